@@ -1,0 +1,104 @@
+/*
+ * mase_amd C ABI: gfx950 (MI355X) kernels for MASE's quantized-inference hot path.
+ *
+ * Every entry point
+ *   - takes plain device pointers, sizes and format integers (no framework types),
+ *   - enqueues its kernels on `stream` (a hipStream_t passed as void*) and returns immediately,
+ *   - never allocates, frees or synchronises,
+ *   - returns MASE_OK (0) or a negative MASE_ERR_* code; it never throws or aborts.
+ * Tensors are dense and contiguous in the order stated for each call.  "dtype" is one of MASE_DT_*.
+ *
+ * Reference interfaces replaced (paths relative to the reference's src/chop/):
+ *   mase_mxint_qdq          nn/quantizers/mxint/mxint.py:211-251  (mxint_quantizer, non-search branch :145-169;
+ *                           arithmetic nn/quantizers/mxint/fake.py:11-80)
+ *   mase_block_fp_qdq       nn/quantizers/block_fp.py:111-142     (block_fp_quantizer; arithmetic :7-82,
+ *                           blocking nn/quantizers/utils.py:350-629)
+ *   mase_integer_qdq        nn/quantizers/integer.py:97-122       (integer_quantizer / integer_floor_quantizer)
+ *   mase_minifloat_qdq      nn/quantizers/minifloat.py:90-117, :200-225 (minifloat_denorm/ieee_quantizer)
+ *   mase_minifloat_mx_qdq   nn/quantizers/_minifloat_mx/minifloat.py:12-33 (minifloat_quantizer_sim)
+ *   mase_mxfp_qdq           nn/quantizers/mxfp/mxfp.py:187-230    (mxfp_quantizer, non-search branch)
+ *   mase_mx_linear_bf16     nn/quantized/modules/linear.py:956-972 (LinearMXInt.forward: F.linear on the
+ *                           quantize-dequantized operands) and :877-895 (LinearMXFP.forward)
+ *   mase_mxfp_linear_scaled nn/quantized/modules/linear.py:877-895 (LinearMXFP.forward, native scaled MFMA)
+ */
+#ifndef MASE_AMD_H
+#define MASE_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MASE_OK 0
+#define MASE_ERR_NULL (-1)      /* a required pointer is NULL */
+#define MASE_ERR_SHAPE (-2)     /* sizes inconsistent (e.g. numel not divisible by the block size) */
+#define MASE_ERR_ALIGN (-3)     /* a pointer is not aligned as the call requires */
+#define MASE_ERR_DTYPE (-4)     /* unknown dtype code */
+#define MASE_ERR_PARAM (-5)     /* format parameter outside the supported domain */
+#define MASE_ERR_LAUNCH (-6)    /* the HIP runtime rejected a launch */
+#define MASE_ERR_WORKSPACE (-7) /* workspace missing or too small */
+
+#define MASE_DT_F32 0
+#define MASE_DT_BF16 1
+#define MASE_DT_F16 2
+
+/* number of uint32 entries in a log2 correction table (see mase_log2_table_layout below) */
+#define MASE_LOG2_TABLE_WORDS 576
+
+int mase_abi_version(void);
+const char* mase_error_string(int code);
+
+/*
+ * log2 correction tables.  The reference evaluates ceil(log2(v)) / floor(log2(v)) with the host math
+ * library *in the tensor dtype*, whose rounded result differs from the exact integer answer for values
+ * a few ulps away from a power of two.  To be bit-exact the kernels take a table measured on the host
+ * (one per dtype), in device memory, MASE_LOG2_TABLE_WORDS uint32 words:
+ *   tab[k+149]       largest normalised 23-bit mantissa M>0 with ceil(log2(2^k*(1+M/2^23))) == k, else 0
+ *   tab[288+k+149]   smallest M with floor(log2(2^k*(1+M/2^23))) == k+1, else 0x800000
+ * for k = floor(log2 v) in [-149, 127].  A table of zeros / 0x800000 gives the exact integer answers.
+ */
+
+/* MXINT quantize-dequantize over contiguous runs of `block_size` elements of a flat array.
+ * in/out: numel elements of `dtype`.  codes (int8, numel) and scales (uint8, numel/block_size) are
+ * optional packed outputs (both or neither; element_bits <= 8): value = codes * 2^(scales - 134). */
+int mase_mxint_qdq(const void* in, void* out, int8_t* codes, uint8_t* scales, size_t numel, int dtype,
+                   int block_size, int element_bits, int scale_bits, const uint32_t* log2_tab, void* stream);
+
+/* Block floating point over [batch, rows, cols] with tiles of tile_rows x tile_cols inside each batch
+ * item (ragged edges behave as if zero padded).  exponent_bias < 0 selects 2^(exponent_width-1)-1.
+ * workspace: mase_block_fp_workspace_bytes() bytes of device memory (may be NULL when that is 0). */
+size_t mase_block_fp_workspace_bytes(size_t batch, size_t rows, size_t cols, int tile_rows, int tile_cols,
+                                     int dtype);
+int mase_block_fp_qdq(const void* in, void* out, size_t batch, size_t rows, size_t cols, int tile_rows,
+                      int tile_cols, int dtype, int width, int exponent_width, int exponent_bias,
+                      const uint32_t* log2_tab, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Fixed point: clamp(round_or_floor(x * 2^frac_width)) / 2^frac_width. */
+int mase_integer_qdq(const void* in, void* out, size_t numel, int dtype, int width, int frac_width,
+                     int is_signed, int use_floor, void* stream);
+
+/* Element-wise minifloat, ieee = 0 (no implicit leading bit) or 1 (implicit leading bit). */
+int mase_minifloat_qdq(const void* in, void* out, size_t numel, int dtype, int width, int exponent_width,
+                       int exponent_bias, int ieee, const uint32_t* log2_tab, void* stream);
+
+/* Bit-level minifloat cast used by the MX formats.  round_mode: 0 rn, 1 ru, 2 rd, 3 rz. */
+int mase_minifloat_mx_qdq(const void* in, void* out, size_t numel, int in_dtype, int out_dtype, int exp_bits,
+                          int frac_bits, int is_finite, int round_mode, void* stream);
+
+/* MXFP quantize-dequantize over contiguous runs of block_size elements.  log2_tab is the fp32 table.
+ * Optional packed outputs: codes (uint8, numel; sign|exp|frac in the low 1+E+F bits) and scales
+ * (uint8 E8M0, numel/block_size). */
+int mase_mxfp_qdq(const void* in, void* out, uint8_t* codes, uint8_t* scales, size_t numel, int in_dtype,
+                  int out_dtype, int block_size, int exp_bits, int frac_bits, const uint32_t* log2_tab,
+                  void* stream);
+
+/* test/diagnostic helpers (host only, no device work) */
+uint32_t mase_isclose_zero_threshold_bits(int dtype); /* largest |x| (fp32 bits) that isclose(x, 0) accepts */
+float mase_round_scalar_to_dtype(double v, int dtype); /* how a clamp bound is represented in dtype */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MASE_AMD_H */

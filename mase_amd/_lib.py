@@ -1,0 +1,84 @@
+"""ctypes binding of ``libmase_amd.so`` (the C ABI declared in ``include/mase_amd.h``).
+
+The library is the only compute path of this package: if it is missing, or a call fails, an exception is
+raised.  There is no fallback to framework ops.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_double, c_float, c_int, c_size_t, c_uint32, c_void_p
+
+import torch
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libmase_amd.so")
+
+DT_F32, DT_BF16, DT_F16 = 0, 1, 2
+DTYPE_CODE = {torch.float32: DT_F32, torch.bfloat16: DT_BF16, torch.float16: DT_F16}
+LOG2_TABLE_WORDS = 576
+
+
+class MaseAmdError(RuntimeError):
+    pass
+
+
+# name -> (restype, argtypes); one entry per symbol declared in include/mase_amd.h
+SIGNATURES = {
+    "mase_abi_version": (c_int, []),
+    "mase_error_string": (c_char_p, [c_int]),
+    "mase_mxint_qdq": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "mase_block_fp_workspace_bytes": (c_size_t, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int]),
+    "mase_block_fp_qdq": (c_int, [c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "mase_integer_qdq": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "mase_minifloat_qdq": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "mase_minifloat_mx_qdq": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "mase_mxfp_qdq": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "mase_isclose_zero_threshold_bits": (c_uint32, [c_int]),
+    "mase_round_scalar_to_dtype": (c_float, [c_double, c_int]),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Loads the shared library (once).  Raises MaseAmdError when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise MaseAmdError(
+            f"{LIB_PATH} not found: build it with `python -m mase_amd.build` (hipcc, gfx950). "
+            "mase_amd has no CPU or framework fallback."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        msg = load().mase_error_string(code).decode()
+        raise MaseAmdError(f"{what} failed: {msg} (code {code})")
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    try:
+        return DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise MaseAmdError(f"mase_amd kernels support float32, bfloat16 and float16 tensors, got {t.dtype}") from None
+
+
+def require_device(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise MaseAmdError(
+            f"{what}: expected a tensor on a ROCm device, got device '{t.device}'. "
+            "mase_amd runs on MI355X only and has no CPU path."
+        )
+
+
+def stream_ptr(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream

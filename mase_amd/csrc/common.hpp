@@ -1,0 +1,188 @@
+// Shared device helpers for the gfx950 quantize-dequantize kernels.
+//
+// All arithmetic is carried in fp32 registers.  Every reference operation on a bf16/fp16 tensor is
+// "compute in fp32, round once to the tensor dtype", so a kernel only needs an explicit rounding step
+// where the fp32 result is not already representable in the tensor dtype; the places where that can
+// happen are listed next to each kernel.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mase_amd.h"
+
+namespace mase {
+
+constexpr int kThreads = 256;
+
+// ---------------------------------------------------------------------------------------------
+// dtype traits: 16-byte vectors of the storage type <-> fp32 registers
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float bits2f(uint32_t b) { return __builtin_bit_cast(float, b); }
+__device__ __forceinline__ uint32_t f2bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// fp32 -> bf16 bits, round-to-nearest-even (NaN kept quiet)
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t b = f2bits(f);
+  uint32_t r = (b + 0x7FFFu + ((b >> 16) & 1u)) >> 16;
+  return ((b & 0x7FFFFFFFu) > 0x7F800000u) ? ((b >> 16) | 0x40u) : r;
+}
+__device__ __forceinline__ float round_to_bf16(float f) { return bits2f(f32_to_bf16_bits(f) << 16); }
+__device__ __forceinline__ float round_to_f16(float f) { return (float)(_Float16)f; }
+
+// streaming (non-temporal) 16-byte accesses: inputs are read once and outputs never re-read
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load_nt(const uint4* p) {
+  u32x4_t v = __builtin_nontemporal_load((const u32x4_t*)p);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void store_nt(uint4* p, const uint4& v) {
+  u32x4_t w = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(w, (u32x4_t*)p);
+}
+
+template <int DT> struct DTypeTraits;
+
+template <> struct DTypeTraits<MASE_DT_F32> {
+  static constexpr int kVec = 4;       // elements per 16-byte vector
+  static constexpr int kBytes = 4;
+  static constexpr int kMaxPow2 = 127; // largest k with 2^k finite
+  static constexpr uint32_t kTinyBits = 0x00800000u;  // finfo.tiny as fp32 bits
+  __device__ static __forceinline__ float round(float f) { return f; }
+  __device__ static __forceinline__ void unpack(const uint4& v, float* x) {
+    x[0] = bits2f(v.x); x[1] = bits2f(v.y); x[2] = bits2f(v.z); x[3] = bits2f(v.w);
+  }
+  __device__ static __forceinline__ uint4 pack(const float* x) {
+    return make_uint4(f2bits(x[0]), f2bits(x[1]), f2bits(x[2]), f2bits(x[3]));
+  }
+  __device__ static __forceinline__ float load1(const void* p, size_t i) { return ((const float*)p)[i]; }
+  __device__ static __forceinline__ void store1(void* p, size_t i, float f) { ((float*)p)[i] = f; }
+};
+
+template <> struct DTypeTraits<MASE_DT_BF16> {
+  static constexpr int kVec = 8;
+  static constexpr int kBytes = 2;
+  static constexpr int kMaxPow2 = 127;
+  static constexpr uint32_t kTinyBits = 0x00800000u;
+  __device__ static __forceinline__ float round(float f) { return round_to_bf16(f); }
+  __device__ static __forceinline__ void unpack(const uint4& v, float* x) {
+    x[0] = bits2f(v.x << 16); x[1] = bits2f(v.x & 0xFFFF0000u);
+    x[2] = bits2f(v.y << 16); x[3] = bits2f(v.y & 0xFFFF0000u);
+    x[4] = bits2f(v.z << 16); x[5] = bits2f(v.z & 0xFFFF0000u);
+    x[6] = bits2f(v.w << 16); x[7] = bits2f(v.w & 0xFFFF0000u);
+  }
+  __device__ static __forceinline__ uint4 pack(const float* x) {
+    uint4 v;
+    v.x = f32_to_bf16_bits(x[0]) | (f32_to_bf16_bits(x[1]) << 16);
+    v.y = f32_to_bf16_bits(x[2]) | (f32_to_bf16_bits(x[3]) << 16);
+    v.z = f32_to_bf16_bits(x[4]) | (f32_to_bf16_bits(x[5]) << 16);
+    v.w = f32_to_bf16_bits(x[6]) | (f32_to_bf16_bits(x[7]) << 16);
+    return v;
+  }
+  __device__ static __forceinline__ float load1(const void* p, size_t i) {
+    return bits2f((uint32_t)((const uint16_t*)p)[i] << 16);
+  }
+  __device__ static __forceinline__ void store1(void* p, size_t i, float f) {
+    ((uint16_t*)p)[i] = (uint16_t)f32_to_bf16_bits(f);
+  }
+};
+
+template <> struct DTypeTraits<MASE_DT_F16> {
+  static constexpr int kVec = 8;
+  static constexpr int kBytes = 2;
+  static constexpr int kMaxPow2 = 15;
+  static constexpr uint32_t kTinyBits = 0x38800000u;  // 2^-14 as fp32 bits
+  __device__ static __forceinline__ float round(float f) { return round_to_f16(f); }
+  __device__ static __forceinline__ float h2f(uint32_t h) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+  }
+  __device__ static __forceinline__ uint32_t f2h(float f) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+  }
+  __device__ static __forceinline__ void unpack(const uint4& v, float* x) {
+    x[0] = h2f(v.x & 0xFFFFu); x[1] = h2f(v.x >> 16);
+    x[2] = h2f(v.y & 0xFFFFu); x[3] = h2f(v.y >> 16);
+    x[4] = h2f(v.z & 0xFFFFu); x[5] = h2f(v.z >> 16);
+    x[6] = h2f(v.w & 0xFFFFu); x[7] = h2f(v.w >> 16);
+  }
+  __device__ static __forceinline__ uint4 pack(const float* x) {
+    uint4 v;
+    v.x = f2h(x[0]) | (f2h(x[1]) << 16);
+    v.y = f2h(x[2]) | (f2h(x[3]) << 16);
+    v.z = f2h(x[4]) | (f2h(x[5]) << 16);
+    v.w = f2h(x[6]) | (f2h(x[7]) << 16);
+    return v;
+  }
+  __device__ static __forceinline__ float load1(const void* p, size_t i) { return h2f(((const uint16_t*)p)[i]); }
+  __device__ static __forceinline__ void store1(void* p, size_t i, float f) { ((uint16_t*)p)[i] = (uint16_t)f2h(f); }
+};
+
+// ---------------------------------------------------------------------------------------------
+// wave64 lane exchange: max over aligned groups of LANES consecutive lanes (LANES = 1..64, power of 2)
+// quad_perm / row_half_mirror / row_mirror DPP for 2..16 lanes, ds_bpermute beyond a 16-lane row.
+// ---------------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_mov(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, 0xF, 0xF, false);
+}
+
+template <int LANES>
+__device__ __forceinline__ uint32_t group_max_u32(uint32_t v) {
+  if constexpr (LANES >= 2) v = max(v, dpp_mov<0xB1>(v));   // quad_perm:[1,0,3,2]
+  if constexpr (LANES >= 4) v = max(v, dpp_mov<0x4E>(v));   // quad_perm:[2,3,0,1]
+  if constexpr (LANES >= 8) v = max(v, dpp_mov<0x141>(v));  // row_half_mirror
+  if constexpr (LANES >= 16) v = max(v, dpp_mov<0x140>(v)); // row_mirror
+  if constexpr (LANES >= 32) v = max(v, (uint32_t)__shfl_xor((int)v, 16, 64));
+  if constexpr (LANES >= 64) v = max(v, (uint32_t)__shfl_xor((int)v, 32, 64));
+  return v;
+}
+
+// ---------------------------------------------------------------------------------------------
+// ceil(log2(v)) / floor(log2(v)) "as the host library evaluates them in the tensor dtype".
+//
+// v is a positive, finite, non-zero value of the tensor dtype, given as fp32 bits.  The exact integer
+// answer is corrected with per-exponent thresholds measured on the host at start-up:
+//   tab[k + 149]        largest normalised 23-bit mantissa M > 0 for which ceil(log2(2^k (1+M/2^23))) == k
+//                       (0 when there is none: the exact answer k+1 is what the library returns)
+//   tab[288 + k + 149]  smallest M for which floor(log2(2^k (1+M/2^23))) == k+1 (0x800000 when none)
+// ---------------------------------------------------------------------------------------------
+constexpr int kLog2TabHalf = 288;
+
+__device__ __forceinline__ int split_pow2(uint32_t b, uint32_t& M) {
+  int E = (int)(b >> 23);
+  M = b & 0x7FFFFFu;
+  if (E == 0) {  // fp32 subnormal: normalise
+    int sh = __clz(M) - 8;
+    M = (M << sh) & 0x7FFFFFu;
+    E = 1 - sh;
+  }
+  return E - 127;
+}
+
+__device__ __forceinline__ int ceil_log2_lib(uint32_t b, const uint32_t* __restrict__ tab) {
+  uint32_t M;
+  int k = split_pow2(b, M);
+  if (M == 0) return k;
+  return (M <= tab[k + 149]) ? k : k + 1;
+}
+
+__device__ __forceinline__ int floor_log2_lib(uint32_t b, const uint32_t* __restrict__ tab) {
+  uint32_t M;
+  int k = split_pow2(b, M);
+  return (M >= tab[kLog2TabHalf + k + 149]) ? k + 1 : k;
+}
+
+// 2^e as fp32 for e in [-149, 127]; callers handle e > 127 themselves
+__device__ __forceinline__ float pow2f(int e) {
+  return (e >= -126) ? bits2f((uint32_t)(e + 127) << 23) : bits2f(1u << (e + 149));
+}
+
+__device__ __forceinline__ float qnan() { return bits2f(0x7FC00000u); }
+
+// host-side launch geometry
+static inline unsigned blocks_for(size_t items, size_t per_block) {
+  return (unsigned)((items + per_block - 1) / per_block);
+}
+
+static inline bool aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
+
+}  // namespace mase

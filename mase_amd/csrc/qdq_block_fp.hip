@@ -1,0 +1,248 @@
+// Block floating point (MSFP) quantize-dequantize for gfx950.
+//
+// Reference arithmetic (nn/quantizers/block_fp.py:7-82), every op in the tensor dtype T, per tile
+// (blocking: nn/quantizers/utils.py:350-629), mb = width-1, bias = 2^(ew-1)-1 unless given:
+//   mx  = max|x| over the tile (ragged edges zero padded)
+//   e   = clamp(ceil(log2(mx)), -bias, 2^ew-1-bias)            (log2 as the library rounds it in T)
+//   v_i = |x_i| + 1e-9                                          (rounded to T)
+//   q_i = clamp(rne(v_i / 2^e * 2^mb), 0, 2^mb-1)               (bounds cast to T)
+//   y_i = sign(x_i + 1e-9) * 2^e * (q_i / 2^mb)
+//   out = isclose(x_i, 0) ? x_i (with -0 -> +0) : y_i carrying the sign of x_i (also on zero results)
+// The reference's substitute exponent for all-zero tiles never reaches an output (all elements of such a
+// tile take the isclose branch), so tiles are independent.  Power-of-two scalings are exact in fp32
+// registers; T-rounding is applied to v_i and to the final product.  Tiles holding Inf/NaN, or whose 2^e
+// overflows T, come out as NaN like the reference's 0*inf.
+//
+// Two schedules:
+//  * run kernel   tile_rows == 1 and cols % tile_cols == 0: tiles are contiguous runs; one pass, 16-byte
+//                 loads/stores, tile maximum by DPP inside the wavefront.
+//  * tile kernels any tile shape / ragged edge: pass 1 reduces |x| per tile with atomicMax into a caller
+//                 workspace, pass 2 quantizes; both are coalesced along the last dimension.
+#include "common.hpp"
+
+namespace mase {
+namespace {
+
+struct BfpParams {
+  int mb;            // mantissa bits = width - 1
+  int e_lo, e_hi;    // exponent clamp
+  float qmax;        // 2^mb - 1 as T represents it
+  uint32_t close_thr;  // |x| bits <= close_thr  <=>  isclose(x, 0)
+  const uint32_t* tab;
+};
+
+constexpr int kUnroll = 4;
+
+// returns 0: zero tile, 1: regular (e valid), 2: NaN tile
+template <int DT>
+__device__ __forceinline__ int tile_exponent(uint32_t mbits, const BfpParams& p, int& e) {
+  using TR = DTypeTraits<DT>;
+  if (mbits == 0) return 0;
+  if (mbits >= 0x7F800000u) return 2;
+  e = min(max(ceil_log2_lib(mbits, p.tab), p.e_lo), p.e_hi);
+  return (e > TR::kMaxPow2) ? 2 : 1;
+}
+
+template <int DT>
+__device__ __forceinline__ float bfp_element(float x, int state, int e, const BfpParams& p) {
+  using TR = DTypeTraits<DT>;
+  uint32_t xb = f2bits(x);
+  uint32_t ab = xb & 0x7FFFFFFFu;
+  if (state == 2) return qnan();
+  if (ab <= p.close_thr) return (ab == 0) ? 0.0f : x;
+  float v = TR::round(bits2f(ab) + 1e-9f);
+  float q = fminf(fmaxf(rintf(ldexpf(v, p.mb - e)), 0.0f), p.qmax);
+  float y = ldexpf(q, e - p.mb);
+  return bits2f(f2bits(y) | (xb & 0x80000000u));
+}
+
+template <int DT, int LPB, int SUB>
+__global__ __launch_bounds__(kThreads) void bfp_run_kernel(const uint4* __restrict__ in, uint4* __restrict__ out,
+                                                           size_t n_vec, BfpParams p) {
+  using TR = DTypeTraits<DT>;
+  constexpr int V = TR::kVec;
+  constexpr int EPS = V / SUB;
+  const size_t base = (size_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+  uint4 raw[kUnroll];
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    size_t idx = base + (size_t)u * kThreads;
+    raw[u] = (idx < n_vec) ? load_nt(in + idx) : make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    size_t idx = base + (size_t)u * kThreads;
+    float x[V], y[V];
+    TR::unpack(raw[u], x);
+#pragma unroll
+    for (int s = 0; s < SUB; ++s) {
+      uint32_t m = 0;
+#pragma unroll
+      for (int j = 0; j < EPS; ++j) m = max(m, f2bits(x[s * EPS + j]) & 0x7FFFFFFFu);
+      m = group_max_u32<LPB>(m);
+      int e = 0;
+      int state = tile_exponent<DT>(m, p, e);
+#pragma unroll
+      for (int j = 0; j < EPS; ++j) y[s * EPS + j] = bfp_element<DT>(x[s * EPS + j], state, e, p);
+    }
+    if (idx < n_vec) store_nt(out + idx, TR::pack(y));
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void fill_u32_kernel(uint32_t* __restrict__ p, size_t n, uint32_t v) {
+  size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+struct TileGeom {
+  size_t rows, cols;        // per batch item
+  size_t tiles_r, tiles_c;  // tiles per batch item along rows / cols
+  int b0, b1;
+  size_t col_groups;        // groups of kGroup consecutive columns per row
+  size_t total_groups;      // batch * rows * col_groups
+};
+constexpr int kGroup = 8;
+
+// One work-item per group of kGroup consecutive columns of one row.
+template <int DT, int PASS>
+__global__ __launch_bounds__(kThreads) void bfp_tile_kernel(const void* __restrict__ in, void* __restrict__ out,
+                                                            uint32_t* __restrict__ tile_max, TileGeom g,
+                                                            BfpParams p) {
+  using TR = DTypeTraits<DT>;
+  size_t gid = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  if (gid >= g.total_groups) return;
+  size_t cg = gid % g.col_groups;
+  size_t row_all = gid / g.col_groups;  // batch * rows + row
+  size_t b = row_all / g.rows, r = row_all % g.rows;
+  size_t c0 = cg * kGroup;
+  size_t c1 = min(c0 + (size_t)kGroup, g.cols);
+  size_t tile_row_base = (b * g.tiles_r + r / g.b0) * g.tiles_c;
+  size_t off = row_all * g.cols;
+  if constexpr (PASS == 1) {
+    size_t cur = c0 / g.b1;
+    uint32_t m = 0;
+    for (size_t c = c0; c < c1; ++c) {
+      size_t t = c / g.b1;
+      if (t != cur) {
+        if (m) atomicMax(&tile_max[tile_row_base + cur], m);
+        cur = t;
+        m = 0;
+      }
+      m = max(m, f2bits(TR::load1(in, off + c)) & 0x7FFFFFFFu);
+    }
+    if (m) atomicMax(&tile_max[tile_row_base + cur], m);
+  } else {
+    size_t cur = (size_t)-1;
+    int e = 0, state = 0;
+    for (size_t c = c0; c < c1; ++c) {
+      size_t t = c / g.b1;
+      if (t != cur) {
+        cur = t;
+        state = tile_exponent<DT>(tile_max[tile_row_base + cur], p, e);
+      }
+      TR::store1(out, off + c, bfp_element<DT>(TR::load1(in, off + c), state, e, p));
+    }
+  }
+}
+
+bool run_path_ok(const void* in, const void* out, size_t numel, size_t cols, int b0, int b1, int V) {
+  return b0 == 1 && (b1 & (b1 - 1)) == 0 && b1 <= 64 * V && cols % (size_t)b1 == 0 && numel % (size_t)V == 0 &&
+         aligned16(in) && aligned16(out);
+}
+
+template <int DT>
+int launch_bfp(const void* in, void* out, size_t batch, size_t rows, size_t cols, int b0, int b1, const BfpParams& p,
+               void* ws, size_t ws_bytes, hipStream_t st) {
+  using TR = DTypeTraits<DT>;
+  constexpr int V = TR::kVec;
+  size_t numel = batch * rows * cols;
+  if (run_path_ok(in, out, numel, cols, b0, b1, V)) {
+    size_t n_vec = numel / V;
+    dim3 grid(blocks_for(n_vec, (size_t)kThreads * kUnroll)), block(kThreads);
+#define MASE_BFP_CASE(LPB_, SUB_) \
+  hipLaunchKernelGGL((bfp_run_kernel<DT, LPB_, SUB_>), grid, block, 0, st, (const uint4*)in, (uint4*)out, n_vec, p)
+    if (b1 >= V) {
+      switch (b1 / V) {
+        case 1: MASE_BFP_CASE(1, 1); break;
+        case 2: MASE_BFP_CASE(2, 1); break;
+        case 4: MASE_BFP_CASE(4, 1); break;
+        case 8: MASE_BFP_CASE(8, 1); break;
+        case 16: MASE_BFP_CASE(16, 1); break;
+        case 32: MASE_BFP_CASE(32, 1); break;
+        default: MASE_BFP_CASE(64, 1); break;
+      }
+    } else {
+      switch (V / b1) {
+        case 2: MASE_BFP_CASE(1, 2); break;
+        case 4: MASE_BFP_CASE(1, 4); break;
+        default:
+          if constexpr (V == 8) MASE_BFP_CASE(1, 8);
+          break;
+      }
+    }
+#undef MASE_BFP_CASE
+    return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+  }
+  TileGeom g;
+  g.rows = rows;
+  g.cols = cols;
+  g.b0 = b0;
+  g.b1 = b1;
+  g.tiles_r = (rows + b0 - 1) / b0;
+  g.tiles_c = (cols + b1 - 1) / b1;
+  g.col_groups = (cols + kGroup - 1) / kGroup;
+  g.total_groups = batch * rows * g.col_groups;
+  size_t n_tiles = batch * g.tiles_r * g.tiles_c;
+  if (ws == nullptr || ws_bytes < n_tiles * sizeof(uint32_t)) return MASE_ERR_WORKSPACE;
+  uint32_t* tm = (uint32_t*)ws;
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(blocks_for(n_tiles, kThreads)), dim3(kThreads), 0, st, tm, n_tiles, 0u);
+  dim3 grid(blocks_for(g.total_groups, kThreads)), block(kThreads);
+  hipLaunchKernelGGL((bfp_tile_kernel<DT, 1>), grid, block, 0, st, in, out, tm, g, p);
+  hipLaunchKernelGGL((bfp_tile_kernel<DT, 2>), grid, block, 0, st, in, out, tm, g, p);
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+int vec_of(int dtype) { return dtype == MASE_DT_F32 ? 4 : 8; }
+int min_pow2_of(int dtype) { return dtype == MASE_DT_F32 ? -149 : (dtype == MASE_DT_BF16 ? -133 : -24); }
+
+}  // namespace
+}  // namespace mase
+
+extern "C" size_t mase_block_fp_workspace_bytes(size_t batch, size_t rows, size_t cols, int tile_rows, int tile_cols,
+                                                int dtype) {
+  using namespace mase;
+  if (tile_rows <= 0 || tile_cols <= 0) return 0;
+  // the run path additionally needs 16-byte aligned pointers; a caller that cannot guarantee them must
+  // provide the workspace, so report the tile-path size whenever the shape alone does not decide
+  size_t tiles = batch * ((rows + tile_rows - 1) / tile_rows) * ((cols + tile_cols - 1) / tile_cols);
+  return tiles * sizeof(uint32_t);
+}
+
+extern "C" int mase_block_fp_qdq(const void* in, void* out, size_t batch, size_t rows, size_t cols, int tile_rows,
+                                 int tile_cols, int dtype, int width, int exponent_width, int exponent_bias,
+                                 const uint32_t* log2_tab, void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace mase;
+  if (batch == 0 || rows == 0 || cols == 0) return MASE_OK;
+  if (in == nullptr || out == nullptr || log2_tab == nullptr) return MASE_ERR_NULL;
+  if (tile_rows <= 0 || tile_cols <= 0) return MASE_ERR_SHAPE;
+  if (dtype != MASE_DT_F32 && dtype != MASE_DT_BF16 && dtype != MASE_DT_F16) return MASE_ERR_DTYPE;
+  if (width < 2 || width > 25 || exponent_width < 1 || exponent_width > 16) return MASE_ERR_PARAM;
+  BfpParams p;
+  p.mb = width - 1;
+  int bias = exponent_bias < 0 ? (1 << (exponent_width - 1)) - 1 : exponent_bias;
+  p.e_lo = -bias;
+  p.e_hi = (1 << exponent_width) - 1 - bias;
+  if (p.e_hi < min_pow2_of(dtype)) return MASE_ERR_PARAM;  // 2^e would underflow to zero in the dtype
+  p.qmax = mase_round_scalar_to_dtype((double)((1 << p.mb) - 1), dtype);
+  p.close_thr = mase_isclose_zero_threshold_bits(dtype);
+  p.tab = log2_tab;
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case MASE_DT_F32:
+      return launch_bfp<MASE_DT_F32>(in, out, batch, rows, cols, tile_rows, tile_cols, p, workspace, workspace_bytes, st);
+    case MASE_DT_BF16:
+      return launch_bfp<MASE_DT_BF16>(in, out, batch, rows, cols, tile_rows, tile_cols, p, workspace, workspace_bytes, st);
+    default:
+      return launch_bfp<MASE_DT_F16>(in, out, batch, rows, cols, tile_rows, tile_cols, p, workspace, workspace_bytes, st);
+  }
+}

@@ -1,0 +1,270 @@
+// Element-wise quantize-dequantize kernels for gfx950: fixed point, minifloat (denorm / ieee flavours) and
+// the bit-level minifloat cast used by the MX formats.
+//
+// The two minifloat flavours are restated operation by operation: each reference op on a tensor of dtype
+// T is "fp32 op, then round to T", written R(.) below, because with narrow T the intermediate values
+// (2^e underflowing to 0 in fp16, clamp bounds that T cannot represent, ...) are part of the result.
+#include "common.hpp"
+#include "minifloat_mx.hpp"
+
+namespace mase {
+namespace {
+
+// ---------------------------------------------------------------------------------------------
+// generic driver: 8 elements per work-item through 16-byte accesses, scalar tail
+// ---------------------------------------------------------------------------------------------
+template <int DT>
+__device__ __forceinline__ void load8(const void* p, size_t i8, float* x) {
+  using TR = DTypeTraits<DT>;
+  if constexpr (TR::kVec == 4) {
+    const uint4* q = (const uint4*)p + 2 * i8;
+    uint4 a = load_nt(q), b = load_nt(q + 1);
+    TR::unpack(a, x);
+    TR::unpack(b, x + 4);
+  } else {
+    uint4 a = load_nt((const uint4*)p + i8);
+    TR::unpack(a, x);
+  }
+}
+template <int DT>
+__device__ __forceinline__ void store8(void* p, size_t i8, const float* y) {
+  using TR = DTypeTraits<DT>;
+  if constexpr (TR::kVec == 4) {
+    uint4* q = (uint4*)p + 2 * i8;
+    store_nt(q, TR::pack(y));
+    store_nt(q + 1, TR::pack(y + 4));
+  } else {
+    store_nt((uint4*)p + i8, TR::pack(y));
+  }
+}
+
+template <int DTI, int DTO, typename F>
+__global__ __launch_bounds__(kThreads) void elementwise_kernel(const void* __restrict__ in, void* __restrict__ out,
+                                                               size_t n8, size_t numel, F f) {
+  __shared__ uint32_t lds_tab[F::kUsesTable ? MASE_LOG2_TABLE_WORDS : 1];
+  if constexpr (F::kUsesTable) {
+    for (int i = threadIdx.x; i < MASE_LOG2_TABLE_WORDS; i += kThreads) lds_tab[i] = f.tab[i];
+    __syncthreads();
+  }
+  size_t t = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  if (t < n8) {
+    float x[8], y[8];
+    load8<DTI>(in, t, x);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) y[j] = f(x[j], lds_tab);
+    store8<DTO>(out, t, y);
+  } else {
+    size_t i = n8 * 8 + (t - n8);
+    if (i < numel) DTypeTraits<DTO>::store1(out, i, f(DTypeTraits<DTI>::load1(in, i), lds_tab));
+  }
+}
+
+template <int DTI, int DTO, typename F>
+int launch_elementwise(const void* in, void* out, size_t numel, const F& f, hipStream_t st) {
+  size_t n8 = (aligned16(in) && aligned16(out)) ? numel / 8 : 0;
+  size_t threads = n8 + (numel - n8 * 8);
+  hipLaunchKernelGGL((elementwise_kernel<DTI, DTO, F>), dim3(blocks_for(threads, kThreads)), dim3(kThreads), 0, st, in,
+                     out, n8, numel, f);
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+// clamp as "min(max(a, lo), hi)" with the library's scalar-compare semantics: NaN propagates and
+// -0.0 is not replaced by a +0.0 bound.
+__device__ __forceinline__ float clamp_cmp(float a, float lo, float hi) {
+  a = (a < lo) ? lo : a;
+  a = (a > hi) ? hi : a;
+  return a;
+}
+
+// ---------------------------------------------------------------------------------------------
+// fixed point: integer.py:10-66
+// ---------------------------------------------------------------------------------------------
+template <int DT>
+struct IntegerOp {
+  static constexpr bool kUsesTable = false;
+  const uint32_t* tab;
+  int frac;
+  int use_floor;
+  float lo, hi;
+  __device__ __forceinline__ float operator()(float x, const uint32_t*) const {
+    float t = ldexpf(x, frac);
+    float r = use_floor ? floorf(t) : rintf(t);
+    r = clamp_cmp(r, lo, hi);
+    return ldexpf(r, -frac);  // rounded to T by the store
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+// minifloat denorm / ieee: minifloat.py:7-68 and :120-182
+// ---------------------------------------------------------------------------------------------
+template <int DT, bool IEEE>
+struct MinifloatOp {
+  using TR = DTypeTraits<DT>;
+  static constexpr bool kUsesTable = true;
+  const uint32_t* tab;
+  int mb;
+  float e_lo, e_hi;  // exponent clamp (as floats; representable in every T for exponent_width <= 8)
+  float qmax;        // 2^mb - 1 as T represents it
+  float shift;       // 2^mb
+  uint32_t close_thr;
+  float neg_bias;    // -exponent_bias as T represents it (ieee)
+
+  __device__ static __forceinline__ float R(float f) { return TR::round(f); }
+
+  // library log2 of a T value followed by ceil (denorm) or floor (ieee), as a float
+  __device__ __forceinline__ float log2_rounded(float l, const uint32_t* t) const {
+    uint32_t b = f2bits(l);
+    if (b == 0) return -__builtin_inff();
+    if (b >= 0x7F800000u) return (b == 0x7F800000u) ? __builtin_inff() : qnan();  // l >= 0 here or NaN
+    return (float)(IEEE ? floor_log2_lib(b, t) : ceil_log2_lib(b, t));
+  }
+  // 2^e evaluated in T for an integer-valued float e
+  __device__ static __forceinline__ float pow2_T(float e) {
+    if (e != e) return e;
+    if (e > (float)TR::kMaxPow2) return __builtin_inff();
+    if (e < -160.0f) return 0.0f;
+    return R(ldexpf(1.0f, (int)e));
+  }
+
+  __device__ __forceinline__ float operator()(float x, const uint32_t* t) const {
+    float xs = R(x + 1e-9f);
+    float sgn = (xs > 0.0f) ? 1.0f : ((xs < 0.0f) ? -1.0f : xs);
+    float val = fabsf(x);
+    float l = R(val + 1e-9f);
+    float e = clamp_cmp(log2_rounded(l, t), e_lo, e_hi);
+    float p2 = pow2_T(e);
+    float man = R(val / p2);
+    float mant;
+    if constexpr (!IEEE) {
+      float q = clamp_cmp(rintf(R(man * shift)), 0.0f, qmax);
+      mant = R(q / shift);
+    } else {
+      bool normal = !(e == neg_bias);
+      float ms = R(man * shift);
+      float a1 = clamp_cmp(rintf(R(ms - shift)), 0.0f, qmax);
+      float a2 = clamp_cmp(rintf(R(ms / 2.0f)), 0.0f, qmax);
+      float q = normal ? R(a1 + R(0.0f * a2)) : R(R(0.0f * a1) + a2);
+      float m1 = R(1.0f + R(q / shift));
+      float m2 = R(R(q / shift) * 2.0f);
+      mant = normal ? R(m1 + R(0.0f * m2)) : R(R(0.0f * m1) + m2);
+    }
+    float y = R(R(sgn * p2) * mant);
+    bool close = (f2bits(val) <= close_thr);
+    return close ? R(R(0.0f * y) + x) : R(y + R(0.0f * x));
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+// bit-level minifloat cast: _minifloat_mx/fake.py:11-149 (encode to a code, decode it back)
+// ---------------------------------------------------------------------------------------------
+struct MinifloatMxOp {
+  static constexpr bool kUsesTable = false;
+  const uint32_t* tab;
+  MinifloatMxFmt m;
+  __device__ __forceinline__ float operator()(float x, const uint32_t*) const {
+    return minifloat_mx_decode(minifloat_mx_encode(x, m), m);
+  }
+};
+
+template <typename MakeOp>
+int dispatch_same_dtype(int dtype, MakeOp&& mk) {
+  switch (dtype) {
+    case MASE_DT_F32: return mk.template run<MASE_DT_F32>();
+    case MASE_DT_BF16: return mk.template run<MASE_DT_BF16>();
+    case MASE_DT_F16: return mk.template run<MASE_DT_F16>();
+    default: return MASE_ERR_DTYPE;
+  }
+}
+
+struct IntegerRun {
+  const void* in; void* out; size_t numel; int dtype, width, frac, is_signed, use_floor; hipStream_t st;
+  template <int DT> int run() {
+    IntegerOp<DT> op;
+    op.tab = nullptr;
+    op.frac = frac;
+    op.use_floor = use_floor;
+    double lo = is_signed ? -(double)(1ull << (width - 1)) : 0.0;
+    double hi = is_signed ? (double)((1ull << (width - 1)) - 1) : (double)((1ull << width) - 1);
+    op.lo = mase_round_scalar_to_dtype(lo, dtype);
+    op.hi = mase_round_scalar_to_dtype(hi, dtype);
+    return launch_elementwise<DT, DT>(in, out, numel, op, st);
+  }
+};
+
+struct MinifloatRun {
+  const void* in; void* out; size_t numel; int dtype, width, ew, bias, ieee; const uint32_t* tab; hipStream_t st;
+  template <int DT, bool IEEE> int go() {
+    MinifloatOp<DT, IEEE> op;
+    op.tab = tab;
+    op.mb = width - ew - 1;
+    op.e_lo = (float)(-bias);
+    op.e_hi = (float)((1 << ew) - 1 - bias);
+    op.qmax = mase_round_scalar_to_dtype((double)((1 << op.mb) - 1), dtype);
+    op.shift = (float)(1 << op.mb);
+    op.close_thr = mase_isclose_zero_threshold_bits(dtype);
+    op.neg_bias = -mase_round_scalar_to_dtype((double)bias, dtype);
+    return launch_elementwise<DT, DT>(in, out, numel, op, st);
+  }
+  template <int DT> int run() { return ieee ? go<DT, true>() : go<DT, false>(); }
+};
+
+struct MinifloatMxRun {
+  const void* in; void* out; size_t numel; int out_dtype; MinifloatMxFmt m; hipStream_t st;
+  template <int DTI> int run() {
+    MinifloatMxOp op;
+    op.tab = nullptr;
+    op.m = m;
+    switch (out_dtype) {
+      case MASE_DT_F32: return launch_elementwise<DTI, MASE_DT_F32>(in, out, numel, op, st);
+      case MASE_DT_BF16: return launch_elementwise<DTI, MASE_DT_BF16>(in, out, numel, op, st);
+      case MASE_DT_F16: return launch_elementwise<DTI, MASE_DT_F16>(in, out, numel, op, st);
+      default: return MASE_ERR_DTYPE;
+    }
+  }
+};
+
+}  // namespace
+}  // namespace mase
+
+extern "C" int mase_integer_qdq(const void* in, void* out, size_t numel, int dtype, int width, int frac_width,
+                                int is_signed, int use_floor, void* stream) {
+  using namespace mase;
+  if (numel == 0) return MASE_OK;
+  if (in == nullptr || out == nullptr) return MASE_ERR_NULL;
+  if (width < 1 || width > 32 || frac_width < -64 || frac_width > 64) return MASE_ERR_PARAM;
+  IntegerRun r{in, out, numel, dtype, width, frac_width, is_signed, use_floor, (hipStream_t)stream};
+  return dispatch_same_dtype(dtype, r);
+}
+
+extern "C" int mase_minifloat_qdq(const void* in, void* out, size_t numel, int dtype, int width, int exponent_width,
+                                  int exponent_bias, int ieee, const uint32_t* log2_tab, void* stream) {
+  using namespace mase;
+  if (numel == 0) return MASE_OK;
+  if (in == nullptr || out == nullptr || log2_tab == nullptr) return MASE_ERR_NULL;
+  if (exponent_width < 1 || exponent_width > 8 || width - exponent_width - 1 < 0 || width - exponent_width - 1 > 23)
+    return MASE_ERR_PARAM;
+  int bias = exponent_bias < 0 ? (1 << (exponent_width - 1)) - 1 : exponent_bias;
+  if (bias > 255) return MASE_ERR_PARAM;
+  MinifloatRun r{in, out, numel, dtype, width, exponent_width, bias, ieee, log2_tab, (hipStream_t)stream};
+  return dispatch_same_dtype(dtype, r);
+}
+
+extern "C" int mase_minifloat_mx_qdq(const void* in, void* out, size_t numel, int in_dtype, int out_dtype, int exp_bits,
+                                     int frac_bits, int is_finite, int round_mode, void* stream) {
+  using namespace mase;
+  if (numel == 0) return MASE_OK;
+  if (in == nullptr || out == nullptr) return MASE_ERR_NULL;
+  if (exp_bits <= 0 || frac_bits <= 0 || exp_bits + frac_bits >= 16 || round_mode < 0 || round_mode > 3)
+    return MASE_ERR_PARAM;
+  if (exp_bits > 8) return MASE_ERR_PARAM;  // exponent range beyond fp32's is not representable in the decode
+  MinifloatMxFmt m;
+  m.E = exp_bits;
+  m.F = frac_bits;
+  m.bias = (1 << (exp_bits - 1)) - 1;
+  m.e_hi = is_finite ? (1 << exp_bits) - 1 : (1 << exp_bits) - 2;
+  m.frac_hi = (1 << frac_bits) - 1;
+  m.is_finite = is_finite;
+  m.round_mode = round_mode;
+  MinifloatMxRun r{in, out, numel, out_dtype, m, (hipStream_t)stream};
+  return dispatch_same_dtype(in_dtype, r);
+}

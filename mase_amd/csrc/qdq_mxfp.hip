@@ -1,0 +1,221 @@
+// MXFP quantize-dequantize (and optional packing) for gfx950.
+//
+// Reference arithmetic (nn/quantizers/mxfp/fake.py:12-104), always in fp32 whatever the tensor dtype, per
+// block of B consecutive elements, element format (E, F) with el_emax = 2^E-1-bias_E (finite elements,
+// round-to-nearest):
+//   t_i  = x_i with fp32 subnormals flushed to +0
+//   sh   = clamp(floor(log2(max|t|)) - el_emax, -127, 128)       (log2 as the library rounds it in fp32)
+//   c_i  = minifloat_encode(t_i / 2^sh)                           (bit-level, see minifloat_mx.hpp)
+//   y_i  = minifloat_decode(c_i) * 2^sh, converted to the output dtype;  scale byte = sh + 127
+// An all-flushed block has scale byte 0 and decodes to +0.  A block holding Inf/NaN decodes to NaN in the
+// reference (its int32 conversion of log2 wraps to the largest scale, 0 * inf), and does here.
+#include "common.hpp"
+#include "minifloat_mx.hpp"
+
+namespace mase {
+namespace {
+
+struct MxfpParams {
+  MinifloatMxFmt m;
+  int el_emax;
+  const uint32_t* tab;  // fp32 table (floor half is used)
+};
+
+constexpr int kUnroll = 2;
+
+// state 0: all flushed, 1: regular (sh valid), 2: NaN block
+__device__ __forceinline__ int mxfp_block_scale(uint32_t mbits, const MxfpParams& p, int& sh) {
+  if (mbits == 0) return 0;
+  if (mbits >= 0x7F800000u) return 2;
+  sh = min(max(floor_log2_lib(mbits, p.tab) - p.el_emax, -127), 128);
+  return 1;
+}
+
+__device__ __forceinline__ float mxfp_element(float t, int state, int sh, const MxfpParams& p, uint32_t& code) {
+  code = 0;
+  if (state == 0) return 0.0f;
+  if (state == 2) return qnan();
+  code = minifloat_mx_encode(ldexpf(t, -sh), p.m);
+  return minifloat_mx_decode(code, p.m) * pow2f(sh);
+}
+
+__device__ __forceinline__ float flush_subnormal(float x) {
+  return ((f2bits(x) & 0x7F800000u) == 0) ? 0.0f : x;
+}
+
+template <int DTI, int DTO, int LPB, int SUB>
+__global__ __launch_bounds__(kThreads) void mxfp_qdq_vec_kernel(const void* __restrict__ in, void* __restrict__ out,
+                                                                uint8_t* __restrict__ codes,
+                                                                uint8_t* __restrict__ scales, size_t n_vec,
+                                                                MxfpParams p) {
+  using TI = DTypeTraits<DTI>;
+  using TO = DTypeTraits<DTO>;
+  // work in units of 8 elements when either side is a 16-bit type, else 4
+  constexpr int V = (TI::kVec == 8 || TO::kVec == 8) ? 8 : 4;
+  constexpr int EPS = V / SUB;
+  const size_t base = (size_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    size_t idx = base + (size_t)u * kThreads;
+    bool live = idx < n_vec;
+    float x[V], y[V];
+    uint32_t c[V];
+    if (live) {
+      if constexpr (TI::kVec == V) {
+        TI::unpack(load_nt((const uint4*)in + idx), x);
+      } else {  // fp32 input, 8 per item
+        TI::unpack(load_nt((const uint4*)in + 2 * idx), x);
+        TI::unpack(load_nt((const uint4*)in + 2 * idx + 1), x + 4);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < V; ++j) x[j] = 0.0f;
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) x[j] = flush_subnormal(x[j]);
+#pragma unroll
+    for (int s = 0; s < SUB; ++s) {
+      uint32_t m = 0;
+#pragma unroll
+      for (int j = 0; j < EPS; ++j) m = max(m, f2bits(x[s * EPS + j]) & 0x7FFFFFFFu);
+      m = group_max_u32<LPB>(m);
+      int sh = 0;
+      int state = mxfp_block_scale(m, p, sh);
+#pragma unroll
+      for (int j = 0; j < EPS; ++j) y[s * EPS + j] = mxfp_element(x[s * EPS + j], state, sh, p, c[s * EPS + j]);
+      if (codes != nullptr && live) {
+        int sb = (state == 1) ? sh + 127 : (state == 0 ? 0 : 255);
+        if constexpr (LPB > 1) {
+          if ((idx & (LPB - 1)) == 0) scales[idx / LPB] = (uint8_t)sb;
+        } else {
+          scales[idx * SUB + s] = (uint8_t)sb;
+        }
+      }
+    }
+    if (live) {
+      if constexpr (TO::kVec == V) {
+        store_nt((uint4*)out + idx, TO::pack(y));
+      } else {
+        store_nt((uint4*)out + 2 * idx, TO::pack(y));
+        store_nt((uint4*)out + 2 * idx + 1, TO::pack(y + 4));
+      }
+      if (codes != nullptr) {
+        if constexpr (V == 4) {
+          ((uint32_t*)codes)[idx] = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+        } else {
+          uint2 w;
+          w.x = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+          w.y = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
+          ((uint2*)codes)[idx] = w;
+        }
+      }
+    }
+  }
+}
+
+template <int DTI, int DTO>
+__global__ __launch_bounds__(kThreads) void mxfp_qdq_generic_kernel(const void* __restrict__ in, void* __restrict__ out,
+                                                                    uint8_t* __restrict__ codes,
+                                                                    uint8_t* __restrict__ scales, size_t n_blocks,
+                                                                    int B, MxfpParams p) {
+  size_t blk = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  if (blk >= n_blocks) return;
+  size_t off = blk * (size_t)B;
+  uint32_t m = 0;
+  for (int j = 0; j < B; ++j) m = max(m, f2bits(flush_subnormal(DTypeTraits<DTI>::load1(in, off + j))) & 0x7FFFFFFFu);
+  int sh = 0;
+  int state = mxfp_block_scale(m, p, sh);
+  for (int j = 0; j < B; ++j) {
+    uint32_t c;
+    float y = mxfp_element(flush_subnormal(DTypeTraits<DTI>::load1(in, off + j)), state, sh, p, c);
+    DTypeTraits<DTO>::store1(out, off + j, y);
+    if (codes != nullptr) codes[off + j] = (uint8_t)c;
+  }
+  if (codes != nullptr) scales[blk] = (uint8_t)((state == 1) ? sh + 127 : (state == 0 ? 0 : 255));
+}
+
+template <int DTI, int DTO>
+int launch_mxfp(const void* in, void* out, uint8_t* codes, uint8_t* scales, size_t numel, int B, const MxfpParams& p,
+                hipStream_t st) {
+  constexpr int V = (DTypeTraits<DTI>::kVec == 8 || DTypeTraits<DTO>::kVec == 8) ? 8 : 4;
+  const bool pow2 = (B & (B - 1)) == 0;
+  const bool vec_ok = pow2 && B <= 64 * V && (numel % V) == 0 && aligned16(in) && aligned16(out) &&
+                      (codes == nullptr || (((uintptr_t)codes) & 7u) == 0);
+  if (vec_ok) {
+    size_t n_vec = numel / V;
+    dim3 grid(blocks_for(n_vec, (size_t)kThreads * kUnroll)), block(kThreads);
+#define MASE_MXFP_CASE(LPB_, SUB_)                                                                               \
+  hipLaunchKernelGGL((mxfp_qdq_vec_kernel<DTI, DTO, LPB_, SUB_>), grid, block, 0, st, in, out, codes, scales, n_vec, p)
+    if (B >= V) {
+      switch (B / V) {
+        case 1: MASE_MXFP_CASE(1, 1); break;
+        case 2: MASE_MXFP_CASE(2, 1); break;
+        case 4: MASE_MXFP_CASE(4, 1); break;
+        case 8: MASE_MXFP_CASE(8, 1); break;
+        case 16: MASE_MXFP_CASE(16, 1); break;
+        case 32: MASE_MXFP_CASE(32, 1); break;
+        default: MASE_MXFP_CASE(64, 1); break;
+      }
+    } else {
+      switch (V / B) {
+        case 2: MASE_MXFP_CASE(1, 2); break;
+        case 4: MASE_MXFP_CASE(1, 4); break;
+        default:
+          if constexpr (V == 8) MASE_MXFP_CASE(1, 8);
+          break;
+      }
+    }
+#undef MASE_MXFP_CASE
+  } else {
+    size_t n_blocks = numel / (size_t)B;
+    hipLaunchKernelGGL((mxfp_qdq_generic_kernel<DTI, DTO>), dim3(blocks_for(n_blocks, kThreads)), dim3(kThreads), 0, st,
+                       in, out, codes, scales, n_blocks, B, p);
+  }
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+template <int DTI>
+int launch_mxfp_out(int out_dtype, const void* in, void* out, uint8_t* codes, uint8_t* scales, size_t numel, int B,
+                    const MxfpParams& p, hipStream_t st) {
+  switch (out_dtype) {
+    case MASE_DT_F32: return launch_mxfp<DTI, MASE_DT_F32>(in, out, codes, scales, numel, B, p, st);
+    case MASE_DT_BF16: return launch_mxfp<DTI, MASE_DT_BF16>(in, out, codes, scales, numel, B, p, st);
+    case MASE_DT_F16: return launch_mxfp<DTI, MASE_DT_F16>(in, out, codes, scales, numel, B, p, st);
+    default: return MASE_ERR_DTYPE;
+  }
+}
+
+}  // namespace
+}  // namespace mase
+
+extern "C" int mase_mxfp_qdq(const void* in, void* out, uint8_t* codes, uint8_t* scales, size_t numel, int in_dtype,
+                             int out_dtype, int block_size, int exp_bits, int frac_bits, const uint32_t* log2_tab,
+                             void* stream) {
+  using namespace mase;
+  if (numel == 0) return MASE_OK;
+  if (in == nullptr || out == nullptr || log2_tab == nullptr) return MASE_ERR_NULL;
+  if ((codes == nullptr) != (scales == nullptr)) return MASE_ERR_NULL;
+  if (block_size <= 0 || numel % (size_t)block_size != 0) return MASE_ERR_SHAPE;
+  // legal element formats of the reference (nn/quantizers/mxfp/meta.py:41)
+  const int legal[6][2] = {{4, 3}, {5, 2}, {2, 3}, {3, 2}, {2, 1}, {1, 2}};
+  bool ok = false;
+  for (auto& l : legal) ok = ok || (l[0] == exp_bits && l[1] == frac_bits);
+  if (!ok) return MASE_ERR_PARAM;
+  MxfpParams p;
+  p.m.E = exp_bits;
+  p.m.F = frac_bits;
+  p.m.bias = (1 << (exp_bits - 1)) - 1;
+  p.m.e_hi = (1 << exp_bits) - 1;
+  p.m.frac_hi = (1 << frac_bits) - 1;
+  p.m.is_finite = 1;
+  p.m.round_mode = 0;
+  p.el_emax = p.m.e_hi - p.m.bias;
+  p.tab = log2_tab;
+  hipStream_t st = (hipStream_t)stream;
+  switch (in_dtype) {
+    case MASE_DT_F32: return launch_mxfp_out<MASE_DT_F32>(out_dtype, in, out, codes, scales, numel, block_size, p, st);
+    case MASE_DT_BF16: return launch_mxfp_out<MASE_DT_BF16>(out_dtype, in, out, codes, scales, numel, block_size, p, st);
+    case MASE_DT_F16: return launch_mxfp_out<MASE_DT_F16>(out_dtype, in, out, codes, scales, numel, block_size, p, st);
+    default: return MASE_ERR_DTYPE;
+  }
+}

@@ -1,0 +1,205 @@
+// MXINT quantize-dequantize (and optional packing) for gfx950.
+//
+// Reference arithmetic (nn/quantizers/mxint/fake.py:11-80), per block of B consecutive elements, b =
+// element_bits, s = scale_bits, bias = 2^(s-1)-1, all in the tensor dtype T:
+//   mx  = max(max|x|, tiny(T));  k = ceil(log2(mx)) as the library rounds it in T
+//   m_i = clamp(rne(x_i / 2^k * 2^(b-1)), -2^(b-1), 2^(b-1)-1)        (bounds cast to T)
+//   kc  = clamp(k + bias, 0, 2^s-1) - bias
+//   y_i = m_i / 2^(b-1) * 2^kc
+// Scaling by powers of two is exact in fp32 registers; the only roundings are rne() and the final
+// conversion to T (which matters only for subnormal results).  x_i/2^k can be inexact only when it is
+// subnormal, and then m_i is 0 either way.  A block whose 2^k overflows T (or holds Inf/NaN) comes out
+// as NaN in the reference (0 * inf), and does here.
+//
+// Bandwidth-bound: one 16-byte load and one 16-byte store per lane per vector, kUnroll independent loads
+// in flight per lane, block maximum by DPP inside the wavefront, no LDS.
+#include "common.hpp"
+
+namespace mase {
+namespace {
+
+struct MxintParams {
+  int qshift;     // b - 1
+  int bias;       // 2^(s-1) - 1
+  int scale_max;  // 2^s - 1
+  float lo, hi;   // clamp bounds as T represents them
+  const uint32_t* tab;
+};
+
+constexpr int kUnroll = 4;
+
+template <int DT>
+__device__ __forceinline__ bool block_exponent(uint32_t mbits, const MxintParams& p, int& k, int& kc) {
+  using TR = DTypeTraits<DT>;
+  mbits = max(mbits, TR::kTinyBits);
+  if (mbits >= 0x7F800000u) return false;
+  k = ceil_log2_lib(mbits, p.tab);
+  if (k > TR::kMaxPow2) return false;
+  kc = min(max(k + p.bias, 0), p.scale_max) - p.bias;
+  return true;
+}
+
+__device__ __forceinline__ float quantize_mant(float x, int k, const MxintParams& p) {
+  float r = rintf(ldexpf(x, p.qshift - k));
+  return fminf(fmaxf(r, p.lo), p.hi);
+}
+
+// LPB lanes share one block (B = LPB * kVec) or one lane holds SUB blocks (B = kVec / SUB).
+template <int DT, int LPB, int SUB>
+__global__ __launch_bounds__(kThreads) void mxint_qdq_vec_kernel(const uint4* __restrict__ in, uint4* __restrict__ out,
+                                                                 int8_t* __restrict__ codes,
+                                                                 uint8_t* __restrict__ scales, size_t n_vec,
+                                                                 MxintParams p) {
+  using TR = DTypeTraits<DT>;
+  constexpr int V = TR::kVec;
+  constexpr int EPS = V / SUB;  // elements per sub-block held by this lane
+  const size_t base = (size_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+
+  uint4 raw[kUnroll];
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    size_t idx = base + (size_t)u * kThreads;
+    raw[u] = (idx < n_vec) ? load_nt(in + idx) : make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    size_t idx = base + (size_t)u * kThreads;
+    float x[V];
+    TR::unpack(raw[u], x);
+    float y[V];
+    int8_t c[V];
+#pragma unroll
+    for (int s = 0; s < SUB; ++s) {
+      uint32_t m = 0;
+#pragma unroll
+      for (int j = 0; j < EPS; ++j) m = max(m, f2bits(x[s * EPS + j]) & 0x7FFFFFFFu);
+      m = group_max_u32<LPB>(m);
+      int k = 0, kc = 0;
+      bool ok = block_exponent<DT>(m, p, k, kc);
+#pragma unroll
+      for (int j = 0; j < EPS; ++j) {
+        float r = quantize_mant(x[s * EPS + j], k, p);
+        y[s * EPS + j] = ok ? ldexpf(r, kc - p.qshift) : qnan();
+        c[s * EPS + j] = ok ? (int8_t)(int)r : (int8_t)0;
+      }
+      if (codes != nullptr && idx < n_vec) {
+        int sb = ok ? min(max(kc - p.qshift + 134, 0), 255) : 255;
+        if constexpr (LPB > 1) {
+          if ((idx & (LPB - 1)) == 0) scales[idx / LPB] = (uint8_t)sb;
+        } else {
+          scales[idx * SUB + s] = (uint8_t)sb;
+        }
+      }
+    }
+    if (idx < n_vec) {
+      store_nt(out + idx, TR::pack(y));
+      if (codes != nullptr) {
+        if constexpr (V == 4) {
+          uint32_t w = (uint32_t)(uint8_t)c[0] | ((uint32_t)(uint8_t)c[1] << 8) | ((uint32_t)(uint8_t)c[2] << 16) |
+                       ((uint32_t)(uint8_t)c[3] << 24);
+          ((uint32_t*)codes)[idx] = w;
+        } else {
+          uint2 w;
+          w.x = (uint32_t)(uint8_t)c[0] | ((uint32_t)(uint8_t)c[1] << 8) | ((uint32_t)(uint8_t)c[2] << 16) |
+                ((uint32_t)(uint8_t)c[3] << 24);
+          w.y = (uint32_t)(uint8_t)c[4] | ((uint32_t)(uint8_t)c[5] << 8) | ((uint32_t)(uint8_t)c[6] << 16) |
+                ((uint32_t)(uint8_t)c[7] << 24);
+          ((uint2*)codes)[idx] = w;
+        }
+      }
+    }
+  }
+}
+
+// Any block size / alignment: one work-item per block, two passes over its elements.
+template <int DT>
+__global__ __launch_bounds__(kThreads) void mxint_qdq_generic_kernel(const void* __restrict__ in, void* __restrict__ out,
+                                                                     int8_t* __restrict__ codes,
+                                                                     uint8_t* __restrict__ scales, size_t n_blocks,
+                                                                     int B, MxintParams p) {
+  using TR = DTypeTraits<DT>;
+  size_t blk = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  if (blk >= n_blocks) return;
+  size_t off = blk * (size_t)B;
+  uint32_t m = 0;
+  for (int j = 0; j < B; ++j) m = max(m, f2bits(TR::load1(in, off + j)) & 0x7FFFFFFFu);
+  int k = 0, kc = 0;
+  bool ok = block_exponent<DT>(m, p, k, kc);
+  for (int j = 0; j < B; ++j) {
+    float r = quantize_mant(TR::load1(in, off + j), k, p);
+    TR::store1(out, off + j, ok ? ldexpf(r, kc - p.qshift) : qnan());
+    if (codes != nullptr) codes[off + j] = ok ? (int8_t)(int)r : (int8_t)0;
+  }
+  if (codes != nullptr) scales[blk] = (uint8_t)(ok ? min(max(kc - p.qshift + 134, 0), 255) : 255);
+}
+
+template <int DT>
+int launch_mxint(const void* in, void* out, int8_t* codes, uint8_t* scales, size_t numel, int B, const MxintParams& p,
+                 hipStream_t st) {
+  using TR = DTypeTraits<DT>;
+  constexpr int V = TR::kVec;
+  const bool pow2 = (B & (B - 1)) == 0;
+  const bool vec_ok = pow2 && B <= 64 * V && (numel % V) == 0 && aligned16(in) && aligned16(out) &&
+                      (codes == nullptr || (((uintptr_t)codes) & 7u) == 0);
+  if (vec_ok) {
+    size_t n_vec = numel / V;
+    dim3 grid(blocks_for(n_vec, (size_t)kThreads * kUnroll)), block(kThreads);
+#define MASE_MXINT_CASE(LPB_, SUB_)                                                                          \
+  hipLaunchKernelGGL((mxint_qdq_vec_kernel<DT, LPB_, SUB_>), grid, block, 0, st, (const uint4*)in, (uint4*)out, \
+                     codes, scales, n_vec, p)
+    if (B >= V) {
+      switch (B / V) {
+        case 1: MASE_MXINT_CASE(1, 1); break;
+        case 2: MASE_MXINT_CASE(2, 1); break;
+        case 4: MASE_MXINT_CASE(4, 1); break;
+        case 8: MASE_MXINT_CASE(8, 1); break;
+        case 16: MASE_MXINT_CASE(16, 1); break;
+        case 32: MASE_MXINT_CASE(32, 1); break;
+        default: MASE_MXINT_CASE(64, 1); break;
+      }
+    } else {
+      switch (V / B) {
+        case 2: MASE_MXINT_CASE(1, 2); break;
+        case 4: MASE_MXINT_CASE(1, 4); break;
+        default:
+          if constexpr (V == 8) MASE_MXINT_CASE(1, 8);
+          break;
+      }
+    }
+#undef MASE_MXINT_CASE
+  } else {
+    size_t n_blocks = numel / (size_t)B;
+    hipLaunchKernelGGL((mxint_qdq_generic_kernel<DT>), dim3(blocks_for(n_blocks, kThreads)), dim3(kThreads), 0, st, in,
+                       out, codes, scales, n_blocks, B, p);
+  }
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+}  // namespace
+}  // namespace mase
+
+extern "C" int mase_mxint_qdq(const void* in, void* out, int8_t* codes, uint8_t* scales, size_t numel, int dtype,
+                              int block_size, int element_bits, int scale_bits, const uint32_t* log2_tab,
+                              void* stream) {
+  using namespace mase;
+  if (numel == 0) return MASE_OK;
+  if (in == nullptr || out == nullptr || log2_tab == nullptr) return MASE_ERR_NULL;
+  if ((codes == nullptr) != (scales == nullptr)) return MASE_ERR_NULL;
+  if (block_size <= 0 || numel % (size_t)block_size != 0) return MASE_ERR_SHAPE;
+  if (element_bits < 2 || element_bits > 24 || scale_bits < 1 || scale_bits > 8) return MASE_ERR_PARAM;
+  if (codes != nullptr && element_bits > 8) return MASE_ERR_PARAM;
+  if (dtype != MASE_DT_F32 && dtype != MASE_DT_BF16 && dtype != MASE_DT_F16) return MASE_ERR_DTYPE;
+  MxintParams p;
+  p.qshift = element_bits - 1;
+  p.bias = (1 << (scale_bits - 1)) - 1;
+  p.scale_max = (1 << scale_bits) - 1;
+  p.lo = mase_round_scalar_to_dtype(-(double)(1 << (element_bits - 1)), dtype);
+  p.hi = mase_round_scalar_to_dtype((double)((1 << (element_bits - 1)) - 1), dtype);
+  p.tab = log2_tab;
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case MASE_DT_F32: return launch_mxint<MASE_DT_F32>(in, out, codes, scales, numel, block_size, p, st);
+    case MASE_DT_BF16: return launch_mxint<MASE_DT_BF16>(in, out, codes, scales, numel, block_size, p, st);
+    default: return launch_mxint<MASE_DT_F16>(in, out, codes, scales, numel, block_size, p, st);
+  }
+}

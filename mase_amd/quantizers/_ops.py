@@ -1,0 +1,223 @@
+"""Host side of the quantize-dequantize functions: argument handling, layout, launches through the C ABI.
+
+Mirrors the public functions of the reference's ``chop.nn.quantizers`` (same names, argument meaning,
+defaults and error behaviour); the arithmetic itself lives in ``mase_amd/csrc``.
+"""
+from __future__ import annotations
+
+from math import ceil
+from typing import List, Sequence
+
+import torch
+from torch import Tensor
+
+from .. import _lib
+from .._tables import log2_table
+
+
+def _contig(x: Tensor) -> Tensor:
+    x = x.contiguous()
+    if x.data_ptr() % 16 != 0:  # views with odd storage offsets: realign so the 16-byte path applies
+        x = x.clone(memory_format=torch.contiguous_format)
+    return x
+
+
+# ------------------------------------------------------------------------------------------------
+# layout helpers with the semantics of mxfp/helpers.py:8-63
+# ------------------------------------------------------------------------------------------------
+def _to_block_last_flat(x: Tensor, block_dim: int) -> Tensor:
+    nd = x.dim()
+    d = block_dim % nd
+    if d == nd - 1:
+        return _contig(x).view(-1)
+    order = [i for i in range(nd) if i != d] + [d]
+    return _contig(x.permute(order)).view(-1)
+
+
+def _from_block_last_flat(flat: Tensor, shape: Sequence[int], block_dim: int) -> Tensor:
+    nd = len(shape)
+    d = block_dim % nd
+    if d == nd - 1:
+        return flat.view(shape)
+    moved = [s for i, s in enumerate(shape) if i != d] + [shape[d]]
+    back = list(range(nd - 1))
+    back.insert(d, nd - 1)
+    return flat.view(moved).permute(back)
+
+
+# ------------------------------------------------------------------------------------------------
+# MXINT  (reference: mxint/mxint.py:211-251)
+# ------------------------------------------------------------------------------------------------
+def mxint_qdq(x: Tensor, block_size: int, element_bits: int, block_dim: int, scale_bits: int, pack: bool = False):
+    """Returns the dequantized tensor, or (dequantized, codes int8, scales uint8) when ``pack``."""
+    _lib.require_device(x, "mxint_quantizer")
+    lib = _lib.load()
+    shape = tuple(x.shape)
+    nd = len(shape)
+    assert block_dim < nd and block_dim >= -nd
+    assert x.numel() % block_size == 0, f"Input tensor size {x.numel()} is not divisible by block size {block_size}."
+    flat = _to_block_last_flat(x, block_dim)
+    out = torch.empty_like(flat)
+    codes = scales = None
+    if pack:
+        codes = torch.empty(flat.numel(), dtype=torch.int8, device=x.device)
+        scales = torch.empty(flat.numel() // block_size, dtype=torch.uint8, device=x.device)
+    tab = log2_table(x.dtype, x.device)
+    rc = lib.mase_mxint_qdq(
+        flat.data_ptr(), out.data_ptr(),
+        codes.data_ptr() if pack else None, scales.data_ptr() if pack else None,
+        flat.numel(), _lib.dtype_code(x), block_size, element_bits, scale_bits, tab.data_ptr(), _lib.stream_ptr(x),
+    )
+    _lib.check(rc, "mase_mxint_qdq")
+    res = _from_block_last_flat(out, shape, block_dim)
+    return (res, codes, scales) if pack else res
+
+
+# ------------------------------------------------------------------------------------------------
+# MXFP  (reference: mxfp/mxfp.py:187-230)
+# ------------------------------------------------------------------------------------------------
+_LEGAL_MXFP = ((4, 3), (5, 2), (2, 3), (3, 2), (2, 1), (1, 2))
+
+
+def mxfp_qdq(x: Tensor, block_size: int, exp_bits: int, frac_bits: int, block_dim: int, scale_exp_bits: int,
+             pack: bool = False):
+    _lib.require_device(x, "mxfp_quantizer")
+    lib = _lib.load()
+    assert scale_exp_bits in (8,), f"Invalid scale exponent bits: {scale_exp_bits}. Legal values are: (8,)."
+    assert (exp_bits, frac_bits) in _LEGAL_MXFP, (
+        f"Invalid element exp/frac bits: {(exp_bits, frac_bits)}. Legal values are: {_LEGAL_MXFP}."
+    )
+    shape = tuple(x.shape)
+    nd = len(shape)
+    assert block_dim < nd and block_dim >= -nd
+    assert x.numel() % block_size == 0
+    flat = _to_block_last_flat(x, block_dim)
+    out = torch.empty_like(flat)
+    codes = scales = None
+    if pack:
+        codes = torch.empty(flat.numel(), dtype=torch.uint8, device=x.device)
+        scales = torch.empty(flat.numel() // block_size, dtype=torch.uint8, device=x.device)
+    tab = log2_table(torch.float32, x.device)
+    dt = _lib.dtype_code(x)
+    rc = lib.mase_mxfp_qdq(
+        flat.data_ptr(), out.data_ptr(),
+        codes.data_ptr() if pack else None, scales.data_ptr() if pack else None,
+        flat.numel(), dt, dt, block_size, exp_bits, frac_bits, tab.data_ptr(), _lib.stream_ptr(x),
+    )
+    _lib.check(rc, "mase_mxfp_qdq")
+    res = _from_block_last_flat(out, shape, block_dim)
+    return (res, codes, scales) if pack else res
+
+
+# ------------------------------------------------------------------------------------------------
+# block floating point  (reference: block_fp.py:111-142; blocking utils.py:350-629)
+# ------------------------------------------------------------------------------------------------
+def _infer_block_shape(x_shape: List[int], block_shape: List[int]) -> List[int]:
+    nd, nb = len(x_shape), len(block_shape)
+    inferred = list(block_shape[-nd:]) if nb >= nd else [-1] * (nd - nb) + list(block_shape)
+    return [x_shape[i] if (inferred[i] == -1 or inferred[i] > x_shape[i]) else inferred[i] for i in range(nd)]
+
+
+def block_fp_geometry(shape: Sequence[int], block_size, skip_first_dim: bool):
+    """(batch, rows, cols, tile_rows, tile_cols) the reference's ``block`` dispatch (utils.py:569-592) implies."""
+    if isinstance(block_size, int):
+        block_size = [block_size]
+    block_size = list(block_size)
+    nd = len(shape)
+    if nd == 1:
+        assert skip_first_dim is False, "skip_first_dim must be False for bias to be blocked"
+        bs = _infer_block_shape([shape[0]], block_size)
+        return 1, 1, shape[0], 1, bs[0]
+    if nd == 2:
+        if skip_first_dim:
+            bs = _infer_block_shape([1, shape[1]], block_size)
+            return 1, shape[0], shape[1], 1, bs[-1]
+        bs = _infer_block_shape([shape[0], shape[1]], block_size)
+        return 1, shape[0], shape[1], bs[0], bs[1]
+    if nd == 3:
+        if skip_first_dim:
+            bs = _infer_block_shape([1, shape[1], shape[2]], block_size)
+            return shape[0], shape[1], shape[2], bs[1], bs[2]
+        raise NotImplementedError("block 3d weight is not supported.")
+    raise RuntimeError(f"Unsupported x.ndim = {nd}")
+
+
+def block_fp_qdq(x: Tensor, width: int, exponent_width: int, exponent_bias, block_size, skip_first_dim: bool) -> Tensor:
+    _lib.require_device(x, "block_fp_quantizer")
+    lib = _lib.load()
+    batch, rows, cols, b0, b1 = block_fp_geometry(tuple(x.shape), block_size, skip_first_dim)
+    if exponent_bias in (None, "none", "None"):
+        exponent_bias = -1
+    xin = _contig(x)
+    out = torch.empty_like(xin)
+    if xin.numel() == 0:
+        return out
+    if b0 <= 0 or b1 <= 0:
+        raise RuntimeError(f"invalid block shape {(b0, b1)}")
+    dt = _lib.dtype_code(x)
+    vec = 4 if x.dtype == torch.float32 else 8
+    run_path = b0 == 1 and (b1 & (b1 - 1)) == 0 and b1 <= 64 * vec and cols % b1 == 0 and xin.numel() % vec == 0
+    ws = None
+    ws_bytes = 0
+    if not run_path:
+        ws_bytes = lib.mase_block_fp_workspace_bytes(batch, rows, cols, b0, b1, dt)
+        ws = torch.empty(max(1, ws_bytes // 4), dtype=torch.int32, device=x.device)
+    tab = log2_table(x.dtype, x.device)
+    rc = lib.mase_block_fp_qdq(
+        xin.data_ptr(), out.data_ptr(), batch, rows, cols, b0, b1, dt, width, exponent_width, int(exponent_bias),
+        tab.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes, _lib.stream_ptr(x),
+    )
+    _lib.check(rc, "mase_block_fp_qdq")
+    return out
+
+
+# ------------------------------------------------------------------------------------------------
+# element-wise formats
+# ------------------------------------------------------------------------------------------------
+def integer_qdq(x: Tensor, width: int, frac_width, is_signed: bool, use_floor: bool) -> Tensor:
+    _lib.require_device(x, "integer_quantizer")
+    lib = _lib.load()
+    if frac_width is None:
+        frac_width = width // 2
+    xin = _contig(x)
+    out = torch.empty_like(xin)
+    rc = lib.mase_integer_qdq(xin.data_ptr(), out.data_ptr(), xin.numel(), _lib.dtype_code(x), int(width),
+                              int(frac_width), int(bool(is_signed)), int(bool(use_floor)), _lib.stream_ptr(x))
+    _lib.check(rc, "mase_integer_qdq")
+    return out
+
+
+def minifloat_qdq(x: Tensor, width: int, exponent_width: int, exponent_bias, ieee: bool) -> Tensor:
+    _lib.require_device(x, "minifloat quantizer")
+    lib = _lib.load()
+    if exponent_bias in (None, "none", "None"):
+        exponent_bias = -1
+    xin = _contig(x)
+    out = torch.empty_like(xin)
+    tab = log2_table(x.dtype, x.device)
+    rc = lib.mase_minifloat_qdq(xin.data_ptr(), out.data_ptr(), xin.numel(), _lib.dtype_code(x), int(width),
+                                int(exponent_width), int(exponent_bias), int(bool(ieee)), tab.data_ptr(),
+                                _lib.stream_ptr(x))
+    _lib.check(rc, "mase_minifloat_qdq")
+    return out
+
+
+_ROUND_MODES = {"rn": 0, "ru": 1, "rd": 2, "rz": 3}
+
+
+def minifloat_mx_qdq(x: Tensor, exp_bits: int, frac_bits: int, is_finite: bool, round_mode: str,
+                     output_dtype: torch.dtype | None) -> Tensor:
+    _lib.require_device(x, "minifloat_quantizer_sim")
+    lib = _lib.load()
+    if round_mode not in _ROUND_MODES:
+        raise ValueError(f"Unknown rounding mode: {round_mode}")
+    xin = _contig(x)
+    odt = output_dtype or x.dtype
+    out = torch.empty(xin.shape, dtype=odt, device=x.device)
+    if odt not in _lib.DTYPE_CODE:
+        raise _lib.MaseAmdError(f"unsupported output dtype {odt}")
+    rc = lib.mase_minifloat_mx_qdq(xin.data_ptr(), out.data_ptr(), xin.numel(), _lib.dtype_code(x),
+                                   _lib.DTYPE_CODE[odt], int(exp_bits), int(frac_bits), int(bool(is_finite)),
+                                   _ROUND_MODES[round_mode], _lib.stream_ptr(x))
+    _lib.check(rc, "mase_minifloat_mx_qdq")
+    return out

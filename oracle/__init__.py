@@ -1,0 +1,54 @@
+"""CPU oracle for the quantize-dequantize / quantized-Linear path.  TEST INFRASTRUCTURE ONLY.
+
+This package restates, op for op with plain ``torch`` CPU calls, the arithmetic of the reference's
+``chop.nn.quantizers`` functions and of the quantized ``Linear`` forward that consumes them.  It is the
+checker the HIP kernels are compared against and the timed CPU baseline of the benchmark; nothing in
+the shipped package ``mase_amd`` may import it.  Only ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` use it.
+
+Why torch and not numpy/C: the reference's results depend on library behaviour of torch itself
+(``Tensor.log2`` evaluated *in the tensor dtype*, ``pow(2, t)``, ``round`` half-to-even keeping the
+sign of zero, bf16/fp16 ops computing in fp32 and rounding once, ``clamp`` casting its bounds to the
+tensor dtype, ``isclose`` thresholds).  Restating those in another library would replace the very
+behaviour that has to be matched.  Integer/bit arithmetic (`_minifloat_mx`) is additionally restated
+as a scalar pure-integer routine in ``oracle/scalar.py`` so the two can be checked against each other.
+
+Pinning status (what fixes each function besides reading the source):
+
+* ``integer_quantizer``            closed form (exact rational arithmetic), exhaustive over bf16   -> pinned
+* ``mxint_quantizer``              closed form with torch's own ``log2().ceil()``, invariants       -> pinned
+* ``block_fp_quantizer``           closed form; blocking checked against a brute-force index map   -> pinned
+                                   except the per-op rounding order in bf16/fp16 for width > 9,
+                                   which only the reference could confirm             -> parity unpinned (that part)
+* ``minifloat_denorm/ieee``        closed form in fp32; bf16/fp16 per-op rounding      -> parity unpinned (low-precision part)
+* ``_minifloat_mx`` encode/decode  nearest-value brute force away from the documented quirks; the quirks
+  and ``mxfp_quantizer``           (``>> 8`` double rounding, lost carry in odd binades, truncating subnormals)
+                                   are source-defined                                   -> parity unpinned (quirk regions)
+
+The reference ships no golden vectors or value-asserting tests for this path, and running the reference
+to produce vectors was refused by the environment, so "parity unpinned" above means: restated from the
+source text (file:line cited at each function), cross-checked by an independent scalar restatement, but
+never compared with an execution of the reference.
+"""
+from .quantizers import (  # noqa: F401
+    block_fp_quantizer,
+    integer_floor_quantizer,
+    integer_quantizer,
+    minifloat_denorm_quantizer,
+    minifloat_ieee_quantizer,
+    minifloat_mx_compose,
+    minifloat_mx_extract,
+    minifloat_quantizer_sim,
+    mxfp_components,
+    mxfp_quantizer,
+    mxint_components,
+    mxint_quantizer,
+)
+from .linear import (  # noqa: F401
+    linear_block_fp,
+    linear_integer,
+    linear_minifloat_denorm,
+    linear_minifloat_ieee,
+    linear_mxfp_forward,
+    linear_mxint_forward,
+)
