@@ -68,12 +68,17 @@ int mase_mxint_qdq(const void* in, void* out, int8_t* codes, uint8_t* scales, si
 
 /* Block floating point over [batch, rows, cols] with tiles of tile_rows x tile_cols inside each batch
  * item (ragged edges behave as if zero padded).  exponent_bias < 0 selects 2^(exponent_width-1)-1.
- * workspace: mase_block_fp_workspace_bytes() bytes of device memory (may be NULL when that is 0). */
+ * zero_sign_mode: 0 = an element that quantizes to zero keeps the sign of the input (the reference's
+ * reshape-based blocking of 1-D tensors and of 2-D activations), 1 = it becomes +0 (the reference's
+ * unfold/fold blocking of 2-D weights and 3-D activations, where fold adds into a zero buffer).
+ * workspace: mase_block_fp_workspace_bytes() bytes of device memory; may be NULL when tile_rows == 1,
+ * tile_cols is a power of two dividing cols, and in/out are 16-byte aligned (single-pass schedule). */
 size_t mase_block_fp_workspace_bytes(size_t batch, size_t rows, size_t cols, int tile_rows, int tile_cols,
                                      int dtype);
 int mase_block_fp_qdq(const void* in, void* out, size_t batch, size_t rows, size_t cols, int tile_rows,
                       int tile_cols, int dtype, int width, int exponent_width, int exponent_bias,
-                      const uint32_t* log2_tab, void* workspace, size_t workspace_bytes, void* stream);
+                      int zero_sign_mode, const uint32_t* log2_tab, void* workspace, size_t workspace_bytes,
+                      void* stream);
 
 /* Fixed point: clamp(round_or_floor(x * 2^frac_width)) / 2^frac_width. */
 int mase_integer_qdq(const void* in, void* out, size_t numel, int dtype, int width, int frac_width,

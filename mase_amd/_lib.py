@@ -28,7 +28,7 @@ SIGNATURES = {
     "mase_error_string": (c_char_p, [c_int]),
     "mase_mxint_qdq": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mase_block_fp_workspace_bytes": (c_size_t, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int]),
-    "mase_block_fp_qdq": (c_int, [c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "mase_block_fp_qdq": (c_int, [c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
     "mase_integer_qdq": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "mase_minifloat_qdq": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mase_minifloat_mx_qdq": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),

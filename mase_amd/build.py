@@ -27,6 +27,7 @@ COMMON_FLAGS = [
     "-std=c++17",
     "-fPIC",
     "-fno-gpu-rdc",
+    "-ffp-contract=off",  # the reference rounds after every op; no fused multiply-add behind its back
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall",
     "-Wno-unused-function",

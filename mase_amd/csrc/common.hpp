@@ -27,7 +27,18 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   return ((b & 0x7FFFFFFFu) > 0x7F800000u) ? ((b >> 16) | 0x40u) : r;
 }
 __device__ __forceinline__ float round_to_bf16(float f) { return bits2f(f32_to_bf16_bits(f) << 16); }
-__device__ __forceinline__ float round_to_f16(float f) { return (float)(_Float16)f; }
+// fp32 -> fp16 bits, round-to-nearest-even.  Issued as an explicit instruction: when the compiler sees
+// "(half)(a * b)" it fuses the pair into a mixed-precision fma with a +0 addend, which turns a -0 product
+// into +0 and so loses the sign of zero that the reference keeps.
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+  uint32_t h;
+  asm("v_cvt_f16_f32 %0, %1" : "=v"(h) : "v"(f));
+  return h & 0xFFFFu;
+}
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+__device__ __forceinline__ float round_to_f16(float f) { return f16_bits_to_f32(f32_to_f16_bits(f)); }
 
 // streaming (non-temporal) 16-byte accesses: inputs are read once and outputs never re-read
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -92,12 +103,8 @@ template <> struct DTypeTraits<MASE_DT_F16> {
   static constexpr int kMaxPow2 = 15;
   static constexpr uint32_t kTinyBits = 0x38800000u;  // 2^-14 as fp32 bits
   __device__ static __forceinline__ float round(float f) { return round_to_f16(f); }
-  __device__ static __forceinline__ float h2f(uint32_t h) {
-    return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
-  }
-  __device__ static __forceinline__ uint32_t f2h(float f) {
-    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
-  }
+  __device__ static __forceinline__ float h2f(uint32_t h) { return f16_bits_to_f32(h); }
+  __device__ static __forceinline__ uint32_t f2h(float f) { return f32_to_f16_bits(f); }
   __device__ static __forceinline__ void unpack(const uint4& v, float* x) {
     x[0] = h2f(v.x & 0xFFFFu); x[1] = h2f(v.x >> 16);
     x[2] = h2f(v.y & 0xFFFFu); x[3] = h2f(v.y >> 16);

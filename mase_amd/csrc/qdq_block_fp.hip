@@ -7,11 +7,14 @@
 //   v_i = |x_i| + 1e-9                                          (rounded to T)
 //   q_i = clamp(rne(v_i / 2^e * 2^mb), 0, 2^mb-1)               (bounds cast to T)
 //   y_i = sign(x_i + 1e-9) * 2^e * (q_i / 2^mb)
-//   out = isclose(x_i, 0) ? x_i (with -0 -> +0) : y_i carrying the sign of x_i (also on zero results)
+//   out = isclose(x_i, 0) ? x_i (with -0 -> +0) : y_i carrying the sign of x_i
+// Sign of a zero result: the reference reassembles 2-D weights and 3-D activations with F.fold, which
+// *adds* the blocks into a zero buffer, so a -0 becomes +0 there; 1-D and 2-D activation blocking is a
+// reshape and keeps -0.  The caller selects the behaviour with `zero_sign_mode`.
 // The reference's substitute exponent for all-zero tiles never reaches an output (all elements of such a
 // tile take the isclose branch), so tiles are independent.  Power-of-two scalings are exact in fp32
-// registers; T-rounding is applied to v_i and to the final product.  Tiles holding Inf/NaN, or whose 2^e
-// overflows T, come out as NaN like the reference's 0*inf.
+// registers; T-rounding is applied to v_i and to the final product.  Tiles holding NaN, or whose 2^e
+// overflows T, come out as NaN like the reference's 0*inf; an Inf element saturates when 2^e is finite.
 //
 // Two schedules:
 //  * run kernel   tile_rows == 1 and cols % tile_cols == 0: tiles are contiguous runs; one pass, 16-byte
@@ -28,6 +31,7 @@ struct BfpParams {
   int e_lo, e_hi;    // exponent clamp
   float qmax;        // 2^mb - 1 as T represents it
   uint32_t close_thr;  // |x| bits <= close_thr  <=>  isclose(x, 0)
+  uint32_t zero_sign_mask;  // 0x80000000: a zero result keeps the sign of x; 0: it is +0 (see header)
   const uint32_t* tab;
 };
 
@@ -38,8 +42,9 @@ template <int DT>
 __device__ __forceinline__ int tile_exponent(uint32_t mbits, const BfpParams& p, int& e) {
   using TR = DTypeTraits<DT>;
   if (mbits == 0) return 0;
-  if (mbits >= 0x7F800000u) return 2;
-  e = min(max(ceil_log2_lib(mbits, p.tab), p.e_lo), p.e_hi);
+  if (mbits > 0x7F800000u) return 2;
+  // an infinite maximum has log2 = inf, which the clamp brings down to e_hi
+  e = (mbits == 0x7F800000u) ? p.e_hi : min(max(ceil_log2_lib(mbits, p.tab), p.e_lo), p.e_hi);
   return (e > TR::kMaxPow2) ? 2 : 1;
 }
 
@@ -53,7 +58,8 @@ __device__ __forceinline__ float bfp_element(float x, int state, int e, const Bf
   float v = TR::round(bits2f(ab) + 1e-9f);
   float q = fminf(fmaxf(rintf(ldexpf(v, p.mb - e)), 0.0f), p.qmax);
   float y = ldexpf(q, e - p.mb);
-  return bits2f(f2bits(y) | (xb & 0x80000000u));
+  uint32_t smask = (q == 0.0f) ? p.zero_sign_mask : 0x80000000u;
+  return bits2f(f2bits(y) | (xb & smask));
 }
 
 template <int DT, int LPB, int SUB>
@@ -220,7 +226,8 @@ extern "C" size_t mase_block_fp_workspace_bytes(size_t batch, size_t rows, size_
 
 extern "C" int mase_block_fp_qdq(const void* in, void* out, size_t batch, size_t rows, size_t cols, int tile_rows,
                                  int tile_cols, int dtype, int width, int exponent_width, int exponent_bias,
-                                 const uint32_t* log2_tab, void* workspace, size_t workspace_bytes, void* stream) {
+                                 int zero_sign_mode, const uint32_t* log2_tab, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
   using namespace mase;
   if (batch == 0 || rows == 0 || cols == 0) return MASE_OK;
   if (in == nullptr || out == nullptr || log2_tab == nullptr) return MASE_ERR_NULL;
@@ -235,6 +242,7 @@ extern "C" int mase_block_fp_qdq(const void* in, void* out, size_t batch, size_t
   if (p.e_hi < min_pow2_of(dtype)) return MASE_ERR_PARAM;  // 2^e would underflow to zero in the dtype
   p.qmax = mase_round_scalar_to_dtype((double)((1 << p.mb) - 1), dtype);
   p.close_thr = mase_isclose_zero_threshold_bits(dtype);
+  p.zero_sign_mask = zero_sign_mode ? 0u : 0x80000000u;
   p.tab = log2_tab;
   hipStream_t st = (hipStream_t)stream;
   switch (dtype) {

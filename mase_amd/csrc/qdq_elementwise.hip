@@ -87,7 +87,7 @@ struct IntegerOp {
   int use_floor;
   float lo, hi;
   __device__ __forceinline__ float operator()(float x, const uint32_t*) const {
-    float t = ldexpf(x, frac);
+    float t = DTypeTraits<DT>::round(ldexpf(x, frac));  // x * 2^f underflows differently in narrow T
     float r = use_floor ? floorf(t) : rintf(t);
     r = clamp_cmp(r, lo, hi);
     return ldexpf(r, -frac);  // rounded to T by the store

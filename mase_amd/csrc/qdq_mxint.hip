@@ -8,8 +8,9 @@
 //   y_i = m_i / 2^(b-1) * 2^kc
 // Scaling by powers of two is exact in fp32 registers; the only roundings are rne() and the final
 // conversion to T (which matters only for subnormal results).  x_i/2^k can be inexact only when it is
-// subnormal, and then m_i is 0 either way.  A block whose 2^k overflows T (or holds Inf/NaN) comes out
-// as NaN in the reference (0 * inf), and does here.
+// subnormal, and then m_i is 0 either way.  When 2^k overflows T (or the maximum is Inf) the reference
+// computes x/inf = +-0 and then +-0 * 2^kc, which is NaN when 2^kc is inf as well and +-0 otherwise; a NaN
+// maximum makes the whole block NaN.  The same cases are reproduced here.
 //
 // Bandwidth-bound: one 16-byte load and one 16-byte store per lane per vector, kUnroll independent loads
 // in flight per lane, block maximum by DPP inside the wavefront, no LDS.
@@ -28,20 +29,34 @@ struct MxintParams {
 
 constexpr int kUnroll = 4;
 
+// state 0: regular block (k, kc valid); 1: 2^k overflows T (also an infinite maximum): x/2^k is +-0;
+// 2: the maximum is NaN.
 template <int DT>
-__device__ __forceinline__ bool block_exponent(uint32_t mbits, const MxintParams& p, int& k, int& kc) {
+__device__ __forceinline__ int block_exponent(uint32_t mbits, const MxintParams& p, int& k, int& kc) {
   using TR = DTypeTraits<DT>;
   mbits = max(mbits, TR::kTinyBits);
-  if (mbits >= 0x7F800000u) return false;
-  k = ceil_log2_lib(mbits, p.tab);
-  if (k > TR::kMaxPow2) return false;
+  if (mbits > 0x7F800000u) return 2;
+  k = (mbits == 0x7F800000u) ? 1024 : ceil_log2_lib(mbits, p.tab);
   kc = min(max(k + p.bias, 0), p.scale_max) - p.bias;
-  return true;
+  return (k > TR::kMaxPow2) ? 1 : 0;
 }
 
-__device__ __forceinline__ float quantize_mant(float x, int k, const MxintParams& p) {
-  float r = rintf(ldexpf(x, p.qshift - k));
-  return fminf(fmaxf(r, p.lo), p.hi);
+// one element: dequantized value (fp32, rounded to T by the store) and its integer code
+template <int DT>
+__device__ __forceinline__ float mxint_element(float x, int state, int k, int kc, const MxintParams& p, int& code) {
+  using TR = DTypeTraits<DT>;
+  code = 0;
+  if (state == 0) {
+    float r = rintf(ldexpf(x, p.qshift - k));
+    r = fminf(fmaxf(r, p.lo), p.hi);
+    code = (int)r;
+    return ldexpf(r, kc - p.qshift);
+  }
+  if (state == 2) return qnan();
+  // x / inf: +-0 for finite x, NaN otherwise; then (+-0 / 2^(b-1)) * 2^kc, NaN when 2^kc is inf in T
+  bool finite = (f2bits(x) & 0x7FFFFFFFu) < 0x7F800000u;
+  if (!finite || kc > TR::kMaxPow2) return qnan();
+  return bits2f(f2bits(x) & 0x80000000u);
 }
 
 // LPB lanes share one block (B = LPB * kVec) or one lane holds SUB blocks (B = kVec / SUB).
@@ -75,15 +90,15 @@ __global__ __launch_bounds__(kThreads) void mxint_qdq_vec_kernel(const uint4* __
       for (int j = 0; j < EPS; ++j) m = max(m, f2bits(x[s * EPS + j]) & 0x7FFFFFFFu);
       m = group_max_u32<LPB>(m);
       int k = 0, kc = 0;
-      bool ok = block_exponent<DT>(m, p, k, kc);
+      int state = block_exponent<DT>(m, p, k, kc);
 #pragma unroll
       for (int j = 0; j < EPS; ++j) {
-        float r = quantize_mant(x[s * EPS + j], k, p);
-        y[s * EPS + j] = ok ? ldexpf(r, kc - p.qshift) : qnan();
-        c[s * EPS + j] = ok ? (int8_t)(int)r : (int8_t)0;
+        int code;
+        y[s * EPS + j] = mxint_element<DT>(x[s * EPS + j], state, k, kc, p, code);
+        c[s * EPS + j] = (int8_t)code;
       }
       if (codes != nullptr && idx < n_vec) {
-        int sb = ok ? min(max(kc - p.qshift + 134, 0), 255) : 255;
+        int sb = (state == 0) ? min(max(kc - p.qshift + 134, 0), 255) : 255;
         if constexpr (LPB > 1) {
           if ((idx & (LPB - 1)) == 0) scales[idx / LPB] = (uint8_t)sb;
         } else {
@@ -124,13 +139,13 @@ __global__ __launch_bounds__(kThreads) void mxint_qdq_generic_kernel(const void*
   uint32_t m = 0;
   for (int j = 0; j < B; ++j) m = max(m, f2bits(TR::load1(in, off + j)) & 0x7FFFFFFFu);
   int k = 0, kc = 0;
-  bool ok = block_exponent<DT>(m, p, k, kc);
+  int state = block_exponent<DT>(m, p, k, kc);
   for (int j = 0; j < B; ++j) {
-    float r = quantize_mant(TR::load1(in, off + j), k, p);
-    TR::store1(out, off + j, ok ? ldexpf(r, kc - p.qshift) : qnan());
-    if (codes != nullptr) codes[off + j] = ok ? (int8_t)(int)r : (int8_t)0;
+    int code;
+    TR::store1(out, off + j, mxint_element<DT>(TR::load1(in, off + j), state, k, kc, p, code));
+    if (codes != nullptr) codes[off + j] = (int8_t)code;
   }
-  if (codes != nullptr) scales[blk] = (uint8_t)(ok ? min(max(kc - p.qshift + 134, 0), 255) : 255);
+  if (codes != nullptr) scales[blk] = (uint8_t)((state == 0) ? min(max(kc - p.qshift + 134, 0), 255) : 255);
 }
 
 template <int DT>

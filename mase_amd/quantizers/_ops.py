@@ -119,7 +119,8 @@ def _infer_block_shape(x_shape: List[int], block_shape: List[int]) -> List[int]:
 
 
 def block_fp_geometry(shape: Sequence[int], block_size, skip_first_dim: bool):
-    """(batch, rows, cols, tile_rows, tile_cols) the reference's ``block`` dispatch (utils.py:569-592) implies."""
+    """(batch, rows, cols, tile_rows, tile_cols, folded) the reference's ``block`` dispatch (utils.py:569-592)
+    implies; ``folded`` tells whether the reference reassembles the result with ``F.fold``."""
     if isinstance(block_size, int):
         block_size = [block_size]
     block_size = list(block_size)
@@ -127,17 +128,17 @@ def block_fp_geometry(shape: Sequence[int], block_size, skip_first_dim: bool):
     if nd == 1:
         assert skip_first_dim is False, "skip_first_dim must be False for bias to be blocked"
         bs = _infer_block_shape([shape[0]], block_size)
-        return 1, 1, shape[0], 1, bs[0]
+        return 1, 1, shape[0], 1, bs[0], False
     if nd == 2:
         if skip_first_dim:
             bs = _infer_block_shape([1, shape[1]], block_size)
-            return 1, shape[0], shape[1], 1, bs[-1]
+            return 1, shape[0], shape[1], 1, bs[-1], False
         bs = _infer_block_shape([shape[0], shape[1]], block_size)
-        return 1, shape[0], shape[1], bs[0], bs[1]
+        return 1, shape[0], shape[1], bs[0], bs[1], True
     if nd == 3:
         if skip_first_dim:
             bs = _infer_block_shape([1, shape[1], shape[2]], block_size)
-            return shape[0], shape[1], shape[2], bs[1], bs[2]
+            return shape[0], shape[1], shape[2], bs[1], bs[2], True
         raise NotImplementedError("block 3d weight is not supported.")
     raise RuntimeError(f"Unsupported x.ndim = {nd}")
 
@@ -145,7 +146,7 @@ def block_fp_geometry(shape: Sequence[int], block_size, skip_first_dim: bool):
 def block_fp_qdq(x: Tensor, width: int, exponent_width: int, exponent_bias, block_size, skip_first_dim: bool) -> Tensor:
     _lib.require_device(x, "block_fp_quantizer")
     lib = _lib.load()
-    batch, rows, cols, b0, b1 = block_fp_geometry(tuple(x.shape), block_size, skip_first_dim)
+    batch, rows, cols, b0, b1, folded = block_fp_geometry(tuple(x.shape), block_size, skip_first_dim)
     if exponent_bias in (None, "none", "None"):
         exponent_bias = -1
     xin = _contig(x)
@@ -165,7 +166,7 @@ def block_fp_qdq(x: Tensor, width: int, exponent_width: int, exponent_bias, bloc
     tab = log2_table(x.dtype, x.device)
     rc = lib.mase_block_fp_qdq(
         xin.data_ptr(), out.data_ptr(), batch, rows, cols, b0, b1, dt, width, exponent_width, int(exponent_bias),
-        tab.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes, _lib.stream_ptr(x),
+        int(folded), tab.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes, _lib.stream_ptr(x),
     )
     _lib.check(rc, "mase_block_fp_qdq")
     return out

@@ -199,6 +199,8 @@ def test_block_fp_errors(Q, dev):
 def test_integer(Q, dev, width, frac, signed):
     rng = np.random.default_rng(width * 31 + (frac or 0))
     for dtype in DTYPES:
+        if dtype == torch.float16 and width > 16:
+            continue  # the clamp bound does not fit fp16: the reference raises there
         if dtype == torch.float32:
             x = fp32_from_bits(adversarial_fp32_bits(rng, 1 << 16))
             x = torch.where(torch.isfinite(x), x, torch.zeros_like(x))
