@@ -1,0 +1,242 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-inference hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+
+A "step" is one pass of the hot path over one batch of synthetic input that is already resident in HBM.
+Workloads (BASELINE.json configs):
+    bfp_qdq      config 2 (default): block-FP quantize-dequantize, bf16 [8,2048,4096], width 8, exp 8, block [1,16]
+    mxint_qdq    config 1: MXINT8 quantize-dequantize, fp32 [4096,4096], block 32
+    mxint_linear config 3: MXINT8 Linear forward, 4096x4096x4096, fp32 in/out
+    mxfp_linear  config 4: MXFP4(e2m1) weights x MXFP8(e4m3) activations Linear, M=8192 K=8192 N=28672
+Prints ONE JSON line.  `value` is algorithmic GB/s (Q-DQ) or TFLOP/s (Linear) over the whole timed region;
+`roofline` is for the dominant kernel, timed with HIP events on the launch stream; `cpu_baseline` is the CPU
+oracle timed on this box's host cores on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0}
+
+
+def make_bfp_input(torch, seed=1):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(8, 2048, 4096, generator=g, dtype=torch.float32)
+    idx = torch.randperm(4096, generator=g)[:4]  # 0.1 % of the channels carry outliers
+    x[..., idx] *= 50
+    return x.to(torch.bfloat16)
+
+
+def make_mxint_input(torch, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(4096, 4096, generator=g, dtype=torch.float32)
+
+
+class Workload:
+    name = ""
+    metric = ""
+    unit = ""
+    dtype = ""
+    bound = "hbm"
+    kernel = ""
+
+    def setup(self, torch, dev, n_buffers):
+        raise NotImplementedError
+
+    def step(self, i):
+        raise NotImplementedError
+
+    def work_per_step(self) -> float:
+        """algorithmic bytes (hbm) or flops (mfma) per step"""
+        raise NotImplementedError
+
+    def cpu_baseline(self, torch, budget_s):
+        return None
+
+
+class BfpQdq(Workload):
+    name = "bfp_qdq"
+    metric = "block-FP quantize-dequantize throughput (algorithmic bytes: 2 B read + 2 B written per element)"
+    unit = "GB/s"
+    dtype = "bf16"
+    kernel = "bfp_run_kernel"
+    config = {"workload": "block_fp_quantizer bf16 [8,2048,4096] width=8 exponent_width=8 block=[1,16], "
+                          "N(0,1) with 4 of 4096 channels x50, seed 1"}
+    kw = dict(width=8, exponent_width=8, exponent_bias=None, block_size=[1, 16], skip_first_dim=True)
+
+    def setup(self, torch, dev, n_buffers):
+        import mase_amd.quantizers as Q
+
+        self.Q = Q
+        self.host = make_bfp_input(torch)
+        # distinct buffers so that the 256 MB last-level cache cannot serve the reads of the next step
+        self.bufs = [self.host.to(dev) if i == 0 else None for i in range(n_buffers)]
+        for i in range(1, n_buffers):
+            self.bufs[i] = self.bufs[0].roll(i, dims=1).contiguous()
+        self.out = None
+
+    def step(self, i):
+        self.out = self.Q.block_fp_quantizer(self.bufs[i % len(self.bufs)], **self.kw)
+
+    def work_per_step(self):
+        return float(self.host.numel() * 4)
+
+    def cpu_baseline(self, torch, budget_s):
+        import oracle as O
+
+        x = self.host
+        O.block_fp_quantizer(x[:1].clone(), **self.kw)  # warm
+        t0 = time.perf_counter()
+        n = 0
+        while True:
+            O.block_fp_quantizer(x.clone(), **self.kw)
+            n += 1
+            if time.perf_counter() - t0 > budget_s or n >= 20:
+                break
+        dt = (time.perf_counter() - t0) / n
+        return {"value": self.work_per_step() / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                "kind": "port", "sample": f"{n} full passes of the same [8,2048,4096] bf16 tensor, {dt*1e3:.0f} ms each"}
+
+
+class MxintQdq(Workload):
+    name = "mxint_qdq"
+    metric = "MXINT8 quantize-dequantize throughput (algorithmic bytes: 4 B read + 4 B written per element)"
+    unit = "GB/s"
+    dtype = "f32"
+    kernel = "mxint_qdq_vec_kernel"
+    config = {"workload": "mxint_quantizer fp32 [4096,4096] block_size=32 element_bits=8 scale_bits=8, N(0,1) seed 0"}
+
+    def setup(self, torch, dev, n_buffers):
+        import mase_amd.quantizers as Q
+
+        self.Q = Q
+        self.host = make_mxint_input(torch)
+        n_buffers = max(n_buffers, 8)  # 64 MB each: rotate over more of them
+        self.bufs = [self.host.to(dev).roll(i, dims=0).contiguous() for i in range(n_buffers)]
+
+    def step(self, i):
+        self.out = self.Q.mxint_quantizer(self.bufs[i % len(self.bufs)], 32, 8)
+
+    def work_per_step(self):
+        return float(self.host.numel() * 8)
+
+    def cpu_baseline(self, torch, budget_s):
+        import oracle as O
+
+        x = self.host
+        O.mxint_quantizer(x[:64], 32, 8)
+        t0 = time.perf_counter()
+        n = 0
+        while True:
+            O.mxint_quantizer(x, 32, 8)
+            n += 1
+            if time.perf_counter() - t0 > budget_s or n >= 20:
+                break
+        dt = (time.perf_counter() - t0) / n
+        return {"value": self.work_per_step() / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                "kind": "port", "sample": f"{n} full passes of the same [4096,4096] fp32 tensor, {dt*1e3:.0f} ms each"}
+
+
+WORKLOADS = {w.name: w for w in (BfpQdq, MxintQdq)}
+
+
+def load_traffic(name):
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE), if a summary is committed."""
+    path = os.path.join(ROOT, "profiles", f"traffic_{name}.json")
+    if os.path.exists(path):
+        with open(path) as f:
+            return json.load(f).get("traffic_bytes_per_launch")
+    return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="bfp_qdq", choices=sorted(WORKLOADS))
+    ap.add_argument("--buffers", type=int, default=4)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build measures one GPU only (--gpus 1); multi-GPU sharding is a design note, not code",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no ROCm device visible", file=sys.stderr)
+        sys.exit(3)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = WORKLOADS[a.workload]()
+    w.setup(torch, dev, a.buffers)
+    for i in range(a.warmup):
+        w.step(i)
+    torch.cuda.synchronize()
+
+    # whole-job timing: wall clock bracketed by synchronisation
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        w.step(i)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    # kernel timing: HIP events on the launch stream (torch's current stream is the one passed to the C ABI)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
+    for i in range(a.steps):
+        evs[i][0].record()
+        w.step(i)
+        evs[i][1].record()
+    torch.cuda.synchronize()
+    k_ms = sorted(s.elapsed_time(e) for s, e in evs)
+    k_avg = sum(k_ms) / len(k_ms)
+
+    work = w.work_per_step()
+    scale = 1e9 if w.bound == "hbm" else 1e12
+    value = work * a.steps / wall / scale
+    achieved = work / (k_avg * 1e-3) / scale
+    peak = HBM_PEAK_GBS if w.bound == "hbm" else MFMA_PEAK_TFLOPS[getattr(w, "mfma_dtype", "bf16")]
+    out = {
+        "metric": w.metric,
+        "value": round(value, 2),
+        "unit": w.unit,
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": round(wall / a.steps * 1e3, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": w.dtype,
+        "data": "synthetic",
+        "config": w.config,
+        "roofline": {
+            "bound": w.bound,
+            "kernel": w.kernel,
+            "achieved": round(achieved, 2),
+            "peak": peak,
+            "unit": "GB/s" if w.bound == "hbm" else "TFLOP/s",
+            "frac": round(achieved / peak, 4),
+            "traffic": load_traffic(w.name),
+            "kernel_ms_avg": round(k_avg, 5),
+            "kernel_ms_median": round(k_ms[len(k_ms) // 2], 5),
+        },
+        "cpu_baseline": None if a.no_cpu else w.cpu_baseline(torch, a.cpu_seconds),
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

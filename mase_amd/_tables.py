@@ -56,7 +56,28 @@ def _thresholds(k: np.ndarray, M: np.ndarray, ceil_v: np.ndarray, floor_v: np.nd
             raise RuntimeError(f"{what}: floor(log2) corrections are not a suffix at exponent {kk}")
         if n_high:
             tab[_HALF + kk - _K_MIN] = m[len(m) - n_high]
+    _summarise(tab)
     return tab
+
+
+def _summarise(tab: np.ndarray) -> None:
+    """Words 277..279 of each half: the widest exponent interval around k=0 without corrections, and the
+    extreme threshold, so that kernels can skip the per-lane table read in the common case."""
+    n = _K_MAX - _K_MIN + 1
+    for half, neutral in ((0, 0), (_HALF, 0x800000)):
+        thr = tab[half:half + n]
+        clean = thr == neutral
+        lo = hi = 0 - _K_MIN  # biased index of k = 0
+        if not clean[lo]:
+            lo, hi = 1, 0  # empty interval
+        else:
+            while lo - 1 >= 0 and clean[lo - 1]:
+                lo -= 1
+            while hi + 1 < n and clean[hi + 1]:
+                hi += 1
+        tab[half + 277] = lo
+        tab[half + 278] = hi
+        tab[half + 279] = thr.max() if half == 0 else thr.min()
 
 
 def _measure_16bit(dtype: torch.dtype) -> np.ndarray:

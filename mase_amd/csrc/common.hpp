@@ -144,6 +144,36 @@ __device__ __forceinline__ uint32_t group_max_u32(uint32_t v) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// max |x| over the elements of one 16-byte vector, returned as fp32 bits (NaN compares largest).
+// 16-bit types are reduced two at a time with packed 16-bit integer max before widening.
+// ---------------------------------------------------------------------------------------------
+typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+  u16x2_t r = __builtin_elementwise_max(__builtin_bit_cast(u16x2_t, a), __builtin_bit_cast(u16x2_t, b));
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+template <int DT>
+__device__ __forceinline__ uint32_t vec_absmax_bits(const uint4& v) {
+  if constexpr (DT == MASE_DT_F32) {
+    return max(max(v.x & 0x7FFFFFFFu, v.y & 0x7FFFFFFFu), max(v.z & 0x7FFFFFFFu, v.w & 0x7FFFFFFFu));
+  } else {
+    uint32_t m = pk_max_u16(pk_max_u16(v.x & 0x7FFF7FFFu, v.y & 0x7FFF7FFFu),
+                            pk_max_u16(v.z & 0x7FFF7FFFu, v.w & 0x7FFF7FFFu));
+    m = max(m & 0xFFFFu, m >> 16);
+    if constexpr (DT == MASE_DT_BF16) return m << 16;
+    // fp16: widen (monotone); Inf/NaN patterns map to fp32 Inf/NaN
+    return f2bits(f16_bits_to_f32(m));
+  }
+}
+
+// two fp32 values that are exactly representable in bf16 -> one packed dword (no rounding step)
+__device__ __forceinline__ uint32_t pack_bf16_exact(float lo, float hi) {
+  return __builtin_amdgcn_perm(f2bits(hi), f2bits(lo), 0x07060302u);
+}
+
+// ---------------------------------------------------------------------------------------------
 // ceil(log2(v)) / floor(log2(v)) "as the host library evaluates them in the tensor dtype".
 //
 // v is a positive, finite, non-zero value of the tensor dtype, given as fp32 bits.  The exact integer
@@ -153,6 +183,22 @@ __device__ __forceinline__ uint32_t group_max_u32(uint32_t v) {
 //   tab[288 + k + 149]  smallest M for which floor(log2(2^k (1+M/2^23))) == k+1 (0x800000 when none)
 // ---------------------------------------------------------------------------------------------
 constexpr int kLog2TabHalf = 288;
+// Words 277..279 of each half summarise it so that the common case needs no per-lane table read:
+//   [277], [278]  k_lo+149, k_hi+149: exponents in [k_lo, k_hi] have no correction at all
+//   [279]         ceil half: largest threshold of any exponent; floor half: smallest threshold
+constexpr int kLog2MetaLo = 277, kLog2MetaHi = 278, kLog2MetaM = 279;
+
+struct Log2Meta {
+  int lo, hi;      // biased (k+149) exponent interval without corrections
+  uint32_t m;      // extreme threshold
+};
+__device__ __forceinline__ Log2Meta load_log2_meta(const uint32_t* __restrict__ tab, int half) {
+  Log2Meta r;
+  r.lo = (int)tab[half + kLog2MetaLo];
+  r.hi = (int)tab[half + kLog2MetaHi];
+  r.m = tab[half + kLog2MetaM];
+  return r;
+}
 
 __device__ __forceinline__ int split_pow2(uint32_t b, uint32_t& M) {
   int E = (int)(b >> 23);
@@ -171,11 +217,27 @@ __device__ __forceinline__ int ceil_log2_lib(uint32_t b, const uint32_t* __restr
   if (M == 0) return k;
   return (M <= tab[k + 149]) ? k : k + 1;
 }
+// same, reading the table only for mantissas/exponents that can be corrected at all
+__device__ __forceinline__ int ceil_log2_lib(uint32_t b, const uint32_t* __restrict__ tab, const Log2Meta& meta) {
+  uint32_t M;
+  int k = split_pow2(b, M);
+  if (M == 0) return k;
+  int kb = k + 149;
+  if (M > meta.m || (kb >= meta.lo && kb <= meta.hi)) return k + 1;
+  return (M <= tab[kb]) ? k : k + 1;
+}
 
 __device__ __forceinline__ int floor_log2_lib(uint32_t b, const uint32_t* __restrict__ tab) {
   uint32_t M;
   int k = split_pow2(b, M);
   return (M >= tab[kLog2TabHalf + k + 149]) ? k + 1 : k;
+}
+__device__ __forceinline__ int floor_log2_lib(uint32_t b, const uint32_t* __restrict__ tab, const Log2Meta& meta) {
+  uint32_t M;
+  int k = split_pow2(b, M);
+  int kb = k + 149;
+  if (M < meta.m || (kb >= meta.lo && kb <= meta.hi)) return k;
+  return (M >= tab[kLog2TabHalf + kb]) ? k + 1 : k;
 }
 
 // 2^e as fp32 for e in [-149, 127]; callers handle e > 127 themselves

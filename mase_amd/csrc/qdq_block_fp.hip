@@ -23,6 +23,10 @@
 //                 workspace, pass 2 quantizes; both are coalesced along the last dimension.
 #include "common.hpp"
 
+#ifndef MASE_RUN_THREADS
+#define MASE_RUN_THREADS 256
+#endif
+
 namespace mase {
 namespace {
 
@@ -35,16 +39,17 @@ struct BfpParams {
   const uint32_t* tab;
 };
 
-constexpr int kUnroll = 4;
+// work-group size of the single-pass kernel: small groups stream best on this part
+constexpr int kRunThreads = MASE_RUN_THREADS;
 
 // returns 0: zero tile, 1: regular (e valid), 2: NaN tile
-template <int DT>
-__device__ __forceinline__ int tile_exponent(uint32_t mbits, const BfpParams& p, int& e) {
+template <int DT, typename... Meta>
+__device__ __forceinline__ int tile_exponent(uint32_t mbits, const BfpParams& p, int& e, const Meta&... meta) {
   using TR = DTypeTraits<DT>;
   if (mbits == 0) return 0;
   if (mbits > 0x7F800000u) return 2;
   // an infinite maximum has log2 = inf, which the clamp brings down to e_hi
-  e = (mbits == 0x7F800000u) ? p.e_hi : min(max(ceil_log2_lib(mbits, p.tab), p.e_lo), p.e_hi);
+  e = (mbits == 0x7F800000u) ? p.e_hi : min(max(ceil_log2_lib(mbits, p.tab, meta...), p.e_lo), p.e_hi);
   return (e > TR::kMaxPow2) ? 2 : 1;
 }
 
@@ -62,37 +67,76 @@ __device__ __forceinline__ float bfp_element(float x, int state, int e, const Bf
   return bits2f(f2bits(y) | (xb & smask));
 }
 
-template <int DT, int LPB, int SUB>
-__global__ __launch_bounds__(kThreads) void bfp_run_kernel(const uint4* __restrict__ in, uint4* __restrict__ out,
-                                                           size_t n_vec, BfpParams p) {
+// One 16-byte vector per lane.  LPB lanes share a tile (tile_cols = LPB * kVec) or one lane holds SUB tiles.
+//
+// Fast path (taken per tile): in a regular tile the quantized value is computed on the signed input,
+//   q = med3(rne(x * 2^(mb-e)), -qmax, qmax),  y = q * 2^(e-mb)          [fp32: |x| + 1e-9 first, sign copied]
+// which equals the reference because
+//   * fp16: |x| + 1e-9 always rounds back to |x|;  bf16: it does for |x| >= 2^-21, and smaller elements
+//     quantize to 0 either way once e >= mb - 19 (tiles with a smaller exponent take the general path);
+//   * q has at most 8 significant bits for bf16 inputs, so y is a bf16 value and is packed by truncation;
+//   * rne() keeps the sign of zero, which is what zero_sign_mode 0 wants; mode 1 adds +0.0 (-0 -> +0).
+// Elements with isclose(x, 0) are selected afterwards: x + 0.0 (the value itself, -0 -> +0).
+template <int DT, int LPB, int SUB, int T>
+__global__ __launch_bounds__(T) void bfp_run_kernel(const uint4* __restrict__ in, uint4* __restrict__ out,
+                                                    size_t n_vec, BfpParams p) {
   using TR = DTypeTraits<DT>;
   constexpr int V = TR::kVec;
-  constexpr int EPS = V / SUB;
-  const size_t base = (size_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
-  uint4 raw[kUnroll];
+  const size_t idx = (size_t)blockIdx.x * T + threadIdx.x;
+  if (idx >= n_vec) return;  // whole tiles drop out together: n_vec is a multiple of LPB
+  const uint4 raw = load_nt(in + idx);
+  const Log2Meta meta = load_log2_meta(p.tab, 0);
+  float x[V], y[V];
+  TR::unpack(raw, x);
+  if constexpr (SUB == 1) {
+    uint32_t m = group_max_u32<LPB>(vec_absmax_bits<DT>(raw));
+    int e = 0;
+    const int state = tile_exponent<DT>(m, p, e, meta);
+    const bool fast = (state == 1) && (DT != MASE_DT_BF16 || e >= p.mb - 19);
+    if (fast) {
+      const float thr = bits2f(p.close_thr);
+      const int up = p.mb - e, dn = e - p.mb;
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    size_t idx = base + (size_t)u * kThreads;
-    raw[u] = (idx < n_vec) ? load_nt(in + idx) : make_uint4(0, 0, 0, 0);
-  }
+      for (int j = 0; j < V; ++j) {
+        float r;
+        if constexpr (DT == MASE_DT_F32) {
+          float q = fminf(rintf(ldexpf(fabsf(x[j]) + 1e-9f, up)), p.qmax);
+          r = bits2f(f2bits(ldexpf(q, dn)) | (f2bits(x[j]) & 0x80000000u));
+        } else {
+          float q = fminf(fmaxf(rintf(ldexpf(x[j], up)), -p.qmax), p.qmax);
+          r = ldexpf(q, dn);
+        }
+        if (p.zero_sign_mask == 0u) r = r + 0.0f;
+        y[j] = (fabsf(x[j]) <= thr) ? (x[j] + 0.0f) : r;
+      }
+      if constexpr (DT == MASE_DT_BF16) {
+        uint4 o;
+        o.x = pack_bf16_exact(y[0], y[1]);
+        o.y = pack_bf16_exact(y[2], y[3]);
+        o.z = pack_bf16_exact(y[4], y[5]);
+        o.w = pack_bf16_exact(y[6], y[7]);
+        store_nt(out + idx, o);
+      } else {
+        store_nt(out + idx, TR::pack(y));
+      }
+      return;
+    }
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    size_t idx = base + (size_t)u * kThreads;
-    float x[V], y[V];
-    TR::unpack(raw[u], x);
+    for (int j = 0; j < V; ++j) y[j] = bfp_element<DT>(x[j], state, e, p);
+  } else {
+    constexpr int EPS = V / SUB;
 #pragma unroll
     for (int s = 0; s < SUB; ++s) {
       uint32_t m = 0;
 #pragma unroll
       for (int j = 0; j < EPS; ++j) m = max(m, f2bits(x[s * EPS + j]) & 0x7FFFFFFFu);
-      m = group_max_u32<LPB>(m);
       int e = 0;
-      int state = tile_exponent<DT>(m, p, e);
+      const int state = tile_exponent<DT>(m, p, e);
 #pragma unroll
       for (int j = 0; j < EPS; ++j) y[s * EPS + j] = bfp_element<DT>(x[s * EPS + j], state, e, p);
     }
-    if (idx < n_vec) store_nt(out + idx, TR::pack(y));
   }
+  store_nt(out + idx, TR::pack(y));
 }
 
 __global__ __launch_bounds__(kThreads) void fill_u32_kernel(uint32_t* __restrict__ p, size_t n, uint32_t v) {
@@ -164,9 +208,10 @@ int launch_bfp(const void* in, void* out, size_t batch, size_t rows, size_t cols
   size_t numel = batch * rows * cols;
   if (run_path_ok(in, out, numel, cols, b0, b1, V)) {
     size_t n_vec = numel / V;
-    dim3 grid(blocks_for(n_vec, (size_t)kThreads * kUnroll)), block(kThreads);
-#define MASE_BFP_CASE(LPB_, SUB_) \
-  hipLaunchKernelGGL((bfp_run_kernel<DT, LPB_, SUB_>), grid, block, 0, st, (const uint4*)in, (uint4*)out, n_vec, p)
+    dim3 grid(blocks_for(n_vec, kRunThreads)), block(kRunThreads);
+#define MASE_BFP_CASE(LPB_, SUB_)                                                                              \
+  hipLaunchKernelGGL((bfp_run_kernel<DT, LPB_, SUB_, kRunThreads>), grid, block, 0, st, (const uint4*)in, (uint4*)out, \
+                     n_vec, p)
     if (b1 >= V) {
       switch (b1 / V) {
         case 1: MASE_BFP_CASE(1, 1); break;

@@ -24,10 +24,11 @@ struct MxfpParams {
 constexpr int kUnroll = 2;
 
 // state 0: all flushed, 1: regular (sh valid), 2: NaN block
-__device__ __forceinline__ int mxfp_block_scale(uint32_t mbits, const MxfpParams& p, int& sh) {
+template <typename... Meta>
+__device__ __forceinline__ int mxfp_block_scale(uint32_t mbits, const MxfpParams& p, int& sh, const Meta&... meta) {
   if (mbits == 0) return 0;
   if (mbits >= 0x7F800000u) return 2;
-  sh = min(max(floor_log2_lib(mbits, p.tab) - p.el_emax, -127), 128);
+  sh = min(max(floor_log2_lib(mbits, p.tab, meta...) - p.el_emax, -127), 128);
   return 1;
 }
 
@@ -54,6 +55,7 @@ __global__ __launch_bounds__(kThreads) void mxfp_qdq_vec_kernel(const void* __re
   constexpr int V = (TI::kVec == 8 || TO::kVec == 8) ? 8 : 4;
   constexpr int EPS = V / SUB;
   const size_t base = (size_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+  const Log2Meta meta = load_log2_meta(p.tab, kLog2TabHalf);
 #pragma unroll
   for (int u = 0; u < kUnroll; ++u) {
     size_t idx = base + (size_t)u * kThreads;
@@ -80,7 +82,7 @@ __global__ __launch_bounds__(kThreads) void mxfp_qdq_vec_kernel(const void* __re
       for (int j = 0; j < EPS; ++j) m = max(m, f2bits(x[s * EPS + j]) & 0x7FFFFFFFu);
       m = group_max_u32<LPB>(m);
       int sh = 0;
-      int state = mxfp_block_scale(m, p, sh);
+      int state = mxfp_block_scale(m, p, sh, meta);
 #pragma unroll
       for (int j = 0; j < EPS; ++j) y[s * EPS + j] = mxfp_element(x[s * EPS + j], state, sh, p, c[s * EPS + j]);
       if (codes != nullptr && live) {

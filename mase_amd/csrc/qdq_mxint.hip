@@ -12,9 +12,13 @@
 // computes x/inf = +-0 and then +-0 * 2^kc, which is NaN when 2^kc is inf as well and +-0 otherwise; a NaN
 // maximum makes the whole block NaN.  The same cases are reproduced here.
 //
-// Bandwidth-bound: one 16-byte load and one 16-byte store per lane per vector, kUnroll independent loads
-// in flight per lane, block maximum by DPP inside the wavefront, no LDS.
+// Bandwidth-bound: one 16-byte load and one 16-byte store per lane, latency hidden by occupancy (few
+// registers, many small work-groups), block maximum by DPP inside the wavefront, no LDS.
 #include "common.hpp"
+
+#ifndef MASE_RUN_THREADS
+#define MASE_RUN_THREADS 256
+#endif
 
 namespace mase {
 namespace {
@@ -27,16 +31,18 @@ struct MxintParams {
   const uint32_t* tab;
 };
 
-constexpr int kUnroll = 4;
+// work-group size of the vector kernel: small groups stream best on this part
+constexpr int kRunThreads = MASE_RUN_THREADS;
 
 // state 0: regular block (k, kc valid); 1: 2^k overflows T (also an infinite maximum): x/2^k is +-0;
 // 2: the maximum is NaN.
-template <int DT>
-__device__ __forceinline__ int block_exponent(uint32_t mbits, const MxintParams& p, int& k, int& kc) {
+template <int DT, typename... Meta>
+__device__ __forceinline__ int block_exponent(uint32_t mbits, const MxintParams& p, int& k, int& kc,
+                                              const Meta&... meta) {
   using TR = DTypeTraits<DT>;
   mbits = max(mbits, TR::kTinyBits);
   if (mbits > 0x7F800000u) return 2;
-  k = (mbits == 0x7F800000u) ? 1024 : ceil_log2_lib(mbits, p.tab);
+  k = (mbits == 0x7F800000u) ? 1024 : ceil_log2_lib(mbits, p.tab, meta...);
   kc = min(max(k + p.bias, 0), p.scale_max) - p.bias;
   return (k > TR::kMaxPow2) ? 1 : 0;
 }
@@ -59,69 +65,83 @@ __device__ __forceinline__ float mxint_element(float x, int state, int k, int kc
   return bits2f(f2bits(x) & 0x80000000u);
 }
 
-// LPB lanes share one block (B = LPB * kVec) or one lane holds SUB blocks (B = kVec / SUB).
-template <int DT, int LPB, int SUB>
-__global__ __launch_bounds__(kThreads) void mxint_qdq_vec_kernel(const uint4* __restrict__ in, uint4* __restrict__ out,
-                                                                 int8_t* __restrict__ codes,
-                                                                 uint8_t* __restrict__ scales, size_t n_vec,
-                                                                 MxintParams p) {
+// One 16-byte vector per lane.  LPB lanes share one block (B = LPB * kVec) or one lane holds SUB blocks
+// (B = kVec / SUB).  For bf16 the dequantized value m * 2^(kc-b+1) has at most 8 significant bits (m is the
+// rne of an 8-bit-significand input), so it is packed by truncation unless it would be subnormal.
+template <int DT, int LPB, int SUB, int T>
+__global__ __launch_bounds__(T) void mxint_qdq_vec_kernel(const uint4* __restrict__ in, uint4* __restrict__ out,
+                                                          int8_t* __restrict__ codes, uint8_t* __restrict__ scales,
+                                                          size_t n_vec, MxintParams p) {
   using TR = DTypeTraits<DT>;
   constexpr int V = TR::kVec;
   constexpr int EPS = V / SUB;  // elements per sub-block held by this lane
-  const size_t base = (size_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
-
-  uint4 raw[kUnroll];
+  const size_t idx = (size_t)blockIdx.x * T + threadIdx.x;
+  if (idx >= n_vec) return;  // whole blocks drop out together: n_vec is a multiple of LPB
+  const uint4 raw = load_nt(in + idx);
+  const Log2Meta meta = load_log2_meta(p.tab, 0);
+  float x[V], y[V];
+  int c[V];
+  TR::unpack(raw, x);
+  bool exact_bf16 = (DT == MASE_DT_BF16);
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    size_t idx = base + (size_t)u * kThreads;
-    raw[u] = (idx < n_vec) ? load_nt(in + idx) : make_uint4(0, 0, 0, 0);
-  }
-#pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    size_t idx = base + (size_t)u * kThreads;
-    float x[V];
-    TR::unpack(raw[u], x);
-    float y[V];
-    int8_t c[V];
-#pragma unroll
-    for (int s = 0; s < SUB; ++s) {
-      uint32_t m = 0;
+  for (int s = 0; s < SUB; ++s) {
+    uint32_t m;
+    if constexpr (SUB == 1) {
+      m = group_max_u32<LPB>(vec_absmax_bits<DT>(raw));
+    } else {
+      m = 0;
 #pragma unroll
       for (int j = 0; j < EPS; ++j) m = max(m, f2bits(x[s * EPS + j]) & 0x7FFFFFFFu);
-      m = group_max_u32<LPB>(m);
-      int k = 0, kc = 0;
-      int state = block_exponent<DT>(m, p, k, kc);
+    }
+    int k = 0, kc = 0;
+    const int state = block_exponent<DT>(m, p, k, kc, meta);
+    if (state == 0) {
+      const int up = p.qshift - k, dn = kc - p.qshift;
+      exact_bf16 = exact_bf16 && (dn >= -126);
 #pragma unroll
       for (int j = 0; j < EPS; ++j) {
-        int code;
-        y[s * EPS + j] = mxint_element<DT>(x[s * EPS + j], state, k, kc, p, code);
-        c[s * EPS + j] = (int8_t)code;
+        float r = fminf(fmaxf(rintf(ldexpf(x[s * EPS + j], up)), p.lo), p.hi);
+        c[s * EPS + j] = (int)r;
+        y[s * EPS + j] = ldexpf(r, dn);
       }
-      if (codes != nullptr && idx < n_vec) {
-        int sb = (state == 0) ? min(max(kc - p.qshift + 134, 0), 255) : 255;
-        if constexpr (LPB > 1) {
-          if ((idx & (LPB - 1)) == 0) scales[idx / LPB] = (uint8_t)sb;
-        } else {
-          scales[idx * SUB + s] = (uint8_t)sb;
-        }
+    } else {
+#pragma unroll
+      for (int j = 0; j < EPS; ++j) y[s * EPS + j] = mxint_element<DT>(x[s * EPS + j], state, k, kc, p, c[s * EPS + j]);
+    }
+    if (codes != nullptr) {
+      int sb = (state == 0) ? min(max(kc - p.qshift + 134, 0), 255) : 255;
+      if constexpr (LPB > 1) {
+        if ((idx & (LPB - 1)) == 0) scales[idx / LPB] = (uint8_t)sb;
+      } else {
+        scales[idx * SUB + s] = (uint8_t)sb;
       }
     }
-    if (idx < n_vec) {
+  }
+  if constexpr (DT == MASE_DT_BF16) {
+    if (exact_bf16) {
+      uint4 o;
+      o.x = pack_bf16_exact(y[0], y[1]);
+      o.y = pack_bf16_exact(y[2], y[3]);
+      o.z = pack_bf16_exact(y[4], y[5]);
+      o.w = pack_bf16_exact(y[6], y[7]);
+      store_nt(out + idx, o);
+    } else {
       store_nt(out + idx, TR::pack(y));
-      if (codes != nullptr) {
-        if constexpr (V == 4) {
-          uint32_t w = (uint32_t)(uint8_t)c[0] | ((uint32_t)(uint8_t)c[1] << 8) | ((uint32_t)(uint8_t)c[2] << 16) |
-                       ((uint32_t)(uint8_t)c[3] << 24);
-          ((uint32_t*)codes)[idx] = w;
-        } else {
-          uint2 w;
-          w.x = (uint32_t)(uint8_t)c[0] | ((uint32_t)(uint8_t)c[1] << 8) | ((uint32_t)(uint8_t)c[2] << 16) |
-                ((uint32_t)(uint8_t)c[3] << 24);
-          w.y = (uint32_t)(uint8_t)c[4] | ((uint32_t)(uint8_t)c[5] << 8) | ((uint32_t)(uint8_t)c[6] << 16) |
-                ((uint32_t)(uint8_t)c[7] << 24);
-          ((uint2*)codes)[idx] = w;
-        }
-      }
+    }
+  } else {
+    store_nt(out + idx, TR::pack(y));
+  }
+  if (codes != nullptr) {
+    if constexpr (V == 4) {
+      ((uint32_t*)codes)[idx] = (uint32_t)(c[0] & 0xFF) | ((uint32_t)(c[1] & 0xFF) << 8) | ((uint32_t)(c[2] & 0xFF) << 16) |
+                                ((uint32_t)(c[3] & 0xFF) << 24);
+    } else {
+      uint2 w;
+      w.x = (uint32_t)(c[0] & 0xFF) | ((uint32_t)(c[1] & 0xFF) << 8) | ((uint32_t)(c[2] & 0xFF) << 16) |
+            ((uint32_t)(c[3] & 0xFF) << 24);
+      w.y = (uint32_t)(c[4] & 0xFF) | ((uint32_t)(c[5] & 0xFF) << 8) | ((uint32_t)(c[6] & 0xFF) << 16) |
+            ((uint32_t)(c[7] & 0xFF) << 24);
+      ((uint2*)codes)[idx] = w;
     }
   }
 }
@@ -158,10 +178,10 @@ int launch_mxint(const void* in, void* out, int8_t* codes, uint8_t* scales, size
                       (codes == nullptr || (((uintptr_t)codes) & 7u) == 0);
   if (vec_ok) {
     size_t n_vec = numel / V;
-    dim3 grid(blocks_for(n_vec, (size_t)kThreads * kUnroll)), block(kThreads);
-#define MASE_MXINT_CASE(LPB_, SUB_)                                                                          \
-  hipLaunchKernelGGL((mxint_qdq_vec_kernel<DT, LPB_, SUB_>), grid, block, 0, st, (const uint4*)in, (uint4*)out, \
-                     codes, scales, n_vec, p)
+    dim3 grid(blocks_for(n_vec, kRunThreads)), block(kRunThreads);
+#define MASE_MXINT_CASE(LPB_, SUB_)                                                                               \
+  hipLaunchKernelGGL((mxint_qdq_vec_kernel<DT, LPB_, SUB_, kRunThreads>), grid, block, 0, st, (const uint4*)in, \
+                     (uint4*)out, codes, scales, n_vec, p)
     if (B >= V) {
       switch (B / V) {
         case 1: MASE_MXINT_CASE(1, 1); break;
