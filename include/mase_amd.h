@@ -17,9 +17,8 @@
  *   mase_minifloat_qdq      nn/quantizers/minifloat.py:90-117, :200-225 (minifloat_denorm/ieee_quantizer)
  *   mase_minifloat_mx_qdq   nn/quantizers/_minifloat_mx/minifloat.py:12-33 (minifloat_quantizer_sim)
  *   mase_mxfp_qdq           nn/quantizers/mxfp/mxfp.py:187-230    (mxfp_quantizer, non-search branch)
- *   mase_mx_linear_bf16     nn/quantized/modules/linear.py:956-972 (LinearMXInt.forward: F.linear on the
- *                           quantize-dequantized operands) and :877-895 (LinearMXFP.forward)
- *   mase_mxfp_linear_scaled nn/quantized/modules/linear.py:877-895 (LinearMXFP.forward, native scaled MFMA)
+ *   mase_gemm_bf16_tn       nn/quantized/modules/linear.py:972 and :895 (the F.linear of LinearMXInt.forward /
+ *                           LinearMXFP.forward on the quantize-dequantized operands)
  */
 #ifndef MASE_AMD_H
 #define MASE_AMD_H
@@ -103,6 +102,13 @@ int mase_minifloat_mx_qdq(const void* in, void* out, size_t numel, int in_dtype,
 int mase_mxfp_qdq(const void* in, void* out, uint8_t* codes, uint8_t* scales, size_t numel, int in_dtype,
                   int out_dtype, int block_size, int exp_bits, int frac_bits, const uint32_t* log2_tab,
                   void* stream);
+
+/* C[M,N] = A[M,K] * B[N,K]^T (+ bias[N]): bf16 operands (both K-major, 16-byte aligned, K % 8 == 0), fp32
+ * accumulation on the matrix cores, C written in out_dtype.  bias may be NULL; bias_dtype is its MASE_DT_*.
+ * This is the contraction of LinearMXInt.forward / LinearMXFP.forward (nn/quantized/modules/linear.py:972,
+ * :895) on operands whose MX values are held exactly in bf16. */
+int mase_gemm_bf16_tn(const void* A, const void* B, const void* bias, void* C, size_t M, size_t N, size_t K,
+                      int out_dtype, int bias_dtype, void* stream);
 
 /* test/diagnostic helpers (host only, no device work) */
 uint32_t mase_isclose_zero_threshold_bits(int dtype); /* largest |x| (fp32 bits) that isclose(x, 0) accepts */

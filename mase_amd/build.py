@@ -34,6 +34,10 @@ COMMON_FLAGS = [
 ]
 
 
+# extra compiler flags for experiments, e.g. MASE_EXTRA_HIPCC_FLAGS="-DMASE_RUN_THREADS=64"
+COMMON_FLAGS += os.environ.get("MASE_EXTRA_HIPCC_FLAGS", "").split()
+
+
 def sources() -> list[str]:
     return sorted(os.path.join(SRC_DIR, f) for f in os.listdir(SRC_DIR) if f.endswith(".hip"))
 

@@ -17,7 +17,7 @@
 #include "common.hpp"
 
 #ifndef MASE_RUN_THREADS
-#define MASE_RUN_THREADS 256
+#define MASE_RUN_THREADS 64
 #endif
 
 namespace mase {

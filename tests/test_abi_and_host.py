@@ -1,0 +1,156 @@
+"""CPU-side checks of the C-ABI library and of the host logic (no GPU, no kernel launches)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from mase_amd import _lib
+
+    if not os.path.exists(_lib.LIB_PATH):
+        import __graft_entry__ as g
+
+        g.build()
+    return _lib.load()
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "mase_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mase_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(lib):
+    from mase_amd import _lib
+
+    names = declared_symbols()
+    assert len(names) >= 10
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/mase_amd.h but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature in mase_amd/_lib.py"
+    assert sorted(_lib.SIGNATURES) == names
+    assert lib.mase_abi_version() >= 1
+    assert lib.mase_error_string(0) == b"ok" and b"NULL" in lib.mase_error_string(-1)
+
+
+def test_entry_points_reject_bad_arguments_without_a_gpu(lib):
+    """argument validation happens before any HIP call, so it can be exercised on the CPU"""
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    assert lib.mase_mxint_qdq(None, p, None, None, 64, 0, 32, 8, 8, p, None) == -1
+    assert lib.mase_mxint_qdq(p, p, None, None, 65, 0, 32, 8, 8, p, None) == -2
+    assert lib.mase_mxint_qdq(p, p, None, None, 64, 7, 32, 8, 8, p, None) == -4
+    assert lib.mase_mxint_qdq(p, p, None, None, 64, 0, 32, 1, 8, p, None) == -5
+    assert lib.mase_mxint_qdq(p, p, p, None, 64, 0, 32, 8, 8, p, None) == -1
+    assert lib.mase_mxint_qdq(p, p, None, None, 0, 0, 32, 8, 8, p, None) == 0  # empty input is a no-op
+    assert lib.mase_mxfp_qdq(p, p, None, None, 64, 0, 0, 32, 3, 3, p, None) == -5  # illegal element format
+    assert lib.mase_mxfp_qdq(p, p, None, None, 63, 0, 0, 32, 4, 3, p, None) == -2
+    assert lib.mase_block_fp_qdq(p, p, 1, 4, 16, 0, 16, 0, 8, 8, -1, 0, p, None, 0, None) == -2
+    assert lib.mase_block_fp_qdq(p, p, 1, 4, 16, 2, 16, 0, 8, 8, -1, 1, p, None, 0, None) == -7  # needs a workspace
+    assert lib.mase_block_fp_qdq(p, p, 1, 4, 16, 1, 16, 2, 8, 2, 60, 0, p, None, 0, None) == -5  # 2^e underflows fp16
+    assert lib.mase_integer_qdq(p, p, 16, 0, 40, 4, 1, 0, None) == -5
+    assert lib.mase_minifloat_qdq(p, p, 16, 0, 8, 9, -1, 0, p, None) == -5
+    assert lib.mase_minifloat_mx_qdq(p, p, 16, 0, 0, 4, 3, 1, 7, None) == -5
+    assert lib.mase_block_fp_workspace_bytes(2, 5, 40, 2, 16, 1) == 2 * 3 * 3 * 4
+
+
+@pytest.mark.parametrize("dtype,code", [(torch.float32, 0), (torch.bfloat16, 1), (torch.float16, 2)])
+def test_host_scalar_conversions_match_torch(lib, dtype, code):
+    for v in (127, 255, 2047, 4095, 32767, 65535, -128, -2048, 1e-8, 3.3):
+        want = torch.tensor(float(v)).to(dtype).float().item()
+        assert lib.mase_round_scalar_to_dtype(float(v), code) == want
+    # clamp really does cast its bounds to the tensor dtype
+    if dtype != torch.float32:
+        assert torch.tensor([5000.0], dtype=dtype).clamp(0, 2047).float().item() == lib.mase_round_scalar_to_dtype(2047.0, code)
+    # isclose(x, 0) threshold
+    thr = np.array([lib.mase_isclose_zero_threshold_bits(code)], dtype=np.uint32).view(np.float32)[0]
+    zero = torch.tensor([0.0], dtype=dtype)
+    t = torch.tensor([thr], dtype=torch.float32).to(dtype)
+    assert t.float().item() == thr
+    assert bool(torch.isclose(t, zero)) or thr == 0.0
+    bigger = (t.view(torch.int16 if dtype != torch.float32 else torch.int32) + 1).view(dtype)
+    assert not bool(torch.isclose(bigger, zero))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_log2_tables_reproduce_the_library(dtype):
+    """the kernels' table lookup, replayed in numpy, equals torch.log2().ceil()/.floor() on the host"""
+    from mase_amd._tables import log2_table_cpu
+
+    tab = log2_table_cpu(dtype).astype(np.int64)
+    if dtype == torch.float32:
+        rng = np.random.default_rng(0)
+        bits = np.concatenate([rng.integers(1, 0x7F800000, size=400000), 
+                               (np.arange(1, 255)[:, None] << 23 | np.arange(0, 300)[None, :]).reshape(-1),
+                               (np.arange(1, 255)[:, None] << 23 | (0x7FFFFF - np.arange(0, 300)[None, :])).reshape(-1),
+                               np.arange(1, 5000)]).astype(np.uint32)
+        v = torch.from_numpy(bits.view(np.int32).copy()).view(torch.float32)
+    else:
+        top = 0x7F80 if dtype == torch.bfloat16 else 0x7C00
+        v = torch.arange(1, top, dtype=torch.int32).to(torch.int16).view(dtype)
+    lg = v.log2()
+    want_c = lg.ceil().float().numpy().astype(np.int64)
+    want_f = lg.floor().float().numpy().astype(np.int64)
+    mant, exp = np.frexp(v.double().numpy())
+    k = exp.astype(np.int64) - 1
+    M = np.rint((mant * 2 - 1) * (1 << 23)).astype(np.int64)
+    got_c = np.where(M == 0, k, np.where(M <= tab[k + 149], k, k + 1))
+    got_f = np.where(M >= tab[288 + k + 149], k + 1, k)
+    assert np.array_equal(got_c, want_c) and np.array_equal(got_f, want_f)
+    # summary words: inside [lo, hi] no correction exists; the extreme thresholds bound every entry
+    lo, hi, mx = tab[277], tab[278], tab[279]
+    assert np.all(tab[lo:hi + 1] == 0) and tab[:277].max() == mx
+    lo, hi, mn = tab[288 + 277], tab[288 + 278], tab[288 + 279]
+    assert np.all(tab[288 + lo:288 + hi + 1] == 0x800000) and tab[288:288 + 277].min() == mn
+
+
+def test_block_fp_geometry_follows_the_reference_dispatch():
+    from mase_amd.quantizers._ops import block_fp_geometry as g
+
+    assert g((8, 2048, 4096), [1, 16], True) == (8, 2048, 4096, 1, 16, True)
+    assert g((8, 2048, 4096), [16], True) == (8, 2048, 4096, 2048, 16, True)   # -1 prepended: whole token dim
+    assert g((64, 128), [16], True) == (1, 64, 128, 1, 16, False)
+    assert g((64, 128), [16], False) == (1, 64, 128, 64, 16, True)
+    assert g((64, 128), [4, 256], False) == (1, 64, 128, 4, 128, True)            # oversize -> full dim
+    assert g((100,), [16], False) == (1, 1, 100, 1, 16, False)
+    assert g((100,), 16, False) == (1, 1, 100, 1, 16, False)
+    assert g((10,), [2, 3, 16], False) == (1, 1, 10, 1, 10, False)
+    with pytest.raises(AssertionError):
+        g((100,), [16], True)
+    with pytest.raises(NotImplementedError):
+        g((2, 3, 4), [16], False)
+    with pytest.raises(RuntimeError):
+        g((2, 3, 4, 5), [16], True)
+
+
+def test_product_has_no_cpu_path():
+    import mase_amd.quantizers as Q
+    from mase_amd._lib import MaseAmdError
+
+    x = torch.randn(4, 32)
+    for call in (lambda: Q.mxint_quantizer(x, 32, 8), lambda: Q.mxfp_quantizer(x, 32, 4, 3),
+                 lambda: Q.block_fp_quantizer(x, 8, 8, None, [16]), lambda: Q.integer_quantizer(x, 8, 4),
+                 lambda: Q.minifloat_denorm_quantizer(x, 8, 4), lambda: Q.minifloat_ieee_quantizer(x, 8, 4)):
+        with pytest.raises(MaseAmdError):
+            call()
+    with pytest.raises(NotImplementedError):
+        Q.mxint_quantizer(x, 32, 8, quantile_search=True)
+
+
+def test_product_does_not_import_the_oracle():
+    import subprocess
+    import sys
+
+    code = "import sys; import mase_amd.quantizers, mase_amd.quantized, mase_amd.passes; assert not any(m == 'oracle' or m.startswith('oracle.') for m in sys.modules), 'oracle imported'"
+    subprocess.run([sys.executable, "-c", code], check=True, cwd=ROOT)
+    for dirpath, _, files in os.walk(os.path.join(ROOT, "mase_amd")):
+        for f in files:
+            if f.endswith(".py"):
+                assert not re.search(r"^\s*(from|import)\s+oracle\b", open(os.path.join(dirpath, f)).read(), flags=re.M), f

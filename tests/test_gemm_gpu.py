@@ -1,0 +1,54 @@
+"""GPU parity of the bf16 matrix-core contraction against an fp32 reference of the same operands."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_err(y, ref):
+    """max |y - ref| / max |ref|: the error measure used for every Linear comparison in this repo"""
+    return float((y.double() - ref.double()).abs().max() / ref.double().abs().max())
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (256, 256, 32), (512, 768, 128), (300, 200, 96), (1, 256, 64), (257, 513, 32),
+                                   (1024, 1024, 1024), (4096, 4096, 4096), (130, 11008, 4096)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_gemm_bf16_tn(dev, M, N, K, out_dtype):
+    from mase_amd._gemm import gemm_bf16_tn
+
+    g = torch.Generator().manual_seed(M * 7 + N * 3 + K)
+    a = torch.randn(M, K, generator=g).bfloat16()
+    b = (torch.randn(N, K, generator=g) * 0.05).bfloat16()
+    bias = torch.randn(N, generator=g)
+    print(f"gemm case M={M} N={N} K={K} out={out_dtype}", flush=True)
+    ad, bd = a.to(dev), b.to(dev)
+    ref = (ad.float() @ bd.float().t()).double().cpu() if M * N * K > 2 ** 28 else a.double() @ b.double().t()
+    y = gemm_bf16_tn(ad, bd, None, out_dtype)
+    tol = 2e-6 if out_dtype == torch.float32 else 4e-3  # fp32: summation order only; bf16: output rounding
+    if M * N * K > 2 ** 28:
+        tol = max(tol, 2e-5)  # the fp32 device reference itself carries rounding error at this size
+    assert rel_err(y.cpu(), ref) < tol
+    yb = gemm_bf16_tn(ad, bd, bias.to(dev), out_dtype)
+    assert rel_err(yb.cpu(), ref + bias.double()) < tol
+    yb2 = gemm_bf16_tn(ad, bd, bias.bfloat16().to(dev), out_dtype)
+    assert rel_err(yb2.cpu(), ref + bias.bfloat16().double()) < tol
+
+
+def test_gemm_exact_on_small_integers(dev):
+    """integer-valued operands with small K: every product and partial sum is exact in fp32, so the result
+    must equal the integer matrix product bit for bit whatever the summation order"""
+    from mase_amd._gemm import gemm_bf16_tn
+
+    g = torch.Generator().manual_seed(5)
+    a = torch.randint(-128, 128, (384, 256), generator=g).float()
+    b = torch.randint(-128, 128, (320, 256), generator=g).float()
+    y = gemm_bf16_tn(a.bfloat16().to(dev), b.bfloat16().to(dev), None, torch.float32)
+    assert torch.equal(y.cpu(), a @ b.t())
+
+
+def test_gemm_rejects_bad_k(dev):
+    from mase_amd._gemm import gemm_bf16_tn
+    from mase_amd._lib import MaseAmdError
+
+    with pytest.raises(MaseAmdError):
+        gemm_bf16_tn(torch.zeros(4, 24, device=dev).bfloat16(), torch.zeros(4, 24, device=dev).bfloat16(), None, torch.float32)
