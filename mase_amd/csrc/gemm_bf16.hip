@@ -10,9 +10,12 @@
 // Schedule: 256x256 output tile per work-group (4 wavefronts, 2x2, 128x128 each = 4x4 MFMA tiles, 256
 // accumulator registers per lane), K step 32, four LDS stages of 32 KB (128 of the CU's 160 KB).  Operand
 // tiles go from HBM/L2 straight into LDS with global_load_lds_dwordx4 (no staging registers, no ds_write);
-// the loads of K tile t+3 are issued before the MFMAs of tile t.  A wavefront-wide load deposits 64
-// consecutive 16-byte chunks = 16 LDS rows of 64 B, so the bank-conflict swizzle (chunk ^ ((row>>1)&3)) is
-// applied on the global-address side: each lane fetches the chunk that belongs at its LDS position.
+// the copies of K tile t+3 are issued while the MFMAs of tile t execute.  A wavefront-wide load deposits 64
+// consecutive 16-byte chunks = 16 LDS rows of 64 B, so the bank-conflict swizzle is applied on the
+// global-address side: each lane fetches the chunk that belongs at its LDS position.  The swizzle is
+// chunk ^ ((row>>2)&3): this LDS serves a ds_read_b128 sixteen lanes at a time out of 64 four-byte banks, so
+// the 16-byte slots (address/16 mod 16) of 16 consecutive rows must all differ; rows r, r+4, r+8, r+12 share
+// the same 64-byte quarter of the 256-byte bank period and get distinct slots from the XOR.
 // Rows beyond M or N are clamped to the last valid row (their products land in accumulators that are never
 // stored), so the main loop has no bounds checks.  Work-groups are renumbered so that each XCD
 // (blockIdx % 8) owns a contiguous band of tiles and re-reads operand panels from its own L2.
@@ -43,7 +46,7 @@ struct GemmParams {
 };
 
 __device__ __forceinline__ int lds_off(int row, int chunk) {
-  return row * kRowBytes + ((chunk ^ ((row >> 1) & 3)) << 4);
+  return row * kRowBytes + ((chunk ^ ((row >> 2) & 3)) << 4);
 }
 
 __device__ __forceinline__ float load_bias(const void* bias, int dt, int col) {
@@ -66,6 +69,7 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8) | ((N >> 4) << 14));
 }
 
+template <int OUT_DT>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int tid = threadIdx.x;
@@ -87,7 +91,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
 
   // global side of the async copies: wave w fills row groups g = w + 4*j (16 rows each), j = 0..3
   const int cp_row = lane >> 2;                              // row inside the 16-row group
-  const int cp_chunk = (lane & 3) ^ ((cp_row >> 1) & 3);     // chunk that belongs at LDS position lane&3
+  const int cp_chunk = (lane & 3) ^ ((cp_row >> 2) & 3);     // chunk that belongs at LDS position lane&3
   const size_t ldb = (size_t)p.K * 2;                        // bytes per operand row
   const unsigned char* ga[kWaveLoadsPerTile];
   const unsigned char* gb[kWaveLoadsPerTile];
@@ -97,15 +101,15 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     ga[j] = p.A + (size_t)min(m0 + r, p.M - 1) * ldb + cp_chunk * 16;
     gb[j] = p.B + (size_t)min(n0 + r, p.N - 1) * ldb + cp_chunk * 16;
   }
-  auto issue_tile = [&](int kt) {
-    unsigned char* sa = lds + (kt % kStages) * kStageBytes;
-    unsigned char* sb = sa + kTileBytes;
-    const size_t koff = (size_t)kt * kRowBytes;
-#pragma unroll
-    for (int j = 0; j < kWaveLoadsPerTile; ++j) {
-      async_copy_16(ga[j] + koff, sa + (wave + 4 * j) * 1024);
-      async_copy_16(gb[j] + koff, sb + (wave + 4 * j) * 1024);
-    }
+  // Tile numbers past the end are clamped to the last tile: the copy then lands in a stage that nobody
+  // reads any more, which keeps the main loop free of branches (and the vmcnt bookkeeping uniform).
+  const int nk = p.K / BK;
+  // copy number c (0..7) of K tile kt: row group c/2 of A (even c) or B (odd c)
+  auto issue_copy = [&](int kt, int c) {
+    unsigned char* st = lds + (kt % kStages) * kStageBytes + (c & 1) * kTileBytes;
+    const size_t koff = (size_t)min(kt, nk - 1) * kRowBytes;
+    const int j = c >> 1;
+    async_copy_16(((c & 1) ? gb[j] : ga[j]) + koff, st + (wave + 4 * j) * 1024);
   };
 
   f32x16_t acc[4][4];
@@ -116,63 +120,136 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  const int nk = p.K / BK;
   constexpr int kAhead = kStages - 1;  // tiles in flight beyond the one being consumed
+  constexpr int kLoadsPerTile = 2 * kWaveLoadsPerTile;  // async copies one wavefront issues per K tile
 #pragma unroll
   for (int t = 0; t < kAhead; ++t)
-    if (t < nk) issue_tile(t);
+#pragma unroll
+    for (int c = 0; c < kLoadsPerTile; ++c) issue_copy(t, c);
 
   const int frag_row = lane & 31;
   const int kgrp = lane >> 5;
+  // fragment f (0..3: A row tile f, 4..7: B column tile f-4) of K step s of tile kt
+  auto load_frag = [&](int kt, int s, int f) -> bf16x8_t {
+    const unsigned char* st = lds + (kt % kStages) * kStageBytes +
+                              ((f < 4) ? (wm * 128) * kRowBytes : kTileBytes + (wn * 128) * kRowBytes);
+    return __builtin_bit_cast(bf16x8_t, *(const uint4*)(st + lds_off((f & 3) * 32 + frag_row, s * 2 + kgrp)));
+  };
+
+  // Software pipeline, written out instruction by instruction and pinned with scheduling barriers, because a
+  // wavefront issues in order: an MFMA occupies the matrix pipe for 32 cycles, and whatever else has to be
+  // issued (LDS reads of the next K step, async copies of tile kt+3) must sit *between* MFMAs to be free.
+  //   step 0: 16 MFMAs on fragment set 0, interleaved with the 8 LDS reads of step 1 (set 1)
+  //   hand-over: own copies of tile kt+1 complete (vmcnt), barrier -> tile kt+1 visible, stage of kt-1 free
+  //   step 1: 16 MFMAs on set 1, interleaved with the 8 LDS reads of step 0 of tile kt+1 (set 0) and the
+  //           8 async copies of tile kt+3
+  // The barrier is a bare s_barrier: the fence of __syncthreads() would wait for all copies in flight.
+  bf16x8_t fr[2][8];
+#ifdef MASE_GEMM_DBG_CLOCK
+  const long long dbg_c0 = clock64(), dbg_w0 = wall_clock64();
+#endif
+  wait_vmcnt<2 * kLoadsPerTile>();  // tiles 1 and 2 may still be in flight
+  asm volatile("s_barrier" ::: "memory");
+#pragma unroll
+  for (int f = 0; f < 8; ++f) fr[0][f] = load_frag(0, 0, f);
   for (int kt = 0; kt < nk; ++kt) {
-    // tile kt has landed once at most the loads of the tiles issued after it are outstanding
-    const int newer = min(nk - 1 - kt, kAhead - 1);
-    if (newer >= 2) wait_vmcnt<2 * 2 * kWaveLoadsPerTile>();
-    else if (newer == 1) wait_vmcnt<2 * kWaveLoadsPerTile>();
-    else wait_vmcnt<0>();
-    // everyone's part of tile kt is in LDS, and everyone is done reading tile kt-1.  A bare s_barrier: the
-    // fence of __syncthreads() would also wait for the copies of the tiles still in flight.
-    __builtin_amdgcn_s_barrier();
-    if (kt + kAhead < nk) issue_tile(kt + kAhead);
-
-    const unsigned char* sa = lds + (kt % kStages) * kStageBytes + (wm * 128) * kRowBytes;
-    const unsigned char* sb = lds + (kt % kStages) * kStageBytes + kTileBytes + (wn * 128) * kRowBytes;
 #pragma unroll
-    for (int s = 0; s < BK / 16; ++s) {
-      bf16x8_t a[4], b[4];
+    for (int t = 0; t < 16; ++t) {
+      acc[t >> 2][t & 3] =
+          __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[0][t >> 2], fr[0][4 + (t & 3)], acc[t >> 2][t & 3], 0, 0, 0);
+      if (t < 8) fr[1][t] = load_frag(kt, 1, t);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#ifndef MASE_GEMM_DBG_NOLOAD
+    wait_vmcnt<kLoadsPerTile>();  // tiles kt+1 and kt+2 are in flight; kt+1 must have landed
+#endif
+#ifndef MASE_GEMM_DBG_NOBARRIER
+    asm volatile("s_barrier" ::: "memory");
+#endif
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        a[i] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(sa + lds_off(i * 32 + frag_row, s * 2 + kgrp)));
-        b[i] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(sb + lds_off(i * 32 + frag_row, s * 2 + kgrp)));
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    for (int t = 0; t < 16; ++t) {
+      acc[t >> 2][t & 3] =
+          __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[1][t >> 2], fr[1][4 + (t & 3)], acc[t >> 2][t & 3], 0, 0, 0);
+      if (t < 8) fr[0][t] = load_frag(kt + 1, 0, t);
+#ifndef MASE_GEMM_DBG_NOLOAD
+      else issue_copy(kt + kAhead, t - 8);  // into the stage of tile kt-1, which everybody has left
+#endif
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
+  wait_vmcnt<0>();  // no copy may still be in flight towards LDS when the work-group retires
+#ifdef MASE_GEMM_DBG_CLOCK
+  const long long dbg_c1 = clock64(), dbg_w1 = wall_clock64();
+#endif
 
-  // epilogue: acc[i][j][r] is C[row, col] with row = i*32 + (r/4)*8 + kgrp*4 + r%4, col = j*32 + lane%32
+  // Epilogue.  acc[i][j][r] is C[row, col] with row = i*32 + (r/4)*8 + kgrp*4 + r%4, col = j*32 + lane%32:
+  // stored directly that would be 256 four-byte stores per lane.  Instead each wavefront transposes one
+  // 32-row band at a time through its own LDS slice (32 x 128 fp32, rows padded to 136 floats so that the
+  // two half-waves of a ds_write_b32 hit disjoint banks) and writes 4 consecutive columns per lane: a
+  // half-wave covers 512 contiguous bytes of a C row.  LDS ops of one wavefront complete in order, so the
+  // slice needs no barrier; the one barrier below only separates it from the operand stages.
+  asm volatile("s_barrier" ::: "memory");
+  constexpr int kStgStride = 136;
+  float* stg = (float*)(lds + wave * (32 * kStgStride * 4));
+  const int c4 = (lane & 31) * 4;                      // first of this lane's 4 columns inside the wave tile
+  const int col0 = n0 + wn * 128 + c4;
+  const bool vec_ok = ((p.N & 3) == 0) && ((((uintptr_t)p.C) & 15u) == 0);
+  float bv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (p.bias != nullptr) {
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int col = n0 + wn * 128 + j * 32 + frag_row;
-    if (col >= p.N) continue;
-    const float bv = p.bias ? load_bias(p.bias, p.bias_dtype, col) : 0.0f;
+    for (int e = 0; e < 4; ++e)
+      if (col0 + e < p.N) bv[e] = load_bias(p.bias, p.bias_dtype, col0 + e);
+  }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < 4; ++i) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = m0 + wm * 128 + i * 32 + (r >> 2) * 8 + kgrp * 4 + (r & 3);
-        if (row >= p.M) continue;
-        const float v = acc[i][j][r] + bv;
-        const size_t o = (size_t)row * p.N + col;
-        if (p.out_dtype == MASE_DT_F32) ((float*)p.C)[o] = v;
-        else if (p.out_dtype == MASE_DT_BF16) ((uint16_t*)p.C)[o] = (uint16_t)f32_to_bf16_bits(v);
-        else ((uint16_t*)p.C)[o] = (uint16_t)f32_to_f16_bits(v);
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        stg[((r >> 2) * 8 + kgrp * 4 + (r & 3)) * kStgStride + j * 32 + frag_row] = acc[i][j][r];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const int rr = q * 2 + kgrp;
+      const int row = m0 + wm * 128 + i * 32 + rr;
+      const float4 v4 = *(const float4*)(stg + rr * kStgStride + c4);
+      const float v[4] = {v4.x + bv[0], v4.y + bv[1], v4.z + bv[2], v4.w + bv[3]};
+      if (row >= p.M) continue;
+      const size_t o = (size_t)row * p.N + col0;
+      if (vec_ok && col0 + 3 < p.N) {
+        if constexpr (OUT_DT == MASE_DT_F32) {
+          *(float4*)((float*)p.C + o) = make_float4(v[0], v[1], v[2], v[3]);
+        } else if constexpr (OUT_DT == MASE_DT_BF16) {
+          uint2 w;
+          w.x = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
+          w.y = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
+          *(uint2*)((uint16_t*)p.C + o) = w;
+        } else {
+          uint2 w;
+          w.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
+          w.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
+          *(uint2*)((uint16_t*)p.C + o) = w;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (col0 + e >= p.N) continue;
+          if constexpr (OUT_DT == MASE_DT_F32) ((float*)p.C)[o + e] = v[e];
+          else if constexpr (OUT_DT == MASE_DT_BF16) ((uint16_t*)p.C)[o + e] = (uint16_t)f32_to_bf16_bits(v[e]);
+          else ((uint16_t*)p.C)[o + e] = (uint16_t)f32_to_f16_bits(v[e]);
+        }
       }
     }
   }
+#ifdef MASE_GEMM_DBG_CLOCK
+  const long long dbg_c2 = clock64(), dbg_w2 = wall_clock64();
+  if (blockIdx.x == 7 && tid == 0) {
+    float* o = (float*)p.C;
+    __threadfence();
+    o[0] = (float)(dbg_c1 - dbg_c0); o[1] = (float)(dbg_w1 - dbg_w0);
+    o[2] = (float)(dbg_c2 - dbg_c1); o[3] = (float)(dbg_w2 - dbg_w1);
+  }
+#endif
 }
 
 }  // namespace
@@ -200,13 +277,18 @@ extern "C" int mase_gemm_bf16_tn(const void* A, const void* B, const void* bias,
   p.tiles_n = (int)((N + BN - 1) / BN);
   static bool attr_set = false;
   const size_t lds_bytes = (size_t)kStages * kStageBytes;
+  const void* kernels[3] = {(const void*)gemm_bf16_tn_kernel<MASE_DT_F32>, (const void*)gemm_bf16_tn_kernel<MASE_DT_BF16>,
+                            (const void*)gemm_bf16_tn_kernel<MASE_DT_F16>};
   if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)gemm_bf16_tn_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds_bytes) != hipSuccess)
-      return MASE_ERR_LAUNCH;
+    for (const void* k : kernels)
+      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
+        return MASE_ERR_LAUNCH;
     attr_set = true;
   }
-  hipLaunchKernelGGL(gemm_bf16_tn_kernel, dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(kGemmThreads), lds_bytes,
-                     (hipStream_t)stream, p);
+  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kGemmThreads);
+  hipStream_t st = (hipStream_t)stream;
+  if (out_dtype == MASE_DT_F32) hipLaunchKernelGGL(gemm_bf16_tn_kernel<MASE_DT_F32>, grid, block, lds_bytes, st, p);
+  else if (out_dtype == MASE_DT_BF16) hipLaunchKernelGGL(gemm_bf16_tn_kernel<MASE_DT_BF16>, grid, block, lds_bytes, st, p);
+  else hipLaunchKernelGGL(gemm_bf16_tn_kernel<MASE_DT_F16>, grid, block, lds_bytes, st, p);
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
