@@ -103,7 +103,7 @@ int mase_mxfp_qdq(const void* in, void* out, uint8_t* codes, uint8_t* scales, si
                   int out_dtype, int block_size, int exp_bits, int frac_bits, const uint32_t* log2_tab,
                   void* stream);
 
-/* C[M,N] = A[M,K] * B[N,K]^T (+ bias[N]): bf16 operands (both K-major, 16-byte aligned, K % 8 == 0), fp32
+/* C[M,N] = A[M,K] * B[N,K]^T (+ bias[N]): bf16 operands (both K-major, 16-byte aligned, K % 64 == 0), fp32
  * accumulation on the matrix cores, C written in out_dtype.  bias may be NULL; bias_dtype is its MASE_DT_*.
  * This is the contraction of LinearMXInt.forward / LinearMXFP.forward (nn/quantized/modules/linear.py:972,
  * :895) on operands whose MX values are held exactly in bf16. */

@@ -6,6 +6,8 @@ from torch import Tensor
 
 from . import _lib
 
+GEMM_K_MULTIPLE = 64  # K tile of mase_gemm_bf16_tn
+
 
 def gemm_bf16_tn(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dtype) -> Tensor:
     """``a[M,K] @ b[N,K].T + bias`` with bf16 operands and fp32 accumulation; result in ``out_dtype``."""
@@ -13,6 +15,11 @@ def gemm_bf16_tn(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dty
     lib = _lib.load()
     assert a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16
     assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[1]
+    if a.shape[1] % GEMM_K_MULTIPLE:
+        # the kernel consumes K in whole tiles; zero columns do not change the product
+        pad = GEMM_K_MULTIPLE - a.shape[1] % GEMM_K_MULTIPLE
+        a = torch.nn.functional.pad(a, (0, pad))
+        b = torch.nn.functional.pad(b, (0, pad))
     a = a.contiguous()
     b = b.contiguous()
     M, K = a.shape

@@ -8,14 +8,15 @@
 // differs.
 //
 // Schedule: 256x256 output tile per work-group (4 wavefronts, 2x2, 128x128 each = 4x4 MFMA tiles, 256
-// accumulator registers per lane), K step 32, four LDS stages of 32 KB (128 of the CU's 160 KB).  Operand
-// tiles go from HBM/L2 straight into LDS with global_load_lds_dwordx4 (no staging registers, no ds_write);
-// the copies of K tile t+3 are issued while the MFMAs of tile t execute.  A wavefront-wide load deposits 64
-// consecutive 16-byte chunks = 16 LDS rows of 64 B, so the bank-conflict swizzle is applied on the
-// global-address side: each lane fetches the chunk that belongs at its LDS position.  The swizzle is
-// chunk ^ ((row>>2)&3): this LDS serves a ds_read_b128 sixteen lanes at a time out of 64 four-byte banks, so
-// the 16-byte slots (address/16 mod 16) of 16 consecutive rows must all differ; rows r, r+4, r+8, r+12 share
-// the same 64-byte quarter of the 256-byte bank period and get distinct slots from the XOR.
+// accumulator registers per lane), K step 64 so that every operand row of a tile is one full 128-byte cache
+// line (64-byte rows made the L1 fetch every line twice and bound the loop), two LDS stages of 64 KB.
+// Operand tiles go from HBM/L2 straight into LDS with global_load_lds_dwordx4 (no staging registers, no
+// ds_write); the copies of K tile t+2 are issued while the last MFMAs of tile t execute.  A wavefront-wide
+// load deposits 64 consecutive 16-byte chunks = 8 LDS rows of 128 B, so the bank-conflict swizzle is applied
+// on the global-address side: each lane fetches the chunk that belongs at its LDS position.  The swizzle
+// is chunk ^ ((row>>1)&7): this LDS serves a ds_read_b128 sixteen lanes at a time out of 64 four-byte
+// banks, so the 16-byte slots (address/16 mod 16) of 16 consecutive rows must all differ; rows of equal
+// parity share a 128-byte half of the 256-byte bank period and get distinct slots from the XOR.
 // Rows beyond M or N are clamped to the last valid row (their products land in accumulators that are never
 // stored), so the main loop has no bounds checks.  Work-groups are renumbered so that each XCD
 // (blockIdx % 8) owns a contiguous band of tiles and re-reads operand panels from its own L2.
@@ -27,13 +28,15 @@ namespace {
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 256, BN = 256, BK = 32;
-constexpr int kStages = 4;
+constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int kStages = 2;
 constexpr int kGemmThreads = 256;
-constexpr int kRowBytes = BK * 2;                 // 64
-constexpr int kTileBytes = BM * kRowBytes;        // 16 KB per operand per stage
+constexpr int kRowBytes = BK * 2;                 // 128: one cache line per operand row per K tile
+constexpr int kTileBytes = BM * kRowBytes;        // 32 KB per operand per stage
 constexpr int kStageBytes = 2 * kTileBytes;       // A then B
-constexpr int kWaveLoadsPerTile = kTileBytes / 1024 / 4;  // per wavefront per operand per stage = 4
+constexpr int kWaveLoadsPerTile = kTileBytes / 1024 / 4;  // per wavefront per operand per stage = 8
+constexpr int kLoadsPerTile = 2 * kWaveLoadsPerTile;      // async copies one wavefront issues per K tile = 16
+constexpr int kSteps = BK / 16;                   // MFMA K steps per tile = 4
 
 struct GemmParams {
   const unsigned char* A;
@@ -46,7 +49,7 @@ struct GemmParams {
 };
 
 __device__ __forceinline__ int lds_off(int row, int chunk) {
-  return row * kRowBytes + ((chunk ^ ((row >> 2) & 3)) << 4);
+  return row * kRowBytes + ((chunk ^ ((row >> 1) & 7)) << 4);
 }
 
 __device__ __forceinline__ float load_bias(const void* bias, int dt, int col) {
@@ -80,8 +83,13 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // XCD-aware tile numbering (see header comment), then groups of 8 tile rows
   int bid = blockIdx.x;
   const int total = p.tiles_m * p.tiles_n;
+#ifndef MASE_GEMM_DBG_NOXCD
   if ((total & 7) == 0) bid = (bid & 7) * (total >> 3) + (bid >> 3);
-  constexpr int GROUP_M = 8;
+#endif
+#ifndef MASE_GEMM_GROUP_M
+#define MASE_GEMM_GROUP_M 4
+#endif
+  constexpr int GROUP_M = MASE_GEMM_GROUP_M;
   const int in_group = GROUP_M * p.tiles_n;
   const int first_m = (bid / in_group) * GROUP_M;
   const int gsz = min(p.tiles_m - first_m, GROUP_M);
@@ -89,22 +97,22 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   const int tile_n = (bid % in_group) / gsz;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-  // global side of the async copies: wave w fills row groups g = w + 4*j (16 rows each), j = 0..3
-  const int cp_row = lane >> 2;                              // row inside the 16-row group
-  const int cp_chunk = (lane & 3) ^ ((cp_row >> 2) & 3);     // chunk that belongs at LDS position lane&3
-  const size_t ldb = (size_t)p.K * 2;                        // bytes per operand row
+  // global side of the async copies: wave w fills row groups g = w + 4*j (8 rows of 128 B each), j = 0..7
+  const int cp_row = lane >> 3;  // row inside the 8-row group
+  const size_t ldb = (size_t)p.K * 2;  // bytes per operand row
   const unsigned char* ga[kWaveLoadsPerTile];
   const unsigned char* gb[kWaveLoadsPerTile];
 #pragma unroll
   for (int j = 0; j < kWaveLoadsPerTile; ++j) {
-    const int r = (wave + 4 * j) * 16 + cp_row;
+    const int r = (wave + 4 * j) * 8 + cp_row;
+    const int cp_chunk = (lane & 7) ^ ((r >> 1) & 7);  // chunk that belongs at LDS position lane&7 of row r
     ga[j] = p.A + (size_t)min(m0 + r, p.M - 1) * ldb + cp_chunk * 16;
     gb[j] = p.B + (size_t)min(n0 + r, p.N - 1) * ldb + cp_chunk * 16;
   }
   // Tile numbers past the end are clamped to the last tile: the copy then lands in a stage that nobody
   // reads any more, which keeps the main loop free of branches (and the vmcnt bookkeeping uniform).
   const int nk = p.K / BK;
-  // copy number c (0..7) of K tile kt: row group c/2 of A (even c) or B (odd c)
+  // copy number c (0..15) of K tile kt: row group c/2 of A (even c) or B (odd c)
   auto issue_copy = [&](int kt, int c) {
     unsigned char* st = lds + (kt % kStages) * kStageBytes + (c & 1) * kTileBytes;
     const size_t koff = (size_t)min(kt, nk - 1) * kRowBytes;
@@ -120,12 +128,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  constexpr int kAhead = kStages - 1;  // tiles in flight beyond the one being consumed
-  constexpr int kLoadsPerTile = 2 * kWaveLoadsPerTile;  // async copies one wavefront issues per K tile
 #pragma unroll
-  for (int t = 0; t < kAhead; ++t)
+  for (int c = 0; c < kLoadsPerTile; ++c) issue_copy(0, c);
 #pragma unroll
-    for (int c = 0; c < kLoadsPerTile; ++c) issue_copy(t, c);
+  for (int c = 0; c < kLoadsPerTile; ++c) issue_copy(1, c);
 
   const int frag_row = lane & 31;
   const int kgrp = lane >> 5;
@@ -138,44 +144,53 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
 
   // Software pipeline, written out instruction by instruction and pinned with scheduling barriers, because a
   // wavefront issues in order: an MFMA occupies the matrix pipe for 32 cycles, and whatever else has to be
-  // issued (LDS reads of the next K step, async copies of tile kt+3) must sit *between* MFMAs to be free.
-  //   step 0: 16 MFMAs on fragment set 0, interleaved with the 8 LDS reads of step 1 (set 1)
-  //   hand-over: own copies of tile kt+1 complete (vmcnt), barrier -> tile kt+1 visible, stage of kt-1 free
-  //   step 1: 16 MFMAs on set 1, interleaved with the 8 LDS reads of step 0 of tile kt+1 (set 0) and the
-  //           8 async copies of tile kt+3
+  // issued (LDS reads of the next K step, async copies of the tile after next) must sit *between* MFMAs to
+  // be free.  Per K tile (4 steps of 16 MFMAs, fragment sets ping-pong between fr[0] and fr[1]):
+  //   steps 0..2: MFMAs of step s, interleaved with the 8 LDS reads of step s+1
+  //   hand-over (after the MFMAs of step 2 are issued): this wavefront's reads of the tile are complete
+  //     (lgkmcnt) and its copies of tile kt+1 have landed (vmcnt); barrier -> tile kt+1 is visible to all
+  //     and nobody reads tile kt's stage any more
+  //   step 3: MFMAs, interleaved with the LDS reads of step 0 of tile kt+1 and the 16 copies of tile kt+2
+  //     (into the stage just vacated), which then have a whole tile's worth of MFMAs to land
   // The barrier is a bare s_barrier: the fence of __syncthreads() would wait for all copies in flight.
   bf16x8_t fr[2][8];
 #ifdef MASE_GEMM_DBG_CLOCK
   const long long dbg_c0 = clock64(), dbg_w0 = wall_clock64();
 #endif
-  wait_vmcnt<2 * kLoadsPerTile>();  // tiles 1 and 2 may still be in flight
+  wait_vmcnt<kLoadsPerTile>();  // tile 1 may still be in flight
   asm volatile("s_barrier" ::: "memory");
 #pragma unroll
   for (int f = 0; f < 8; ++f) fr[0][f] = load_frag(0, 0, f);
   for (int kt = 0; kt < nk; ++kt) {
 #pragma unroll
-    for (int t = 0; t < 16; ++t) {
-      acc[t >> 2][t & 3] =
-          __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[0][t >> 2], fr[0][4 + (t & 3)], acc[t >> 2][t & 3], 0, 0, 0);
-      if (t < 8) fr[1][t] = load_frag(kt, 1, t);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-#ifndef MASE_GEMM_DBG_NOLOAD
-    wait_vmcnt<kLoadsPerTile>();  // tiles kt+1 and kt+2 are in flight; kt+1 must have landed
-#endif
-#ifndef MASE_GEMM_DBG_NOBARRIER
-    asm volatile("s_barrier" ::: "memory");
-#endif
-    __builtin_amdgcn_sched_barrier(0);
+    for (int s = 0; s < kSteps; ++s) {
+      const int cur = s & 1, nxt = cur ^ 1;
 #pragma unroll
-    for (int t = 0; t < 16; ++t) {
-      acc[t >> 2][t & 3] =
-          __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[1][t >> 2], fr[1][4 + (t & 3)], acc[t >> 2][t & 3], 0, 0, 0);
-      if (t < 8) fr[0][t] = load_frag(kt + 1, 0, t);
+      for (int t = 0; t < 16; ++t) {
+        acc[t >> 2][t & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[cur][t >> 2], fr[cur][4 + (t & 3)],
+                                                                     acc[t >> 2][t & 3], 0, 0, 0);
+        if (s < kSteps - 1) {
+          if (t < 8) fr[nxt][t] = load_frag(kt, s + 1, t);
+        } else {
+          if (t < 8) {
+            fr[nxt][t] = load_frag(kt + 1, 0, t);
+          } else {  // the 16 copies of tile kt+2, two per MFMA slot, into the stage just vacated
 #ifndef MASE_GEMM_DBG_NOLOAD
-      else issue_copy(kt + kAhead, t - 8);  // into the stage of tile kt-1, which everybody has left
+            issue_copy(kt + 2, 2 * (t - 8));
+            issue_copy(kt + 2, 2 * (t - 8) + 1);
 #endif
-      __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (s == kSteps - 2) {
+        // all LDS reads of tile kt are in registers; the copies of tile kt+1 (issued one tile ago) have landed
+        wait_vmcnt<0>();
+#ifndef MASE_GEMM_DBG_NOBARRIER
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#endif
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   }
   wait_vmcnt<0>();  // no copy may still be in flight towards LDS when the work-group retires

@@ -46,9 +46,11 @@ def test_gemm_exact_on_small_integers(dev):
     assert torch.equal(y.cpu(), a @ b.t())
 
 
-def test_gemm_rejects_bad_k(dev):
-    from mase_amd._gemm import gemm_bf16_tn
-    from mase_amd._lib import MaseAmdError
+def test_gemm_c_abi_rejects_partial_k_tiles(dev):
+    from mase_amd import _lib
 
-    with pytest.raises(MaseAmdError):
-        gemm_bf16_tn(torch.zeros(4, 24, device=dev).bfloat16(), torch.zeros(4, 24, device=dev).bfloat16(), None, torch.float32)
+    lib = _lib.load()
+    a = torch.zeros(4, 96, device=dev).bfloat16()
+    c = torch.zeros(4, 4, device=dev)
+    rc = lib.mase_gemm_bf16_tn(a.data_ptr(), a.data_ptr(), None, c.data_ptr(), 4, 4, 96, 0, 0, None)
+    assert rc == -2
