@@ -146,7 +146,70 @@ class MxintQdq(Workload):
                 "kind": "port", "sample": f"{n} full passes of the same [4096,4096] fp32 tensor, {dt*1e3:.0f} ms each"}
 
 
-WORKLOADS = {w.name: w for w in (BfpQdq, MxintQdq)}
+class MxintLinear(Workload):
+    name = "mxint_linear"
+    metric = "MXINT8 Linear forward throughput (2*M*N*K flop per step; activation quantization included in the step)"
+    unit = "TFLOP/s"
+    dtype = "bf16"
+    bound = "mfma"
+    mfma_dtype = "bf16"
+    kernel = "gemm_bf16_tn_kernel"
+    M = N = K = 4096
+    config = {"workload": "LinearMXInt 4096x4096 (bias zeros), x fp32 [4096,4096] N(0,1), W N(0,0.02), block 32, "
+                          "8-bit mantissas; weights quantized at load_state_dict, seed 2"}
+    cfg = {"weight_block_size": 32, "weight_width": 8, "data_in_block_size": 32, "data_in_width": 8}
+
+    def make(self, torch):
+        g = torch.Generator().manual_seed(2)
+        x = torch.randn(self.M, self.K, generator=g)
+        w = torch.randn(self.N, self.K, generator=g) * 0.02
+        b = torch.zeros(self.N)
+        return x, w, b
+
+    def setup(self, torch, dev, n_buffers):
+        from mase_amd.quantized import LinearMXInt
+        from mase_amd.quantizers import _ops
+        from mase_amd._gemm import gemm_bf16_tn
+
+        self.torch = torch
+        x, w, b = self.make(torch)
+        self.host = (x, w, b)
+        self.m = LinearMXInt(self.K, self.N, bias=True, device=dev, config=dict(self.cfg))
+        self.m.load_state_dict({"weight": w, "bias": b})
+        self.bufs = [x.to(dev).roll(i, dims=0).contiguous() for i in range(max(n_buffers, 4))]
+        self.xq = _ops.mxint_qdq(self.bufs[0], 32, 8, -1, 8, out_dtype=torch.bfloat16)
+        self.wb = self.m._w_cache.get(self.m.weight)
+        assert self.wb is not None
+        self._gemm = gemm_bf16_tn
+
+    def step(self, i):
+        self.out = self.m(self.bufs[i % len(self.bufs)])
+
+    def dominant_step(self, i):
+        self.out = self._gemm(self.xq, self.wb, self.m.bias, self.torch.float32)
+
+    def work_per_step(self):
+        return 2.0 * self.M * self.N * self.K
+
+    def cpu_baseline(self, torch, budget_s):
+        from oracle import linear as OL
+
+        x, w, b = self.host
+        qw, qb = OL.mxint_prepare_weights(w, b, self.cfg)
+        OL.linear_mxint_forward(x[:64], qw, qb, self.cfg)
+        t0 = time.perf_counter()
+        n = 0
+        while True:
+            OL.linear_mxint_forward(x, qw, qb, self.cfg)
+            n += 1
+            if time.perf_counter() - t0 > budget_s or n >= 20:
+                break
+        dt = (time.perf_counter() - t0) / n
+        return {"value": self.work_per_step() / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+                "kind": "port", "sample": f"{n} full forwards (activation quantize-dequantize + fp32 F.linear), {dt*1e3:.0f} ms each"}
+
+
+WORKLOADS = {w.name: w for w in (BfpQdq, MxintQdq, MxintLinear)}
 
 
 def load_traffic(name):
@@ -196,9 +259,10 @@ def main():
     # kernel timing: one HIP event pair on the launch stream (torch's current stream is the one handed to the
     # C ABI) around K back-to-back launches; average launch duration = elapsed / K
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    dominant = getattr(w, "dominant_step", w.step)
     e0.record()
     for i in range(a.steps):
-        w.step(i)
+        dominant(i)
     e1.record()
     torch.cuda.synchronize()
     k_avg = e0.elapsed_time(e1) / a.steps

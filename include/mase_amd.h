@@ -65,10 +65,13 @@ const char* mase_error_string(int code);
  */
 
 /* MXINT quantize-dequantize over contiguous runs of `block_size` elements of a flat array.
- * in/out: numel elements of `dtype`.  codes (int8, numel) and scales (uint8, numel/block_size) are
- * optional packed outputs (both or neither; element_bits <= 8): value = codes * 2^(scales - 134). */
+ * in: numel elements of `dtype` (all arithmetic follows that dtype); out: numel elements of `out_dtype` (the
+ * reference's final `.to(dtype)`; MXINT8 values are exact in bf16, which is how the Linear path takes them).
+ * codes (int8, numel) and scales (uint8, numel/block_size) are optional packed outputs (both or neither;
+ * element_bits <= 8): value = codes * 2^(scales - 134). */
 int mase_mxint_qdq(const void* in, void* out, int8_t* codes, uint8_t* scales, size_t numel, int dtype,
-                   int block_size, int element_bits, int scale_bits, const uint32_t* log2_tab, void* stream);
+                   int out_dtype, int block_size, int element_bits, int scale_bits, const uint32_t* log2_tab,
+                   void* stream);
 
 /* Block floating point over [batch, rows, cols] with tiles of tile_rows x tile_cols inside each batch
  * item (ragged edges behave as if zero padded).  exponent_bias < 0 selects 2^(exponent_width-1)-1.

@@ -26,7 +26,7 @@ class MaseAmdError(RuntimeError):
 SIGNATURES = {
     "mase_abi_version": (c_int, []),
     "mase_error_string": (c_char_p, [c_int]),
-    "mase_mxint_qdq": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "mase_mxint_qdq": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mase_block_fp_workspace_bytes": (c_size_t, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int]),
     "mase_block_fp_qdq": (c_int, [c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
     "mase_integer_qdq": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_void_p]),

@@ -68,8 +68,39 @@ __device__ __forceinline__ float mxint_element(float x, int state, int k, int kc
 // One 16-byte vector per lane.  LPB lanes share one block (B = LPB * kVec) or one lane holds SUB blocks
 // (B = kVec / SUB).  For bf16 the dequantized value m * 2^(kc-b+1) has at most 8 significant bits (m is the
 // rne of an 8-bit-significand input), so it is packed by truncation unless it would be subnormal.
-template <int DT, int LPB, int SUB, int T>
-__global__ __launch_bounds__(T) void mxint_qdq_vec_kernel(const uint4* __restrict__ in, uint4* __restrict__ out,
+// out-of-place store of V fp32 registers as DTO elements at vector index idx
+template <int DTO, int V>
+__device__ __forceinline__ void store_vec(void* out, size_t idx, const float* y, bool exact_bf16) {
+  using TO = DTypeTraits<DTO>;
+  if constexpr (DTO == MASE_DT_F32) {
+    store_nt((uint4*)out + idx * (V / 4), TO::pack(y));
+    if constexpr (V == 8) store_nt((uint4*)out + idx * 2 + 1, TO::pack(y + 4));
+  } else if constexpr (V == 8) {
+    if (DTO == MASE_DT_BF16 && exact_bf16) {
+      uint4 o;
+      o.x = pack_bf16_exact(y[0], y[1]);
+      o.y = pack_bf16_exact(y[2], y[3]);
+      o.z = pack_bf16_exact(y[4], y[5]);
+      o.w = pack_bf16_exact(y[6], y[7]);
+      store_nt((uint4*)out + idx, o);
+    } else {
+      store_nt((uint4*)out + idx, TO::pack(y));
+    }
+  } else {  // 4 sixteen-bit results: 8 bytes
+    uint2 o;
+    if constexpr (DTO == MASE_DT_BF16) {
+      o.x = f32_to_bf16_bits(y[0]) | (f32_to_bf16_bits(y[1]) << 16);
+      o.y = f32_to_bf16_bits(y[2]) | (f32_to_bf16_bits(y[3]) << 16);
+    } else {
+      o.x = f32_to_f16_bits(y[0]) | (f32_to_f16_bits(y[1]) << 16);
+      o.y = f32_to_f16_bits(y[2]) | (f32_to_f16_bits(y[3]) << 16);
+    }
+    ((uint2*)out)[idx] = o;
+  }
+}
+
+template <int DT, int DTO, int LPB, int SUB, int T>
+__global__ __launch_bounds__(T) void mxint_qdq_vec_kernel(const uint4* __restrict__ in, void* __restrict__ out,
                                                           int8_t* __restrict__ codes, uint8_t* __restrict__ scales,
                                                           size_t n_vec, MxintParams p) {
   using TR = DTypeTraits<DT>;
@@ -82,7 +113,7 @@ __global__ __launch_bounds__(T) void mxint_qdq_vec_kernel(const uint4* __restric
   float x[V], y[V];
   int c[V];
   TR::unpack(raw, x);
-  bool exact_bf16 = (DT == MASE_DT_BF16);
+  bool exact_bf16 = (DT == MASE_DT_BF16);  // 8-bit-significand inputs: results need no rounding to bf16
 #pragma unroll
   for (int s = 0; s < SUB; ++s) {
     uint32_t m;
@@ -117,20 +148,7 @@ __global__ __launch_bounds__(T) void mxint_qdq_vec_kernel(const uint4* __restric
       }
     }
   }
-  if constexpr (DT == MASE_DT_BF16) {
-    if (exact_bf16) {
-      uint4 o;
-      o.x = pack_bf16_exact(y[0], y[1]);
-      o.y = pack_bf16_exact(y[2], y[3]);
-      o.z = pack_bf16_exact(y[4], y[5]);
-      o.w = pack_bf16_exact(y[6], y[7]);
-      store_nt(out + idx, o);
-    } else {
-      store_nt(out + idx, TR::pack(y));
-    }
-  } else {
-    store_nt(out + idx, TR::pack(y));
-  }
+  store_vec<DTO, V>(out, idx, y, exact_bf16);
   if (codes != nullptr) {
     if constexpr (V == 4) {
       ((uint32_t*)codes)[idx] = (uint32_t)(c[0] & 0xFF) | ((uint32_t)(c[1] & 0xFF) << 8) | ((uint32_t)(c[2] & 0xFF) << 16) |
@@ -147,7 +165,7 @@ __global__ __launch_bounds__(T) void mxint_qdq_vec_kernel(const uint4* __restric
 }
 
 // Any block size / alignment: one work-item per block, two passes over its elements.
-template <int DT>
+template <int DT, int DTO>
 __global__ __launch_bounds__(kThreads) void mxint_qdq_generic_kernel(const void* __restrict__ in, void* __restrict__ out,
                                                                      int8_t* __restrict__ codes,
                                                                      uint8_t* __restrict__ scales, size_t n_blocks,
@@ -162,13 +180,13 @@ __global__ __launch_bounds__(kThreads) void mxint_qdq_generic_kernel(const void*
   int state = block_exponent<DT>(m, p, k, kc);
   for (int j = 0; j < B; ++j) {
     int code;
-    TR::store1(out, off + j, mxint_element<DT>(TR::load1(in, off + j), state, k, kc, p, code));
+    DTypeTraits<DTO>::store1(out, off + j, mxint_element<DT>(TR::load1(in, off + j), state, k, kc, p, code));
     if (codes != nullptr) codes[off + j] = (int8_t)code;
   }
   if (codes != nullptr) scales[blk] = (uint8_t)((state == 0) ? min(max(kc - p.qshift + 134, 0), 255) : 255);
 }
 
-template <int DT>
+template <int DT, int DTO>
 int launch_mxint(const void* in, void* out, int8_t* codes, uint8_t* scales, size_t numel, int B, const MxintParams& p,
                  hipStream_t st) {
   using TR = DTypeTraits<DT>;
@@ -180,8 +198,8 @@ int launch_mxint(const void* in, void* out, int8_t* codes, uint8_t* scales, size
     size_t n_vec = numel / V;
     dim3 grid(blocks_for(n_vec, kRunThreads)), block(kRunThreads);
 #define MASE_MXINT_CASE(LPB_, SUB_)                                                                               \
-  hipLaunchKernelGGL((mxint_qdq_vec_kernel<DT, LPB_, SUB_, kRunThreads>), grid, block, 0, st, (const uint4*)in, \
-                     (uint4*)out, codes, scales, n_vec, p)
+  hipLaunchKernelGGL((mxint_qdq_vec_kernel<DT, DTO, LPB_, SUB_, kRunThreads>), grid, block, 0, st, (const uint4*)in, \
+                     out, codes, scales, n_vec, p)
     if (B >= V) {
       switch (B / V) {
         case 1: MASE_MXINT_CASE(1, 1); break;
@@ -204,7 +222,7 @@ int launch_mxint(const void* in, void* out, int8_t* codes, uint8_t* scales, size
 #undef MASE_MXINT_CASE
   } else {
     size_t n_blocks = numel / (size_t)B;
-    hipLaunchKernelGGL((mxint_qdq_generic_kernel<DT>), dim3(blocks_for(n_blocks, kThreads)), dim3(kThreads), 0, st, in,
+    hipLaunchKernelGGL((mxint_qdq_generic_kernel<DT, DTO>), dim3(blocks_for(n_blocks, kThreads)), dim3(kThreads), 0, st, in,
                        out, codes, scales, n_blocks, B, p);
   }
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
@@ -213,9 +231,24 @@ int launch_mxint(const void* in, void* out, int8_t* codes, uint8_t* scales, size
 }  // namespace
 }  // namespace mase
 
+namespace mase {
+namespace {
+template <int DT>
+int launch_mxint_out(int out_dtype, const void* in, void* out, int8_t* codes, uint8_t* scales, size_t numel, int B,
+                     const MxintParams& p, hipStream_t st) {
+  switch (out_dtype) {
+    case MASE_DT_F32: return launch_mxint<DT, MASE_DT_F32>(in, out, codes, scales, numel, B, p, st);
+    case MASE_DT_BF16: return launch_mxint<DT, MASE_DT_BF16>(in, out, codes, scales, numel, B, p, st);
+    case MASE_DT_F16: return launch_mxint<DT, MASE_DT_F16>(in, out, codes, scales, numel, B, p, st);
+    default: return MASE_ERR_DTYPE;
+  }
+}
+}  // namespace
+}  // namespace mase
+
 extern "C" int mase_mxint_qdq(const void* in, void* out, int8_t* codes, uint8_t* scales, size_t numel, int dtype,
-                              int block_size, int element_bits, int scale_bits, const uint32_t* log2_tab,
-                              void* stream) {
+                              int out_dtype, int block_size, int element_bits, int scale_bits,
+                              const uint32_t* log2_tab, void* stream) {
   using namespace mase;
   if (numel == 0) return MASE_OK;
   if (in == nullptr || out == nullptr || log2_tab == nullptr) return MASE_ERR_NULL;
@@ -224,6 +257,7 @@ extern "C" int mase_mxint_qdq(const void* in, void* out, int8_t* codes, uint8_t*
   if (element_bits < 2 || element_bits > 24 || scale_bits < 1 || scale_bits > 8) return MASE_ERR_PARAM;
   if (codes != nullptr && element_bits > 8) return MASE_ERR_PARAM;
   if (dtype != MASE_DT_F32 && dtype != MASE_DT_BF16 && dtype != MASE_DT_F16) return MASE_ERR_DTYPE;
+  if (out_dtype != MASE_DT_F32 && out_dtype != MASE_DT_BF16 && out_dtype != MASE_DT_F16) return MASE_ERR_DTYPE;
   MxintParams p;
   p.qshift = element_bits - 1;
   p.bias = (1 << (scale_bits - 1)) - 1;
@@ -233,8 +267,8 @@ extern "C" int mase_mxint_qdq(const void* in, void* out, int8_t* codes, uint8_t*
   p.tab = log2_tab;
   hipStream_t st = (hipStream_t)stream;
   switch (dtype) {
-    case MASE_DT_F32: return launch_mxint<MASE_DT_F32>(in, out, codes, scales, numel, block_size, p, st);
-    case MASE_DT_BF16: return launch_mxint<MASE_DT_BF16>(in, out, codes, scales, numel, block_size, p, st);
-    default: return launch_mxint<MASE_DT_F16>(in, out, codes, scales, numel, block_size, p, st);
+    case MASE_DT_F32: return launch_mxint_out<MASE_DT_F32>(out_dtype, in, out, codes, scales, numel, block_size, p, st);
+    case MASE_DT_BF16: return launch_mxint_out<MASE_DT_BF16>(out_dtype, in, out, codes, scales, numel, block_size, p, st);
+    default: return launch_mxint_out<MASE_DT_F16>(out_dtype, in, out, codes, scales, numel, block_size, p, st);
   }
 }

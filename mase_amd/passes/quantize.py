@@ -1,0 +1,122 @@
+"""Module-level quantize pass with the contract of the reference's
+``chop/passes/module/transforms/quantize/quantize.py:95-151`` for ``nn.Linear`` targets:
+
+    network, info = quantize_module_transform_pass(network, {"by": "type", "linear": {"config": {"name": "mxint", ...}}})
+
+Like the reference it pops ``"by"`` (and ``"gptq"``) from ``pass_args`` and ``"name"`` from a by-type/by-name config
+(:28, :48, :140), instantiates ``quantized_module_map["linear_<name>"]`` with the original module's shape, bias,
+device and dtype (``module_modify_helper.py:149-176``), hands the weights over with
+``load_state_dict(deepcopy(state_dict), strict=False)`` (:103-114) and swaps the module in by name (:137-141).
+Model-family wrappers (attention, MLP, embeddings) and the GPTQ pre-pass are outside this build.
+"""
+from __future__ import annotations
+
+import inspect
+import logging
+import re
+from copy import deepcopy
+
+import torch
+
+from ..quantized.modules import quantized_module_map
+
+
+def _instantiate_linear(module, postfix, module_map, additional_module_args):
+    linear_cls = module_map[f"linear_{postfix}"]
+    has_bias = module.bias is not None
+    kwargs = dict(in_features=module.in_features, out_features=module.out_features, bias=has_bias,
+                  device=module.weight.device, dtype=module.weight.dtype)
+    if "config" in inspect.signature(linear_cls.__init__).parameters:
+        return linear_cls(**kwargs, config=additional_module_args)
+    return linear_cls(**kwargs, **additional_module_args)
+
+
+def _instantiate_module(module, postfix, module_map, additional_module_args):
+    module_args = additional_module_args["config"]
+    if isinstance(module, torch.nn.Linear):
+        return _instantiate_linear(module, postfix, module_map, module_args)
+    raise ValueError(f"{module} is not supported.")
+
+
+def _weight_replacement(x, y):
+    target_state_dict = deepcopy(x.state_dict())
+    missing_keys, unexpected_keys = y.load_state_dict(target_state_dict, strict=False)
+    if missing_keys:
+        logging.warning(f"Missing keys when loading state_dict: {missing_keys} from {x} to {y}")
+    if unexpected_keys:
+        logging.warning(f"Unexpected keys when loading state_dict: {unexpected_keys} from {x} to {y}")
+    return y
+
+
+def _replace_by_name(network, name, module):
+    original = network.get_submodule(name)
+    new = _weight_replacement(original, module)
+    parent_name, _, child = name.rpartition(".")
+    parent = network.get_submodule(parent_name) if parent_name else network
+    setattr(parent, child, new)
+    return network
+
+
+def _quantize_by_type(network, pass_args):
+    for type_name, config in pass_args.items():
+        n_m = dict(network.named_modules())
+        if type_name == "linear":
+            module = torch.nn.Linear
+        elif type_name == "conv2d":
+            raise ValueError("conv2d is outside this build (Linear only)")
+        else:
+            raise ValueError(f"{type_name} is not supported!")
+        config = config["config"]
+        postfix = config.pop("name")
+        for n, m in n_m.items():
+            if isinstance(m, module):
+                new_m = _instantiate_module(m, postfix, quantized_module_map, {"config": config})
+                network = _replace_by_name(network, n, new_m)
+    return network
+
+
+def _quantize_by_name(network, pass_args):
+    n_m = dict(network.named_modules())
+    for n, m in n_m.items():
+        if n in pass_args:
+            quan_config = pass_args[n]["config"]
+            postfix = quan_config.pop("name")
+            new_m = _instantiate_module(m, postfix, quantized_module_map, {"config": quan_config})
+            network = _replace_by_name(network, n, new_m)
+    return network
+
+
+def _match_a_pattern(name: str, patterns):
+    for pattern in patterns:
+        if re.fullmatch(pattern, name):
+            return pattern
+    return None
+
+
+def _quantize_by_regex_name(network, pass_args):
+    patterns = list(pass_args.keys())
+    n_m = dict(network.named_modules())
+    for n, m in n_m.items():
+        matched = _match_a_pattern(n, patterns)
+        if not matched:
+            continue
+        quan_config = pass_args[matched]["config"]
+        postfix = quan_config["name"]
+        new_m = _instantiate_module(m, postfix, quantized_module_map, {"config": quan_config})
+        network = _replace_by_name(network, n, new_m)
+    return network
+
+
+def quantize_module_transform_pass(network, pass_args):
+    if pass_args.pop("gptq", None) is not None:
+        raise NotImplementedError("the GPTQ pre-pass (calibration data) is outside this build")
+    by = pass_args.pop("by")
+    if by == "type":
+        network = _quantize_by_type(network, pass_args)
+    elif by == "name":
+        network = _quantize_by_name(network, pass_args)
+    elif by == "regex_name":
+        network = _quantize_by_regex_name(network, pass_args)
+    else:
+        raise ValueError(f'Unsupported quantize "by": {by}')
+    return network, {}

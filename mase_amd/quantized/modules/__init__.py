@@ -1,0 +1,20 @@
+"""``quantized_module_map``: the in-scope entries of the reference's registry
+(``chop/nn/quantized/modules/__init__.py:236-251, 388-408``), same keys."""
+from .linear import (
+    LinearBlockFP,
+    LinearInteger,
+    LinearMinifloatDenorm,
+    LinearMinifloatIEEE,
+    LinearMXFP,
+    LinearMXInt,
+)
+
+quantized_module_map = {
+    "linear_block_fp": LinearBlockFP,
+    "linear_integer": LinearInteger,
+    "linear_fixed": LinearInteger,
+    "linear_minifloat_denorm": LinearMinifloatDenorm,
+    "linear_minifloat_ieee": LinearMinifloatIEEE,
+    "linear_mxint": LinearMXInt,
+    "linear_mxfp": LinearMXFP,
+}

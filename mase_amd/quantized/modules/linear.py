@@ -1,0 +1,161 @@
+"""Quantized ``nn.Linear`` modules with the constructors, config keys and ``load_state_dict`` behaviour of the
+reference's ``chop/nn/quantized/modules/linear.py`` (``_LinearBase`` :61-83, ``LinearInteger`` :100-126,
+``LinearMinifloatDenorm/IEEE`` :129-173, ``LinearBlockFP`` :199-219, ``LinearMXFP`` :817-895, ``LinearMXInt``
+:898-972), so that the quantize pass can instantiate them through ``quantized_module_map`` unchanged.
+"""
+from __future__ import annotations
+
+import torch
+from torch.nn import functional as F
+
+from ...quantizers import _ops, mxfp_quantizer, mxint_quantizer
+from ..functional.linear import linearBlockFP, linearInteger, linearMinifloatDenorm, linearMinifloatIEEE
+from ..functional.mx_linear import WeightCache, mx_linear
+
+
+class _LinearBase(torch.nn.Linear):
+    def __init__(self, in_features: int, out_features: int, bias: bool = False, device=None, dtype=None) -> None:
+        super().__init__(in_features, out_features, bias, device, dtype)
+        self.bypass = False
+        self.pruning_masks = None
+
+
+class LinearInteger(_LinearBase):
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, dtype=None, config=None,
+                 out_config=None, floor=None) -> None:
+        super().__init__(in_features, out_features, bias, device, dtype)
+        assert config is not None, "config is None!"
+        if floor is not None:
+            config["floor"] = floor
+        self.config = config
+        self.out_config = out_config
+        self.bypass = config.get("bypass", False)
+
+    def forward(self, x):
+        if self.bypass:
+            return F.linear(x, self.weight, self.bias)
+        return linearInteger(x, self.weight, self.bias, self.config, self.out_config)
+
+
+class _ConfigLinear(_LinearBase):
+    _functional = None
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, dtype=None,
+                 config=None) -> None:
+        super().__init__(in_features, out_features, bias, device, dtype)
+        assert config is not None, "config is None!"
+        self.config = config
+        self.bypass = config.get("bypass", False)
+
+    def forward(self, x):
+        if self.bypass:
+            return F.linear(x, self.weight, self.bias)
+        return type(self)._functional(x, self.weight, self.bias, self.config)
+
+
+class LinearMinifloatDenorm(_ConfigLinear):
+    _functional = staticmethod(linearMinifloatDenorm)
+
+
+class LinearMinifloatIEEE(_ConfigLinear):
+    _functional = staticmethod(linearMinifloatIEEE)
+
+
+class LinearBlockFP(_ConfigLinear):
+    _functional = staticmethod(linearBlockFP)
+
+
+class _LinearMX(_LinearBase):
+    """Shared shape of LinearMXInt / LinearMXFP: weights (and optionally the bias) are quantized in place when a
+    state dict is loaded; the forward quantizes the activations and contracts.  Inference only."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, dtype=None,
+                 config=None) -> None:
+        super().__init__(in_features, out_features, bias, device, dtype)
+        assert config is not None, "config is None!"
+        self.config = config
+        self.bypass = config.get("bypass", False)
+        self.gptq = config.get("gptq", False)
+        self.clip_search = config.get("clip_search", False)
+        self._w_cache = WeightCache()
+
+    def _quantize_params(self):
+        raise NotImplementedError
+
+    def invalidate_weight_cache(self):
+        """Forget the bf16 image of the weight (needed only after an in-place edit through ``weight.data``)."""
+        self._w_cache.invalidate()
+
+    def load_state_dict(self, state_dict, strict=True, assign=False):
+        """Load pretrained weights, then quantize them in place."""
+        result = super().load_state_dict(state_dict, strict=strict, assign=assign)
+        if self.bypass or self.gptq:
+            return result
+        self._quantize_params()
+        self._w_cache.invalidate()
+        return result
+
+
+class LinearMXInt(_LinearMX):
+    def _quantize_params(self):
+        cfg = self.config
+        self.weight.data.copy_(
+            mxint_quantizer(self.weight.data, block_size=cfg["weight_block_size"], element_bits=cfg["weight_width"],
+                            block_dim=1, quantile_search=self.clip_search)
+        )
+        b_block_size = cfg.get("bias_block_size")
+        b_element_bits = cfg.get("bias_width")
+        if self.bias is not None and b_block_size is not None and b_element_bits is not None:
+            self.bias.data.copy_(
+                mxint_quantizer(self.bias.data, block_size=b_block_size, element_bits=b_element_bits, block_dim=0,
+                                quantile_search=self.clip_search)
+            )
+
+    @torch.no_grad()
+    def forward(self, x):
+        if self.bypass:
+            return F.linear(x, self.weight, self.bias)
+        bs = self.config.get("data_in_block_size")
+        bits = self.config.get("data_in_width")
+        if bs is None or bits is None:
+            return F.linear(x, self.weight, self.bias)
+        return mx_linear(
+            x, self.weight, self.bias,
+            lambda t: _ops.mxint_qdq(t, bs, bits, -1, 8, out_dtype=torch.bfloat16),
+            lambda t: mxint_quantizer(t, block_size=bs, element_bits=bits, block_dim=-1),
+            self._w_cache,
+        )
+
+
+class LinearMXFP(_LinearMX):
+    def _quantize_params(self):
+        cfg = self.config
+        self.weight.data.copy_(
+            mxfp_quantizer(self.weight.data, block_size=cfg["weight_block_size"],
+                           element_exp_bits=cfg["weight_exponent_width"], element_frac_bits=cfg["weight_frac_width"],
+                           block_dim=1)
+        )
+        b_block_size = cfg.get("bias_block_size")
+        b_exp_bits = cfg.get("bias_exponent_width")
+        b_frac_bits = cfg.get("bias_frac_width")
+        if self.bias is not None and b_block_size is not None and b_exp_bits is not None:
+            self.bias.data.copy_(
+                mxfp_quantizer(self.bias.data, block_size=b_block_size, element_exp_bits=b_exp_bits,
+                               element_frac_bits=b_frac_bits, block_dim=0)
+            )
+
+    @torch.no_grad()
+    def forward(self, x):
+        if self.bypass:
+            return F.linear(x, self.weight, self.bias)
+        bs = self.config.get("data_in_block_size")
+        eb = self.config.get("data_in_exponent_width")
+        fb = self.config.get("data_in_frac_width")
+        if bs is None or eb is None:
+            return F.linear(x, self.weight, self.bias)
+        return mx_linear(
+            x, self.weight, self.bias,
+            lambda t: _ops.mxfp_qdq(t, bs, eb, fb, -1, 8, out_dtype=torch.bfloat16),
+            lambda t: mxfp_quantizer(t, block_size=bs, element_exp_bits=eb, element_frac_bits=fb, block_dim=-1),
+            self._w_cache,
+        )

@@ -48,8 +48,10 @@ def _from_block_last_flat(flat: Tensor, shape: Sequence[int], block_dim: int) ->
 # ------------------------------------------------------------------------------------------------
 # MXINT  (reference: mxint/mxint.py:211-251)
 # ------------------------------------------------------------------------------------------------
-def mxint_qdq(x: Tensor, block_size: int, element_bits: int, block_dim: int, scale_bits: int, pack: bool = False):
-    """Returns the dequantized tensor, or (dequantized, codes int8, scales uint8) when ``pack``."""
+def mxint_qdq(x: Tensor, block_size: int, element_bits: int, block_dim: int, scale_bits: int, pack: bool = False,
+              out_dtype: torch.dtype | None = None):
+    """Returns the dequantized tensor (in ``out_dtype``, default the input dtype), or
+    (dequantized, codes int8, scales uint8) when ``pack``."""
     _lib.require_device(x, "mxint_quantizer")
     lib = _lib.load()
     shape = tuple(x.shape)
@@ -57,7 +59,7 @@ def mxint_qdq(x: Tensor, block_size: int, element_bits: int, block_dim: int, sca
     assert block_dim < nd and block_dim >= -nd
     assert x.numel() % block_size == 0, f"Input tensor size {x.numel()} is not divisible by block size {block_size}."
     flat = _to_block_last_flat(x, block_dim)
-    out = torch.empty_like(flat)
+    out = torch.empty_like(flat, dtype=out_dtype or x.dtype)
     codes = scales = None
     if pack:
         codes = torch.empty(flat.numel(), dtype=torch.int8, device=x.device)
@@ -66,7 +68,8 @@ def mxint_qdq(x: Tensor, block_size: int, element_bits: int, block_dim: int, sca
     rc = lib.mase_mxint_qdq(
         flat.data_ptr(), out.data_ptr(),
         codes.data_ptr() if pack else None, scales.data_ptr() if pack else None,
-        flat.numel(), _lib.dtype_code(x), block_size, element_bits, scale_bits, tab.data_ptr(), _lib.stream_ptr(x),
+        flat.numel(), _lib.dtype_code(x), _lib.dtype_code(out), block_size, element_bits, scale_bits, tab.data_ptr(),
+        _lib.stream_ptr(x),
     )
     _lib.check(rc, "mase_mxint_qdq")
     res = _from_block_last_flat(out, shape, block_dim)
@@ -80,7 +83,7 @@ _LEGAL_MXFP = ((4, 3), (5, 2), (2, 3), (3, 2), (2, 1), (1, 2))
 
 
 def mxfp_qdq(x: Tensor, block_size: int, exp_bits: int, frac_bits: int, block_dim: int, scale_exp_bits: int,
-             pack: bool = False):
+             pack: bool = False, out_dtype: torch.dtype | None = None):
     _lib.require_device(x, "mxfp_quantizer")
     lib = _lib.load()
     assert scale_exp_bits in (8,), f"Invalid scale exponent bits: {scale_exp_bits}. Legal values are: (8,)."
@@ -92,7 +95,7 @@ def mxfp_qdq(x: Tensor, block_size: int, exp_bits: int, frac_bits: int, block_di
     assert block_dim < nd and block_dim >= -nd
     assert x.numel() % block_size == 0
     flat = _to_block_last_flat(x, block_dim)
-    out = torch.empty_like(flat)
+    out = torch.empty_like(flat, dtype=out_dtype or x.dtype)
     codes = scales = None
     if pack:
         codes = torch.empty(flat.numel(), dtype=torch.uint8, device=x.device)
@@ -102,7 +105,7 @@ def mxfp_qdq(x: Tensor, block_size: int, exp_bits: int, frac_bits: int, block_di
     rc = lib.mase_mxfp_qdq(
         flat.data_ptr(), out.data_ptr(),
         codes.data_ptr() if pack else None, scales.data_ptr() if pack else None,
-        flat.numel(), dt, dt, block_size, exp_bits, frac_bits, tab.data_ptr(), _lib.stream_ptr(x),
+        flat.numel(), dt, _lib.dtype_code(out), block_size, exp_bits, frac_bits, tab.data_ptr(), _lib.stream_ptr(x),
     )
     _lib.check(rc, "mase_mxfp_qdq")
     res = _from_block_last_flat(out, shape, block_dim)

@@ -44,12 +44,15 @@ def test_entry_points_reject_bad_arguments_without_a_gpu(lib):
     """argument validation happens before any HIP call, so it can be exercised on the CPU"""
     buf = ctypes.create_string_buffer(4096)
     p = ctypes.cast(buf, ctypes.c_void_p)
-    assert lib.mase_mxint_qdq(None, p, None, None, 64, 0, 32, 8, 8, p, None) == -1
-    assert lib.mase_mxint_qdq(p, p, None, None, 65, 0, 32, 8, 8, p, None) == -2
-    assert lib.mase_mxint_qdq(p, p, None, None, 64, 7, 32, 8, 8, p, None) == -4
-    assert lib.mase_mxint_qdq(p, p, None, None, 64, 0, 32, 1, 8, p, None) == -5
-    assert lib.mase_mxint_qdq(p, p, p, None, 64, 0, 32, 8, 8, p, None) == -1
-    assert lib.mase_mxint_qdq(p, p, None, None, 0, 0, 32, 8, 8, p, None) == 0  # empty input is a no-op
+    assert lib.mase_mxint_qdq(None, p, None, None, 64, 0, 0, 32, 8, 8, p, None) == -1
+    assert lib.mase_mxint_qdq(p, p, None, None, 65, 0, 0, 32, 8, 8, p, None) == -2
+    assert lib.mase_mxint_qdq(p, p, None, None, 64, 7, 0, 32, 8, 8, p, None) == -4
+    assert lib.mase_mxint_qdq(p, p, None, None, 64, 0, 9, 32, 8, 8, p, None) == -4
+    assert lib.mase_mxint_qdq(p, p, None, None, 64, 0, 0, 32, 1, 8, p, None) == -5
+    assert lib.mase_mxint_qdq(p, p, p, None, 64, 0, 0, 32, 8, 8, p, None) == -1
+    assert lib.mase_mxint_qdq(p, p, None, None, 0, 0, 0, 32, 8, 8, p, None) == 0  # empty input is a no-op
+    assert lib.mase_gemm_bf16_tn(p, p, None, p, 4, 4, 96, 0, 0, None) == -2  # K must be whole 64-wide tiles
+    assert lib.mase_gemm_bf16_tn(p, None, None, p, 4, 4, 64, 0, 0, None) == -1
     assert lib.mase_mxfp_qdq(p, p, None, None, 64, 0, 0, 32, 3, 3, p, None) == -5  # illegal element format
     assert lib.mase_mxfp_qdq(p, p, None, None, 63, 0, 0, 32, 4, 3, p, None) == -2
     assert lib.mase_block_fp_qdq(p, p, 1, 4, 16, 0, 16, 0, 8, 8, -1, 0, p, None, 0, None) == -2

@@ -1,0 +1,216 @@
+"""GPU parity of the quantized Linear modules against the CPU oracle.
+
+Error measure everywhere: max|y - y_ref| / max|y_ref|, bound 1e-2 (the north-star tolerance; the measured
+values are printed and are orders of magnitude below it for fp32).  Quantized parameters are compared bit-exactly.
+"""
+import copy
+
+import pytest
+import torch
+from torch import nn
+
+import oracle as O
+from oracle import linear as OL
+from helpers import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def rel_err(y, ref):
+    return float((y.double().cpu() - ref.double()).abs().max() / ref.double().abs().max())
+
+
+MXINT_CFG = {"weight_block_size": 32, "weight_width": 8, "data_in_block_size": 32, "data_in_width": 8}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape,out_f,bias", [((16, 128), 96, True), ((4, 33, 256), 64, False), ((300, 64), 257, True)])
+def test_linear_mxint(dev, dtype, shape, out_f, bias):
+    from mase_amd.quantized import LinearMXInt
+
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(*shape, generator=g).to(dtype)
+    w = (torch.randn(out_f, shape[-1], generator=g) * 0.02).to(dtype)
+    b = torch.randn(out_f, generator=g).to(dtype) if bias else None
+    cfg = dict(MXINT_CFG)
+    m = LinearMXInt(shape[-1], out_f, bias=bias, device=dev, dtype=dtype, config=copy.deepcopy(cfg))
+    sd = {"weight": w} if b is None else {"weight": w, "bias": b}
+    res = m.load_state_dict(copy.deepcopy(sd))
+    missing, unexpected = res
+    assert not missing and not unexpected
+    qw, qb = OL.mxint_prepare_weights(w, b, cfg)
+    assert_bits_equal(m.weight.data, qw, "LinearMXInt weight after load_state_dict")
+    y = m(x.to(dev))
+    ref = OL.linear_mxint_forward(x, qw, qb, cfg)
+    assert y.shape == ref.shape and y.dtype == ref.dtype
+    e = rel_err(y, ref)
+    print(f"LinearMXInt {dtype} {shape}->{out_f}: rel err {e:.3e}")
+    assert e < (TOL if dtype != torch.float32 else 1e-5)
+    assert m._w_cache.get(m.weight) is not None  # the matrix-core path was taken
+
+
+def test_linear_mxint_config3_full_size(dev):
+    """BASELINE config 3: activations [4096,4096] N(0,1), weight [4096,4096] N(0,0.02), bias zeros, fp32."""
+    from mase_amd.quantized import LinearMXInt
+
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(4096, 4096, generator=g)
+    w = torch.randn(4096, 4096, generator=g) * 0.02
+    b = torch.zeros(4096)
+    cfg = dict(MXINT_CFG)
+    m = LinearMXInt(4096, 4096, bias=True, device=dev, config=dict(cfg))
+    m.load_state_dict({"weight": w, "bias": b})
+    qw, qb = OL.mxint_prepare_weights(w, b, cfg)
+    assert_bits_equal(m.weight.data, qw, "config 3 weight")
+    y = m(x.to(dev))
+    ref = OL.linear_mxint_forward(x, qw, qb, cfg)
+    e = rel_err(y, ref)
+    print(f"config 3 rel err {e:.3e}")
+    assert e < 1e-5 < TOL
+
+
+def test_linear_mxint_bias_quantization_bypass_and_fallbacks(dev):
+    from mase_amd.quantized import LinearMXInt
+
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(8, 64, generator=g)
+    w = torch.randn(32, 64, generator=g)
+    b = torch.randn(32, generator=g)
+    cfg = {**MXINT_CFG, "bias_block_size": 16, "bias_width": 6}
+    m = LinearMXInt(64, 32, device=dev, config=dict(cfg))
+    m.load_state_dict({"weight": w, "bias": b})
+    qw, qb = OL.mxint_prepare_weights(w, b, cfg)
+    assert_bits_equal(m.bias.data, qb, "quantized bias")
+    assert rel_err(m(x.to(dev)), OL.linear_mxint_forward(x, qw, qb, cfg)) < 1e-5
+    # bypass: a plain linear on untouched weights
+    mb = LinearMXInt(64, 32, device=dev, config={**cfg, "bypass": True})
+    mb.load_state_dict({"weight": w, "bias": b})
+    assert_bits_equal(mb.weight.data, w, "bypass keeps the weight")
+    assert rel_err(mb(x.to(dev)), torch.nn.functional.linear(x, w, b)) < 1e-5
+    # gptq: weights are not quantized at load; they have no exact bf16 image -> library GEMM on q(x)
+    mg = LinearMXInt(64, 32, device=dev, config={**cfg, "gptq": True})
+    mg.load_state_dict({"weight": w, "bias": b})
+    assert mg._w_cache.get(mg.weight) is None
+    assert rel_err(mg(x.to(dev)), torch.nn.functional.linear(O.mxint_quantizer(x, 32, 8), w, b)) < 1e-5
+    # no activation config: weights only
+    mw = LinearMXInt(64, 32, device=dev, config={"weight_block_size": 32, "weight_width": 8})
+    mw.load_state_dict({"weight": w, "bias": b})
+    assert rel_err(mw(x.to(dev)), torch.nn.functional.linear(x, qw, b)) < 1e-5
+    # a weight modified after loading is picked up (version counter), also when it leaves the MXINT grid
+    with torch.no_grad():
+        m.weight.mul_(2.0)
+    assert rel_err(m(x.to(dev)), OL.linear_mxint_forward(x, qw * 2, qb, cfg)) < 1e-5
+    with torch.no_grad():
+        m.weight.add_(0.001)
+    assert rel_err(m(x.to(dev)), OL.linear_mxint_forward(x, qw * 2 + 0.001, qb, cfg)) < 1e-5
+    assert m._w_cache.get(m.weight) is None
+    m.weight.data.copy_(qw.to(dev))          # an edit through .data needs an explicit invalidation
+    m.invalidate_weight_cache()
+    assert rel_err(m(x.to(dev)), OL.linear_mxint_forward(x, qw, qb, cfg)) < 1e-5
+    with pytest.raises(AssertionError):
+        LinearMXInt(64, 32, device=dev)
+
+
+@pytest.mark.parametrize("wfmt,xfmt", [((2, 1), (4, 3)), ((4, 3), (4, 3)), ((5, 2), (5, 2)), ((2, 3), (3, 2)), ((1, 2), (2, 1))])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_linear_mxfp(dev, dtype, wfmt, xfmt):
+    from mase_amd.quantized import LinearMXFP
+
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(5, 40, 128, generator=g)
+    x[..., 7] *= 20
+    x = x.to(dtype)
+    w = (torch.randn(96, 128, generator=g) * 0.02).to(dtype)
+    cfg = {"weight_block_size": 32, "weight_exponent_width": wfmt[0], "weight_frac_width": wfmt[1],
+           "data_in_block_size": 32, "data_in_exponent_width": xfmt[0], "data_in_frac_width": xfmt[1]}
+    m = LinearMXFP(128, 96, bias=False, device=dev, dtype=dtype, config=dict(cfg))
+    m.load_state_dict({"weight": w})
+    qw, _ = OL.mxfp_prepare_weights(w, None, cfg)
+    assert_bits_equal(m.weight.data, qw, "LinearMXFP weight")
+    y = m(x.to(dev))
+    ref = OL.linear_mxfp_forward(x, qw, None, cfg)
+    e = rel_err(y, ref)
+    print(f"LinearMXFP {dtype} w=e{wfmt[0]}m{wfmt[1]} x=e{xfmt[0]}m{xfmt[1]}: rel err {e:.3e}")
+    assert e < (TOL if dtype != torch.float32 else 1e-5)
+
+
+def test_linear_block_fp_integer_minifloat(dev):
+    from mase_amd.quantized import LinearBlockFP, LinearInteger, LinearMinifloatDenorm, LinearMinifloatIEEE
+
+    g = torch.Generator().manual_seed(5)
+    x3 = torch.randn(2, 24, 64, generator=g)
+    x2 = torch.randn(24, 64, generator=g)
+    w = torch.randn(48, 64, generator=g) * 0.1
+    b = torch.randn(48, generator=g)
+    sd = {"weight": w, "bias": b}
+    bfp = {f"{k}_{s}": v for k in ("weight", "data_in", "bias")
+           for s, v in (("width", 8), ("exponent_width", 8), ("exponent_bias", None), ("block_size", [16]))}
+    m = LinearBlockFP(64, 48, device=dev, config=dict(bfp))
+    m.load_state_dict(sd)
+    for x in (x3, x2):
+        assert rel_err(m(x.to(dev)), OL.linear_block_fp(x, w, b, bfp)) < 1e-5
+    icfg = {"weight_width": 8, "weight_frac_width": 6, "data_in_width": 8, "data_in_frac_width": 4, "bias_width": 8,
+            "bias_frac_width": 5}
+    mi = LinearInteger(64, 48, device=dev, config=dict(icfg))
+    mi.load_state_dict(sd)
+    assert rel_err(mi(x3.to(dev)), OL.linear_integer(x3, w, b, icfg)) < 1e-5
+    mo = LinearInteger(64, 48, device=dev, config={**icfg, "data_out_width": 8, "data_out_frac_width": 3}, floor=True)
+    mo.load_state_dict(sd)
+    ref = OL.linear_integer(x3, w, b, {**icfg, "data_out_width": 8, "data_out_frac_width": 3, "floor": True})
+    got = mo(x3.to(dev)).cpu()
+    # the output re-quantization can flip a value sitting on a rounding boundary by one step of 2^-3
+    assert float((got - ref).abs().max()) <= 0.125 and float(((got - ref) != 0).float().mean()) < 1e-3
+    mcfg = {f"{k}_{s}": v for k in ("weight", "data_in", "bias") for s, v in (("width", 8), ("exponent_width", 4), ("exponent_bias", None))}
+    for cls, fn in ((LinearMinifloatDenorm, OL.linear_minifloat_denorm), (LinearMinifloatIEEE, OL.linear_minifloat_ieee)):
+        mm = cls(64, 48, device=dev, config=dict(mcfg))
+        mm.load_state_dict(sd)
+        assert rel_err(mm(x3.to(dev)), fn(x3, w, b, mcfg)) < 1e-5
+
+
+class MLP(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.fc1 = nn.Linear(64, 128)
+        self.act = nn.ReLU()
+        self.fc2 = nn.Linear(128, 32, bias=False)
+        self.head = nn.ModuleDict({"out": nn.Linear(32, 32)})
+
+    def forward(self, x):
+        return self.head["out"](self.fc2(self.act(self.fc1(x))))
+
+
+def test_quantize_module_transform_pass(dev):
+    from mase_amd.passes import quantize_module_transform_pass
+    from mase_amd.quantized import LinearInteger, LinearMXInt, quantized_module_map
+
+    torch.manual_seed(0)
+    net = MLP().to(dev)
+    ref_net = copy.deepcopy(net).cpu()
+    x = torch.randn(16, 64)
+    pass_args = {"by": "type", "linear": {"config": {"name": "mxint", **MXINT_CFG}}}
+    out, info = quantize_module_transform_pass(net, pass_args)
+    assert info == {} and out is net
+    assert "by" not in pass_args and "name" not in pass_args["linear"]["config"]  # popped like the reference does
+    assert all(isinstance(m, LinearMXInt) for m in (net.fc1, net.fc2, net.head["out"]))
+    assert net.fc2.bias is None and net.fc1.config is pass_args["linear"]["config"]
+    h = x
+    for lin, act in ((ref_net.fc1, True), (ref_net.fc2, False), (ref_net.head["out"], False)):
+        qw, qb = OL.mxint_prepare_weights(lin.weight.data, lin.bias.data if lin.bias is not None else None, MXINT_CFG)
+        h = OL.linear_mxint_forward(h, qw, qb, MXINT_CFG)
+        h = torch.relu(h) if act else h
+    assert rel_err(net(x.to(dev)), h) < 1e-4
+    # by name and by regex
+    net2 = MLP().to(dev)
+    quantize_module_transform_pass(net2, {"by": "name", "fc1": {"config": {"name": "integer", "weight_width": 8,
+        "weight_frac_width": 4, "data_in_width": 8, "data_in_frac_width": 4, "bias_width": 8, "bias_frac_width": 4}}})
+    assert isinstance(net2.fc1, LinearInteger) and type(net2.fc2) is nn.Linear
+    net3 = MLP().to(dev)
+    quantize_module_transform_pass(net3, {"by": "regex_name", r"head\.\w+": {"config": {"name": "mxint", **MXINT_CFG}}})
+    assert isinstance(net3.head["out"], LinearMXInt) and type(net3.fc1) is nn.Linear
+    with pytest.raises(ValueError):
+        quantize_module_transform_pass(MLP().to(dev), {"by": "type", "default": {"config": {"name": None}}})
+    with pytest.raises(ValueError):
+        quantize_module_transform_pass(MLP().to(dev), {"by": "layer"})
+    assert set(quantized_module_map) >= {"linear_mxint", "linear_mxfp", "linear_block_fp", "linear_integer",
+                                         "linear_fixed", "linear_minifloat_ieee", "linear_minifloat_denorm"}
