@@ -146,6 +146,32 @@ class MxintQdq(Workload):
                 "kind": "port", "sample": f"{n} full passes of the same [4096,4096] fp32 tensor, {dt*1e3:.0f} ms each"}
 
 
+class CopyBytes(Workload):
+    """calibration: a plain streaming copy of the same size as the default workload (128 MiB in, 128 MiB out)"""
+    name = "copy"
+    metric = "streaming copy throughput (bytes read + bytes written)"
+    unit = "GB/s"
+    dtype = "u8"
+    kernel = "copy_bytes_kernel"
+    config = {"workload": "mase_copy_bytes of 134217728 bytes (calibration: achievable HBM ceiling, counter scale)"}
+    nbytes = 134217728
+
+    def setup(self, torch, dev, n_buffers):
+        from mase_amd import _lib
+
+        self.lib = _lib.load()
+        self._lib = _lib
+        self.bufs = [torch.randint(0, 255, (self.nbytes,), dtype=torch.uint8, device=dev) for _ in range(max(n_buffers, 4))]
+        self.outs = [torch.empty(self.nbytes, dtype=torch.uint8, device=dev) for _ in range(2)]
+
+    def step(self, i):
+        src, dst = self.bufs[i % len(self.bufs)], self.outs[i % 2]
+        self._lib.check(self.lib.mase_copy_bytes(src.data_ptr(), dst.data_ptr(), self.nbytes, self._lib.stream_ptr(src)), "copy")
+
+    def work_per_step(self):
+        return 2.0 * self.nbytes
+
+
 class MxintLinear(Workload):
     name = "mxint_linear"
     metric = "MXINT8 Linear forward throughput (2*M*N*K flop per step; activation quantization included in the step)"
@@ -209,7 +235,7 @@ class MxintLinear(Workload):
                 "kind": "port", "sample": f"{n} full forwards (activation quantize-dequantize + fp32 F.linear), {dt*1e3:.0f} ms each"}
 
 
-WORKLOADS = {w.name: w for w in (BfpQdq, MxintQdq, MxintLinear)}
+WORKLOADS = {w.name: w for w in (BfpQdq, MxintQdq, MxintLinear, CopyBytes)}
 
 
 def load_traffic(name):

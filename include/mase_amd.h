@@ -113,6 +113,10 @@ int mase_mxfp_qdq(const void* in, void* out, uint8_t* codes, uint8_t* scales, si
 int mase_gemm_bf16_tn(const void* A, const void* B, const void* bias, void* C, size_t M, size_t N, size_t K,
                       int out_dtype, int bias_dtype, void* stream);
 
+/* Plain streaming copy of `bytes` (multiple of 16, 16-byte aligned pointers).  No counterpart in the reference:
+ * it is the calibration kernel for the achievable-bandwidth ceiling and for scaling hardware byte counters. */
+int mase_copy_bytes(const void* in, void* out, size_t bytes, void* stream);
+
 /* test/diagnostic helpers (host only, no device work) */
 uint32_t mase_isclose_zero_threshold_bits(int dtype); /* largest |x| (fp32 bits) that isclose(x, 0) accepts */
 float mase_round_scalar_to_dtype(double v, int dtype); /* how a clamp bound is represented in dtype */

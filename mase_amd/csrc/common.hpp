@@ -227,6 +227,38 @@ __device__ __forceinline__ int ceil_log2_lib(uint32_t b, const uint32_t* __restr
   return (M <= tab[kb]) ? k : k + 1;
 }
 
+// Wave-resident copy of the table entries for k in [-32, 31] (lane i holds k = i - 32), read with one
+// coalesced load per wavefront that is in flight together with the data load.  A lookup is then a
+// ds_bpermute (cross-lane read, no memory access); exponents outside the window fall back to the table.
+// Every lane of the wavefront must call init() and lookups before any lane exits.
+struct WaveLog2 {
+  uint32_t reg;
+  const uint32_t* tab;
+  int half;
+  __device__ __forceinline__ void init(const uint32_t* __restrict__ t, int h) {
+    tab = t;
+    half = h;
+    reg = t[h + 149 - 32 + (int)(threadIdx.x & 63)];
+  }
+  __device__ __forceinline__ uint32_t threshold(int k) const {
+    int kb = k + 32;
+    uint32_t thr = (uint32_t)__builtin_amdgcn_ds_bpermute((kb & 63) << 2, (int)reg);
+    if ((unsigned)kb >= 64u) thr = tab[half + k + 149];
+    return thr;
+  }
+};
+__device__ __forceinline__ int ceil_log2_lib(uint32_t b, const uint32_t* __restrict__, const WaveLog2& w) {
+  uint32_t M;
+  int k = split_pow2(b, M);
+  uint32_t thr = w.threshold(k);
+  return (M == 0 || M <= thr) ? k : k + 1;
+}
+__device__ __forceinline__ int floor_log2_lib(uint32_t b, const uint32_t* __restrict__, const WaveLog2& w) {
+  uint32_t M;
+  int k = split_pow2(b, M);
+  return (M >= w.threshold(k)) ? k + 1 : k;
+}
+
 __device__ __forceinline__ int floor_log2_lib(uint32_t b, const uint32_t* __restrict__ tab) {
   uint32_t M;
   int k = split_pow2(b, M);

@@ -42,14 +42,18 @@ struct BfpParams {
 // work-group size of the single-pass kernel: small groups stream best on this part
 constexpr int kRunThreads = MASE_RUN_THREADS;
 
-// returns 0: zero tile, 1: regular (e valid), 2: NaN tile
+// returns 0: zero tile, 1: regular (e valid), 2: NaN tile.  The log2 lookup runs for every lane (on a
+// harmless stand-in when the maximum is zero or not finite): the wave-resident table is read with a
+// cross-lane operation that needs all lanes of the wavefront to take part.
 template <int DT, typename... Meta>
 __device__ __forceinline__ int tile_exponent(uint32_t mbits, const BfpParams& p, int& e, const Meta&... meta) {
   using TR = DTypeTraits<DT>;
+  const bool special = (mbits == 0) || (mbits >= 0x7F800000u);
+  const int k = ceil_log2_lib(special ? 0x3F800000u : mbits, p.tab, meta...);
   if (mbits == 0) return 0;
   if (mbits > 0x7F800000u) return 2;
   // an infinite maximum has log2 = inf, which the clamp brings down to e_hi
-  e = (mbits == 0x7F800000u) ? p.e_hi : min(max(ceil_log2_lib(mbits, p.tab, meta...), p.e_lo), p.e_hi);
+  e = (mbits == 0x7F800000u) ? p.e_hi : min(max(k, p.e_lo), p.e_hi);
   return (e > TR::kMaxPow2) ? 2 : 1;
 }
 
@@ -83,9 +87,10 @@ __global__ __launch_bounds__(T) void bfp_run_kernel(const uint4* __restrict__ in
   using TR = DTypeTraits<DT>;
   constexpr int V = TR::kVec;
   const size_t idx = (size_t)blockIdx.x * T + threadIdx.x;
-  if (idx >= n_vec) return;  // whole tiles drop out together: n_vec is a multiple of LPB
-  const uint4 raw = load_nt(in + idx);
-  const Log2Meta meta = load_log2_meta(p.tab, 0);
+  const bool live = idx < n_vec;  // whole tiles are live or dead together: n_vec is a multiple of LPB
+  const uint4 raw = live ? load_nt(in + idx) : make_uint4(0, 0, 0, 0);
+  WaveLog2 meta;
+  meta.init(p.tab, 0);
   float x[V], y[V];
   TR::unpack(raw, x);
   if constexpr (SUB == 1) {
@@ -109,6 +114,7 @@ __global__ __launch_bounds__(T) void bfp_run_kernel(const uint4* __restrict__ in
         if (p.zero_sign_mask == 0u) r = r + 0.0f;
         y[j] = (fabsf(x[j]) <= thr) ? (x[j] + 0.0f) : r;
       }
+      if (!live) return;
       if constexpr (DT == MASE_DT_BF16) {
         uint4 o;
         o.x = pack_bf16_exact(y[0], y[1]);
@@ -131,12 +137,12 @@ __global__ __launch_bounds__(T) void bfp_run_kernel(const uint4* __restrict__ in
 #pragma unroll
       for (int j = 0; j < EPS; ++j) m = max(m, f2bits(x[s * EPS + j]) & 0x7FFFFFFFu);
       int e = 0;
-      const int state = tile_exponent<DT>(m, p, e);
+      const int state = tile_exponent<DT>(m, p, e, meta);
 #pragma unroll
       for (int j = 0; j < EPS; ++j) y[s * EPS + j] = bfp_element<DT>(x[s * EPS + j], state, e, p);
     }
   }
-  store_nt(out + idx, TR::pack(y));
+  if (live) store_nt(out + idx, TR::pack(y));
 }
 
 __global__ __launch_bounds__(kThreads) void fill_u32_kernel(uint32_t* __restrict__ p, size_t n, uint32_t v) {

@@ -26,9 +26,12 @@ constexpr int kUnroll = 2;
 // state 0: all flushed, 1: regular (sh valid), 2: NaN block
 template <typename... Meta>
 __device__ __forceinline__ int mxfp_block_scale(uint32_t mbits, const MxfpParams& p, int& sh, const Meta&... meta) {
+  // the lookup runs for every lane (see WaveLog2), on a stand-in when the maximum is zero or not finite
+  const bool special = (mbits == 0) || (mbits >= 0x7F800000u);
+  const int kf = floor_log2_lib(special ? 0x3F800000u : mbits, p.tab, meta...);
   if (mbits == 0) return 0;
   if (mbits >= 0x7F800000u) return 2;
-  sh = min(max(floor_log2_lib(mbits, p.tab, meta...) - p.el_emax, -127), 128);
+  sh = min(max(kf - p.el_emax, -127), 128);
   return 1;
 }
 
@@ -55,7 +58,8 @@ __global__ __launch_bounds__(kThreads) void mxfp_qdq_vec_kernel(const void* __re
   constexpr int V = (TI::kVec == 8 || TO::kVec == 8) ? 8 : 4;
   constexpr int EPS = V / SUB;
   const size_t base = (size_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
-  const Log2Meta meta = load_log2_meta(p.tab, kLog2TabHalf);
+  WaveLog2 meta;
+  meta.init(p.tab, kLog2TabHalf);
 #pragma unroll
   for (int u = 0; u < kUnroll; ++u) {
     size_t idx = base + (size_t)u * kThreads;

@@ -41,8 +41,10 @@ __device__ __forceinline__ int block_exponent(uint32_t mbits, const MxintParams&
                                               const Meta&... meta) {
   using TR = DTypeTraits<DT>;
   mbits = max(mbits, TR::kTinyBits);
+  // the lookup runs for every lane (see WaveLog2), on a stand-in when the maximum is not finite
+  const int kf = ceil_log2_lib(mbits >= 0x7F800000u ? 0x3F800000u : mbits, p.tab, meta...);
   if (mbits > 0x7F800000u) return 2;
-  k = (mbits == 0x7F800000u) ? 1024 : ceil_log2_lib(mbits, p.tab, meta...);
+  k = (mbits == 0x7F800000u) ? 1024 : kf;
   kc = min(max(k + p.bias, 0), p.scale_max) - p.bias;
   return (k > TR::kMaxPow2) ? 1 : 0;
 }
@@ -107,9 +109,10 @@ __global__ __launch_bounds__(T) void mxint_qdq_vec_kernel(const uint4* __restric
   constexpr int V = TR::kVec;
   constexpr int EPS = V / SUB;  // elements per sub-block held by this lane
   const size_t idx = (size_t)blockIdx.x * T + threadIdx.x;
-  if (idx >= n_vec) return;  // whole blocks drop out together: n_vec is a multiple of LPB
-  const uint4 raw = load_nt(in + idx);
-  const Log2Meta meta = load_log2_meta(p.tab, 0);
+  const bool live = idx < n_vec;  // whole blocks are live or dead together: n_vec is a multiple of LPB
+  const uint4 raw = live ? load_nt(in + idx) : make_uint4(0, 0, 0, 0);
+  WaveLog2 meta;
+  meta.init(p.tab, 0);
   float x[V], y[V];
   int c[V];
   TR::unpack(raw, x);
@@ -139,7 +142,7 @@ __global__ __launch_bounds__(T) void mxint_qdq_vec_kernel(const uint4* __restric
 #pragma unroll
       for (int j = 0; j < EPS; ++j) y[s * EPS + j] = mxint_element<DT>(x[s * EPS + j], state, k, kc, p, c[s * EPS + j]);
     }
-    if (codes != nullptr) {
+    if (codes != nullptr && live) {
       int sb = (state == 0) ? min(max(kc - p.qshift + 134, 0), 255) : 255;
       if constexpr (LPB > 1) {
         if ((idx & (LPB - 1)) == 0) scales[idx / LPB] = (uint8_t)sb;
@@ -148,6 +151,7 @@ __global__ __launch_bounds__(T) void mxint_qdq_vec_kernel(const uint4* __restric
       }
     }
   }
+  if (!live) return;
   store_vec<DTO, V>(out, idx, y, exact_bf16);
   if (codes != nullptr) {
     if constexpr (V == 4) {
