@@ -17,6 +17,8 @@
  *   mase_minifloat_qdq      nn/quantizers/minifloat.py:90-117, :200-225 (minifloat_denorm/ieee_quantizer)
  *   mase_minifloat_mx_qdq   nn/quantizers/_minifloat_mx/minifloat.py:12-33 (minifloat_quantizer_sim)
  *   mase_mxfp_qdq           nn/quantizers/mxfp/mxfp.py:187-230    (mxfp_quantizer, non-search branch)
+ *   mase_mxfp_pack, mase_gemm_mxfp_scaled   nn/quantized/modules/linear.py:877-895 (LinearMXFP.forward on
+ *                           formats the block-scaled matrix instruction supports)
  *   mase_gemm_bf16_tn       nn/quantized/modules/linear.py:972 and :895 (the F.linear of LinearMXInt.forward /
  *                           LinearMXFP.forward on the quantize-dequantized operands)
  */
@@ -112,6 +114,22 @@ int mase_mxfp_qdq(const void* in, void* out, uint8_t* codes, uint8_t* scales, si
  * :895) on operands whose MX values are held exactly in bf16. */
 int mase_gemm_bf16_tn(const void* A, const void* B, const void* bias, void* C, size_t M, size_t N, size_t K,
                       int out_dtype, int bias_dtype, void* stream);
+
+/* MXFP packing for the block-scaled matrix instruction.  in: numel elements (numel % 32 == 0, blocks of 32
+ * consecutive elements); element format (exp_bits, frac_bits) in {(4,3), (5,2), (2,1)}.  codes: one byte per
+ * element for 8-bit formats, two elements per byte (even element in the low nibble) for (2,1); scales: one E8M0
+ * byte per block.  codes/scales decode to the values of mase_mxfp_qdq, except that a block using a code the
+ * OCP format reserves (e4m3 S.1111.111, e5m2 exponent 31) is stored with scale+1 and halved elements.
+ * Quantizer part: nn/quantizers/mxfp/fake.py:12-72. */
+int mase_mxfp_pack(const void* in, uint8_t* codes, uint8_t* scales, size_t numel, int in_dtype, int exp_bits,
+                   int frac_bits, const uint32_t* log2_tab, void* stream);
+
+/* C[M,N] = A[M,K] * B[N,K]^T (+ bias[N]) on packed MXFP operands (layout of mase_mxfp_pack, K % 128 == 0), using
+ * the block-scaled MFMA.  a_format / b_format: 0 = e4m3, 1 = e5m2, 4 = e2m1 (B only).  The contraction of
+ * LinearMXFP.forward (nn/quantized/modules/linear.py:877-895) for hardware formats. */
+int mase_gemm_mxfp_scaled(const void* A, const void* A_scales, int a_format, const void* B, const void* B_scales,
+                          int b_format, const void* bias, void* C, size_t M, size_t N, size_t K, int out_dtype,
+                          int bias_dtype, void* stream);
 
 /* Plain streaming copy of `bytes` (multiple of 16, 16-byte aligned pointers).  No counterpart in the reference:
  * it is the calibration kernel for the achievable-bandwidth ceiling and for scaling hardware byte counters. */

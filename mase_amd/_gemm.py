@@ -33,3 +33,49 @@ def gemm_bf16_tn(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dty
     )
     _lib.check(rc, "mase_gemm_bf16_tn")
     return out
+
+
+# element formats of the block-scaled matrix instruction: (exp_bits, frac_bits) -> format code of the C ABI
+MXFP_HW_FORMATS = {(4, 3): 0, (5, 2): 1, (2, 1): 4}
+MXFP_K_MULTIPLE = 128  # K tile of mase_gemm_mxfp_scaled
+
+
+def mxfp_pack(x: Tensor, exp_bits: int, frac_bits: int):
+    """Quantize ``x`` (blocks of 32 along the last dim) to packed MXFP codes + E8M0 scales for the matrix
+    instruction.  Returns ``(codes uint8 [..., K] or [..., K/2], scales uint8 [..., K/32])``."""
+    from ._tables import log2_table
+
+    _lib.require_device(x, "mxfp_pack")
+    lib = _lib.load()
+    assert (exp_bits, frac_bits) in MXFP_HW_FORMATS
+    x = x.contiguous()
+    K = x.shape[-1]
+    assert K % 32 == 0, "the last dimension must hold whole blocks of 32"
+    per_byte = 2 if exp_bits + frac_bits + 1 <= 4 else 1
+    codes = torch.empty(*x.shape[:-1], K // per_byte, dtype=torch.uint8, device=x.device)
+    scales = torch.empty(*x.shape[:-1], K // 32, dtype=torch.uint8, device=x.device)
+    tab = log2_table(torch.float32, x.device)
+    rc = lib.mase_mxfp_pack(x.data_ptr(), codes.data_ptr(), scales.data_ptr(), x.numel(), _lib.dtype_code(x),
+                            exp_bits, frac_bits, tab.data_ptr(), _lib.stream_ptr(x))
+    _lib.check(rc, "mase_mxfp_pack")
+    return codes, scales
+
+
+def gemm_mxfp_scaled(a_codes: Tensor, a_scales: Tensor, a_fmt, b_codes: Tensor, b_scales: Tensor, b_fmt,
+                     bias: Tensor | None, out_dtype: torch.dtype) -> Tensor:
+    """``dequant(A)[M,K] @ dequant(B)[N,K].T + bias`` on packed MXFP operands (``mxfp_pack`` layout)."""
+    _lib.require_device(a_codes, "gemm_mxfp_scaled")
+    lib = _lib.load()
+    M, K = a_codes.shape[0], a_scales.shape[1] * 32
+    N = b_codes.shape[0]
+    assert b_scales.shape[1] * 32 == K and K % MXFP_K_MULTIPLE == 0
+    out = torch.empty((M, N), dtype=out_dtype, device=a_codes.device)
+    if bias is not None:
+        bias = bias.contiguous()
+    rc = lib.mase_gemm_mxfp_scaled(
+        a_codes.data_ptr(), a_scales.data_ptr(), MXFP_HW_FORMATS[tuple(a_fmt)], b_codes.data_ptr(), b_scales.data_ptr(),
+        MXFP_HW_FORMATS[tuple(b_fmt)], bias.data_ptr() if bias is not None else None, out.data_ptr(), M, N, K,
+        _lib.DTYPE_CODE[out_dtype], _lib.DTYPE_CODE[bias.dtype] if bias is not None else 0, _lib.stream_ptr(a_codes),
+    )
+    _lib.check(rc, "mase_gemm_mxfp_scaled")
+    return out

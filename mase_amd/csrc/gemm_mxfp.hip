@@ -1,0 +1,343 @@
+// C[M,N] = A[M,K] * B[N,K]^T (+ bias[N]) with MX-format operands on gfx950's block-scaled matrix instruction
+// v_mfma_scale_f32_32x32x64_f8f6f4: A holds 8-bit codes (e4m3 or e5m2), B holds 8-bit or 4-bit (e2m1) codes,
+// each with one E8M0 scale byte per 32 consecutive K elements, fp32 accumulation.
+//
+// This is the contraction of LinearMXFP.forward for formats the hardware has (the other formats go through
+// the bf16 kernel).  In the instruction lane l supplies the 32 K-elements [32*(l/32), +32) of row/column l%32,
+// which is exactly one MX block, together with that block's scale byte; the hardware multiplies the two
+// scales into the block's partial product, so the result equals the dot product of the dequantized operands.
+//
+// Schedule: the 256x256 tile, 2x2 wavefronts of 4x4 MFMA tiles and the LDS-transposed epilogue are those of the
+// bf16 kernel (gemm_bf16.hip).  K tile 128: per stage A 256 x 128 B, B 256 x 64 B (4-bit) or 256 x 128 B (8-bit),
+// plus 4 scale bytes per row for each operand = one dword per row per K tile.  Three stages when B is 4-bit
+// (50 KB each), two when it is 8-bit (66 KB).  All of it travels HBM/L2 -> LDS with global_load_lds (16-byte
+// form for codes, 4-byte form for scales); copies of tile t+S are issued while the last MFMAs of tile t run.
+// A lane's scale dword is pre-shifted by 8*(l/32) so that K step s finds its byte at position 2s in both
+// half-waves (the byte select of the instruction is an immediate).
+#include "common.hpp"
+
+namespace mase {
+namespace {
+
+typedef int i32x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 256, BN = 256, BK = 128;
+constexpr int kThreadsG = 256;
+
+struct MxGemmParams {
+  const unsigned char* A;
+  const unsigned char* B;
+  const unsigned char* SA;
+  const unsigned char* SB;
+  const void* bias;
+  void* C;
+  int M, N, K;
+  int bias_dtype;
+  int tiles_m, tiles_n;
+};
+
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_n() {
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8) | ((N >> 4) << 14));
+}
+
+__device__ __forceinline__ float load_bias_v(const void* bias, int dt, int col) {
+  if (dt == MASE_DT_F32) return ((const float*)bias)[col];
+  if (dt == MASE_DT_BF16) return bits2f((uint32_t)((const uint16_t*)bias)[col] << 16);
+  return f16_bits_to_f32(((const uint16_t*)bias)[col]);
+}
+
+// LDS offset of 16-byte chunk `chunk` of row `row` for rows of RB bytes (64 or 128); conflict-free for
+// ds_read_b128 on a 64-bank LDS that serves 16 lanes at a time (see gemm_bf16.hip)
+template <int RB>
+__device__ __forceinline__ int lds_off(int row, int chunk) {
+  if constexpr (RB == 128) return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4);
+  else return row * 64 + ((chunk ^ ((row >> 2) & 3)) << 4);
+}
+
+template <int B_BITS, int CBSZ, int BLGP, int OUT_DT>
+__global__ __launch_bounds__(kThreadsG) void gemm_mxfp_kernel(MxGemmParams p) {
+  constexpr int RA = BK;               // bytes per A row per K tile (8-bit codes)
+  constexpr int RB = BK * B_BITS / 8;  // bytes per B row per K tile
+  constexpr int kTileA = BM * RA, kTileB = BN * RB;
+  constexpr int kStage = kTileA + kTileB + 2 * 1024;  // + one scale dword per row for A and for B
+  constexpr int S = (kStage <= 53 * 1024) ? 3 : 2;
+  constexpr int kCopiesA = kTileA / 1024 / 4;          // 16-byte copies per wavefront per tile
+  constexpr int kCopiesB = kTileB / 1024 / 4;
+  constexpr int kCopies = kCopiesA + kCopiesB + 2;     // + one 4-byte copy each for the A and B scales
+  constexpr int kChunksB = RB / 64;                    // 16-byte chunks of B per lane per K step: 2 (8-bit) or 1 (4-bit)
+  constexpr int kReads = 8 + 4 * kChunksB;             // ds_read_b128 per K step
+
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+
+  int bid = blockIdx.x;
+  const int total = p.tiles_m * p.tiles_n;
+  if ((total & 7) == 0) bid = (bid & 7) * (total >> 3) + (bid >> 3);
+  constexpr int GROUP_M = 4;
+  const int in_group = GROUP_M * p.tiles_n;
+  const int first_m = (bid / in_group) * GROUP_M;
+  const int gsz = min(p.tiles_m - first_m, GROUP_M);
+  const int tile_m = first_m + (bid % in_group) % gsz;
+  const int tile_n = (bid % in_group) / gsz;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int nk = p.K / BK;
+
+  // ---- global side of the async copies
+  const size_t lda = (size_t)p.K;                 // bytes per A row
+  const size_t ldbb = (size_t)p.K * B_BITS / 8;   // bytes per B row
+  const size_t lds_sc = (size_t)p.K / 32;         // scale bytes per row
+  const unsigned char* ga[kCopiesA];
+  const unsigned char* gb[kCopiesB];
+#pragma unroll
+  for (int j = 0; j < kCopiesA; ++j) {  // 8 rows of 128 B per copy
+    const int r = (wave + 4 * j) * 8 + (lane >> 3);
+    ga[j] = p.A + (size_t)min(m0 + r, p.M - 1) * lda + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
+  }
+#pragma unroll
+  for (int j = 0; j < kCopiesB; ++j) {
+    if constexpr (RB == 128) {
+      const int r = (wave + 4 * j) * 8 + (lane >> 3);
+      gb[j] = p.B + (size_t)min(n0 + r, p.N - 1) * ldbb + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
+    } else {  // 16 rows of 64 B per copy
+      const int r = (wave + 4 * j) * 16 + (lane >> 2);
+      gb[j] = p.B + (size_t)min(n0 + r, p.N - 1) * ldbb + (((lane & 3) ^ ((r >> 2) & 3)) << 4);
+    }
+  }
+  // scales: wave w copies the dwords of rows [64w, 64w+64) of each operand
+  const unsigned char* gsa = p.SA + (size_t)min(m0 + wave * 64 + lane, p.M - 1) * lds_sc;
+  const unsigned char* gsb = p.SB + (size_t)min(n0 + wave * 64 + lane, p.N - 1) * lds_sc;
+
+  auto issue_copy = [&](int kt, int c) {
+    unsigned char* st = lds + (kt % S) * kStage;
+    const int ktc = min(kt, nk - 1);
+    if (c < kCopiesA) {
+      __builtin_amdgcn_global_load_lds((gptr_t)(ga[c] + (size_t)ktc * RA), (lptr_t)(st + (wave + 4 * c) * 1024), 16, 0, 0);
+    } else if (c < kCopiesA + kCopiesB) {
+      const int j = c - kCopiesA;
+      __builtin_amdgcn_global_load_lds((gptr_t)(gb[j] + (size_t)ktc * RB), (lptr_t)(st + kTileA + (wave + 4 * j) * 1024), 16, 0, 0);
+    } else if (c == kCopiesA + kCopiesB) {
+      __builtin_amdgcn_global_load_lds((gptr_t)(gsa + (size_t)ktc * 4), (lptr_t)(st + kTileA + kTileB + wave * 256), 4, 0, 0);
+    } else {
+      __builtin_amdgcn_global_load_lds((gptr_t)(gsb + (size_t)ktc * 4), (lptr_t)(st + kTileA + kTileB + 1024 + wave * 256), 4, 0, 0);
+    }
+  };
+
+  f32x16_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+#pragma unroll
+  for (int t = 0; t < S; ++t)
+#pragma unroll
+    for (int c = 0; c < kCopies; ++c) issue_copy(t, c);
+
+  const int frag_row = lane & 31;
+  const int kgrp = lane >> 5;
+  // Fragment registers of one K step: A row tile i -> fa[i] (8 dwords), B column tile j -> fb[j] (8 dwords, the
+  // upper 4 unused for 4-bit codes).  Read number q of a step: q < 8 -> 16-byte half (q&1) of A tile q>>1;
+  // then the B chunks.
+  uint4 fa[2][4][2], fb[2][4][2];
+  auto load_part = [&](int kt, int s, int set, int q) {
+    const unsigned char* st = lds + (kt % S) * kStage;
+    if (q < 8) {
+      const int i = q >> 1, h = q & 1;
+      fa[set][i][h] = *(const uint4*)(st + (wm * 128) * RA + lds_off<RA>(i * 32 + frag_row, s * 4 + h * 2 + kgrp));
+    } else {
+      const int qq = q - 8;
+      const int j = qq / kChunksB, h = qq % kChunksB;
+      fb[set][j][h] = *(const uint4*)(st + kTileA + (wn * 128) * RB +
+                                      lds_off<RB>(j * 32 + frag_row, kChunksB == 2 ? s * 4 + h * 2 + kgrp : s * 2 + kgrp));
+    }
+  };
+  // scale dwords of the current tile (sa/sb) and of the next one (san/sbn), pre-shifted so that K step s
+  // uses byte 2s
+  int sa[4], sb[4], san[4], sbn[4];
+  auto load_scales = [&](int kt, int* a, int* b) {
+    const unsigned char* st = lds + (kt % S) * kStage + kTileA + kTileB;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      a[i] = (int)(*(const uint32_t*)(st + (wm * 128 + i * 32 + frag_row) * 4) >> (8 * kgrp));
+      b[i] = (int)(*(const uint32_t*)(st + 1024 + (wn * 128 + i * 32 + frag_row) * 4) >> (8 * kgrp));
+    }
+  };
+  auto mfma = [&](int set, int s, int t) {
+    const int i = t >> 2, j = t & 3;
+    i32x8_t a, b;
+    a[0] = (int)fa[set][i][0].x; a[1] = (int)fa[set][i][0].y; a[2] = (int)fa[set][i][0].z; a[3] = (int)fa[set][i][0].w;
+    a[4] = (int)fa[set][i][1].x; a[5] = (int)fa[set][i][1].y; a[6] = (int)fa[set][i][1].z; a[7] = (int)fa[set][i][1].w;
+    b[0] = (int)fb[set][j][0].x; b[1] = (int)fb[set][j][0].y; b[2] = (int)fb[set][j][0].z; b[3] = (int)fb[set][j][0].w;
+    if constexpr (kChunksB == 2) {
+      b[4] = (int)fb[set][j][1].x; b[5] = (int)fb[set][j][1].y; b[6] = (int)fb[set][j][1].z; b[7] = (int)fb[set][j][1].w;
+    } else {
+      b[4] = 0; b[5] = 0; b[6] = 0; b[7] = 0;
+    }
+    if (s == 0)
+      acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], CBSZ, BLGP, 0, sa[i], 0, sb[j]);
+    else
+      acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], CBSZ, BLGP, 2, sa[i], 2, sb[j]);
+  };
+
+  // Pipeline (see gemm_bf16.hip for the reasoning): per K tile two steps of 16 MFMAs; fragment sets ping-pong.
+  //   step 0: MFMAs on set 0, interleaved with the LDS reads of step 1 (set 1)
+  //   hand-over: own LDS reads done (lgkmcnt), own copies of tile kt+1 landed (vmcnt), barrier
+  //   step 1: MFMAs on set 1, interleaved with the LDS reads of step 0 and the scales of tile kt+1 and with
+  //           the copies of tile kt+S into the stage tile kt just vacated
+  constexpr int kCopiesPerSlot = (kCopies + 15) / 16;
+  wait_vmcnt_n<(S - 1) * kCopies>();  // tile 0 landed; the other stages may still be filling
+  asm volatile("s_barrier" ::: "memory");
+#pragma unroll
+  for (int q = 0; q < kReads; ++q) load_part(0, 0, 0, q);
+  load_scales(0, sa, sb);
+  for (int kt = 0; kt < nk; ++kt) {
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      mfma(0, 0, t);
+      if (t < kReads) load_part(kt, 1, 1, t);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    wait_vmcnt_n<(S - 2) * kCopies>();  // tiles kt+1 .. kt+S-1 are in flight; kt+1 must have landed
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      mfma(1, 1, t);
+      if (t < kReads) load_part(kt + 1, 0, 0, t);
+      if (t == 12) load_scales(kt + 1, san, sbn);
+#pragma unroll
+      for (int c = t * kCopiesPerSlot; c < (t + 1) * kCopiesPerSlot; ++c)
+        if (c < kCopies) issue_copy(kt + S, c);  // into the stage tile kt just vacated
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { sa[i] = san[i]; sb[i] = sbn[i]; }
+  }
+  wait_vmcnt_n<0>();
+
+  // ---- epilogue (as in gemm_bf16.hip): transpose 32-row bands through LDS, 4 consecutive columns per lane
+  asm volatile("s_barrier" ::: "memory");
+  constexpr int kStgStride = 136;
+  float* stg = (float*)(lds + wave * (32 * kStgStride * 4));
+  const int c4 = (lane & 31) * 4;
+  const int col0 = n0 + wn * 128 + c4;
+  const bool vec_ok = ((p.N & 3) == 0) && ((((uintptr_t)p.C) & 15u) == 0);
+  float bv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (p.bias != nullptr) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (col0 + e < p.N) bv[e] = load_bias_v(p.bias, p.bias_dtype, col0 + e);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        stg[((r >> 2) * 8 + kgrp * 4 + (r & 3)) * kStgStride + j * 32 + frag_row] = acc[i][j][r];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const int rr = q * 2 + kgrp;
+      const int row = m0 + wm * 128 + i * 32 + rr;
+      const float4 v4 = *(const float4*)(stg + rr * kStgStride + c4);
+      const float v[4] = {v4.x + bv[0], v4.y + bv[1], v4.z + bv[2], v4.w + bv[3]};
+      if (row >= p.M) continue;
+      const size_t o = (size_t)row * p.N + col0;
+      if (vec_ok && col0 + 3 < p.N) {
+        if constexpr (OUT_DT == MASE_DT_F32) {
+          *(float4*)((float*)p.C + o) = make_float4(v[0], v[1], v[2], v[3]);
+        } else if constexpr (OUT_DT == MASE_DT_BF16) {
+          uint2 w;
+          w.x = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
+          w.y = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
+          *(uint2*)((uint16_t*)p.C + o) = w;
+        } else {
+          uint2 w;
+          w.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
+          w.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
+          *(uint2*)((uint16_t*)p.C + o) = w;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (col0 + e >= p.N) continue;
+          if constexpr (OUT_DT == MASE_DT_F32) ((float*)p.C)[o + e] = v[e];
+          else if constexpr (OUT_DT == MASE_DT_BF16) ((uint16_t*)p.C)[o + e] = (uint16_t)f32_to_bf16_bits(v[e]);
+          else ((uint16_t*)p.C)[o + e] = (uint16_t)f32_to_f16_bits(v[e]);
+        }
+      }
+    }
+  }
+}
+
+template <int B_BITS, int CBSZ, int BLGP>
+int launch_mx_gemm(const MxGemmParams& p, int out_dtype, hipStream_t st) {
+  constexpr int kStage = BM * BK + BN * BK * B_BITS / 8 + 2048;
+  constexpr int S = (kStage <= 53 * 1024) ? 3 : 2;
+  const size_t lds_bytes = (size_t)S * kStage;
+  const void* kernels[3] = {(const void*)gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, MASE_DT_F32>,
+                            (const void*)gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, MASE_DT_BF16>,
+                            (const void*)gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, MASE_DT_F16>};
+  static bool attr_set = false;
+  if (!attr_set) {
+    for (const void* k : kernels)
+      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
+        return MASE_ERR_LAUNCH;
+    attr_set = true;
+  }
+  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kThreadsG);
+  if (out_dtype == MASE_DT_F32)
+    hipLaunchKernelGGL((gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, MASE_DT_F32>), grid, block, lds_bytes, st, p);
+  else if (out_dtype == MASE_DT_BF16)
+    hipLaunchKernelGGL((gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, MASE_DT_BF16>), grid, block, lds_bytes, st, p);
+  else
+    hipLaunchKernelGGL((gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, MASE_DT_F16>), grid, block, lds_bytes, st, p);
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+}  // namespace
+}  // namespace mase
+
+// a_format / b_format: 0 = e4m3 (8-bit), 1 = e5m2 (8-bit), 4 = e2m1 (4-bit, two codes per byte); A must be 8-bit.
+extern "C" int mase_gemm_mxfp_scaled(const void* A, const void* A_scales, int a_format, const void* B,
+                                     const void* B_scales, int b_format, const void* bias, void* C, size_t M, size_t N,
+                                     size_t K, int out_dtype, int bias_dtype, void* stream) {
+  using namespace mase;
+  if (M == 0 || N == 0) return MASE_OK;
+  if (A == nullptr || B == nullptr || A_scales == nullptr || B_scales == nullptr || C == nullptr) return MASE_ERR_NULL;
+  if (K == 0 || (K % BK) != 0 || M > (1u << 30) || N > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
+  if (!aligned16(A) || !aligned16(B) || (((uintptr_t)A_scales) & 3u) != 0 || (((uintptr_t)B_scales) & 3u) != 0)
+    return MASE_ERR_ALIGN;
+  if (out_dtype < 0 || out_dtype > 2 || (bias != nullptr && (bias_dtype < 0 || bias_dtype > 2))) return MASE_ERR_DTYPE;
+  if ((a_format != 0 && a_format != 1) || (b_format != 0 && b_format != 1 && b_format != 4)) return MASE_ERR_PARAM;
+  MxGemmParams p;
+  p.A = (const unsigned char*)A;
+  p.B = (const unsigned char*)B;
+  p.SA = (const unsigned char*)A_scales;
+  p.SB = (const unsigned char*)B_scales;
+  p.bias = bias;
+  p.C = C;
+  p.M = (int)M;
+  p.N = (int)N;
+  p.K = (int)K;
+  p.bias_dtype = bias_dtype;
+  p.tiles_m = (int)((M + BM - 1) / BM);
+  p.tiles_n = (int)((N + BN - 1) / BN);
+  hipStream_t st = (hipStream_t)stream;
+  if (a_format == 0 && b_format == 4) return launch_mx_gemm<4, 0, 4>(p, out_dtype, st);
+  if (a_format == 1 && b_format == 4) return launch_mx_gemm<4, 1, 4>(p, out_dtype, st);
+  if (a_format == 0 && b_format == 0) return launch_mx_gemm<8, 0, 0>(p, out_dtype, st);
+  if (a_format == 0 && b_format == 1) return launch_mx_gemm<8, 0, 1>(p, out_dtype, st);
+  if (a_format == 1 && b_format == 0) return launch_mx_gemm<8, 1, 0>(p, out_dtype, st);
+  return launch_mx_gemm<8, 1, 1>(p, out_dtype, st);
+}

@@ -180,6 +180,112 @@ int launch_mxfp(const void* in, void* out, uint8_t* codes, uint8_t* scales, size
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Packing for the block-scaled matrix instructions (v_mfma_scale_f32_*_f8f6f4).
+//
+// Codes and scales are first computed exactly as above (so they decode to the reference's values), then
+// adapted to what the hardware formats can express: the reference's element formats are "all finite" (the top
+// exponent field holds ordinary values), whereas OCP e4m3 reserves S.1111.111 for NaN and e5m2 reserves the
+// whole top exponent field.  A block that uses such a code is re-expressed with the next scale (scale + 1)
+// and every element halved: exact for elements with exponent field >= 2, round-to-nearest-even into the
+// subnormal range below that (error <= 2^-10 of an element unit while the block maximum is >= 2^8 units).
+// 8-bit codes are stored one per byte, 4-bit codes two per byte (even element in the low nibble).
+// ---------------------------------------------------------------------------------------------
+template <int E, int F>
+__device__ __forceinline__ uint32_t halve_code(uint32_t c) {
+  const uint32_t sgn = c & (1u << (E + F));
+  uint32_t e = (c >> F) & ((1u << E) - 1u);
+  uint32_t f = c & ((1u << F) - 1u);
+  if (e >= 2) {
+    e -= 1;
+  } else {
+    uint32_t v = (e == 1) ? ((1u << F) + f) : f;
+    uint32_t q = (v >> 1) + ((v & 1u) & ((v >> 1) & 1u));  // round half to even
+    if (q == (1u << F)) { e = 1; f = 0; }
+    else { e = 0; f = q; }
+  }
+  return sgn | (e << F) | f;
+}
+
+template <int E, int F>
+__device__ __forceinline__ bool code_is_reserved(uint32_t c) {
+  const uint32_t e = (c >> F) & ((1u << E) - 1u);
+  const uint32_t f = c & ((1u << F) - 1u);
+  if constexpr (E == 4 && F == 3) return e == 15u && f == 7u;  // OCP e4m3: NaN
+  if constexpr (E == 5 && F == 2) return e == 31u;             // OCP e5m2: Inf / NaN
+  return false;
+}
+
+template <int DTI, int E, int F>
+__global__ __launch_bounds__(64) void mxfp_pack_kernel(const void* __restrict__ in, uint8_t* __restrict__ codes,
+                                                       uint8_t* __restrict__ scales, size_t n8, MxfpParams p) {
+  using TI = DTypeTraits<DTI>;
+  const size_t idx = (size_t)blockIdx.x * 64 + threadIdx.x;  // 8 elements per lane, 4 lanes per block of 32
+  const bool live = idx < n8;
+  WaveLog2 meta;
+  meta.init(p.tab, kLog2TabHalf);
+  float x[8];
+  if (live) {
+    if constexpr (TI::kVec == 8) {
+      TI::unpack(load_nt((const uint4*)in + idx), x);
+    } else {
+      TI::unpack(load_nt((const uint4*)in + 2 * idx), x);
+      TI::unpack(load_nt((const uint4*)in + 2 * idx + 1), x + 4);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] = 0.0f;
+  }
+  uint32_t m = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    x[j] = flush_subnormal(x[j]);
+    m = max(m, f2bits(x[j]) & 0x7FFFFFFFu);
+  }
+  m = group_max_u32<4>(m);
+  int sh = 0;
+  const int state = mxfp_block_scale(m, p, sh, meta);
+  uint32_t c[8];
+  uint32_t reserved = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    mxfp_element(x[j], state, sh, p, c[j]);
+    reserved |= code_is_reserved<E, F>(c[j]) ? 1u : 0u;
+  }
+  reserved = group_max_u32<4>(reserved);
+  int sb = (state == 1) ? sh + 127 : (state == 0 ? 0 : 255);
+  if (reserved && state == 1) {
+    sb = min(sb + 1, 254);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) c[j] = halve_code<E, F>(c[j]);
+  }
+  if (!live) return;
+  if ((idx & 3) == 0) scales[idx >> 2] = (uint8_t)sb;
+  if constexpr (E + F + 1 <= 4) {
+    uint32_t w = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) w |= (c[j] & 0xFu) << (4 * j);
+    ((uint32_t*)codes)[idx] = w;
+  } else {
+    uint2 w;
+    w.x = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+    w.y = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
+    ((uint2*)codes)[idx] = w;
+  }
+}
+
+template <int DTI>
+int launch_mxfp_pack(const void* in, uint8_t* codes, uint8_t* scales, size_t numel, int E, int F, const MxfpParams& p,
+                     hipStream_t st) {
+  const size_t n8 = numel / 8;
+  const dim3 grid(blocks_for(n8, 64)), block(64);
+  if (E == 4 && F == 3) hipLaunchKernelGGL((mxfp_pack_kernel<DTI, 4, 3>), grid, block, 0, st, in, codes, scales, n8, p);
+  else if (E == 5 && F == 2) hipLaunchKernelGGL((mxfp_pack_kernel<DTI, 5, 2>), grid, block, 0, st, in, codes, scales, n8, p);
+  else if (E == 2 && F == 1) hipLaunchKernelGGL((mxfp_pack_kernel<DTI, 2, 1>), grid, block, 0, st, in, codes, scales, n8, p);
+  else return MASE_ERR_PARAM;
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
 template <int DTI>
 int launch_mxfp_out(int out_dtype, const void* in, void* out, uint8_t* codes, uint8_t* scales, size_t numel, int B,
                     const MxfpParams& p, hipStream_t st) {
@@ -222,6 +328,34 @@ extern "C" int mase_mxfp_qdq(const void* in, void* out, uint8_t* codes, uint8_t*
     case MASE_DT_F32: return launch_mxfp_out<MASE_DT_F32>(out_dtype, in, out, codes, scales, numel, block_size, p, st);
     case MASE_DT_BF16: return launch_mxfp_out<MASE_DT_BF16>(out_dtype, in, out, codes, scales, numel, block_size, p, st);
     case MASE_DT_F16: return launch_mxfp_out<MASE_DT_F16>(out_dtype, in, out, codes, scales, numel, block_size, p, st);
+    default: return MASE_ERR_DTYPE;
+  }
+}
+
+extern "C" int mase_mxfp_pack(const void* in, uint8_t* codes, uint8_t* scales, size_t numel, int in_dtype, int exp_bits,
+                              int frac_bits, const uint32_t* log2_tab, void* stream) {
+  using namespace mase;
+  if (numel == 0) return MASE_OK;
+  if (in == nullptr || codes == nullptr || scales == nullptr || log2_tab == nullptr) return MASE_ERR_NULL;
+  if (numel % 32 != 0) return MASE_ERR_SHAPE;
+  if (!aligned16(in) || (((uintptr_t)codes) & 7u) != 0) return MASE_ERR_ALIGN;
+  if (!((exp_bits == 4 && frac_bits == 3) || (exp_bits == 5 && frac_bits == 2) || (exp_bits == 2 && frac_bits == 1)))
+    return MASE_ERR_PARAM;
+  MxfpParams p;
+  p.m.E = exp_bits;
+  p.m.F = frac_bits;
+  p.m.bias = (1 << (exp_bits - 1)) - 1;
+  p.m.e_hi = (1 << exp_bits) - 1;
+  p.m.frac_hi = (1 << frac_bits) - 1;
+  p.m.is_finite = 1;
+  p.m.round_mode = 0;
+  p.el_emax = p.m.e_hi - p.m.bias;
+  p.tab = log2_tab;
+  hipStream_t st = (hipStream_t)stream;
+  switch (in_dtype) {
+    case MASE_DT_F32: return launch_mxfp_pack<MASE_DT_F32>(in, codes, scales, numel, exp_bits, frac_bits, p, st);
+    case MASE_DT_BF16: return launch_mxfp_pack<MASE_DT_BF16>(in, codes, scales, numel, exp_bits, frac_bits, p, st);
+    case MASE_DT_F16: return launch_mxfp_pack<MASE_DT_F16>(in, codes, scales, numel, exp_bits, frac_bits, p, st);
     default: return MASE_ERR_DTYPE;
   }
 }

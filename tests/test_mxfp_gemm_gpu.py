@@ -1,0 +1,103 @@
+"""GPU tests of the packed-MXFP path: the packer against the oracle quantizer, and the block-scaled MFMA
+contraction against an fp64 product of the decoded operands."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from helpers import adversarial
+
+pytestmark = pytest.mark.gpu
+
+
+def decode_ocp(codes: torch.Tensor, scales: torch.Tensor, fmt):
+    """packed hardware codes + E8M0 scales -> float64 values, decoded per the OCP MX formats"""
+    E, F = fmt
+    c = codes.cpu().to(torch.int64)
+    if E + F + 1 <= 4:
+        c = torch.stack([c & 0xF, c >> 4], dim=-1).reshape(*c.shape[:-1], -1)
+    bias = (1 << (E - 1)) - 1
+    sgn = (c >> (E + F)) & 1
+    e = (c >> F) & ((1 << E) - 1)
+    f = c & ((1 << F) - 1)
+    mag = torch.where(e == 0, f.double() / (1 << F) * 2.0 ** (1 - bias), (1 + f.double() / (1 << F)) * torch.exp2((e - bias).double()))
+    if (E, F) == (4, 3):
+        assert not bool(((e == 15) & (f == 7)).any()), "packed e4m3 must not contain the NaN code"
+    if (E, F) == (5, 2):
+        assert not bool((e == 31).any()), "packed e5m2 must not contain Inf/NaN codes"
+    v = torch.where(sgn == 1, -mag, mag)
+    s = torch.exp2(scales.cpu().double() - 127).repeat_interleave(32, dim=-1)
+    return v * s
+
+
+@pytest.mark.parametrize("fmt", [(4, 3), (5, 2), (2, 1)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_mxfp_pack_decodes_to_the_quantizer_output(dev, fmt, dtype):
+    from mase_amd._gemm import mxfp_pack
+
+    rng = np.random.default_rng(fmt[0] * 4 + fmt[1])
+    x = adversarial(rng, (64, 512), dtype, block=32)
+    x = torch.where(x.float().abs() < 1e20, x, torch.zeros_like(x))
+    x[3, :32] = torch.linspace(-1, 1, 32).to(dtype) * 479.0 / 256  # a block whose maximum rounds to the top e4m3 code
+    want = O.mxfp_quantizer(x.float(), 32, fmt[0], fmt[1]).double()
+    codes, scales = mxfp_pack(x.to(dev), *fmt)
+    got = decode_ocp(codes, scales, fmt)
+    blk_max = want.abs().reshape(64, -1, 32).amax(-1, keepdim=True).repeat_interleave(32, -1).reshape(64, 512)
+    diff = (got - want).abs()
+    # exact except in blocks re-expressed with the next scale, where elements far below the block maximum
+    # are rounded into the format's subnormal range
+    assert float((diff / blk_max.clamp_min(1e-300)).max()) <= 2.0 ** -9
+    exact = float((diff == 0).double().mean())
+    print(f"pack e{fmt[0]}m{fmt[1]} {dtype}: {exact:.4f} of elements exact")
+    assert exact > (0.97 if fmt != (5, 2) else 0.5)
+    assert bool(((got == 0) == (want == 0)).all()) or fmt == (5, 2)
+
+
+@pytest.mark.parametrize("bfmt", [(2, 1), (4, 3), (5, 2)])
+@pytest.mark.parametrize("afmt", [(4, 3), (5, 2)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 200, 384), (512, 768, 1024), (1, 33, 256)])
+def test_gemm_mxfp_scaled_against_decoded_operands(dev, afmt, bfmt, M, N, K):
+    from mase_amd._gemm import gemm_mxfp_scaled, mxfp_pack
+
+    g = torch.Generator().manual_seed(M + N + K)
+    a = torch.randn(M, K, generator=g)
+    a[:, 5] *= 20
+    b = torch.randn(N, K, generator=g) * 0.02
+    bias = torch.randn(N, generator=g)
+    print(f"mxfp gemm {afmt}x{bfmt} M={M} N={N} K={K}", flush=True)
+    ac, asc = mxfp_pack(a.to(dev), *afmt)
+    bc, bsc = mxfp_pack(b.to(dev), *bfmt)
+    da, db = decode_ocp(ac, asc, afmt), decode_ocp(bc, bsc, bfmt)
+    ref = da @ db.t()
+    # The instruction adds the 8 products of one register pair after aligning them to the largest of the 8
+    # and dropping what lies more than about 12 bits below its leading bit (measured: e4m3 x e2m1 keeps a
+    # granularity of 2^-12 of that product); sums across such groups and across instructions are fp32.
+    # Hence |error| <= 7 * 2^-12 * sum|a_k b_k| in the worst case; typical errors are ~1e-5 of the result.
+    bound = (da.abs() @ db.abs().t()) * 2.0 ** -9 + ref.abs() * 2.0 ** -21
+    y = gemm_mxfp_scaled(ac, asc, afmt, bc, bsc, bfmt, None, torch.float32)
+    d = (y.cpu().double() - ref).abs()
+    assert bool((d <= bound).all()), float((d / bound).max())
+    err = float(d.max() / ref.abs().max())
+    print(f"  max |err| / max |ref| = {err:.2e}")
+    assert err < 5e-4, err
+    yb = gemm_mxfp_scaled(ac, asc, afmt, bc, bsc, bfmt, bias.to(dev), torch.bfloat16)
+    want = ref + bias.double()
+    d = (yb.cpu().double() - want).abs()
+    assert bool((d <= want.abs() * 2.0 ** -8 + ref.abs().max() * 5e-4).all())  # bf16 rounding of the output
+
+
+def test_gemm_mxfp_exact_small_integers(dev):
+    """e2m1 x e4m3 with unit scales and values that both formats hold exactly: every product is a multiple of 32
+    below 2^11, so neither the 12-bit alignment inside the instruction nor fp32 accumulation rounds anything"""
+    from mase_amd._gemm import gemm_mxfp_scaled, mxfp_pack
+
+    g = torch.Generator().manual_seed(1)
+    a = torch.randint(-8, 9, (256, 256), generator=g).float() * 32   # multiples of 32 up to 256: exact in e4m3
+    a[:, ::32] = 256.0  # pins every block's scale
+    b = torch.tensor([0, 1, 1.5, 2, 3, 4, 6, 6])[torch.randint(0, 8, (256, 256), generator=g)] * torch.where(torch.rand(256, 256, generator=g) < 0.5, -1.0, 1.0)
+    b[:, ::32] = 6.0
+    ac, asc = mxfp_pack(a.to(dev), 4, 3)
+    bc, bsc = mxfp_pack(b.to(dev), 2, 1)
+    assert torch.equal(decode_ocp(ac, asc, (4, 3)), a.double()) and torch.equal(decode_ocp(bc, bsc, (2, 1)), b.double())
+    y = gemm_mxfp_scaled(ac, asc, (4, 3), bc, bsc, (2, 1), None, torch.float32)
+    assert torch.equal(y.cpu().double(), a.double() @ b.double().t())
