@@ -11,7 +11,7 @@ import torch
 from torch import Tensor
 from torch.nn import functional as F
 
-from ..._gemm import gemm_bf16_tn
+from ..._gemm import MXFP_HW_FORMATS, MXFP_K_MULTIPLE, gemm_bf16_tn, gemm_mxfp_scaled, mxfp_pack
 
 
 class WeightCache:
@@ -60,3 +60,58 @@ def mx_linear(x: Tensor, weight: Tensor, bias: Tensor | None, quantize_to_bf16, 
     xq = quantize_to_bf16(x2)
     y = gemm_bf16_tn(xq, wb, bias, x.dtype)
     return y.reshape(*lead, weight.shape[0])
+
+
+def _weight_key(weight: Tensor):
+    return (weight.data_ptr(), weight._version, weight.dtype, weight.device, tuple(weight.shape))
+
+
+class PackedMXFPWeight:
+    """Hardware image (element codes + E8M0 block scales) of an MXFP-quantized weight for the block-scaled
+    matrix instruction.
+
+    It is packed from the *unquantized* weight when a state dict is loaded (packing the quantized weight again
+    could pick a different block scale) and is valid only while the parameter is the tensor that load produced:
+    the same identity/version test as ``WeightCache``.  The packed values equal the reference's quantized
+    weight except in blocks whose largest element takes the format's top code, which the hardware reserves
+    for NaN/Inf (e4m3 0x7F, e5m2 exponent 31): those blocks are stored with the next scale and halved codes,
+    which only rounds elements more than 2^9 below the block maximum.  e2m1 has no reserved code and is exact.
+    """
+
+    def __init__(self):
+        self._key = None
+        self.codes = None
+        self.scales = None
+        self.fmt = None
+
+    def invalidate(self):
+        self._key = None
+        self.codes = self.scales = self.fmt = None
+
+    @staticmethod
+    def eligible(weight: Tensor, block_size: int, fmt) -> bool:
+        return (weight.is_cuda and weight.dim() == 2 and block_size == 32 and tuple(fmt) in MXFP_HW_FORMATS
+                and weight.shape[1] % MXFP_K_MULTIPLE == 0
+                and weight.dtype in (torch.float32, torch.bfloat16, torch.float16))
+
+    def pack(self, weight: Tensor, fmt):
+        self.codes, self.scales = mxfp_pack(weight.detach(), *fmt)
+        self.fmt = tuple(fmt)
+
+    def bind(self, weight: Tensor):
+        """declare the image current for ``weight`` as it is now (after its in-place quantization)"""
+        self._key = _weight_key(weight)
+
+    def valid_for(self, weight: Tensor) -> bool:
+        return self.codes is not None and self._key == _weight_key(weight)
+
+
+def mxfp_linear_native(x: Tensor, packed: PackedMXFPWeight, bias: Tensor | None, act_fmt) -> Tensor:
+    """``F.linear(q(x), W, b)`` on the block-scaled matrix instruction: the activations are quantized straight to
+    element codes + scales (one pass over x, 1.03 bytes written per element) and contracted with the packed
+    weight; accumulation is fp32 and the result is written in x's dtype."""
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, x.shape[-1])
+    xc, xs = mxfp_pack(x2, *act_fmt)
+    y = gemm_mxfp_scaled(xc, xs, act_fmt, packed.codes, packed.scales, packed.fmt, bias, x.dtype)
+    return y.reshape(*lead, packed.codes.shape[0])

@@ -10,7 +10,7 @@ from torch.nn import functional as F
 
 from ...quantizers import _ops, mxfp_quantizer, mxint_quantizer
 from ..functional.linear import linearBlockFP, linearInteger, linearMinifloatDenorm, linearMinifloatIEEE
-from ..functional.mx_linear import WeightCache, mx_linear
+from ..functional.mx_linear import PackedMXFPWeight, WeightCache, mx_linear, mxfp_linear_native
 
 
 class _LinearBase(torch.nn.Linear):
@@ -89,11 +89,19 @@ class _LinearMX(_LinearBase):
     def load_state_dict(self, state_dict, strict=True, assign=False):
         """Load pretrained weights, then quantize them in place."""
         result = super().load_state_dict(state_dict, strict=strict, assign=assign)
+        self._w_cache.invalidate()
         if self.bypass or self.gptq:
             return result
+        self._before_quantize_params()
         self._quantize_params()
-        self._w_cache.invalidate()
+        self._after_quantize_params()
         return result
+
+    def _before_quantize_params(self):
+        pass
+
+    def _after_quantize_params(self):
+        pass
 
 
 class LinearMXInt(_LinearMX):
@@ -128,6 +136,33 @@ class LinearMXInt(_LinearMX):
 
 
 class LinearMXFP(_LinearMX):
+    """``config["native_mx"]`` (default True; not a key of the reference) lets the forward use the block-scaled
+    matrix instruction when activations are e4m3/e5m2, weights e4m3/e5m2/e2m1, both block sizes are 32 and
+    in_features is a multiple of 128; otherwise, or with ``native_mx=False``, the contraction runs in bf16 on the
+    dequantized operands."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, dtype=None,
+                 config=None) -> None:
+        super().__init__(in_features, out_features, bias, device, dtype, config)
+        self._w_packed = PackedMXFPWeight()
+
+    def invalidate_weight_cache(self):
+        super().invalidate_weight_cache()
+        self._w_packed.invalidate()
+
+    def _weight_fmt(self):
+        return (self.config["weight_exponent_width"], self.config["weight_frac_width"])
+
+    def _before_quantize_params(self):
+        self._w_packed.invalidate()
+        if self.config.get("native_mx", True) and PackedMXFPWeight.eligible(
+                self.weight, self.config["weight_block_size"], self._weight_fmt()):
+            self._w_packed.pack(self.weight.data, self._weight_fmt())
+
+    def _after_quantize_params(self):
+        if self._w_packed.codes is not None:
+            self._w_packed.bind(self.weight)
+
     def _quantize_params(self):
         cfg = self.config
         self.weight.data.copy_(
@@ -153,6 +188,9 @@ class LinearMXFP(_LinearMX):
         fb = self.config.get("data_in_frac_width")
         if bs is None or eb is None:
             return F.linear(x, self.weight, self.bias)
+        if (bs == 32 and (eb, fb) in ((4, 3), (5, 2)) and x.is_cuda and x.dtype == self.weight.dtype
+                and x.numel() > 0 and self._w_packed.valid_for(self.weight)):
+            return mxfp_linear_native(x, self._w_packed, self.bias, (eb, fb))
         return mx_linear(
             x, self.weight, self.bias,
             lambda t: _ops.mxfp_qdq(t, bs, eb, fb, -1, 8, out_dtype=torch.bfloat16),
