@@ -235,7 +235,77 @@ class MxintLinear(Workload):
                 "kind": "port", "sample": f"{n} full forwards (activation quantize-dequantize + fp32 F.linear), {dt*1e3:.0f} ms each"}
 
 
-WORKLOADS = {w.name: w for w in (BfpQdq, MxintQdq, MxintLinear, CopyBytes)}
+class MxfpLinear(Workload):
+    name = "mxfp_linear"
+    metric = ("MXFP8 x MXFP4 Linear forward throughput (2*M*N*K flop per step; activation quantization to packed "
+              "codes included in the step)")
+    unit = "TFLOP/s"
+    dtype = "fp8"
+    bound = "mfma"
+    mfma_dtype = "fp8"
+    kernel = "gemm_mxfp_kernel"
+    M, K, N = 8192, 8192, 28672
+    config = {"workload": "LinearMXFP 8192->28672 (no bias), x bf16 [8192,8192] N(0,1) with 8 of 8192 channels x20, "
+                          "W N(0,0.02); weights e2m1, activations e4m3, block 32, E8M0 scales; block-scaled MFMA, "
+                          "fp32 accumulate, bf16 out; seed 3"}
+    cfg = {"weight_block_size": 32, "weight_exponent_width": 2, "weight_frac_width": 1,
+           "data_in_block_size": 32, "data_in_exponent_width": 4, "data_in_frac_width": 3}
+
+    def make_x(self, torch, rows):
+        g = torch.Generator().manual_seed(3)
+        idx = torch.randperm(self.K, generator=g)[: self.K // 1000]
+        x = torch.randn(rows, self.K, generator=g)
+        x[:, idx] *= 20
+        return x.to(torch.bfloat16)
+
+    def make_w(self, torch, rows):
+        g = torch.Generator().manual_seed(33)
+        return (torch.randn(rows, self.K, generator=g) * 0.02).to(torch.bfloat16)
+
+    def setup(self, torch, dev, n_buffers):
+        from mase_amd.quantized import LinearMXFP
+        from mase_amd._gemm import gemm_mxfp_scaled, mxfp_pack
+
+        self.torch = torch
+        self.m = LinearMXFP(self.K, self.N, bias=False, device=dev, dtype=torch.bfloat16, config=dict(self.cfg))
+        self.m.load_state_dict({"weight": self.make_w(torch, self.N)})
+        assert self.m._w_packed.valid_for(self.m.weight)
+        x = self.make_x(torch, self.M).to(dev)
+        self.bufs = [x.roll(i, dims=0).contiguous() for i in range(max(n_buffers, 2))]
+        self.xc, self.xs = mxfp_pack(self.bufs[0], 4, 3)
+        self._gemm = gemm_mxfp_scaled
+
+    def step(self, i):
+        self.out = self.m(self.bufs[i % len(self.bufs)])
+
+    def dominant_step(self, i):
+        p = self.m._w_packed
+        self.out = self._gemm(self.xc, self.xs, (4, 3), p.codes, p.scales, p.fmt, None, self.torch.bfloat16)
+
+    def work_per_step(self):
+        return 2.0 * self.M * self.N * self.K
+
+    def cpu_baseline(self, torch, budget_s):
+        from oracle import linear as OL
+
+        ms, ns = 1024, 4096  # bounded sample: the first 1024 activation rows against the first 4096 weight rows
+        x = self.make_x(torch, ms)
+        qw, _ = OL.mxfp_prepare_weights(self.make_w(torch, ns), None, self.cfg)
+        OL.linear_mxfp_forward(x[:64], qw, None, self.cfg)
+        t0 = time.perf_counter()
+        n = 0
+        while True:
+            OL.linear_mxfp_forward(x, qw, None, self.cfg)
+            n += 1
+            if time.perf_counter() - t0 > budget_s or n >= 20:
+                break
+        dt = (time.perf_counter() - t0) / n
+        return {"value": 2.0 * ms * ns * self.K / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+                "kind": "port", "sample": f"{n} forwards of a [{ms},{self.K}] x [{ns},{self.K}] slice of the workload "
+                                          f"(activation quantize-dequantize + bf16 F.linear), {dt*1e3:.0f} ms each"}
+
+
+WORKLOADS = {w.name: w for w in (BfpQdq, MxintQdq, MxintLinear, MxfpLinear, CopyBytes)}
 
 
 def load_traffic(name):

@@ -21,7 +21,7 @@ struct MxfpParams {
   const uint32_t* tab;  // fp32 table (floor half is used)
 };
 
-constexpr int kUnroll = 2;
+constexpr int kVecThreads = 64;
 
 // state 0: all flushed, 1: regular (sh valid), 2: NaN block
 template <typename... Meta>
@@ -47,74 +47,110 @@ __device__ __forceinline__ float flush_subnormal(float x) {
   return ((f2bits(x) & 0x7F800000u) == 0) ? 0.0f : x;
 }
 
+// Integer fast path of mxfp_element for an element of a regular block (state 1): the same steps as
+// minifloat_mx_encode / minifloat_mx_decode written on the bit fields of the already flushed fp32 input.
+//   exponent field of t / 2^sh is  ef = exp(t) - sh  (ldexp is exact while ef stays >= 1)
+//   fraction: 23 -> 15 bits by truncation, 15 -> F bits round-half-even; a carry out of the fraction is OR-ed
+//   into the exponent field (lost when that field is odd), exponent field 0 takes the truncating shift
+//   value = code's [exponent|fraction] field moved to fp32's, exponent rebased by sh + 127 - bias
+// Returns false (caller takes mxfp_element) when t / 2^sh leaves the fp32 normal range or the format's
+// exponent range, which only happens for elements more than 2^100 below the block maximum or clamped scales.
+__device__ __forceinline__ bool mxfp_element_fast(uint32_t xb, int sh, const MxfpParams& p, uint32_t& code,
+                                                  uint32_t& ybits) {
+  const int F = p.m.F;
+  const uint32_t ab = xb & 0x7FFFFFFFu;
+  const uint32_t sgn32 = xb & 0x80000000u;
+  const int ef = (int)(ab >> 23) - sh;
+  const int ye = ef - 127 + p.m.bias;
+  const int shn = 15 - F;
+  const uint32_t m15 = (ab >> 8) & 0x7FFFu;
+  const uint32_t yf = (m15 + ((1u << (shn - 1)) - 1u) + ((m15 >> shn) & 1u)) >> shn;  // 0 .. 2^F
+  const uint32_t cn = ((uint32_t)ye << F) | yf;
+  const uint32_t cs = yf ? ((yf | (1u << F)) >> 1) : 0u;
+  uint32_t c = ye > 0 ? cn : (ye == 0 ? cs : 0u);
+  if (ab == 0) c = 0;
+  // decode: normal codes move as a bit field; codes with exponent field 0 are integers times a power of two
+  const uint32_t yn = (c << (23 - F)) + ((uint32_t)(sh + 127 - p.m.bias) << 23);
+  const uint32_t ys = f2bits(ldexpf((float)c, 1 - p.m.bias - F + sh));
+  ybits = sgn32 | ((c >> F) != 0 ? yn : ys);
+  code = c | (sgn32 >> (31 - p.m.E - F));
+  return (ab == 0) || (ef > 0 && ye <= p.m.e_hi);
+}
+
+// one element of a block in any state: fast path when it applies, else the step-by-step functions
+__device__ __forceinline__ uint32_t mxfp_element_bits(float t, int state, int sh, const MxfpParams& p, uint32_t& code) {
+  uint32_t yb;
+  const bool ok = mxfp_element_fast(f2bits(t), sh, p, code, yb);
+  if (__builtin_expect(state != 1 || !ok, 0)) yb = f2bits(mxfp_element(t, state, sh, p, code));
+  return yb;
+}
+
+// One 16-byte vector of the wider side per lane, 64-lane work-groups (the shape that streams best on this
+// part); a block of B elements spans LPB lanes, or a lane holds SUB blocks.  No lane leaves before the table
+// lookups: they are wave-wide register permutes.
 template <int DTI, int DTO, int LPB, int SUB>
-__global__ __launch_bounds__(kThreads) void mxfp_qdq_vec_kernel(const void* __restrict__ in, void* __restrict__ out,
-                                                                uint8_t* __restrict__ codes,
-                                                                uint8_t* __restrict__ scales, size_t n_vec,
-                                                                MxfpParams p) {
+__global__ __launch_bounds__(kVecThreads) void mxfp_qdq_vec_kernel(const void* __restrict__ in, void* __restrict__ out,
+                                                                   uint8_t* __restrict__ codes,
+                                                                   uint8_t* __restrict__ scales, size_t n_vec,
+                                                                   MxfpParams p) {
   using TI = DTypeTraits<DTI>;
   using TO = DTypeTraits<DTO>;
   // work in units of 8 elements when either side is a 16-bit type, else 4
   constexpr int V = (TI::kVec == 8 || TO::kVec == 8) ? 8 : 4;
   constexpr int EPS = V / SUB;
-  const size_t base = (size_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+  const size_t idx = (size_t)blockIdx.x * kVecThreads + threadIdx.x;
+  const bool live = idx < n_vec;
   WaveLog2 meta;
   meta.init(p.tab, kLog2TabHalf);
-#pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    size_t idx = base + (size_t)u * kThreads;
-    bool live = idx < n_vec;
-    float x[V], y[V];
-    uint32_t c[V];
-    if (live) {
-      if constexpr (TI::kVec == V) {
-        TI::unpack(load_nt((const uint4*)in + idx), x);
-      } else {  // fp32 input, 8 per item
-        TI::unpack(load_nt((const uint4*)in + 2 * idx), x);
-        TI::unpack(load_nt((const uint4*)in + 2 * idx + 1), x + 4);
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < V; ++j) x[j] = 0.0f;
+  float x[V], y[V];
+  uint32_t c[V];
+  if (live) {
+    if constexpr (TI::kVec == V) {
+      TI::unpack(load_nt((const uint4*)in + idx), x);
+    } else {  // fp32 input, 8 per item
+      TI::unpack(load_nt((const uint4*)in + 2 * idx), x);
+      TI::unpack(load_nt((const uint4*)in + 2 * idx + 1), x + 4);
     }
+  } else {
 #pragma unroll
-    for (int j = 0; j < V; ++j) x[j] = flush_subnormal(x[j]);
+    for (int j = 0; j < V; ++j) x[j] = 0.0f;
+  }
 #pragma unroll
-    for (int s = 0; s < SUB; ++s) {
-      uint32_t m = 0;
+  for (int j = 0; j < V; ++j) x[j] = flush_subnormal(x[j]);
 #pragma unroll
-      for (int j = 0; j < EPS; ++j) m = max(m, f2bits(x[s * EPS + j]) & 0x7FFFFFFFu);
-      m = group_max_u32<LPB>(m);
-      int sh = 0;
-      int state = mxfp_block_scale(m, p, sh, meta);
+  for (int s = 0; s < SUB; ++s) {
+    uint32_t m = 0;
 #pragma unroll
-      for (int j = 0; j < EPS; ++j) y[s * EPS + j] = mxfp_element(x[s * EPS + j], state, sh, p, c[s * EPS + j]);
-      if (codes != nullptr && live) {
-        int sb = (state == 1) ? sh + 127 : (state == 0 ? 0 : 255);
-        if constexpr (LPB > 1) {
-          if ((idx & (LPB - 1)) == 0) scales[idx / LPB] = (uint8_t)sb;
-        } else {
-          scales[idx * SUB + s] = (uint8_t)sb;
-        }
-      }
-    }
-    if (live) {
-      if constexpr (TO::kVec == V) {
-        store_nt((uint4*)out + idx, TO::pack(y));
+    for (int j = 0; j < EPS; ++j) m = max(m, f2bits(x[s * EPS + j]) & 0x7FFFFFFFu);
+    m = group_max_u32<LPB>(m);
+    int sh = 0;
+    const int state = mxfp_block_scale(m, p, sh, meta);
+#pragma unroll
+    for (int j = 0; j < EPS; ++j) y[s * EPS + j] = bits2f(mxfp_element_bits(x[s * EPS + j], state, sh, p, c[s * EPS + j]));
+    if (codes != nullptr && live) {
+      int sb = (state == 1) ? sh + 127 : (state == 0 ? 0 : 255);
+      if constexpr (LPB > 1) {
+        if ((idx & (LPB - 1)) == 0) scales[idx / LPB] = (uint8_t)sb;
       } else {
-        store_nt((uint4*)out + 2 * idx, TO::pack(y));
-        store_nt((uint4*)out + 2 * idx + 1, TO::pack(y + 4));
+        scales[idx * SUB + s] = (uint8_t)sb;
       }
-      if (codes != nullptr) {
-        if constexpr (V == 4) {
-          ((uint32_t*)codes)[idx] = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
-        } else {
-          uint2 w;
-          w.x = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
-          w.y = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
-          ((uint2*)codes)[idx] = w;
-        }
-      }
+    }
+  }
+  if (!live) return;
+  if constexpr (TO::kVec == V) {
+    store_nt((uint4*)out + idx, TO::pack(y));
+  } else {
+    store_nt((uint4*)out + 2 * idx, TO::pack(y));
+    store_nt((uint4*)out + 2 * idx + 1, TO::pack(y + 4));
+  }
+  if (codes != nullptr) {
+    if constexpr (V == 4) {
+      ((uint32_t*)codes)[idx] = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+    } else {
+      uint2 w;
+      w.x = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+      w.y = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
+      ((uint2*)codes)[idx] = w;
     }
   }
 }
@@ -149,7 +185,7 @@ int launch_mxfp(const void* in, void* out, uint8_t* codes, uint8_t* scales, size
                       (codes == nullptr || (((uintptr_t)codes) & 7u) == 0);
   if (vec_ok) {
     size_t n_vec = numel / V;
-    dim3 grid(blocks_for(n_vec, (size_t)kThreads * kUnroll)), block(kThreads);
+    dim3 grid(blocks_for(n_vec, (size_t)kVecThreads)), block(kVecThreads);
 #define MASE_MXFP_CASE(LPB_, SUB_)                                                                               \
   hipLaunchKernelGGL((mxfp_qdq_vec_kernel<DTI, DTO, LPB_, SUB_>), grid, block, 0, st, in, out, codes, scales, n_vec, p)
     if (B >= V) {
@@ -246,15 +282,16 @@ __global__ __launch_bounds__(64) void mxfp_pack_kernel(const void* __restrict__ 
   int sh = 0;
   const int state = mxfp_block_scale(m, p, sh, meta);
   uint32_t c[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) mxfp_element_bits(x[j], state, sh, p, c[j]);
+  // any element may hold the reserved code, not only the largest: a fraction carry that the encoder loses
+  // in an odd exponent field leaves the block maximum below a neighbour's code
   uint32_t reserved = 0;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    mxfp_element(x[j], state, sh, p, c[j]);
-    reserved |= code_is_reserved<E, F>(c[j]) ? 1u : 0u;
-  }
+  for (int j = 0; j < 8; ++j) reserved |= code_is_reserved<E, F>(c[j]) ? 1u : 0u;
   reserved = group_max_u32<4>(reserved);
   int sb = (state == 1) ? sh + 127 : (state == 0 ? 0 : 255);
-  if (reserved && state == 1) {
+  if (state == 1 && reserved) {
     sb = min(sb + 1, 254);
 #pragma unroll
     for (int j = 0; j < 8; ++j) c[j] = halve_code<E, F>(c[j]);
