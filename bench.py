@@ -9,6 +9,7 @@ Workloads (BASELINE.json configs):
     mxint_qdq    config 1: MXINT8 quantize-dequantize, fp32 [4096,4096], block 32
     mxint_linear config 3: MXINT8 Linear forward, 4096x4096x4096, fp32 in/out
     mxfp_linear  config 4: MXFP4(e2m1) weights x MXFP8(e4m3) activations Linear, M=8192 K=8192 N=28672
+    decoder_layer config 5: Llama-style decoder layer, every nn.Linear -> LinearMXInt, batch 8 x seq 2048, bf16
 Prints ONE JSON line.  `value` is algorithmic GB/s (Q-DQ) or TFLOP/s (Linear) over the whole timed region;
 `roofline` is for the dominant kernel, timed with HIP events on the launch stream; `cpu_baseline` is the CPU
 oracle timed on this box's host cores on a bounded sample of the same workload.
@@ -305,7 +306,101 @@ class MxfpLinear(Workload):
                                           f"(activation quantize-dequantize + bf16 F.linear), {dt*1e3:.0f} ms each"}
 
 
-WORKLOADS = {w.name: w for w in (BfpQdq, MxintQdq, MxintLinear, MxfpLinear, CopyBytes)}
+class DecoderLayerMxint(Workload):
+    name = "decoder_layer"
+    metric = ("Llama-style decoder layer forward with MXINT8 Linears (flop per step = 7 Linears + causal attention; "
+              "RMSNorm, rotary embedding, attention and SwiGLU glue run as torch ops inside the step)")
+    unit = "TFLOP/s"
+    dtype = "bf16"
+    bound = "mfma"
+    mfma_dtype = "bf16"
+    kernel = "gemm_bf16_tn_kernel"
+    B, T = 8, 2048
+    config = {"workload": "decoder layer hidden 4096, 32 heads x 128, SwiGLU 11008, RMSNorm eps 1e-6, RoPE theta 1e4, "
+                          "causal, batch 8 x seq 2048, bf16, weights N(0,0.02) seed 40, x N(0,1) seed 4; every nn.Linear "
+                          "-> LinearMXInt (block 32, 8-bit) through quantize_module_transform_pass"}
+    cfg = {"weight_block_size": 32, "weight_width": 8, "data_in_block_size": 32, "data_in_width": 8}
+
+    def build(self, torch, device):
+        from mase_amd.workloads import DecoderLayer, DecoderLayerConfig
+
+        return DecoderLayer(DecoderLayerConfig(), device=device, dtype=torch.bfloat16, seed=40)
+
+    def setup(self, torch, dev, n_buffers):
+        from mase_amd.passes import quantize_module_transform_pass
+        from mase_amd.quantizers import _ops
+        from mase_amd._gemm import gemm_bf16_tn
+
+        self.torch = torch
+        layer = self.build(torch, dev)
+        self.layer, _ = quantize_module_transform_pass(
+            layer, {"by": "type", "linear": {"config": dict(self.cfg, name="mxint")}})
+        x = torch.randn(self.B, self.T, 4096, generator=torch.Generator().manual_seed(4)).bfloat16().to(dev)
+        self.bufs = [x.roll(i, dims=1).contiguous() for i in range(max(n_buffers, 2))]
+        # operands of the seven contractions alone, for the kernel-only timing
+        tok = self.B * self.T
+        a4096 = _ops.mxint_qdq(self.bufs[0].reshape(tok, 4096), 32, 8, -1, 8, out_dtype=torch.bfloat16)
+        a11008 = _ops.mxint_qdq(torch.randn(tok, 11008, device=dev, dtype=torch.bfloat16), 32, 8, -1, 8,
+                                out_dtype=torch.bfloat16)
+        self.gemms = []
+        for name in ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"):
+            m = getattr(self.layer, name)
+            wb = m._w_cache.get(m.weight)
+            assert wb is not None
+            self.gemms.append((a11008 if name == "down_proj" else a4096, wb))
+        self._gemm = gemm_bf16_tn
+        self.linear_flops = self.layer.linear_flops(tok)
+        self.attn_flops = 4.0 * self.B * 32 * self.T * self.T * 128 / 2  # causal: half of the score matrix
+
+    def step(self, i):
+        with self.torch.no_grad():
+            self.out = self.layer(self.bufs[i % len(self.bufs)])
+
+    def dominant_step(self, i):
+        for a, w in self.gemms:
+            self.out = self._gemm(a, w, None, self.torch.bfloat16)
+
+    def work_per_step(self):
+        return self.linear_flops + self.attn_flops
+
+    def dominant_work(self):
+        return self.linear_flops
+
+    def cpu_baseline(self, torch, budget_s):
+        from oracle import linear as OL
+
+        class _OracleLinear(torch.nn.Module):
+            def __init__(self, qw, cfg):
+                super().__init__()
+                self.qw, self.cfg = qw, cfg
+
+            def forward(self, x):
+                return OL.linear_mxint_forward(x, self.qw, None, self.cfg)
+
+        layer = self.build(torch, None)
+        for name, m in list(layer.named_children()):
+            if isinstance(m, torch.nn.Linear):
+                qw, _ = OL.mxint_prepare_weights(m.weight.data, None, self.cfg)
+                setattr(layer, name, _OracleLinear(qw, self.cfg))
+        tokens = 128
+        x = torch.randn(1, tokens, 4096, generator=torch.Generator().manual_seed(4)).bfloat16()
+        with torch.no_grad():
+            layer(x[:, :16])
+            t0 = time.perf_counter()
+            n = 0
+            while True:
+                layer(x)
+                n += 1
+                if time.perf_counter() - t0 > budget_s or n >= 20:
+                    break
+        dt = (time.perf_counter() - t0) / n
+        flops = layer.linear_flops(tokens) + 4.0 * 32 * tokens * tokens * 128 / 2
+        return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+                "sample": f"{n} forwards of the same layer on 1 x {tokens} tokens (bf16, reference Linear forward), "
+                          f"{dt*1e3:.0f} ms each"}
+
+
+WORKLOADS = {w.name: w for w in (BfpQdq, MxintQdq, MxintLinear, MxfpLinear, DecoderLayerMxint, CopyBytes)}
 
 
 def load_traffic(name):
@@ -366,7 +461,8 @@ def main():
     work = w.work_per_step()
     scale = 1e9 if w.bound == "hbm" else 1e12
     value = work * a.steps / wall / scale
-    achieved = work / (k_avg * 1e-3) / scale
+    dominant_work = w.dominant_work() if hasattr(w, "dominant_work") else work
+    achieved = dominant_work / (k_avg * 1e-3) / scale
     peak = HBM_PEAK_GBS if w.bound == "hbm" else MFMA_PEAK_TFLOPS[getattr(w, "mfma_dtype", "bf16")]
     out = {
         "metric": w.metric,

@@ -1,0 +1,106 @@
+"""A Llama-style decoder layer out of plain ``torch.nn`` parts: the workload whose ``nn.Linear`` modules the
+quantize pass replaces (RMSNorm -> q/k/v projections -> rotary embedding -> causal attention -> o projection ->
+residual; RMSNorm -> SwiGLU MLP -> residual).
+
+Semantics follow the reference's Llama block (``chop/models/llama/modeling_llama.py:79-93`` RMSNorm, ``:99-147,
+185-216`` rotary embedding with ``rotate_half``, ``:219-236`` MLP ``down(silu(gate(x)) * up(x))``, ``:362-480``
+attention, ``:843-918`` layer with pre-norm residuals); no KV cache, no dropout, no attention bias.
+Everything except the seven Linears is ordinary torch and runs identically on CPU and GPU, which is what lets the
+same class serve as the CPU reference once its Linears are swapped for reference ones.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+from torch import nn
+from torch.nn import functional as F
+
+
+@dataclass
+class DecoderLayerConfig:
+    hidden_size: int = 4096
+    num_heads: int = 32
+    head_dim: int = 128
+    intermediate_size: int = 11008
+    rms_norm_eps: float = 1e-6
+    rope_theta: float = 10000.0
+    init_std: float = 0.02
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, hidden_size: int, eps: float):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(hidden_size))
+        self.eps = eps
+
+    def forward(self, x):
+        dtype = x.dtype
+        h = x.to(torch.float32)
+        h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + self.eps)
+        return self.weight * h.to(dtype)
+
+
+def rotate_half(x):
+    x1, x2 = x[..., : x.shape[-1] // 2], x[..., x.shape[-1] // 2:]
+    return torch.cat((-x2, x1), dim=-1)
+
+
+def rope_tables(seq_len: int, head_dim: int, theta: float, device, dtype):
+    inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32, device=device) / head_dim))
+    t = torch.arange(seq_len, dtype=torch.float32, device=device)
+    freqs = torch.outer(t, inv_freq)
+    emb = torch.cat((freqs, freqs), dim=-1)
+    return emb.cos().to(dtype), emb.sin().to(dtype)
+
+
+class DecoderLayer(nn.Module):
+    def __init__(self, cfg: DecoderLayerConfig = DecoderLayerConfig(), device=None, dtype=None, seed: int | None = None):
+        super().__init__()
+        self.cfg = cfg
+        kw = dict(bias=False, device=device, dtype=dtype)
+        H, D, I = cfg.hidden_size, cfg.num_heads * cfg.head_dim, cfg.intermediate_size
+        self.input_layernorm = RMSNorm(H, cfg.rms_norm_eps).to(device=device, dtype=dtype)
+        self.q_proj = nn.Linear(H, D, **kw)
+        self.k_proj = nn.Linear(H, D, **kw)
+        self.v_proj = nn.Linear(H, D, **kw)
+        self.o_proj = nn.Linear(D, H, **kw)
+        self.post_attention_layernorm = RMSNorm(H, cfg.rms_norm_eps).to(device=device, dtype=dtype)
+        self.gate_proj = nn.Linear(H, I, **kw)
+        self.up_proj = nn.Linear(H, I, **kw)
+        self.down_proj = nn.Linear(I, H, **kw)
+        # the attention core is a plain torch library call; tests replace it to keep both sides of a comparison on
+        # the same implementation (the library's CPU and GPU kernels differ by a few bf16 ulps)
+        self.attention_fn = lambda q, k, v: F.scaled_dot_product_attention(q, k, v, is_causal=True)
+        if seed is not None:
+            self.reset_parameters_seeded(seed)
+
+    @torch.no_grad()
+    def reset_parameters_seeded(self, seed: int):
+        """N(0, init_std) weights drawn on the CPU from one generator, so that a CPU and a GPU instance built with
+        the same seed hold identical parameters"""
+        g = torch.Generator().manual_seed(seed)
+        for name in ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"):
+            w = getattr(self, name).weight
+            w.copy_((torch.randn(w.shape, generator=g) * self.cfg.init_std).to(w.dtype))
+
+    def forward(self, x):
+        cfg = self.cfg
+        B, T, _ = x.shape
+        h = self.input_layernorm(x)
+        q = self.q_proj(h).view(B, T, cfg.num_heads, cfg.head_dim).transpose(1, 2)
+        k = self.k_proj(h).view(B, T, cfg.num_heads, cfg.head_dim).transpose(1, 2)
+        v = self.v_proj(h).view(B, T, cfg.num_heads, cfg.head_dim).transpose(1, 2)
+        cos, sin = rope_tables(T, cfg.head_dim, cfg.rope_theta, x.device, x.dtype)
+        q = q * cos + rotate_half(q) * sin
+        k = k * cos + rotate_half(k) * sin
+        a = self.attention_fn(q, k, v)
+        a = a.transpose(1, 2).reshape(B, T, cfg.num_heads * cfg.head_dim)
+        x = x + self.o_proj(a)
+        h = self.post_attention_layernorm(x)
+        x = x + self.down_proj(F.silu(self.gate_proj(h)) * self.up_proj(h))
+        return x
+
+    def linear_flops(self, tokens: int) -> float:
+        H, D, I = self.cfg.hidden_size, self.cfg.num_heads * self.cfg.head_dim, self.cfg.intermediate_size
+        return 2.0 * tokens * (3 * H * D + D * H + 3 * H * I)
