@@ -13,8 +13,8 @@
 // the largest of them and truncated about 12 bits below its leading bit before they are added; sums across
 // such groups of 8 and across instructions are carried in fp32.
 //
-// Schedule: the 256x256 tile, 2x2 wavefronts of 4x4 MFMA tiles and the LDS-transposed epilogue are those of the
-// bf16 kernel (gemm_bf16.hip).  K tile 128: per stage A 256 x 128 B, B 256 x 64 B (4-bit) or 256 x 128 B (8-bit),
+// Schedule: the 256x256 tile and the 2x2 wavefronts of 4x4 MFMA tiles are those of the bf16 kernel
+// (gemm_bf16.hip); the kernel is persistent (one work-group per CU walks its output tiles).  K tile 128: per stage A 256 x 128 B, B 256 x 64 B (4-bit) or 256 x 128 B (8-bit),
 // plus 4 scale bytes per row for each operand = one dword per row per K tile.  Three stages when B is 4-bit
 // (50 KB each), two when it is 8-bit (66 KB).  All of it travels HBM/L2 -> LDS with global_load_lds (16-byte
 // form for codes, 4-byte form for scales); copies of tile t+S are issued while the last MFMAs of tile t run.
@@ -46,14 +46,15 @@ struct MxGemmParams {
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
-// one wavefront-wide async copy HBM/L2 -> LDS: lane i's BYTES bytes at `g` land at LDS address lds_addr + BYTES*i
+// one wavefront-wide async copy HBM/L2 -> LDS: lane i's BYTES bytes at base + off_i land at LDS address
+// lds_addr + BYTES*i (base and lds_addr wavefront-uniform, off_i a 32-bit byte offset)
 template <int BYTES>
-__device__ __forceinline__ void async_copy(const unsigned char* g, uint32_t lds_addr) {
-  const uint32_t base = __builtin_amdgcn_readfirstlane(lds_addr);
+__device__ __forceinline__ void async_copy(const unsigned char* base, uint32_t off, uint32_t lds_addr) {
+  const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_addr);
   if constexpr (BYTES == 16)
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(base) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
   else
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(base) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
 }
 
 template <int N>
@@ -75,13 +76,29 @@ __device__ __forceinline__ int lds_off(int row, int chunk) {
   else return row * 64 + ((chunk ^ ((row >> 2) & 3)) << 4);
 }
 
-template <int B_BITS, int CBSZ, int BLGP, int OUT_DT>
+template <int B_BITS>
+struct MxGemmGeom {
+  static constexpr int RA = BK;               // bytes per A row per K tile (8-bit codes)
+  static constexpr int RB = BK * B_BITS / 8;  // bytes per B row per K tile
+  static constexpr int kTileA = BM * RA, kTileB = BN * RB;
+  static constexpr int kStage = kTileA + kTileB + 2 * 1024;  // + one scale dword per row for A and for B
+  static constexpr int S = (kStage <= 53 * 1024) ? 3 : 2;
+  // epilogue staging, separate from the stages (copies of the next tile are in flight during the epilogue):
+  // per wavefront 8 rows x 64 columns of fp32, row stride 68 floats (4 rows per half-wave)
+  static constexpr int kStgStride = 68;
+  static constexpr int kStgWave = 8 * kStgStride * 4;
+  static constexpr int kLdsBytes = S * kStage + 4 * kStgWave;
+};
+
+// Persistent kernel: one work-group per CU walks a list of output tiles.  The K tiles of all its output tiles
+// form one stream through the LDS stages, so the copies of the next output tile's first K tiles are already
+// in flight while the epilogue of the current one runs, and its stores drain behind the next main loop.
+// STREAM: K holds at least S tiles, so the copy stream is never more than one output tile ahead and advances
+// without branches; the other instantiation (short K) advances it with the general, branching step.
+template <int B_BITS, int CBSZ, int BLGP, int OUT_DT, bool STREAM>
 __global__ __launch_bounds__(kThreadsG) void gemm_mxfp_kernel(MxGemmParams p) {
-  constexpr int RA = BK;               // bytes per A row per K tile (8-bit codes)
-  constexpr int RB = BK * B_BITS / 8;  // bytes per B row per K tile
-  constexpr int kTileA = BM * RA, kTileB = BN * RB;
-  constexpr int kStage = kTileA + kTileB + 2 * 1024;  // + one scale dword per row for A and for B
-  constexpr int S = (kStage <= 53 * 1024) ? 3 : 2;
+  using G = MxGemmGeom<B_BITS>;
+  constexpr int RA = G::RA, RB = G::RB, kTileA = G::kTileA, kTileB = G::kTileB, kStage = G::kStage, S = G::S;
   constexpr int kCopiesA = kTileA / 1024 / 4;          // 16-byte copies per wavefront per tile
   constexpr int kCopiesB = kTileB / 1024 / 4;
   constexpr int kCopies = kCopiesA + kCopiesB + 2;     // + one 4-byte copy each for the A and B scales
@@ -90,79 +107,123 @@ __global__ __launch_bounds__(kThreadsG) void gemm_mxfp_kernel(MxGemmParams p) {
 
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int tid = threadIdx.x;
-  const int lane = tid & 63;
+  const int lane_id = tid & 63;
+  const int lane = lane_id;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
-
-  int bid = blockIdx.x;
-  const int total = p.tiles_m * p.tiles_n;
-  if ((total & 7) == 0) bid = (bid & 7) * (total >> 3) + (bid >> 3);
-  constexpr int GROUP_M = 4;
-  const int in_group = GROUP_M * p.tiles_n;
-  const int first_m = (bid / in_group) * GROUP_M;
-  const int gsz = min(p.tiles_m - first_m, GROUP_M);
-  const int tile_m = first_m + (bid % in_group) % gsz;
-  const int tile_n = (bid % in_group) / gsz;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int nk = p.K / BK;
 
-  // ---- global side of the async copies
+  // ---- this work-group's output tiles.  Work-groups are dealt to the 8 XCDs round-robin; when the counts
+  // divide, XCD x owns the contiguous tile range [x*total/8, (x+1)*total/8) and its work-groups walk it
+  // together (at any time they hold neighbouring tiles, which share operand rows in that XCD's L2).
+  const int total = p.tiles_m * p.tiles_n;
+  const int nwg = (int)gridDim.x;
+  int t_first, t_step, t_end;
+  if ((total & 7) == 0 && (nwg & 7) == 0) {
+    const int per_xcd = total >> 3;
+    t_first = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+    t_step = nwg >> 3;
+    t_end = (((int)blockIdx.x & 7) + 1) * per_xcd;
+  } else {
+    t_first = (int)blockIdx.x;
+    t_step = nwg;
+    t_end = total;
+  }
+  const int n_my = (t_first < t_end) ? (t_end - t_first + t_step - 1) / t_step : 0;
+  if (n_my == 0) return;
+  constexpr int GROUP_M = 4;
+  const int in_group = GROUP_M * p.tiles_n;
+  auto tile_origin = [&](int ord, int& m0, int& n0) {  // ord-th tile of this work-group
+    const int t = t_first + min(ord, n_my - 1) * t_step;
+    const int first_m = (t / in_group) * GROUP_M;
+    const int gsz = min(p.tiles_m - first_m, GROUP_M);
+    m0 = (first_m + (t % in_group) % gsz) * BM;
+    n0 = ((t % in_group) / gsz) * BN;
+  };
+
+  // ---- global side of the async copies (the copy stream runs S K-tiles ahead of the MFMAs)
   const size_t lda = (size_t)p.K;                 // bytes per A row
   const size_t ldbb = (size_t)p.K * B_BITS / 8;   // bytes per B row
   const size_t lds_sc = (size_t)p.K / 32;         // scale bytes per row
-  const unsigned char* ga[kCopiesA];
-  const unsigned char* gb[kCopiesB];
+  uint32_t ga[kCopiesA], gb[kCopiesB], gsa, gsb;  // byte offsets of this lane's pieces from the operand bases
+  auto set_copy_tile = [&](int ord) __attribute__((always_inline)) {
+    int m0, n0;
+    tile_origin(ord, m0, n0);
+    int lane = lane_id;
+    asm volatile("" : "+v"(lane));  // keeps the lane-derived terms below out of the K loop's live registers
 #pragma unroll
-  for (int j = 0; j < kCopiesA; ++j) {  // 8 rows of 128 B per copy
-    const int r = (wave + 4 * j) * 8 + (lane >> 3);
-    ga[j] = p.A + (size_t)min(m0 + r, p.M - 1) * lda + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
-  }
-#pragma unroll
-  for (int j = 0; j < kCopiesB; ++j) {
-    if constexpr (RB == 128) {
+    for (int j = 0; j < kCopiesA; ++j) {  // 8 rows of 128 B per copy
       const int r = (wave + 4 * j) * 8 + (lane >> 3);
-      gb[j] = p.B + (size_t)min(n0 + r, p.N - 1) * ldbb + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
-    } else {  // 16 rows of 64 B per copy
-      const int r = (wave + 4 * j) * 16 + (lane >> 2);
-      gb[j] = p.B + (size_t)min(n0 + r, p.N - 1) * ldbb + (((lane & 3) ^ ((r >> 2) & 3)) << 4);
+      ga[j] = (uint32_t)((size_t)min(m0 + r, p.M - 1) * lda) + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
     }
-  }
-  // scales: wave w copies the dwords of rows [64w, 64w+64) of each operand
-  const unsigned char* gsa = p.SA + (size_t)min(m0 + wave * 64 + lane, p.M - 1) * lds_sc;
-  const unsigned char* gsb = p.SB + (size_t)min(n0 + wave * 64 + lane, p.N - 1) * lds_sc;
+#pragma unroll
+    for (int j = 0; j < kCopiesB; ++j) {
+      if constexpr (RB == 128) {
+        const int r = (wave + 4 * j) * 8 + (lane >> 3);
+        gb[j] = (uint32_t)((size_t)min(n0 + r, p.N - 1) * ldbb) + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
+      } else {  // 16 rows of 64 B per copy
+        const int r = (wave + 4 * j) * 16 + (lane >> 2);
+        gb[j] = (uint32_t)((size_t)min(n0 + r, p.N - 1) * ldbb) + (((lane & 3) ^ ((r >> 2) & 3)) << 4);
+      }
+    }
+    // scales: wave w copies the dwords of rows [64w, 64w+64) of each operand
+    gsa = (uint32_t)((size_t)min(m0 + wave * 64 + lane, p.M - 1) * lds_sc);
+    gsb = (uint32_t)((size_t)min(n0 + wave * 64 + lane, p.N - 1) * lds_sc);
+  };
 
   // The copies are issued from inline assembly rather than through the compiler's builtin: the compiler
   // orders every LDS read after all async copies it knows to be in flight (s_waitcnt vmcnt(0) before each
   // ds_read), which would serialize the pipeline; completion is tracked by hand with wait_vmcnt_n below.
   // M0 carries the wavefront-uniform LDS base; nothing else in this kernel uses M0.
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;
-  auto issue_copy = [&](int kt, int c) {
-    const uint32_t st = lds_base + (uint32_t)((kt % S) * kStage);
-    const int ktc = min(kt, nk - 1);
+  // copy-stream position: K tile c_kt of this work-group's c_ord-th output tile goes to stage c_stage.  Past the
+  // last tile the stream keeps re-copying the final K tile into stages nobody reads any more, which keeps
+  // the main loop free of branches around the copies and the vmcnt bookkeeping uniform.
+  int c_kt = 0, c_ord = 0, c_stage = 0;
+  auto issue_copy = [&](int c) __attribute__((always_inline)) {
+    const uint32_t st = lds_base + (uint32_t)(c_stage * kStage);
     if (c < kCopiesA) {
-      async_copy<16>(ga[c] + (size_t)ktc * RA, st + (wave + 4 * c) * 1024);
+      async_copy<16>(p.A + (size_t)c_kt * RA, ga[c], st + (wave + 4 * c) * 1024);
     } else if (c < kCopiesA + kCopiesB) {
       const int j = c - kCopiesA;
-      async_copy<16>(gb[j] + (size_t)ktc * RB, st + kTileA + (wave + 4 * j) * 1024);
+      async_copy<16>(p.B + (size_t)c_kt * RB, gb[j], st + kTileA + (wave + 4 * j) * 1024);
     } else if (c == kCopiesA + kCopiesB) {
-      async_copy<4>(gsa + (size_t)ktc * 4, st + kTileA + kTileB + wave * 256);
+      async_copy<4>(p.SA + (size_t)c_kt * 4, gsa, st + kTileA + kTileB + wave * 256);
     } else {
-      async_copy<4>(gsb + (size_t)ktc * 4, st + kTileA + kTileB + 1024 + wave * 256);
+      async_copy<4>(p.SB + (size_t)c_kt * 4, gsb, st + kTileA + kTileB + 1024 + wave * 256);
+    }
+  };
+  auto advance_copy_stream = [&]() __attribute__((always_inline)) {
+    c_stage = (c_stage + 1 == S) ? 0 : c_stage + 1;
+    if (c_ord >= n_my) return;          // past the end: stay on the final K tile
+    if (++c_kt == nk) {
+      if (++c_ord < n_my) {
+        c_kt = 0;
+        set_copy_tile(c_ord);
+      } else {
+        c_kt = nk - 1;
+      }
     }
   };
 
   f32x16_t acc[4][4];
+  auto zero_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  };
+  zero_acc();
 
+  set_copy_tile(0);
 #pragma unroll
-  for (int t = 0; t < S; ++t)
+  for (int t = 0; t < S; ++t) {
 #pragma unroll
-    for (int c = 0; c < kCopies; ++c) issue_copy(t, c);
+    for (int c = 0; c < kCopies; ++c) issue_copy(c);
+    advance_copy_stream();
+  }
 
   const int frag_row = lane & 31;
   const int kgrp = lane >> 5;
@@ -170,8 +231,8 @@ __global__ __launch_bounds__(kThreadsG) void gemm_mxfp_kernel(MxGemmParams p) {
   // upper 4 unused for 4-bit codes).  Read number q of a step: q < 8 -> 16-byte half (q&1) of A tile q>>1;
   // then the B chunks.
   uint4 fa[2][4][2], fb[2][4][2];
-  auto load_part = [&](int kt, int s, int set, int q) {
-    const unsigned char* st = lds + (kt % S) * kStage;
+  auto load_part = [&](int stage, int s, int set, int q) __attribute__((always_inline)) {
+    const unsigned char* st = lds + stage * kStage;
     if (q < 8) {
       const int i = q >> 1, h = q & 1;
       fa[set][i][h] = *(const uint4*)(st + (wm * 128) * RA + lds_off<RA>(i * 32 + frag_row, s * 4 + h * 2 + kgrp));
@@ -182,18 +243,18 @@ __global__ __launch_bounds__(kThreadsG) void gemm_mxfp_kernel(MxGemmParams p) {
                                       lds_off<RB>(j * 32 + frag_row, kChunksB == 2 ? s * 4 + h * 2 + kgrp : s * 2 + kgrp));
     }
   };
-  // scale dwords of the current tile (sa/sb) and of the next one (san/sbn), pre-shifted so that K step s
+  // scale dwords of the current K tile (sa/sb) and of the next one (san/sbn), pre-shifted so that K step s
   // uses byte 2s
   int sa[4], sb[4], san[4], sbn[4];
-  auto load_scales = [&](int kt, int* a, int* b) {
-    const unsigned char* st = lds + (kt % S) * kStage + kTileA + kTileB;
+  auto load_scales = [&](int stage, int* a, int* b) {
+    const unsigned char* st = lds + stage * kStage + kTileA + kTileB;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       a[i] = (int)(*(const uint32_t*)(st + (wm * 128 + i * 32 + frag_row) * 4) >> (8 * kgrp));
       b[i] = (int)(*(const uint32_t*)(st + 1024 + (wn * 128 + i * 32 + frag_row) * 4) >> (8 * kgrp));
     }
   };
-  auto mfma = [&](int set, int s, int t) {
+  auto mfma = [&](int set, int s, int t) __attribute__((always_inline)) {
     const int i = t >> 2, j = t & 3;
     i32x8_t a, b;
     a[0] = (int)fa[set][i][0].x; a[1] = (int)fa[set][i][0].y; a[2] = (int)fa[set][i][0].z; a[3] = (int)fa[set][i][0].w;
@@ -210,119 +271,195 @@ __global__ __launch_bounds__(kThreadsG) void gemm_mxfp_kernel(MxGemmParams p) {
       acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], CBSZ, BLGP, 2, sa[i], 2, sb[j]);
   };
 
+  // ---- epilogue of one output tile: accumulators -> bands of 8 rows x 64 columns through the wavefront's own
+  // staging rows -> 16 bytes of consecutive columns per lane (bias added, converted) -> global.
+  // In the accumulator layout lanes 0-31 hold rows q*8+0..3 and lanes 32-63 rows q*8+4..7 of each 32-row MFMA
+  // tile (one column per lane); each half-wave writes its 4 rows and reads the same 4 rows back, so no lane
+  // depends on LDS writes of the other half-wave or of another wavefront: no barrier and no wait for write
+  // completion is needed (the LDS executes one half-wave's accesses in order).
+  const bool vec_ok = ((p.N & 3) == 0) && ((((uintptr_t)p.C) & 15u) == 0);
+  auto epilogue = [&](int ord) __attribute__((always_inline)) {
+    int m0, n0;
+    tile_origin(ord, m0, n0);
+    int lane = lane_id;
+    asm volatile("" : "+v"(lane));  // keeps the lane-derived terms below out of the K loop's live registers
+    const int frag_row = lane & 31, kgrp = lane >> 5;
+    float* stg = (float*)(lds + S * kStage + wave * G::kStgWave) + kgrp * (4 * G::kStgStride);
+    const int c4 = (lane & 15) * 4;          // columns within the 64-column band
+    const int rl0 = (lane & 31) >> 4;        // this lane reads rows rl0 and rl0 + 2 of its half-wave's 4
+    float bv[2][4] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+    if (p.bias != nullptr) {
+#pragma unroll
+      for (int jh = 0; jh < 2; ++jh)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int col = n0 + wn * 128 + jh * 64 + c4 + e;
+          if (col < p.N) bv[jh][e] = load_bias_v(p.bias, p.bias_dtype, col);
+        }
+      // The bias loads are the only vector-memory loads the compiler itself tracks in this kernel.  Completing
+      // them here, with a wait it can see, keeps it from guarding their registers with s_waitcnt vmcnt(0)
+      // inside the K loop, where that would also wait for every async copy in flight.
+      wait_vmcnt_n<0>();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+#pragma unroll
+        for (int jh = 0; jh < 2; ++jh) {
+#pragma unroll
+          for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr)
+              stg[rr * G::kStgStride + jj * 32 + frag_row] = acc[i][jh * 2 + jj][q * 4 + rr];
+          asm volatile("" ::: "memory");  // lanes exchange data through LDS: no value may be carried across
+          __builtin_amdgcn_sched_barrier(0);  // bands stay in program order: bounded register use
+          const int col0 = n0 + wn * 128 + jh * 64 + c4;
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            const int rl = rl0 + 2 * u;
+            const float4 v4 = *(const float4*)(stg + rl * G::kStgStride + c4);
+            const float v[4] = {v4.x + bv[jh][0], v4.y + bv[jh][1], v4.z + bv[jh][2], v4.w + bv[jh][3]};
+            const int row = m0 + wm * 128 + i * 32 + q * 8 + kgrp * 4 + rl;
+            if (row >= p.M) continue;
+            const size_t o = (size_t)row * p.N + col0;
+            if (vec_ok && col0 + 3 < p.N) {
+              if constexpr (OUT_DT == MASE_DT_F32) {
+                *(float4*)((float*)p.C + o) = make_float4(v[0], v[1], v[2], v[3]);
+              } else if constexpr (OUT_DT == MASE_DT_BF16) {
+                uint2 w;
+                w.x = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
+                w.y = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
+                *(uint2*)((uint16_t*)p.C + o) = w;
+              } else {
+                uint2 w;
+                w.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
+                w.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
+                *(uint2*)((uint16_t*)p.C + o) = w;
+              }
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                if (col0 + e >= p.N) continue;
+                if constexpr (OUT_DT == MASE_DT_F32) ((float*)p.C)[o + e] = v[e];
+                else if constexpr (OUT_DT == MASE_DT_BF16) ((uint16_t*)p.C)[o + e] = (uint16_t)f32_to_bf16_bits(v[e]);
+                else ((uint16_t*)p.C)[o + e] = (uint16_t)f32_to_f16_bits(v[e]);
+              }
+            }
+          }
+        }
+      }
+    }
+  };
+
   // Pipeline (see gemm_bf16.hip for the reasoning): per K tile two steps of 16 MFMAs; fragment sets ping-pong.
   //   step 0: MFMAs on set 0, interleaved with the LDS reads of step 1 (set 1)
-  //   hand-over: own LDS reads done (lgkmcnt), own copies of tile kt+1 landed (vmcnt), barrier
-  //   step 1: MFMAs on set 1, interleaved with the LDS reads of step 0 and the scales of tile kt+1 and with
-  //           the copies of tile kt+S into the stage tile kt just vacated
+  //   hand-over: own LDS reads done (lgkmcnt), own copies of the next K tile landed (vmcnt), barrier
+  //   step 1: MFMAs on set 1, interleaved with the LDS reads of step 0 and the scales of the next K tile and
+  //           with the copies of the K tile S positions ahead into the stage just vacated
+  // After the last K tile of an output tile: epilogue, accumulators cleared; the stream carries on.
+  // The epilogue's stores count in vmcnt like the copies.  Loads retire in order among themselves, so
+  // "at most (S-2)*kCopies outstanding" still proves the next K tile has landed (if one of its loads were
+  // pending, all kCopies loads of the K tile after it would be too); it may additionally wait for stores.
   constexpr int kCopiesPerSlot = (kCopies + 15) / 16;
-  wait_vmcnt_n<(S - 1) * kCopies>();  // tile 0 landed; the other stages may still be filling
+  wait_vmcnt_n<(S - 1) * kCopies>();  // K tile 0 landed; the other stages may still be filling
   asm volatile("s_barrier" ::: "memory");
 #pragma unroll
   for (int q = 0; q < kReads; ++q) load_part(0, 0, 0, q);
   load_scales(0, sa, sb);
-  for (int kt = 0; kt < nk; ++kt) {
+  int stage = 0;
+  // One K tile.  The body must stay a single basic block: with a branch inside, the compiler sinks the MFMAs
+  // (whose results are only consumed by the next iteration) below it and the interleave is lost.  Hence the
+  // copy stream is advanced by a caller-supplied, branch-free step.
+  auto k_iteration = [&](auto&& advance) __attribute__((always_inline)) {
+    const int next_stage = (stage + 1 == S) ? 0 : stage + 1;
 #pragma unroll
     for (int t = 0; t < 16; ++t) {
       mfma(0, 0, t);
-      if (t < kReads) load_part(kt, 1, 1, t);
+      if (t < kReads) load_part(stage, 1, 1, t);
       __builtin_amdgcn_sched_barrier(0);
     }
-    wait_vmcnt_n<(S - 2) * kCopies>();  // tiles kt+1 .. kt+S-1 are in flight; kt+1 must have landed
+    wait_vmcnt_n<(S - 2) * kCopies>();  // the next K tile must have landed; later ones may be in flight
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = 0; t < 16; ++t) {
       mfma(1, 1, t);
-      if (t < kReads) load_part(kt + 1, 0, 0, t);
-      if (t == 12) load_scales(kt + 1, san, sbn);
+      if (t < kReads) load_part(next_stage, 0, 0, t);
+      if (t == 12) load_scales(next_stage, san, sbn);
 #pragma unroll
       for (int c = t * kCopiesPerSlot; c < (t + 1) * kCopiesPerSlot; ++c)
-        if (c < kCopies) issue_copy(kt + S, c);  // into the stage tile kt just vacated
+        if (c < kCopies) issue_copy(c);  // into the stage this K tile just vacated (c_stage == stage)
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) { sa[i] = san[i]; sb[i] = sbn[i]; }
-  }
-  wait_vmcnt_n<0>();
-
-  // ---- epilogue (as in gemm_bf16.hip): transpose 32-row bands through LDS, 4 consecutive columns per lane
-  asm volatile("s_barrier" ::: "memory");
-  constexpr int kStgStride = 136;
-  float* stg = (float*)(lds + wave * (32 * kStgStride * 4));
-  const int c4 = (lane & 31) * 4;
-  const int col0 = n0 + wn * 128 + c4;
-  const bool vec_ok = ((p.N & 3) == 0) && ((((uintptr_t)p.C) & 15u) == 0);
-  float bv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  if (p.bias != nullptr) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e)
-      if (col0 + e < p.N) bv[e] = load_bias_v(p.bias, p.bias_dtype, col0 + e);
-  }
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        stg[((r >> 2) * 8 + kgrp * 4 + (r & 3)) * kStgStride + j * 32 + frag_row] = acc[i][j][r];
-#pragma unroll
-    for (int q = 0; q < 16; ++q) {
-      const int rr = q * 2 + kgrp;
-      const int row = m0 + wm * 128 + i * 32 + rr;
-      const float4 v4 = *(const float4*)(stg + rr * kStgStride + c4);
-      const float v[4] = {v4.x + bv[0], v4.y + bv[1], v4.z + bv[2], v4.w + bv[3]};
-      if (row >= p.M) continue;
-      const size_t o = (size_t)row * p.N + col0;
-      if (vec_ok && col0 + 3 < p.N) {
-        if constexpr (OUT_DT == MASE_DT_F32) {
-          *(float4*)((float*)p.C + o) = make_float4(v[0], v[1], v[2], v[3]);
-        } else if constexpr (OUT_DT == MASE_DT_BF16) {
-          uint2 w;
-          w.x = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
-          w.y = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
-          *(uint2*)((uint16_t*)p.C + o) = w;
-        } else {
-          uint2 w;
-          w.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
-          w.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
-          *(uint2*)((uint16_t*)p.C + o) = w;
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if (col0 + e >= p.N) continue;
-          if constexpr (OUT_DT == MASE_DT_F32) ((float*)p.C)[o + e] = v[e];
-          else if constexpr (OUT_DT == MASE_DT_BF16) ((uint16_t*)p.C)[o + e] = (uint16_t)f32_to_bf16_bits(v[e]);
-          else ((uint16_t*)p.C)[o + e] = (uint16_t)f32_to_f16_bits(v[e]);
-        }
-      }
+    advance();
+    stage = next_stage;
+  };
+  auto step_within_tile = [&]() {
+    c_stage = (c_stage + 1 == S) ? 0 : c_stage + 1;
+    ++c_kt;
+  };
+  for (int ord = 0; ord < n_my; ++ord) {
+    if constexpr (STREAM) {
+      // the copy stream stands at K tile S of this output tile (or, if nk == S, at K tile 0 of the next)
+#pragma unroll 1
+      for (int kt = 0; kt < nk - S; ++kt) k_iteration(step_within_tile);
+      // it moves on to the next output tile (past the last one: harmless re-copies of its first K tiles)
+      set_copy_tile(ord + 1);
+      c_kt = 0;
+#pragma unroll 1
+      for (int kt = 0; kt < S; ++kt) k_iteration(step_within_tile);
+    } else {
+      for (int kt = 0; kt < nk; ++kt) k_iteration(advance_copy_stream);
     }
+    epilogue(ord);
+    zero_acc();
   }
+  wait_vmcnt_n<0>();  // no copy may still be in flight towards LDS when the work-group retires
+}
+
+// number of work-groups of the persistent kernel: one per CU (each takes the whole LDS of its CU)
+int persistent_grid(int total_tiles) {
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return -1;
+    n_cu = prop.multiProcessorCount;
+  }
+  return total_tiles < n_cu ? total_tiles : n_cu;
 }
 
 template <int B_BITS, int CBSZ, int BLGP>
 int launch_mx_gemm(const MxGemmParams& p, int out_dtype, hipStream_t st) {
-  constexpr int kStage = BM * BK + BN * BK * B_BITS / 8 + 2048;
-  constexpr int S = (kStage <= 53 * 1024) ? 3 : 2;
-  const size_t lds_bytes = (size_t)S * kStage;
-  const void* kernels[3] = {(const void*)gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, MASE_DT_F32>,
-                            (const void*)gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, MASE_DT_BF16>,
-                            (const void*)gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, MASE_DT_F16>};
-  static bool attr_set = false;
-  if (!attr_set) {
-    for (const void* k : kernels)
-      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
-        return MASE_ERR_LAUNCH;
-    attr_set = true;
+  const size_t lds_bytes = (size_t)MxGemmGeom<B_BITS>::kLdsBytes;
+  const int nwg = persistent_grid(p.tiles_m * p.tiles_n);
+  if (nwg <= 0) return MASE_ERR_LAUNCH;
+  const dim3 grid((unsigned)nwg), block(kThreadsG);
+  const bool stream = p.K / BK >= MxGemmGeom<B_BITS>::S;
+#define MASE_MX_LAUNCH(DT_, STREAM_)                                                                              \
+  do {                                                                                                            \
+    static bool attr_set = false;                                                                                 \
+    const void* k = (const void*)gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, DT_, STREAM_>;                              \
+    if (!attr_set) {                                                                                              \
+      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)       \
+        return MASE_ERR_LAUNCH;                                                                                   \
+      attr_set = true;                                                                                            \
+    }                                                                                                             \
+    hipLaunchKernelGGL((gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, DT_, STREAM_>), grid, block, lds_bytes, st, p);      \
+  } while (0)
+  if (stream) {
+    if (out_dtype == MASE_DT_F32) MASE_MX_LAUNCH(MASE_DT_F32, true);
+    else if (out_dtype == MASE_DT_BF16) MASE_MX_LAUNCH(MASE_DT_BF16, true);
+    else MASE_MX_LAUNCH(MASE_DT_F16, true);
+  } else {
+    if (out_dtype == MASE_DT_F32) MASE_MX_LAUNCH(MASE_DT_F32, false);
+    else if (out_dtype == MASE_DT_BF16) MASE_MX_LAUNCH(MASE_DT_BF16, false);
+    else MASE_MX_LAUNCH(MASE_DT_F16, false);
   }
-  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kThreadsG);
-  if (out_dtype == MASE_DT_F32)
-    hipLaunchKernelGGL((gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, MASE_DT_F32>), grid, block, lds_bytes, st, p);
-  else if (out_dtype == MASE_DT_BF16)
-    hipLaunchKernelGGL((gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, MASE_DT_BF16>), grid, block, lds_bytes, st, p);
-  else
-    hipLaunchKernelGGL((gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, MASE_DT_F16>), grid, block, lds_bytes, st, p);
+#undef MASE_MX_LAUNCH
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
 
@@ -337,6 +474,8 @@ extern "C" int mase_gemm_mxfp_scaled(const void* A, const void* A_scales, int a_
   if (M == 0 || N == 0) return MASE_OK;
   if (A == nullptr || B == nullptr || A_scales == nullptr || B_scales == nullptr || C == nullptr) return MASE_ERR_NULL;
   if (K == 0 || (K % BK) != 0 || M > (1u << 30) || N > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
+  // the kernel addresses each operand with a 32-bit byte offset from its base
+  if ((unsigned long long)M * K > 0xFFFFFFFFull || (unsigned long long)N * K > 0xFFFFFFFFull) return MASE_ERR_SHAPE;
   if (!aligned16(A) || !aligned16(B) || (((uintptr_t)A_scales) & 3u) != 0 || (((uintptr_t)B_scales) & 3u) != 0)
     return MASE_ERR_ALIGN;
   if (out_dtype < 0 || out_dtype > 2 || (bias != nullptr && (bias_dtype < 0 || bias_dtype > 2))) return MASE_ERR_DTYPE;

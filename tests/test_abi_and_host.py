@@ -62,6 +62,18 @@ def test_entry_points_reject_bad_arguments_without_a_gpu(lib):
     assert lib.mase_minifloat_qdq(p, p, 16, 0, 8, 9, -1, 0, p, None) == -5
     assert lib.mase_minifloat_mx_qdq(p, p, 16, 0, 0, 4, 3, 1, 7, None) == -5
     assert lib.mase_block_fp_workspace_bytes(2, 5, 40, 2, 16, 1) == 2 * 3 * 3 * 4
+    # packed-MXFP path: mase_mxfp_pack(in, codes, scales, numel, in_dtype, E, F, tab, stream)
+    assert lib.mase_mxfp_pack(p, p, p, 48, 0, 4, 3, p, None) == -2       # whole blocks of 32
+    assert lib.mase_mxfp_pack(p, p, p, 64, 0, 2, 3, p, None) == -5       # e2m3 has no matrix-instruction format
+    assert lib.mase_mxfp_pack(p, None, p, 64, 0, 4, 3, p, None) == -1
+    assert lib.mase_mxfp_pack(p, p, p, 64, 5, 4, 3, p, None) == -4
+    # mase_gemm_mxfp_scaled(A, SA, a_fmt, B, SB, b_fmt, bias, C, M, N, K, out_dtype, bias_dtype, stream)
+    assert lib.mase_gemm_mxfp_scaled(p, p, 0, p, p, 4, None, p, 4, 4, 192, 1, 0, None) == -2   # K in whole 128-tiles
+    assert lib.mase_gemm_mxfp_scaled(p, p, 4, p, p, 4, None, p, 4, 4, 128, 1, 0, None) == -5   # A must be 8-bit
+    assert lib.mase_gemm_mxfp_scaled(p, p, 0, p, p, 2, None, p, 4, 4, 128, 1, 0, None) == -5   # fp6 not provided
+    assert lib.mase_gemm_mxfp_scaled(p, None, 0, p, p, 4, None, p, 4, 4, 128, 1, 0, None) == -1
+    assert lib.mase_gemm_mxfp_scaled(p, p, 0, p, p, 4, None, p, 4, 4, 128, 3, 0, None) == -4
+    assert lib.mase_gemm_mxfp_scaled(p, p, 0, p, p, 4, None, p, 0, 4, 128, 1, 0, None) == 0    # empty output
 
 
 @pytest.mark.parametrize("dtype,code", [(torch.float32, 0), (torch.bfloat16, 1), (torch.float16, 2)])
@@ -157,3 +169,26 @@ def test_product_does_not_import_the_oracle():
         for f in files:
             if f.endswith(".py"):
                 assert not re.search(r"^\s*(from|import)\s+oracle\b", open(os.path.join(dirpath, f)).read(), flags=re.M), f
+
+
+def test_packed_mxfp_weight_eligibility_and_decoder_layer_host_side():
+    """host logic that needs no GPU: which weights may take the block-scaled matrix instruction, and the synthetic
+    decoder layer's shape/flop bookkeeping (it runs on the CPU with plain nn.Linear)"""
+    from mase_amd.quantized.functional.mx_linear import PackedMXFPWeight
+    from mase_amd.workloads import DecoderLayer, DecoderLayerConfig
+
+    w = torch.zeros(64, 256)
+    assert not PackedMXFPWeight.eligible(w, 32, (2, 1))            # not on a GPU
+    assert not PackedMXFPWeight().valid_for(w)
+    cfg = DecoderLayerConfig(hidden_size=256, num_heads=2, head_dim=128, intermediate_size=512)
+    layer = DecoderLayer(cfg, dtype=torch.bfloat16, seed=3)
+    again = DecoderLayer(cfg, dtype=torch.bfloat16, seed=3)
+    assert torch.equal(layer.down_proj.weight, again.down_proj.weight)
+    x = torch.randn(2, 16, 256).bfloat16()
+    with torch.no_grad():
+        y = layer(x)
+        # causal: the first 8 positions do not depend on the rest
+        y8 = layer(x[:, :8])
+    assert y.shape == x.shape and y.dtype == torch.bfloat16
+    assert (y[:, :8].float() - y8.float()).abs().max() < 0.1
+    assert DecoderLayer(DecoderLayerConfig(), dtype=torch.bfloat16, device="meta").linear_flops(16384) == pytest.approx(6.632e12, rel=1e-3)
