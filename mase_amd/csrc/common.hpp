@@ -21,12 +21,15 @@ __device__ __forceinline__ float bits2f(uint32_t b) { return __builtin_bit_cast(
 __device__ __forceinline__ uint32_t f2bits(float f) { return __builtin_bit_cast(uint32_t, f); }
 
 // fp32 -> bf16 bits, round-to-nearest-even (NaN kept quiet)
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  uint32_t b = f2bits(f);
-  uint32_t r = (b + 0x7FFFu + ((b >> 16) & 1u)) >> 16;
-  return ((b & 0x7FFFFFFFu) > 0x7F800000u) ? ((b >> 16) | 0x40u) : r;
+// fp32 -> bf16, round-to-nearest-even, with the hardware conversion of this part (two values per instruction,
+// first operand in the low half); NaN stays NaN
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
+  uint32_t r;
+  asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+  return r;
 }
-__device__ __forceinline__ float round_to_bf16(float f) { return bits2f(f32_to_bf16_bits(f) << 16); }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) { return f32x2_to_bf16x2_bits(f, 0.0f) & 0xFFFFu; }
+__device__ __forceinline__ float round_to_bf16(float f) { return bits2f(f32x2_to_bf16x2_bits(0.0f, f) & 0xFFFF0000u); }
 // fp32 -> fp16 bits, round-to-nearest-even.  Issued as an explicit instruction: when the compiler sees
 // "(half)(a * b)" it fuses the pair into a mixed-precision fma with a +0 addend, which turns a -0 product
 // into +0 and so loses the sign of zero that the reference keeps.
@@ -83,10 +86,10 @@ template <> struct DTypeTraits<MASE_DT_BF16> {
   }
   __device__ static __forceinline__ uint4 pack(const float* x) {
     uint4 v;
-    v.x = f32_to_bf16_bits(x[0]) | (f32_to_bf16_bits(x[1]) << 16);
-    v.y = f32_to_bf16_bits(x[2]) | (f32_to_bf16_bits(x[3]) << 16);
-    v.z = f32_to_bf16_bits(x[4]) | (f32_to_bf16_bits(x[5]) << 16);
-    v.w = f32_to_bf16_bits(x[6]) | (f32_to_bf16_bits(x[7]) << 16);
+    v.x = f32x2_to_bf16x2_bits(x[0], x[1]);
+    v.y = f32x2_to_bf16x2_bits(x[2], x[3]);
+    v.z = f32x2_to_bf16x2_bits(x[4], x[5]);
+    v.w = f32x2_to_bf16x2_bits(x[6], x[7]);
     return v;
   }
   __device__ static __forceinline__ float load1(const void* p, size_t i) {

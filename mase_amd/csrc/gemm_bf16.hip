@@ -251,8 +251,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
                 *(float4*)((float*)p.C + o) = make_float4(v[0], v[1], v[2], v[3]);
               } else if constexpr (OUT_DT == MASE_DT_BF16) {
                 uint2 w;
-                w.x = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
-                w.y = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
+                w.x = f32x2_to_bf16x2_bits(v[0], v[1]);
+                w.y = f32x2_to_bf16x2_bits(v[2], v[3]);
                 *(uint2*)((uint16_t*)p.C + o) = w;
               } else {
                 uint2 w;

@@ -11,7 +11,7 @@ namespace mase {
 namespace {
 
 // ---------------------------------------------------------------------------------------------
-// generic driver: 8 elements per work-item through 16-byte accesses, scalar tail
+// generic driver: 8 elements per lane through 16-byte accesses, one element per lane for the tail
 // ---------------------------------------------------------------------------------------------
 template <int DT>
 __device__ __forceinline__ void load8(const void* p, size_t i8, float* x) {
@@ -38,33 +38,38 @@ __device__ __forceinline__ void store8(void* p, size_t i8, const float* y) {
   }
 }
 
+// One item of 8 elements per lane (16 bytes of a 16-bit type, 32 of fp32), 64-lane work-groups: the shape
+// that streams best on this part.  Lanes past the vector part each take one element of the unaligned tail.
+// Every lane runs the functor on all 8 slots (the log2 lookups inside are wave-wide register permutes and
+// need all lanes present); unused slots hold 1.0.
+constexpr int kEwThreads = 64;
+
 template <int DTI, int DTO, typename F>
-__global__ __launch_bounds__(kThreads) void elementwise_kernel(const void* __restrict__ in, void* __restrict__ out,
-                                                               size_t n8, size_t numel, F f) {
-  __shared__ uint32_t lds_tab[F::kUsesTable ? MASE_LOG2_TABLE_WORDS : 1];
-  if constexpr (F::kUsesTable) {
-    for (int i = threadIdx.x; i < MASE_LOG2_TABLE_WORDS; i += kThreads) lds_tab[i] = f.tab[i];
-    __syncthreads();
-  }
-  size_t t = (size_t)blockIdx.x * kThreads + threadIdx.x;
-  if (t < n8) {
-    float x[8], y[8];
-    load8<DTI>(in, t, x);
+__global__ __launch_bounds__(kEwThreads) void elementwise_kernel(const void* __restrict__ in, void* __restrict__ out,
+                                                                 size_t n8, size_t numel, F f) {
+  WaveLog2 meta;
+  if constexpr (F::kUsesTable) meta.init(f.tab, F::kTableHalf);
+  const size_t t = (size_t)blockIdx.x * kEwThreads + threadIdx.x;
+  const size_t tail = n8 * 8 + (t - n8);
+  const bool vec = t < n8;
+  const bool one = !vec && tail < numel;
+  float x[8], y[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) y[j] = f(x[j], lds_tab);
-    store8<DTO>(out, t, y);
-  } else {
-    size_t i = n8 * 8 + (t - n8);
-    if (i < numel) DTypeTraits<DTO>::store1(out, i, f(DTypeTraits<DTI>::load1(in, i), lds_tab));
-  }
+  for (int j = 0; j < 8; ++j) x[j] = 1.0f;
+  if (vec) load8<DTI>(in, t, x);
+  else if (one) x[0] = DTypeTraits<DTI>::load1(in, tail);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) y[j] = f(x[j], meta);
+  if (vec) store8<DTO>(out, t, y);
+  else if (one) DTypeTraits<DTO>::store1(out, tail, y[0]);
 }
 
 template <int DTI, int DTO, typename F>
 int launch_elementwise(const void* in, void* out, size_t numel, const F& f, hipStream_t st) {
   size_t n8 = (aligned16(in) && aligned16(out)) ? numel / 8 : 0;
   size_t threads = n8 + (numel - n8 * 8);
-  hipLaunchKernelGGL((elementwise_kernel<DTI, DTO, F>), dim3(blocks_for(threads, kThreads)), dim3(kThreads), 0, st, in,
-                     out, n8, numel, f);
+  hipLaunchKernelGGL((elementwise_kernel<DTI, DTO, F>), dim3(blocks_for(threads, kEwThreads)), dim3(kEwThreads), 0, st,
+                     in, out, n8, numel, f);
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
 
@@ -82,11 +87,12 @@ __device__ __forceinline__ float clamp_cmp(float a, float lo, float hi) {
 template <int DT>
 struct IntegerOp {
   static constexpr bool kUsesTable = false;
+  static constexpr int kTableHalf = 0;
   const uint32_t* tab;
   int frac;
   int use_floor;
   float lo, hi;
-  __device__ __forceinline__ float operator()(float x, const uint32_t*) const {
+  __device__ __forceinline__ float operator()(float x, const WaveLog2&) const {
     float t = DTypeTraits<DT>::round(ldexpf(x, frac));  // x * 2^f underflows differently in narrow T
     float r = use_floor ? floorf(t) : rintf(t);
     r = clamp_cmp(r, lo, hi);
@@ -101,6 +107,7 @@ template <int DT, bool IEEE>
 struct MinifloatOp {
   using TR = DTypeTraits<DT>;
   static constexpr bool kUsesTable = true;
+  static constexpr int kTableHalf = IEEE ? kLog2TabHalf : 0;  // floor thresholds (ieee) or ceil thresholds (denorm)
   const uint32_t* tab;
   int mb;
   float e_lo, e_hi;  // exponent clamp (as floats; representable in every T for exponent_width <= 8)
@@ -112,11 +119,24 @@ struct MinifloatOp {
   __device__ static __forceinline__ float R(float f) { return TR::round(f); }
 
   // library log2 of a T value followed by ceil (denorm) or floor (ieee), as a float
-  __device__ __forceinline__ float log2_rounded(float l, const uint32_t* t) const {
-    uint32_t b = f2bits(l);
+  __device__ __forceinline__ float log2_rounded(float l, const WaveLog2& w) const {
+    const uint32_t b = f2bits(l);
+    // the lookup runs for every lane (wave-wide register permute), on a stand-in for zero / non-finite values
+    const bool special = (b == 0) || (b >= 0x7F800000u);
+    const uint32_t bb = special ? 0x3F800000u : b;
+    const float k = (float)(IEEE ? floor_log2_lib(bb, tab, w) : ceil_log2_lib(bb, tab, w));
     if (b == 0) return -__builtin_inff();
     if (b >= 0x7F800000u) return (b == 0x7F800000u) ? __builtin_inff() : qnan();  // l >= 0 here or NaN
-    return (float)(IEEE ? floor_log2_lib(b, t) : ceil_log2_lib(b, t));
+    return k;
+  }
+  // x / p for p = 2^k evaluated in T: an exact scaling while p is a finite non-zero power of two (the quotient
+  // of an IEEE division by a power of two is the correctly rounded scaled value, which is what ldexp gives);
+  // zero, infinite or NaN p take the division
+  __device__ static __forceinline__ float div_pow2(float x, float p) {
+    const uint32_t pb = f2bits(p);
+    const uint32_t ex = pb >> 23;  // p >= 0 here
+    if (__builtin_expect((pb & 0x7FFFFFu) == 0 && ex >= 1 && ex <= 254, 1)) return ldexpf(x, 127 - (int)ex);
+    return x / p;
   }
   // 2^e evaluated in T for an integer-valued float e
   __device__ static __forceinline__ float pow2_T(float e) {
@@ -126,26 +146,27 @@ struct MinifloatOp {
     return R(ldexpf(1.0f, (int)e));
   }
 
-  __device__ __forceinline__ float operator()(float x, const uint32_t* t) const {
+  __device__ __forceinline__ float operator()(float x, const WaveLog2& t) const {
     float xs = R(x + 1e-9f);
     float sgn = (xs > 0.0f) ? 1.0f : ((xs < 0.0f) ? -1.0f : xs);
     float val = fabsf(x);
     float l = R(val + 1e-9f);
     float e = clamp_cmp(log2_rounded(l, t), e_lo, e_hi);
     float p2 = pow2_T(e);
-    float man = R(val / p2);
+    float man = R(div_pow2(val, p2));
     float mant;
     if constexpr (!IEEE) {
       float q = clamp_cmp(rintf(R(man * shift)), 0.0f, qmax);
-      mant = R(q / shift);
+      mant = R(ldexpf(q, -mb));  // q / 2^mb
     } else {
       bool normal = !(e == neg_bias);
       float ms = R(man * shift);
       float a1 = clamp_cmp(rintf(R(ms - shift)), 0.0f, qmax);
-      float a2 = clamp_cmp(rintf(R(ms / 2.0f)), 0.0f, qmax);
+      float a2 = clamp_cmp(rintf(R(ms * 0.5f)), 0.0f, qmax);
       float q = normal ? R(a1 + R(0.0f * a2)) : R(R(0.0f * a1) + a2);
-      float m1 = R(1.0f + R(q / shift));
-      float m2 = R(R(q / shift) * 2.0f);
+      const float qs = R(ldexpf(q, -mb));  // q / 2^mb
+      float m1 = R(1.0f + qs);
+      float m2 = R(qs * 2.0f);
       mant = normal ? R(m1 + R(0.0f * m2)) : R(R(0.0f * m1) + m2);
     }
     float y = R(R(sgn * p2) * mant);
@@ -159,9 +180,10 @@ struct MinifloatOp {
 // ---------------------------------------------------------------------------------------------
 struct MinifloatMxOp {
   static constexpr bool kUsesTable = false;
+  static constexpr int kTableHalf = 0;
   const uint32_t* tab;
   MinifloatMxFmt m;
-  __device__ __forceinline__ float operator()(float x, const uint32_t*) const {
+  __device__ __forceinline__ float operator()(float x, const WaveLog2&) const {
     return minifloat_mx_decode(minifloat_mx_encode(x, m), m);
   }
 };
