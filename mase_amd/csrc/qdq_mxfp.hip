@@ -53,8 +53,8 @@ __device__ __forceinline__ float flush_subnormal(float x) {
 //   fraction: 23 -> 15 bits by truncation, 15 -> F bits round-half-even; a carry out of the fraction is OR-ed
 //   into the exponent field (lost when that field is odd), exponent field 0 takes the truncating shift
 //   value = code's [exponent|fraction] field moved to fp32's, exponent rebased by sh + 127 - bias
-// Returns false (caller takes mxfp_element) when t / 2^sh leaves the fp32 normal range or the format's
-// exponent range, which only happens for elements more than 2^100 below the block maximum or clamped scales.
+// Takes the raw (unflushed) input bits.  Returns false (caller takes mxfp_element) when t / 2^sh leaves the
+// fp32 normal range, which only happens for elements more than 2^100 below the block maximum.
 __device__ __forceinline__ bool mxfp_element_fast(uint32_t xb, int sh, const MxfpParams& p, uint32_t& code,
                                                   uint32_t& ybits) {
   const int F = p.m.F;
@@ -68,21 +68,32 @@ __device__ __forceinline__ bool mxfp_element_fast(uint32_t xb, int sh, const Mxf
   const uint32_t cn = ((uint32_t)ye << F) | yf;
   const uint32_t cs = yf ? ((yf | (1u << F)) >> 1) : 0u;
   uint32_t c = ye > 0 ? cn : (ye == 0 ? cs : 0u);
-  if (ab == 0) c = 0;
+  const bool zero = (ab >> 23) == 0;  // zero or an fp32 subnormal, which the reference flushes to +0
+  if (zero) c = 0;
   // decode: normal codes move as a bit field; codes with exponent field 0 are integers times a power of two
   const uint32_t yn = (c << (23 - F)) + ((uint32_t)(sh + 127 - p.m.bias) << 23);
   const uint32_t ys = f2bits(ldexpf((float)c, 1 - p.m.bias - F + sh));
-  ybits = sgn32 | ((c >> F) != 0 ? yn : ys);
-  code = c | (sgn32 >> (31 - p.m.E - F));
-  return (ab == 0) || (ef > 0 && ye <= p.m.e_hi);
+  const uint32_t sg = zero ? 0u : sgn32;
+  ybits = sg | ((c >> F) != 0 ? yn : ys);
+  code = c | (sg >> (31 - p.m.E - F));
+  // ye <= e_hi always holds in a regular block: sh >= floor(log2 max) - el_emax unless clamped from above,
+  // which fp32 exponents cannot reach
+  return zero || ef > 0;
 }
 
 // one element of a block in any state: fast path when it applies, else the step-by-step functions
-__device__ __forceinline__ uint32_t mxfp_element_bits(float t, int state, int sh, const MxfpParams& p, uint32_t& code) {
+__device__ __forceinline__ uint32_t mxfp_element_bits(float x, int state, int sh, const MxfpParams& p, uint32_t& code) {
   uint32_t yb;
-  const bool ok = mxfp_element_fast(f2bits(t), sh, p, code, yb);
-  if (__builtin_expect(state != 1 || !ok, 0)) yb = f2bits(mxfp_element(t, state, sh, p, code));
+  const bool ok = mxfp_element_fast(f2bits(x), sh, p, code, yb);
+  if (__builtin_expect(state != 1 || !ok, 0)) yb = f2bits(mxfp_element(flush_subnormal(x), state, sh, p, code));
   return yb;
+}
+
+// largest magnitude (fp32 bits) of the flushed elements of one 16-byte input vector
+template <int DTI>
+__device__ __forceinline__ uint32_t vec_flushed_absmax(const uint4& v) {
+  const uint32_t m = vec_absmax_bits<DTI>(v);
+  return ((m & 0x7F800000u) == 0) ? 0u : m;  // a subnormal maximum means every element is flushed
 }
 
 // One 16-byte vector of the wider side per lane, 64-lane work-groups (the shape that streams best on this
@@ -104,24 +115,27 @@ __global__ __launch_bounds__(kVecThreads) void mxfp_qdq_vec_kernel(const void* _
   meta.init(p.tab, kLog2TabHalf);
   float x[V], y[V];
   uint32_t c[V];
+  uint4 raw[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
   if (live) {
     if constexpr (TI::kVec == V) {
-      TI::unpack(load_nt((const uint4*)in + idx), x);
+      raw[0] = load_nt((const uint4*)in + idx);
     } else {  // fp32 input, 8 per item
-      TI::unpack(load_nt((const uint4*)in + 2 * idx), x);
-      TI::unpack(load_nt((const uint4*)in + 2 * idx + 1), x + 4);
+      raw[0] = load_nt((const uint4*)in + 2 * idx);
+      raw[1] = load_nt((const uint4*)in + 2 * idx + 1);
     }
-  } else {
-#pragma unroll
-    for (int j = 0; j < V; ++j) x[j] = 0.0f;
   }
-#pragma unroll
-  for (int j = 0; j < V; ++j) x[j] = flush_subnormal(x[j]);
+  TI::unpack(raw[0], x);
+  if constexpr (TI::kVec != V) TI::unpack(raw[1], x + 4);
 #pragma unroll
   for (int s = 0; s < SUB; ++s) {
     uint32_t m = 0;
+    if constexpr (SUB == 1) {  // the lane's whole item belongs to one block: packed maximum of the raw vector(s)
+      m = vec_flushed_absmax<DTI>(raw[0]);
+      if constexpr (TI::kVec != V) m = max(m, vec_flushed_absmax<DTI>(raw[1]));
+    } else {
 #pragma unroll
-    for (int j = 0; j < EPS; ++j) m = max(m, f2bits(x[s * EPS + j]) & 0x7FFFFFFFu);
+      for (int j = 0; j < EPS; ++j) m = max(m, f2bits(flush_subnormal(x[s * EPS + j])) & 0x7FFFFFFFu);
+    }
     m = group_max_u32<LPB>(m);
     int sh = 0;
     const int state = mxfp_block_scale(m, p, sh, meta);
@@ -261,23 +275,19 @@ __global__ __launch_bounds__(64) void mxfp_pack_kernel(const void* __restrict__ 
   WaveLog2 meta;
   meta.init(p.tab, kLog2TabHalf);
   float x[8];
+  uint4 raw[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
   if (live) {
     if constexpr (TI::kVec == 8) {
-      TI::unpack(load_nt((const uint4*)in + idx), x);
+      raw[0] = load_nt((const uint4*)in + idx);
     } else {
-      TI::unpack(load_nt((const uint4*)in + 2 * idx), x);
-      TI::unpack(load_nt((const uint4*)in + 2 * idx + 1), x + 4);
+      raw[0] = load_nt((const uint4*)in + 2 * idx);
+      raw[1] = load_nt((const uint4*)in + 2 * idx + 1);
     }
-  } else {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) x[j] = 0.0f;
   }
-  uint32_t m = 0;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    x[j] = flush_subnormal(x[j]);
-    m = max(m, f2bits(x[j]) & 0x7FFFFFFFu);
-  }
+  TI::unpack(raw[0], x);
+  if constexpr (TI::kVec != 8) TI::unpack(raw[1], x + 4);
+  uint32_t m = vec_flushed_absmax<DTI>(raw[0]);
+  if constexpr (TI::kVec != 8) m = max(m, vec_flushed_absmax<DTI>(raw[1]));
   m = group_max_u32<4>(m);
   int sh = 0;
   const int state = mxfp_block_scale(m, p, sh, meta);
