@@ -34,6 +34,26 @@ def test_gemm_bf16_tn(dev, M, N, K, out_dtype):
     assert rel_err(yb2.cpu(), ref + bias.bfloat16().double()) < tol
 
 
+@pytest.mark.parametrize("M,N,K", [(4096, 8192, 192), (4352, 4352, 128), (2048, 8448, 64), (4100, 4200, 320)])
+def test_gemm_bf16_tn_several_tiles_per_work_group(dev, M, N, K):
+    """more 256x256 output tiles than CUs: every work-group walks several tiles and its K-tile stream crosses from
+    one output tile to the next (tile counts divisible by 8 and not, K of 1, 2, 3 and 5 tiles).  Small-integer
+    operands make every partial sum exact, so the result must equal the integer product bit for bit."""
+    from mase_amd._gemm import gemm_bf16_tn
+
+    g = torch.Generator().manual_seed(M + N + K)
+    a = torch.randint(-16, 17, (M, K), generator=g).float()
+    b = torch.randint(-16, 17, (N, K), generator=g).float()
+    bias = torch.randint(-8, 9, (N,), generator=g).float()
+    print(f"gemm multi-tile M={M} N={N} K={K}", flush=True)
+    ad, bd = a.bfloat16().to(dev), b.bfloat16().to(dev)
+    ref = (ad.float() @ bd.float().t()).cpu()   # exact in fp32 as well: |sums| < 2^24
+    assert torch.equal(gemm_bf16_tn(ad, bd, None, torch.float32).cpu(), ref)
+    assert torch.equal(gemm_bf16_tn(ad, bd, bias.to(dev), torch.float32).cpu(), ref + bias)
+    yb = gemm_bf16_tn(ad, bd, None, torch.bfloat16).cpu()
+    assert torch.equal(yb, ref.bfloat16())
+
+
 def test_gemm_exact_on_small_integers(dev):
     """integer-valued operands with small K: every product and partial sum is exact in fp32, so the result
     must equal the integer matrix product bit for bit whatever the summation order"""

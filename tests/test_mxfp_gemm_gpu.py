@@ -101,3 +101,26 @@ def test_gemm_mxfp_exact_small_integers(dev):
     assert torch.equal(decode_ocp(ac, asc, (4, 3)), a.double()) and torch.equal(decode_ocp(bc, bsc, (2, 1)), b.double())
     y = gemm_mxfp_scaled(ac, asc, (4, 3), bc, bsc, (2, 1), None, torch.float32)
     assert torch.equal(y.cpu().double(), a.double() @ b.double().t())
+
+
+@pytest.mark.parametrize("bfmt", [(2, 1), (4, 3)])
+@pytest.mark.parametrize("M,N,K", [(4096, 8192, 384), (4352, 4352, 256), (2048, 8448, 128), (4100, 4200, 640)])
+def test_gemm_mxfp_several_tiles_per_work_group(dev, bfmt, M, N, K):
+    """more output tiles than CUs (the K-tile stream of a work-group crosses from one output tile to the next), with
+    K of 1 to 5 tiles; operands chosen so that every product and partial sum is exact: bit-exact result required"""
+    from mase_amd._gemm import gemm_mxfp_scaled, mxfp_pack
+
+    g = torch.Generator().manual_seed(M + N + K + bfmt[0])
+    a = torch.randint(-8, 9, (M, K), generator=g).float() * 32
+    a[:, ::32] = 256.0  # pins every block's scale
+    vals = torch.tensor([0, 1, 1.5, 2, 3, 4, 6, 6]) if bfmt == (2, 1) else torch.tensor([0, 32, 64, 96, 128, 160, 192, 224.0])
+    top = 6.0 if bfmt == (2, 1) else 256.0
+    b = vals[torch.randint(0, 8, (N, K), generator=g)] * torch.where(torch.rand(N, K, generator=g) < 0.5, -1.0, 1.0)
+    b[:, ::32] = top
+    print(f"mxfp gemm multi-tile {bfmt} M={M} N={N} K={K}", flush=True)
+    ad, bd = a.to(dev), b.to(dev)
+    ac, asc = mxfp_pack(ad, 4, 3)
+    bc, bsc = mxfp_pack(bd, *bfmt)
+    ref = (ad @ bd.t()).cpu()  # exact in fp32: multiples of 32 (or 1024) well below 2^24 units
+    y = gemm_mxfp_scaled(ac, asc, (4, 3), bc, bsc, bfmt, None, torch.float32)
+    assert torch.equal(y.cpu(), ref)
