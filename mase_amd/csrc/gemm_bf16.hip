@@ -284,7 +284,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   //     (lgkmcnt) and its copies of the next K tile have landed (vmcnt); barrier -> the next K tile is visible
   //     to all and nobody reads this one's stage any more
   //   step 3: MFMAs, interleaved with the LDS reads of step 0 of the next K tile and the 16 copies of the K tile
-  //     after next (into the stage just vacated), which then have a whole K tile's worth of MFMAs to land
+  //     after next (into the stage just vacated), which then have a whole K tile's worth of MFMAs to land.
+  //     One copy per MFMA slot: issuing them in a shorter burst makes their data arrive in a burst too, the LDS
+  //     is then busy with the writes when the wavefronts want their fragment reads, and the wavefronts drift
+  //     apart (measured: the barrier costs nothing without the copies and a quarter of the loop with them).
   // The barrier is a bare s_barrier: the fence of __syncthreads() would wait for all copies in flight.
   // The body must stay a single basic block: with a branch inside, the compiler sinks the MFMAs (whose
   // results are only consumed by the next iteration) below it and the interleave is lost.  Hence the copy
@@ -308,12 +311,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
         if (s < kSteps - 1) {
           if (t < 8) fr[nxt][t] = load_frag(stage, s + 1, t);
         } else {
-          if (t < 8) {
-            fr[nxt][t] = load_frag(stage ^ 1, 0, t);
-          } else {  // the 16 copies of the K tile after next, two per MFMA slot, into the stage just vacated
-            issue_copy(2 * (t - 8));
-            issue_copy(2 * (t - 8) + 1);
-          }
+          if (t < 8) fr[nxt][t] = load_frag(stage ^ 1, 0, t);
+          issue_copy(t);  // the 16 copies of the K tile after next, one per MFMA slot, into the stage just vacated
         }
         __builtin_amdgcn_sched_barrier(0);
       }
