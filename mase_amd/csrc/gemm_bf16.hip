@@ -38,7 +38,7 @@ constexpr int kTileBytes = BM * kRowBytes;        // 32 KB per operand per stage
 constexpr int kStageBytes = 2 * kTileBytes;       // A then B
 constexpr int kWaveCopies = kTileBytes / 1024 / 4;  // copies per wavefront per operand per K tile = 8
 constexpr int kCopies = 2 * kWaveCopies;          // async copies one wavefront issues per K tile = 16
-constexpr int kSteps = BK / 16;                   // MFMA K steps per K tile = 4
+constexpr int kSteps = BK / 16;                   // MFMA K steps per K tile = 4                   // MFMA K steps per K tile = 4
 // epilogue staging, separate from the stages: per wavefront 8 rows x 64 columns of fp32, row stride 68 floats
 constexpr int kStgStride = 68;
 constexpr int kStgWave = 8 * kStgStride * 4;
@@ -277,24 +277,26 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
 
   // Software pipeline, written out instruction by instruction and pinned with scheduling barriers, because a
   // wavefront issues in order: an MFMA occupies the matrix pipe for 32 cycles, and whatever else has to be
-  // issued (LDS reads of the next K step, async copies of the K tile after next) must sit *between* MFMAs to
-  // be free.  Per K tile (4 steps of 16 MFMAs, fragment sets ping-pong between fr[0] and fr[1]):
-  //   steps 0..2: MFMAs of step s, interleaved with the 8 LDS reads of step s+1
-  //   hand-over (after the MFMAs of step 2 are issued): this wavefront's reads of the K tile are complete
+  // issued (LDS reads of later K steps, async copies of the K tile after next) must sit *between* MFMAs to be
+  // free.  Per K tile: 4 steps of 16 MFMAs, one fragment set fr[s] per step:
+  //   step 0: MFMAs on fr[0], interleaved with the 8 LDS reads of step 1
+  //   step 1: MFMAs on fr[1], interleaved with the 16 LDS reads of steps 2 and 3
+  //   hand-over (after the MFMAs of step 1 are issued): this wavefront's reads of the K tile are complete
   //     (lgkmcnt) and its copies of the next K tile have landed (vmcnt); barrier -> the next K tile is visible
   //     to all and nobody reads this one's stage any more
-  //   step 3: MFMAs, interleaved with the LDS reads of step 0 of the next K tile and the 16 copies of the K tile
-  //     after next (into the stage just vacated), which then have a whole K tile's worth of MFMAs to land.
-  //     One copy per MFMA slot: issuing them in a shorter burst makes their data arrive in a burst too, the LDS
-  //     is then busy with the writes when the wavefronts want their fragment reads, and the wavefronts drift
-  //     apart (measured: the barrier costs nothing without the copies and a quarter of the loop with them).
+  //   steps 2, 3: MFMAs on fr[2], fr[3], interleaved with the LDS reads of step 0 of the next K tile and the 16
+  //     copies of the K tile after next into the stage just vacated, one every other MFMA slot.
+  // Handing the stage over half-way through the K tile (which costs two more fragment sets) lets the copies be
+  // issued over two steps instead of one: issued in a burst their data arrives in a burst, the LDS is then busy
+  // with the writes when the wavefronts want their fragment reads, and the wavefronts drift apart (measured:
+  // the barrier costs nothing without the copies and a quarter of the loop with them in a 16-slot burst).
   // The barrier is a bare s_barrier: the fence of __syncthreads() would wait for all copies in flight.
   // The body must stay a single basic block: with a branch inside, the compiler sinks the MFMAs (whose
   // results are only consumed by the next iteration) below it and the interleave is lost.  Hence the copy
   // stream is advanced by a caller-supplied, branch-free step.
-  // The epilogue's stores count in vmcnt like the copies, so the first hand-over of an output tile may also
-  // wait for the previous tile's stores to be acknowledged; by then they have had three K steps to drain.
-  bf16x8_t fr[2][8];
+  // The epilogue's stores count in vmcnt like the copies, so the first hand-over of an output tile also waits
+  // for the previous tile's stores to be acknowledged.
+  bf16x8_t fr[4][8];
   wait_vmcnt<kCopies>();  // K tile 0 landed; K tile 1 may still be in flight
   asm volatile("s_barrier" ::: "memory");
 #pragma unroll
@@ -303,20 +305,24 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   auto k_iteration = [&](auto&& advance) __attribute__((always_inline)) {
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
-      const int cur = s & 1, nxt = cur ^ 1;
 #pragma unroll
       for (int t = 0; t < 16; ++t) {
-        acc[t >> 2][t & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[cur][t >> 2], fr[cur][4 + (t & 3)],
+        acc[t >> 2][t & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[s][t >> 2], fr[s][4 + (t & 3)],
                                                                      acc[t >> 2][t & 3], 0, 0, 0);
-        if (s < kSteps - 1) {
-          if (t < 8) fr[nxt][t] = load_frag(stage, s + 1, t);
+        if (s == 0) {
+          if (t < 8) fr[1][t] = load_frag(stage, 1, t);
+        } else if (s == 1) {
+          if (t < 8) fr[2][t] = load_frag(stage, 2, t);
+          else fr[3][t - 8] = load_frag(stage, 3, t - 8);
+        } else if (s == 2) {
+          if (t < 8) fr[0][t] = load_frag(stage ^ 1, 0, t);
+          if (t & 1) issue_copy(t >> 1);
         } else {
-          if (t < 8) fr[nxt][t] = load_frag(stage ^ 1, 0, t);
-          issue_copy(t);  // the 16 copies of the K tile after next, one per MFMA slot, into the stage just vacated
+          if (t & 1) issue_copy(8 + (t >> 1));
         }
         __builtin_amdgcn_sched_barrier(0);
       }
-      if (s == kSteps - 2) {
+      if (s == 1) {
         wait_vmcnt<0>();
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
