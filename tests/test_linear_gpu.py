@@ -201,12 +201,20 @@ def test_linear_block_fp_integer_minifloat(dev):
     m = LinearBlockFP(64, 48, device=dev, config=dict(bfp))
     m.load_state_dict(sd)
     for x in (x3, x2):
-        assert rel_err(m(x.to(dev)), OL.linear_block_fp(x, w, b, bfp)) < 1e-5
+        assert rel_err(m(x.to(dev)), OL.linear_block_fp(x, w, b, bfp)) < 1e-5      # grad recorded: library GEMM
+        with torch.no_grad():
+            assert rel_err(m(x.to(dev)), OL.linear_block_fp(x, w, b, bfp)) < 1e-5  # inference: matrix-core kernel
+    # training still works: straight-through quantizers + differentiable GEMM
+    xg = x2.to(dev).requires_grad_(True)
+    m(xg).sum().backward()
+    assert xg.grad is not None and m.weight.grad is not None and bool(torch.isfinite(m.weight.grad).all())
     icfg = {"weight_width": 8, "weight_frac_width": 6, "data_in_width": 8, "data_in_frac_width": 4, "bias_width": 8,
             "bias_frac_width": 5}
     mi = LinearInteger(64, 48, device=dev, config=dict(icfg))
     mi.load_state_dict(sd)
     assert rel_err(mi(x3.to(dev)), OL.linear_integer(x3, w, b, icfg)) < 1e-5
+    with torch.no_grad():
+        assert rel_err(mi(x3.to(dev)), OL.linear_integer(x3, w, b, icfg)) < 1e-5
     mo = LinearInteger(64, 48, device=dev, config={**icfg, "data_out_width": 8, "data_out_frac_width": 3}, floor=True)
     mo.load_state_dict(sd)
     ref = OL.linear_integer(x3, w, b, {**icfg, "data_out_width": 8, "data_out_frac_width": 3, "floor": True})
@@ -218,6 +226,38 @@ def test_linear_block_fp_integer_minifloat(dev):
         mm = cls(64, 48, device=dev, config=dict(mcfg))
         mm.load_state_dict(sd)
         assert rel_err(mm(x3.to(dev)), fn(x3, w, b, mcfg)) < 1e-5
+        with torch.no_grad():
+            assert rel_err(mm(x3.to(dev)), fn(x3, w, b, mcfg)) < 1e-5
+
+
+def test_linear_block_fp_integer_wide_formats_take_the_library_gemm(dev):
+    """widths beyond 9 bits are not exact in bf16: the forward must still match (library GEMM in the tensor dtype),
+    and the narrow formats must match in bf16 and fp16 tensors too"""
+    from mase_amd.quantized import LinearBlockFP, LinearInteger
+
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(3, 40, 128, generator=g)
+    w = torch.randn(72, 128, generator=g) * 0.1
+    b = torch.randn(72, generator=g)
+    for width, tol in ((12, 1e-5), (8, 1e-5)):
+        bfp = {f"{k}_{s}": v for k in ("weight", "data_in", "bias")
+               for s, v in (("width", width), ("exponent_width", 8), ("exponent_bias", None), ("block_size", [16]))}
+        m = LinearBlockFP(128, 72, device=dev, config=dict(bfp)).requires_grad_(False)
+        m.load_state_dict({"weight": w, "bias": b})
+        assert rel_err(m(x.to(dev)), OL.linear_block_fp(x, w, b, bfp)) < tol
+        icfg = {"weight_width": width, "weight_frac_width": width - 2, "data_in_width": width, "data_in_frac_width": width - 4,
+                "bias_width": width, "bias_frac_width": width - 3}
+        mi = LinearInteger(128, 72, device=dev, config=dict(icfg)).requires_grad_(False)
+        mi.load_state_dict({"weight": w, "bias": b})
+        assert rel_err(mi(x.to(dev)), OL.linear_integer(x, w, b, icfg)) < tol
+    for dtype in (torch.bfloat16, torch.float16):
+        bfp = {f"{k}_{s}": v for k in ("weight", "data_in", "bias")
+               for s, v in (("width", 8), ("exponent_width", 8), ("exponent_bias", None), ("block_size", [16]))}
+        m = LinearBlockFP(128, 72, device=dev, dtype=dtype, config=dict(bfp)).requires_grad_(False)
+        m.load_state_dict({"weight": w.to(dtype), "bias": b.to(dtype)})
+        e = rel_err(m(x.to(dtype).to(dev)), OL.linear_block_fp(x.to(dtype), w.to(dtype), b.to(dtype), bfp))
+        print(f"LinearBlockFP {dtype}: rel err {e:.3e}")
+        assert e < TOL
 
 
 class MLP(nn.Module):
