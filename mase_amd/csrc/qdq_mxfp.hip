@@ -55,6 +55,10 @@ __device__ __forceinline__ float flush_subnormal(float x) {
 //   value = code's [exponent|fraction] field moved to fp32's, exponent rebased by sh + 127 - bias
 // Takes the raw (unflushed) input bits.  Returns false (caller takes mxfp_element) when t / 2^sh leaves the
 // fp32 normal range, which only happens for elements more than 2^100 below the block maximum.
+// INLINE_SUB = false leaves codes with exponent field 0 (elements more than 2^(el_emax + bias) below the block
+// maximum) to the caller's slow path as well: right for the wide-exponent formats (e4m3, e5m2), where such
+// elements are rare, and it halves the instruction count; the narrow-exponent formats handle them in line.
+template <bool INLINE_SUB>
 __device__ __forceinline__ bool mxfp_element_fast(uint32_t xb, int sh, const MxfpParams& p, uint32_t& code,
                                                   uint32_t& ybits) {
   const int F = p.m.F;
@@ -66,6 +70,13 @@ __device__ __forceinline__ bool mxfp_element_fast(uint32_t xb, int sh, const Mxf
   const uint32_t m15 = (ab >> 8) & 0x7FFFu;
   const uint32_t yf = (m15 + ((1u << (shn - 1)) - 1u) + ((m15 >> shn) & 1u)) >> shn;  // 0 .. 2^F
   const uint32_t cn = ((uint32_t)ye << F) | yf;
+  if constexpr (!INLINE_SUB) {
+    const bool zero = (ab >> 23) == 0;  // zero or an fp32 subnormal, which the reference flushes to +0
+    const uint32_t yn = sgn32 | ((cn << (23 - F)) + ((uint32_t)(sh + 127 - p.m.bias) << 23));
+    ybits = zero ? 0u : yn;
+    code = zero ? 0u : (cn | (sgn32 >> (31 - p.m.E - F)));
+    return zero || ye > 0;  // ye > 0 implies ef > 0 (bias <= 127)
+  }
   const uint32_t cs = yf ? ((yf | (1u << F)) >> 1) : 0u;
   uint32_t c = ye > 0 ? cn : (ye == 0 ? cs : 0u);
   const bool zero = (ab >> 23) == 0;  // zero or an fp32 subnormal, which the reference flushes to +0
@@ -81,12 +92,23 @@ __device__ __forceinline__ bool mxfp_element_fast(uint32_t xb, int sh, const Mxf
   return zero || ef > 0;
 }
 
-// one element of a block in any state: fast path when it applies, else the step-by-step functions
-__device__ __forceinline__ uint32_t mxfp_element_bits(float x, int state, int sh, const MxfpParams& p, uint32_t& code) {
-  uint32_t yb;
-  const bool ok = mxfp_element_fast(f2bits(x), sh, p, code, yb);
-  if (__builtin_expect(state != 1 || !ok, 0)) yb = f2bits(mxfp_element(flush_subnormal(x), state, sh, p, code));
-  return yb;
+// N elements of one block in any state: fast path for all of them, and one (rarely taken) branch that redoes
+// the lane's elements with the step-by-step functions when the block is not regular or any element fell out
+// of the fast path's range
+template <bool INLINE_SUB, int N>
+__device__ __forceinline__ void mxfp_elements(const float* x, int state, int sh, const MxfpParams& p, uint32_t* code,
+                                              float* y) {
+  bool slow = state != 1;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    uint32_t yb;
+    slow |= !mxfp_element_fast<INLINE_SUB>(f2bits(x[j]), sh, p, code[j], yb);
+    y[j] = bits2f(yb);
+  }
+  if (__builtin_expect(slow, 0)) {
+#pragma unroll
+    for (int j = 0; j < N; ++j) y[j] = mxfp_element(flush_subnormal(x[j]), state, sh, p, code[j]);
+  }
 }
 
 // largest magnitude (fp32 bits) of the flushed elements of one 16-byte input vector
@@ -99,7 +121,7 @@ __device__ __forceinline__ uint32_t vec_flushed_absmax(const uint4& v) {
 // One 16-byte vector of the wider side per lane, 64-lane work-groups (the shape that streams best on this
 // part); a block of B elements spans LPB lanes, or a lane holds SUB blocks.  No lane leaves before the table
 // lookups: they are wave-wide register permutes.
-template <int DTI, int DTO, int LPB, int SUB>
+template <int DTI, int DTO, int LPB, int SUB, bool CODES>
 __global__ __launch_bounds__(kVecThreads) void mxfp_qdq_vec_kernel(const void* __restrict__ in, void* __restrict__ out,
                                                                    uint8_t* __restrict__ codes,
                                                                    uint8_t* __restrict__ scales, size_t n_vec,
@@ -139,9 +161,11 @@ __global__ __launch_bounds__(kVecThreads) void mxfp_qdq_vec_kernel(const void* _
     m = group_max_u32<LPB>(m);
     int sh = 0;
     const int state = mxfp_block_scale(m, p, sh, meta);
-#pragma unroll
-    for (int j = 0; j < EPS; ++j) y[s * EPS + j] = bits2f(mxfp_element_bits(x[s * EPS + j], state, sh, p, c[s * EPS + j]));
-    if (codes != nullptr && live) {
+    if (p.m.E >= 4)  // uniform: wide-exponent formats
+      mxfp_elements<false, EPS>(x + s * EPS, state, sh, p, c + s * EPS, y + s * EPS);
+    else
+      mxfp_elements<true, EPS>(x + s * EPS, state, sh, p, c + s * EPS, y + s * EPS);
+    if (CODES && live) {
       int sb = (state == 1) ? sh + 127 : (state == 0 ? 0 : 255);
       if constexpr (LPB > 1) {
         if ((idx & (LPB - 1)) == 0) scales[idx / LPB] = (uint8_t)sb;
@@ -157,7 +181,7 @@ __global__ __launch_bounds__(kVecThreads) void mxfp_qdq_vec_kernel(const void* _
     store_nt((uint4*)out + 2 * idx, TO::pack(y));
     store_nt((uint4*)out + 2 * idx + 1, TO::pack(y + 4));
   }
-  if (codes != nullptr) {
+  if constexpr (CODES) {
     if constexpr (V == 4) {
       ((uint32_t*)codes)[idx] = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
     } else {
@@ -201,7 +225,14 @@ int launch_mxfp(const void* in, void* out, uint8_t* codes, uint8_t* scales, size
     size_t n_vec = numel / V;
     dim3 grid(blocks_for(n_vec, (size_t)kVecThreads)), block(kVecThreads);
 #define MASE_MXFP_CASE(LPB_, SUB_)                                                                               \
-  hipLaunchKernelGGL((mxfp_qdq_vec_kernel<DTI, DTO, LPB_, SUB_>), grid, block, 0, st, in, out, codes, scales, n_vec, p)
+  do {                                                                                                           \
+    if (codes != nullptr)                                                                                        \
+      hipLaunchKernelGGL((mxfp_qdq_vec_kernel<DTI, DTO, LPB_, SUB_, true>), grid, block, 0, st, in, out, codes,  \
+                         scales, n_vec, p);                                                                      \
+    else                                                                                                         \
+      hipLaunchKernelGGL((mxfp_qdq_vec_kernel<DTI, DTO, LPB_, SUB_, false>), grid, block, 0, st, in, out, codes, \
+                         scales, n_vec, p);                                                                      \
+  } while (0)
     if (B >= V) {
       switch (B / V) {
         case 1: MASE_MXFP_CASE(1, 1); break;
@@ -292,8 +323,8 @@ __global__ __launch_bounds__(64) void mxfp_pack_kernel(const void* __restrict__ 
   int sh = 0;
   const int state = mxfp_block_scale(m, p, sh, meta);
   uint32_t c[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) mxfp_element_bits(x[j], state, sh, p, c[j]);
+  float y_unused[8];
+  mxfp_elements<(E < 4), 8>(x, state, sh, p, c, y_unused);
   // any element may hold the reserved code, not only the largest: a fraction carry that the encoder loses
   // in an odd exponent field leaves the block maximum below a neighbour's code
   uint32_t reserved = 0;
