@@ -1,5 +1,6 @@
 """``quantized_module_map``: the in-scope entries of the reference's registry
-(``chop/nn/quantized/modules/__init__.py:236-251, 388-408``), same keys."""
+(``chop/nn/quantized/modules/__init__.py:236-251, 334-335, 388-408``), same keys."""
+from .embedding import EmbeddingMXFP, EmbeddingMXInt
 from .linear import (
     LinearBlockFP,
     LinearInteger,
@@ -17,4 +18,6 @@ quantized_module_map = {
     "linear_minifloat_ieee": LinearMinifloatIEEE,
     "linear_mxint": LinearMXInt,
     "linear_mxfp": LinearMXFP,
+    "embedding_mxint": EmbeddingMXInt,
+    "embedding_mxfp": EmbeddingMXFP,
 }

@@ -25,6 +25,9 @@ Pinning status (what fixes each function besides reading the source):
   and ``mxfp_quantizer``           (``>> 8`` double rounding, lost carry in odd binades, truncating subnormals)
                                    are source-defined                                   -> parity unpinned (quirk regions)
 
+``tests/golden/known_answers.json`` holds small vectors computed with the exact scalar restatement; the vectorised
+restatement (and the kernels) must reproduce them bit for bit.
+
 The reference ships no golden vectors or value-asserting tests for this path, and running the reference
 to produce vectors was refused by the environment, so "parity unpinned" above means: restated from the
 source text (file:line cited at each function), cross-checked by an independent scalar restatement, but
