@@ -67,3 +67,42 @@ def test_embedding_mx_quantizes_only_looked_up_rows_bit_exactly(dev, dtype):
         with torch.no_grad():
             mb.weight.copy_(table.to(dev))
         assert_bits_equal(mb(idx.to(dev)), table[idx], "bypass")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_quantized_softmax_silu_rope_kvcache(dev, dtype):
+    """thin callers of the quantizers (reference functional/softmax.py, silu.py, rope.py, kvcache.py): the quantized
+    tensors are compared bit-exactly, the torch op applied on top within the library's CPU/GPU difference"""
+    import oracle as O
+    from mase_amd.quantized import functional as QF
+
+    g = torch.Generator().manual_seed(13)
+    x = (torch.randn(2, 4, 48, 64, generator=g) * 3).to(dtype)
+    fcfg = {"data_in_block_size": 32, "data_in_exponent_width": 4, "data_in_frac_width": 3}
+    icfg = {"data_in_block_size": 32, "data_in_width": 8}
+    mcfg = {"data_in_exponent_width": 4, "data_in_frac_width": 3}
+    q_fp = lambda t: O.mxfp_quantizer(t, 32, 4, 3)
+    q_int = lambda t: O.mxint_quantizer(t, 32, 8)
+    q_mf = lambda t: O.minifloat_quantizer_sim(t, 4, 3, True, "rn", None)
+    sm = lambda t: torch.softmax(t.float(), -1).to(t.dtype)
+    tol = 2e-6 if dtype == torch.float32 else 8e-3
+    xd = x.to(dev)
+    for fn, q, cfg in ((QF.softmax_mxfp, q_fp, fcfg), (QF.softmax_mxint, q_int, icfg), (QF.softmax_minifloat, q_mf, mcfg)):
+        assert rel_err(fn(xd, cfg), sm(q(x))) < tol
+    for fn, q, cfg in ((QF.silu_mxfp, q_fp, fcfg), (QF.silu_mxint, q_int, icfg), (QF.silu_minifloat, q_mf, mcfg)):
+        assert rel_err(fn(xd, cfg), torch.nn.functional.silu(q(x))) < tol
+    k, v = QF.kv_cache_mxfp(xd, xd * 0.5, fcfg)
+    assert_bits_equal(k, q_fp(x), "kv_cache_mxfp k")
+    assert_bits_equal(v, q_fp(x * 0.5), "kv_cache_mxfp v")
+    k, v = QF.kv_cache_mxint(xd, xd * 0.5, icfg)
+    assert_bits_equal(k, q_int(x), "kv_cache_mxint k")
+    # rotary embedding: cos/sin tables quantized, q/k untouched
+    t = torch.arange(48, dtype=torch.float32)
+    freqs = torch.outer(t, 1.0 / (10000 ** (torch.arange(0, 64, 2).float() / 64)))
+    emb = torch.cat((freqs, freqs), -1)
+    cos, sin = emb.cos()[None].to(dtype), emb.sin()[None].to(dtype)
+    for fn, q, cfg in ((QF.rope_mxfp, q_fp, fcfg), (QF.rope_mxint, q_int, icfg), (QF.rope_minifloat, q_mf, mcfg)):
+        qe, ke = fn(xd, xd * 2, cos.to(dev), sin.to(dev), cfg)
+        c, s_ = q(cos).unsqueeze(1), q(sin).unsqueeze(1)
+        rot = lambda u: torch.cat((-u[..., 32:], u[..., :32]), -1)
+        assert rel_err(qe, x * c + rot(x) * s_) < tol and rel_err(ke, (x * 2) * c + rot(x * 2) * s_) < tol
