@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident in HBM.
-Workloads (BASELINE.json configs):
+Workloads (the headline configurations):
     bfp_qdq      config 2 (default): block-FP quantize-dequantize, bf16 [8,2048,4096], width 8, exp 8, block [1,16]
     mxint_qdq    config 1: MXINT8 quantize-dequantize, fp32 [4096,4096], block 32
     mxint_linear config 3: MXINT8 Linear forward, 4096x4096x4096, fp32 in/out

@@ -58,12 +58,9 @@ const char* mase_error_string(int code);
  * (one per dtype), in device memory, MASE_LOG2_TABLE_WORDS uint32 words:
  *   tab[k+149]       largest normalised 23-bit mantissa M>0 with ceil(log2(2^k*(1+M/2^23))) == k, else 0
  *   tab[288+k+149]   smallest M with floor(log2(2^k*(1+M/2^23))) == k+1, else 0x800000
- * for k = floor(log2 v) in [-149, 127], plus three summary words per half that let a kernel skip the table
- * read for most inputs:
- *   tab[277], tab[278]           kb_lo, kb_hi: biased exponents k+149 in [kb_lo, kb_hi] have no ceil correction
- *   tab[279]                     the largest ceil threshold of any exponent
- *   tab[288+277], tab[288+278]   the same interval for floor;  tab[288+279] the smallest floor threshold
- * A table of {0.., 0, 276, 0} / {0x800000.., 0, 276, 0x800000} gives the exact integer answers.
+ * for k = floor(log2 v) in [-149, 127].  Words 277..279 of each half are reserved (the host tooling stores a
+ * summary there; the kernels do not read them).  A table of all 0 in the first half and all 0x800000 in the
+ * second gives the exact integer answers.  Kernels keep the entries for k in [-32, 31] in one register per lane.
  */
 
 /* MXINT quantize-dequantize over contiguous runs of `block_size` elements of a flat array.

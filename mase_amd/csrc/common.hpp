@@ -186,22 +186,7 @@ __device__ __forceinline__ uint32_t pack_bf16_exact(float lo, float hi) {
 //   tab[288 + k + 149]  smallest M for which floor(log2(2^k (1+M/2^23))) == k+1 (0x800000 when none)
 // ---------------------------------------------------------------------------------------------
 constexpr int kLog2TabHalf = 288;
-// Words 277..279 of each half summarise it so that the common case needs no per-lane table read:
-//   [277], [278]  k_lo+149, k_hi+149: exponents in [k_lo, k_hi] have no correction at all
-//   [279]         ceil half: largest threshold of any exponent; floor half: smallest threshold
-constexpr int kLog2MetaLo = 277, kLog2MetaHi = 278, kLog2MetaM = 279;
-
-struct Log2Meta {
-  int lo, hi;      // biased (k+149) exponent interval without corrections
-  uint32_t m;      // extreme threshold
-};
-__device__ __forceinline__ Log2Meta load_log2_meta(const uint32_t* __restrict__ tab, int half) {
-  Log2Meta r;
-  r.lo = (int)tab[half + kLog2MetaLo];
-  r.hi = (int)tab[half + kLog2MetaHi];
-  r.m = tab[half + kLog2MetaM];
-  return r;
-}
+// (Words 277..279 of each half hold a host-side summary of the table; the kernels do not read them.)
 
 __device__ __forceinline__ int split_pow2(uint32_t b, uint32_t& M) {
   int E = (int)(b >> 23);
@@ -219,15 +204,6 @@ __device__ __forceinline__ int ceil_log2_lib(uint32_t b, const uint32_t* __restr
   int k = split_pow2(b, M);
   if (M == 0) return k;
   return (M <= tab[k + 149]) ? k : k + 1;
-}
-// same, reading the table only for mantissas/exponents that can be corrected at all
-__device__ __forceinline__ int ceil_log2_lib(uint32_t b, const uint32_t* __restrict__ tab, const Log2Meta& meta) {
-  uint32_t M;
-  int k = split_pow2(b, M);
-  if (M == 0) return k;
-  int kb = k + 149;
-  if (M > meta.m || (kb >= meta.lo && kb <= meta.hi)) return k + 1;
-  return (M <= tab[kb]) ? k : k + 1;
 }
 
 // Wave-resident copy of the table entries for k in [-32, 31] (lane i holds k = i - 32), read with one
@@ -266,13 +242,6 @@ __device__ __forceinline__ int floor_log2_lib(uint32_t b, const uint32_t* __rest
   uint32_t M;
   int k = split_pow2(b, M);
   return (M >= tab[kLog2TabHalf + k + 149]) ? k + 1 : k;
-}
-__device__ __forceinline__ int floor_log2_lib(uint32_t b, const uint32_t* __restrict__ tab, const Log2Meta& meta) {
-  uint32_t M;
-  int k = split_pow2(b, M);
-  int kb = k + 149;
-  if (M < meta.m || (kb >= meta.lo && kb <= meta.hi)) return k;
-  return (M >= tab[kLog2TabHalf + kb]) ? k + 1 : k;
 }
 
 // 2^e as fp32 for e in [-149, 127]; callers handle e > 127 themselves

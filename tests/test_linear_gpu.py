@@ -51,7 +51,7 @@ def test_linear_mxint(dev, dtype, shape, out_f, bias):
 
 
 def test_linear_mxint_config3_full_size(dev):
-    """BASELINE config 3: activations [4096,4096] N(0,1), weight [4096,4096] N(0,0.02), bias zeros, fp32."""
+    """Headline configuration 3: activations [4096,4096] N(0,1), weight [4096,4096] N(0,0.02), bias zeros, fp32."""
     from mase_amd.quantized import LinearMXInt
 
     g = torch.Generator().manual_seed(2)
