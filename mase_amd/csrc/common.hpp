@@ -54,6 +54,12 @@ __device__ __forceinline__ void store_nt(uint4* p, const uint4& v) {
   __builtin_nontemporal_store(w, (u32x4_t*)p);
 }
 
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void store_nt(uint2* p, const uint2& v) {
+  u32x2_t w = {v.x, v.y};
+  __builtin_nontemporal_store(w, (u32x2_t*)p);
+}
+
 template <int DT> struct DTypeTraits;
 
 template <> struct DTypeTraits<MASE_DT_F32> {

@@ -97,7 +97,7 @@ __device__ __forceinline__ void store_vec(void* out, size_t idx, const float* y,
       o.x = f32_to_f16_bits(y[0]) | (f32_to_f16_bits(y[1]) << 16);
       o.y = f32_to_f16_bits(y[2]) | (f32_to_f16_bits(y[3]) << 16);
     }
-    ((uint2*)out)[idx] = o;
+    store_nt((uint2*)out + idx, o);
   }
 }
 
