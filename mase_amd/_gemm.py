@@ -7,6 +7,7 @@ from torch import Tensor
 from . import _lib
 
 GEMM_K_MULTIPLE = 64  # K tile of mase_gemm_bf16_tn
+OPERAND_BYTES_LIMIT = (1 << 32) - 1  # per-call operand size the GEMM entry points accept
 
 
 def gemm_bf16_tn(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dtype) -> Tensor:
@@ -27,11 +28,16 @@ def gemm_bf16_tn(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dty
     out = torch.empty((M, N), dtype=out_dtype, device=a.device)
     if bias is not None:
         bias = bias.contiguous()
-    rc = lib.mase_gemm_bf16_tn(
-        a.data_ptr(), b.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(), M, N, K,
-        _lib.DTYPE_CODE[out_dtype], _lib.DTYPE_CODE[bias.dtype] if bias is not None else 0, _lib.stream_ptr(a),
-    )
-    _lib.check(rc, "mase_gemm_bf16_tn")
+    # the kernel addresses an operand with 32-bit byte offsets: activations beyond 4 GiB go in row chunks
+    rows_per_call = max(1, min(M, (OPERAND_BYTES_LIMIT // (2 * K)) // 256 * 256 or 1))
+    for r0 in range(0, M, rows_per_call):
+        r1 = min(M, r0 + rows_per_call)
+        rc = lib.mase_gemm_bf16_tn(
+            a[r0:r1].data_ptr(), b.data_ptr(), bias.data_ptr() if bias is not None else None, out[r0:r1].data_ptr(),
+            r1 - r0, N, K, _lib.DTYPE_CODE[out_dtype], _lib.DTYPE_CODE[bias.dtype] if bias is not None else 0,
+            _lib.stream_ptr(a),
+        )
+        _lib.check(rc, "mase_gemm_bf16_tn")
     return out
 
 
@@ -72,10 +78,14 @@ def gemm_mxfp_scaled(a_codes: Tensor, a_scales: Tensor, a_fmt, b_codes: Tensor, 
     out = torch.empty((M, N), dtype=out_dtype, device=a_codes.device)
     if bias is not None:
         bias = bias.contiguous()
-    rc = lib.mase_gemm_mxfp_scaled(
-        a_codes.data_ptr(), a_scales.data_ptr(), MXFP_HW_FORMATS[tuple(a_fmt)], b_codes.data_ptr(), b_scales.data_ptr(),
-        MXFP_HW_FORMATS[tuple(b_fmt)], bias.data_ptr() if bias is not None else None, out.data_ptr(), M, N, K,
-        _lib.DTYPE_CODE[out_dtype], _lib.DTYPE_CODE[bias.dtype] if bias is not None else 0, _lib.stream_ptr(a_codes),
-    )
-    _lib.check(rc, "mase_gemm_mxfp_scaled")
+    rows_per_call = max(1, min(M, (OPERAND_BYTES_LIMIT // K) // 256 * 256 or 1))  # M*K < 2^32 per call
+    for r0 in range(0, M, rows_per_call):
+        r1 = min(M, r0 + rows_per_call)
+        rc = lib.mase_gemm_mxfp_scaled(
+            a_codes[r0:r1].data_ptr(), a_scales[r0:r1].data_ptr(), MXFP_HW_FORMATS[tuple(a_fmt)], b_codes.data_ptr(),
+            b_scales.data_ptr(), MXFP_HW_FORMATS[tuple(b_fmt)], bias.data_ptr() if bias is not None else None,
+            out[r0:r1].data_ptr(), r1 - r0, N, K, _lib.DTYPE_CODE[out_dtype],
+            _lib.DTYPE_CODE[bias.dtype] if bias is not None else 0, _lib.stream_ptr(a_codes),
+        )
+        _lib.check(rc, "mase_gemm_mxfp_scaled")
     return out

@@ -74,3 +74,24 @@ def test_gemm_c_abi_rejects_partial_k_tiles(dev):
     c = torch.zeros(4, 4, device=dev)
     rc = lib.mase_gemm_bf16_tn(a.data_ptr(), a.data_ptr(), None, c.data_ptr(), 4, 4, 96, 0, 0, None)
     assert rc == -2
+
+
+def test_gemm_wrappers_split_oversized_activations(dev, monkeypatch):
+    """operands beyond the per-call size limit of the C entry points are fed in row chunks (limit lowered here so
+    that a small problem exercises the split)"""
+    from mase_amd import _gemm
+
+    g = torch.Generator().manual_seed(3)
+    a = torch.randint(-8, 9, (1000, 128), generator=g).float()
+    b = torch.randint(-8, 9, (320, 128), generator=g).float()
+    ad, bd = a.bfloat16().to(dev), b.bfloat16().to(dev)
+    whole = _gemm.gemm_bf16_tn(ad, bd, None, torch.float32)
+    monkeypatch.setattr(_gemm, "OPERAND_BYTES_LIMIT", 2 * 128 * 300)   # -> 256 rows per call
+    assert torch.equal(_gemm.gemm_bf16_tn(ad, bd, None, torch.float32), whole)
+    assert torch.equal(whole.cpu(), a @ b.t())
+    monkeypatch.setattr(_gemm, "OPERAND_BYTES_LIMIT", (1 << 32) - 1)
+    ac, asc = _gemm.mxfp_pack((a * 32).to(dev), 4, 3)
+    bc, bsc = _gemm.mxfp_pack(b.to(dev), 4, 3)
+    whole = _gemm.gemm_mxfp_scaled(ac, asc, (4, 3), bc, bsc, (4, 3), None, torch.float32)
+    monkeypatch.setattr(_gemm, "OPERAND_BYTES_LIMIT", 128 * 300)
+    assert torch.equal(_gemm.gemm_mxfp_scaled(ac, asc, (4, 3), bc, bsc, (4, 3), None, torch.float32), whole)
