@@ -84,9 +84,11 @@ struct MxGemmGeom {
   static constexpr int kStage = kTileA + kTileB + 2 * 1024;  // + one scale dword per row for A and for B
   static constexpr int S = (kStage <= 53 * 1024) ? 3 : 2;
   // epilogue staging, separate from the stages (copies of the next tile are in flight during the epilogue):
-  // per wavefront 8 rows x 64 columns of fp32, row stride 68 floats (4 rows per half-wave)
-  static constexpr int kStgStride = 68;
-  static constexpr int kStgWave = 8 * kStgStride * 4;
+  // per wavefront two buffers of 8 rows x 32 columns of fp32 (4 rows per half-wave).  Row stride 32 floats is
+  // conflict-free both for the half-wave row writes and for the 16-lane phases of the 16-byte reads.
+  static constexpr int kStgStride = 32;
+  static constexpr int kStgBuf = 8 * kStgStride;       // floats per buffer
+  static constexpr int kStgWave = 2 * kStgBuf * 4;     // bytes per wavefront
   static constexpr int kLdsBytes = S * kStage + 4 * kStgWave;
 };
 
@@ -271,12 +273,13 @@ __global__ __launch_bounds__(kThreadsG) void gemm_mxfp_kernel(MxGemmParams p) {
       acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], CBSZ, BLGP, 2, sa[i], 2, sb[j]);
   };
 
-  // ---- epilogue of one output tile: accumulators -> bands of 8 rows x 64 columns through the wavefront's own
+  // ---- epilogue of one output tile: accumulators -> bands of 8 rows x 32 columns through the wavefront's own
   // staging rows -> 16 bytes of consecutive columns per lane (bias added, converted) -> global.
   // In the accumulator layout lanes 0-31 hold rows q*8+0..3 and lanes 32-63 rows q*8+4..7 of each 32-row MFMA
   // tile (one column per lane); each half-wave writes its 4 rows and reads the same 4 rows back, so no lane
   // depends on LDS writes of the other half-wave or of another wavefront: no barrier and no wait for write
-  // completion is needed (the LDS executes one half-wave's accesses in order).
+  // completion is needed (the LDS executes one half-wave's accesses in order).  Two staging buffers alternate:
+  // the writes of band b+1 are issued while the read of band b is still in flight.
   const bool vec_ok = ((p.N & 3) == 0) && ((((uintptr_t)p.C) & 15u) == 0);
   auto epilogue = [&](int ord) __attribute__((always_inline)) {
     int m0, n0;
@@ -285,70 +288,69 @@ __global__ __launch_bounds__(kThreadsG) void gemm_mxfp_kernel(MxGemmParams p) {
     asm volatile("" : "+v"(lane));  // keeps the lane-derived terms below out of the K loop's live registers
     const int frag_row = lane & 31, kgrp = lane >> 5;
     float* stg = (float*)(lds + S * kStage + wave * G::kStgWave) + kgrp * (4 * G::kStgStride);
-    const int c4 = (lane & 15) * 4;          // columns within the 64-column band
-    const int rl0 = (lane & 31) >> 4;        // this lane reads rows rl0 and rl0 + 2 of its half-wave's 4
-    float bv[2][4] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+    const int c4 = (lane & 7) * 4;           // columns within the 32-column band
+    const int rl = (lane & 31) >> 3;         // the row of its half-wave's 4 that this lane reads back
+    float bv[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bv[j][e] = 0.0f;
     if (p.bias != nullptr) {
 #pragma unroll
-      for (int jh = 0; jh < 2; ++jh)
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const int col = n0 + wn * 128 + jh * 64 + c4 + e;
-          if (col < p.N) bv[jh][e] = load_bias_v(p.bias, p.bias_dtype, col);
+          const int col = n0 + wn * 128 + j * 32 + c4 + e;
+          if (col < p.N) bv[j][e] = load_bias_v(p.bias, p.bias_dtype, col);
         }
       // The bias loads are the only vector-memory loads the compiler itself tracks in this kernel.  Completing
       // them here, with a wait it can see, keeps it from guarding their registers with s_waitcnt vmcnt(0)
       // inside the K loop, where that would also wait for every async copy in flight.
       wait_vmcnt_n<0>();
     }
+    auto write_band = [&](int band) __attribute__((always_inline)) {  // band = (i*4 + q)*4 + j
+      const int i = band >> 4, q = (band >> 2) & 3, j = band & 3;
+      float* b = stg + (band & 1) * G::kStgBuf;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+      for (int rr = 0; rr < 4; ++rr) b[rr * G::kStgStride + frag_row] = acc[i][j][q * 4 + rr];
+    };
+    write_band(0);
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
+    for (int band = 0; band < 64; ++band) {
+      const int i = band >> 4, q = (band >> 2) & 3, j = band & 3;
+      asm volatile("" ::: "memory");  // lanes exchange data through LDS: no value may be carried across
+      const float4 v4 = *(const float4*)(stg + (band & 1) * G::kStgBuf + rl * G::kStgStride + c4);
+      if (band + 1 < 64) write_band(band + 1);
+      const float v[4] = {v4.x + bv[j][0], v4.y + bv[j][1], v4.z + bv[j][2], v4.w + bv[j][3]};
+      const int row = m0 + wm * 128 + i * 32 + q * 8 + kgrp * 4 + rl;
+      const int col0 = n0 + wn * 128 + j * 32 + c4;
+      if (row < p.M) {
+        const size_t o = (size_t)row * p.N + col0;
+        if (vec_ok && col0 + 3 < p.N) {
+          if constexpr (OUT_DT == MASE_DT_F32) {
+            *(float4*)((float*)p.C + o) = make_float4(v[0], v[1], v[2], v[3]);
+          } else if constexpr (OUT_DT == MASE_DT_BF16) {
+            uint2 w;
+            w.x = f32x2_to_bf16x2_bits(v[0], v[1]);
+            w.y = f32x2_to_bf16x2_bits(v[2], v[3]);
+            *(uint2*)((uint16_t*)p.C + o) = w;
+          } else {
+            uint2 w;
+            w.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
+            w.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
+            *(uint2*)((uint16_t*)p.C + o) = w;
+          }
+        } else {
 #pragma unroll
-        for (int jh = 0; jh < 2; ++jh) {
-#pragma unroll
-          for (int jj = 0; jj < 2; ++jj)
-#pragma unroll
-            for (int rr = 0; rr < 4; ++rr)
-              stg[rr * G::kStgStride + jj * 32 + frag_row] = acc[i][jh * 2 + jj][q * 4 + rr];
-          asm volatile("" ::: "memory");  // lanes exchange data through LDS: no value may be carried across
-          __builtin_amdgcn_sched_barrier(0);  // bands stay in program order: bounded register use
-          const int col0 = n0 + wn * 128 + jh * 64 + c4;
-#pragma unroll
-          for (int u = 0; u < 2; ++u) {
-            const int rl = rl0 + 2 * u;
-            const float4 v4 = *(const float4*)(stg + rl * G::kStgStride + c4);
-            const float v[4] = {v4.x + bv[jh][0], v4.y + bv[jh][1], v4.z + bv[jh][2], v4.w + bv[jh][3]};
-            const int row = m0 + wm * 128 + i * 32 + q * 8 + kgrp * 4 + rl;
-            if (row >= p.M) continue;
-            const size_t o = (size_t)row * p.N + col0;
-            if (vec_ok && col0 + 3 < p.N) {
-              if constexpr (OUT_DT == MASE_DT_F32) {
-                *(float4*)((float*)p.C + o) = make_float4(v[0], v[1], v[2], v[3]);
-              } else if constexpr (OUT_DT == MASE_DT_BF16) {
-                uint2 w;
-                w.x = f32x2_to_bf16x2_bits(v[0], v[1]);
-                w.y = f32x2_to_bf16x2_bits(v[2], v[3]);
-                *(uint2*)((uint16_t*)p.C + o) = w;
-              } else {
-                uint2 w;
-                w.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
-                w.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
-                *(uint2*)((uint16_t*)p.C + o) = w;
-              }
-            } else {
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                if (col0 + e >= p.N) continue;
-                if constexpr (OUT_DT == MASE_DT_F32) ((float*)p.C)[o + e] = v[e];
-                else if constexpr (OUT_DT == MASE_DT_BF16) ((uint16_t*)p.C)[o + e] = (uint16_t)f32_to_bf16_bits(v[e]);
-                else ((uint16_t*)p.C)[o + e] = (uint16_t)f32_to_f16_bits(v[e]);
-              }
-            }
+          for (int e = 0; e < 4; ++e) {
+            if (col0 + e >= p.N) continue;
+            if constexpr (OUT_DT == MASE_DT_F32) ((float*)p.C)[o + e] = v[e];
+            else if constexpr (OUT_DT == MASE_DT_BF16) ((uint16_t*)p.C)[o + e] = (uint16_t)f32_to_bf16_bits(v[e]);
+            else ((uint16_t*)p.C)[o + e] = (uint16_t)f32_to_f16_bits(v[e]);
           }
         }
       }
+      __builtin_amdgcn_sched_barrier(0);  // bands stay in program order: bounded register use
     }
   };
 
