@@ -115,6 +115,8 @@ struct MinifloatOp {
   float shift;       // 2^mb
   uint32_t close_thr;
   float neg_bias;    // -exponent_bias as T represents it (ieee)
+  int fast_ok;       // every intermediate of a finite element is exact in T (set by the launcher): value-level path
+  int e_lo_i, e_hi_i;
 
   __device__ static __forceinline__ float R(float f) { return TR::round(f); }
 
@@ -146,12 +148,45 @@ struct MinifloatOp {
     return R(ldexpf(1.0f, (int)e));
   }
 
+  // Value-level evaluation of a finite element when the launcher has established that no intermediate needs a
+  // rounding to T (mantissa no wider than T's, 2^e and the smallest grid step representable in T): with k the
+  // rounded logarithm of R(|x| + 1e-9),
+  //   e = clamp(k, e_lo, e_hi);  man = R(|x| / 2^e);  ms = R(man * 2^mb)
+  //   denorm: q = clamp(rint(ms), 0, qmax),                         |y| = q * 2^(e-mb)
+  //   ieee:   e != -bias: q = clamp(rint(ms - 2^mb), 0, qmax),       |y| = (2^mb + q) * 2^(e-mb)
+  //           e == -bias: q = clamp(rint(ms / 2), 0, qmax),          |y| = q * 2^(e-mb+1)
+  //   result = isclose(x, 0) ? (x == 0 ? +0 : x) : copysign(|y|, x)
+  // (for close elements 0*y + x keeps x, except that +0 + -0 is +0; for the others y carries the sign of
+  // x + 1e-9, which is the sign of x, and adding 0*x changes nothing).
+  __device__ __forceinline__ float fast(float x, uint32_t ab, float val, int k) const {
+    const int e = min(max(k, e_lo_i), e_hi_i);
+    const float man = R(ldexpf(val, -e));
+    const float ms = R(ldexpf(man, mb));
+    float yabs;
+    if constexpr (!IEEE) {
+      const float q = fminf(fmaxf(rintf(ms), 0.0f), qmax);
+      yabs = ldexpf(q, e - mb);
+    } else {
+      const bool normal = (float)e != neg_bias;
+      const float a = normal ? R(ms - shift) : R(ms * 0.5f);
+      const float q = fminf(fmaxf(rintf(a), 0.0f), qmax);
+      yabs = normal ? ldexpf(shift + q, e - mb) : ldexpf(q, e - mb + 1);
+    }
+    if (ab <= close_thr) return (ab == 0) ? 0.0f : x;
+    return bits2f(f2bits(yabs) | (f2bits(x) & 0x80000000u));
+  }
+
   __device__ __forceinline__ float operator()(float x, const WaveLog2& t) const {
-    float xs = R(x + 1e-9f);
-    float sgn = (xs > 0.0f) ? 1.0f : ((xs < 0.0f) ? -1.0f : xs);
     float val = fabsf(x);
     float l = R(val + 1e-9f);
-    float e = clamp_cmp(log2_rounded(l, t), e_lo, e_hi);
+    const float lr = log2_rounded(l, t);  // the table lookup inside runs for every lane, before any divergence
+    if (fast_ok) {  // uniform
+      const uint32_t ab = f2bits(val);
+      if (__builtin_expect(ab < 0x7F800000u, 1)) return fast(x, ab, val, (int)lr);
+    }
+    float xs = R(x + 1e-9f);
+    float sgn = (xs > 0.0f) ? 1.0f : ((xs < 0.0f) ? -1.0f : xs);
+    float e = clamp_cmp(lr, e_lo, e_hi);
     float p2 = pow2_T(e);
     float man = R(div_pow2(val, p2));
     float mant;
@@ -225,6 +260,17 @@ struct MinifloatRun {
     op.shift = (float)(1 << op.mb);
     op.close_thr = mase_isclose_zero_threshold_bits(dtype);
     op.neg_bias = -mase_round_scalar_to_dtype((double)bias, dtype);
+    op.e_lo_i = -bias;
+    op.e_hi_i = (1 << ew) - 1 - bias;
+    // exactness conditions of the value-level path: significand of the result fits T, 2^e_hi finite in T, the
+    // smallest grid step 2^(e_lo - mb) exactly representable in T (fp16: down to its smallest subnormal), the
+    // clamp bounds and -bias exact in T
+    const int sig_T = (DT == MASE_DT_F32) ? 24 : (DT == MASE_DT_BF16 ? 8 : 11);
+    const int max_e = DTypeTraits<DT>::kMaxPow2;
+    const int min_step = (DT == MASE_DT_F16) ? -24 : -126;
+    const int sig = op.mb + (IEEE ? 1 : 0);
+    op.fast_ok = sig <= sig_T && op.e_hi_i <= max_e && op.e_lo_i - op.mb >= min_step &&
+                 op.qmax == (float)((1 << op.mb) - 1) && op.neg_bias == (float)(-bias) && bias < 256;
     return launch_elementwise<DT, DT>(in, out, numel, op, st);
   }
   template <int DT> int run() { return ieee ? go<DT, true>() : go<DT, false>(); }
