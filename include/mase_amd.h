@@ -19,6 +19,7 @@
  *   mase_mxfp_qdq           nn/quantizers/mxfp/mxfp.py:187-230    (mxfp_quantizer, non-search branch)
  *   mase_mxfp_pack, mase_gemm_mxfp_scaled   nn/quantized/modules/linear.py:877-895 (LinearMXFP.forward on
  *                           formats the block-scaled matrix instruction supports)
+ *   mase_gemm_bf16_skinny   same call sites as mase_gemm_bf16_tn, for at most 128 rows of activations
  *   mase_gemm_bf16_tn       nn/quantized/modules/linear.py:972 and :895 (the F.linear of LinearMXInt.forward /
  *                           LinearMXFP.forward on the quantize-dequantized operands)
  */
@@ -112,6 +113,15 @@ int mase_mxfp_qdq(const void* in, void* out, uint8_t* codes, uint8_t* scales, si
  * :895) on operands whose MX values are held exactly in bf16. */
 int mase_gemm_bf16_tn(const void* A, const void* B, const void* bias, void* C, size_t M, size_t N, size_t K,
                       int out_dtype, int bias_dtype, void* stream);
+
+/* The same product for few rows of A (M <= 128, the token-by-token shape of serving): bound by streaming B once
+ * from HBM.  The work is split over N and over K ranges; the partial results of the K ranges go through
+ * `workspace` (device memory, 16-byte aligned, at least mase_gemm_bf16_skinny_workspace_bytes(M, N, K) bytes, which
+ * is at most 64*M*N*4) and are added in a fixed order, so results are reproducible.  K % 64 == 0.
+ * Replaces the same F.linear as mase_gemm_bf16_tn (nn/quantized/modules/linear.py:972, :895). */
+size_t mase_gemm_bf16_skinny_workspace_bytes(size_t M, size_t N, size_t K);
+int mase_gemm_bf16_skinny(const void* A, const void* B, const void* bias, void* C, size_t M, size_t N, size_t K,
+                          int out_dtype, int bias_dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* MXFP packing for the block-scaled matrix instruction.  in: numel elements (numel % 32 == 0, blocks of 32
  * consecutive elements); element format (exp_bits, frac_bits) in {(4,3), (5,2), (2,1)}.  codes: one byte per

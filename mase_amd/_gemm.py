@@ -7,6 +7,7 @@ from torch import Tensor
 from . import _lib
 
 GEMM_K_MULTIPLE = 64  # K tile of mase_gemm_bf16_tn
+SKINNY_MAX_ROWS = 128  # at most this many rows of activations take mase_gemm_bf16_skinny
 OPERAND_BYTES_LIMIT = (1 << 32) - 1  # per-call operand size the GEMM entry points accept
 
 
@@ -28,6 +29,17 @@ def gemm_bf16_tn(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dty
     out = torch.empty((M, N), dtype=out_dtype, device=a.device)
     if bias is not None:
         bias = bias.contiguous()
+    if M <= SKINNY_MAX_ROWS:
+        # few rows (token-by-token serving): the weight-streaming kernel, which spreads N and K over the whole chip
+        nbytes = lib.mase_gemm_bf16_skinny_workspace_bytes(M, N, K)
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=a.device)
+        rc = lib.mase_gemm_bf16_skinny(
+            a.data_ptr(), b.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(), M, N, K,
+            _lib.DTYPE_CODE[out_dtype], _lib.DTYPE_CODE[bias.dtype] if bias is not None else 0, ws.data_ptr(), nbytes,
+            _lib.stream_ptr(a),
+        )
+        _lib.check(rc, "mase_gemm_bf16_skinny")
+        return out
     # the kernel addresses an operand with 32-bit byte offsets: activations beyond 4 GiB go in row chunks
     rows_per_call = max(1, min(M, (OPERAND_BYTES_LIMIT // (2 * K)) // 256 * 256 or 1))
     for r0 in range(0, M, rows_per_call):

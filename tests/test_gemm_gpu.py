@@ -95,3 +95,28 @@ def test_gemm_wrappers_split_oversized_activations(dev, monkeypatch):
     whole = _gemm.gemm_mxfp_scaled(ac, asc, (4, 3), bc, bsc, (4, 3), None, torch.float32)
     monkeypatch.setattr(_gemm, "OPERAND_BYTES_LIMIT", 128 * 300)
     assert torch.equal(_gemm.gemm_mxfp_scaled(ac, asc, (4, 3), bc, bsc, (4, 3), None, torch.float32), whole)
+
+
+@pytest.mark.parametrize("M", [1, 7, 32, 33, 64, 100, 128])
+@pytest.mark.parametrize("N,K", [(33, 64), (256, 4096), (4100, 1024), (11008, 4096), (4096, 11008)])
+def test_gemm_few_rows_takes_the_weight_streaming_kernel(dev, M, N, K):
+    """M <= 128: the kernel that splits N and K over the chip and adds the K ranges in a fixed order.  Exact on
+    small-integer operands, within fp32 summation error on random ones, and reproducible run to run."""
+    from mase_amd import _gemm
+
+    assert M <= _gemm.SKINNY_MAX_ROWS
+    g = torch.Generator().manual_seed(M * 13 + N + K)
+    a = torch.randint(-8, 9, (M, K), generator=g).float()
+    b = torch.randint(-8, 9, (N, K), generator=g).float()
+    bias = torch.randint(-8, 9, (N,), generator=g).float()
+    ad, bd = a.bfloat16().to(dev), b.bfloat16().to(dev)
+    ref = a.double() @ b.double().t()
+    assert torch.equal(_gemm.gemm_bf16_tn(ad, bd, None, torch.float32).cpu().double(), ref)
+    assert torch.equal(_gemm.gemm_bf16_tn(ad, bd, bias.to(dev), torch.float32).cpu().double(), ref + bias.double())
+    assert torch.equal(_gemm.gemm_bf16_tn(ad, bd, bias.bfloat16().to(dev), torch.bfloat16).cpu(), (ref + bias.double()).float().bfloat16())
+    ar = torch.randn(M, K, generator=g).bfloat16()
+    br = (torch.randn(N, K, generator=g) * 0.05).bfloat16()
+    y1 = _gemm.gemm_bf16_tn(ar.to(dev), br.to(dev), None, torch.float32)
+    y2 = _gemm.gemm_bf16_tn(ar.to(dev), br.to(dev), None, torch.float32)
+    assert torch.equal(y1, y2)
+    assert rel_err(y1.cpu(), ar.double() @ br.double().t()) < 2e-6
