@@ -13,12 +13,27 @@ namespace {
 // ---------------------------------------------------------------------------------------------
 // generic driver: 8 elements per lane through 16-byte accesses, one element per lane for the tail
 // ---------------------------------------------------------------------------------------------
-template <int DT>
-__device__ __forceinline__ void load8(const void* p, size_t i8, float* x) {
+// fp32 items are two 16-byte vectors.  Inside a complete group of 64 items (one wavefront) lane l takes vectors l
+// and l + 64 of the group's 128, so that each access of the wavefront covers 1 KB of consecutive memory; the items
+// of the incomplete last group take adjacent vectors.
+// SPLIT is set when input and output are both fp32 (the two sides must agree on which elements an item holds).
+template <bool SPLIT>
+__device__ __forceinline__ size_t vec4_first(size_t i8, size_t n8) {
+  if constexpr (!SPLIT) return 2 * i8;
+  return ((i8 | 63) < n8) ? ((i8 & ~(size_t)63) * 2 + (i8 & 63)) : 2 * i8;
+}
+template <bool SPLIT>
+__device__ __forceinline__ size_t vec4_step(size_t i8, size_t n8) {
+  if constexpr (!SPLIT) return 1;
+  return ((i8 | 63) < n8) ? 64 : 1;
+}
+
+template <int DT, bool SPLIT>
+__device__ __forceinline__ void load8(const void* p, size_t i8, size_t n8, float* x) {
   using TR = DTypeTraits<DT>;
   if constexpr (TR::kVec == 4) {
-    const uint4* q = (const uint4*)p + 2 * i8;
-    uint4 a = load_nt(q), b = load_nt(q + 1);
+    const uint4* q = (const uint4*)p + vec4_first<SPLIT>(i8, n8);
+    uint4 a = load_nt(q), b = load_nt(q + vec4_step<SPLIT>(i8, n8));
     TR::unpack(a, x);
     TR::unpack(b, x + 4);
   } else {
@@ -26,13 +41,13 @@ __device__ __forceinline__ void load8(const void* p, size_t i8, float* x) {
     TR::unpack(a, x);
   }
 }
-template <int DT>
-__device__ __forceinline__ void store8(void* p, size_t i8, const float* y) {
+template <int DT, bool SPLIT>
+__device__ __forceinline__ void store8(void* p, size_t i8, size_t n8, const float* y) {
   using TR = DTypeTraits<DT>;
   if constexpr (TR::kVec == 4) {
-    uint4* q = (uint4*)p + 2 * i8;
+    uint4* q = (uint4*)p + vec4_first<SPLIT>(i8, n8);
     store_nt(q, TR::pack(y));
-    store_nt(q + 1, TR::pack(y + 4));
+    store_nt(q + vec4_step<SPLIT>(i8, n8), TR::pack(y + 4));
   } else {
     store_nt((uint4*)p + i8, TR::pack(y));
   }
@@ -47,6 +62,7 @@ constexpr int kEwThreads = 64;
 template <int DTI, int DTO, typename F>
 __global__ __launch_bounds__(kEwThreads) void elementwise_kernel(const void* __restrict__ in, void* __restrict__ out,
                                                                  size_t n8, size_t numel, F f) {
+  constexpr bool kSplit = DTypeTraits<DTI>::kVec == 4 && DTypeTraits<DTO>::kVec == 4;
   WaveLog2 meta;
   if constexpr (F::kUsesTable) meta.init(f.tab, F::kTableHalf);
   const size_t t = (size_t)blockIdx.x * kEwThreads + threadIdx.x;
@@ -56,11 +72,15 @@ __global__ __launch_bounds__(kEwThreads) void elementwise_kernel(const void* __r
   float x[8], y[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) x[j] = 1.0f;
-  if (vec) load8<DTI>(in, t, x);
+  if (vec) load8<DTI, kSplit>(in, t, n8, x);
   else if (one) x[0] = DTypeTraits<DTI>::load1(in, tail);
+  if constexpr (F::kBatch) {
+    f.batch8(x, y);
+  } else {
 #pragma unroll
-  for (int j = 0; j < 8; ++j) y[j] = f(x[j], meta);
-  if (vec) store8<DTO>(out, t, y);
+    for (int j = 0; j < 8; ++j) y[j] = f(x[j], meta);
+  }
+  if (vec) store8<DTO, kSplit>(out, t, n8, y);
   else if (one) DTypeTraits<DTO>::store1(out, tail, y[0]);
 }
 
@@ -88,6 +108,7 @@ template <int DT>
 struct IntegerOp {
   static constexpr bool kUsesTable = false;
   static constexpr int kTableHalf = 0;
+  static constexpr bool kBatch = false;
   const uint32_t* tab;
   int frac;
   int use_floor;
@@ -108,6 +129,7 @@ struct MinifloatOp {
   using TR = DTypeTraits<DT>;
   static constexpr bool kUsesTable = true;
   static constexpr int kTableHalf = IEEE ? kLog2TabHalf : 0;  // floor thresholds (ieee) or ceil thresholds (denorm)
+  static constexpr bool kBatch = false;
   const uint32_t* tab;
   int mb;
   float e_lo, e_hi;  // exponent clamp (as floats; representable in every T for exponent_width <= 8)
@@ -121,12 +143,15 @@ struct MinifloatOp {
   __device__ static __forceinline__ float R(float f) { return TR::round(f); }
 
   // library log2 of a T value followed by ceil (denorm) or floor (ieee), as a float
+  template <bool WAVE = true>
   __device__ __forceinline__ float log2_rounded(float l, const WaveLog2& w) const {
     const uint32_t b = f2bits(l);
     // the lookup runs for every lane (wave-wide register permute), on a stand-in for zero / non-finite values
     const bool special = (b == 0) || (b >= 0x7F800000u);
     const uint32_t bb = special ? 0x3F800000u : b;
-    const float k = (float)(IEEE ? floor_log2_lib(bb, tab, w) : ceil_log2_lib(bb, tab, w));
+    float k;
+    if constexpr (WAVE) k = (float)(IEEE ? floor_log2_lib(bb, tab, w) : ceil_log2_lib(bb, tab, w));
+    else k = (float)(IEEE ? floor_log2_lib(bb, tab) : ceil_log2_lib(bb, tab));  // table from memory: any lane subset
     if (b == 0) return -__builtin_inff();
     if (b >= 0x7F800000u) return (b == 0x7F800000u) ? __builtin_inff() : qnan();  // l >= 0 here or NaN
     return k;
@@ -184,6 +209,18 @@ struct MinifloatOp {
       const uint32_t ab = f2bits(val);
       if (__builtin_expect(ab < 0x7F800000u, 1)) return fast(x, ab, val, (int)lr);
     }
+    return stepwise(x, val, lr);
+  }
+
+  // the same element evaluated with the table read from memory: callable from a divergent branch
+  __device__ __forceinline__ float stepwise_from_memory(float x) const {
+    const float val = fabsf(x);
+    const WaveLog2 unused{};
+    return stepwise(x, val, log2_rounded<false>(R(val + 1e-9f), unused));
+  }
+
+  // operation-by-operation evaluation; lr = rounded library logarithm of R(|x| + 1e-9)
+  __device__ __forceinline__ float stepwise(float x, float val, float lr) const {
     float xs = R(x + 1e-9f);
     float sgn = (xs > 0.0f) ? 1.0f : ((xs < 0.0f) ? -1.0f : xs);
     float e = clamp_cmp(lr, e_lo, e_hi);
@@ -211,15 +248,169 @@ struct MinifloatOp {
 };
 
 // ---------------------------------------------------------------------------------------------
+// minifloat denorm / ieee, value-level kernel.  Preconditions (checked by the launcher): fast_ok of the op (no
+// intermediate needs rounding to T) and the exponent clamp range inside [-32, 31].  Then, with k the rounded library
+// logarithm and e = clamp(k, e_lo, e_hi),
+//   denorm: |y| = min(rint(|x| * 2^(mb-e)), qmax) * 2^(e-mb)
+//   ieee:   e != e_lo: |y| = (2^mb + clamp(rint(|x| * 2^(mb-e) - 2^mb), 0, qmax)) * 2^(e-mb)
+//           e == e_lo: |y| = min(rint(|x| * 2^(mb-e-1)), qmax) * 2^(e-mb+1)
+// (two exact scalings by powers of two collapse into one; where the stepwise form would round a subnormal
+// intermediate the product is far below 1/2 and rounds to 0 either way).  rint on the grid is done in place by
+// adding and subtracting 1.5 * 2^(23+e-mb), and the clamps are applied to |y| itself.  k comes from one add and one shift: lane L
+// keeps, for the biased exponent E = L (mod 64) in [95, 158], delta = 2^23 - 1 - thr (ceil flavour: k = E-127 + (M >
+// thr)) or 2^23 - thr (floor flavour: M >= thr), so that (bits + delta) >> 23 = E + carry.  Exponents outside the
+// window read some other lane's delta and come out as E or E + 1, which the clamp maps to the same bound as the true
+// k.  EPS selects how log2's argument R(|x| + 1e-9) is formed: 0 = it equals |x| for every element whose k can land
+// inside the clamp range (fp16 always; bf16 when e_lo >= -20), 1 = fp32 add, 2 = add and round to bf16.
+// Non-finite elements take the stepwise evaluation with the table read from memory.
+// ---------------------------------------------------------------------------------------------
+template <int DT, bool IEEE, int EPS>
+__global__ __launch_bounds__(kEwThreads) void minifloat_value_kernel(const void* __restrict__ in, void* __restrict__ out,
+                                                                     size_t n8, MinifloatOp<DT, IEEE> op) {
+  using TR = DTypeTraits<DT>;
+  const int lane = (int)(threadIdx.x & 63);
+  // this lane's biased exponent in [95, 158] and its delta
+  const int E_l = 95 + ((lane - 95) & 63);
+  const uint32_t thr = op.tab[(IEEE ? kLog2TabHalf : 0) + 149 + (E_l - 127)];
+  const uint32_t delta = IEEE ? (0x800000u - thr) : (0x7FFFFFu - thr);
+  const size_t t = (size_t)blockIdx.x * kEwThreads + threadIdx.x;
+  const bool live = t < n8;
+  const size_t item = live ? t : n8 - 1;  // every lane takes part in the register permutes
+  float x[8], y[8];
+  load8<DT, true>(in, item, n8, x);
+  // clamp bounds of the exponent in place, and the constants that turn (e + 127) << 23 into the rounding constant
+  // and into the upper bound of |y| (mb >= 1 for the denorm flavour, checked by the launcher)
+  const uint32_t lo_f = (uint32_t)(op.e_lo_i + 127) << 23, hi_f = ((uint32_t)(op.e_hi_i + 127) << 23) | 0x7FFFFFu;
+  const uint32_t k_magic = ((uint32_t)(23 - op.mb) << 23) + 0x400000u;
+  const uint32_t k_cap = IEEE ? (0x800000u - (0x800000u >> op.mb))                    // (2 - 2^-mb) * 2^e
+                              : (0x800000u - (0x1000000u >> op.mb)) - 0x800000u;      // (2 - 2^(1-mb)) * 2^(e-1)
+  [[maybe_unused]] const float c_sub = bits2f(lo_f + k_magic + 0x800000u);
+  [[maybe_unused]] const float cap_sub = op.mb == 0 ? 0.0f : bits2f(lo_f + (0x800000u - (0x1000000u >> op.mb)));
+  uint32_t worst = 0;
+  uint32_t lbs[8], ds[8];
+  // all eight permutes are issued before the first result is needed
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const uint32_t ab = f2bits(x[j]) & 0x7FFFFFFFu;
+    uint32_t lb = ab;
+    if constexpr (EPS == 1) lb = f2bits(bits2f(ab) + 1e-9f);
+    if constexpr (EPS == 2) lb = f2bits(TR::round(bits2f(ab) + 1e-9f));
+    lbs[j] = lb;
+    ds[j] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((lb >> 21) & 0xFCu), (int)delta);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const uint32_t xb = f2bits(x[j]);
+    const uint32_t ab = xb & 0x7FFFFFFFu;
+    const float val = bits2f(ab);
+    worst = max(worst, ab);
+    const uint32_t lb = lbs[j], d = ds[j];
+    // e clamped, kept in place as the exponent field: ebs = (e + 127) << 23
+    uint32_t c;
+    asm("v_med3_u32 %0, %1, %2, %3" : "=v"(c) : "v"(lb + d), "s"(lo_f), "v"(hi_f));  // one scalar operand at most
+    const uint32_t ebs = c & 0x7F800000u;
+    // rounding to the grid 2^(e-mb) by adding and subtracting 1.5 * 2^(23+e-mb) (exact while |x| < 2^(22+e-mb);
+    // beyond that the result only has to stay at or above the upper clamp bound, which it does)
+    float yabs;
+    if constexpr (!IEEE) {
+      const float C = bits2f(ebs + k_magic);
+      const float r = (val + C) - C;
+      yabs = fminf(r, bits2f(ebs + k_cap));  // qmax * 2^(e-mb)
+    } else {
+      // e == e_lo: grid 2^(e-mb+1), range [0, qmax * 2^(e-mb+1)];  otherwise [2^e, (2^(mb+1) - 1) * 2^(e-mb)]
+      const bool sub = c < lo_f + 0x800000u;
+      const float C = sub ? c_sub : bits2f(ebs + k_magic);
+      const float lo = sub ? 0.0f : bits2f(ebs);
+      const float hi = sub ? cap_sub : bits2f(ebs + k_cap);
+      const float r = (val + C) - C;
+      yabs = __builtin_amdgcn_fmed3f(r, lo, hi);
+    }
+    const uint32_t yb = (f2bits(yabs) & 0x7FFFFFFFu) | (xb & 0x80000000u);
+    // isclose(x, 0): the element passes through, and both zeros become +0 (x + 0.0).  A bitwise select: a
+    // conditional here would be compiled into a branch around the arithmetic, with a wait for each permute
+    const uint32_t xz = f2bits(x[j] + 0.0f);
+    const uint32_t keep = (uint32_t)-(int32_t)(ab <= op.close_thr);
+    y[j] = bits2f((xz & keep) | (yb & ~keep));
+  }
+  if (__builtin_expect(worst >= 0x7F800000u, 0)) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if ((f2bits(x[j]) & 0x7FFFFFFFu) >= 0x7F800000u) y[j] = op.stepwise_from_memory(x[j]);
+  }
+  if (live) store8<DT, true>(out, item, n8, y);
+}
+
+// ---------------------------------------------------------------------------------------------
 // bit-level minifloat cast: _minifloat_mx/fake.py:11-149 (encode to a code, decode it back)
 // ---------------------------------------------------------------------------------------------
 struct MinifloatMxOp {
   static constexpr bool kUsesTable = false;
   static constexpr int kTableHalf = 0;
+  static constexpr bool kBatch = true;
   const uint32_t* tab;
   MinifloatMxFmt m;
   __device__ __forceinline__ float operator()(float x, const WaveLog2&) const {
     return minifloat_mx_decode(minifloat_mx_encode(x, m), m);
+  }
+
+  // Integer form of decode(encode(x)) on the fp32 bit fields, for elements whose code is an ordinary one:
+  //   ye = exponent field + bias - 127; fraction 23 -> 15 bits by truncation, 15 -> F bits in the format's rounding
+  //   mode; a carry out of the fraction is OR-ed into the exponent field; ye > e_hi saturates; ye == 0 takes the
+  //   shifted fraction, ye < 0 gives zero; the value is the code's [exponent|fraction] field moved to fp32's place
+  //   (codes with exponent field 0: the integer fraction times 2^(1-bias-F)).
+  // Returns false for what is left to the stepwise functions: fp32 subnormals and non-finite inputs, codes of the
+  // inf/nan exponent of a format that has them and, with INLINE_SUB = false (formats whose subnormal range is
+  // rarely reached), every code with exponent field 0.
+  template <bool INLINE_SUB>
+  __device__ __forceinline__ bool fast(float x, uint32_t addc, uint32_t tie, int ye_limit, float& y) const {
+    const int F = m.F;
+    const uint32_t xb = f2bits(x + 0.0f);  // -0.0 is "not negative" in the encode
+    const uint32_t ab = xb & 0x7FFFFFFFu;
+    const uint32_t Ef = ab >> 23;
+    const int ye = (int)Ef + (m.bias - 127);
+    const int shn = 15 - F;
+    const uint32_t m15 = (ab >> 8) & 0x7FFFu;
+    const uint32_t yf = (m15 + addc + ((m15 >> shn) & tie)) >> shn;  // 0 .. 2^F
+    const uint32_t cn = ((uint32_t)ye << F) | yf;
+    const uint32_t cmax = ((uint32_t)m.e_hi << F) | (uint32_t)m.frac_hi;
+    const uint32_t rebias = (uint32_t)(127 - m.bias) << 23;
+    const bool ordinary = (Ef - 1u < 254u) || ab == 0;
+    if constexpr (!INLINE_SUB) {
+      const uint32_t c = ye > m.e_hi ? cmax : cn;
+      const uint32_t yn = (c << (23 - F)) + rebias;
+      y = bits2f(ab == 0 ? 0u : ((xb & 0x80000000u) | yn));
+      return ordinary && (ye > 0 || ab == 0) && ye < ye_limit;
+    }
+    const uint32_t cs = yf ? ((yf | (1u << F)) >> 1) : 0u;
+    uint32_t c = ye > 0 ? cn : (ye == 0 ? cs : 0u);
+    c = ye > m.e_hi ? cmax : c;
+    c = ab == 0 ? 0u : c;
+    const uint32_t yn = (c << (23 - F)) + rebias;
+    const uint32_t ys = f2bits(ldexpf((float)c, 1 - m.bias - F));
+    y = bits2f((xb & 0x80000000u) | ((c >> F) != 0 ? yn : ys));
+    return ordinary && ye < ye_limit;
+  }
+
+  __device__ __forceinline__ void batch8(const float* x, float* y) const {
+    const int shn = 15 - m.F;
+    // rounding of the 15-bit fraction as one addition: nearest-even, up (any remainder), down / toward zero
+    const uint32_t addc = m.round_mode == 0 ? (1u << (shn - 1)) - 1u : (m.round_mode == 1 ? (1u << shn) - 1u : 0u);
+    const uint32_t tie = m.round_mode == 0 ? 1u : 0u;
+    // formats with inf/nan codes: an element that reaches the top ordinary exponent may carry into the inf/nan one
+    const int ye_limit = m.is_finite ? 0x7FFFFFFF : m.e_hi;
+    bool ok = true;
+    if (m.bias < 12) {  // uniform
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ok &= fast<true>(x[j], addc, tie, ye_limit, y[j]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ok &= fast<false>(x[j], addc, tie, ye_limit, y[j]);
+    }
+    if (__builtin_expect(!ok, 0)) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) y[j] = minifloat_mx_decode(minifloat_mx_encode(x[j], m), m);
+    }
   }
 };
 
@@ -271,7 +462,22 @@ struct MinifloatRun {
     const int sig = op.mb + (IEEE ? 1 : 0);
     op.fast_ok = sig <= sig_T && op.e_hi_i <= max_e && op.e_lo_i - op.mb >= min_step &&
                  op.qmax == (float)((1 << op.mb) - 1) && op.neg_bias == (float)(-bias) && bias < 256;
-    return launch_elementwise<DT, DT>(in, out, numel, op, st);
+    // value-level kernel on the 16-byte-aligned vector part, the general kernel on what is left
+    const bool window = op.e_lo_i >= -32 && op.e_hi_i <= 31 && op.mb <= 16 && (IEEE || op.mb >= 1);
+    size_t done = 0;
+    if (op.fast_ok && window && aligned16(in) && aligned16(out) && numel >= 8) {
+      const size_t n8 = numel / 8;
+      const int eps = (DT == MASE_DT_F16) ? 0 : (DT == MASE_DT_F32 ? 1 : (op.e_lo_i >= -20 ? 0 : 2));
+      const dim3 grid(blocks_for(n8, kEwThreads)), block(kEwThreads);
+      if (eps == 0) hipLaunchKernelGGL((minifloat_value_kernel<DT, IEEE, 0>), grid, block, 0, st, in, out, n8, op);
+      else if (eps == 1) hipLaunchKernelGGL((minifloat_value_kernel<DT, IEEE, 1>), grid, block, 0, st, in, out, n8, op);
+      else hipLaunchKernelGGL((minifloat_value_kernel<DT, IEEE, 2>), grid, block, 0, st, in, out, n8, op);
+      if (hipGetLastError() != hipSuccess) return MASE_ERR_LAUNCH;
+      done = n8 * 8;
+      if (done == numel) return MASE_OK;
+    }
+    const size_t eb = DTypeTraits<DT>::kBytes;
+    return launch_elementwise<DT, DT>((const char*)in + done * eb, (char*)out + done * eb, numel - done, op, st);
   }
   template <int DT> int run() { return ieee ? go<DT, true>() : go<DT, false>(); }
 };

@@ -215,7 +215,7 @@ def test_integer(Q, dev, width, frac, signed):
 
 # ------------------------------------------------------------------ element-wise minifloat
 @pytest.mark.parametrize("cfg", [(8, 4, None), (8, 5, None), (6, 3, None), (8, 4, 11), (12, 5, None), (16, 8, None),
-                                 (8, 2, None), (4, 2, 0)])
+                                 (8, 2, None), (4, 2, 0), (8, 5, 25), (8, 6, None), (6, 5, 31)])
 @pytest.mark.parametrize("dtype", DTYPES, ids=_ID.get)
 def test_minifloat_denorm_ieee(Q, dev, dtype, cfg):
     w, ew, eb = cfg
