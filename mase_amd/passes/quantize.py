@@ -7,7 +7,12 @@ Like the reference it pops ``"by"`` (and ``"gptq"``) from ``pass_args`` and ``"n
 (:28, :48, :140), instantiates ``quantized_module_map["linear_<name>"]`` with the original module's shape, bias,
 device and dtype (``module_modify_helper.py:149-176``), hands the weights over with
 ``load_state_dict(deepcopy(state_dict), strict=False)`` (:103-114) and swaps the module in by name (:137-141).
-Model-family wrappers (attention, MLP, embeddings) and the GPTQ pre-pass are outside this build.
+``nn.Embedding`` targets (:191-216) and Llama attention / MLP / RMSNorm targets (:264-275, selected by name or
+regex with a ``llama_self_attention_* / llama_mlp_* / llama_rms_norm_*`` entry of the registry) are handled the same
+way; the Llama replacements receive ``config=network.config`` like the reference's (quantize.py:52-56, 82-86).  A
+module counts as a Llama attention / MLP / RMSNorm when a class of that name is among its bases, so that the
+``transformers`` classes match without being imported here.  Other model families, conv2d and the GPTQ pre-pass are
+outside this build.
 """
 from __future__ import annotations
 
@@ -31,11 +36,53 @@ def _instantiate_linear(module, postfix, module_map, additional_module_args):
     return linear_cls(**kwargs, **additional_module_args)
 
 
+def _instantiate_embedding(module, postfix, module_map, additional_module_args):
+    embedding_cls = module_map[f"embedding_{postfix}"]
+    kwargs = dict(num_embeddings=module.num_embeddings, embedding_dim=module.embedding_dim,
+                  padding_idx=module.padding_idx, max_norm=module.max_norm, norm_type=module.norm_type,
+                  scale_grad_by_freq=module.scale_grad_by_freq, sparse=module.sparse)
+    if "config" in inspect.signature(embedding_cls.__init__).parameters:
+        return embedding_cls(**kwargs, config=additional_module_args)
+    return embedding_cls(**kwargs, **additional_module_args)
+
+
+_LLAMA_PREFIX = {"LlamaAttention": "llama_self_attention", "LlamaMLP": "llama_mlp", "LlamaRMSNorm": "llama_rms_norm"}
+
+
+def _llama_prefix(module):
+    for cls in type(module).__mro__:
+        if cls.__name__ in _LLAMA_PREFIX:
+            return _LLAMA_PREFIX[cls.__name__]
+    return None
+
+
+def _instantiate_llama_module(module, postfix, prefix, module_map, module_args, network_args):
+    llama_cls = module_map[f"{prefix}_{postfix}"]
+    new = llama_cls(config=network_args, layer_idx=getattr(module, "layer_idx", None), q_config=module_args)
+    first = next(module.parameters(), None)
+    return new if first is None else new.to(device=first.device, dtype=first.dtype)
+
+
 def _instantiate_module(module, postfix, module_map, additional_module_args):
     module_args = additional_module_args["config"]
+    network_args = additional_module_args.get("network_config", None)
     if isinstance(module, torch.nn.Linear):
         return _instantiate_linear(module, postfix, module_map, module_args)
+    if isinstance(module, torch.nn.Embedding):
+        return _instantiate_embedding(module, postfix, module_map, module_args)
+    prefix = _llama_prefix(module)
+    if prefix is not None:
+        return _instantiate_llama_module(module, postfix, prefix, module_map, module_args, network_args)
     raise ValueError(f"{module} is not supported.")
+
+
+def _module_args(network, quan_config):
+    """``network_config`` travels with the module config when the network carries a model config (the reference
+    tests for a ``transformers`` model; any network with a ``config`` attribute is treated the same here)"""
+    network_config = getattr(network, "config", None)
+    if network_config is not None:
+        return {"config": quan_config, "network_config": network_config}
+    return {"config": quan_config}
 
 
 def _weight_replacement(x, y):
@@ -81,7 +128,7 @@ def _quantize_by_name(network, pass_args):
         if n in pass_args:
             quan_config = pass_args[n]["config"]
             postfix = quan_config.pop("name")
-            new_m = _instantiate_module(m, postfix, quantized_module_map, {"config": quan_config})
+            new_m = _instantiate_module(m, postfix, quantized_module_map, _module_args(network, quan_config))
             network = _replace_by_name(network, n, new_m)
     return network
 
@@ -102,7 +149,7 @@ def _quantize_by_regex_name(network, pass_args):
             continue
         quan_config = pass_args[matched]["config"]
         postfix = quan_config["name"]
-        new_m = _instantiate_module(m, postfix, quantized_module_map, {"config": quan_config})
+        new_m = _instantiate_module(m, postfix, quantized_module_map, _module_args(network, quan_config))
         network = _replace_by_name(network, n, new_m)
     return network
 

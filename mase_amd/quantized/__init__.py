@@ -9,5 +9,10 @@ from .modules import (  # noqa: F401
     LinearMinifloatIEEE,
     LinearMXFP,
     LinearMXInt,
+    LlamaAttentionMXFP,
+    LlamaAttentionMXInt,
+    LlamaMLPMXFP,
+    LlamaMLPMXInt,
+    LlamaRMSNormMinifloat,
     quantized_module_map,
 )

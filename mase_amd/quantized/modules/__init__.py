@@ -1,6 +1,14 @@
 """``quantized_module_map``: the in-scope entries of the reference's registry
-(``chop/nn/quantized/modules/__init__.py:236-251, 334-335, 388-408``), same keys."""
+(``chop/nn/quantized/modules/__init__.py:236-251, 334-335, 352-360, 388-408``), same keys."""
 from .embedding import EmbeddingMXFP, EmbeddingMXInt
+from .llama import (
+    LlamaAttentionMXFP,
+    LlamaAttentionMXInt,
+    LlamaMLPMXFP,
+    LlamaMLPMXInt,
+    LlamaRMSNormMinifloat,
+    quantized_llama_module_map,
+)
 from .linear import (
     LinearBlockFP,
     LinearInteger,
@@ -20,4 +28,4 @@ quantized_module_map = {
     "linear_mxfp": LinearMXFP,
     "embedding_mxint": EmbeddingMXInt,
     "embedding_mxfp": EmbeddingMXFP,
-}
+} | quantized_llama_module_map

@@ -1,0 +1,240 @@
+"""MX-quantized Llama attention, MLP and RMSNorm with the constructor, attributes, config keys and forward contract
+of the reference's ``chop/nn/quantized/modules/llama/attention.py:130-457`` (``LlamaAttentionMXFP``,
+``LlamaAttentionMXInt``, ``_eager_attention_forward_mxfp/_mxint``), ``llama/mlp.py:49-77`` (``LlamaMLPMXFP``,
+``LlamaMLPMXInt``) and ``llama/rms_norm.py:34-84`` (``LlamaRMSNormMinifloat``).
+
+The reference derives these classes from the ``transformers`` Llama modules; here they are plain ``nn.Module``s with
+the same parameter names (``q_proj/k_proj/v_proj/o_proj``, ``gate_proj/up_proj/down_proj``, ``weight``), so a state
+dict of the original module loads with ``strict=True`` and no ``transformers`` import is needed.  ``config`` is any
+object with the Llama config fields read below (a ``LlamaConfig`` works).  Every quantizer is a HIP kernel; the
+contractions are the library's batched GEMMs, the operations the reference performs at those points.
+
+What is quantized (``q_config`` sub-dicts, each with an optional ``bypass``):
+  ``rope``      cos/sin tables, minifloat cast                       (attention.py:163-177)
+  ``kv_cache``  new key/value states before ``past_key_value.update``  (attention.py:182-187)
+  ``qk_matmul`` the query (not the key) along head_dim                (attention.py:352-361)
+  ``softmax``   the masked scores, minifloat cast, softmax in fp32    (attention.py:369-375)
+  ``av_matmul`` the probabilities (not the values) along the key axis (attention.py:383-392)
+MLP: ``silu_minifloat`` on the gate projection (mlp.py:60-62, 75-77); RMSNorm: minifloat cast of the input and of the
+weight (rms_norm.py:72-84).
+"""
+from __future__ import annotations
+
+from functools import partial
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor, nn
+
+from ...quantizers import mxfp_quantizer, mxint_quantizer
+from ...quantizers._ops import minifloat_mx_qdq
+from ..functional.activations import kv_cache_mxfp, kv_cache_mxint, rope_minifloat, rotate_half, silu_minifloat, softmax_minifloat
+
+
+def repeat_kv(hidden_states: Tensor, n_rep: int) -> Tensor:
+    """(batch, kv_heads, seq, head_dim) -> (batch, kv_heads * n_rep, seq, head_dim), each head repeated in place"""
+    batch, num_key_value_heads, slen, head_dim = hidden_states.shape
+    if n_rep == 1:
+        return hidden_states
+    hidden_states = hidden_states[:, :, None, :, :].expand(batch, num_key_value_heads, n_rep, slen, head_dim)
+    return hidden_states.reshape(batch, num_key_value_heads * n_rep, slen, head_dim)
+
+
+def apply_rotary_pos_emb(q, k, cos, sin, unsqueeze_dim=1):
+    cos = cos.unsqueeze(unsqueeze_dim)
+    sin = sin.unsqueeze(unsqueeze_dim)
+    return (q * cos) + (rotate_half(q) * sin), (k * cos) + (rotate_half(k) * sin)
+
+
+def _mx_quantizer(kind: str, config: dict):
+    if kind == "mxfp":
+        return partial(mxfp_quantizer, block_size=config["data_in_block_size"],
+                       element_exp_bits=config["data_in_exponent_width"],
+                       element_frac_bits=config["data_in_frac_width"], block_dim=-1)
+    return partial(mxint_quantizer, block_size=config["data_in_block_size"], element_bits=config["data_in_width"],
+                   block_dim=-1)
+
+
+def _eager_attention_forward(kind, module, query, key, value, attention_mask, scaling, dropout=0.0, qk_bypass=False,
+                             qk_config=None, av_bypass=False, av_config=None, softmax_bypass=False, softmax_config=None,
+                             **kwargs):
+    key_states = repeat_kv(key, module.num_key_value_groups)
+    value_states = repeat_kv(value, module.num_key_value_groups)
+    if not qk_bypass:
+        query = _mx_quantizer(kind, qk_config)(query)
+    attn_weights = torch.matmul(query, key_states.transpose(2, 3)) * scaling
+    if attention_mask is not None:
+        causal_mask = attention_mask[:, :, :, : key_states.shape[-2]]
+        attn_weights = attn_weights + causal_mask
+    if not softmax_bypass:
+        attn_weights = softmax_minifloat(attn_weights, softmax_config, dim=-1)
+    else:
+        attn_weights = nn.functional.softmax(attn_weights.to(torch.float32), dim=-1).to(attn_weights.dtype)
+    attn_weights = nn.functional.dropout(attn_weights, p=dropout, training=module.training)
+    if not av_bypass:
+        attn_weights = _mx_quantizer(kind, av_config)(attn_weights)
+    attn_output = torch.matmul(attn_weights, value_states)
+    attn_output = attn_output.transpose(1, 2).contiguous()
+    return attn_output, attn_weights
+
+
+_eager_attention_forward_mxfp = partial(_eager_attention_forward, "mxfp")
+_eager_attention_forward_mxint = partial(_eager_attention_forward, "mxint")
+
+
+class _LlamaAttentionMX(nn.Module):
+    _kind = "mxint"
+
+    def __init__(self, config, layer_idx, q_config: dict = None):
+        super().__init__()
+        self.config = config
+        self.layer_idx = layer_idx
+        self.head_dim = getattr(config, "head_dim", None) or config.hidden_size // config.num_attention_heads
+        self.num_key_value_groups = config.num_attention_heads // config.num_key_value_heads
+        self.scaling = self.head_dim ** -0.5
+        self.attention_dropout = getattr(config, "attention_dropout", 0.0)
+        self.is_causal = True
+        bias = getattr(config, "attention_bias", False)
+        self.q_proj = nn.Linear(config.hidden_size, config.num_attention_heads * self.head_dim, bias=bias)
+        self.k_proj = nn.Linear(config.hidden_size, config.num_key_value_heads * self.head_dim, bias=bias)
+        self.v_proj = nn.Linear(config.hidden_size, config.num_key_value_heads * self.head_dim, bias=bias)
+        self.o_proj = nn.Linear(config.num_attention_heads * self.head_dim, config.hidden_size, bias=bias)
+        q_config = q_config or {}
+        self.qk_config = q_config.get("qk_matmul", {})
+        self.av_config = q_config.get("av_matmul", {})
+        self.rope_config = q_config.get("rope", {})
+        self.softmax_config = q_config.get("softmax", {})
+        self.kv_cache_config = q_config.get("kv_cache", {})
+        self.qk_bypass = self.qk_config.get("bypass", False)
+        self.av_bypass = self.av_config.get("bypass", False)
+        self.rope_bypass = self.rope_config.get("bypass", False)
+        self.softmax_bypass = self.softmax_config.get("bypass", False)
+        self.kv_cache_bypass = self.kv_cache_config.get("bypass", False)
+
+    def forward(self, hidden_states: Tensor, position_embeddings: Tuple[Tensor, Tensor],
+                attention_mask: Optional[Tensor], past_key_value=None, cache_position=None, **kwargs):
+        input_shape = hidden_states.shape[:-1]
+        hidden_shape = (*input_shape, -1, self.head_dim)
+        query_states = self.q_proj(hidden_states).view(hidden_shape).transpose(1, 2)
+        key_states = self.k_proj(hidden_states).view(hidden_shape).transpose(1, 2)
+        value_states = self.v_proj(hidden_states).view(hidden_shape).transpose(1, 2)
+
+        cos, sin = position_embeddings
+        if not self.rope_bypass:
+            query_states, key_states = rope_minifloat(query_states, key_states, cos, sin, self.rope_config)
+        else:
+            query_states, key_states = apply_rotary_pos_emb(query_states, key_states, cos, sin)
+
+        if past_key_value is not None:
+            cache_kwargs = {"sin": sin, "cos": cos, "cache_position": cache_position}
+            if not self.kv_cache_bypass:
+                kv_cache = kv_cache_mxfp if self._kind == "mxfp" else kv_cache_mxint
+                key_states, value_states = kv_cache(key_states, value_states, self.kv_cache_config)
+            key_states, value_states = past_key_value.update(key_states, value_states, self.layer_idx, cache_kwargs)
+
+        attn_output, attn_weights = _eager_attention_forward(
+            self._kind, self, query_states, key_states, value_states, attention_mask,
+            dropout=0.0 if not self.training else self.attention_dropout, scaling=self.scaling,
+            qk_bypass=self.qk_bypass, qk_config=self.qk_config, av_bypass=self.av_bypass, av_config=self.av_config,
+            softmax_bypass=self.softmax_bypass, softmax_config=self.softmax_config, **kwargs)
+        attn_output = attn_output.reshape(*input_shape, -1).contiguous()
+        attn_output = self.o_proj(attn_output)
+        return attn_output, attn_weights
+
+    @classmethod
+    def from_attention(cls, attention: nn.Module, q_config: dict = None):
+        new_attn = cls(config=attention.config, layer_idx=attention.layer_idx, q_config=q_config)
+        first = next(attention.parameters())
+        new_attn = new_attn.to(dtype=first.dtype, device=first.device)
+        new_attn.load_state_dict(attention.state_dict(), strict=True)
+        return new_attn
+
+
+class LlamaAttentionMXFP(_LlamaAttentionMX):
+    """MXFP-quantized Llama attention."""
+    _kind = "mxfp"
+
+
+class LlamaAttentionMXInt(_LlamaAttentionMX):
+    """MXInt-quantized Llama attention."""
+    _kind = "mxint"
+
+
+class _LlamaMLPMX(nn.Module):
+    """Llama MLP whose SiLU input goes through the minifloat cast."""
+
+    def __init__(self, config, layer_idx=None, q_config: dict = None):
+        super().__init__()
+        self.config = config
+        self.hidden_size = config.hidden_size
+        self.intermediate_size = config.intermediate_size
+        bias = getattr(config, "mlp_bias", False)
+        self.gate_proj = nn.Linear(self.hidden_size, self.intermediate_size, bias=bias)
+        self.up_proj = nn.Linear(self.hidden_size, self.intermediate_size, bias=bias)
+        self.down_proj = nn.Linear(self.intermediate_size, self.hidden_size, bias=bias)
+        hidden_act = getattr(config, "hidden_act", "silu")
+        if hidden_act != "silu":
+            raise NotImplementedError(f"hidden_act={hidden_act!r}: the quantized form is defined for SiLU only")
+        self.act_fn = nn.SiLU()
+        self.layer_idx = layer_idx
+        self.q_config = q_config or {}
+        self.bypass = self.q_config.get("bypass", False)
+
+    def forward(self, x: Tensor) -> Tensor:
+        if self.bypass:
+            return self.down_proj(self.act_fn(self.gate_proj(x)) * self.up_proj(x))
+        x = silu_minifloat(self.gate_proj(x), self.q_config) * self.up_proj(x)
+        return self.down_proj(x)
+
+
+class LlamaMLPMXFP(_LlamaMLPMX):
+    """MXFP-quantized LlamaMLP. SiLU uses minifloat quantization."""
+
+
+class LlamaMLPMXInt(_LlamaMLPMX):
+    """MXInt-quantized LlamaMLP. SiLU uses minifloat quantization."""
+
+
+class LlamaRMSNormMinifloat(nn.Module):
+    """Minifloat-quantized Llama RMSNorm: weight and input go through the minifloat cast at forward time."""
+
+    def __init__(self, config=None, layer_idx=None, q_config: dict = None):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(config.hidden_size))
+        self.variance_epsilon = config.rms_norm_eps
+        self.layer_idx = layer_idx
+        self.q_config = q_config or {}
+        self.bypass = self.q_config.get("bypass", False)
+        self.weight_bypass = self.q_config.get("weight_bypass", False)
+        self.data_in_bypass = self.q_config.get("data_in_bypass", False)
+
+        def cast(prefix):
+            return partial(minifloat_mx_qdq, exp_bits=self.q_config[f"{prefix}_exponent_width"],
+                           frac_bits=self.q_config[f"{prefix}_frac_width"],
+                           is_finite=self.q_config.get(f"{prefix}_is_finite", True),
+                           round_mode=self.q_config.get(f"{prefix}_round_mode", "rn"), output_dtype=None)
+
+        self.w_quantizer = cast("weight") if not self.bypass and not self.weight_bypass else None
+        self.x_quantizer = cast("data_in") if not self.bypass and not self.data_in_bypass else None
+
+    def forward(self, hidden_states):
+        input_dtype = hidden_states.dtype
+        if self.x_quantizer is not None:
+            hidden_states = self.x_quantizer(hidden_states)
+        hidden_states = hidden_states.to(torch.float32)
+        variance = hidden_states.pow(2).mean(-1, keepdim=True)
+        hidden_states = hidden_states * torch.rsqrt(variance + self.variance_epsilon)
+        weight = self.w_quantizer(self.weight) if self.w_quantizer is not None else self.weight
+        return weight * hidden_states.to(input_dtype)
+
+    def extra_repr(self):
+        return f"{tuple(self.weight.shape)}, eps={self.variance_epsilon}"
+
+
+quantized_llama_module_map = {
+    "llama_self_attention_mxfp": LlamaAttentionMXFP,
+    "llama_self_attention_mxint": LlamaAttentionMXInt,
+    "llama_rms_norm_minifloat": LlamaRMSNormMinifloat,
+    "llama_mlp_mxfp": LlamaMLPMXFP,
+    "llama_mlp_mxint": LlamaMLPMXInt,
+}

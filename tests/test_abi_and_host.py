@@ -199,3 +199,49 @@ def test_packed_mxfp_weight_eligibility_and_decoder_layer_host_side():
     assert y.shape == x.shape and y.dtype == torch.bfloat16
     assert (y[:, :8].float() - y8.float()).abs().max() < 0.1
     assert DecoderLayer(DecoderLayerConfig(), dtype=torch.bfloat16, device="meta").linear_flops(16384) == pytest.approx(6.632e12, rel=1e-3)
+
+
+def test_module_pass_swaps_llama_blocks_on_the_host():
+    """the swap itself needs no device: classes named like the Llama modules are matched through their bases, the
+    replacements get network.config and the original weights"""
+    from types import SimpleNamespace
+
+    from mase_amd.passes import quantize_module_transform_pass
+    from mase_amd.quantized import LlamaMLPMXFP, LlamaRMSNormMinifloat, quantized_module_map
+
+    assert {"llama_self_attention_mxint", "llama_self_attention_mxfp", "llama_mlp_mxint", "llama_mlp_mxfp",
+            "llama_rms_norm_minifloat"} <= set(quantized_module_map)
+
+    class LlamaMLP(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.gate_proj = torch.nn.Linear(64, 96, bias=False)
+            self.up_proj = torch.nn.Linear(64, 96, bias=False)
+            self.down_proj = torch.nn.Linear(96, 64, bias=False)
+
+    class MyMLP(LlamaMLP):  # a subclass still matches
+        pass
+
+    class LlamaRMSNorm(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.weight = torch.nn.Parameter(torch.full((64,), 1.5))
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.config = SimpleNamespace(hidden_size=64, intermediate_size=96, rms_norm_eps=1e-5)
+            self.mlp, self.norm, self.act = MyMLP(), LlamaRMSNorm(), torch.nn.GELU()
+
+    net = Net()
+    up = net.mlp.up_proj.weight.detach().clone()
+    args = {"by": "name",
+            "mlp": {"config": {"name": "mxfp", "data_in_exponent_width": 4, "data_in_frac_width": 3}},
+            "norm": {"config": {"name": "minifloat", "bypass": True}}}
+    net, _ = quantize_module_transform_pass(net, args)
+    assert isinstance(net.mlp, LlamaMLPMXFP) and torch.equal(net.mlp.up_proj.weight, up)
+    assert net.mlp.q_config == {"data_in_exponent_width": 4, "data_in_frac_width": 3}  # "name" popped, as by name does
+    assert isinstance(net.norm, LlamaRMSNormMinifloat) and float(net.norm.weight[0]) == 1.5
+    assert net.norm.variance_epsilon == 1e-5 and net.norm.x_quantizer is None
+    with pytest.raises(ValueError):
+        quantize_module_transform_pass(net, {"by": "name", "act": {"config": {"name": "mxint"}}})
