@@ -17,6 +17,7 @@
  *   mase_minifloat_qdq      nn/quantizers/minifloat.py:90-117, :200-225 (minifloat_denorm/ieee_quantizer)
  *   mase_minifloat_mx_qdq   nn/quantizers/_minifloat_mx/minifloat.py:12-33 (minifloat_quantizer_sim)
  *   mase_mxfp_qdq           nn/quantizers/mxfp/mxfp.py:187-230    (mxfp_quantizer, non-search branch)
+ *   mase_mx_unpack          nn/quantizers/mxint/fake.py:59-80, nn/quantizers/mxfp/fake.py:75-104 (compose_*)
  *   mase_mxfp_pack, mase_gemm_mxfp_scaled   nn/quantized/modules/linear.py:877-895 (LinearMXFP.forward on
  *                           formats the block-scaled matrix instruction supports)
  *   mase_gemm_bf16_skinny   same call sites as mase_gemm_bf16_tn, for at most 128 rows of activations
@@ -105,6 +106,14 @@ int mase_minifloat_mx_qdq(const void* in, void* out, size_t numel, int in_dtype,
 int mase_mxfp_qdq(const void* in, void* out, uint8_t* codes, uint8_t* scales, size_t numel, int in_dtype,
                   int out_dtype, int block_size, int exp_bits, int frac_bits, const uint32_t* log2_tab,
                   void* stream);
+
+/* Dequantization of the packed outputs of mase_mxint_qdq (kind 0: p0 = element_bits, p1 unused; value = code *
+ * 2^(scale - 134)) or mase_mxfp_qdq (kind 1: p0 = exp_bits, p1 = frac_bits; value = minifloat(code) * 2^(scale - 127),
+ * NaN for a block whose scale byte is 255): codes (numel bytes), scales (numel / block_size bytes) -> out (numel
+ * elements of out_dtype).  The "compose" half of the reference's quantizers (nn/quantizers/mxint/fake.py:59-80,
+ * nn/quantizers/mxfp/fake.py:75-104), for loading checkpoints that store codes and scales. */
+int mase_mx_unpack(const uint8_t* codes, const uint8_t* scales, void* out, size_t numel, int block_size, int out_dtype,
+                   int kind, int p0, int p1, void* stream);
 
 /* C[M,N] = A[M,K] * B[N,K]^T (+ bias[N]): bf16 operands (both K-major, 16-byte aligned, K % 64 == 0), fp32
  * accumulation on the matrix cores, C written in out_dtype.  bias may be NULL; bias_dtype is its MASE_DT_*.

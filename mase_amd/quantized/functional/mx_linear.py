@@ -102,6 +102,32 @@ class PackedMXFPWeight:
         """declare the image current for ``weight`` as it is now (after its in-place quantization)"""
         self._key = _weight_key(weight)
 
+    def from_reference_codes(self, codes: Tensor, scales: Tensor, fmt) -> bool:
+        """Build the image from the quantizer's own element codes (one ``sign|exp|frac`` byte per element) and scale
+        bytes, e.g. those of a packed checkpoint.  The bit fields are the hardware's; e2m1 codes are put two to a
+        byte.  Returns False (no image) when a block uses a code the hardware format reserves."""
+        fmt = tuple(fmt)
+        codes = codes.contiguous()
+        if fmt == (2, 1):
+            hw = (codes[..., 0::2] & 0xF) | (codes[..., 1::2] << 4)
+        else:
+            reserved = ((codes & 0x7F) == 0x7F) if fmt == (4, 3) else (((codes >> 2) & 0x1F) == 0x1F)
+            if bool(reserved.any()):
+                return False
+            hw = codes
+        self.codes, self.scales, self.fmt = hw.contiguous(), scales.contiguous(), fmt
+        return True
+
+    def decodes_to(self, weight: Tensor) -> bool:
+        """whether the image holds exactly the values of ``weight``"""
+        from ...quantizers._ops import mx_unpack
+
+        codes = self.codes
+        if self.fmt == (2, 1):  # two codes per byte, even element in the low nibble
+            codes = torch.stack((codes & 0xF, codes >> 4), dim=-1).reshape(*codes.shape[:-1], -1)
+        got = mx_unpack(codes, self.scales, 32, weight.dtype, "mxfp", *self.fmt).view(weight.shape)
+        return bool(torch.equal(got, weight))
+
     def valid_for(self, weight: Tensor) -> bool:
         return self.codes is not None and self._key == _weight_key(weight)
 

@@ -103,6 +103,11 @@ class _LinearMX(_LinearBase):
     def _after_quantize_params(self):
         pass
 
+    def weights_loaded_quantized(self):
+        """Tell the module that its parameters were just set to already quantized values (a packed checkpoint): the
+        cached images are rebuilt from them on the next forward."""
+        self._w_cache.invalidate()
+
 
 class LinearMXInt(_LinearMX):
     def _quantize_params(self):
@@ -162,6 +167,24 @@ class LinearMXFP(_LinearMX):
     def _after_quantize_params(self):
         if self._w_packed.codes is not None:
             self._w_packed.bind(self.weight)
+
+    def weights_loaded_quantized(self, codes=None, scales=None):
+        """``codes`` / ``scales``: the quantizer's element codes and scale bytes of the weight, when the caller has
+        them (a packed checkpoint).  The matrix-instruction image is built from them; it cannot be rebuilt from the
+        quantized weight alone, because quantizing is not idempotent (an element equal to the smallest subnormal of
+        the format quantizes to zero).  The image is kept only if it decodes to exactly the weight."""
+        super().weights_loaded_quantized()
+        self._w_packed.invalidate()
+        if codes is None or self.bypass or self.gptq or not self.config.get("native_mx", True):
+            return
+        fmt = self._weight_fmt()
+        if not PackedMXFPWeight.eligible(self.weight, self.config["weight_block_size"], fmt):
+            return
+        if self._w_packed.from_reference_codes(codes.to(self.weight.device), scales.to(self.weight.device), fmt) \
+                and self._w_packed.decodes_to(self.weight.data):
+            self._w_packed.bind(self.weight)
+        else:
+            self._w_packed.invalidate()
 
     def _quantize_params(self):
         cfg = self.config

@@ -112,6 +112,24 @@ def mxfp_qdq(x: Tensor, block_size: int, exp_bits: int, frac_bits: int, block_di
     return (res, codes, scales) if pack else res
 
 
+def mx_unpack(codes: Tensor, scales: Tensor, block_size: int, dtype: torch.dtype, kind: str, p0: int, p1: int = 0) -> Tensor:
+    """Dequantize packed MX codes (flat, one byte per element, blocks of ``block_size`` consecutive elements) and
+    their scale bytes, as produced by ``mxint_qdq(..., pack=True)`` (``kind="mxint"``, ``p0`` = element bits) or
+    ``mxfp_qdq(..., pack=True)`` (``kind="mxfp"``, ``p0``/``p1`` = exponent / fraction bits).  Returns a flat tensor
+    of ``dtype`` (reference: compose_mxint_tensor mxint/fake.py:59-80, mxfp compose mxfp/fake.py:75-104)."""
+    _lib.require_device(codes, "mx_unpack")
+    lib = _lib.load()
+    codes, scales = codes.contiguous().reshape(-1), scales.contiguous().reshape(-1)
+    assert codes.dtype in (torch.int8, torch.uint8) and scales.dtype == torch.uint8
+    assert codes.numel() == scales.numel() * block_size
+    out = torch.empty(codes.numel(), dtype=dtype, device=codes.device)
+    rc = lib.mase_mx_unpack(codes.data_ptr(), scales.data_ptr(), out.data_ptr(), codes.numel(), int(block_size),
+                            _lib.DTYPE_CODE[dtype], {"mxint": 0, "mxfp": 1}[kind], int(p0), int(p1),
+                            _lib.stream_ptr(codes))
+    _lib.check(rc, "mase_mx_unpack")
+    return out
+
+
 # ------------------------------------------------------------------------------------------------
 # block floating point  (reference: block_fp.py:111-142; blocking utils.py:350-629)
 # ------------------------------------------------------------------------------------------------

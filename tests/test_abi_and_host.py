@@ -245,3 +245,16 @@ def test_module_pass_swaps_llama_blocks_on_the_host():
     assert net.norm.variance_epsilon == 1e-5 and net.norm.x_quantizer is None
     with pytest.raises(ValueError):
         quantize_module_transform_pass(net, {"by": "name", "act": {"config": {"name": "mxint"}}})
+
+
+def test_unpack_rejects_bad_arguments_without_a_gpu(lib):
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    # mase_mx_unpack(codes, scales, out, numel, block_size, out_dtype, kind, p0, p1, stream)
+    assert lib.mase_mx_unpack(p, p, p, 0, 32, 0, 0, 8, 0, None) == 0
+    assert lib.mase_mx_unpack(None, p, p, 64, 32, 0, 0, 8, 0, None) == -1
+    assert lib.mase_mx_unpack(p, p, p, 65, 32, 0, 0, 8, 0, None) == -2
+    assert lib.mase_mx_unpack(p, p, p, 64, 32, 0, 0, 9, 0, None) == -5     # codes are one byte
+    assert lib.mase_mx_unpack(p, p, p, 64, 32, 0, 1, 5, 3, None) == -5     # sign + 5 + 3 bits do not fit a byte
+    assert lib.mase_mx_unpack(p, p, p, 64, 32, 0, 2, 8, 0, None) == -5     # unknown kind
+    assert lib.mase_mx_unpack(p, p, p, 64, 32, 7, 0, 8, 0, None) == -4
