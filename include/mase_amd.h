@@ -17,6 +17,7 @@
  *   mase_minifloat_qdq      nn/quantizers/minifloat.py:90-117, :200-225 (minifloat_denorm/ieee_quantizer)
  *   mase_minifloat_mx_qdq   nn/quantizers/_minifloat_mx/minifloat.py:12-33 (minifloat_quantizer_sim)
  *   mase_mxfp_qdq           nn/quantizers/mxfp/mxfp.py:187-230    (mxfp_quantizer, non-search branch)
+ *   mase_attn_softmax_mx    nn/quantized/modules/llama/attention.py:363-392 (scores -> quantized probabilities)
  *   mase_mx_unpack          nn/quantizers/mxint/fake.py:59-80, nn/quantizers/mxfp/fake.py:75-104 (compose_*)
  *   mase_mxfp_pack, mase_gemm_mxfp_scaled   nn/quantized/modules/linear.py:877-895 (LinearMXFP.forward on
  *                           formats the block-scaled matrix instruction supports)
@@ -150,6 +151,21 @@ int mase_mxfp_pack(const void* in, uint8_t* codes, uint8_t* scales, size_t numel
 int mase_gemm_mxfp_scaled(const void* A, const void* A_scales, int a_format, const void* B, const void* B_scales,
                           int b_format, const void* bias, void* C, size_t M, size_t N, size_t K, int out_dtype,
                           int bias_dtype, void* stream);
+
+/* Attention probabilities of the MX-quantized Llama attention in one pass: for scores [batch, heads, q_len, kv_len]
+ * (dense, dtype) and an optional additive mask [batch, 1, q_len, kv_len] of the same dtype (rows mask_row_stride
+ * elements apart, batches q_len rows apart):
+ *   w = scores * scaling; w += mask; w = minifloat cast (cast_exp_bits > 0; bit-level cast of mase_minifloat_mx_qdq);
+ *   p = softmax(float(w)) along kv_len, rounded to dtype; p = MX quantize-dequantize in blocks of 32 along kv_len
+ *   (mx_kind 0 none, 1 MXINT with mx_p0 element bits, 2 MXFP with mx_p0 / mx_p1 exponent / fraction bits),
+ * each intermediate rounded to dtype as the separate tensor operations would.  kv_len % 32 == 0, kv_len <= 8192.
+ * log2_tab_dtype: table of `dtype` (MXINT), log2_tab_f32: fp32 table (MXFP); the one not needed may be NULL.
+ * Replaces the score-to-probability part of _eager_attention_forward_mxfp / _mxint
+ * (nn/quantized/modules/llama/attention.py:363-392) with softmax_minifloat (nn/quantized/functional/softmax.py:41-57). */
+int mase_attn_softmax_mx(const void* scores, const void* mask, void* out, size_t batch, size_t heads, size_t q_len,
+                         size_t kv_len, size_t mask_row_stride, int dtype, float scaling, int cast_exp_bits,
+                         int cast_frac_bits, int cast_is_finite, int cast_round_mode, int mx_kind, int mx_p0, int mx_p1,
+                         const uint32_t* log2_tab_dtype, const uint32_t* log2_tab_f32, void* stream);
 
 /* Plain streaming copy of `bytes` (multiple of 16, 16-byte aligned pointers).  No counterpart in the reference:
  * it is the calibration kernel for the achievable-bandwidth ceiling and for scaling hardware byte counters. */

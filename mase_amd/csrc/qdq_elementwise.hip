@@ -354,64 +354,7 @@ struct MinifloatMxOp {
     return minifloat_mx_decode(minifloat_mx_encode(x, m), m);
   }
 
-  // Integer form of decode(encode(x)) on the fp32 bit fields, for elements whose code is an ordinary one:
-  //   ye = exponent field + bias - 127; fraction 23 -> 15 bits by truncation, 15 -> F bits in the format's rounding
-  //   mode; a carry out of the fraction is OR-ed into the exponent field; ye > e_hi saturates; ye == 0 takes the
-  //   shifted fraction, ye < 0 gives zero; the value is the code's [exponent|fraction] field moved to fp32's place
-  //   (codes with exponent field 0: the integer fraction times 2^(1-bias-F)).
-  // Returns false for what is left to the stepwise functions: fp32 subnormals and non-finite inputs, codes of the
-  // inf/nan exponent of a format that has them and, with INLINE_SUB = false (formats whose subnormal range is
-  // rarely reached), every code with exponent field 0.
-  template <bool INLINE_SUB>
-  __device__ __forceinline__ bool fast(float x, uint32_t addc, uint32_t tie, int ye_limit, float& y) const {
-    const int F = m.F;
-    const uint32_t xb = f2bits(x + 0.0f);  // -0.0 is "not negative" in the encode
-    const uint32_t ab = xb & 0x7FFFFFFFu;
-    const uint32_t Ef = ab >> 23;
-    const int ye = (int)Ef + (m.bias - 127);
-    const int shn = 15 - F;
-    const uint32_t m15 = (ab >> 8) & 0x7FFFu;
-    const uint32_t yf = (m15 + addc + ((m15 >> shn) & tie)) >> shn;  // 0 .. 2^F
-    const uint32_t cn = ((uint32_t)ye << F) | yf;
-    const uint32_t cmax = ((uint32_t)m.e_hi << F) | (uint32_t)m.frac_hi;
-    const uint32_t rebias = (uint32_t)(127 - m.bias) << 23;
-    const bool ordinary = (Ef - 1u < 254u) || ab == 0;
-    if constexpr (!INLINE_SUB) {
-      const uint32_t c = ye > m.e_hi ? cmax : cn;
-      const uint32_t yn = (c << (23 - F)) + rebias;
-      y = bits2f(ab == 0 ? 0u : ((xb & 0x80000000u) | yn));
-      return ordinary && (ye > 0 || ab == 0) && ye < ye_limit;
-    }
-    const uint32_t cs = yf ? ((yf | (1u << F)) >> 1) : 0u;
-    uint32_t c = ye > 0 ? cn : (ye == 0 ? cs : 0u);
-    c = ye > m.e_hi ? cmax : c;
-    c = ab == 0 ? 0u : c;
-    const uint32_t yn = (c << (23 - F)) + rebias;
-    const uint32_t ys = f2bits(ldexpf((float)c, 1 - m.bias - F));
-    y = bits2f((xb & 0x80000000u) | ((c >> F) != 0 ? yn : ys));
-    return ordinary && ye < ye_limit;
-  }
-
-  __device__ __forceinline__ void batch8(const float* x, float* y) const {
-    const int shn = 15 - m.F;
-    // rounding of the 15-bit fraction as one addition: nearest-even, up (any remainder), down / toward zero
-    const uint32_t addc = m.round_mode == 0 ? (1u << (shn - 1)) - 1u : (m.round_mode == 1 ? (1u << shn) - 1u : 0u);
-    const uint32_t tie = m.round_mode == 0 ? 1u : 0u;
-    // formats with inf/nan codes: an element that reaches the top ordinary exponent may carry into the inf/nan one
-    const int ye_limit = m.is_finite ? 0x7FFFFFFF : m.e_hi;
-    bool ok = true;
-    if (m.bias < 12) {  // uniform
-#pragma unroll
-      for (int j = 0; j < 8; ++j) ok &= fast<true>(x[j], addc, tie, ye_limit, y[j]);
-    } else {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) ok &= fast<false>(x[j], addc, tie, ye_limit, y[j]);
-    }
-    if (__builtin_expect(!ok, 0)) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) y[j] = minifloat_mx_decode(minifloat_mx_encode(x[j], m), m);
-    }
-  }
+  __device__ __forceinline__ void batch8(const float* x, float* y) const { minifloat_mx_qdq8(x, y, m); }
 };
 
 template <typename MakeOp>

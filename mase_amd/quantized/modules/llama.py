@@ -27,7 +27,7 @@ import torch
 from torch import Tensor, nn
 
 from ...quantizers import mxfp_quantizer, mxint_quantizer
-from ...quantizers._ops import minifloat_mx_qdq
+from ...quantizers._ops import attn_softmax_mx, attn_softmax_mx_supported, minifloat_mx_qdq
 from ..functional.activations import kv_cache_mxfp, kv_cache_mxint, rope_minifloat, rotate_half, silu_minifloat, softmax_minifloat
 
 
@@ -62,7 +62,13 @@ def _eager_attention_forward(kind, module, query, key, value, attention_mask, sc
     value_states = repeat_kv(value, module.num_key_value_groups)
     if not qk_bypass:
         query = _mx_quantizer(kind, qk_config)(query)
-    attn_weights = torch.matmul(query, key_states.transpose(2, 3)) * scaling
+    scores = torch.matmul(query, key_states.transpose(2, 3))
+    fused = _fused_probabilities(kind, module, scores, key_states, attention_mask, scaling, dropout, av_bypass, av_config,
+                                 softmax_bypass, softmax_config)
+    if fused is not None:
+        attn_output = torch.matmul(fused, value_states).transpose(1, 2).contiguous()
+        return attn_output, fused
+    attn_weights = scores * scaling
     if attention_mask is not None:
         causal_mask = attention_mask[:, :, :, : key_states.shape[-2]]
         attn_weights = attn_weights + causal_mask
@@ -76,6 +82,35 @@ def _eager_attention_forward(kind, module, query, key, value, attention_mask, sc
     attn_output = torch.matmul(attn_weights, value_states)
     attn_output = attn_output.transpose(1, 2).contiguous()
     return attn_output, attn_weights
+
+
+def _fused_probabilities(kind, module, scores, key_states, attention_mask, scaling, dropout, av_bypass, av_config,
+                         softmax_bypass, softmax_config):
+    """scores -> scaled, masked, minifloat-cast, softmax, MX-quantized probabilities in one kernel when the operands
+    allow it (device tensors, key length a multiple of 32 up to 8192, blocks of 32, no dropout); else None and the
+    caller runs the separate passes.  ``module.fused_probabilities = False`` switches it off."""
+    if not getattr(module, "fused_probabilities", True) or not scores.is_cuda:
+        return None
+    if dropout != 0.0 and module.training:
+        return None
+    if torch.is_grad_enabled() and scores.requires_grad:
+        return None
+    mx = None
+    if not av_bypass:
+        if av_config["data_in_block_size"] != 32:
+            return None
+        mx = ("mxfp", av_config["data_in_exponent_width"], av_config["data_in_frac_width"]) if kind == "mxfp" \
+            else ("mxint", av_config["data_in_width"])
+    cast = None
+    if not softmax_bypass:
+        cast = (softmax_config["data_in_exponent_width"], softmax_config["data_in_frac_width"],
+                softmax_config.get("data_in_is_finite", True), softmax_config.get("data_in_round_mode", "rn"))
+    mask = None
+    if attention_mask is not None:
+        mask = attention_mask[:, :, :, : key_states.shape[-2]]
+    if not attn_softmax_mx_supported(scores, mask):
+        return None
+    return attn_softmax_mx(scores, mask, scaling, cast, mx)
 
 
 _eager_attention_forward_mxfp = partial(_eager_attention_forward, "mxfp")

@@ -112,6 +112,48 @@ def mxfp_qdq(x: Tensor, block_size: int, exp_bits: int, frac_bits: int, block_di
     return (res, codes, scales) if pack else res
 
 
+ATTN_PROB_MAX_KV = 8192
+
+
+def attn_softmax_mx_supported(scores: Tensor, mask: Tensor | None) -> bool:
+    """whether ``attn_softmax_mx`` can take these operands (otherwise the caller runs the separate tensor passes)"""
+    if not (scores.is_cuda and scores.dim() == 4 and scores.dtype in _lib.DTYPE_CODE and scores.numel() > 0):
+        return False
+    B, H, S, T = scores.shape
+    if T % 32 != 0 or T > ATTN_PROB_MAX_KV:
+        return False
+    if mask is None:
+        return True
+    return (mask.dim() == 4 and mask.dtype == scores.dtype and mask.device == scores.device
+            and tuple(mask.shape) == (B, 1, S, T) and mask.stride(3) == 1 and mask.stride(2) % 8 == 0
+            and mask.stride(2) >= T and (B == 1 or mask.stride(0) == S * mask.stride(2)) and mask.data_ptr() % 16 == 0)
+
+
+def attn_softmax_mx(scores: Tensor, mask: Tensor | None, scaling: float, cast: tuple | None, mx: tuple | None) -> Tensor:
+    """Quantized attention probabilities from the raw query-key products in one pass (``mase_attn_softmax_mx``).
+    ``cast``: (exp_bits, frac_bits, is_finite, round_mode) of the softmax input's minifloat cast or None;
+    ``mx``: ("mxint", element_bits) / ("mxfp", exp_bits, frac_bits) for blocks of 32 along the last dim, or None."""
+    _lib.require_device(scores, "attn_softmax_mx")
+    lib = _lib.load()
+    assert attn_softmax_mx_supported(scores, mask)
+    scores = scores.contiguous()
+    B, H, S, T = scores.shape
+    out = torch.empty_like(scores)
+    ce, cf, cfin, crm = (0, 0, 1, 0) if cast is None else (int(cast[0]), int(cast[1]), int(bool(cast[2])), _ROUND_MODES[cast[3]])
+    kind, p0, p1, tab_t, tab_f = 0, 0, 0, None, None
+    if mx is not None and mx[0] == "mxint":
+        kind, p0 = 1, int(mx[1])
+        tab_t = log2_table(scores.dtype, scores.device).data_ptr()
+    elif mx is not None:
+        kind, p0, p1 = 2, int(mx[1]), int(mx[2])
+        tab_f = log2_table(torch.float32, scores.device).data_ptr()
+    rc = lib.mase_attn_softmax_mx(scores.data_ptr(), None if mask is None else mask.data_ptr(), out.data_ptr(), B, H, S, T,
+                                  0 if mask is None else mask.stride(2), _lib.dtype_code(scores), float(scaling), ce, cf,
+                                  cfin, crm, kind, p0, p1, tab_t, tab_f, _lib.stream_ptr(scores))
+    _lib.check(rc, "mase_attn_softmax_mx")
+    return out
+
+
 def mx_unpack(codes: Tensor, scales: Tensor, block_size: int, dtype: torch.dtype, kind: str, p0: int, p1: int = 0) -> Tensor:
     """Dequantize packed MX codes (flat, one byte per element, blocks of ``block_size`` consecutive elements) and
     their scale bytes, as produced by ``mxint_qdq(..., pack=True)`` (``kind="mxint"``, ``p0`` = element bits) or

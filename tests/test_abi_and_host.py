@@ -258,3 +258,21 @@ def test_unpack_rejects_bad_arguments_without_a_gpu(lib):
     assert lib.mase_mx_unpack(p, p, p, 64, 32, 0, 1, 5, 3, None) == -5     # sign + 5 + 3 bits do not fit a byte
     assert lib.mase_mx_unpack(p, p, p, 64, 32, 0, 2, 8, 0, None) == -5     # unknown kind
     assert lib.mase_mx_unpack(p, p, p, 64, 32, 7, 0, 8, 0, None) == -4
+
+
+def test_attention_probability_entry_point_rejects_bad_arguments_without_a_gpu(lib):
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    # (scores, mask, out, batch, heads, q_len, kv_len, mask_row_stride, dtype, scaling, cast E, F, finite, round,
+    #  mx_kind, p0, p1, tab_dtype, tab_f32, stream)
+    call = lib.mase_attn_softmax_mx
+    assert call(p, None, p, 0, 4, 8, 64, 0, 1, 0.125, 4, 3, 1, 0, 1, 8, 0, p, None, None) == 0       # empty
+    assert call(None, None, p, 1, 4, 8, 64, 0, 1, 0.125, 4, 3, 1, 0, 1, 8, 0, p, None, None) == -1
+    assert call(p, None, p, 1, 4, 8, 48, 0, 1, 0.125, 4, 3, 1, 0, 1, 8, 0, p, None, None) == -2      # whole blocks of 32
+    assert call(p, None, p, 1, 4, 8, 16384, 0, 1, 0.125, 4, 3, 1, 0, 1, 8, 0, p, None, None) == -2   # row too long
+    assert call(p, p, p, 1, 4, 8, 64, 32, 1, 0.125, 4, 3, 1, 0, 1, 8, 0, p, None, None) == -2        # mask rows overlap
+    assert call(p, None, p, 1, 4, 8, 64, 0, 5, 0.125, 4, 3, 1, 0, 1, 8, 0, p, None, None) == -4
+    assert call(p, None, p, 1, 4, 8, 64, 0, 1, 0.125, 9, 3, 1, 0, 1, 8, 0, p, None, None) == -5      # cast format
+    assert call(p, None, p, 1, 4, 8, 64, 0, 1, 0.125, 4, 3, 1, 0, 2, 3, 3, None, p, None) == -5      # MXFP format
+    assert call(p, None, p, 1, 4, 8, 64, 0, 1, 0.125, 4, 3, 1, 0, 1, 8, 0, None, None, None) == -1   # table missing
+    assert call(p, None, p, 1, 4, 8, 64, 0, 1, 0.125, 4, 3, 1, 0, 3, 8, 0, p, p, None) == -5         # unknown kind
