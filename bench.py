@@ -10,6 +10,11 @@ Workloads (the headline configurations):
     mxint_linear config 3: MXINT8 Linear forward, 4096x4096x4096, fp32 in/out
     mxfp_linear  config 4: MXFP4(e2m1) weights x MXFP8(e4m3) activations Linear, M=8192 K=8192 N=28672
     decoder_layer config 5: Llama-style decoder layer, every nn.Linear -> LinearMXInt, batch 8 x seq 2048, bf16
+Secondary workloads (other rows of the path, same JSON; --dtype bf16|f32|f16 where it applies):
+    integer_qdq, minifloat_denorm_qdq, minifloat_ieee_qdq, minifloat_mx_qdq, mxfp_qdq   on [8,2048,4096]
+    attn_prob    score -> probability chain of the MX-quantized attention on [4,32,2048,2048]
+    decode_linear  LinearMXInt 8192 -> 28672 for 16 tokens (weight-streaming kernel)
+    copy         calibration copy
 Prints ONE JSON line.  `value` is algorithmic GB/s (Q-DQ) or TFLOP/s (Linear) over the whole timed region;
 `roofline` is for the dominant kernel, timed with HIP events on the launch stream; `cpu_baseline` is the CPU
 oracle timed on this box's host cores on a bounded sample of the same workload.
@@ -400,7 +405,190 @@ class DecoderLayerMxint(Workload):
                           f"{dt*1e3:.0f} ms each"}
 
 
-WORKLOADS = {w.name: w for w in (BfpQdq, MxintQdq, MxintLinear, MxfpLinear, DecoderLayerMxint, CopyBytes)}
+class _ElementwiseQdq(Workload):
+    """the element-wise / per-block quantizers on a tensor of config 2's size ([8,2048,4096], N(0,1), seed 5) in the
+    dtype given by --dtype (default bf16)"""
+    shape = (8, 2048, 4096)
+    torch_dtype = None
+    fn_name = ""
+    args = ()
+
+    def setup(self, torch, dev, n_buffers):
+        import mase_amd.quantizers as Q
+
+        self.fn = getattr(Q, self.fn_name)
+        g = torch.Generator().manual_seed(5)
+        self.host = torch.randn(*self.shape, generator=g).to(self.torch_dtype)
+        self.bufs = [self.host.to(dev).roll(i, dims=1).contiguous() for i in range(n_buffers)]
+        self.dtype = {torch.bfloat16: "bf16", torch.float32: "f32", torch.float16: "f16"}[self.torch_dtype]
+        self.config = {"workload": f"{self.fn_name}{self.args} on {self.dtype} {list(self.shape)}, N(0,1) seed 5"}
+        self.metric = (f"{self.fn_name} throughput (algorithmic bytes: {self.host.element_size()} B read + "
+                       f"{self.host.element_size()} B written per element)")
+
+    def step(self, i):
+        self.out = self.fn(self.bufs[i % len(self.bufs)], *self.args)
+
+    def work_per_step(self):
+        return float(self.host.numel() * 2 * self.host.element_size())
+
+    def cpu_baseline(self, torch, budget_s):
+        import oracle as O
+
+        fn = getattr(O, self.oracle_name)
+        x = self.host[:1].contiguous()  # one of the 8 batch items
+        fn(x[:, :64].contiguous(), *self.oracle_args)
+        t0 = time.perf_counter()
+        n = 0
+        while True:
+            fn(x, *self.oracle_args)
+            n += 1
+            if time.perf_counter() - t0 > budget_s or n >= 20:
+                break
+        dt = (time.perf_counter() - t0) / n
+        return {"value": self.work_per_step() / 8 / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                "kind": "port", "sample": f"{n} passes over one batch item [1,2048,4096], {dt*1e3:.0f} ms each"}
+
+
+class IntegerQdq(_ElementwiseQdq):
+    name, unit, kernel = "integer_qdq", "GB/s", "elementwise_kernel<IntegerOp>"
+    fn_name, args = "integer_quantizer", (8, 4)
+    oracle_name, oracle_args = "integer_quantizer", (8, 4)
+
+
+class MinifloatDenormQdq(_ElementwiseQdq):
+    name, unit, kernel = "minifloat_denorm_qdq", "GB/s", "minifloat_value_kernel"
+    fn_name, args = "minifloat_denorm_quantizer", (8, 4, None)
+    oracle_name, oracle_args = "minifloat_denorm_quantizer", (8, 4, None)
+
+
+class MinifloatIeeeQdq(_ElementwiseQdq):
+    name, unit, kernel = "minifloat_ieee_qdq", "GB/s", "minifloat_value_kernel"
+    fn_name, args = "minifloat_ieee_quantizer", (8, 4, None)
+    oracle_name, oracle_args = "minifloat_ieee_quantizer", (8, 4, None)
+
+
+class MxfpQdq(_ElementwiseQdq):
+    name, unit, kernel = "mxfp_qdq", "GB/s", "mxfp_qdq_vec_kernel"
+    fn_name, args = "mxfp_quantizer", (32, 4, 3)
+    oracle_name, oracle_args = "mxfp_quantizer", (32, 4, 3)
+
+
+class MinifloatMxQdq(_ElementwiseQdq):
+    name, unit, kernel = "minifloat_mx_qdq", "GB/s", "elementwise_kernel<MinifloatMxOp>"
+    oracle_name, oracle_args = "minifloat_quantizer_sim", (4, 3, True, "rn")
+
+    def setup(self, torch, dev, n_buffers):
+        import mase_amd.quantizers as Q
+
+        self.fn_name = "minifloat_quantizer_sim"
+        super().setup(torch, dev, n_buffers)
+        meta = Q.MinifloatMeta(exp_bits=4, frac_bits=3, is_finite=True, round_mode="rn")
+        self.fn = lambda t: Q.minifloat_quantizer_sim(t, meta)
+        self.config = {"workload": f"minifloat_quantizer_sim e4m3 finite rn on {self.dtype} {list(self.shape)}, N(0,1) seed 5"}
+
+
+class AttnProb(Workload):
+    """score -> probability chain of the MX-quantized Llama attention (scale, causal mask, minifloat cast e5m8,
+    fp32 softmax, MXINT8 blocks of 32) on [4,32,2048,2048]"""
+    name = "attn_prob"
+    unit = "GB/s"
+    kernel = "attn_prob_kernel"
+    shape = (4, 32, 2048, 2048)
+    torch_dtype = None
+
+    def setup(self, torch, dev, n_buffers):
+        from mase_amd.quantizers._ops import attn_softmax_mx
+
+        self.op = attn_softmax_mx
+        B, H, S, T = self.shape
+        dt = self.torch_dtype
+        self.dtype = {torch.bfloat16: "bf16", torch.float32: "f32", torch.float16: "f16"}[dt]
+        g = torch.Generator(device=dev).manual_seed(6)
+        self.bufs = [(torch.randn(B, H, S, T, device=dev, generator=g) * 4).to(dt) for _ in range(max(2, min(n_buffers, 3)))]
+        self.mask = torch.triu(torch.full((S, T), torch.finfo(dt).min, dtype=dt, device=dev), diagonal=1)[None, None] \
+            .expand(B, 1, S, T).contiguous()
+        self.esize = self.bufs[0].element_size()
+        self.metric = (f"attention probability chain throughput (algorithmic bytes: {self.esize} B of scores read + "
+                       f"{self.esize} B of probabilities written per element)")
+        self.config = {"workload": f"scores {self.dtype} {list(self.shape)} N(0,16) seed 6, scaling 0.0884, causal mask, "
+                                   "cast e5m8, softmax, MXINT8 block 32"}
+
+    def step(self, i):
+        self.out = self.op(self.bufs[i % len(self.bufs)], self.mask, 0.0884, (5, 8, True, "rn"), ("mxint", 8))
+
+    def work_per_step(self):
+        B, H, S, T = self.shape
+        return float(B * H * S * T * 2 * self.esize)
+
+    def cpu_baseline(self, torch, budget_s):
+        import oracle as O
+
+        x = self.bufs[0][0, :2].cpu()[None]           # 2 heads of one batch item
+        m = self.mask[:1].cpu()
+        t0 = time.perf_counter()
+        n = 0
+        while True:
+            w = x * 0.0884 + m
+            w = O.minifloat_quantizer_sim(w, 5, 8, True, "rn")
+            w = torch.softmax(w.to(torch.float32), dim=-1).to(x.dtype)
+            O.mxint_quantizer(w, 32, 8, block_dim=-1)
+            n += 1
+            if time.perf_counter() - t0 > budget_s or n >= 10:
+                break
+        dt = (time.perf_counter() - t0) / n
+        return {"value": x.numel() * 2 * self.esize / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                "kind": "port", "sample": f"{n} passes of the separate tensor operations over 2 heads [1,2,2048,2048], {dt*1e3:.0f} ms each"}
+
+
+class DecodeLinear(Workload):
+    """LinearMXInt forward for a handful of tokens: bound by streaming the weight once"""
+    name = "decode_linear"
+    unit = "GB/s"
+    dtype = "bf16"
+    kernel = "gemm_skinny_partial_kernel"
+    M, N, K = 16, 28672, 8192
+    metric = "MXINT8 Linear forward for 16 tokens (algorithmic bytes: the bf16 weight image, 2 B per weight, read once)"
+    config = {"workload": "LinearMXInt 8192 -> 28672, 16 tokens, bf16, weights N(0,0.02) seed 7"}
+
+    def setup(self, torch, dev, n_buffers):
+        from mase_amd.quantized import LinearMXInt
+
+        cfg = {"weight_block_size": 32, "weight_width": 8, "data_in_block_size": 32, "data_in_width": 8}
+        g = torch.Generator().manual_seed(7)
+        self.mods = []
+        for i in range(2):  # two layers, alternated: the 470 MB weight cannot stay in the last-level cache
+            m = LinearMXInt(self.K, self.N, bias=False, device=dev, dtype=torch.bfloat16, config=dict(cfg))
+            m.load_state_dict({"weight": (torch.randn(self.N, self.K, generator=g) * 0.02).bfloat16()})
+            self.mods.append(m)
+        self.x = torch.randn(self.M, self.K, generator=g).bfloat16().to(dev)
+
+    def step(self, i):
+        self.out = self.mods[i % 2](self.x)
+
+    def work_per_step(self):
+        return float(self.N * self.K * 2)
+
+    def cpu_baseline(self, torch, budget_s):
+        from oracle import linear as OL
+
+        cfg = {"weight_block_size": 32, "weight_width": 8, "data_in_block_size": 32, "data_in_width": 8}
+        n_rows = 2048
+        w = self.mods[0].weight.data[:n_rows].float().cpu()
+        x = self.x.float().cpu()
+        t0 = time.perf_counter()
+        n = 0
+        while True:
+            OL.linear_mxint_forward(x, w, None, cfg)
+            n += 1
+            if time.perf_counter() - t0 > budget_s or n >= 20:
+                break
+        dt = (time.perf_counter() - t0) / n
+        return {"value": n_rows * self.K * 2 / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                "sample": f"{n} forwards with {n_rows} of the {self.N} output rows (fp32 on the CPU), {dt*1e3:.0f} ms each"}
+
+
+WORKLOADS = {w.name: w for w in (BfpQdq, MxintQdq, MxintLinear, MxfpLinear, DecoderLayerMxint, CopyBytes, IntegerQdq,
+                                 MinifloatDenormQdq, MinifloatIeeeQdq, MinifloatMxQdq, MxfpQdq, AttnProb, DecodeLinear)}
 
 
 def load_traffic(name):
@@ -419,6 +607,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="bfp_qdq", choices=sorted(WORKLOADS))
     ap.add_argument("--buffers", type=int, default=4)
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "f32", "f16"],
+                    help="tensor dtype of the secondary workloads (the headline ones fix theirs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     a = ap.parse_args()
@@ -435,6 +625,8 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     w = WORKLOADS[a.workload]()
+    if hasattr(w, "torch_dtype"):
+        w.torch_dtype = {"bf16": torch.bfloat16, "f32": torch.float32, "f16": torch.float16}[a.dtype]
     w.setup(torch, dev, a.buffers)
     for i in range(a.warmup):
         w.step(i)

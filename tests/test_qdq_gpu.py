@@ -251,9 +251,16 @@ def test_minifloat_mx(Q, dev, fmt, finite):
         assert_bits_equal(got, want, f"minifloat_mx e{e}m{f} finite={finite} {rm}")
     for dtype in (torch.bfloat16, torch.float16):
         x = all_16bit(dtype)
+        for rm in ("rn", "ru", "rd", "rz"):  # every 16-bit value in every mode: the packed 16-bit kernel's domain
+            meta = Q.MinifloatMeta(e, f, finite, rm)
+            assert_bits_equal(Q.minifloat_quantizer_sim(x.to(dev), meta), O.minifloat_quantizer_sim(x, e, f, finite, rm),
+                              f"minifloat_mx {dtype} e{e}m{f} finite={finite} {rm}")
+            # a lane's 8 elements are handled together: shuffled order and an unaligned view
+            perm = torch.randperm(65536, generator=torch.Generator().manual_seed(e * 8 + f))
+            xs = x[perm]
+            assert_bits_equal(Q.minifloat_quantizer_sim(xs.to(dev)[3:], meta), O.minifloat_quantizer_sim(xs[3:], e, f, finite, rm),
+                              f"minifloat_mx {dtype} e{e}m{f} {rm} shuffled")
         meta = Q.MinifloatMeta(e, f, finite, "rn")
-        assert_bits_equal(Q.minifloat_quantizer_sim(x.to(dev), meta), O.minifloat_quantizer_sim(x, e, f, finite, "rn"),
-                          f"minifloat_mx {dtype} e{e}m{f}")
         assert_bits_equal(Q.minifloat_quantizer_sim(x.to(dev), meta, output_dtype=torch.float32),
                           O.minifloat_quantizer_sim(x, e, f, finite, "rn", torch.float32), "output dtype")
 
