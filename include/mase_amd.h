@@ -167,12 +167,6 @@ int mase_attn_softmax_mx(const void* scores, const void* mask, void* out, size_t
                          int cast_frac_bits, int cast_is_finite, int cast_round_mode, int mx_kind, int mx_p0, int mx_p1,
                          const uint32_t* log2_tab_dtype, const uint32_t* log2_tab_f32, void* stream);
 
-/* out[i] = table[in[i]] over numel 16-bit elements (bf16 / fp16 bit patterns); table: 65536 uint16 in device memory.
- * No counterpart in the reference: it is how the element-wise quantizers (integer.py, minifloat.py,
- * _minifloat_mx/minifloat.py) are evaluated on 16-bit tensors, with a table the caller fills by running the
- * arithmetic entry point (mase_integer_qdq, mase_minifloat_qdq, mase_minifloat_mx_qdq) on all 65536 inputs. */
-int mase_lut16_apply(const void* in, void* out, size_t numel, const uint16_t* table, void* stream);
-
 /* Plain streaming copy of `bytes` (multiple of 16, 16-byte aligned pointers).  No counterpart in the reference:
  * it is the calibration kernel for the achievable-bandwidth ceiling and for scaling hardware byte counters. */
 int mase_copy_bytes(const void* in, void* out, size_t bytes, void* stream);
