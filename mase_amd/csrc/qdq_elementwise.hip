@@ -6,6 +6,7 @@
 // (2^e underflowing to 0 in fp16, clamp bounds that T cannot represent, ...) are part of the result.
 #include "common.hpp"
 #include "minifloat_mx.hpp"
+#include "pk16_cast.hpp"
 
 namespace mase {
 namespace {
@@ -358,88 +359,35 @@ struct MinifloatMxOp {
 };
 
 // ---------------------------------------------------------------------------------------------
-// Bit-level minifloat cast of a 16-bit tensor to the same dtype, two elements per 32-bit register.
-// For an element whose code is an ordinary one (exponent field of the code in [1, e_hi]) the cast only rounds the
-// element's mantissa (MB bits: 7 for bf16, 10 for fp16) to F bits; in the element's own bit pattern that is
-//   t  = |x| + round_add + tie_bit          (a carry out of the mantissa bumps the exponent field)
-//   y  = t with the dropped mantissa bits cleared
-//   the format ORs a carry into its exponent field, so a carry is lost when that field is odd: y -= one exponent step
-//   y  = min(y, largest value of the format), sign put back (a zero keeps no sign)
-// all of it with packed 16-bit integer instructions on both halves of a register at once (about 9 instructions per
-// element instead of 30).  Lanes holding an element outside that domain (codes with exponent field 0, underflow,
-// Inf/NaN, subnormal inputs, the inf/nan exponent of a format that has one) redo their 8 elements with the fp32 form.
-// SUB = true (formats whose smallest normal binade is within reach of ordinary data) also handles, in line, the binade
-// below the normal range, where the format shifts the rounded fraction right by one with truncation
-//   rounded fraction 0 -> zero;  a carry -> 1.0 * 2^e;  otherwise the lowest kept mantissa bit is cleared
-// and everything below that binade, which becomes a signed zero.
+// Bit-level minifloat cast of a 16-bit tensor to the same dtype with the packed 16-bit form (pk16_cast.hpp: about 9
+// instructions per element instead of 30, 17 with the in-line handling of the format's subnormal binade).  Lanes
+// holding an element outside its domain (Inf/NaN, inputs subnormal in the tensor dtype, the inf/nan exponent of a
+// format that has one and, without SUB, codes with exponent field 0) redo their 8 elements with the fp32 form.
 // ---------------------------------------------------------------------------------------------
-typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ u16x2 as_u16x2(uint32_t v) { return __builtin_bit_cast(u16x2, v); }
-__device__ __forceinline__ uint32_t as_u32(u16x2 v) { return __builtin_bit_cast(uint32_t, v); }
-
 struct MinifloatPk16Params {
-  uint32_t round_add2;  // per half: what is added before the dropped bits are cleared
-  uint32_t tie2;        // 0x00010001 for round-to-nearest-even, else 0
-  uint32_t keep2;       // per half: mask of sign-less bits that survive
-  uint32_t exp_lsb2;    // per half: lowest bit of the exponent field
-  uint32_t odd_k2;      // per half: exp_lsb if the code's exponent field is odd when the element's is even
-  uint32_t max2;        // per half: bit pattern of the format's largest value
+  Pk16Format f;
+  Pk16Range r;
   uint32_t lo_thr, hi_thr;  // an element e is in the domain iff e == 0 or lo_thr <= |e| < hi_thr (bit patterns)
-  uint32_t sub_thr;     // SUB: lowest pattern of the binade below lo_thr, whose elements take codes with exponent field 0
-  uint32_t keep_sub2;   // SUB: keep2 without its lowest mantissa bit
-  uint32_t exp_mask2;   // per half: the exponent field
-  int drop;             // mantissa bits dropped
   MinifloatMxFmt m;
 };
-
-// 0xFFFF in the halves where a (as a signed 16-bit number) is negative
-__device__ __forceinline__ uint32_t neg_mask2(uint32_t a) {
-  typedef short i16x2 __attribute__((ext_vector_type(2)));
-  const i16x2 fifteen = {15, 15};
-  return __builtin_bit_cast(uint32_t, __builtin_bit_cast(i16x2, a) >> fifteen);
-}
 
 template <int DT, bool SUB>
 __global__ __launch_bounds__(kEwThreads) void minifloat_mx_pk16_kernel(const uint4* __restrict__ in,
                                                                        uint4* __restrict__ out, size_t n8,
                                                                        MinifloatPk16Params p) {
+  constexpr int MB = (DT == MASE_DT_BF16) ? 7 : 10;
   const size_t i = (size_t)blockIdx.x * kEwThreads + threadIdx.x;
   if (i >= n8) return;
   const uint4 v = load_nt(in + i);
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};
   uint32_t r[4];
   u16x2 lo_acc = as_u16x2(0xFFFFFFFFu), hi_acc = as_u16x2(0u);
-  const u16x2 drop2 = {(unsigned short)p.drop, (unsigned short)p.drop};
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const uint32_t ab = w[j] & 0x7FFF7FFFu;
-    const uint32_t lsb = as_u32(as_u16x2(ab) >> drop2) & p.tie2;
-    const uint32_t t = as_u32(as_u16x2(ab) + as_u16x2(p.round_add2) + as_u16x2(lsb));
-    const uint32_t tm = t & p.keep2;
-    const uint32_t fix = (tm ^ ab) & (ab ^ p.odd_k2) & p.exp_lsb2;  // carry into an odd exponent field of the code
-    u16x2 ya = as_u16x2(tm) - as_u16x2(fix);
-    ya = __builtin_elementwise_min(ya, as_u16x2(p.max2));
-    uint32_t yv = as_u32(ya);
-    if constexpr (SUB) {
-      const uint32_t below_lo = neg_mask2(as_u32(as_u16x2(ab) - as_u16x2(p.lo_thr * 0x00010001u)));
-      const uint32_t below_sub = neg_mask2(as_u32(as_u16x2(ab) - as_u16x2(p.sub_thr * 0x00010001u)));
-      const uint32_t eonly = ab & p.exp_mask2;
-      const uint32_t carry = neg_mask2(((tm ^ ab) & p.exp_lsb2) << (15 - (DT == MASE_DT_BF16 ? 7 : 10)));
-      uint32_t ys = (carry & eonly) | (~carry & tm & p.keep_sub2);
-      const uint32_t z = tm ^ eonly;  // zero iff the rounded fraction is zero (and there was no carry)
-      ys &= neg_mask2(z | as_u32(as_u16x2(0u) - as_u16x2(z)));
-      yv = (below_lo & ys) | (~below_lo & yv);
-      yv &= ~below_sub;
-    }
-    const uint32_t nz = as_u32(as_u16x2(ab) + as_u16x2(0x7FFF7FFFu));  // bit 15 of a half: the element is not zero
-    r[j] = yv | (w[j] & nz & 0x80008000u);
-    lo_acc = __builtin_elementwise_min(lo_acc, as_u16x2(ab) - as_u16x2(0x00010001u));  // zero wraps to 0xFFFF
-    hi_acc = __builtin_elementwise_max(hi_acc, as_u16x2(ab));
-  }
+  for (int j = 0; j < 4; ++j) r[j] = pk16_cast<MB, SUB>(w[j], p.f, p.r, lo_acc, hi_acc);
   const uint32_t lo = min((uint32_t)lo_acc.x, (uint32_t)lo_acc.y), hi = max((uint32_t)hi_acc.x, (uint32_t)hi_acc.y);
   uint4 o = make_uint4(r[0], r[1], r[2], r[3]);
   // SUB: only inputs that are subnormal in T itself (or non-finite) are left over
-  const uint32_t lowest = SUB ? (1u << (DT == MASE_DT_BF16 ? 7 : 10)) : p.lo_thr;
+  const uint32_t lowest = SUB ? (1u << MB) : p.lo_thr;
   if (__builtin_expect(lo + 1u < lowest || hi >= p.hi_thr, 0)) {
     float x[8], y[8];
     DTypeTraits<DT>::unpack(v, x);
@@ -526,20 +474,13 @@ struct MinifloatMxRun {
     const int top = m.e_hi - m.bias + EB;      // exponent field (in T) of the format's largest binade
     const int bottom = 1 - m.bias + EB;        // and of its smallest normal binade
     if (m.F > MB || top > kMaxField || top < 1) return false;
-    const int drop = MB - m.F;
     const uint32_t one = 0x00010001u;
-    const uint32_t add = drop == 0 ? 0u : (m.round_mode == 0 ? (1u << (drop - 1)) - 1u : (m.round_mode == 1 ? (1u << drop) - 1u : 0u));
-    q.drop = drop;
-    q.round_add2 = add * one;
-    q.tie2 = (m.round_mode == 0 && drop > 0) ? one : 0u;
-    q.keep2 = (0x7FFFu & ~((1u << drop) - 1u)) * one;
-    q.exp_lsb2 = (1u << MB) * one;
-    q.odd_k2 = (((m.bias - EB) & 1) ? (1u << MB) : 0u) * one;
-    q.max2 = (((uint32_t)top << MB) | ((uint32_t)m.frac_hi << drop)) * one;
+    q.f = make_pk16_format<MB>(m.F, m.round_mode);
+    q.r.odd_k2 = (((m.bias - EB) & 1) ? (1u << MB) : 0u) * one;
+    q.r.max2 = (((uint32_t)top << MB) | ((uint32_t)m.frac_hi << q.f.drop)) * one;
     q.lo_thr = (uint32_t)(bottom < 1 ? 1 : bottom) << MB;
-    q.sub_thr = (uint32_t)(bottom - 1 < 1 ? 1 : bottom - 1) << MB;
-    q.keep_sub2 = q.keep2 & ~((1u << drop) * one);
-    q.exp_mask2 = (0x7FFFu & ~((1u << MB) - 1u)) * one;
+    q.r.lo_thr2 = q.lo_thr * one;
+    q.r.sub_thr2 = ((uint32_t)(bottom - 1 < 1 ? 1 : bottom - 1) << MB) * one;
     // Inf/NaN inputs, and for a format with inf/nan codes every element of its top ordinary binade
     q.hi_thr = m.is_finite ? ((uint32_t)(kMaxField + 1) << MB) : ((uint32_t)top << MB);
     q.m = m;

@@ -12,6 +12,7 @@
 #include "common.hpp"
 #include "minifloat_mx.hpp"
 #include "mxfp_core.hpp"
+#include "pk16_cast.hpp"
 
 namespace mase {
 namespace {
@@ -100,6 +101,68 @@ __global__ __launch_bounds__(kVecThreads) void mxfp_qdq_vec_kernel(const void* _
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// MXFP quantize-dequantize of a 16-bit tensor to the same dtype with the packed 16-bit cast (pk16_cast.hpp).
+// Dividing an element by 2^sh, casting it and multiplying by 2^sh again is, in the element's own bit pattern, the
+// cast with its thresholds moved up by sh exponent steps: the block's scale only changes per-lane constants (largest
+// value, lowest ordinary pattern, parity of the code's exponent field), the elements are never rescaled.
+// LPB lanes of 8 elements share a block.  SUBN handles the binade below the format's normal range in line (needed
+// for the narrow-exponent formats, where it lies a few binades under the block maximum).  A lane redoes its elements
+// with the fp32 form when its block is not regular (all flushed, non-finite) or when it holds an element outside the
+// packed form's domain (subnormal in the tensor dtype or, without SUBN, below the format's normal range).
+// ---------------------------------------------------------------------------------------------
+struct MxfpPk16Params {
+  Pk16Format f;
+  int top0, bot0;     // exponent fields (in T) of the format's largest / smallest normal binade at scale 2^0
+  uint32_t maxfrac;   // mantissa bits of the format's largest value
+  int parity0;        // (format bias - T bias) & 1
+};
+
+template <int DT, int LPB, bool SUBN>
+__global__ __launch_bounds__(kVecThreads) void mxfp_qdq_pk16_kernel(const uint4* __restrict__ in, uint4* __restrict__ out,
+                                                                    size_t n_vec, MxfpParams p, MxfpPk16Params q) {
+  using TR = DTypeTraits<DT>;
+  constexpr int MB = (DT == MASE_DT_BF16) ? 7 : 10;
+  const size_t idx = (size_t)blockIdx.x * kVecThreads + threadIdx.x;
+  const bool live = idx < n_vec;  // whole blocks are live or dead together: n_vec is a multiple of LPB
+  WaveLog2 meta;
+  meta.init(p.tab, kLog2TabHalf);
+  const uint4 raw = live ? load_nt(in + idx) : make_uint4(0, 0, 0, 0);
+  const uint32_t m = group_max_u32<LPB>(vec_flushed_absmax<DT>(raw));
+  int sh = 0;
+  const int state = mxfp_block_scale(m, p, sh, meta);
+  // the cast's thresholds at this block's scale
+  const uint32_t one = 0x00010001u;
+  const int botf = q.bot0 + sh;
+  Pk16Range r;
+  r.odd_k2 = (((q.parity0 - sh) & 1) ? (1u << MB) : 0u) * one;
+  r.max2 = (((uint32_t)min(max(q.top0 + sh, 1), 0xFF) << MB) | q.maxfrac) * one;
+  const uint32_t lo_thr = (uint32_t)min(max(botf, 1), 0xFF) << MB;
+  r.lo_thr2 = lo_thr * one;
+  r.sub_thr2 = ((uint32_t)min(max(botf - 1, 1), 0xFF) << MB) * one;
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  uint32_t y[4];
+  u16x2 lo_acc = as_u16x2(0xFFFFFFFFu), hi_acc = as_u16x2(0u);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) y[j] = pk16_cast<MB, SUBN>(w[j], q.f, r, lo_acc, hi_acc);
+  const uint32_t lo = min((uint32_t)lo_acc.x, (uint32_t)lo_acc.y);
+  uint4 o = make_uint4(y[0], y[1], y[2], y[3]);
+  // outside the packed form's domain: elements subnormal in T, elements whose quotient by 2^sh leaves the fp32 normal
+  // range (bf16 shares fp32's exponent field: field <= sh; a quotient that underflows to zero loses its sign in the
+  // reference) and, without SUBN, elements below the format's normal range
+  uint32_t lowest = SUBN ? (1u << MB) : lo_thr;
+  if constexpr (DT == MASE_DT_BF16) lowest = max(lowest, (uint32_t)min(max(sh + 1, 1), 0xFF) << MB);
+  if (__builtin_expect(state != 1 || lo + 1u < lowest, 0)) {
+    float x[8], z[8];
+    uint32_t c[8];
+    TR::unpack(raw, x);
+    if (p.m.E >= 4) mxfp_elements<false, 8>(x, state, sh, p, c, z);
+    else mxfp_elements<true, 8>(x, state, sh, p, c, z);
+    o = TR::pack(z);
+  }
+  if (live) store_nt(out + idx, o);
+}
+
 template <int DTI, int DTO>
 __global__ __launch_bounds__(kThreads) void mxfp_qdq_generic_kernel(const void* __restrict__ in, void* __restrict__ out,
                                                                     uint8_t* __restrict__ codes,
@@ -131,6 +194,36 @@ int launch_mxfp(const void* in, void* out, uint8_t* codes, uint8_t* scales, size
   if (vec_ok) {
     size_t n_vec = numel / V;
     dim3 grid(blocks_for(n_vec, (size_t)kVecThreads)), block(kVecThreads);
+    if constexpr (DTI == DTO && DTI != MASE_DT_F32) {
+      // packed 16-bit form: same dtype in and out, no codes wanted, a block is 1, 2, 4 or 8 lanes of 8 elements
+      constexpr int MB = (DTI == MASE_DT_BF16) ? 7 : 10, EB = (DTI == MASE_DT_BF16) ? 127 : 15;
+      const int lpb = B / 8;
+      if (codes == nullptr && B % 8 == 0 && lpb <= 8 && p.m.F <= MB) {
+        MxfpPk16Params q;
+        q.f = make_pk16_format<MB>(p.m.F, 0);
+        q.top0 = p.m.e_hi - p.m.bias + EB;
+        q.bot0 = 1 - p.m.bias + EB;
+        q.maxfrac = (uint32_t)p.m.frac_hi << q.f.drop;
+        q.parity0 = (p.m.bias - EB) & 1;
+        const uint4* src = (const uint4*)in;
+        uint4* dst = (uint4*)out;
+#define MASE_MXFP_PK(LPB_)                                                                                          \
+  do {                                                                                                              \
+    if (p.m.E >= 4)                                                                                                 \
+      hipLaunchKernelGGL((mxfp_qdq_pk16_kernel<DTI, LPB_, false>), grid, block, 0, st, src, dst, n_vec, p, q);      \
+    else                                                                                                            \
+      hipLaunchKernelGGL((mxfp_qdq_pk16_kernel<DTI, LPB_, true>), grid, block, 0, st, src, dst, n_vec, p, q);       \
+  } while (0)
+        switch (lpb) {
+          case 1: MASE_MXFP_PK(1); break;
+          case 2: MASE_MXFP_PK(2); break;
+          case 4: MASE_MXFP_PK(4); break;
+          default: MASE_MXFP_PK(8); break;
+        }
+#undef MASE_MXFP_PK
+        return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+      }
+    }
 #define MASE_MXFP_CASE(LPB_, SUB_)                                                                               \
   do {                                                                                                           \
     if (codes != nullptr)                                                                                        \

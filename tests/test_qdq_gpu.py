@@ -281,6 +281,30 @@ def test_mxfp(Q, dev, dtype, fmt):
                           f"mxfp dim={dim}")
 
 
+@pytest.mark.parametrize("fmt", [(4, 3), (5, 2), (2, 3), (3, 2), (2, 1), (1, 2)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=_ID.get)
+def test_mxfp_every_16bit_value_as_an_element(Q, dev, dtype, fmt):
+    """every finite 16-bit pattern as an element of blocks whose maximum sits 0 .. 100 binades above it (the packed
+    16-bit kernel: ordinary codes, the format's subnormal binade, underflow, quotients that leave the fp32 range)"""
+    e, f = fmt
+    x = all_16bit(dtype)
+    x = x[torch.isfinite(x)]
+    x = x[: (x.numel() // 31) * 31].view(-1, 31)
+    top = float(torch.finfo(dtype).max)
+    for lift in (0, 1, 2, 3, 6, 9, 16, 40, 100):
+        mx = (x.double().abs().max(dim=1, keepdim=True).values * 2.0 ** lift).clamp(max=top / 2).to(dtype)
+        blocks = torch.cat([x, mx], dim=1).contiguous()
+        assert_bits_equal(Q.mxfp_quantizer(blocks.to(dev), 32, e, f), O.mxfp_quantizer(blocks, 32, e, f),
+                          f"mxfp {dtype} e{e}m{f} lift {lift}")
+    g = torch.Generator().manual_seed(e * 8 + f)
+    shuffled = all_16bit(dtype)
+    shuffled = shuffled[torch.isfinite(shuffled)]
+    shuffled = shuffled[torch.randperm(shuffled.numel(), generator=g)][: (shuffled.numel() // 64) * 64].view(-1, 64)
+    for B in (8, 16, 32, 64):
+        assert_bits_equal(Q.mxfp_quantizer(shuffled.to(dev), B, e, f), O.mxfp_quantizer(shuffled, B, e, f),
+                          f"mxfp {dtype} e{e}m{f} shuffled B={B}")
+
+
 def test_mxfp_top_of_range_and_subnormals(Q, dev):
     """Scaled values in [448, 512) (the all-finite e4m3 top codes and the lost-carry binade) and fp32 subnormals."""
     top = torch.tensor([464, 479.9, 480, 495.9, 496, 511.9, 448, 300, 1.9375 * 128, 1.97 * 64, 1.97 * 32], dtype=torch.float32)
