@@ -421,6 +421,8 @@ class _ElementwiseQdq(Workload):
         self.host = torch.randn(*self.shape, generator=g).to(self.torch_dtype)
         self.bufs = [self.host.to(dev).roll(i, dims=1).contiguous() for i in range(n_buffers)]
         self.dtype = {torch.bfloat16: "bf16", torch.float32: "f32", torch.float16: "f16"}[self.torch_dtype]
+        if self.torch_dtype != torch.float32 and getattr(self, "kernel16", None):
+            self.kernel = self.kernel16
         self.config = {"workload": f"{self.fn_name}{self.args} on {self.dtype} {list(self.shape)}, N(0,1) seed 5"}
         self.metric = (f"{self.fn_name} throughput (algorithmic bytes: {self.host.element_size()} B read + "
                        f"{self.host.element_size()} B written per element)")
@@ -469,12 +471,14 @@ class MinifloatIeeeQdq(_ElementwiseQdq):
 
 class MxfpQdq(_ElementwiseQdq):
     name, unit, kernel = "mxfp_qdq", "GB/s", "mxfp_qdq_vec_kernel"
+    kernel16 = "mxfp_qdq_pk16_kernel"
     fn_name, args = "mxfp_quantizer", (32, 4, 3)
     oracle_name, oracle_args = "mxfp_quantizer", (32, 4, 3)
 
 
 class MinifloatMxQdq(_ElementwiseQdq):
     name, unit, kernel = "minifloat_mx_qdq", "GB/s", "elementwise_kernel<MinifloatMxOp>"
+    kernel16 = "minifloat_mx_pk16_kernel"
     oracle_name, oracle_args = "minifloat_quantizer_sim", (4, 3, True, "rn")
 
     def setup(self, torch, dev, n_buffers):

@@ -156,8 +156,7 @@ __global__ __launch_bounds__(kVecThreads) void mxfp_qdq_pk16_kernel(const uint4*
     float x[8], z[8];
     uint32_t c[8];
     TR::unpack(raw, x);
-    if (p.m.E >= 4) mxfp_elements<false, 8>(x, state, sh, p, c, z);
-    else mxfp_elements<true, 8>(x, state, sh, p, c, z);
+    mxfp_elements<true, 8>(x, state, sh, p, c, z);  // the form that handles codes with exponent field 0 in line
     o = TR::pack(z);
   }
   if (live) store_nt(out + idx, o);
