@@ -314,7 +314,8 @@ class MxfpLinear(Workload):
 class DecoderLayerMxint(Workload):
     name = "decoder_layer"
     metric = ("Llama-style decoder layer forward with MXINT8 Linears (flop per step = 7 Linears + causal attention; "
-              "RMSNorm, rotary embedding, attention and SwiGLU glue run as torch ops inside the step)")
+              "RMSNorm and the SwiGLU product run as one-pass kernels, rotary embedding and attention as torch ops, "
+              "all inside the step)")
     unit = "TFLOP/s"
     dtype = "bf16"
     bound = "mfma"

@@ -17,6 +17,8 @@
  *   mase_minifloat_qdq      nn/quantizers/minifloat.py:90-117, :200-225 (minifloat_denorm/ieee_quantizer)
  *   mase_minifloat_mx_qdq   nn/quantizers/_minifloat_mx/minifloat.py:12-33 (minifloat_quantizer_sim)
  *   mase_mxfp_qdq           nn/quantizers/mxfp/mxfp.py:187-230    (mxfp_quantizer, non-search branch)
+ *   mase_rmsnorm_minifloat  nn/quantized/modules/llama/rms_norm.py:72-84 (LlamaRMSNormMinifloat.forward)
+ *   mase_silu_mul_minifloat nn/quantized/modules/llama/mlp.py:60-62 (silu_minifloat(gate) * up)
  *   mase_attn_softmax_mx    nn/quantized/modules/llama/attention.py:363-392 (scores -> quantized probabilities)
  *   mase_mx_unpack          nn/quantizers/mxint/fake.py:59-80, nn/quantizers/mxfp/fake.py:75-104 (compose_*)
  *   mase_mxfp_pack, mase_gemm_mxfp_scaled   nn/quantized/modules/linear.py:877-895 (LinearMXFP.forward on
@@ -166,6 +168,21 @@ int mase_attn_softmax_mx(const void* scores, const void* mask, void* out, size_t
                          size_t kv_len, size_t mask_row_stride, int dtype, float scaling, int cast_exp_bits,
                          int cast_frac_bits, int cast_is_finite, int cast_round_mode, int mx_kind, int mx_p0, int mx_p1,
                          const uint32_t* log2_tab_dtype, const uint32_t* log2_tab_f32, void* stream);
+
+/* RMSNorm over the last dimension of x [rows, cols] with optional bit-level minifloat casts (exp_bits 0 = off) of the
+ * input and of the weight [cols], all in dtype:  h = cast(x);  h = float(h) * rsqrt(mean(h^2) + eps);
+ * out = cast(weight) * dtype(h).  cols % 8 == 0, cols <= 8192.  LlamaRMSNormMinifloat.forward
+ * (nn/quantized/modules/llama/rms_norm.py:72-84); with both casts off the plain Llama RMSNorm
+ * (models/llama/modeling_llama.py:79-93). */
+int mase_rmsnorm_minifloat(const void* x, const void* weight, void* out, size_t rows, size_t cols, int dtype, float eps,
+                           int x_exp_bits, int x_frac_bits, int x_is_finite, int x_round_mode, int w_exp_bits,
+                           int w_frac_bits, int w_is_finite, int w_round_mode, void* stream);
+
+/* out = silu(cast(gate)) * up, element-wise over numel elements of dtype (numel % 8 == 0), the cast optional
+ * (exp_bits 0 = off): LlamaMLPMXInt / LlamaMLPMXFP.forward's silu_minifloat(gate_proj(x)) * up_proj(x)
+ * (nn/quantized/modules/llama/mlp.py:60-62, nn/quantized/functional/silu.py:41-57). */
+int mase_silu_mul_minifloat(const void* gate, const void* up, void* out, size_t numel, int dtype, int exp_bits,
+                            int frac_bits, int is_finite, int round_mode, void* stream);
 
 /* Plain streaming copy of `bytes` (multiple of 16, 16-byte aligned pointers).  No counterpart in the reference:
  * it is the calibration kernel for the achievable-bandwidth ceiling and for scaling hardware byte counters. */

@@ -7,6 +7,8 @@ fp32 accumulation, so the real-number dot products are those of the reference; o
 """
 from __future__ import annotations
 
+import weakref
+
 import torch
 from torch import Tensor
 from torch.nn import functional as F
@@ -48,16 +50,49 @@ class WeightCache:
         return self._w
 
 
+class _SharedActivation:
+    """The quantized form of the activation tensor most recently fed to an MX Linear, so that sibling projections of
+    the same tensor (q/k/v, gate/up) quantize it once.  A hit requires the very same tensor object, unmodified (same
+    version counter) and the same quantizer; the entry holds the tensor only weakly and is dropped when it dies."""
+
+    def __init__(self):
+        self._ref = None
+        self._key = None
+        self._xq = None
+
+    def _drop(self, _ref=None):
+        self._ref = self._key = self._xq = None
+
+    def get(self, x: Tensor, quantizer_key, make):
+        key = (x._version, tuple(x.shape), x.dtype, quantizer_key)
+        if self._ref is not None and self._ref() is x and self._key == key:
+            return self._xq
+        xq = make()
+        try:
+            self._ref, self._key, self._xq = weakref.ref(x, self._drop), key, xq
+        except TypeError:
+            self._drop()
+        return xq
+
+
+_shared_activation = _SharedActivation()
+
+
 def mx_linear(x: Tensor, weight: Tensor, bias: Tensor | None, quantize_to_bf16, quantize_same_dtype,
-              cache: WeightCache) -> Tensor:
+              cache: WeightCache, quantizer_key=None) -> Tensor:
     """``F.linear(q(x), weight, bias)``.  ``quantize_to_bf16(x2d)`` returns q(x) as bf16 (exact);
-    ``quantize_same_dtype(x)`` returns q(x) in x's dtype (used when the weight has no exact bf16 image)."""
+    ``quantize_same_dtype(x)`` returns q(x) in x's dtype (used when the weight has no exact bf16 image).
+    ``quantizer_key`` identifies the activation quantizer (format and block size): with it, projections that are fed
+    the same tensor object share one quantized copy."""
     wb = cache.get(weight) if x.is_cuda and weight.dim() == 2 else None
     if wb is None or x.dtype not in (torch.float32, torch.bfloat16, torch.float16):
         return F.linear(quantize_same_dtype(x), weight, bias)
     lead = x.shape[:-1]
-    x2 = x.reshape(-1, x.shape[-1])
-    xq = quantize_to_bf16(x2)
+    # not while a HIP graph is being captured: a hit would leave the quantizer out of the graph
+    if quantizer_key is not None and not torch.is_grad_enabled() and not torch.cuda.is_current_stream_capturing():
+        xq = _shared_activation.get(x, quantizer_key, lambda: quantize_to_bf16(x.reshape(-1, x.shape[-1])))
+    else:
+        xq = quantize_to_bf16(x.reshape(-1, x.shape[-1]))
     y = gemm_bf16_tn(xq, wb, bias, x.dtype)
     return y.reshape(*lead, weight.shape[0])
 

@@ -136,7 +136,7 @@ class LinearMXInt(_LinearMX):
             x, self.weight, self.bias,
             lambda t: _ops.mxint_qdq(t, bs, bits, -1, 8, out_dtype=torch.bfloat16),
             lambda t: mxint_quantizer(t, block_size=bs, element_bits=bits, block_dim=-1),
-            self._w_cache,
+            self._w_cache, ("mxint", bs, bits),
         )
 
 
@@ -218,5 +218,5 @@ class LinearMXFP(_LinearMX):
             x, self.weight, self.bias,
             lambda t: _ops.mxfp_qdq(t, bs, eb, fb, -1, 8, out_dtype=torch.bfloat16),
             lambda t: mxfp_quantizer(t, block_size=bs, element_exp_bits=eb, element_frac_bits=fb, block_dim=-1),
-            self._w_cache,
+            self._w_cache, ("mxfp", bs, eb, fb),
         )

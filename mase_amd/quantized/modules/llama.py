@@ -27,6 +27,7 @@ import torch
 from torch import Tensor, nn
 
 from ...quantizers import mxfp_quantizer, mxint_quantizer
+from ...quantizers import _ops
 from ...quantizers._ops import attn_softmax_mx, attn_softmax_mx_supported, minifloat_mx_qdq
 from ..functional.activations import kv_cache_mxfp, kv_cache_mxint, rope_minifloat, rotate_half, silu_minifloat, softmax_minifloat
 
@@ -216,10 +217,15 @@ class _LlamaMLPMX(nn.Module):
         self.bypass = self.q_config.get("bypass", False)
 
     def forward(self, x: Tensor) -> Tensor:
+        gate, up = self.gate_proj(x), self.up_proj(x)
+        if _ops.silu_mul_supported(gate, up):  # one pass: cast, SiLU and product
+            cast = None if self.bypass else (self.q_config["data_in_exponent_width"], self.q_config["data_in_frac_width"],
+                                             self.q_config.get("data_in_is_finite", True),
+                                             self.q_config.get("data_in_round_mode", "rn"))
+            return self.down_proj(_ops.silu_mul_minifloat(gate, up, cast))
         if self.bypass:
-            return self.down_proj(self.act_fn(self.gate_proj(x)) * self.up_proj(x))
-        x = silu_minifloat(self.gate_proj(x), self.q_config) * self.up_proj(x)
-        return self.down_proj(x)
+            return self.down_proj(self.act_fn(gate) * up)
+        return self.down_proj(silu_minifloat(gate, self.q_config) * up)
 
 
 class LlamaMLPMXFP(_LlamaMLPMX):
@@ -252,7 +258,17 @@ class LlamaRMSNormMinifloat(nn.Module):
         self.w_quantizer = cast("weight") if not self.bypass and not self.weight_bypass else None
         self.x_quantizer = cast("data_in") if not self.bypass and not self.data_in_bypass else None
 
+    def _cast_spec(self, prefix, quantizer):
+        if quantizer is None:
+            return None
+        return (self.q_config[f"{prefix}_exponent_width"], self.q_config[f"{prefix}_frac_width"],
+                self.q_config.get(f"{prefix}_is_finite", True), self.q_config.get(f"{prefix}_round_mode", "rn"))
+
     def forward(self, hidden_states):
+        if _ops.rmsnorm_supported(hidden_states, self.weight):  # one pass over the activations
+            return _ops.rmsnorm_minifloat(hidden_states, self.weight, self.variance_epsilon,
+                                          self._cast_spec("data_in", self.x_quantizer),
+                                          self._cast_spec("weight", self.w_quantizer))
         input_dtype = hidden_states.dtype
         if self.x_quantizer is not None:
             hidden_states = self.x_quantizer(hidden_states)

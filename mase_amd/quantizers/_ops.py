@@ -112,6 +112,58 @@ def mxfp_qdq(x: Tensor, block_size: int, exp_bits: int, frac_bits: int, block_di
     return (res, codes, scales) if pack else res
 
 
+def _cast_args(cast):
+    """(exp_bits, frac_bits, is_finite, round_mode code) of an optional minifloat cast; exp_bits 0 switches it off"""
+    if cast is None:
+        return 0, 0, 1, 0
+    return int(cast[0]), int(cast[1]), int(bool(cast[2])), _ROUND_MODES[cast[3]]
+
+
+RMSNORM_MAX_COLS = 8192
+
+
+def rmsnorm_supported(x: Tensor, weight: Tensor) -> bool:
+    return (x.is_cuda and x.dtype in _lib.DTYPE_CODE and weight.dtype == x.dtype and weight.device == x.device
+            and weight.dim() == 1 and x.dim() >= 1 and x.shape[-1] == weight.shape[0] and x.shape[-1] % 8 == 0
+            and x.shape[-1] <= RMSNORM_MAX_COLS and x.numel() > 0
+            and not (torch.is_grad_enabled() and (x.requires_grad or weight.requires_grad)))
+
+
+def rmsnorm_minifloat(x: Tensor, weight: Tensor, eps: float, x_cast=None, w_cast=None) -> Tensor:
+    """``cast(weight) * (cast(x).float() * rsqrt(mean(square) + eps)).to(dtype)`` over the last dimension in one pass
+    (``mase_rmsnorm_minifloat``); a cast is (exp_bits, frac_bits, is_finite, round_mode) or None."""
+    _lib.require_device(x, "rmsnorm_minifloat")
+    lib = _lib.load()
+    assert rmsnorm_supported(x, weight)
+    xc = _contig(x)
+    w = weight.detach().contiguous()
+    out = torch.empty_like(xc)
+    cols = xc.shape[-1]
+    rc = lib.mase_rmsnorm_minifloat(xc.data_ptr(), w.data_ptr(), out.data_ptr(), xc.numel() // cols, cols, _lib.dtype_code(xc),
+                                    float(eps), *_cast_args(x_cast), *_cast_args(w_cast), _lib.stream_ptr(xc))
+    _lib.check(rc, "mase_rmsnorm_minifloat")
+    return out
+
+
+def silu_mul_supported(gate: Tensor, up: Tensor) -> bool:
+    return (gate.is_cuda and gate.dtype in _lib.DTYPE_CODE and up.dtype == gate.dtype and up.shape == gate.shape
+            and up.device == gate.device and gate.numel() > 0 and gate.numel() % 8 == 0
+            and not (torch.is_grad_enabled() and (gate.requires_grad or up.requires_grad)))
+
+
+def silu_mul_minifloat(gate: Tensor, up: Tensor, cast=None) -> Tensor:
+    """``silu(cast(gate)) * up`` in one pass (``mase_silu_mul_minifloat``)"""
+    _lib.require_device(gate, "silu_mul_minifloat")
+    lib = _lib.load()
+    assert silu_mul_supported(gate, up)
+    g, u = _contig(gate), _contig(up)
+    out = torch.empty_like(g)
+    rc = lib.mase_silu_mul_minifloat(g.data_ptr(), u.data_ptr(), out.data_ptr(), g.numel(), _lib.dtype_code(g),
+                                     *_cast_args(cast), _lib.stream_ptr(g))
+    _lib.check(rc, "mase_silu_mul_minifloat")
+    return out
+
+
 ATTN_PROB_MAX_KV = 8192
 
 

@@ -5,8 +5,10 @@ residual; RMSNorm -> SwiGLU MLP -> residual).
 Semantics follow the reference's Llama block (``chop/models/llama/modeling_llama.py:79-93`` RMSNorm, ``:99-147,
 185-216`` rotary embedding with ``rotate_half``, ``:219-236`` MLP ``down(silu(gate(x)) * up(x))``, ``:362-480``
 attention, ``:843-918`` layer with pre-norm residuals); no KV cache, no dropout, no attention bias.
-Everything except the seven Linears is ordinary torch and runs identically on CPU and GPU, which is what lets the
-same class serve as the CPU reference once its Linears are swapped for reference ones.
+On the CPU everything except the seven Linears is ordinary torch, which is what lets the same class serve as the CPU
+reference once its Linears are swapped for reference ones; on the GPU (no gradient recorded) RMSNorm and the SwiGLU
+product run as one-pass kernels with the same arithmetic (``mase_rmsnorm_minifloat`` / ``mase_silu_mul_minifloat``
+with their casts off).
 """
 from __future__ import annotations
 
@@ -15,6 +17,8 @@ from dataclasses import dataclass
 import torch
 from torch import nn
 from torch.nn import functional as F
+
+from ..quantizers import _ops
 
 
 @dataclass
@@ -35,6 +39,8 @@ class RMSNorm(nn.Module):
         self.eps = eps
 
     def forward(self, x):
+        if x.is_cuda and _ops.rmsnorm_supported(x, self.weight):
+            return _ops.rmsnorm_minifloat(x, self.weight, self.eps)  # the same arithmetic in one pass
         dtype = x.dtype
         h = x.to(torch.float32)
         h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + self.eps)
@@ -98,7 +104,12 @@ class DecoderLayer(nn.Module):
         a = a.transpose(1, 2).reshape(B, T, cfg.num_heads * cfg.head_dim)
         x = x + self.o_proj(a)
         h = self.post_attention_layernorm(x)
-        x = x + self.down_proj(F.silu(self.gate_proj(h)) * self.up_proj(h))
+        gate, up = self.gate_proj(h), self.up_proj(h)
+        if gate.is_cuda and _ops.silu_mul_supported(gate, up):
+            act = _ops.silu_mul_minifloat(gate, up)  # silu(gate) * up in one pass
+        else:
+            act = F.silu(gate) * up
+        x = x + self.down_proj(act)
         return x
 
     def linear_flops(self, tokens: int) -> float:

@@ -276,3 +276,24 @@ def test_attention_probability_entry_point_rejects_bad_arguments_without_a_gpu(l
     assert call(p, None, p, 1, 4, 8, 64, 0, 1, 0.125, 4, 3, 1, 0, 2, 3, 3, None, p, None) == -5      # MXFP format
     assert call(p, None, p, 1, 4, 8, 64, 0, 1, 0.125, 4, 3, 1, 0, 1, 8, 0, None, None, None) == -1   # table missing
     assert call(p, None, p, 1, 4, 8, 64, 0, 1, 0.125, 4, 3, 1, 0, 3, 8, 0, p, p, None) == -5         # unknown kind
+
+
+def test_layer_op_entry_points_reject_bad_arguments_without_a_gpu(lib):
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    # mase_rmsnorm_minifloat(x, weight, out, rows, cols, dtype, eps, x cast E F fin rm, w cast E F fin rm, stream)
+    r = lib.mase_rmsnorm_minifloat
+    assert r(p, p, p, 0, 64, 1, 1e-6, 0, 0, 1, 0, 0, 0, 1, 0, None) == 0
+    assert r(p, None, p, 4, 64, 1, 1e-6, 0, 0, 1, 0, 0, 0, 1, 0, None) == -1
+    assert r(p, p, p, 4, 60, 1, 1e-6, 0, 0, 1, 0, 0, 0, 1, 0, None) == -2      # whole 16-byte vectors
+    assert r(p, p, p, 4, 16384, 1, 1e-6, 0, 0, 1, 0, 0, 0, 1, 0, None) == -2   # row too long for the registers
+    assert r(p, p, p, 4, 64, 4, 1e-6, 0, 0, 1, 0, 0, 0, 1, 0, None) == -4
+    assert r(p, p, p, 4, 64, 1, 1e-6, 9, 3, 1, 0, 0, 0, 1, 0, None) == -5      # cast format
+    assert r(p, p, p, 4, 64, 1, 1e-6, 4, 3, 1, 0, 4, 3, 1, 7, None) == -5      # rounding mode
+    # mase_silu_mul_minifloat(gate, up, out, numel, dtype, E, F, fin, rm, stream)
+    s = lib.mase_silu_mul_minifloat
+    assert s(p, p, p, 0, 1, 0, 0, 1, 0, None) == 0
+    assert s(p, p, None, 64, 1, 0, 0, 1, 0, None) == -1
+    assert s(p, p, p, 63, 1, 0, 0, 1, 0, None) == -2
+    assert s(p, p, p, 64, 3, 0, 0, 1, 0, None) == -4
+    assert s(p, p, p, 64, 1, 4, 12, 1, 0, None) == -5

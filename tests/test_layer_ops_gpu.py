@@ -1,0 +1,92 @@
+"""One-pass RMSNorm and SiLU-product kernels against the separate tensor operations (torch on the GPU for the plain
+forms, the CPU oracle for the minifloat-cast forms), and the sharing of quantized activations between projections."""
+import pytest
+import torch
+
+import oracle as O
+from oracle import llama as OL
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+ULP = {torch.float32: 2.0 ** -23, torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10}
+
+
+def close_in_ulps(got, want, dtype, n_ulp, frac_equal):
+    got, want = got.float().cpu(), want.float().cpu()
+    err = (got - want).abs() / want.abs().clamp_min(1e-30)
+    assert float(err.max()) <= n_ulp * ULP[dtype], float(err.max())
+    assert float((got == want).float().mean()) >= frac_equal, float((got == want).float().mean())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cols", [8, 256, 4096, 5120, 8192])
+def test_rmsnorm_one_pass(dev, dtype, cols):
+    from mase_amd.quantizers import _ops
+
+    g = torch.Generator().manual_seed(cols)
+    x = (torch.randn(37, cols, generator=g) * 1.7).to(dtype)
+    w = (1.0 + 0.2 * torch.randn(cols, generator=g)).to(dtype)
+    xd, wd = x.to(dev), w.to(dev)
+    assert _ops.rmsnorm_supported(xd, wd)
+    got = _ops.rmsnorm_minifloat(xd, wd, 1e-6)
+    h = xd.float()
+    want = wd * (h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + 1e-6)).to(dtype)
+    # the row sum is taken in another order: a result may land on the neighbouring value of dtype
+    close_in_ulps(got, want, dtype, 1.01 if dtype != torch.float32 else 8, 0.995 if dtype != torch.float32 else 0.5)
+    # with casts: against the oracle's restatement of LlamaRMSNormMinifloat.forward
+    qc = {"data_in_exponent_width": 4, "data_in_frac_width": 3, "weight_exponent_width": 5, "weight_frac_width": 2,
+          "weight_round_mode": "ru"}
+    got = _ops.rmsnorm_minifloat(xd, wd, 1e-6, (4, 3, True, "rn"), (5, 2, True, "ru"))
+    close_in_ulps(got, OL.rms_norm_forward(w, x, 1e-6, qc), dtype, 1.01 if dtype != torch.float32 else 8,
+                  0.995 if dtype != torch.float32 else 0.5)
+    assert not _ops.rmsnorm_supported(xd, wd.float() if dtype != torch.float32 else wd.bfloat16())
+    assert not _ops.rmsnorm_supported(xd[:, : cols - 4], wd[: cols - 4]) or (cols - 4) % 8 == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul_one_pass(dev, dtype):
+    from mase_amd.quantizers import _ops
+
+    g = torch.Generator().manual_seed(3)
+    gate = (torch.randn(33, 1000, generator=g) * 3).to(dtype)
+    up = torch.randn(33, 1000, generator=g).to(dtype)
+    gate[0, :8] = torch.tensor([0.0, -0.0, 30.0, -30.0, 88.0, -88.0, 1e-3, -1e-3]).to(dtype)
+    got = _ops.silu_mul_minifloat(gate.to(dev), up.to(dev))
+    want = torch.nn.functional.silu(gate.to(dev)) * up.to(dev)
+    close_in_ulps(got, want, dtype, 2.02 if dtype != torch.float32 else 8, 0.99 if dtype != torch.float32 else 0.5)
+    got = _ops.silu_mul_minifloat(gate.to(dev), up.to(dev), (4, 3, True, "rn"))
+    want = torch.nn.functional.silu(O.minifloat_quantizer_sim(gate, 4, 3, True, "rn")) * up
+    close_in_ulps(got, want, dtype, 2.02 if dtype != torch.float32 else 8, 0.99 if dtype != torch.float32 else 0.5)
+
+
+def test_sibling_projections_share_one_quantized_activation(dev, monkeypatch):
+    from mase_amd.quantized import LinearMXInt
+    from mase_amd.quantizers import _ops
+
+    cfg = {"weight_block_size": 32, "weight_width": 8, "data_in_block_size": 32, "data_in_width": 8}
+    torch.manual_seed(0)
+    mods = []
+    for _ in range(3):
+        m = LinearMXInt(256, 128, bias=False, device=dev, dtype=torch.bfloat16, config=dict(cfg))
+        m.load_state_dict({"weight": torch.randn(128, 256) * 0.05})
+        mods.append(m)
+    calls = []
+    real = _ops.mxint_qdq
+    monkeypatch.setattr(_ops, "mxint_qdq", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    x = torch.randn(300, 256, device=dev, dtype=torch.bfloat16)
+    ys = [m(x) for m in mods]
+    assert len(calls) == 1                               # q/k/v style: one quantization for three projections
+    ref = [m(x.clone()) for m in mods]                   # other tensor objects: quantized again each time
+    assert len(calls) == 4
+    for a, b in zip(ys, ref):
+        assert torch.equal(a, b)
+    x.mul_(0.5)                                          # modified in place: the cached copy is stale
+    y2 = mods[0](x)
+    assert len(calls) == 5 and torch.equal(y2, mods[0](x.clone()))
+    other = LinearMXInt(256, 128, bias=False, device=dev, dtype=torch.bfloat16,
+                        config={**cfg, "data_in_width": 6})
+    other.load_state_dict({"weight": torch.randn(128, 256) * 0.05})
+    n = len(calls)
+    other(x)                                             # another activation format: not shared
+    assert len(calls) == n + 1
