@@ -314,8 +314,8 @@ class MxfpLinear(Workload):
 class DecoderLayerMxint(Workload):
     name = "decoder_layer"
     metric = ("Llama-style decoder layer forward with MXINT8 Linears (flop per step = 7 Linears + causal attention; "
-              "RMSNorm and the SwiGLU product run as one-pass kernels, rotary embedding and attention as torch ops, "
-              "all inside the step)")
+              "RMSNorm, rotary embedding and the SwiGLU product run as one-pass kernels, attention as the library's "
+              "scaled_dot_product_attention, all inside the step)")
     unit = "TFLOP/s"
     dtype = "bf16"
     bound = "mfma"

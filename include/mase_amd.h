@@ -17,6 +17,7 @@
  *   mase_minifloat_qdq      nn/quantizers/minifloat.py:90-117, :200-225 (minifloat_denorm/ieee_quantizer)
  *   mase_minifloat_mx_qdq   nn/quantizers/_minifloat_mx/minifloat.py:12-33 (minifloat_quantizer_sim)
  *   mase_mxfp_qdq           nn/quantizers/mxfp/mxfp.py:187-230    (mxfp_quantizer, non-search branch)
+ *   mase_rope               nn/quantized/functional/rope.py:17-27 (_apply_rope)
  *   mase_rmsnorm_minifloat  nn/quantized/modules/llama/rms_norm.py:72-84 (LlamaRMSNormMinifloat.forward)
  *   mase_silu_mul_minifloat nn/quantized/modules/llama/mlp.py:60-62 (silu_minifloat(gate) * up)
  *   mase_attn_softmax_mx    nn/quantized/modules/llama/attention.py:363-392 (scores -> quantized probabilities)
@@ -183,6 +184,15 @@ int mase_rmsnorm_minifloat(const void* x, const void* weight, void* out, size_t 
  * (nn/quantized/modules/llama/mlp.py:60-62, nn/quantized/functional/silu.py:41-57). */
 int mase_silu_mul_minifloat(const void* gate, const void* up, void* out, size_t numel, int dtype, int exp_bits,
                             int frac_bits, int is_finite, int round_mode, void* stream);
+
+/* Rotary embedding out = x * cos + rotate_half(x) * sin for x [B, H, T, D] with the last dimension contiguous and
+ * element strides (x_stride_b, x_stride_h, x_stride_t); out has the same strides; cos / sin tables [B or 1, T, D] with
+ * strides (cs_stride_b, cs_stride_t), cs_stride_b = 0 for one table shared by the batch.  Products and sum are rounded to
+ * dtype one by one, as the tensor operations of _apply_rope round them (nn/quantized/functional/rope.py:17-27).
+ * D % 16 == 0, all strides multiples of 8. */
+int mase_rope(const void* x, const void* cos, const void* sin, void* out, size_t B, size_t H, size_t T, size_t D,
+              size_t x_stride_b, size_t x_stride_h, size_t x_stride_t, size_t cs_stride_b, size_t cs_stride_t, int dtype,
+              void* stream);
 
 /* Plain streaming copy of `bytes` (multiple of 16, 16-byte aligned pointers).  No counterpart in the reference:
  * it is the calibration kernel for the achievable-bandwidth ceiling and for scaling hardware byte counters. */

@@ -39,6 +39,8 @@ SIGNATURES = {
     "mase_attn_softmax_mx": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_size_t, c_size_t, c_int,
                                      ctypes.c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
                                      c_void_p]),
+    "mase_rope": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_size_t, c_size_t, c_size_t,
+                          c_size_t, c_size_t, c_size_t, c_int, c_void_p]),
     "mase_rmsnorm_minifloat": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_float, c_int, c_int, c_int,
                                        c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "mase_silu_mul_minifloat": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_void_p]),

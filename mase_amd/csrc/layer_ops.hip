@@ -1,6 +1,8 @@
 // Row-wise and element-wise layers around the quantized Linears of a Llama block, each in one pass (gfx950):
 //   RMSNorm with optional minifloat casts of the input and of the weight (nn/quantized/modules/llama/rms_norm.py:72-84;
 //   with both casts off: the plain RMSNorm, models/llama/modeling_llama.py:79-93)
+//   rotary embedding x * cos + rotate_half(x) * sin (nn/quantized/functional/rope.py:8-27; the minifloat cast of
+//   rope_minifloat applies to the small cos / sin tables and is done by the caller)
 //   SiLU(cast(gate)) * up (nn/quantized/modules/llama/mlp.py:60-62 with functional/silu.py:41-57; cast off: the plain
 //   SwiGLU product, models/llama/modeling_llama.py:219-236)
 // Every intermediate is rounded to the tensor dtype T where the separate tensor operations would round it.  Both are
@@ -134,6 +136,48 @@ __global__ __launch_bounds__(kRowThreads) void silu_mul_kernel(SiluMulParams p) 
   store_vec8<DT>(p.out, i * 8, y);
 }
 
+struct RopeParams {
+  const void* x;
+  const void* cos;
+  const void* sin;
+  void* out;
+  int B, H, T, D;                 // D: head_dim, a multiple of 16 (two halves of whole 16-byte vectors)
+  size_t xs_b, xs_h, xs_t;        // element strides of x and out (last dimension contiguous)
+  size_t cs_b, cs_t;              // element strides of the cos / sin tables [B or 1, T, D]
+};
+
+// out = R(R(x * cos) + R(rotate_half(x) * sin)), rotate_half(x) = cat(-x[D/2:], x[:D/2]); each lane takes 8 elements
+// of one (b, h, t) row and reads the 8 partner elements half a row away
+template <int DT>
+__global__ __launch_bounds__(256) void rope_kernel(RopeParams p) {
+  using TR = DTypeTraits<DT>;
+  const int vec_per_row = p.D / 8;
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t total = (size_t)p.B * p.H * p.T * vec_per_row;
+  if (i >= total) return;
+  const int v = (int)(i % vec_per_row);
+  size_t r = i / vec_per_row;
+  const int h = (int)(r % p.H);
+  r /= p.H;
+  const int t = (int)(r % p.T);
+  const int b = (int)(r / p.T);
+  const size_t row = (size_t)b * p.xs_b + (size_t)h * p.xs_h + (size_t)t * p.xs_t;
+  const size_t crow = (size_t)b * p.cs_b + (size_t)t * p.cs_t;
+  const int d0 = v * 8, half = p.D / 2;
+  const bool low = d0 < half;
+  float x[8], xp[8], c[8], sn[8], y[8];
+  load_vec8<DT>(p.x, row + d0, x);
+  load_vec8<DT>(p.x, row + (low ? d0 + half : d0 - half), xp);
+  load_vec8<DT>(p.cos, crow + d0, c);
+  load_vec8<DT>(p.sin, crow + d0, sn);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float rot = low ? -xp[j] : xp[j];
+    y[j] = TR::round(x[j] * c[j]) + TR::round(rot * sn[j]);
+  }
+  store_vec8<DT>(p.out, row + d0, y);
+}
+
 bool fill_cast(CastSpec& c, int exp_bits, int frac_bits, int is_finite, int round_mode) {
   c.on = exp_bits > 0;
   if (!c.on) return true;
@@ -198,6 +242,41 @@ extern "C" int mase_silu_mul_minifloat(const void* gate, const void* up, void* o
     case MASE_DT_F32: hipLaunchKernelGGL((silu_mul_kernel<MASE_DT_F32>), grid, block, 0, st, p); break;
     case MASE_DT_BF16: hipLaunchKernelGGL((silu_mul_kernel<MASE_DT_BF16>), grid, block, 0, st, p); break;
     default: hipLaunchKernelGGL((silu_mul_kernel<MASE_DT_F16>), grid, block, 0, st, p); break;
+  }
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+extern "C" int mase_rope(const void* x, const void* cos, const void* sin, void* out, size_t B, size_t H, size_t T, size_t D,
+                         size_t x_stride_b, size_t x_stride_h, size_t x_stride_t, size_t cs_stride_b, size_t cs_stride_t,
+                         int dtype, void* stream) {
+  using namespace mase;
+  if (B == 0 || H == 0 || T == 0 || D == 0) return MASE_OK;
+  if (x == nullptr || cos == nullptr || sin == nullptr || out == nullptr) return MASE_ERR_NULL;
+  if (D % 16 != 0 || D > 4096 || B * H * T > 0x7FFFFFFFull) return MASE_ERR_SHAPE;
+  if ((x_stride_b | x_stride_h | x_stride_t | cs_stride_b | cs_stride_t) % 8 != 0) return MASE_ERR_SHAPE;
+  if (!aligned16(x) || !aligned16(cos) || !aligned16(sin) || !aligned16(out)) return MASE_ERR_ALIGN;
+  if (dtype < 0 || dtype > 2) return MASE_ERR_DTYPE;
+  RopeParams p{};
+  p.x = x;
+  p.cos = cos;
+  p.sin = sin;
+  p.out = out;
+  p.B = (int)B;
+  p.H = (int)H;
+  p.T = (int)T;
+  p.D = (int)D;
+  p.xs_b = x_stride_b;
+  p.xs_h = x_stride_h;
+  p.xs_t = x_stride_t;
+  p.cs_b = cs_stride_b;
+  p.cs_t = cs_stride_t;
+  hipStream_t st = (hipStream_t)stream;
+  const size_t total = B * H * T * (D / 8);
+  const dim3 grid(blocks_for(total, (size_t)256)), block(256);
+  switch (dtype) {
+    case MASE_DT_F32: hipLaunchKernelGGL((rope_kernel<MASE_DT_F32>), grid, block, 0, st, p); break;
+    case MASE_DT_BF16: hipLaunchKernelGGL((rope_kernel<MASE_DT_BF16>), grid, block, 0, st, p); break;
+    default: hipLaunchKernelGGL((rope_kernel<MASE_DT_F16>), grid, block, 0, st, p); break;
   }
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }

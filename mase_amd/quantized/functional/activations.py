@@ -9,6 +9,7 @@ import torch
 from torch import Tensor
 
 from ...quantizers import mxfp_quantizer, mxint_quantizer
+from ...quantizers import _ops
 from ...quantizers._ops import minifloat_mx_qdq
 
 
@@ -65,6 +66,11 @@ def rotate_half(x: Tensor) -> Tensor:
 
 
 def _apply_rope(q, k, cos, sin, unsqueeze_dim=1):
+    seq = q.size(-2)
+    if unsqueeze_dim == 1 and cos.dim() == 3 and k.size(-2) == seq:  # one pass per tensor
+        c, s_ = cos[..., :seq, :], sin[..., :seq, :]
+        if _ops.rope_supported(q, c, s_) and _ops.rope_supported(k, c, s_):
+            return _ops.rope(q, c, s_), _ops.rope(k, c, s_)
     cos = cos.unsqueeze(unsqueeze_dim)
     sin = sin.unsqueeze(unsqueeze_dim)
     seq_len = q.size(-2)

@@ -164,6 +164,40 @@ def silu_mul_minifloat(gate: Tensor, up: Tensor, cast=None) -> Tensor:
     return out
 
 
+def rope_supported(x: Tensor, cos: Tensor, sin: Tensor) -> bool:
+    """x [B, H, T, D] (any strides with the last dimension contiguous), cos / sin [B or 1, T, D] or [T, D]"""
+    if not (x.is_cuda and x.dim() == 4 and x.dtype in _lib.DTYPE_CODE and x.numel() > 0 and x.stride(3) == 1):
+        return False
+    if torch.is_grad_enabled() and x.requires_grad:
+        return False
+    B, H, T, D = x.shape
+    if D % 16 != 0 or any(s % 8 for s in x.stride()[:3]) or x.data_ptr() % 16:
+        return False
+    for c in (cos, sin):
+        if c.dtype != x.dtype or c.device != x.device or c.dim() not in (2, 3) or c.shape[-1] != D or c.shape[-2] != T:
+            return False
+        if c.stride(-1) != 1 or c.stride(-2) % 8 or c.data_ptr() % 16:
+            return False
+        if c.dim() == 3 and (c.shape[0] not in (1, B) or c.stride(0) % 8):
+            return False
+    return cos.shape == sin.shape and cos.stride() == sin.stride()
+
+
+def rope(x: Tensor, cos: Tensor, sin: Tensor) -> Tensor:
+    """``x * cos + rotate_half(x) * sin`` with the tables broadcast over heads, in one pass (``mase_rope``); the result has
+    x's strides."""
+    _lib.require_device(x, "rope")
+    lib = _lib.load()
+    assert rope_supported(x, cos, sin)
+    B, H, T, D = x.shape
+    out = torch.empty_strided(x.shape, x.stride(), dtype=x.dtype, device=x.device)
+    cs_b = cos.stride(0) if cos.dim() == 3 and cos.shape[0] == B and B > 1 else 0
+    rc = lib.mase_rope(x.data_ptr(), cos.data_ptr(), sin.data_ptr(), out.data_ptr(), B, H, T, D, x.stride(0), x.stride(1),
+                       x.stride(2), cs_b, cos.stride(-2), _lib.dtype_code(x), _lib.stream_ptr(x))
+    _lib.check(rc, "mase_rope")
+    return out
+
+
 ATTN_PROB_MAX_KV = 8192
 
 

@@ -6,9 +6,9 @@ Semantics follow the reference's Llama block (``chop/models/llama/modeling_llama
 185-216`` rotary embedding with ``rotate_half``, ``:219-236`` MLP ``down(silu(gate(x)) * up(x))``, ``:362-480``
 attention, ``:843-918`` layer with pre-norm residuals); no KV cache, no dropout, no attention bias.
 On the CPU everything except the seven Linears is ordinary torch, which is what lets the same class serve as the CPU
-reference once its Linears are swapped for reference ones; on the GPU (no gradient recorded) RMSNorm and the SwiGLU
-product run as one-pass kernels with the same arithmetic (``mase_rmsnorm_minifloat`` / ``mase_silu_mul_minifloat``
-with their casts off).
+reference once its Linears are swapped for reference ones; on the GPU (no gradient recorded) RMSNorm, the rotary
+embedding and the SwiGLU product run as one-pass kernels with the same arithmetic (``mase_rmsnorm_minifloat``,
+``mase_rope``, ``mase_silu_mul_minifloat`` with their casts off).
 """
 from __future__ import annotations
 
@@ -98,8 +98,11 @@ class DecoderLayer(nn.Module):
         k = self.k_proj(h).view(B, T, cfg.num_heads, cfg.head_dim).transpose(1, 2)
         v = self.v_proj(h).view(B, T, cfg.num_heads, cfg.head_dim).transpose(1, 2)
         cos, sin = rope_tables(T, cfg.head_dim, cfg.rope_theta, x.device, x.dtype)
-        q = q * cos + rotate_half(q) * sin
-        k = k * cos + rotate_half(k) * sin
+        if q.is_cuda and _ops.rope_supported(q, cos, sin) and _ops.rope_supported(k, cos, sin):
+            q, k = _ops.rope(q, cos, sin), _ops.rope(k, cos, sin)  # the same products and sum in one pass
+        else:
+            q = q * cos + rotate_half(q) * sin
+            k = k * cos + rotate_half(k) * sin
         a = self.attention_fn(q, k, v)
         a = a.transpose(1, 2).reshape(B, T, cfg.num_heads * cfg.head_dim)
         x = x + self.o_proj(a)

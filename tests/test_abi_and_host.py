@@ -290,6 +290,13 @@ def test_layer_op_entry_points_reject_bad_arguments_without_a_gpu(lib):
     assert r(p, p, p, 4, 64, 4, 1e-6, 0, 0, 1, 0, 0, 0, 1, 0, None) == -4
     assert r(p, p, p, 4, 64, 1, 1e-6, 9, 3, 1, 0, 0, 0, 1, 0, None) == -5      # cast format
     assert r(p, p, p, 4, 64, 1, 1e-6, 4, 3, 1, 0, 4, 3, 1, 7, None) == -5      # rounding mode
+    # mase_rope(x, cos, sin, out, B, H, T, D, xs_b, xs_h, xs_t, cs_b, cs_t, dtype, stream)
+    ro = lib.mase_rope
+    assert ro(p, p, p, p, 0, 2, 4, 64, 512, 64, 128, 0, 64, 1, None) == 0
+    assert ro(p, p, None, p, 1, 2, 4, 64, 512, 64, 128, 0, 64, 1, None) == -1
+    assert ro(p, p, p, p, 1, 2, 4, 40, 512, 64, 128, 0, 64, 1, None) == -2      # head_dim in whole 16-element halves
+    assert ro(p, p, p, p, 1, 2, 4, 64, 512, 60, 128, 0, 64, 1, None) == -2      # strides in whole vectors
+    assert ro(p, p, p, p, 1, 2, 4, 64, 512, 64, 128, 0, 64, 6, None) == -4
     # mase_silu_mul_minifloat(gate, up, out, numel, dtype, E, F, fin, rm, stream)
     s = lib.mase_silu_mul_minifloat
     assert s(p, p, p, 0, 1, 0, 0, 1, 0, None) == 0

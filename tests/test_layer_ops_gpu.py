@@ -60,6 +60,35 @@ def test_silu_mul_one_pass(dev, dtype):
     close_in_ulps(got, want, dtype, 2.02 if dtype != torch.float32 else 8, 0.99 if dtype != torch.float32 else 0.5)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rope_one_pass_is_bit_identical_to_the_tensor_operations(dev, dtype):
+    """products and sum are single roundings of exact fp32 values on both sides: identical bits"""
+    from mase_amd.quantizers import _ops
+    from mase_amd.quantized.functional.activations import rope_minifloat, rotate_half
+
+    g = torch.Generator().manual_seed(9)
+    B, T, H, D = 2, 50, 6, 64
+    proj = torch.randn(B, T, H * D, generator=g).to(dtype).to(dev)
+    q = proj.view(B, T, H, D).transpose(1, 2)                       # the strided view a projection output gives
+    ang = torch.rand(B, T, D, generator=g) * 6.28
+    cos, sin = ang.cos().to(dtype).to(dev), ang.sin().to(dtype).to(dev)
+    for c, s_ in ((cos, sin), (cos[0], sin[0]), (cos[:1], sin[:1])):
+        assert _ops.rope_supported(q, c, s_)
+        got = _ops.rope(q, c, s_)
+        cc, ss = (c, s_) if c.dim() == 2 else (c.unsqueeze(1), s_.unsqueeze(1))
+        want = q * cc + rotate_half(q) * ss
+        assert got.stride() == q.stride() and torch.equal(got, want)
+    qc = q.contiguous()
+    assert torch.equal(_ops.rope(qc, cos, sin), qc * cos.unsqueeze(1) + rotate_half(qc) * sin.unsqueeze(1))
+    # the quantized caller: cos / sin through the minifloat cast, then the same kernel
+    cfg = {"data_in_exponent_width": 4, "data_in_frac_width": 3}
+    qq, kk = rope_minifloat(q, q * 0.5, cos, sin, cfg)
+    cq = O.minifloat_quantizer_sim(cos.cpu(), 4, 3, True, "rn").to(dev).unsqueeze(1)
+    sq = O.minifloat_quantizer_sim(sin.cpu(), 4, 3, True, "rn").to(dev).unsqueeze(1)
+    assert torch.equal(qq, q * cq + rotate_half(q) * sq) and torch.equal(kk, (q * 0.5) * cq + rotate_half(q * 0.5) * sq)
+    assert not _ops.rope_supported(q[..., :40], cos[..., :40], sin[..., :40])   # head_dim not a multiple of 16
+
+
 def test_sibling_projections_share_one_quantized_activation(dev, monkeypatch):
     from mase_amd.quantized import LinearMXInt
     from mase_amd.quantizers import _ops
