@@ -13,7 +13,8 @@ Workloads (the headline configurations):
 Secondary workloads (other rows of the path, same JSON; --dtype bf16|f32|f16 where it applies):
     integer_qdq, minifloat_denorm_qdq, minifloat_ieee_qdq, minifloat_mx_qdq, mxfp_qdq   on [8,2048,4096]
     attn_prob    score -> probability chain of the MX-quantized attention on [4,32,2048,2048]
-    decode_linear  LinearMXInt 8192 -> 28672 for 16 tokens (weight-streaming kernel)
+    decode_linear  LinearMXInt 8192 -> 28672 for 16 tokens (weight-streaming kernel); decode_linear_packed: the same
+                   with the weight streamed as int8 codes + scale bytes
     copy         calibration copy
 Prints ONE JSON line.  `value` is algorithmic GB/s (Q-DQ) or TFLOP/s (Linear) over the whole timed region;
 `roofline` is for the dominant kernel, timed with HIP events on the launch stream; `cpu_baseline` is the CPU
@@ -554,11 +555,13 @@ class DecodeLinear(Workload):
     M, N, K = 16, 28672, 8192
     metric = "MXINT8 Linear forward for 16 tokens (algorithmic bytes: the bf16 weight image, 2 B per weight, read once)"
     config = {"workload": "LinearMXInt 8192 -> 28672, 16 tokens, bf16, weights N(0,0.02) seed 7"}
+    extra_cfg = {}
+    weight_bytes = 2.0
 
     def setup(self, torch, dev, n_buffers):
         from mase_amd.quantized import LinearMXInt
 
-        cfg = {"weight_block_size": 32, "weight_width": 8, "data_in_block_size": 32, "data_in_width": 8}
+        cfg = {"weight_block_size": 32, "weight_width": 8, "data_in_block_size": 32, "data_in_width": 8, **self.extra_cfg}
         g = torch.Generator().manual_seed(7)
         self.mods = []
         for i in range(2):  # two layers, alternated: the 470 MB weight cannot stay in the last-level cache
@@ -571,7 +574,7 @@ class DecodeLinear(Workload):
         self.out = self.mods[i % 2](self.x)
 
     def work_per_step(self):
-        return float(self.N * self.K * 2)
+        return float(self.N * self.K) * self.weight_bytes
 
     def cpu_baseline(self, torch, budget_s):
         from oracle import linear as OL
@@ -588,12 +591,24 @@ class DecodeLinear(Workload):
             if time.perf_counter() - t0 > budget_s or n >= 20:
                 break
         dt = (time.perf_counter() - t0) / n
-        return {"value": n_rows * self.K * 2 / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+        return {"value": n_rows * self.K * self.weight_bytes / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
                 "sample": f"{n} forwards with {n_rows} of the {self.N} output rows (fp32 on the CPU), {dt*1e3:.0f} ms each"}
 
 
+class DecodeLinearPacked(DecodeLinear):
+    """the same forward with the weight streamed as MXINT8 codes + scale bytes (config packed_decode)"""
+    name = "decode_linear_packed"
+    kernel = "gemm_skinny_mxint8_partial_kernel"
+    metric = ("MXINT8 Linear forward for 16 tokens, weight streamed as int8 codes + scale bytes (algorithmic bytes: "
+              "1.03125 B per weight, read once)")
+    config = {"workload": "LinearMXInt 8192 -> 28672 with packed_decode, 16 tokens, bf16, weights N(0,0.02) seed 7"}
+    extra_cfg = {"packed_decode": True}
+    weight_bytes = 1.03125
+
+
 WORKLOADS = {w.name: w for w in (BfpQdq, MxintQdq, MxintLinear, MxfpLinear, DecoderLayerMxint, CopyBytes, IntegerQdq,
-                                 MinifloatDenormQdq, MinifloatIeeeQdq, MinifloatMxQdq, MxfpQdq, AttnProb, DecodeLinear)}
+                                 MinifloatDenormQdq, MinifloatIeeeQdq, MinifloatMxQdq, MxfpQdq, AttnProb, DecodeLinear,
+                                 DecodeLinearPacked)}
 
 
 def load_traffic(name):

@@ -24,6 +24,7 @@
  *   mase_mx_unpack          nn/quantizers/mxint/fake.py:59-80, nn/quantizers/mxfp/fake.py:75-104 (compose_*)
  *   mase_mxfp_pack, mase_gemm_mxfp_scaled   nn/quantized/modules/linear.py:877-895 (LinearMXFP.forward on
  *                           formats the block-scaled matrix instruction supports)
+ *   mase_gemm_mxint8_skinny nn/quantized/modules/linear.py:972 for at most 128 rows, weights as int8 codes + scales
  *   mase_gemm_bf16_skinny   same call sites as mase_gemm_bf16_tn, for at most 128 rows of activations
  *   mase_gemm_bf16_tn       nn/quantized/modules/linear.py:972 and :895 (the F.linear of LinearMXInt.forward /
  *                           LinearMXFP.forward on the quantize-dequantized operands)
@@ -135,6 +136,16 @@ int mase_gemm_bf16_tn(const void* A, const void* B, const void* bias, void* C, s
 size_t mase_gemm_bf16_skinny_workspace_bytes(size_t M, size_t N, size_t K);
 int mase_gemm_bf16_skinny(const void* A, const void* B, const void* bias, void* C, size_t M, size_t N, size_t K,
                           int out_dtype, int bias_dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* The few-rows product with B held as packed MXINT8: int8 codes [N, K] and one scale byte per 32 codes [N, K/32]
+ * (value = code * 2^(scale - 134): the packed outputs of mase_mxint_qdq with element_bits 8, block 32), so the weight
+ * stream is half the bytes of the bf16 image.  Codes are widened to the same bf16 values in registers; A is bf16.
+ * M <= 128, K % 128 == 0, N*K < 2^32; workspace as for mase_gemm_bf16_skinny.  Replaces the F.linear of
+ * LinearMXInt.forward (nn/quantized/modules/linear.py:972) for decode-sized batches. */
+size_t mase_gemm_mxint8_skinny_workspace_bytes(size_t M, size_t N, size_t K);
+int mase_gemm_mxint8_skinny(const void* A, const int8_t* B_codes, const uint8_t* B_scales, const void* bias, void* C,
+                            size_t M, size_t N, size_t K, int out_dtype, int bias_dtype, void* workspace,
+                            size_t workspace_bytes, void* stream);
 
 /* MXFP packing for the block-scaled matrix instruction.  in: numel elements (numel % 32 == 0, blocks of 32
  * consecutive elements); element format (exp_bits, frac_bits) in {(4,3), (5,2), (2,1)}.  codes: one byte per

@@ -53,6 +53,37 @@ def gemm_bf16_tn(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dty
     return out
 
 
+MXINT8_SKINNY_K_MULTIPLE = 128
+
+
+def gemm_mxint8_skinny_supported(M: int, N: int, K: int) -> bool:
+    return 0 < M <= SKINNY_MAX_ROWS and K % MXINT8_SKINNY_K_MULTIPLE == 0 and N * K < (1 << 32)
+
+
+def gemm_mxint8_skinny(a: Tensor, codes: Tensor, scales: Tensor, bias: Tensor | None, out_dtype: torch.dtype) -> Tensor:
+    """``a[M,K] @ dequant(codes, scales)[N,K].T + bias`` for at most 128 rows of bf16 activations, with the weight held
+    as MXINT8 codes (int8 [N,K]) and scale bytes (uint8 [N,K/32]): half the weight bytes of the bf16 image."""
+    _lib.require_device(a, "gemm_mxint8_skinny")
+    lib = _lib.load()
+    assert a.dtype == torch.bfloat16 and codes.dtype == torch.int8 and scales.dtype == torch.uint8
+    a, codes, scales = a.contiguous(), codes.contiguous(), scales.contiguous()
+    M, K = a.shape
+    N = codes.shape[0]
+    assert codes.shape == (N, K) and scales.shape == (N, K // 32) and gemm_mxint8_skinny_supported(M, N, K)
+    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    if bias is not None:
+        bias = bias.contiguous()
+    nbytes = lib.mase_gemm_mxint8_skinny_workspace_bytes(M, N, K)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=a.device)
+    rc = lib.mase_gemm_mxint8_skinny(
+        a.data_ptr(), codes.data_ptr(), scales.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(),
+        M, N, K, _lib.DTYPE_CODE[out_dtype], _lib.DTYPE_CODE[bias.dtype] if bias is not None else 0, ws.data_ptr(), nbytes,
+        _lib.stream_ptr(a),
+    )
+    _lib.check(rc, "mase_gemm_mxint8_skinny")
+    return out
+
+
 # element formats of the block-scaled matrix instruction: (exp_bits, frac_bits) -> format code of the C ABI
 MXFP_HW_FORMATS = {(4, 3): 0, (5, 2): 1, (2, 1): 4}
 MXFP_K_MULTIPLE = 128  # K tile of mase_gemm_mxfp_scaled

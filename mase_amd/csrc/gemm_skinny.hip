@@ -21,11 +21,11 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 constexpr int kSkinnyThreads = 256;   // 4 wavefronts = 4 slabs of 32 weight rows, same K range
 constexpr int kSkChunk = 64;          // K elements per chunk: one 128-byte line per row
 // XC = async copies that carry the rows of A (8 rows each): 1..4.  A stage holds the B slab chunk (4 KB) and XC KB
-// of A; the ring is as deep as 32 KB per wavefront allow (6 stages for up to 8 rows of A, 4 for 32).
+// of A; the ring is as deep as 40 KB per wavefront allow (8 stages for up to 8 rows of A, 5 for 32).
 template <int XC>
 struct SkGeom {
   static constexpr int kStageBytes = 4096 + XC * 1024;
-  static constexpr int kStages = (32 * 1024) / kStageBytes;
+  static constexpr int kStages = (40 * 1024) / kStageBytes;
   static constexpr int kCopies = 4 + XC;                       // async copies per chunk per wavefront
   static constexpr int kLdsBytes = 4 * kStages * kStageBytes;  // per work-group of 4 wavefronts
 };
@@ -130,6 +130,144 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_partial_kernel(Ski
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same product with B held as packed MXINT8: int8 codes [N, K] and one scale byte per 32 codes [N, K/32]
+// (value = code * 2^(scale - 134), the packed outputs of the MXINT quantizer).  The weight stream is half the bytes of
+// the bf16 image, which is what bounds this product.  A wavefront streams 128-element chunks of its 32 code rows (4 KB),
+// their 4 scale bytes per row and the matching chunk of A through its LDS ring; codes become bf16 in registers:
+// byte ^ 0x80 is the code plus 128 as an unsigned byte, v_cvt_f32_ubyte converts it, one fma subtracts the 128 and
+// applies the block's power-of-two scale, and the exact product is truncated to bf16 (at most 8 significant bits).
+// The MFMA operands are therefore the same bf16 values the bf16 path multiplies.  Scale bytes below 8 (weights under
+// 2^-119) are treated as zero.
+// ---------------------------------------------------------------------------------------------
+constexpr int kSqChunk = 128;  // K elements per chunk: one 128-byte line of codes per row
+constexpr int kSqWaves = 4;     // wavefronts (slabs of 32 weight rows) per work-group, as in the bf16 kernel
+constexpr int kSqThreads = kSqWaves * 64;
+template <int XC>
+struct SqGeom {
+  static constexpr int kCodeBytes = 32 * 128, kScaleBytes = 256, kABytes = XC * 8 * 256;
+  static constexpr int kStageBytes = kCodeBytes + kScaleBytes + kABytes;
+  static constexpr int kStages = ((160 / kSqWaves) * 1024) / kStageBytes;
+  static constexpr int kCopies = 4 + 1 + 2 * XC;
+  static constexpr int kLdsBytes = kSqWaves * kStages * kStageBytes;
+};
+
+struct SkinnyQParams {
+  const unsigned char* A;    // [M, K] bf16, M <= 32
+  const unsigned char* Bc;   // [N, K] int8 codes
+  const unsigned char* Bs;   // [N, K/32] scale bytes
+  float* P;
+  int M, N, K;
+  int kc;                    // K elements per split (multiple of 128)
+};
+
+__device__ __forceinline__ void sk_async_copy4(const unsigned char* base, uint32_t off, uint32_t lds_addr) {
+  const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_addr);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
+}
+
+// four codes of one dword -> two registers of two bf16 values each (code * scale, exact)
+__device__ __forceinline__ void codes4_to_bf16(uint32_t c, float scale, float bias, uint32_t& lo, uint32_t& hi) {
+  const uint32_t u = c ^ 0x80808080u;
+  const float f0 = __builtin_fmaf((float)(u & 0xFFu), scale, bias);
+  const float f1 = __builtin_fmaf((float)((u >> 8) & 0xFFu), scale, bias);
+  const float f2 = __builtin_fmaf((float)((u >> 16) & 0xFFu), scale, bias);
+  const float f3 = __builtin_fmaf((float)(u >> 24), scale, bias);
+  lo = (f2bits(f0) >> 16) | (f2bits(f1) & 0xFFFF0000u);
+  hi = (f2bits(f2) >> 16) | (f2bits(f3) & 0xFFFF0000u);
+}
+
+template <int XC>
+__global__ __launch_bounds__(kSqThreads) void gemm_skinny_mxint8_partial_kernel(SkinnyQParams p) {
+  using G = SqGeom<XC>;
+  constexpr int S = G::kStages;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  const int r = lane & 31, g = lane >> 5;
+  const int n0 = ((int)blockIdx.x * kSqWaves + wave) * 32;
+  if (n0 >= p.N) return;  // whole wavefront; there is no barrier in this kernel
+  const int ks = blockIdx.y;
+  // codes: copy j (0..3) moves rows 8j .. 8j+7 (128 bytes each): lane -> row 8j + lane/8, LDS chunk position lane%8
+  uint32_t offc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = 8 * j + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    offc[j] = (uint32_t)((size_t)min(n0 + row, p.N - 1) * (size_t)p.K) + chunk * 16;
+  }
+  // scales: lane -> the dword of row lane%32 for this chunk
+  const uint32_t offs = (uint32_t)((size_t)min(n0 + r, p.N - 1) * (size_t)(p.K / 32));
+  // A: copy j (0 .. 2*XC-1) moves rows 4j .. 4j+3 (256 bytes each): lane -> row 4j + lane/16, LDS chunk position lane%16
+  uint32_t offa[2 * XC];
+#pragma unroll
+  for (int j = 0; j < 2 * XC; ++j) {
+    const int row = 4 * j + (lane >> 4);
+    const int chunk = (lane & 15) ^ (row & 15);
+    offa[j] = (uint32_t)((size_t)min(row, p.M - 1) * (size_t)p.K * 2) + chunk * 16;
+  }
+  const unsigned char* cbase = p.Bc + (size_t)ks * p.kc;
+  const unsigned char* sbase = p.Bs + (size_t)ks * (p.kc / 32);
+  const unsigned char* abase = p.A + (size_t)ks * p.kc * 2;
+  unsigned char* ring = lds + wave * (S * G::kStageBytes);
+  const uint32_t ring_addr = (uint32_t)(uintptr_t)(lptr_t)ring;
+  const int chunks = p.kc / kSqChunk;
+  auto issue = [&](int c) __attribute__((always_inline)) {  // chunk c (clamped: past the end re-copies the last chunk)
+    const int cc = min(c, chunks - 1);
+    const uint32_t st = ring_addr + (uint32_t)((c % S) * G::kStageBytes);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sk_async_copy(cbase + (size_t)cc * 128, offc[j], st + j * 1024);
+    sk_async_copy4(sbase + (size_t)cc * 4, offs, st + G::kCodeBytes);
+#pragma unroll
+    for (int j = 0; j < 2 * XC; ++j)
+      sk_async_copy(abase + (size_t)cc * 256, offa[j], st + G::kCodeBytes + G::kScaleBytes + j * 1024);
+  };
+
+  f32x16_t acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+  for (int c = 0; c < S - 1; ++c) issue(c);
+  const int arow = min(r, 8 * XC - 1);
+  for (int c = 0; c < chunks; ++c) {
+    issue(c + S - 1);
+    sk_wait_vmcnt<(S - 1) * G::kCopies>();  // chunk c has landed; the later ones may be in flight
+    const unsigned char* st = ring + (c % S) * G::kStageBytes;
+    const uint32_t sc4 = *(const uint32_t*)(st + G::kCodeBytes + r * 4);  // the row's 4 scale bytes of this chunk
+#pragma unroll
+    for (int step = 0; step < 8; ++step) {
+      // 8 codes of row r at K offset step*16 + g*8, and the 8 values of A row r at the same K offset
+      const uint2 cw = *(const uint2*)(st + r * 128 + ((step ^ ((r >> 1) & 7)) << 4) + g * 8);
+      const uint4 xv = *(const uint4*)(st + G::kCodeBytes + G::kScaleBytes + arow * 256 + (((2 * step + g) ^ (arow & 15)) << 4));
+      const uint32_t sb = (sc4 >> (8 * (step >> 1))) & 0xFFu;
+      const float scale = bits2f(sb >= 8u ? (sb - 7u) << 23 : 0u);  // 2^(sb - 134)
+      const float bias = -128.0f * scale;
+      uint4 wv;
+      codes4_to_bf16(cw.x, scale, bias, wv.x, wv.y);
+      codes4_to_bf16(cw.y, scale, bias, wv.z, wv.w);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wv), __builtin_bit_cast(bf16x8_t, xv), acc,
+                                                    0, 0, 0);
+    }
+  }
+  sk_wait_vmcnt<0>();  // no copy may still be in flight towards LDS when the wavefront retires
+  float* out = p.P + (size_t)ks * p.M * p.N;
+  const int m = r;
+  if (m < p.M) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int n = n0 + q * 8 + g * 4;
+      float* o = out + (size_t)m * p.N + n;
+      if (n + 3 < p.N && (p.N & 3) == 0) {
+        *(float4*)o = make_float4(acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (n + j < p.N) o[j] = acc[q * 4 + j];
+      }
+    }
+  }
+}
+
 __device__ __forceinline__ float skinny_bias(const void* bias, int dt, int col) {
   if (dt == MASE_DT_F32) return ((const float*)bias)[col];
   if (dt == MASE_DT_BF16) return bits2f((uint32_t)((const uint16_t*)bias)[col] << 16);
@@ -151,20 +289,27 @@ __global__ __launch_bounds__(256) void gemm_skinny_reduce_kernel(const float* __
   else ((uint16_t*)C)[i] = (uint16_t)f32_to_f16_bits(s);
 }
 
-// K ranges: enough of them that the machine is filled (about 8 wavefronts per CU), each a whole number of
-// 64-element chunks, and all equal
+// K ranges (each a whole number of 64-element chunks, all equal).  A work-group takes the CU's whole LDS, so the
+// work-groups run in rounds of n_cu; the number of ranges is chosen for the smallest estimated time
+//   rounds * (time of one work-group, proportional to its K range)  scaled by  (1 + partial-result traffic / B's bytes)
+// where the partial results cost ranges * rows * N * 8 bytes against N * K * 2 of B; ties go to fewer ranges.
 int skinny_splits(int M, int N, int K, int n_cu) {
   const int slabs = (N + 31) / 32;
+  const int groups = (slabs + 3) / 4;
   const int chunks = K / 64;
-  int want = (8 * n_cu + slabs - 1) / slabs;
-  // the partial results cost splits * rows * N * 8 bytes of traffic: keep that below a quarter of B's bytes
   const int rows = M < 32 ? M : 32;
-  const int cap = K / (16 * rows);
-  if (want > cap) want = cap;
-  if (want < 1) want = 1;
   int best = 1;
-  for (int s = 1; s <= chunks && s <= 64; ++s)
-    if (chunks % s == 0 && s <= want) best = s;
+  double best_cost = 1e300;
+  for (int s = 1; s <= chunks && s <= 64; ++s) {
+    if (chunks % s != 0) continue;
+    const long wgs = (long)groups * s;
+    const long rounds = (wgs + n_cu - 1) / n_cu;
+    const double overhead = 4.0 * s * rows / (double)K;
+    // a short K range leaves the ring's start-up (a few chunks) exposed
+    const double per_wg = (double)(chunks / s) + 4.0;
+    const double cost = (double)rounds * per_wg * (1.0 + overhead);
+    if (cost < best_cost * 0.999) { best_cost = cost; best = s; }
+  }
   return best;
 }
 
@@ -234,6 +379,71 @@ extern "C" int mase_gemm_bf16_skinny(const void* A, const void* B, const void* b
     else if (xc == 2) hipLaunchKernelGGL(gemm_skinny_partial_kernel<2>, grid, block, SkGeom<2>::kLdsBytes, st, p);
     else if (xc == 3) hipLaunchKernelGGL(gemm_skinny_partial_kernel<3>, grid, block, SkGeom<3>::kLdsBytes, st, p);
     else hipLaunchKernelGGL(gemm_skinny_partial_kernel<4>, grid, block, SkGeom<4>::kLdsBytes, st, p);
+    const size_t mn_g = rows * N;
+    const dim3 rgrid_g((unsigned)blocks_for(mn_g, 256));
+    void* Cg = (unsigned char*)C + m0 * N * (out_dtype == MASE_DT_F32 ? 4 : 2);
+    if (out_dtype == MASE_DT_F32)
+      hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_F32>, rgrid_g, dim3(256), 0, st, p.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
+    else if (out_dtype == MASE_DT_BF16)
+      hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_BF16>, rgrid_g, dim3(256), 0, st, p.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
+    else
+      hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_F16>, rgrid_g, dim3(256), 0, st, p.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
+  }
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+extern "C" size_t mase_gemm_mxint8_skinny_workspace_bytes(size_t M, size_t N, size_t K) {
+  using namespace mase;
+  if (M == 0 || N == 0 || K == 0 || (K % 128) != 0 || M > 128) return 0;
+  const int n_cu = skinny_cu_count();
+  if (n_cu <= 0) return 0;
+  // chunks of 128: the split search works in units of 64, so hand it K / 2
+  return (size_t)skinny_splits((int)M, (int)N, (int)(K / 2), n_cu) * M * N * sizeof(float);
+}
+
+extern "C" int mase_gemm_mxint8_skinny(const void* A, const int8_t* B_codes, const uint8_t* B_scales, const void* bias,
+                                       void* C, size_t M, size_t N, size_t K, int out_dtype, int bias_dtype,
+                                       void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace mase;
+  if (M == 0 || N == 0) return MASE_OK;
+  if (A == nullptr || B_codes == nullptr || B_scales == nullptr || C == nullptr) return MASE_ERR_NULL;
+  if (K == 0 || (K % 128) != 0 || M > 128 || N > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
+  if ((unsigned long long)N * K > 0xFFFFFFFFull) return MASE_ERR_SHAPE;  // 32-bit byte offsets into the codes
+  if (!aligned16(A) || !aligned16(B_codes) || (((uintptr_t)B_scales) & 3u) != 0) return MASE_ERR_ALIGN;
+  if (out_dtype < 0 || out_dtype > 2 || (bias != nullptr && (bias_dtype < 0 || bias_dtype > 2))) return MASE_ERR_DTYPE;
+  const int n_cu = skinny_cu_count();
+  if (n_cu <= 0) return MASE_ERR_LAUNCH;
+  const int splits = skinny_splits((int)M, (int)N, (int)(K / 2), n_cu);
+  const size_t need = (size_t)splits * M * N * sizeof(float);
+  if (workspace == nullptr || workspace_bytes < need || (((uintptr_t)workspace) & 15u) != 0) return MASE_ERR_WORKSPACE;
+  hipStream_t st = (hipStream_t)stream;
+  static bool attr_set = false;
+  if (!attr_set) {
+    const void* ks[4] = {(const void*)gemm_skinny_mxint8_partial_kernel<1>, (const void*)gemm_skinny_mxint8_partial_kernel<2>,
+                         (const void*)gemm_skinny_mxint8_partial_kernel<3>, (const void*)gemm_skinny_mxint8_partial_kernel<4>};
+    const int sz[4] = {SqGeom<1>::kLdsBytes, SqGeom<2>::kLdsBytes, SqGeom<3>::kLdsBytes, SqGeom<4>::kLdsBytes};
+    for (int i = 0; i < 4; ++i)
+      if (hipFuncSetAttribute(ks[i], hipFuncAttributeMaxDynamicSharedMemorySize, sz[i]) != hipSuccess)
+        return MASE_ERR_LAUNCH;
+    attr_set = true;
+  }
+  const dim3 grid((unsigned)(((N + 31) / 32 + kSqWaves - 1) / kSqWaves), (unsigned)splits), block(kSqThreads);
+  SkinnyQParams p;
+  p.Bc = (const unsigned char*)B_codes;
+  p.Bs = (const unsigned char*)B_scales;
+  p.N = (int)N;
+  p.K = (int)K;
+  p.kc = (int)K / splits;
+  for (size_t m0 = 0; m0 < M; m0 += 32) {
+    const size_t rows = (M - m0 < 32) ? (M - m0) : 32;
+    p.A = (const unsigned char*)A + m0 * K * 2;
+    p.P = (float*)workspace + (size_t)splits * m0 * N;
+    p.M = (int)rows;
+    const int xc = (int)(rows + 7) / 8;
+    if (xc == 1) hipLaunchKernelGGL(gemm_skinny_mxint8_partial_kernel<1>, grid, block, SqGeom<1>::kLdsBytes, st, p);
+    else if (xc == 2) hipLaunchKernelGGL(gemm_skinny_mxint8_partial_kernel<2>, grid, block, SqGeom<2>::kLdsBytes, st, p);
+    else if (xc == 3) hipLaunchKernelGGL(gemm_skinny_mxint8_partial_kernel<3>, grid, block, SqGeom<3>::kLdsBytes, st, p);
+    else hipLaunchKernelGGL(gemm_skinny_mxint8_partial_kernel<4>, grid, block, SqGeom<4>::kLdsBytes, st, p);
     const size_t mn_g = rows * N;
     const dim3 rgrid_g((unsigned)blocks_for(mn_g, 256));
     void* Cg = (unsigned char*)C + m0 * N * (out_dtype == MASE_DT_F32 ? 4 : 2);

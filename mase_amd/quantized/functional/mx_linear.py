@@ -13,7 +13,8 @@ import torch
 from torch import Tensor
 from torch.nn import functional as F
 
-from ..._gemm import MXFP_HW_FORMATS, MXFP_K_MULTIPLE, gemm_bf16_tn, gemm_mxfp_scaled, mxfp_pack
+from ..._gemm import (MXFP_HW_FORMATS, MXFP_K_MULTIPLE, SKINNY_MAX_ROWS, gemm_bf16_tn, gemm_mxfp_scaled,
+                      gemm_mxint8_skinny, gemm_mxint8_skinny_supported, mxfp_pack)
 
 
 class WeightCache:
@@ -165,6 +166,56 @@ class PackedMXFPWeight:
 
     def valid_for(self, weight: Tensor) -> bool:
         return self.codes is not None and self._key == _weight_key(weight)
+
+
+class PackedMXIntWeight:
+    """MXINT8 codes (int8 [N, K]) and scale bytes (uint8 [N, K/32]) of a quantized weight, kept next to the parameter for
+    the weight-streaming product of decode-sized batches (half the bytes of the bf16 image).  Valid only while the
+    parameter is the tensor the codes were made for (identity / version test, as ``WeightCache``)."""
+
+    def __init__(self):
+        self._key = None
+        self.codes = None
+        self.scales = None
+
+    def invalidate(self):
+        self._key = None
+        self.codes = self.scales = None
+
+    @staticmethod
+    def eligible(weight: Tensor, block_size: int, element_bits: int) -> bool:
+        return (weight.is_cuda and weight.dim() == 2 and block_size == 32 and element_bits == 8
+                and weight.shape[1] % 128 == 0 and weight.shape[0] * weight.shape[1] < (1 << 32)
+                and weight.dtype in (torch.float32, torch.bfloat16, torch.float16))
+
+    def set(self, codes: Tensor, scales: Tensor, weight: Tensor):
+        n, k = weight.shape
+        self.codes, self.scales = codes.reshape(n, k).contiguous(), scales.reshape(n, k // 32).contiguous()
+        self._key = _weight_key(weight)
+
+    def decodes_to(self, weight: Tensor) -> bool:
+        from ...quantizers._ops import mx_unpack
+
+        got = mx_unpack(self.codes, self.scales, 32, weight.dtype, "mxint", 8).view(weight.shape)
+        return bool(torch.equal(got, weight))
+
+    def valid_for(self, weight: Tensor) -> bool:
+        return self.codes is not None and self._key == _weight_key(weight)
+
+
+def mxint_linear_decode(x: Tensor, packed: PackedMXIntWeight, bias: Tensor | None, quantize_to_bf16) -> Tensor:
+    """``F.linear(q(x), W, b)`` for at most 128 rows of activations with W as MXINT8 codes + scales"""
+    lead = x.shape[:-1]
+    xq = quantize_to_bf16(x.reshape(-1, x.shape[-1]))
+    y = gemm_mxint8_skinny(xq, packed.codes, packed.scales, bias, x.dtype)
+    return y.reshape(*lead, packed.codes.shape[0])
+
+
+def mxint_decode_applies(x: Tensor, packed: PackedMXIntWeight, weight: Tensor) -> bool:
+    rows = x.numel() // x.shape[-1] if x.numel() else 0
+    return (x.is_cuda and 0 < rows <= SKINNY_MAX_ROWS and x.dtype in (torch.float32, torch.bfloat16, torch.float16)
+            and packed.valid_for(weight) and gemm_mxint8_skinny_supported(rows, weight.shape[0], weight.shape[1])
+            and not torch.is_grad_enabled())
 
 
 def mxfp_linear_native(x: Tensor, packed: PackedMXFPWeight, bias: Tensor | None, act_fmt) -> Tensor:

@@ -10,7 +10,8 @@ from torch.nn import functional as F
 
 from ...quantizers import _ops, mxfp_quantizer, mxint_quantizer
 from ..functional.linear import linearBlockFP, linearInteger, linearMinifloatDenorm, linearMinifloatIEEE
-from ..functional.mx_linear import PackedMXFPWeight, WeightCache, mx_linear, mxfp_linear_native
+from ..functional.mx_linear import (PackedMXFPWeight, PackedMXIntWeight, WeightCache, mx_linear, mxfp_linear_native,
+                                    mxint_decode_applies, mxint_linear_decode)
 
 
 class _LinearBase(torch.nn.Linear):
@@ -110,12 +111,46 @@ class _LinearMX(_LinearBase):
 
 
 class LinearMXInt(_LinearMX):
+    """``config["packed_decode"]`` (default False; not a key of the reference) keeps the weight's MXINT8 codes and scale
+    bytes next to the parameter (1.03 bytes per weight more) and lets forwards of at most 128 rows stream those instead
+    of the bf16 image: the product of decode-sized batches is bound by the weight bytes, which this halves.  A packed
+    checkpoint (``mase_amd.quantized.packed``) hands the codes over without this key."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, dtype=None,
+                 config=None) -> None:
+        super().__init__(in_features, out_features, bias, device, dtype, config)
+        self._w_codes = PackedMXIntWeight()
+
+    def invalidate_weight_cache(self):
+        super().invalidate_weight_cache()
+        self._w_codes.invalidate()
+
+    def weights_loaded_quantized(self, codes=None, scales=None):
+        """``codes`` / ``scales``: the quantizer's codes and scale bytes of the weight when the caller has them (a packed
+        checkpoint); kept for the decode path if they decode to exactly the weight."""
+        super().weights_loaded_quantized()
+        self._w_codes.invalidate()
+        if codes is None or self.bypass or self.gptq:
+            return
+        if not PackedMXIntWeight.eligible(self.weight, self.config["weight_block_size"], self.config["weight_width"]):
+            return
+        self._w_codes.set(codes.to(self.weight.device), scales.to(self.weight.device), self.weight)
+        if not self._w_codes.decodes_to(self.weight.data):
+            self._w_codes.invalidate()
+
     def _quantize_params(self):
         cfg = self.config
-        self.weight.data.copy_(
-            mxint_quantizer(self.weight.data, block_size=cfg["weight_block_size"], element_bits=cfg["weight_width"],
-                            block_dim=1, quantile_search=self.clip_search)
-        )
+        self._w_codes.invalidate()
+        if (cfg.get("packed_decode", False) and not self.clip_search
+                and PackedMXIntWeight.eligible(self.weight, cfg["weight_block_size"], cfg["weight_width"])):
+            deq, codes, scales = _ops.mxint_qdq(self.weight.data, 32, 8, 1, 8, pack=True)
+            self.weight.data.copy_(deq)
+            self._w_codes.set(codes, scales, self.weight)
+        else:
+            self.weight.data.copy_(
+                mxint_quantizer(self.weight.data, block_size=cfg["weight_block_size"], element_bits=cfg["weight_width"],
+                                block_dim=1, quantile_search=self.clip_search)
+            )
         b_block_size = cfg.get("bias_block_size")
         b_element_bits = cfg.get("bias_width")
         if self.bias is not None and b_block_size is not None and b_element_bits is not None:
@@ -132,6 +167,9 @@ class LinearMXInt(_LinearMX):
         bits = self.config.get("data_in_width")
         if bs is None or bits is None:
             return F.linear(x, self.weight, self.bias)
+        if mxint_decode_applies(x, self._w_codes, self.weight):
+            return mxint_linear_decode(x, self._w_codes, self.bias,
+                                       lambda t: _ops.mxint_qdq(t, bs, bits, -1, 8, out_dtype=torch.bfloat16))
         return mx_linear(
             x, self.weight, self.bias,
             lambda t: _ops.mxint_qdq(t, bs, bits, -1, 8, out_dtype=torch.bfloat16),

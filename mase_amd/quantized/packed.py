@@ -119,7 +119,7 @@ def load_packed_state_dict(model: torch.nn.Module, packed: Dict[str, Tensor], st
     result = torch.nn.Module.load_state_dict(model, unpacked_state_dict(packed, device), strict=strict)
     for name, module in model.named_modules():
         key = f"{name}.weight" if name else "weight"
-        if isinstance(module, LinearMXFP) and key + ".mx_codes" in packed:
+        if isinstance(module, (LinearMXFP, LinearMXInt)) and key + ".mx_codes" in packed:
             module.weights_loaded_quantized(packed[key + ".mx_codes"], packed[key + ".mx_scales"])
         elif isinstance(module, (LinearMXInt, LinearMXFP)):
             module.weights_loaded_quantized()

@@ -120,3 +120,39 @@ def test_gemm_few_rows_takes_the_weight_streaming_kernel(dev, M, N, K):
     y2 = _gemm.gemm_bf16_tn(ar.to(dev), br.to(dev), None, torch.float32)
     assert torch.equal(y1, y2)
     assert rel_err(y1.cpu(), ar.double() @ br.double().t()) < 2e-6
+
+
+@pytest.mark.parametrize("M", [1, 7, 16, 32, 33, 100, 128])
+def test_gemm_few_rows_with_mxint8_coded_weights(dev, M):
+    """mase_gemm_mxint8_skinny: the weight as int8 codes + scale bytes.  The codes are widened to exactly the bf16
+    values of the dequantized weight, so the result must agree with the bf16 product to fp32 summation order, and be
+    exact when every partial sum is."""
+    from mase_amd._gemm import gemm_bf16_tn, gemm_mxint8_skinny
+    from mase_amd.quantizers import _ops
+
+    g = torch.Generator().manual_seed(M)
+    for (N, K) in [(256, 128), (4096, 4096), (1000, 1152), (11008, 4096)]:
+        w = (torch.randn(N, K, generator=g) * 0.05)
+        w[3] *= 2.0 ** -40            # a row of tiny blocks (small scale bytes)
+        w[5, :64] = 0.0               # all-zero blocks
+        deq, codes, scales = _ops.mxint_qdq(w.to(dev), 32, 8, 1, 8, pack=True, out_dtype=torch.bfloat16)
+        codes, scales = codes.view(N, K), scales.view(N, K // 32)
+        a = torch.randn(M, K, generator=g).bfloat16().to(dev)
+        bias = torch.randn(N, generator=g).to(dev)
+        want = gemm_bf16_tn(a, deq, bias, torch.float32)
+        got = gemm_mxint8_skinny(a, codes, scales, bias, torch.float32)
+        ref = a.double() @ deq.double().T + bias.double()
+        scale = float(ref.abs().max())
+        assert float((got.double() - ref).abs().max()) / scale < 2e-6, (N, K)
+        assert float((got - want).abs().max()) / scale < 2e-6, (N, K)
+        assert torch.equal(got, gemm_mxint8_skinny(a, codes, scales, bias, torch.float32))   # reproducible
+        got16 = gemm_mxint8_skinny(a, codes, scales, None, torch.bfloat16)
+        assert float((got16.double() - (ref - bias.double())).abs().max()) / scale < 1e-2
+    # exact case: small integers times powers of two, every partial sum exact in fp32
+    N, K = 512, 256
+    wi = torch.randint(-7, 8, (N, K), generator=g).float() * 0.25   # below the block maximum that saturates
+    ai = torch.randint(-4, 5, (M, K), generator=g).float()
+    deq, codes, scales = _ops.mxint_qdq(wi.to(dev), 32, 8, 1, 8, pack=True, out_dtype=torch.bfloat16)
+    assert torch.equal(deq.float().cpu(), wi)
+    got = gemm_mxint8_skinny(ai.bfloat16().to(dev), codes.view(N, K), scales.view(N, K // 32), None, torch.float32)
+    assert torch.equal(got.cpu(), ai @ wi.T)

@@ -118,3 +118,55 @@ def test_model_round_trip_through_a_packed_file(dev, dtype, tmp_path):
     again = unpacked_state_dict(packed_state_dict(net))
     for k, v in net.state_dict().items():
         assert torch.equal(again[k], v), k + " (repacked)"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_linear_mxint_streams_codes_for_decode_sized_batches(dev, dtype, tmp_path):
+    """config["packed_decode"]: forwards of at most 128 rows contract against the int8 codes + scale bytes (the same
+    bf16 operand values, another summation order); larger batches take the bf16 image as before.  A packed checkpoint
+    hands the codes over as well."""
+    from mase_amd.quantized import LinearMXInt
+    from mase_amd.quantized.packed import load_packed_state_dict, packed_state_dict
+    from oracle import linear as OL
+
+    g = torch.Generator().manual_seed(9)
+    w = (torch.randn(384, 512, generator=g) * 0.05).to(dtype)
+    b = torch.randn(384, generator=g).to(dtype)
+    plain = LinearMXInt(512, 384, device=dev, dtype=dtype, config=dict(MXINT))
+    plain.load_state_dict({"weight": w, "bias": b})
+    packed = LinearMXInt(512, 384, device=dev, dtype=dtype, config={**MXINT, "packed_decode": True})
+    packed.load_state_dict({"weight": w, "bias": b})
+    assert packed._w_codes.valid_for(packed.weight) and not plain._w_codes.valid_for(plain.weight)
+    assert torch.equal(packed.weight, plain.weight)                     # the same quantized weight either way
+    qw, qb = OL.mxint_prepare_weights(w, b, MXINT)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    for rows in (1, 5, 128, 129, 300):
+        x = torch.randn(rows, 512, generator=g).to(dtype)
+        y = packed(x.to(dev))
+        ref = OL.linear_mxint_forward(x, qw, qb, MXINT)
+        err = float((y.double().cpu() - ref.double()).abs().max() / ref.double().abs().max())
+        assert err < tol, (rows, err)
+        y0 = plain(x.to(dev))
+        assert float((y.double() - y0.double()).abs().max() / y0.double().abs().max()) < (2e-6 if dtype == torch.float32 else 8e-3)
+    x3 = torch.randn(2, 3, 512, generator=g).to(dtype)                  # leading dimensions
+    assert packed(x3.to(dev)).shape == (2, 3, 384)
+    # an edited weight invalidates the codes: the forward goes back to the parameter
+    with torch.no_grad():
+        packed.weight.mul_(0.0)
+    assert not packed._w_codes.valid_for(packed.weight)
+    assert float(packed(x3.to(dev)).sub(packed.bias).abs().max()) == 0.0
+    # codes arriving through a packed state dict
+    class Net(torch.nn.Module):
+        def __init__(self, lin):
+            super().__init__()
+            self.lin = lin
+    sd = packed_state_dict(Net(plain), float_state_dict={"lin.weight": w.to(dev), "lin.bias": b.to(dev)})
+    assert "lin.weight.mx_codes" in sd
+    fresh = Net(LinearMXInt(512, 384, device=dev, dtype=dtype, config=dict(MXINT)))
+    load_packed_state_dict(fresh, sd)
+    assert fresh.lin._w_codes.valid_for(fresh.lin.weight)
+    x = torch.randn(4, 512, generator=g).to(dtype).to(dev)
+    again = LinearMXInt(512, 384, device=dev, dtype=dtype, config={**MXINT, "packed_decode": True})
+    again.load_state_dict({"weight": w, "bias": b})
+    assert torch.equal(fresh.lin._w_codes.codes, again._w_codes.codes)   # the codes of the original weights both ways
+    assert torch.equal(fresh.lin(x), again(x))
