@@ -54,7 +54,9 @@ class WeightCache:
 class _SharedActivation:
     """The quantized form of the activation tensor most recently fed to an MX Linear, so that sibling projections of
     the same tensor (q/k/v, gate/up) quantize it once.  A hit requires the very same tensor object, unmodified (same
-    version counter) and the same quantizer; the entry holds the tensor only weakly and is dropped when it dies."""
+    version counter) and the same quantizer; the entry holds the tensor only weakly and is dropped when it dies.
+    The quantized copy itself (the size of the activation in bf16) stays allocated until the next miss.  Callers are
+    assumed to run their projections on one stream, and an in-place edit made through ``.data`` is not seen."""
 
     def __init__(self):
         self._ref = None
