@@ -128,6 +128,15 @@ int mase_mx_unpack(const uint8_t* codes, const uint8_t* scales, void* out, size_
 int mase_gemm_bf16_tn(const void* A, const void* B, const void* bias, void* C, size_t M, size_t N, size_t K,
                       int out_dtype, int bias_dtype, void* stream);
 
+/* The same product for shapes whose 256x256 output tiles alone would leave most CUs idle (a few hundred rows of A):
+ * K is cut into ranges, every (tile, range) pair is a work item of the same kernel and writes an fp32 partial tile into
+ * `workspace` (at least mase_gemm_bf16_tn_splitk_workspace_bytes(M, N, K) bytes, 16-byte aligned), and a second kernel
+ * adds the ranges in a fixed order, adds the bias and converts.  _workspace_bytes returns 0 when no split pays, and the
+ * call is then mase_gemm_bf16_tn itself (workspace may be NULL). */
+size_t mase_gemm_bf16_tn_splitk_workspace_bytes(size_t M, size_t N, size_t K);
+int mase_gemm_bf16_tn_splitk(const void* A, const void* B, const void* bias, void* C, size_t M, size_t N, size_t K,
+                             int out_dtype, int bias_dtype, void* workspace, size_t workspace_bytes, void* stream);
+
 /* The same product for few rows of A (M <= 128, the token-by-token shape of serving): bound by streaming B once
  * from HBM.  The work is split over N and over K ranges; the partial results of the K ranges go through
  * `workspace` (device memory, 16-byte aligned, at least mase_gemm_bf16_skinny_workspace_bytes(M, N, K) bytes, which

@@ -40,6 +40,17 @@ def gemm_bf16_tn(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dty
         )
         _lib.check(rc, "mase_gemm_bf16_skinny")
         return out
+    # a few hundred rows: too few output tiles for the chip; K ranges become work items as well
+    nbytes = lib.mase_gemm_bf16_tn_splitk_workspace_bytes(M, N, K) if 2 * M * K <= OPERAND_BYTES_LIMIT else 0
+    if nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=a.device)
+        rc = lib.mase_gemm_bf16_tn_splitk(
+            a.data_ptr(), b.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(), M, N, K,
+            _lib.DTYPE_CODE[out_dtype], _lib.DTYPE_CODE[bias.dtype] if bias is not None else 0, ws.data_ptr(), nbytes,
+            _lib.stream_ptr(a),
+        )
+        _lib.check(rc, "mase_gemm_bf16_tn_splitk")
+        return out
     # the kernel addresses an operand with 32-bit byte offsets: activations beyond 4 GiB go in row chunks
     rows_per_call = max(1, min(M, (OPERAND_BYTES_LIMIT // (2 * K)) // 256 * 256 or 1))
     for r0 in range(0, M, rows_per_call):

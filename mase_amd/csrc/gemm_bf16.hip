@@ -52,6 +52,8 @@ struct GemmParams {
   int M, N, K;
   int bias_dtype;
   int tiles_m, tiles_n;
+  int splits, kc;  // K is cut into `splits` ranges of kc elements; a work item is one output tile over one range and
+                   // (when splits > 1) writes an fp32 partial tile into slice `range` of C, laid out [splits, M, N]
 };
 
 __device__ __forceinline__ int lds_off(int row, int chunk) {
@@ -93,12 +95,13 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   const int lane = lane_id;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
-  const int nk = p.K / BK;
+  const int nk = p.kc / BK;
 
   // ---- this work-group's output tiles.  Work-groups are dealt to the 8 XCDs round-robin; when the counts
   // divide, XCD x owns the contiguous tile range [x*total/8, (x+1)*total/8) and its work-groups walk it
   // together (at any time they hold neighbouring tiles, which share operand rows in that XCD's L2).
-  const int total = p.tiles_m * p.tiles_n;
+  const int tiles_mn = p.tiles_m * p.tiles_n;
+  const int total = tiles_mn * p.splits;
   const int nwg = (int)gridDim.x;
   int t_first, t_step, t_end;
   if ((total & 7) == 0 && (nwg & 7) == 0) {
@@ -115,8 +118,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   if (n_my == 0) return;
   constexpr int GROUP_M = 4;  // tiles are walked in groups of 4 tile rows
   const int in_group = GROUP_M * p.tiles_n;
-  auto tile_origin = [&](int ord, int& m0, int& n0) __attribute__((always_inline)) {  // ord-th tile of this work-group
-    const int t = t_first + min(ord, n_my - 1) * t_step;
+  auto tile_origin = [&](int ord, int& m0, int& n0, int& ks) __attribute__((always_inline)) {  // ord-th item of this work-group
+    const int item = t_first + min(ord, n_my - 1) * t_step;
+    ks = item / tiles_mn;
+    const int t = item - ks * tiles_mn;
     const int first_m = (t / in_group) * GROUP_M;
     const int gsz = min(p.tiles_m - first_m, GROUP_M);
     m0 = (first_m + (t % in_group) % gsz) * BM;
@@ -127,16 +132,17 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   const size_t ldb = (size_t)p.K * 2;  // bytes per operand row
   uint32_t ga[kWaveCopies], gb[kWaveCopies];  // byte offsets of this lane's chunks from the operand bases
   auto set_copy_tile = [&](int ord) __attribute__((always_inline)) {
-    int m0, n0;
-    tile_origin(ord, m0, n0);
+    int m0, n0, ks;
+    tile_origin(ord, m0, n0, ks);
+    const uint32_t k0 = (uint32_t)ks * (uint32_t)p.kc * 2u;  // byte offset of the item's K range inside a row
     int lane = lane_id;
     asm volatile("" : "+v"(lane));  // keeps the lane-derived terms below out of the K loop's live registers
 #pragma unroll
     for (int j = 0; j < kWaveCopies; ++j) {
       const int r = (wave + 4 * j) * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ ((r >> 1) & 7);  // chunk that belongs at LDS position lane&7 of row r
-      ga[j] = (uint32_t)((size_t)min(m0 + r, p.M - 1) * ldb) + chunk * 16;
-      gb[j] = (uint32_t)((size_t)min(n0 + r, p.N - 1) * ldb) + chunk * 16;
+      ga[j] = (uint32_t)((size_t)min(m0 + r, p.M - 1) * ldb) + chunk * 16 + k0;
+      gb[j] = (uint32_t)((size_t)min(n0 + r, p.N - 1) * ldb) + chunk * 16 + k0;
     }
   };
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;
@@ -202,8 +208,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // barrier and no wait for write completion is needed (the LDS executes one half-wave's accesses in order).
   const bool vec_ok = ((p.N & 3) == 0) && ((((uintptr_t)p.C) & 15u) == 0);
   auto epilogue = [&](int ord) __attribute__((always_inline)) {
-    int m0, n0;
-    tile_origin(ord, m0, n0);
+    int m0, n0, ks;
+    tile_origin(ord, m0, n0, ks);
+    // partial tiles of K range ks go to slice ks of C (fp32, no bias: the caller's reduction adds it)
+    unsigned char* const Cs = (unsigned char*)p.C + (size_t)ks * (size_t)p.M * (size_t)p.N * sizeof(float);
     int lane = lane_id;
     asm volatile("" : "+v"(lane));  // keeps the lane-derived terms below out of the K loop's live registers
     const int frag_row = lane & 31, kgrp = lane >> 5;
@@ -248,25 +256,25 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
             const size_t o = (size_t)row * p.N + col0;
             if (vec_ok && col0 + 3 < p.N) {
               if constexpr (OUT_DT == MASE_DT_F32) {
-                *(float4*)((float*)p.C + o) = make_float4(v[0], v[1], v[2], v[3]);
+                *(float4*)((float*)Cs + o) = make_float4(v[0], v[1], v[2], v[3]);
               } else if constexpr (OUT_DT == MASE_DT_BF16) {
                 uint2 w;
                 w.x = f32x2_to_bf16x2_bits(v[0], v[1]);
                 w.y = f32x2_to_bf16x2_bits(v[2], v[3]);
-                *(uint2*)((uint16_t*)p.C + o) = w;
+                *(uint2*)((uint16_t*)Cs + o) = w;
               } else {
                 uint2 w;
                 w.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
                 w.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
-                *(uint2*)((uint16_t*)p.C + o) = w;
+                *(uint2*)((uint16_t*)Cs + o) = w;
               }
             } else {
 #pragma unroll
               for (int e = 0; e < 4; ++e) {
                 if (col0 + e >= p.N) continue;
-                if constexpr (OUT_DT == MASE_DT_F32) ((float*)p.C)[o + e] = v[e];
-                else if constexpr (OUT_DT == MASE_DT_BF16) ((uint16_t*)p.C)[o + e] = (uint16_t)f32_to_bf16_bits(v[e]);
-                else ((uint16_t*)p.C)[o + e] = (uint16_t)f32_to_f16_bits(v[e]);
+                if constexpr (OUT_DT == MASE_DT_F32) ((float*)Cs)[o + e] = v[e];
+                else if constexpr (OUT_DT == MASE_DT_BF16) ((uint16_t*)Cs)[o + e] = (uint16_t)f32_to_bf16_bits(v[e]);
+                else ((uint16_t*)Cs)[o + e] = (uint16_t)f32_to_f16_bits(v[e]);
               }
             }
           }
@@ -362,6 +370,66 @@ int persistent_grid_bf16(int total_tiles) {
   return total_tiles < n_cu ? total_tiles : n_cu;
 }
 
+// launch of the persistent kernel for the work items of p (tiles x K ranges), output dtype out_dtype
+int launch_gemm_bf16(const GemmParams& p, int out_dtype, hipStream_t st) {
+  const size_t lds_bytes = (size_t)kLdsBytes;
+  const int nwg = persistent_grid_bf16(p.tiles_m * p.tiles_n * p.splits);
+  if (nwg <= 0) return MASE_ERR_LAUNCH;
+  const dim3 grid((unsigned)nwg), block(kGemmThreads);
+  const bool stream_fits = p.kc / BK >= S;
+#define MASE_GEMM_LAUNCH(DT_, STREAM_)                                                                            \
+  do {                                                                                                            \
+    static bool attr_set = false;                                                                                 \
+    const void* k = (const void*)gemm_bf16_tn_kernel<DT_, STREAM_>;                                               \
+    if (!attr_set) {                                                                                              \
+      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)       \
+        return MASE_ERR_LAUNCH;                                                                                   \
+      attr_set = true;                                                                                            \
+    }                                                                                                             \
+    hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, STREAM_>), grid, block, lds_bytes, st, p);                       \
+  } while (0)
+  if (stream_fits) {
+    if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH(MASE_DT_F32, true);
+    else if (out_dtype == MASE_DT_BF16) MASE_GEMM_LAUNCH(MASE_DT_BF16, true);
+    else MASE_GEMM_LAUNCH(MASE_DT_F16, true);
+  } else {
+    if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH(MASE_DT_F32, false);
+    else if (out_dtype == MASE_DT_BF16) MASE_GEMM_LAUNCH(MASE_DT_BF16, false);
+    else MASE_GEMM_LAUNCH(MASE_DT_F16, false);
+  }
+#undef MASE_GEMM_LAUNCH
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+// C[m][n] = sum over the K ranges, in order, of P[range][m][n]  (+ bias[n]), converted to the output dtype
+template <int OUT_DT>
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ P, void* __restrict__ C,
+                                                                 const void* __restrict__ bias, int bias_dtype,
+                                                                 size_t mn, int N, int splits) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= mn) return;
+  float s = 0.0f;
+  for (int k = 0; k < splits; ++k) s += P[(size_t)k * mn + i];
+  if (bias != nullptr) s += load_bias(bias, bias_dtype, (int)(i % (size_t)N));
+  if constexpr (OUT_DT == MASE_DT_F32) ((float*)C)[i] = s;
+  else if constexpr (OUT_DT == MASE_DT_BF16) ((uint16_t*)C)[i] = (uint16_t)f32_to_bf16_bits(s);
+  else ((uint16_t*)C)[i] = (uint16_t)f32_to_f16_bits(s);
+}
+
+// K ranges for a product whose output tiles alone would leave most CUs idle: as many as fill the machine once, each a
+// whole number of K tiles and at least 4 of them; 1 when the tiles already fill three quarters of the CUs
+int splitk_ranges(size_t M, size_t N, size_t K) {
+  const int n_cu = persistent_grid_bf16(1 << 30);
+  if (n_cu <= 0 || K % BK != 0) return 1;
+  const long tiles = (long)((M + BM - 1) / BM) * (long)((N + BN - 1) / BN);
+  if (tiles * 4 >= (long)n_cu * 3) return 1;
+  const int kt = (int)(K / BK);
+  int best = 1;
+  for (int s = 2; s <= 16 && (long)s * tiles <= n_cu; ++s)
+    if (kt % s == 0 && kt / s >= 4) best = s;
+  return best;
+}
+
 }  // namespace
 }  // namespace mase
 
@@ -386,32 +454,56 @@ extern "C" int mase_gemm_bf16_tn(const void* A, const void* B, const void* bias,
   p.bias_dtype = bias_dtype;
   p.tiles_m = (int)((M + BM - 1) / BM);
   p.tiles_n = (int)((N + BN - 1) / BN);
-  const size_t lds_bytes = (size_t)kLdsBytes;
-  const int nwg = persistent_grid_bf16(p.tiles_m * p.tiles_n);
-  if (nwg <= 0) return MASE_ERR_LAUNCH;
-  const dim3 grid((unsigned)nwg), block(kGemmThreads);
+  p.splits = 1;
+  p.kc = (int)K;
+  return launch_gemm_bf16(p, out_dtype, (hipStream_t)stream);
+}
+
+extern "C" size_t mase_gemm_bf16_tn_splitk_workspace_bytes(size_t M, size_t N, size_t K) {
+  using namespace mase;
+  if (M == 0 || N == 0 || K == 0) return 0;
+  const int splits = splitk_ranges(M, N, K);
+  return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
+}
+
+extern "C" int mase_gemm_bf16_tn_splitk(const void* A, const void* B, const void* bias, void* C, size_t M, size_t N,
+                                        size_t K, int out_dtype, int bias_dtype, void* workspace, size_t workspace_bytes,
+                                        void* stream) {
+  using namespace mase;
+  if (M == 0 || N == 0) return MASE_OK;
+  const int splits = (K % BK == 0) ? splitk_ranges(M, N, K) : 1;
+  if (splits <= 1) return mase_gemm_bf16_tn(A, B, bias, C, M, N, K, out_dtype, bias_dtype, stream);
+  if (A == nullptr || B == nullptr || C == nullptr) return MASE_ERR_NULL;
+  if (M > (1u << 30) || N > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
+  if ((unsigned long long)M * K * 2 > 0xFFFFFFFFull || (unsigned long long)N * K * 2 > 0xFFFFFFFFull) return MASE_ERR_SHAPE;
+  if (!aligned16(A) || !aligned16(B)) return MASE_ERR_ALIGN;
+  if (out_dtype < 0 || out_dtype > 2 || (bias != nullptr && (bias_dtype < 0 || bias_dtype > 2))) return MASE_ERR_DTYPE;
+  const size_t need = (size_t)splits * M * N * sizeof(float);
+  if (workspace == nullptr || workspace_bytes < need || (((uintptr_t)workspace) & 15u) != 0) return MASE_ERR_WORKSPACE;
+  GemmParams p;
+  p.A = (const unsigned char*)A;
+  p.B = (const unsigned char*)B;
+  p.bias = nullptr;
+  p.C = workspace;
+  p.M = (int)M;
+  p.N = (int)N;
+  p.K = (int)K;
+  p.bias_dtype = 0;
+  p.tiles_m = (int)((M + BM - 1) / BM);
+  p.tiles_n = (int)((N + BN - 1) / BN);
+  p.splits = splits;
+  p.kc = (int)(K / splits);
   hipStream_t st = (hipStream_t)stream;
-  const bool stream_fits = p.K / BK >= S;
-#define MASE_GEMM_LAUNCH(DT_, STREAM_)                                                                            \
-  do {                                                                                                            \
-    static bool attr_set = false;                                                                                 \
-    const void* k = (const void*)gemm_bf16_tn_kernel<DT_, STREAM_>;                                               \
-    if (!attr_set) {                                                                                              \
-      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)       \
-        return MASE_ERR_LAUNCH;                                                                                   \
-      attr_set = true;                                                                                            \
-    }                                                                                                             \
-    hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, STREAM_>), grid, block, lds_bytes, st, p);                       \
-  } while (0)
-  if (stream_fits) {
-    if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH(MASE_DT_F32, true);
-    else if (out_dtype == MASE_DT_BF16) MASE_GEMM_LAUNCH(MASE_DT_BF16, true);
-    else MASE_GEMM_LAUNCH(MASE_DT_F16, true);
-  } else {
-    if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH(MASE_DT_F32, false);
-    else if (out_dtype == MASE_DT_BF16) MASE_GEMM_LAUNCH(MASE_DT_BF16, false);
-    else MASE_GEMM_LAUNCH(MASE_DT_F16, false);
-  }
-#undef MASE_GEMM_LAUNCH
+  const int rc = launch_gemm_bf16(p, MASE_DT_F32, st);
+  if (rc != MASE_OK) return rc;
+  const size_t mn = M * N;
+  const dim3 grid(blocks_for(mn, (size_t)256)), block(256);
+  const float* P = (const float*)workspace;
+  if (out_dtype == MASE_DT_F32)
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<MASE_DT_F32>, grid, block, 0, st, P, C, bias, bias_dtype, mn, (int)N, splits);
+  else if (out_dtype == MASE_DT_BF16)
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<MASE_DT_BF16>, grid, block, 0, st, P, C, bias, bias_dtype, mn, (int)N, splits);
+  else
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel<MASE_DT_F16>, grid, block, 0, st, P, C, bias, bias_dtype, mn, (int)N, splits);
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }

@@ -60,6 +60,10 @@ def test_entry_points_reject_bad_arguments_without_a_gpu(lib):
     assert lib.mase_gemm_bf16_skinny(p, p, None, p, 4, 4, 64, 5, 0, p, 4096, None) == -4
     assert lib.mase_gemm_bf16_skinny_workspace_bytes(129, 4096, 4096) == 0   # outside the kernel's domain
     assert lib.mase_gemm_bf16_skinny_workspace_bytes(32, 4096, 100) == 0
+    # mase_gemm_bf16_tn_splitk falls back to the plain entry point's checks when nothing is split (no device here)
+    assert lib.mase_gemm_bf16_tn_splitk(p, p, None, p, 4, 4, 96, 0, 0, None, 0, None) == -2
+    assert lib.mase_gemm_bf16_tn_splitk(p, None, None, p, 4, 4, 64, 0, 0, None, 0, None) == -1
+    assert lib.mase_gemm_bf16_tn_splitk_workspace_bytes(0, 4, 64) == 0
     # mase_gemm_mxint8_skinny(A, codes, scales, bias, C, M, N, K, out_dtype, bias_dtype, workspace, workspace_bytes, stream)
     assert lib.mase_gemm_mxint8_skinny(p, p, p, None, p, 4, 4, 192, 0, 0, p, 4096, None) == -2    # K in whole 128-chunks
     assert lib.mase_gemm_mxint8_skinny(p, p, p, None, p, 129, 4, 128, 0, 0, p, 4096, None) == -2

@@ -156,3 +156,34 @@ def test_gemm_few_rows_with_mxint8_coded_weights(dev, M):
     assert torch.equal(deq.float().cpu(), wi)
     got = gemm_mxint8_skinny(ai.bfloat16().to(dev), codes.view(N, K), scales.view(N, K // 32), None, torch.float32)
     assert torch.equal(got.cpu(), ai @ wi.T)
+
+
+@pytest.mark.parametrize("M", [129, 256, 300, 512, 1000])
+def test_gemm_a_few_hundred_rows_cuts_k_into_work_items(dev, M):
+    """mase_gemm_bf16_tn_splitk through the dispatch of gemm_bf16_tn: exact on integer operands, agrees with fp64
+    otherwise, reproducible, bias and all output dtypes; a shape with enough tiles reports no workspace"""
+    from mase_amd import _lib
+    from mase_amd._gemm import gemm_bf16_tn
+
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(M)
+    for (N, K) in [(4096, 4096), (1024, 8192), (768, 1536), (11008, 4096)]:
+        assert lib.mase_gemm_bf16_tn_splitk_workspace_bytes(M, N, K) % (M * N * 4) == 0
+        ai = torch.randint(-3, 4, (M, K), generator=g).bfloat16().to(dev)
+        bi = torch.randint(-3, 4, (N, K), generator=g).bfloat16().to(dev)
+        bias = torch.randint(-5, 6, (N,), generator=g).float().to(dev)
+        want = ai.double() @ bi.double().T + bias.double()
+        for dt in (torch.float32, torch.bfloat16):
+            got = gemm_bf16_tn(ai, bi, bias, dt)
+            if dt == torch.float32:
+                assert torch.equal(got.double(), want), (N, K)
+            else:
+                assert torch.equal(got, want.to(dt)), (N, K)
+        a = torch.randn(M, K, generator=g).bfloat16().to(dev)
+        b = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(dev)
+        got = gemm_bf16_tn(a, b, None, torch.float32)
+        ref = a.double() @ b.double().T
+        assert float((got.double() - ref).abs().max() / ref.abs().max()) < 2e-6
+        assert torch.equal(got, gemm_bf16_tn(a, b, None, torch.float32))
+    assert lib.mase_gemm_bf16_tn_splitk_workspace_bytes(4096, 4096, 4096) == 0      # 256 tiles: nothing to split
+    assert lib.mase_gemm_bf16_tn_splitk_workspace_bytes(512, 4096, 4096) > 0
