@@ -14,7 +14,8 @@ Secondary workloads (other rows of the path, same JSON; --dtype bf16|f32|f16 whe
     integer_qdq, minifloat_denorm_qdq, minifloat_ieee_qdq, minifloat_mx_qdq, mxfp_qdq   on [8,2048,4096]
     attn_prob    score -> probability chain of the MX-quantized attention on [4,32,2048,2048]
     decode_linear  LinearMXInt 8192 -> 28672 for 16 tokens (weight-streaming kernel); decode_linear_packed: the same
-                   with the weight streamed as int8 codes + scale bytes
+                   with the weight streamed as int8 codes + scale bytes; decode_linear_mxfp4: LinearMXFP with e2m1
+                   weights on the block-scaled MFMA
     copy         calibration copy
 Prints ONE JSON line.  `value` is algorithmic GB/s (Q-DQ) or TFLOP/s (Linear) over the whole timed region;
 `roofline` is for the dominant kernel, timed with HIP events on the launch stream; `cpu_baseline` is the CPU
@@ -606,9 +607,59 @@ class DecodeLinearPacked(DecodeLinear):
     weight_bytes = 1.03125
 
 
+class DecodeLinearMxfp4(Workload):
+    """LinearMXFP (e2m1 weights, e4m3 activations) forward for a handful of tokens: the weight codes streamed once"""
+    name = "decode_linear_mxfp4"
+    unit = "GB/s"
+    dtype = "fp8"
+    kernel = "gemm_skinny_mxfp4_partial_kernel"
+    M, N, K = 16, 28672, 8192
+    metric = ("MXFP4-weight Linear forward for 16 tokens (algorithmic bytes: e2m1 codes + E8M0 scales, 0.53125 B per "
+              "weight, read once)")
+    config = {"workload": "LinearMXFP 8192 -> 28672 (e2m1 weights, e4m3 activations, block 32), 16 tokens, bf16, "
+                          "weights N(0,0.02) seed 7"}
+    cfg = {"weight_block_size": 32, "weight_exponent_width": 2, "weight_frac_width": 1,
+           "data_in_block_size": 32, "data_in_exponent_width": 4, "data_in_frac_width": 3}
+
+    def setup(self, torch, dev, n_buffers):
+        from mase_amd.quantized import LinearMXFP
+
+        g = torch.Generator().manual_seed(7)
+        self.mods = []
+        for i in range(3):  # alternated layers: 3 x 125 MB of codes, beyond what the last-level cache keeps hot
+            m = LinearMXFP(self.K, self.N, bias=False, device=dev, dtype=torch.bfloat16, config=dict(self.cfg))
+            m.load_state_dict({"weight": (torch.randn(self.N, self.K, generator=g) * 0.02).bfloat16()})
+            assert m._w_packed.valid_for(m.weight)
+            self.mods.append(m)
+        self.x = torch.randn(self.M, self.K, generator=g).bfloat16().to(dev)
+
+    def step(self, i):
+        self.out = self.mods[i % 3](self.x)
+
+    def work_per_step(self):
+        return float(self.N * self.K) * 0.53125
+
+    def cpu_baseline(self, torch, budget_s):
+        from oracle import linear as OL
+
+        n_rows = 2048
+        w = self.mods[0].weight.data[:n_rows].float().cpu()
+        x = self.x.float().cpu()
+        t0 = time.perf_counter()
+        n = 0
+        while True:
+            OL.linear_mxfp_forward(x, w, None, self.cfg)
+            n += 1
+            if time.perf_counter() - t0 > budget_s or n >= 20:
+                break
+        dt = (time.perf_counter() - t0) / n
+        return {"value": n_rows * self.K * 0.53125 / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                "kind": "port", "sample": f"{n} forwards with {n_rows} of the {self.N} output rows (fp32 on the CPU), {dt*1e3:.0f} ms each"}
+
+
 WORKLOADS = {w.name: w for w in (BfpQdq, MxintQdq, MxintLinear, MxfpLinear, DecoderLayerMxint, CopyBytes, IntegerQdq,
                                  MinifloatDenormQdq, MinifloatIeeeQdq, MinifloatMxQdq, MxfpQdq, AttnProb, DecodeLinear,
-                                 DecodeLinearPacked)}
+                                 DecodeLinearPacked, DecodeLinearMxfp4)}
 
 
 def load_traffic(name):

@@ -24,6 +24,7 @@
  *   mase_mx_unpack          nn/quantizers/mxint/fake.py:59-80, nn/quantizers/mxfp/fake.py:75-104 (compose_*)
  *   mase_mxfp_pack, mase_gemm_mxfp_scaled   nn/quantized/modules/linear.py:877-895 (LinearMXFP.forward on
  *                           formats the block-scaled matrix instruction supports)
+ *   mase_gemm_mxfp4_skinny  nn/quantized/modules/linear.py:877-895 for at most 128 rows, MXFP4 weights
  *   mase_gemm_mxint8_skinny nn/quantized/modules/linear.py:972 for at most 128 rows, weights as int8 codes + scales
  *   mase_gemm_bf16_skinny   same call sites as mase_gemm_bf16_tn, for at most 128 rows of activations
  *   mase_gemm_bf16_tn       nn/quantized/modules/linear.py:972 and :895 (the F.linear of LinearMXInt.forward /
@@ -155,6 +156,15 @@ size_t mase_gemm_mxint8_skinny_workspace_bytes(size_t M, size_t N, size_t K);
 int mase_gemm_mxint8_skinny(const void* A, const int8_t* B_codes, const uint8_t* B_scales, const void* bias, void* C,
                             size_t M, size_t N, size_t K, int out_dtype, int bias_dtype, void* workspace,
                             size_t workspace_bytes, void* stream);
+
+/* The few-rows product on packed MXFP operands (layout of mase_mxfp_pack): activations e4m3 (a_format 0) or e5m2 (1)
+ * codes [M, K] with scales [M, K/32], weights e2m1 codes [N, K/2] with scales [N, K/32], on the block-scaled MFMA.
+ * The weight stream is 0.53 bytes per element.  M <= 128, K % 128 == 0; workspace as for mase_gemm_bf16_skinny.
+ * LinearMXFP.forward (nn/quantized/modules/linear.py:877-895) for decode-sized batches with MXFP4 weights. */
+size_t mase_gemm_mxfp4_skinny_workspace_bytes(size_t M, size_t N, size_t K);
+int mase_gemm_mxfp4_skinny(const void* A_codes, const void* A_scales, int a_format, const void* B_codes,
+                           const void* B_scales, const void* bias, void* C, size_t M, size_t N, size_t K, int out_dtype,
+                           int bias_dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* MXFP packing for the block-scaled matrix instruction.  in: numel elements (numel % 32 == 0, blocks of 32
  * consecutive elements); element format (exp_bits, frac_bits) in {(4,3), (5,2), (2,1)}.  codes: one byte per

@@ -143,3 +143,33 @@ def gemm_mxfp_scaled(a_codes: Tensor, a_scales: Tensor, a_fmt, b_codes: Tensor, 
         )
         _lib.check(rc, "mase_gemm_mxfp_scaled")
     return out
+
+
+def gemm_mxfp4_skinny_supported(M: int, N: int, K: int, b_fmt) -> bool:
+    return 0 < M <= SKINNY_MAX_ROWS and K % 128 == 0 and tuple(b_fmt) == (2, 1) and N * K // 2 < (1 << 32)
+
+
+def gemm_mxfp4_skinny(a_codes: Tensor, a_scales: Tensor, a_fmt, b_codes: Tensor, b_scales: Tensor, bias: Tensor | None,
+                      out_dtype: torch.dtype) -> Tensor:
+    """``dequant(A)[M,K] @ dequant(B)[N,K].T + bias`` for at most 128 rows of e4m3 / e5m2 activations and e2m1 weights
+    (``mxfp_pack`` layout): the weight-streaming form of ``gemm_mxfp_scaled``."""
+    _lib.require_device(a_codes, "gemm_mxfp4_skinny")
+    lib = _lib.load()
+    a_codes, a_scales = a_codes.contiguous(), a_scales.contiguous()
+    b_codes, b_scales = b_codes.contiguous(), b_scales.contiguous()
+    M, K = a_codes.shape
+    N = b_codes.shape[0]
+    assert b_codes.shape == (N, K // 2) and a_scales.shape == (M, K // 32) and b_scales.shape == (N, K // 32)
+    assert gemm_mxfp4_skinny_supported(M, N, K, (2, 1)) and tuple(a_fmt) in ((4, 3), (5, 2))
+    out = torch.empty((M, N), dtype=out_dtype, device=a_codes.device)
+    if bias is not None:
+        bias = bias.contiguous()
+    nbytes = lib.mase_gemm_mxfp4_skinny_workspace_bytes(M, N, K)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=a_codes.device)
+    rc = lib.mase_gemm_mxfp4_skinny(
+        a_codes.data_ptr(), a_scales.data_ptr(), MXFP_HW_FORMATS[tuple(a_fmt)], b_codes.data_ptr(), b_scales.data_ptr(),
+        bias.data_ptr() if bias is not None else None, out.data_ptr(), M, N, K, _lib.DTYPE_CODE[out_dtype],
+        _lib.DTYPE_CODE[bias.dtype] if bias is not None else 0, ws.data_ptr(), nbytes, _lib.stream_ptr(a_codes),
+    )
+    _lib.check(rc, "mase_gemm_mxfp4_skinny")
+    return out

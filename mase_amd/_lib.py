@@ -50,6 +50,9 @@ SIGNATURES = {
     "mase_gemm_mxint8_skinny_workspace_bytes": (c_size_t, [c_size_t, c_size_t, c_size_t]),
     "mase_gemm_mxint8_skinny": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_int,
                                         c_int, c_void_p, c_size_t, c_void_p]),
+    "mase_gemm_mxfp4_skinny_workspace_bytes": (c_size_t, [c_size_t, c_size_t, c_size_t]),
+    "mase_gemm_mxfp4_skinny": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t,
+                                       c_size_t, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "mase_mxfp_pack": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mase_gemm_mxfp_scaled": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_int, c_int, c_void_p]),
     "mase_copy_bytes": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),

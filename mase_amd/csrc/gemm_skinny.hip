@@ -268,6 +268,126 @@ __global__ __launch_bounds__(kSqThreads) void gemm_skinny_mxint8_partial_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The few-rows product on packed MXFP operands with the block-scaled matrix instruction: activations as e4m3 / e5m2
+// codes [M, K] and weights as e2m1 codes [N, K/2] (two per byte), one E8M0 scale byte per 32 elements each (the
+// layout of mase_mxfp_pack).  The weight stream is 0.53 bytes per element, a quarter of the bf16 image, and the
+// instruction dequantizes in hardware: nothing but the copies, four LDS reads and one MFMA per 64 elements of K.
+// Operand roles as in gemm_mxfp.hip: A = activations (rows = tokens), B = weights (rows = the wavefront's 32 weight
+// rows); a chunk is 128 elements of K = two instructions; the scale dword of a row holds the chunk's 4 block scales,
+// lane group g uses byte 2*step + g.
+// ---------------------------------------------------------------------------------------------
+typedef int i32x8_t __attribute__((ext_vector_type(8)));
+template <int XC>
+struct SfGeom {
+  static constexpr int kWBytes = 32 * 64, kScaleBytes = 256, kXBytes = XC * 8 * 128;
+  static constexpr int kStageBytes = kWBytes + kScaleBytes + kXBytes + kScaleBytes;
+  static constexpr int kFit = (40 * 1024) / kStageBytes;
+  static constexpr int kStages = kFit > 8 ? 8 : kFit;   // outstanding copies stay below the 6-bit counter's range
+  static constexpr int kCopies = 2 + 1 + XC + 1;
+  static constexpr int kLdsBytes = 4 * kStages * kStageBytes;
+};
+
+struct SkinnyFParams {
+  const unsigned char* Xc;   // [M, K] 8-bit activation codes, M <= 32
+  const unsigned char* Xs;   // [M, K/32]
+  const unsigned char* Wc;   // [N, K/2] e2m1 codes
+  const unsigned char* Ws;   // [N, K/32]
+  float* P;
+  int M, N, K;
+  int kc;                    // K elements per split (multiple of 128)
+};
+
+template <int XC, int CBSZ>
+__global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_mxfp4_partial_kernel(SkinnyFParams p) {
+  using G = SfGeom<XC>;
+  constexpr int S = G::kStages;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  const int r = lane & 31, g = lane >> 5;
+  const int n0 = ((int)blockIdx.x * 4 + wave) * 32;
+  if (n0 >= p.N) return;  // whole wavefront; there is no barrier in this kernel
+  const int ks = blockIdx.y;
+  // weights: copy j (0, 1) moves rows 16j .. 16j+15 (64 bytes per row per chunk): lane -> row 16j + lane/4, position lane%4
+  uint32_t offw[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int row = 16 * j + (lane >> 2);
+    const int chunk = (lane & 3) ^ ((row >> 2) & 3);
+    offw[j] = (uint32_t)((size_t)min(n0 + row, p.N - 1) * (size_t)(p.K / 2)) + chunk * 16;
+  }
+  // activations: copy j moves rows 8j .. 8j+7 (128 bytes per row per chunk)
+  uint32_t offx[XC];
+#pragma unroll
+  for (int j = 0; j < XC; ++j) {
+    const int row = 8 * j + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    offx[j] = (uint32_t)((size_t)min(row, p.M - 1) * (size_t)p.K) + chunk * 16;
+  }
+  // scales: lane -> the dword of row lane%32 for this chunk
+  const uint32_t offws = (uint32_t)((size_t)min(n0 + r, p.N - 1) * (size_t)(p.K / 32));
+  const uint32_t offxs = (uint32_t)((size_t)min(r, p.M - 1) * (size_t)(p.K / 32));
+  const unsigned char* wbase = p.Wc + (size_t)ks * (p.kc / 2);
+  const unsigned char* xbase = p.Xc + (size_t)ks * p.kc;
+  const unsigned char* wsbase = p.Ws + (size_t)ks * (p.kc / 32);
+  const unsigned char* xsbase = p.Xs + (size_t)ks * (p.kc / 32);
+  unsigned char* ring = lds + wave * (S * G::kStageBytes);
+  const uint32_t ring_addr = (uint32_t)(uintptr_t)(lptr_t)ring;
+  const int chunks = p.kc / 128;
+  constexpr int kOffWs = G::kWBytes, kOffX = G::kWBytes + G::kScaleBytes, kOffXs = kOffX + G::kXBytes;
+  auto issue = [&](int c) __attribute__((always_inline)) {  // chunk c (clamped: past the end re-copies the last chunk)
+    const int cc = min(c, chunks - 1);
+    const uint32_t st = ring_addr + (uint32_t)((c % S) * G::kStageBytes);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) sk_async_copy(wbase + (size_t)cc * 64, offw[j], st + j * 1024);
+    sk_async_copy4(wsbase + (size_t)cc * 4, offws, st + kOffWs);
+#pragma unroll
+    for (int j = 0; j < XC; ++j) sk_async_copy(xbase + (size_t)cc * 128, offx[j], st + kOffX + j * 1024);
+    sk_async_copy4(xsbase + (size_t)cc * 4, offxs, st + kOffXs);
+  };
+
+  f32x16_t acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+  for (int c = 0; c < S - 1; ++c) issue(c);
+  const int xrow = min(r, 8 * XC - 1);
+  for (int c = 0; c < chunks; ++c) {
+    issue(c + S - 1);
+    sk_wait_vmcnt<(S - 1) * G::kCopies>();  // chunk c has landed; the later ones may be in flight
+    const unsigned char* st = ring + (c % S) * G::kStageBytes;
+    const int sw = (int)(*(const uint32_t*)(st + kOffWs + r * 4) >> (8 * g));
+    const int sx = (int)(*(const uint32_t*)(st + kOffXs + r * 4) >> (8 * g));
+#pragma unroll
+    for (int step = 0; step < 2; ++step) {
+      const uint4 x0 = *(const uint4*)(st + kOffX + xrow * 128 + (((step * 4 + g) ^ ((xrow >> 1) & 7)) << 4));
+      const uint4 x1 = *(const uint4*)(st + kOffX + xrow * 128 + (((step * 4 + 2 + g) ^ ((xrow >> 1) & 7)) << 4));
+      const uint4 w0 = *(const uint4*)(st + r * 64 + (((step * 2 + g) ^ ((r >> 2) & 3)) << 4));
+      i32x8_t a, b;
+      a[0] = (int)x0.x; a[1] = (int)x0.y; a[2] = (int)x0.z; a[3] = (int)x0.w;
+      a[4] = (int)x1.x; a[5] = (int)x1.y; a[6] = (int)x1.z; a[7] = (int)x1.w;
+      b[0] = (int)w0.x; b[1] = (int)w0.y; b[2] = (int)w0.z; b[3] = (int)w0.w;
+      b[4] = 0; b[5] = 0; b[6] = 0; b[7] = 0;
+      if (step == 0) acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc, CBSZ, 4, 0, sx, 0, sw);
+      else acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc, CBSZ, 4, 2, sx, 2, sw);
+    }
+  }
+  sk_wait_vmcnt<0>();  // no copy may still be in flight towards LDS when the wavefront retires
+  // acc[q*4 + j] = C[token q*8 + g*4 + j][weight row n0 + r]
+  float* out = p.P + (size_t)ks * p.M * p.N;
+  const int n = n0 + r;
+  if (n < p.N) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int m = q * 8 + g * 4 + j;
+        if (m < p.M) out[(size_t)m * p.N + n] = acc[q * 4 + j];
+      }
+  }
+}
+
 __device__ __forceinline__ float skinny_bias(const void* bias, int dt, int col) {
   if (dt == MASE_DT_F32) return ((const float*)bias)[col];
   if (dt == MASE_DT_BF16) return bits2f((uint32_t)((const uint16_t*)bias)[col] << 16);
@@ -444,6 +564,82 @@ extern "C" int mase_gemm_mxint8_skinny(const void* A, const int8_t* B_codes, con
     else if (xc == 2) hipLaunchKernelGGL(gemm_skinny_mxint8_partial_kernel<2>, grid, block, SqGeom<2>::kLdsBytes, st, p);
     else if (xc == 3) hipLaunchKernelGGL(gemm_skinny_mxint8_partial_kernel<3>, grid, block, SqGeom<3>::kLdsBytes, st, p);
     else hipLaunchKernelGGL(gemm_skinny_mxint8_partial_kernel<4>, grid, block, SqGeom<4>::kLdsBytes, st, p);
+    const size_t mn_g = rows * N;
+    const dim3 rgrid_g((unsigned)blocks_for(mn_g, 256));
+    void* Cg = (unsigned char*)C + m0 * N * (out_dtype == MASE_DT_F32 ? 4 : 2);
+    if (out_dtype == MASE_DT_F32)
+      hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_F32>, rgrid_g, dim3(256), 0, st, p.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
+    else if (out_dtype == MASE_DT_BF16)
+      hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_BF16>, rgrid_g, dim3(256), 0, st, p.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
+    else
+      hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_F16>, rgrid_g, dim3(256), 0, st, p.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
+  }
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+extern "C" size_t mase_gemm_mxfp4_skinny_workspace_bytes(size_t M, size_t N, size_t K) {
+  using namespace mase;
+  if (M == 0 || N == 0 || K == 0 || (K % 128) != 0 || M > 128) return 0;
+  const int n_cu = skinny_cu_count();
+  if (n_cu <= 0) return 0;
+  return (size_t)skinny_splits((int)M, (int)N, (int)(K / 2), n_cu) * M * N * sizeof(float);
+}
+
+extern "C" int mase_gemm_mxfp4_skinny(const void* A_codes, const void* A_scales, int a_format, const void* B_codes,
+                                      const void* B_scales, const void* bias, void* C, size_t M, size_t N, size_t K,
+                                      int out_dtype, int bias_dtype, void* workspace, size_t workspace_bytes,
+                                      void* stream) {
+  using namespace mase;
+  if (M == 0 || N == 0) return MASE_OK;
+  if (A_codes == nullptr || A_scales == nullptr || B_codes == nullptr || B_scales == nullptr || C == nullptr) return MASE_ERR_NULL;
+  if (K == 0 || (K % 128) != 0 || M > 128 || N > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
+  if ((unsigned long long)N * K / 2 > 0xFFFFFFFFull) return MASE_ERR_SHAPE;
+  if (!aligned16(A_codes) || !aligned16(B_codes) || (((uintptr_t)A_scales) & 3u) != 0 || (((uintptr_t)B_scales) & 3u) != 0)
+    return MASE_ERR_ALIGN;
+  if (a_format != 0 && a_format != 1) return MASE_ERR_PARAM;
+  if (out_dtype < 0 || out_dtype > 2 || (bias != nullptr && (bias_dtype < 0 || bias_dtype > 2))) return MASE_ERR_DTYPE;
+  const int n_cu = skinny_cu_count();
+  if (n_cu <= 0) return MASE_ERR_LAUNCH;
+  const int splits = skinny_splits((int)M, (int)N, (int)(K / 2), n_cu);
+  const size_t need = (size_t)splits * M * N * sizeof(float);
+  if (workspace == nullptr || workspace_bytes < need || (((uintptr_t)workspace) & 15u) != 0) return MASE_ERR_WORKSPACE;
+  hipStream_t st = (hipStream_t)stream;
+  static bool attr_set = false;
+  if (!attr_set) {
+    const void* ks[8] = {(const void*)gemm_skinny_mxfp4_partial_kernel<1, 0>, (const void*)gemm_skinny_mxfp4_partial_kernel<2, 0>,
+                         (const void*)gemm_skinny_mxfp4_partial_kernel<3, 0>, (const void*)gemm_skinny_mxfp4_partial_kernel<4, 0>,
+                         (const void*)gemm_skinny_mxfp4_partial_kernel<1, 1>, (const void*)gemm_skinny_mxfp4_partial_kernel<2, 1>,
+                         (const void*)gemm_skinny_mxfp4_partial_kernel<3, 1>, (const void*)gemm_skinny_mxfp4_partial_kernel<4, 1>};
+    const int sz[4] = {SfGeom<1>::kLdsBytes, SfGeom<2>::kLdsBytes, SfGeom<3>::kLdsBytes, SfGeom<4>::kLdsBytes};
+    for (int i = 0; i < 8; ++i)
+      if (hipFuncSetAttribute(ks[i], hipFuncAttributeMaxDynamicSharedMemorySize, sz[i & 3]) != hipSuccess)
+        return MASE_ERR_LAUNCH;
+    attr_set = true;
+  }
+  const dim3 grid((unsigned)(((N + 31) / 32 + 3) / 4), (unsigned)splits), block(kSkinnyThreads);
+  SkinnyFParams p;
+  p.Wc = (const unsigned char*)B_codes;
+  p.Ws = (const unsigned char*)B_scales;
+  p.N = (int)N;
+  p.K = (int)K;
+  p.kc = (int)K / splits;
+  for (size_t m0 = 0; m0 < M; m0 += 32) {
+    const size_t rows = (M - m0 < 32) ? (M - m0) : 32;
+    p.Xc = (const unsigned char*)A_codes + m0 * K;
+    p.Xs = (const unsigned char*)A_scales + m0 * (K / 32);
+    p.P = (float*)workspace + (size_t)splits * m0 * N;
+    p.M = (int)rows;
+    const int xc = (int)(rows + 7) / 8;
+#define MASE_SF_LAUNCH(XC_)                                                                                           \
+  do {                                                                                                                \
+    if (a_format == 0) hipLaunchKernelGGL((gemm_skinny_mxfp4_partial_kernel<XC_, 0>), grid, block, SfGeom<XC_>::kLdsBytes, st, p); \
+    else hipLaunchKernelGGL((gemm_skinny_mxfp4_partial_kernel<XC_, 1>), grid, block, SfGeom<XC_>::kLdsBytes, st, p);  \
+  } while (0)
+    if (xc == 1) MASE_SF_LAUNCH(1);
+    else if (xc == 2) MASE_SF_LAUNCH(2);
+    else if (xc == 3) MASE_SF_LAUNCH(3);
+    else MASE_SF_LAUNCH(4);
+#undef MASE_SF_LAUNCH
     const size_t mn_g = rows * N;
     const dim3 rgrid_g((unsigned)blocks_for(mn_g, 256));
     void* Cg = (unsigned char*)C + m0 * N * (out_dtype == MASE_DT_F32 ? 4 : 2);

@@ -13,8 +13,9 @@ import torch
 from torch import Tensor
 from torch.nn import functional as F
 
-from ..._gemm import (MXFP_HW_FORMATS, MXFP_K_MULTIPLE, SKINNY_MAX_ROWS, gemm_bf16_tn, gemm_mxfp_scaled,
-                      gemm_mxint8_skinny, gemm_mxint8_skinny_supported, mxfp_pack)
+from ..._gemm import (MXFP_HW_FORMATS, MXFP_K_MULTIPLE, SKINNY_MAX_ROWS, gemm_bf16_tn, gemm_mxfp4_skinny,
+                      gemm_mxfp4_skinny_supported, gemm_mxfp_scaled, gemm_mxint8_skinny, gemm_mxint8_skinny_supported,
+                      mxfp_pack)
 
 
 class WeightCache:
@@ -227,5 +228,9 @@ def mxfp_linear_native(x: Tensor, packed: PackedMXFPWeight, bias: Tensor | None,
     lead = x.shape[:-1]
     x2 = x.reshape(-1, x.shape[-1])
     xc, xs = mxfp_pack(x2, *act_fmt)
-    y = gemm_mxfp_scaled(xc, xs, act_fmt, packed.codes, packed.scales, packed.fmt, bias, x.dtype)
+    if gemm_mxfp4_skinny_supported(x2.shape[0], packed.scales.shape[0], x2.shape[1], packed.fmt):
+        # decode-sized batch with MXFP4 weights: bound by streaming the weight codes once (0.53 bytes per weight)
+        y = gemm_mxfp4_skinny(xc, xs, act_fmt, packed.codes, packed.scales, bias, x.dtype)
+    else:
+        y = gemm_mxfp_scaled(xc, xs, act_fmt, packed.codes, packed.scales, packed.fmt, bias, x.dtype)
     return y.reshape(*lead, packed.codes.shape[0])

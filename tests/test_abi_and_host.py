@@ -70,6 +70,14 @@ def test_entry_points_reject_bad_arguments_without_a_gpu(lib):
     assert lib.mase_gemm_mxint8_skinny(p, p, None, None, p, 4, 4, 128, 0, 0, p, 4096, None) == -1
     assert lib.mase_gemm_mxint8_skinny(p, p, p, None, p, 4, 4, 128, 9, 0, p, 4096, None) == -4
     assert lib.mase_gemm_mxint8_skinny_workspace_bytes(4, 4, 192) == 0
+    # mase_gemm_mxfp4_skinny(A_codes, A_scales, a_format, B_codes, B_scales, bias, C, M, N, K, out_dtype, bias_dtype,
+    #                        workspace, workspace_bytes, stream)
+    assert lib.mase_gemm_mxfp4_skinny(p, p, 0, p, p, None, p, 4, 4, 192, 0, 0, p, 4096, None) == -2
+    assert lib.mase_gemm_mxfp4_skinny(p, p, 0, p, p, None, p, 129, 4, 128, 0, 0, p, 4096, None) == -2
+    assert lib.mase_gemm_mxfp4_skinny(p, None, 0, p, p, None, p, 4, 4, 128, 0, 0, p, 4096, None) == -1
+    assert lib.mase_gemm_mxfp4_skinny(p, p, 2, p, p, None, p, 4, 4, 128, 0, 0, p, 4096, None) == -5   # activations: e4m3 or e5m2
+    assert lib.mase_gemm_mxfp4_skinny(p, p, 0, p, p, None, p, 4, 4, 128, 7, 0, p, 4096, None) == -4
+    assert lib.mase_gemm_mxfp4_skinny_workspace_bytes(4, 4, 192) == 0
     assert lib.mase_mxfp_qdq(p, p, None, None, 64, 0, 0, 32, 3, 3, p, None) == -5  # illegal element format
     assert lib.mase_mxfp_qdq(p, p, None, None, 63, 0, 0, 32, 4, 3, p, None) == -2
     assert lib.mase_block_fp_qdq(p, p, 1, 4, 16, 0, 16, 0, 8, 8, -1, 0, p, None, 0, None) == -2

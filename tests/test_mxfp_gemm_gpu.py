@@ -124,3 +124,45 @@ def test_gemm_mxfp_several_tiles_per_work_group(dev, bfmt, M, N, K):
     ref = (ad @ bd.t()).cpu()  # exact in fp32: multiples of 32 (or 1024) well below 2^24 units
     y = gemm_mxfp_scaled(ac, asc, (4, 3), bc, bsc, bfmt, None, torch.float32)
     assert torch.equal(y.cpu(), ref)
+
+
+@pytest.mark.parametrize("afmt", [(4, 3), (5, 2)])
+@pytest.mark.parametrize("M", [1, 9, 16, 32, 33, 100, 128])
+def test_gemm_mxfp4_few_rows_streams_the_weight_codes(dev, afmt, M):
+    """mase_gemm_mxfp4_skinny against the decoded operands (same bound as the tiled kernel: the instruction is the
+    same) and against the tiled kernel itself; reproducible; bias and output dtypes"""
+    from mase_amd._gemm import gemm_mxfp4_skinny, gemm_mxfp_scaled, mxfp_pack
+
+    g = torch.Generator().manual_seed(M * 7 + afmt[0])
+    for (N, K) in [(64, 128), (4096, 4096), (1000, 1152), (11008, 2048)]:
+        a = torch.randn(M, K, generator=g)
+        a[:, 5] *= 20
+        b = torch.randn(N, K, generator=g) * 0.02
+        b[3] *= 2.0 ** -30
+        b[5, :64] = 0.0
+        bias = torch.randn(N, generator=g)
+        ac, asc = mxfp_pack(a.to(dev), *afmt)
+        bc, bsc = mxfp_pack(b.to(dev), 2, 1)
+        da, db = decode_ocp(ac, asc, afmt), decode_ocp(bc, bsc, (2, 1))
+        ref = da @ db.t()
+        bound = (da.abs() @ db.abs().t()) * 2.0 ** -9 + ref.abs() * 2.0 ** -21
+        y = gemm_mxfp4_skinny(ac, asc, afmt, bc, bsc, None, torch.float32)
+        d = (y.cpu().double() - ref).abs()
+        assert bool((d <= bound).all()), (N, K, float((d / bound).max()))
+        assert float(d.max() / ref.abs().max()) < 5e-4
+        tiled = gemm_mxfp_scaled(ac, asc, afmt, bc, bsc, (2, 1), None, torch.float32)
+        assert float((y - tiled).abs().max() / ref.abs().max()) < 5e-4
+        assert torch.equal(y, gemm_mxfp4_skinny(ac, asc, afmt, bc, bsc, None, torch.float32))
+        yb = gemm_mxfp4_skinny(ac, asc, afmt, bc, bsc, bias.to(dev), torch.bfloat16)
+        want = ref + bias.double()
+        assert bool(((yb.cpu().double() - want).abs() <= want.abs() * 2.0 ** -8 + ref.abs().max() * 5e-4).all())
+    # exact case: unit scales, small integers both formats hold exactly
+    N, K = 96, 256
+    ai = torch.randint(-4, 5, (M, K), generator=g).float()
+    bi = torch.randint(-3, 4, (N, K), generator=g).float()
+    ai[:, 0], bi[:, 0] = 4.0, 3.0
+    ac, asc = mxfp_pack(ai.to(dev), *afmt)
+    bc, bsc = mxfp_pack(bi.to(dev), 2, 1)
+    da, db = decode_ocp(ac, asc, afmt), decode_ocp(bc, bsc, (2, 1))
+    if torch.equal(da.float(), ai) and torch.equal(db.float(), bi):
+        assert torch.equal(gemm_mxfp4_skinny(ac, asc, afmt, bc, bsc, None, torch.float32).cpu().double(), da @ db.t())
