@@ -479,6 +479,14 @@ class MxfpQdq(_ElementwiseQdq):
     oracle_name, oracle_args = "mxfp_quantizer", (32, 4, 3)
 
 
+class MxintClipSearch(_ElementwiseQdq):
+    """mxint_quantizer(quantile_search=True): 11 candidate scales per block of 32, the weight-loading path of LinearMXInt
+    with config["clip_search"]"""
+    name, unit, kernel = "mxint_clip_search", "GB/s", "mxint_clip_search_kernel"
+    fn_name, args = "mxint_quantizer", (32, 4, -1, 8, True)
+    oracle_name, oracle_args = "mxint_quantizer", (32, 4, -1, 8, True)
+
+
 class MinifloatMxQdq(_ElementwiseQdq):
     name, unit, kernel = "minifloat_mx_qdq", "GB/s", "elementwise_kernel<MinifloatMxOp>"
     kernel16 = "minifloat_mx_pk16_kernel"
@@ -657,7 +665,7 @@ class DecodeLinearMxfp4(Workload):
                 "kind": "port", "sample": f"{n} forwards with {n_rows} of the {self.N} output rows (fp32 on the CPU), {dt*1e3:.0f} ms each"}
 
 
-WORKLOADS = {w.name: w for w in (BfpQdq, MxintQdq, MxintLinear, MxfpLinear, DecoderLayerMxint, CopyBytes, IntegerQdq,
+WORKLOADS = {w.name: w for w in (MxintClipSearch, BfpQdq, MxintQdq, MxintLinear, MxfpLinear, DecoderLayerMxint, CopyBytes, IntegerQdq,
                                  MinifloatDenormQdq, MinifloatIeeeQdq, MinifloatMxQdq, MxfpQdq, AttnProb, DecodeLinear,
                                  DecodeLinearPacked, DecodeLinearMxfp4)}
 

@@ -17,6 +17,8 @@
  *   mase_minifloat_qdq      nn/quantizers/minifloat.py:90-117, :200-225 (minifloat_denorm/ieee_quantizer)
  *   mase_minifloat_mx_qdq   nn/quantizers/_minifloat_mx/minifloat.py:12-33 (minifloat_quantizer_sim)
  *   mase_mxfp_qdq           nn/quantizers/mxfp/mxfp.py:187-230    (mxfp_quantizer, non-search branch)
+ *   mase_mxint_clip_search  nn/quantizers/mxint/mxint.py:40-143 (quantile_search=True without calibration activations)
+ *   mase_mxfp_clip_search   nn/quantizers/mxfp/mxfp.py:40-105   (quantile_search=True without calibration activations)
  *   mase_rope               nn/quantized/functional/rope.py:17-27 (_apply_rope)
  *   mase_rmsnorm_minifloat  nn/quantized/modules/llama/rms_norm.py:72-84 (LlamaRMSNormMinifloat.forward)
  *   mase_silu_mul_minifloat nn/quantized/modules/llama/mlp.py:60-62 (silu_minifloat(gate) * up)
@@ -112,6 +114,21 @@ int mase_minifloat_mx_qdq(const void* in, void* out, size_t numel, int in_dtype,
 int mase_mxfp_qdq(const void* in, void* out, uint8_t* codes, uint8_t* scales, size_t numel, int in_dtype,
                   int out_dtype, int block_size, int exp_bits, int frac_bits, const uint32_t* log2_tab,
                   void* stream);
+
+/* Clip search (quantile_search=True, act_tensor=None): per block of 32 elements, 11 quantize-dequantize candidates
+ * whose scale comes from the 1.0, 0.995, 0.99, 0.97, 0.95, 0.93, 0.90, 0.80, 0.70, 0.60, 0.50 quantile of |x| (linear
+ * interpolation, as the library's quantile) instead of the maximum; the candidate the reference's error measure
+ * prefers is written to `out` (same dtype as `in`), its index 0..10 to `choice` (optional, one byte per block).
+ * in: the tensor with block_dim moved last, flattened; ref: the tensor in its plain flattening (the reference
+ * measures the error against that one; the same array when block_dim is the last dimension).  block_size must be 32;
+ * in / ref / out 16-byte aligned.  MXINT (nn/quantizers/mxint/mxint.py:40-143): error = L2 norm in `dtype`, first
+ * minimum wins.  MXFP (nn/quantizers/mxfp/mxfp.py:40-105): the reference's score on the integer codes, strictly
+ * smaller replaces.  Candidates whose errors differ only by the summation order of the 32 squares may swap with respect
+ * to the library's reductions. */
+int mase_mxint_clip_search(const void* in, const void* ref, void* out, uint8_t* choice, size_t numel, int dtype,
+                           int block_size, int element_bits, int scale_bits, const uint32_t* log2_tab, void* stream);
+int mase_mxfp_clip_search(const void* in, const void* ref, void* out, uint8_t* choice, size_t numel, int dtype,
+                          int block_size, int exp_bits, int frac_bits, const uint32_t* log2_tab, void* stream);
 
 /* Dequantization of the packed outputs of mase_mxint_qdq (kind 0: p0 = element_bits, p1 unused; value = code *
  * 2^(scale - 134)) or mase_mxfp_qdq (kind 1: p0 = exp_bits, p1 = frac_bits; value = minifloat(code) * 2^(scale - 127),

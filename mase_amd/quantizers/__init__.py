@@ -85,18 +85,21 @@ class MXFPMeta:
 # ---------------------------------------------------------------------------------------------
 # MXINT
 # ---------------------------------------------------------------------------------------------
-def _reject_search(quantile_search: bool, name: str):
-    if quantile_search:
+def _reject_calibration(act_tensor, name: str):
+    if act_tensor is not None:
         raise NotImplementedError(
-            f"{name}: quantile_search=True (clip search / GPTQ calibration) is outside the accelerated path"
+            f"{name}: quantile_search with calibration activations (GPTQ) is outside the accelerated path"
         )
 
 
 def mxint_quantizer_sim(tensor: Tensor, block_dim: int, mxint_meta: MXIntMeta, act_tensor: Tensor | None = None,
                         dtype: torch.dtype | None = None, quantile_search: bool = False,
                         cali_batch_size: int = 32) -> Tensor:
-    """mxint/mxint.py:14-171 (non-search branch)."""
-    _reject_search(quantile_search, "mxint_quantizer_sim")
+    """mxint/mxint.py:14-171; the search branch (:40-143) without calibration activations."""
+    if quantile_search:
+        _reject_calibration(act_tensor, "mxint_quantizer_sim")
+        return _ops.mxint_clip_search(tensor, mxint_meta.block_size, mxint_meta.element_bits, block_dim,
+                                      mxint_meta.scale_bits)  # the search branch ignores `dtype` (mxint.py:143)
     out = _ops.mxint_qdq(tensor, mxint_meta.block_size, mxint_meta.element_bits, block_dim, mxint_meta.scale_bits)
     return out.to(dtype or tensor.dtype)
 
@@ -104,7 +107,8 @@ def mxint_quantizer_sim(tensor: Tensor, block_dim: int, mxint_meta: MXIntMeta, a
 def mxint_quantizer(x: Tensor, block_size: int, element_bits: int, block_dim: int = -1, scale_bits: int = 8,
                     quantile_search: bool = False) -> Tensor:
     """MXINT quantize-dequantize with a straight-through gradient (mxint/mxint.py:211-251)."""
-    _reject_search(quantile_search, "mxint_quantizer")
+    if quantile_search:
+        return _ste(_ops.mxint_clip_search, x, block_size, element_bits, block_dim, scale_bits)
     return _ste(_ops.mxint_qdq, x, block_size, element_bits, block_dim, scale_bits)
 
 
@@ -121,10 +125,15 @@ def minifloat_quantizer_sim(tensor: Tensor, minifloat_meta: MinifloatMeta,
 def mxfp_quantizer_sim(tensor: Tensor, block_dim: int, mxfp_meta: MXFPMeta, act_tensor: Tensor | None = None,
                        dtype: torch.dtype | None = None, quantile_search: bool = False,
                        cali_batch_size: int = 32) -> Tensor:
-    """mxfp/mxfp.py:14-115 (non-search branch; finite elements, round-to-nearest as MXFPQuantize fixes them)."""
-    _reject_search(quantile_search, "mxfp_quantizer_sim")
+    """mxfp/mxfp.py:14-115 (finite elements, round-to-nearest as MXFPQuantize fixes them); the search branch
+    (:40-105) without calibration activations."""
     if not (mxfp_meta.element_is_finite and mxfp_meta.round_mode == "rn"):
         raise NotImplementedError("mxfp_quantizer_sim: only finite elements with round mode 'rn' are accelerated")
+    if quantile_search:
+        _reject_calibration(act_tensor, "mxfp_quantizer_sim")
+        out = _ops.mxfp_clip_search(tensor, mxfp_meta.block_size, mxfp_meta.element_exp_bits,
+                                    mxfp_meta.element_frac_bits, block_dim, mxfp_meta.scale_exp_bits)
+        return out.to(dtype or tensor.dtype)
     out = _ops.mxfp_qdq(tensor, mxfp_meta.block_size, mxfp_meta.element_exp_bits, mxfp_meta.element_frac_bits,
                         block_dim, mxfp_meta.scale_exp_bits)
     return out.to(dtype or tensor.dtype)
@@ -133,7 +142,8 @@ def mxfp_quantizer_sim(tensor: Tensor, block_dim: int, mxfp_meta: MXFPMeta, act_
 def mxfp_quantizer(x: Tensor, block_size: int, element_exp_bits: int, element_frac_bits: int, block_dim: int = -1,
                    scale_exp_bits: int = 8, quantile_search: bool = False) -> Tensor:
     """MXFP quantize-dequantize with a straight-through gradient (mxfp/mxfp.py:187-230)."""
-    _reject_search(quantile_search, "mxfp_quantizer")
+    if quantile_search:
+        return _ste(_ops.mxfp_clip_search, x, block_size, element_exp_bits, element_frac_bits, block_dim, scale_exp_bits)
     return _ste(_ops.mxfp_qdq, x, block_size, element_exp_bits, element_frac_bits, block_dim, scale_exp_bits)
 
 

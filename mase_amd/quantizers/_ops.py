@@ -112,6 +112,49 @@ def mxfp_qdq(x: Tensor, block_size: int, exp_bits: int, frac_bits: int, block_di
     return (res, codes, scales) if pack else res
 
 
+CLIP_SEARCH_BLOCK = 32
+
+
+def _clip_search(name: str, x: Tensor, block_size: int, block_dim: int, tab_dtype, params, return_choice: bool):
+    """the search branch of the MX quantizers without calibration activations: blocks along block_dim, the error
+    measured against the blocks of the plain flattening (mxint/mxint.py:41-45, :97; mxfp/mxfp.py:41-45, :94-97)"""
+    _lib.require_device(x, name)
+    lib = _lib.load()
+    if block_size != CLIP_SEARCH_BLOCK:
+        raise NotImplementedError(f"{name}: quantile_search=True is built for block_size {CLIP_SEARCH_BLOCK}, got {block_size}")
+    shape = tuple(x.shape)
+    nd = len(shape)
+    assert block_dim < nd and block_dim >= -nd
+    assert x.numel() % block_size == 0, f"Input tensor size {x.numel()} is not divisible by block size {block_size}."
+    ref = x.contiguous().view(-1)
+    flat = _to_block_last_flat(x, block_dim)
+    out = torch.empty_like(flat)
+    choice = torch.empty(flat.numel() // block_size, dtype=torch.uint8, device=x.device) if return_choice else None
+    tab = log2_table(tab_dtype, x.device)
+    fn = getattr(lib, name)
+    rc = fn(flat.data_ptr(), ref.data_ptr(), out.data_ptr(), choice.data_ptr() if return_choice else None, flat.numel(),
+            _lib.dtype_code(x), block_size, *params, tab.data_ptr(), _lib.stream_ptr(x))
+    _lib.check(rc, name)
+    res = _from_block_last_flat(out, shape, block_dim)
+    return (res, choice) if return_choice else res
+
+
+def mxint_clip_search(x: Tensor, block_size: int, element_bits: int, block_dim: int, scale_bits: int,
+                      return_choice: bool = False):
+    return _clip_search("mase_mxint_clip_search", x, block_size, block_dim, x.dtype, (element_bits, scale_bits),
+                        return_choice)
+
+
+def mxfp_clip_search(x: Tensor, block_size: int, exp_bits: int, frac_bits: int, block_dim: int, scale_exp_bits: int,
+                     return_choice: bool = False):
+    assert scale_exp_bits in (8,), f"Invalid scale exponent bits: {scale_exp_bits}. Legal values are: (8,)."
+    assert (exp_bits, frac_bits) in _LEGAL_MXFP, (
+        f"Invalid element exp/frac bits: {(exp_bits, frac_bits)}. Legal values are: {_LEGAL_MXFP}."
+    )
+    return _clip_search("mase_mxfp_clip_search", x, block_size, block_dim, torch.float32, (exp_bits, frac_bits),
+                        return_choice)
+
+
 def _cast_args(cast):
     """(exp_bits, frac_bits, is_finite, round_mode code) of an optional minifloat cast; exp_bits 0 switches it off"""
     if cast is None:

@@ -25,6 +25,12 @@ Pinning status (what fixes each function besides reading the source):
   and ``mxfp_quantizer``           (``>> 8`` double rounding, lost carry in odd binades, truncating subnormals)
                                    are source-defined                                   -> parity unpinned (quirk regions)
 
+* clip search (``quantile_search``)   quantile against exact rational interpolation; candidates against the scalar
+                                   restatement; the choice against exact errors (first minimum, strict replace);
+                                   the MXFP score against its formula on integer codes  -> pinned, except the
+                                   library's summation order inside ``norm`` / ``sum`` and the uint8 power wrap,
+                                   which are facts of the host library              -> parity unpinned (that part)
+
 ``tests/golden/known_answers.json`` holds small vectors computed with the exact scalar restatement; the vectorised
 restatement (and the kernels) must reproduce them bit for bit.
 
@@ -42,8 +48,11 @@ from .quantizers import (  # noqa: F401
     minifloat_mx_compose,
     minifloat_mx_extract,
     minifloat_quantizer_sim,
+    CLIP_PERCENTILES,
+    mxfp_clip_search,
     mxfp_components,
     mxfp_quantizer,
+    mxint_clip_search,
     mxint_components,
     mxint_quantizer,
 )

@@ -68,9 +68,10 @@ def mxint_quantizer(
     quantile_search: bool = False,
     dtype: torch.dtype | None = None,
 ) -> Tensor:
-    """mxint/mxint.py:211-251 -> MXIntQuantize.forward :183-202 -> mxint_quantizer_sim else-branch :145-169."""
+    """mxint/mxint.py:211-251 -> MXIntQuantize.forward :183-202 -> mxint_quantizer_sim: else-branch :145-169, or
+    the search branch :40-143 without calibration activations."""
     if quantile_search:
-        raise NotImplementedError("oracle covers the non-search branch only (mxint.py:145-169)")
+        return mxint_clip_search(x, block_size, element_bits, block_dim, scale_bits)[0]
     in_dt = x.dtype
     shape = tuple(x.shape)
     assert -len(shape) <= block_dim < len(shape)
@@ -80,6 +81,38 @@ def mxint_quantizer(
     deq = mant / 2 ** (element_bits - 1) * 2 ** (scale - bias)  # fake.py:75-80
     out = _restore_from_flat(deq, shape, block_dim)
     return out.to(dtype or in_dt)
+
+
+CLIP_PERCENTILES = (1.0, 0.995, 0.99, 0.97, 0.95, 0.93, 0.90, 0.80, 0.70, 0.60, 0.50)  # mxint.py:47-51, mxfp.py:53
+
+
+def mxint_clip_search(x: Tensor, block_size: int, element_bits: int, block_dim: int = -1, scale_bits: int = 8):
+    """The search branch of mxint_quantizer_sim with act_tensor=None (mxint/mxint.py:40-143).
+
+    Returns (dequantized tensor, index of the chosen percentile per block, errors [11, n_blocks], candidates
+    [11, n_blocks, B]).  The candidates are the blocks taken along block_dim; the error is measured against the blocks of the plain flattening (:41-45, :97),
+    which are the same blocks only when block_dim is the last dimension.
+    """
+    B = block_size
+    shape = tuple(x.shape)
+    assert -len(shape) <= block_dim < len(shape)
+    rows = x.flatten().reshape(-1, B)  # :41-45
+    blocks = _move_block_dim_last_and_flatten(x, block_dim).flatten().reshape(-1, B)  # :58-65
+    dt = blocks.dtype
+    pct = torch.tensor(CLIP_PERCENTILES, dtype=torch.float32)
+    mx = blocks.abs().to(torch.float32).quantile(pct, dim=1, keepdim=True).to(dt)  # :68-73  [11, n_blocks, 1]
+    mx = mx.clamp(min=torch.finfo(dt).tiny)  # :76
+    scale = mx.log2().ceil()  # :77
+    bias = 2 ** (scale_bits - 1) - 1
+    mant = (blocks / 2**scale) * 2 ** (element_bits - 1)  # :79-80, broadcast to [11, n_blocks, B]
+    scale = (scale + bias).clamp(min=0, max=2**scale_bits - 1)  # :81-82
+    mant = mant.round().clamp(min=-(2 ** (element_bits - 1)), max=2 ** (element_bits - 1) - 1)  # :83-86
+    cand = mant / 2 ** (element_bits - 1) * 2 ** (scale - bias)  # :88-90
+    err = torch.norm(cand - rows, p=2, dim=-1)  # :97
+    pick = torch.argmin(err, dim=0).reshape(-1)  # :98
+    chosen = cand[pick, torch.arange(cand.shape[1])]  # :132
+    out = _restore_from_flat(chosen, shape, block_dim).to(x.dtype)  # :141-143
+    return out, pick, err, cand
 
 
 # ----------------------------------------------------------------------------------------------
@@ -189,8 +222,8 @@ _LEGAL_MXFP = ((4, 3), (5, 2), (2, 3), (3, 2), (2, 1), (1, 2))  # mxfp/meta.py:4
 
 
 def mxfp_components(flat: Tensor, block_size: int, exp_bits: int, frac_bits: int, scale_exp_bits: int = 8,
-                    is_finite: bool = True, round_mode: str = "rn"):
-    """(scales uint8 [n_blocks,1], element codes uint8 [n_blocks,B]).  mxfp/fake.py:12-72, percentile 1.0."""
+                    is_finite: bool = True, round_mode: str = "rn", percentile: float = 1.0):
+    """(scales uint8 [n_blocks,1], element codes uint8 [n_blocks,B]).  mxfp/fake.py:12-72."""
     assert scale_exp_bits in (8,), f"Invalid scale exponent bits: {scale_exp_bits}."  # meta.py:35-39
     assert (exp_bits, frac_bits) in _LEGAL_MXFP, f"Invalid element exp/frac bits: {(exp_bits, frac_bits)}."
     t = flat.float()
@@ -206,7 +239,7 @@ def mxfp_components(flat: Tensor, block_size: int, exp_bits: int, frac_bits: int
     t = t.flatten().reshape(t.numel() // B, B)
     ftz = (t.view(torch.int32) & 0x7F800000) == 0
     t = torch.where(ftz, 0.0, t)
-    sh = t.abs().quantile(1.0, dim=1, keepdim=True)
+    sh = t.abs().quantile(percentile, dim=1, keepdim=True)
     sh = sh.log2().floor().to(torch.int32)
     sh -= el_hi_unb
     sh = sh.clamp(sc_lo, sc_hi)
@@ -229,9 +262,10 @@ def mxfp_quantizer(
     quantile_search: bool = False,
     dtype: torch.dtype | None = None,
 ) -> Tensor:
-    """mxfp/mxfp.py:187-230 -> MXFPQuantize.forward :154-178 (finite elements, "rn") -> sim :107-115."""
+    """mxfp/mxfp.py:187-230 -> MXFPQuantize.forward :154-178 (finite elements, "rn") -> sim :107-115, or the search
+    branch :40-105 without calibration activations."""
     if quantile_search:
-        raise NotImplementedError("oracle covers the non-search branch only (mxfp.py:107-115)")
+        return mxfp_clip_search(x, block_size, element_exp_bits, element_frac_bits, block_dim, scale_exp_bits, dtype)[0]
     shape = tuple(x.shape)
     assert -len(shape) <= block_dim < len(shape)
     flat = _move_block_dim_last_and_flatten(x, block_dim)
@@ -241,6 +275,50 @@ def mxfp_quantizer(
     mf = minifloat_mx_compose(el.to(torch.uint16), element_exp_bits, element_frac_bits, True, torch.float32)
     deq = (mf * sc_fp).flatten().to(dtype or x.dtype)  # fake.py:102-103
     return _restore_from_flat(deq, shape, block_dim)
+
+
+def mxfp_clip_search(x: Tensor, block_size: int, element_exp_bits: int, element_frac_bits: int, block_dim: int = -1,
+                     scale_exp_bits: int = 8, dtype: torch.dtype | None = None):
+    """The search branch of mxfp_quantizer_sim with act_tensor=None (mxfp/mxfp.py:40-105).
+
+    Returns (dequantized tensor, index of the chosen percentile per block, errors [11, n_blocks], candidates
+    [11, n_blocks, B] dequantized).  The score of a
+    candidate is computed, as there, from the element *codes* as integers and with the power of two in the uint8
+    arithmetic of the scale tensor (:58-63); an incumbent is replaced only by a strictly smaller score (:99-103).
+    """
+    B = block_size
+    shape = tuple(x.shape)
+    assert -len(shape) <= block_dim < len(shape)
+    rows = x.flatten().reshape(-1, B)  # :41-45
+    flat = _move_block_dim_last_and_flatten(x, block_dim)
+    best = torch.full([rows.shape[0]], float("inf"), dtype=x.dtype)  # :46-48
+    best_sc, best_el = mxfp_components(flat, B, element_exp_bits, element_frac_bits, scale_exp_bits, True, "rn", 1.0)
+    pick = torch.zeros(rows.shape[0], dtype=torch.int64)
+    errs, cands = [], []
+    sc_bias = 2 ** (scale_exp_bits - 1) - 1
+
+    def compose(sc, el):  # fake.py:75-104
+        sc_fp = torch.exp2(sc.to(torch.int32) - sc_bias)
+        mf = minifloat_mx_compose(el.to(torch.uint16), element_exp_bits, element_frac_bits, True, torch.float32)
+        return (mf * sc_fp).to(dtype or x.dtype)
+
+    for i, pct in enumerate(CLIP_PERCENTILES):
+        sc, el = mxfp_components(flat, B, element_exp_bits, element_frac_bits, scale_exp_bits, True, "rn", pct)
+        q = el / 2 ** (element_frac_bits - 1) * 2 ** (sc - sc_bias)  # :58-62 (uint8 tensors: sc - bias and 2**() wrap)
+        q = q.to(dtype=rows.dtype)  # :63
+        q -= rows  # :94
+        q.abs_()
+        q.pow_(2)
+        err = torch.sum(q, 1)  # :97
+        errs.append(err)
+        cands.append(compose(sc, el))
+        better = err < best  # :99
+        best[better] = err[better]
+        best_sc[better] = sc[better]
+        best_el[better] = el[better]
+        pick[better] = i
+    deq = compose(best_sc, best_el).flatten()  # :107-113
+    return _restore_from_flat(deq, shape, block_dim), pick, torch.stack(errs), torch.stack(cands)
 
 
 # ----------------------------------------------------------------------------------------------

@@ -78,6 +78,16 @@ def test_entry_points_reject_bad_arguments_without_a_gpu(lib):
     assert lib.mase_gemm_mxfp4_skinny(p, p, 2, p, p, None, p, 4, 4, 128, 0, 0, p, 4096, None) == -5   # activations: e4m3 or e5m2
     assert lib.mase_gemm_mxfp4_skinny(p, p, 0, p, p, None, p, 4, 4, 128, 7, 0, p, 4096, None) == -4
     assert lib.mase_gemm_mxfp4_skinny_workspace_bytes(4, 4, 192) == 0
+    # mase_mxint_clip_search(in, ref, out, choice, numel, dtype, block_size, element_bits, scale_bits, tab, stream)
+    assert lib.mase_mxint_clip_search(p, p, p, None, 64, 0, 16, 8, 8, p, None) == -5     # block size 32 only
+    assert lib.mase_mxint_clip_search(p, p, p, None, 48, 0, 32, 8, 8, p, None) == -2
+    assert lib.mase_mxint_clip_search(p, None, p, None, 64, 0, 32, 8, 8, p, None) == -1
+    assert lib.mase_mxint_clip_search(p, p, p, None, 64, 0, 32, 1, 8, p, None) == -5
+    assert lib.mase_mxint_clip_search(p, p, p, None, 64, 3, 32, 8, 8, p, None) == -4
+    assert lib.mase_mxint_clip_search(p, p, p, None, 0, 0, 32, 8, 8, p, None) == 0
+    assert lib.mase_mxfp_clip_search(p, p, p, None, 64, 0, 32, 3, 3, p, None) == -5      # illegal element format
+    assert lib.mase_mxfp_clip_search(p, p, p, None, 64, 0, 64, 4, 3, p, None) == -5
+    assert lib.mase_mxfp_clip_search(p, p, None, None, 64, 0, 32, 4, 3, p, None) == -1
     assert lib.mase_mxfp_qdq(p, p, None, None, 64, 0, 0, 32, 3, 3, p, None) == -5  # illegal element format
     assert lib.mase_mxfp_qdq(p, p, None, None, 63, 0, 0, 32, 4, 3, p, None) == -2
     assert lib.mase_block_fp_qdq(p, p, 1, 4, 16, 0, 16, 0, 8, 8, -1, 0, p, None, 0, None) == -2
@@ -177,11 +187,13 @@ def test_product_has_no_cpu_path():
     x = torch.randn(4, 32)
     for call in (lambda: Q.mxint_quantizer(x, 32, 8), lambda: Q.mxfp_quantizer(x, 32, 4, 3),
                  lambda: Q.block_fp_quantizer(x, 8, 8, None, [16]), lambda: Q.integer_quantizer(x, 8, 4),
-                 lambda: Q.minifloat_denorm_quantizer(x, 8, 4), lambda: Q.minifloat_ieee_quantizer(x, 8, 4)):
+                 lambda: Q.minifloat_denorm_quantizer(x, 8, 4), lambda: Q.minifloat_ieee_quantizer(x, 8, 4),
+                 lambda: Q.mxint_quantizer(x, 32, 8, quantile_search=True),
+                 lambda: Q.mxfp_quantizer(x, 32, 4, 3, quantile_search=True)):
         with pytest.raises(MaseAmdError):
             call()
-    with pytest.raises(NotImplementedError):
-        Q.mxint_quantizer(x, 32, 8, quantile_search=True)
+    with pytest.raises(NotImplementedError):  # the calibrated (GPTQ) search is not part of the path
+        Q.mxint_quantizer_sim(x, -1, Q.MXIntMeta(block_size=32, scale_bits=8, element_bits=8), act_tensor=x, quantile_search=True)
 
 
 def test_product_does_not_import_the_oracle():

@@ -1,0 +1,183 @@
+"""GPU tests of the clip search (quantile_search=True without calibration activations) against the oracle.
+
+Every block the kernel writes must be, bit for bit, the oracle's candidate of the index the kernel reports; the
+index must be the oracle's except where two candidates' errors agree to within the rounding of the error itself
+(the library's summation order over the 32 squares is not reproduced), and those exceptions must be rare."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from helpers import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+ULP = {torch.float32: 2.0 ** -22, torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10}
+
+
+def search_inputs(seed: int, dtype: torch.dtype, rows: int = 96, cols: int = 256, scale: float = 0.05) -> torch.Tensor:
+    """weight-like rows plus blocks with outliers, many zeros, equal magnitudes, wide ranges and tiny values"""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(rows, cols, generator=g) * scale
+    x[1] *= torch.exp2(torch.randint(-12, 12, (cols,), generator=g).float())          # wide range inside blocks
+    x[2, ::32] *= 50                                                                   # one outlier per block
+    x[3, ::7] *= 9
+    x[4] = torch.where(torch.rand(cols, generator=g) < 0.6, torch.zeros(cols), x[4])   # more than half zeros
+    x[5] = torch.where(torch.rand(cols, generator=g) < 0.97, torch.zeros(cols), x[5])  # almost all zeros
+    x[6] = 0.0
+    x[7] = torch.sign(x[7]) * scale                                                   # equal magnitudes
+    x[8] = torch.exp2(torch.randint(-3, 3, (cols,), generator=g).float()) * scale      # powers of two
+    x[9] *= 2.0 ** -20
+    x[10] *= 2.0 ** 10
+    x[11, :64] = torch.linspace(-1, 1, 64) * scale
+    if dtype != torch.float16:
+        x[12] *= 2.0 ** -100
+        x[13] *= 2.0 ** 60
+        x[14] *= 2.0 ** -120
+    else:
+        x = x.clamp(-60000.0, 60000.0)  # Inf inputs are not specified
+    return x.to(dtype)
+
+
+def check_against_oracle(got, choice, oracle_result, dtype, what, min_agree=0.998):
+    want, pick, err, cand = oracle_result
+    B = cand.shape[-1]
+    nb = cand.shape[1]
+    choice = choice.cpu().long()
+    assert int(choice.max()) <= 10
+    # the block written is the oracle's candidate of the reported index
+    mine = cand[choice, torch.arange(nb)]
+    assert_bits_equal(got, mine.reshape(got.shape).to(dtype), f"{what}: block contents for the reported index")
+    agree = choice == pick
+    rate = float(agree.double().mean())
+    print(f"{what}: same candidate as the oracle in {rate:.5f} of {nb} blocks; histogram {torch.bincount(pick, minlength=11).tolist()}")
+    assert rate >= min_agree
+    if not bool(agree.all()):
+        idx = (~agree).nonzero().flatten()
+        e_mine = err[choice[idx], idx].double()
+        e_ref = err[pick[idx], idx].double()
+        ok = (e_mine - e_ref).abs() <= e_ref.abs() * ULP[dtype] * 2
+        assert bool(ok.all()), (what, idx[~ok][:5].tolist(), e_mine[~ok][:5].tolist(), e_ref[~ok][:5].tolist())
+    else:
+        assert_bits_equal(got, want, what)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("bits", [8, 4, 2, 6])
+def test_mxint_clip_search_matches_the_oracle(dev, dtype, bits):
+    from mase_amd.quantizers import _ops
+
+    x = search_inputs(bits, dtype)
+    print(f"mxint clip search {dtype} bits={bits}", flush=True)
+    got, choice = _ops.mxint_clip_search(x.to(dev), 32, bits, -1, 8, return_choice=True)
+    check_against_oracle(got.cpu(), choice, O.mxint_clip_search(x, 32, bits), dtype, f"mxint{bits} {dtype}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("fmt", [(2, 1), (4, 3), (5, 2), (3, 2), (2, 3), (1, 2)])
+@pytest.mark.parametrize("scale", [0.05, 10.0])
+def test_mxfp_clip_search_matches_the_oracle(dev, dtype, fmt, scale):
+    """the larger scale puts the scale bytes into 127..134, the only range where the reference's score tells candidates
+    apart (elsewhere every candidate scores sum(x^2) and the first one stays)"""
+    from mase_amd.quantizers import _ops
+
+    if scale > 1:
+        scale = scale * 2.0 ** ((1 << fmt[0]) - 1 - ((1 << (fmt[0] - 1)) - 1))  # times 2^(largest element exponent)
+    x = search_inputs(fmt[0] * 8 + fmt[1], dtype, scale=scale)
+    print(f"mxfp clip search {dtype} e{fmt[0]}m{fmt[1]} scale={scale}", flush=True)
+    got, choice = _ops.mxfp_clip_search(x.to(dev), 32, fmt[0], fmt[1], -1, 8, return_choice=True)
+    ref = O.mxfp_clip_search(x, 32, fmt[0], fmt[1])
+    check_against_oracle(got.cpu(), choice, ref, dtype, f"mxfp e{fmt[0]}m{fmt[1]} {dtype} x{scale}")
+    if scale > 1 and dtype != torch.float16:
+        assert int((ref[1] != 0).sum()) > 50  # the case does exercise the other candidates
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_clip_search_along_the_first_dimension(dev, dtype):
+    """block_dim = 0: candidates are blocks along dim 0, the error is taken against the blocks of the plain flattening"""
+    from mase_amd.quantizers import _ops
+
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(64, 48, generator=g) * 0.1).to(dtype)
+    got, choice = _ops.mxint_clip_search(x.to(dev), 32, 4, 0, 8, return_choice=True)
+    want, pick, err, cand = O.mxint_clip_search(x, 32, 4, 0)
+    flat = got.cpu().movedim(0, -1).reshape(-1, 32)
+    check_against_oracle(flat, choice, (want.movedim(0, -1).reshape(-1, 32), pick, err, cand), dtype, f"mxint4 dim0 {dtype}")
+    got, choice = _ops.mxfp_clip_search((x * 300).to(dev), 32, 2, 1, 0, 8, return_choice=True)
+    want, pick, err, cand = O.mxfp_clip_search(x * 300, 32, 2, 1, 0)
+    flat = got.cpu().movedim(0, -1).reshape(-1, 32)
+    check_against_oracle(flat, choice, (want.movedim(0, -1).reshape(-1, 32), pick, err, cand), dtype, f"mxfp4 dim0 {dtype}")
+
+
+def test_quantizer_entry_points_take_the_search_branch(dev):
+    from mase_amd.quantizers import MXFPMeta, MXIntMeta, mxfp_quantizer, mxfp_quantizer_sim, mxint_quantizer, mxint_quantizer_sim
+
+    x = search_inputs(3, torch.bfloat16)
+    xd = x.to(dev)
+    got = mxint_quantizer(xd, 32, 4, quantile_search=True)
+    plain = mxint_quantizer(xd, 32, 4)
+    assert not torch.equal(got, plain)
+    assert torch.equal(got, mxint_quantizer_sim(xd, -1, MXIntMeta(block_size=32, scale_bits=8, element_bits=4), quantile_search=True))
+    want = O.mxint_quantizer(x, 32, 4, quantile_search=True)
+    assert float((got.cpu() == want).float().mean()) > 0.995
+    # the searched result is never worse than the plain one by the reference's own measure, block by block
+    e_s = (got.float() - xd.float()).reshape(-1, 32).norm(dim=1)
+    e_p = (plain.float() - xd.float()).reshape(-1, 32).norm(dim=1)
+    assert bool((e_s <= e_p * (1 + 2.0 ** -6)).all())
+    big = (x.float() * 800).to(torch.bfloat16)
+    got = mxfp_quantizer(big.to(dev), 32, 2, 1, quantile_search=True)
+    want = O.mxfp_quantizer(big, 32, 2, 1, quantile_search=True)
+    same = (got.cpu() == want) | (got.cpu().isnan() & want.isnan())
+    assert float(same.float().mean()) > 0.995
+    meta = MXFPMeta(block_size=32, scale_exp_bits=8, element_exp_bits=2, element_frac_bits=1, element_is_finite=True,
+                    round_mode="rn")
+    assert_bits_equal(mxfp_quantizer_sim(big.to(dev), -1, meta, quantile_search=True), got, "sim entry point")
+    with pytest.raises(NotImplementedError):
+        mxint_quantizer_sim(xd, -1, MXIntMeta(block_size=32, scale_bits=8, element_bits=4), act_tensor=xd, quantile_search=True)
+    with pytest.raises(NotImplementedError):
+        mxint_quantizer(xd, 16, 4, quantile_search=True)
+    # straight-through gradient as for the plain quantizer
+    xr = xd.float().clone().requires_grad_(True)
+    mxint_quantizer(xr, 32, 4, quantile_search=True).sum().backward()
+    assert torch.equal(xr.grad, torch.ones_like(xr))
+
+
+def test_linear_mxint_clip_search_config(dev):
+    """LinearMXInt with config["clip_search"]: the weight is quantized with the search when the state dict is loaded
+    (nn/quantized/modules/linear.py:916-954)"""
+    from mase_amd.quantized.modules.linear import LinearMXInt
+
+    cfg = {"weight_block_size": 32, "weight_width": 4, "data_in_block_size": 32, "data_in_width": 8,
+           "bias_block_size": 32, "bias_width": 8, "clip_search": True}
+    g = torch.Generator().manual_seed(2)
+    w = torch.randn(64, 128, generator=g) * 0.05
+    w[:, ::32] *= 6
+    b = torch.randn(64, generator=g)
+    m = LinearMXInt(128, 64, bias=True, config=cfg, device=dev, dtype=torch.bfloat16)
+    m.load_state_dict({"weight": w.to(torch.bfloat16), "bias": b.to(torch.bfloat16)})
+    want_w = O.mxint_quantizer(w.to(torch.bfloat16), 32, 4, 1, quantile_search=True)
+    want_b = O.mxint_quantizer(b.to(torch.bfloat16), 32, 8, 0, quantile_search=True)
+    assert float((m.weight.detach().cpu() == want_w).float().mean()) > 0.995
+    assert float((m.bias.detach().cpu() == want_b).float().mean()) > 0.98
+    plain = LinearMXInt(128, 64, bias=True, config={**cfg, "clip_search": False}, device=dev, dtype=torch.bfloat16)
+    plain.load_state_dict({"weight": w.to(torch.bfloat16), "bias": b.to(torch.bfloat16)})
+    assert not torch.equal(plain.weight, m.weight)
+    x = torch.randn(8, 128, generator=g).to(torch.bfloat16).to(dev)
+    y = m(x)
+    ref = O.linear_mxint_forward(x.cpu(), m.weight.detach().cpu(), m.bias.detach().cpu(), cfg)
+    assert float((y.cpu().float() - ref.float()).abs().max() / ref.float().abs().max()) < 1e-2
+
+
+def test_clip_search_on_a_weight_sized_tensor(dev):
+    """131072 blocks of a weight-like bf16 tensor: agreement with the oracle's choice where the summation order of the
+    32 squares could matter"""
+    from mase_amd.quantizers import _ops
+
+    g = torch.Generator().manual_seed(9)
+    x = (torch.randn(1024, 4096, generator=g) * 0.02).to(torch.bfloat16)
+    got, choice = _ops.mxint_clip_search(x.to(dev), 32, 4, -1, 8, return_choice=True)
+    check_against_oracle(got.cpu(), choice, O.mxint_clip_search(x, 32, 4), torch.bfloat16, "mxint4 bf16 [1024,4096]", 0.9995)
+    xf = x.float() * 1000
+    got, choice = _ops.mxfp_clip_search(xf.to(dev), 32, 2, 1, -1, 8, return_choice=True)
+    check_against_oracle(got.cpu(), choice, O.mxfp_clip_search(xf, 32, 2, 1), torch.float32, "mxfp4 f32 [1024,4096]", 0.9995)

@@ -324,3 +324,98 @@ def test_linear_forwards_are_f_linear_of_quantized_operands():
     y = OL.linear_mxint_forward(x, qw, qb, cfg)
     assert torch.equal(y, torch.nn.functional.linear(O.mxint_quantizer(x, 32, 8), qw, b))
     assert torch.equal(OL.linear_mxint_forward(x, qw, qb, {**cfg, "bypass": True}), torch.nn.functional.linear(x, qw, b))
+
+
+# ------------------------------------------------------------------------------------------------
+# clip search (quantile_search=True without calibration activations)
+# ------------------------------------------------------------------------------------------------
+def _exact_quantile(sorted_vals, q: float):
+    """the library's linear interpolation as the kernels restate it: fp32 rank and weight, one fused multiply-add"""
+    n = len(sorted_vals)
+    rank = np.float32(q) * np.float32(n - 1)
+    lo = int(math.floor(rank))
+    hi = int(math.ceil(rank))
+    w = np.float32(rank - np.float32(lo))
+    a, b = Fraction(float(sorted_vals[lo])), Fraction(float(sorted_vals[hi]))
+    diff = Fraction(float(np.float32(float(b - a))))  # b - a rounded to fp32
+    if w < 0.5:
+        exact = Fraction(float(w)) * diff + a
+    else:
+        exact = Fraction(float(np.float32(w - np.float32(1)))) * diff + b
+    # one rounding of the exact result to fp32 (float() of a Fraction rounds correctly to double first, which is
+    # harmless here only if the double is not a tie of fp32: compare in rationals instead)
+    lo32 = np.float32(float(exact))
+    cands = [lo32, np.nextafter(lo32, np.float32(np.inf)), np.nextafter(lo32, np.float32(-np.inf))]
+    return min(cands, key=lambda c: (abs(Fraction(float(c)) - exact), int(np.float32(c).view(np.uint32)) & 1))
+
+
+def test_library_quantile_is_the_fused_interpolation():
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(40, 32, generator=g).abs() * torch.exp2(torch.randint(-20, 20, (40, 1), generator=g).float())
+    got = x.quantile(torch.tensor(O.CLIP_PERCENTILES, dtype=torch.float32), dim=1)  # [11, 40]
+    s = x.sort(dim=1).values.numpy()
+    for i, q in enumerate(O.CLIP_PERCENTILES):
+        for r in range(x.shape[0]):
+            assert np.float32(got[i, r].item()) == _exact_quantile(s[r], q), (q, r)
+    assert torch.equal(x.quantile(0.93, dim=1), got[5])  # the scalar overload used by the MXFP extraction
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_mxint_clip_search_picks_the_candidate_with_the_smallest_exact_error(bits):
+    g = torch.Generator().manual_seed(bits)
+    x = torch.randn(24, 32, generator=g) * 0.1
+    x[::3, 0] = 0.2505  # a maximum just above a power of two: clipping it costs little, the finer scale gains more
+    out, pick, err, cand = O.mxint_clip_search(x, 32, bits)
+    assert cand.shape == (11, 24, 32) and err.shape == (11, 24)
+    assert torch.equal(cand[0].reshape(x.shape), O.mxint_quantizer(x, 32, bits))  # percentile 1.0 is the plain quantizer
+    assert torch.equal(out, cand[pick, torch.arange(24)].reshape(x.shape))
+    assert int((pick != 0).sum()) >= (4 if bits == 4 else 1)
+    s = x.abs().sort(dim=1).values.numpy()
+    for r in range(24):
+        xs = [float(v) for v in x[r]]
+        exact = []
+        for i, q in enumerate(O.CLIP_PERCENTILES):
+            mx = max(float(_exact_quantile(s[r], q)), float(torch.finfo(torch.float32).tiny))
+            k, is_pow2 = exact_log2_parts(mx)
+            if not is_pow2:
+                if not far_from_pow2(mx):
+                    break
+                k += 1
+            ys = S.mxint_block(xs, k, bits)
+            assert [float(y) for y in ys] == cand[i, r].tolist(), (r, i)
+            exact.append(sum((y - Fraction(v)) ** 2 for y, v in zip(ys, xs)))
+        else:
+            best = min(exact)
+            first = exact.index(best)
+            chosen = exact[int(pick[r])]
+            assert chosen <= best * (1 + Fraction(1, 1 << 20)), (r, int(pick[r]), first)
+            if all(e == best or e > best * (1 + Fraction(1, 1 << 18)) for e in exact):
+                assert int(pick[r]) == first  # no near-tie: the first minimum, as argmin returns it
+
+
+def test_mxfp_clip_search_score_is_on_the_integer_codes():
+    """mxfp/mxfp.py:58-62: the score compares x with code / 2^(F-1) * (2^(scale-127) in uint8 arithmetic)"""
+    g = torch.Generator().manual_seed(4)
+    E, F = 2, 1
+    x = torch.randn(16, 32, generator=g) * 30
+    x[:, 0] = 100.0  # scale byte 127 + 6 - 2 = 131 for percentile 1.0
+    x[5:8] *= 2.0 ** -10  # scale bytes below 127: every candidate scores sum(x^2)
+    out, pick, err, cand = O.mxfp_clip_search(x, 32, E, F)
+    assert torch.equal(cand[0].reshape(x.shape), O.mxfp_quantizer(x, 32, E, F))
+    assert torch.equal(out, cand[pick, torch.arange(16)].reshape(x.shape))
+    assert bool((pick[5:8] == 0).all()) and int((pick != 0).sum()) >= 4
+    flat = x.reshape(-1)
+    for i, q in enumerate(O.CLIP_PERCENTILES):
+        sc, el = O.mxfp_components(flat, 32, E, F, percentile=q)
+        for r in range(16):
+            s = int(sc[r, 0])
+            pw = (1 << (s - 127)) if 127 <= s <= 134 else 0
+            score = sum((Fraction(int(c)) * pw - Fraction(float(v))) ** 2 for c, v in zip(el[r].tolist(), x[r].tolist()))
+            assert abs(float(err[i, r]) - float(score)) <= float(score) * 1e-5 + 1e-30, (i, r)
+    # the winner is the first strictly smaller score
+    for r in range(16):
+        best, who = float("inf"), 0
+        for i in range(11):
+            if float(err[i, r]) < best:
+                best, who = float(err[i, r]), i
+        assert int(pick[r]) == who
