@@ -419,3 +419,50 @@ def test_mxfp_clip_search_score_is_on_the_integer_codes():
             if float(err[i, r]) < best:
                 best, who = float(err[i, r]), i
         assert int(pick[r]) == who
+
+
+# ------------------------------------------------------------------------------------------------
+# GPTQ
+# ------------------------------------------------------------------------------------------------
+def _correlated_inputs(g, n, tokens, cols):
+    mix = torch.randn(cols, cols, generator=g) * 0.3 + torch.eye(cols)
+    return [torch.randn(2, tokens, cols, generator=g) @ mix for _ in range(n)]
+
+
+def test_gptq_hessian_and_inverse_factor():
+    from oracle import gptq as G
+
+    g = torch.Generator().manual_seed(0)
+    xs = _correlated_inputs(g, 3, 40, 64)
+    H = G.hessian(xs)
+    flat = torch.cat([x.reshape(-1, 64) for x in xs]).double()
+    want = 2.0 / 6 * flat.t() @ flat  # n counts batch items (6), not tokens: gptq.py:31-36
+    assert float((H.double() - want).abs().max() / want.abs().max()) < 1e-5
+    U, dead = G.inverse_factor(H)
+    assert not bool(dead.any()) and bool((U.tril(-1) == 0).all())
+    damped = H.double() + 0.01 * H.diag().double().mean() * torch.eye(64, dtype=torch.float64)
+    assert float(((U.double().t() @ U.double()) @ damped - torch.eye(64, dtype=torch.float64)).abs().max()) < 1e-3
+
+
+@pytest.mark.parametrize("fmt,cfg", [("mxint", {"weight_block_size": 32, "weight_width": 4}),
+                                     ("mxfp", {"weight_block_size": 32, "weight_exponent_width": 2, "weight_frac_width": 1})])
+def test_gptq_feedback_lowers_the_proxy_loss(fmt, cfg):
+    from oracle import gptq as G
+
+    g = torch.Generator().manual_seed(1)
+    W = torch.randn(48, 128, generator=g) * 0.05
+    # uncorrelated inputs: nothing to feed back, the result is the plain clip-search quantization group by group
+    Hd = torch.diag(torch.rand(128, generator=g) + 0.5)
+    Q = G.fasterquant(W, Hd, fmt, cfg)
+    assert torch.equal(Q, G.quantize_group(W, fmt, cfg, True))
+    # correlated inputs: the error feedback must pay off on the calibration data
+    H = G.hessian(_correlated_inputs(g, 4, 64, 128))
+    Q = G.fasterquant(W, H, fmt, cfg)
+    rtn = G.quantize_group(W, fmt, cfg, True)
+    assert not torch.equal(Q, rtn)
+    assert G.proxy_loss(W, Q, H) < 0.9 * G.proxy_loss(W, rtn, H)
+    # a dead column (never active in calibration) is zeroed before quantization (gptq.py:67-69)
+    H2 = H.clone()
+    H2[5, :] = 0
+    H2[:, 5] = 0
+    assert bool((G.fasterquant(W, H2, fmt, cfg)[:, 5] == 0).all())
