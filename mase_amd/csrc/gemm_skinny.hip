@@ -388,6 +388,136 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_mxfp4_partial_kern
   }
 }
 
+// The same product with the activation codes of the work-group's K range resident in LDS.  The kernel above copies
+// the activation chunk once per wavefront and chunk, which doubles its copy instructions, and reads the weight rows in
+// 64-byte pieces.  Here the work-group first copies its [rows, kc] slab of activation codes and scales into LDS (shared
+// by the 4 wavefronts, one barrier), and the per-wavefront rings carry weights only, in chunks of 256 elements of K
+// (128 bytes per weight row, 5 copies per 4 KB).  LDS: slab rows*kc + kc bytes, rings 4 x kSlabStages x 4352 bytes;
+// the host picks the number of K ranges so that this fits.  K % 256 == 0.
+// Slab layout: [chunk][row][256 B] with the 16-byte granule j of a row stored at position j ^ (row & 15), so that the
+// 16 lanes a ds_read_b128 serves together (16 rows, same granule) fall into different banks; scales [chunk][32][8 B].
+constexpr int kSlabStages = 5, kSlabStageBytes = 4096 + 256, kSlabCopies = 5;
+constexpr int kSlabRingBytes = 4 * kSlabStages * kSlabStageBytes;
+constexpr int kSlabLdsMax = 160 * 1024;
+
+template <int XC, int CBSZ>
+__global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_mxfp4_slab_kernel(SkinnyFParams p) {
+  constexpr int XR = 8 * XC, S = kSlabStages;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  const int r = lane & 31, g = lane >> 5;
+  const int n0 = ((int)blockIdx.x * 4 + wave) * 32;  // rows beyond N are clamped: every wavefront reaches the barrier
+  const int ks = blockIdx.y;
+  const int nch = p.kc / 256;
+  const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)lds;
+  const uint32_t xcodes_addr = lds_addr, xscales_addr = lds_addr + (uint32_t)(XR * p.kc);
+  const unsigned char* xcodes = lds;
+  const unsigned char* xscales = lds + XR * p.kc;
+  unsigned char* ring = lds + XR * p.kc + p.kc + wave * (S * kSlabStageBytes);
+  const uint32_t ring_addr = xscales_addr + (uint32_t)p.kc + (uint32_t)(wave * (S * kSlabStageBytes));
+
+  // activation slab: copy t moves rows 4q .. 4q+3 of chunk c (t = c * (XR/4) + q); lane -> row 4q + lane/16, slot lane%16
+  {
+    const unsigned char* xbase = p.Xc + (size_t)ks * p.kc;
+    const int total = nch * (XR / 4);
+    for (int t0 = 0; t0 < total; t0 += 4) {
+      const int t = min(t0 + wave, total - 1);
+      const int c = t / (XR / 4), q = t % (XR / 4);
+      const int row = 4 * q + (lane >> 4);
+      const int gran = (lane & 15) ^ (row & 15);
+      const uint32_t off = (uint32_t)((size_t)min(row, p.M - 1) * (size_t)p.K) + (uint32_t)(gran * 16);
+      sk_async_copy(xbase + (size_t)c * 256, off, xcodes_addr + (uint32_t)(c * (XR * 256) + q * 1024));
+    }
+    const unsigned char* xsbase = p.Xs + (size_t)ks * (p.kc / 32);
+    const uint32_t offs = (uint32_t)((size_t)min(lane >> 1, p.M - 1) * (size_t)(p.K / 32)) + (uint32_t)((lane & 1) * 4);
+    for (int c0 = 0; c0 < nch; c0 += 4) {
+      const int c = min(c0 + wave, nch - 1);
+      sk_async_copy4(xsbase + (size_t)c * 8, offs, xscales_addr + (uint32_t)(c * 256));
+    }
+  }
+  // weights: copy j (0..3) moves rows 8j .. 8j+7 (128 bytes per row per chunk); scales: lane -> row lane/2, dword lane%2
+  uint32_t offw[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = 8 * j + (lane >> 3);
+    const int gran = (lane & 7) ^ ((row >> 1) & 7);
+    offw[j] = (uint32_t)((size_t)min(n0 + row, p.N - 1) * (size_t)(p.K / 2)) + (uint32_t)(gran * 16);
+  }
+  const uint32_t offws = (uint32_t)((size_t)min(n0 + (lane >> 1), p.N - 1) * (size_t)(p.K / 32)) + (uint32_t)((lane & 1) * 4);
+  const unsigned char* wbase = p.Wc + (size_t)ks * (p.kc / 2);
+  const unsigned char* wsbase = p.Ws + (size_t)ks * (p.kc / 32);
+  auto issue = [&](int c) __attribute__((always_inline)) {  // chunk c (clamped: past the end re-copies the last chunk)
+    const int cc = min(c, nch - 1);
+    const uint32_t st = ring_addr + (uint32_t)((c % S) * kSlabStageBytes);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sk_async_copy(wbase + (size_t)cc * 128, offw[j], st + j * 1024);
+    sk_async_copy4(wsbase + (size_t)cc * 8, offws, st + 4096);
+  };
+  f32x16_t acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+  for (int c = 0; c < S - 1; ++c) issue(c);
+  // the slab's copies are older than the ring's: with at most the ring's in flight, this wavefront's part of the slab has
+  // landed; the barrier makes the other wavefronts' parts visible
+  sk_wait_vmcnt<(S - 1) * kSlabCopies>();
+  __builtin_amdgcn_s_barrier();
+  const int xrow = min(r, XR - 1);
+  const int xsw = xrow & 15, wsw = (r >> 1) & 7;
+  for (int c = 0; c < nch; ++c) {
+    issue(c + S - 1);
+    sk_wait_vmcnt<(S - 1) * kSlabCopies>();  // chunk c has landed; the later ones may be in flight
+    const unsigned char* st = ring + (c % S) * kSlabStageBytes;
+    const unsigned char* xc = xcodes + c * (XR * 256) + xrow * 256;
+    const uint2 swv = *(const uint2*)(st + 4096 + r * 8);
+    const uint2 sxv = *(const uint2*)(xscales + c * 256 + xrow * 8);
+#pragma unroll
+    for (int step = 0; step < 4; ++step) {
+      const uint4 x0 = *(const uint4*)(xc + (((step * 4 + g) ^ xsw) << 4));
+      const uint4 x1 = *(const uint4*)(xc + (((step * 4 + 2 + g) ^ xsw) << 4));
+      const uint4 w0 = *(const uint4*)(st + r * 128 + (((step * 2 + g) ^ wsw) << 4));
+      const int sw = (int)((step < 2 ? swv.x : swv.y) >> (8 * g));
+      const int sx = (int)((step < 2 ? sxv.x : sxv.y) >> (8 * g));
+      i32x8_t a, b;
+      a[0] = (int)x0.x; a[1] = (int)x0.y; a[2] = (int)x0.z; a[3] = (int)x0.w;
+      a[4] = (int)x1.x; a[5] = (int)x1.y; a[6] = (int)x1.z; a[7] = (int)x1.w;
+      b[0] = (int)w0.x; b[1] = (int)w0.y; b[2] = (int)w0.z; b[3] = (int)w0.w;
+      b[4] = 0; b[5] = 0; b[6] = 0; b[7] = 0;
+      if ((step & 1) == 0) acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc, CBSZ, 4, 0, sx, 0, sw);
+      else acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc, CBSZ, 4, 2, sx, 2, sw);
+    }
+  }
+  sk_wait_vmcnt<0>();  // no copy may still be in flight towards LDS when the wavefront retires
+  // acc[q*4 + j] = C[token q*8 + g*4 + j][weight row n0 + r]
+  float* out = p.P + (size_t)ks * p.M * p.N;
+  const int n = n0 + r;
+  if (n < p.N) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int m = q * 8 + g * 4 + j;
+        if (m < p.M) out[(size_t)m * p.N + n] = acc[q * 4 + j];
+      }
+  }
+}
+
+int skinny_splits(int M, int N, int K, int n_cu);
+
+// K ranges of the slab kernel: at least as many as the LDS needs (slab rows * kc + kc <= 160 KB - rings), then as many
+// as skinny_splits would take; each a whole number of 256-element chunks
+int slab_splits(int rows8, int M, int N, int K, int n_cu) {
+  const int chunks = K / 256;
+  const int kc_max = ((kSlabLdsMax - kSlabRingBytes) / (rows8 + 1)) / 256 * 256;
+  int want = skinny_splits(M, N, K / 2, n_cu);
+  for (int s = 1; s <= chunks; ++s) {
+    if (chunks % s != 0) continue;
+    if (K / s <= kc_max && s >= want) return s;
+  }
+  return chunks;
+}
+
 __device__ __forceinline__ float skinny_bias(const void* bias, int dt, int col) {
   if (dt == MASE_DT_F32) return ((const float*)bias)[col];
   if (dt == MASE_DT_BF16) return bits2f((uint32_t)((const uint16_t*)bias)[col] << 16);
@@ -577,12 +707,25 @@ extern "C" int mase_gemm_mxint8_skinny(const void* A, const int8_t* B_codes, con
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
 
+namespace mase {
+namespace {
+// K % 256 == 0 takes the slab kernel (the same number of K ranges for every pass of 32 rows), other K the ring-only one
+int mxfp4_skinny_splits(size_t M, size_t N, size_t K, int n_cu) {
+  if (K % 256 == 0) {
+    const int rows = (int)(M < 32 ? M : 32);
+    return slab_splits((rows + 7) / 8 * 8, (int)M, (int)N, (int)K, n_cu);
+  }
+  return skinny_splits((int)M, (int)N, (int)(K / 2), n_cu);
+}
+}  // namespace
+}  // namespace mase
+
 extern "C" size_t mase_gemm_mxfp4_skinny_workspace_bytes(size_t M, size_t N, size_t K) {
   using namespace mase;
   if (M == 0 || N == 0 || K == 0 || (K % 128) != 0 || M > 128) return 0;
   const int n_cu = skinny_cu_count();
   if (n_cu <= 0) return 0;
-  return (size_t)skinny_splits((int)M, (int)N, (int)(K / 2), n_cu) * M * N * sizeof(float);
+  return (size_t)mxfp4_skinny_splits(M, N, K, n_cu) * M * N * sizeof(float);
 }
 
 extern "C" int mase_gemm_mxfp4_skinny(const void* A_codes, const void* A_scales, int a_format, const void* B_codes,
@@ -600,12 +743,20 @@ extern "C" int mase_gemm_mxfp4_skinny(const void* A_codes, const void* A_scales,
   if (out_dtype < 0 || out_dtype > 2 || (bias != nullptr && (bias_dtype < 0 || bias_dtype > 2))) return MASE_ERR_DTYPE;
   const int n_cu = skinny_cu_count();
   if (n_cu <= 0) return MASE_ERR_LAUNCH;
-  const int splits = skinny_splits((int)M, (int)N, (int)(K / 2), n_cu);
+  const int splits = mxfp4_skinny_splits(M, N, K, n_cu);
+  const bool slab = (K % 256) == 0;
   const size_t need = (size_t)splits * M * N * sizeof(float);
   if (workspace == nullptr || workspace_bytes < need || (((uintptr_t)workspace) & 15u) != 0) return MASE_ERR_WORKSPACE;
   hipStream_t st = (hipStream_t)stream;
   static bool attr_set = false;
   if (!attr_set) {
+    const void* sl[8] = {(const void*)gemm_skinny_mxfp4_slab_kernel<1, 0>, (const void*)gemm_skinny_mxfp4_slab_kernel<2, 0>,
+                         (const void*)gemm_skinny_mxfp4_slab_kernel<3, 0>, (const void*)gemm_skinny_mxfp4_slab_kernel<4, 0>,
+                         (const void*)gemm_skinny_mxfp4_slab_kernel<1, 1>, (const void*)gemm_skinny_mxfp4_slab_kernel<2, 1>,
+                         (const void*)gemm_skinny_mxfp4_slab_kernel<3, 1>, (const void*)gemm_skinny_mxfp4_slab_kernel<4, 1>};
+    for (int i = 0; i < 8; ++i)
+      if (hipFuncSetAttribute(sl[i], hipFuncAttributeMaxDynamicSharedMemorySize, kSlabLdsMax) != hipSuccess)
+        return MASE_ERR_LAUNCH;
     const void* ks[8] = {(const void*)gemm_skinny_mxfp4_partial_kernel<1, 0>, (const void*)gemm_skinny_mxfp4_partial_kernel<2, 0>,
                          (const void*)gemm_skinny_mxfp4_partial_kernel<3, 0>, (const void*)gemm_skinny_mxfp4_partial_kernel<4, 0>,
                          (const void*)gemm_skinny_mxfp4_partial_kernel<1, 1>, (const void*)gemm_skinny_mxfp4_partial_kernel<2, 1>,
@@ -630,10 +781,17 @@ extern "C" int mase_gemm_mxfp4_skinny(const void* A_codes, const void* A_scales,
     p.P = (float*)workspace + (size_t)splits * m0 * N;
     p.M = (int)rows;
     const int xc = (int)(rows + 7) / 8;
+    const unsigned slab_lds = (unsigned)(8 * xc * p.kc + p.kc + kSlabRingBytes);
 #define MASE_SF_LAUNCH(XC_)                                                                                           \
   do {                                                                                                                \
-    if (a_format == 0) hipLaunchKernelGGL((gemm_skinny_mxfp4_partial_kernel<XC_, 0>), grid, block, SfGeom<XC_>::kLdsBytes, st, p); \
-    else hipLaunchKernelGGL((gemm_skinny_mxfp4_partial_kernel<XC_, 1>), grid, block, SfGeom<XC_>::kLdsBytes, st, p);  \
+    if (slab) {                                                                                                       \
+      if (a_format == 0) hipLaunchKernelGGL((gemm_skinny_mxfp4_slab_kernel<XC_, 0>), grid, block, slab_lds, st, p);   \
+      else hipLaunchKernelGGL((gemm_skinny_mxfp4_slab_kernel<XC_, 1>), grid, block, slab_lds, st, p);                 \
+    } else if (a_format == 0) {                                                                                       \
+      hipLaunchKernelGGL((gemm_skinny_mxfp4_partial_kernel<XC_, 0>), grid, block, SfGeom<XC_>::kLdsBytes, st, p);     \
+    } else {                                                                                                          \
+      hipLaunchKernelGGL((gemm_skinny_mxfp4_partial_kernel<XC_, 1>), grid, block, SfGeom<XC_>::kLdsBytes, st, p);     \
+    }                                                                                                                 \
   } while (0)
     if (xc == 1) MASE_SF_LAUNCH(1);
     else if (xc == 2) MASE_SF_LAUNCH(2);
