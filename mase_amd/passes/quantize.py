@@ -7,8 +7,8 @@ Like the reference it pops ``"by"`` (and ``"gptq"``) from ``pass_args`` and ``"n
 (:28, :48, :140), instantiates ``quantized_module_map["linear_<name>"]`` with the original module's shape, bias,
 device and dtype (``module_modify_helper.py:149-176``), hands the weights over with
 ``load_state_dict(deepcopy(state_dict), strict=False)`` (:103-114) and swaps the module in by name (:137-141).
-``nn.Embedding`` targets (:191-216) and Llama attention / MLP / RMSNorm targets (:264-275, selected by name or
-regex with a ``llama_self_attention_* / llama_mlp_* / llama_rms_norm_*`` entry of the registry) are handled the same
+``nn.Embedding`` targets (:191-216) and Llama / Qwen3 attention / MLP / RMSNorm targets (:264-275, selected by name or
+regex with a ``llama_* / qwen3_*`` ``self_attention_* / mlp_* / rms_norm_*`` entry of the registry) are handled the same
 way; the Llama replacements receive ``config=network.config`` like the reference's (quantize.py:52-56, 82-86).  A
 module counts as a Llama attention / MLP / RMSNorm when a class of that name is among its bases, so that the
 ``transformers`` classes match without being imported here.  A ``"gptq"`` entry runs ``mase_amd.passes.gptq.run_gptq``
@@ -46,7 +46,8 @@ def _instantiate_embedding(module, postfix, module_map, additional_module_args):
     return embedding_cls(**kwargs, **additional_module_args)
 
 
-_LLAMA_PREFIX = {"LlamaAttention": "llama_self_attention", "LlamaMLP": "llama_mlp", "LlamaRMSNorm": "llama_rms_norm"}
+_LLAMA_PREFIX = {"LlamaAttention": "llama_self_attention", "LlamaMLP": "llama_mlp", "LlamaRMSNorm": "llama_rms_norm",
+                 "Qwen3Attention": "qwen3_self_attention", "Qwen3MLP": "qwen3_mlp", "Qwen3RMSNorm": "qwen3_rms_norm"}
 
 
 def _llama_prefix(module):

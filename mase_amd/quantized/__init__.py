@@ -14,5 +14,10 @@ from .modules import (  # noqa: F401
     LlamaMLPMXFP,
     LlamaMLPMXInt,
     LlamaRMSNormMinifloat,
+    Qwen3AttentionMXFP,
+    Qwen3AttentionMXInt,
+    Qwen3MLPMXFP,
+    Qwen3MLPMXInt,
+    Qwen3RMSNormMinifloat,
     quantized_module_map,
 )

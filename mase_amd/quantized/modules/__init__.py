@@ -1,5 +1,5 @@
 """``quantized_module_map``: the in-scope entries of the reference's registry
-(``chop/nn/quantized/modules/__init__.py:236-251, 334-335, 352-360, 388-408``), same keys."""
+(``chop/nn/quantized/modules/__init__.py:236-251, 334-335, 352-369, 388-408``), same keys."""
 from .embedding import EmbeddingMXFP, EmbeddingMXInt
 from .llama import (
     LlamaAttentionMXFP,
@@ -8,6 +8,14 @@ from .llama import (
     LlamaMLPMXInt,
     LlamaRMSNormMinifloat,
     quantized_llama_module_map,
+)
+from .qwen3 import (
+    Qwen3AttentionMXFP,
+    Qwen3AttentionMXInt,
+    Qwen3MLPMXFP,
+    Qwen3MLPMXInt,
+    Qwen3RMSNormMinifloat,
+    quantized_qwen3_module_map,
 )
 from .linear import (
     LinearBlockFP,
@@ -28,4 +36,4 @@ quantized_module_map = {
     "linear_mxfp": LinearMXFP,
     "embedding_mxint": EmbeddingMXInt,
     "embedding_mxfp": EmbeddingMXFP,
-} | quantized_llama_module_map
+} | quantized_llama_module_map | quantized_qwen3_module_map

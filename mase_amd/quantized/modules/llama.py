@@ -151,9 +151,7 @@ class _LlamaAttentionMX(nn.Module):
                 attention_mask: Optional[Tensor], past_key_value=None, cache_position=None, **kwargs):
         input_shape = hidden_states.shape[:-1]
         hidden_shape = (*input_shape, -1, self.head_dim)
-        query_states = self.q_proj(hidden_states).view(hidden_shape).transpose(1, 2)
-        key_states = self.k_proj(hidden_states).view(hidden_shape).transpose(1, 2)
-        value_states = self.v_proj(hidden_states).view(hidden_shape).transpose(1, 2)
+        query_states, key_states, value_states = self._project(hidden_states, hidden_shape)
 
         cos, sin = position_embeddings
         if not self.rope_bypass:
@@ -176,6 +174,13 @@ class _LlamaAttentionMX(nn.Module):
         attn_output = attn_output.reshape(*input_shape, -1).contiguous()
         attn_output = self.o_proj(attn_output)
         return attn_output, attn_weights
+
+    def _project(self, hidden_states, hidden_shape):
+        """query / key / value states [batch, heads, seq, head_dim] (attention.py:157-159)"""
+        query_states = self.q_proj(hidden_states).view(hidden_shape).transpose(1, 2)
+        key_states = self.k_proj(hidden_states).view(hidden_shape).transpose(1, 2)
+        value_states = self.v_proj(hidden_states).view(hidden_shape).transpose(1, 2)
+        return query_states, key_states, value_states
 
     @classmethod
     def from_attention(cls, attention: nn.Module, q_config: dict = None):

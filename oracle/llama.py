@@ -49,17 +49,31 @@ def repeat_kv(x, n_rep):
     return x[:, :, None, :, :].expand(b, h, n_rep, s, d).reshape(b, h * n_rep, s, d)
 
 
+def head_rms_norm(x, weight, eps):
+    """RMSNorm over head_dim as the Qwen3 attention applies it to the projected queries and keys
+    (qwen3/attention.py:53-59; transformers' Qwen3RMSNorm arithmetic)"""
+    dt = x.dtype
+    x = x.to(torch.float32)
+    x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    return weight * x.to(dt)
+
+
 def attention_forward(kind, weights, hidden_states, cos, sin, attention_mask, n_heads, n_kv_heads, q_config,
-                      past=None):
+                      past=None, qk_norm_eps=None):
     """weights: dict with q_proj/k_proj/v_proj/o_proj ``.weight`` (and optional ``.bias``) tensors.
-    past: optional (key, value) already in the cache; the new (quantized) states are appended along the sequence."""
+    past: optional (key, value) already in the cache; the new (quantized) states are appended along the sequence.
+    qk_norm_eps: the Qwen3 form (``q_norm.weight`` / ``k_norm.weight`` in ``weights``), else the Llama form."""
     lin = lambda name, t: F.linear(t, weights[f"{name}.weight"], weights.get(f"{name}.bias"))
     cfg = lambda name: q_config.get(name, {})
     on = lambda name: not cfg(name).get("bypass", False)
     B, S, _ = hidden_states.shape
     head_dim = weights["q_proj.weight"].shape[0] // n_heads
-    q = lin("q_proj", hidden_states).view(B, S, -1, head_dim).transpose(1, 2)
-    k = lin("k_proj", hidden_states).view(B, S, -1, head_dim).transpose(1, 2)
+    q = lin("q_proj", hidden_states).view(B, S, -1, head_dim)
+    k = lin("k_proj", hidden_states).view(B, S, -1, head_dim)
+    if qk_norm_eps is not None:
+        q = head_rms_norm(q, weights["q_norm.weight"], qk_norm_eps)
+        k = head_rms_norm(k, weights["k_norm.weight"], qk_norm_eps)
+    q, k = q.transpose(1, 2), k.transpose(1, 2)
     v = lin("v_proj", hidden_states).view(B, S, -1, head_dim).transpose(1, 2)
     q, k = rope(q, k, cos, sin, cfg("rope") if on("rope") else None)
     if past is not None:
