@@ -128,6 +128,10 @@ def _clip_search(name: str, x: Tensor, block_size: int, block_dim: int, tab_dtyp
     assert x.numel() % block_size == 0, f"Input tensor size {x.numel()} is not divisible by block size {block_size}."
     ref = x.contiguous().view(-1)
     flat = _to_block_last_flat(x, block_dim)
+    if ref.data_ptr() % 16:  # a view that starts inside an allocation: the kernel reads 16-byte vectors
+        ref = ref.clone()
+    if flat.data_ptr() % 16:
+        flat = flat.clone()
     out = torch.empty_like(flat)
     choice = torch.empty(flat.numel() // block_size, dtype=torch.uint8, device=x.device) if return_choice else None
     tab = log2_table(tab_dtype, x.device)

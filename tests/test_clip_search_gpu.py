@@ -137,6 +137,11 @@ def test_quantizer_entry_points_take_the_search_branch(dev):
         mxint_quantizer_sim(xd, -1, MXIntMeta(block_size=32, scale_bits=8, element_bits=4), act_tensor=xd, quantile_search=True)
     with pytest.raises(NotImplementedError):
         mxint_quantizer(xd, 16, 4, quantile_search=True)
+    # a view that does not start on a 16-byte boundary
+    base = torch.randn(4 * 64 + 3, generator=torch.Generator().manual_seed(8)).to(torch.bfloat16)
+    view = base[3:].view(4, 64)
+    assert_bits_equal(mxint_quantizer(base.to(dev)[3:].view(4, 64), 32, 4, quantile_search=True),
+                      O.mxint_quantizer(view, 32, 4, quantile_search=True), "unaligned view")
     # straight-through gradient as for the plain quantizer
     xr = xd.float().clone().requires_grad_(True)
     mxint_quantizer(xr, 32, 4, quantile_search=True).sum().backward()
