@@ -214,13 +214,14 @@ class MxintLinear(Workload):
         self.xq = _ops.mxint_qdq(self.bufs[0], 32, 8, -1, 8, out_dtype=torch.bfloat16)
         self.wb = self.m._w_cache.get(self.m.weight)
         assert self.wb is not None
+        self.wp = self.m._w_cache.packed()  # the fragment-ordered copy the module's own forward uses
         self._gemm = gemm_bf16_tn
 
     def step(self, i):
         self.out = self.m(self.bufs[i % len(self.bufs)])
 
     def dominant_step(self, i):
-        self.out = self._gemm(self.xq, self.wb, self.m.bias, self.torch.float32)
+        self.out = self._gemm(self.xq, self.wb, self.m.bias, self.torch.float32, b_packed=self.wp)
 
     def work_per_step(self):
         return 2.0 * self.M * self.N * self.K
@@ -355,7 +356,7 @@ class DecoderLayerMxint(Workload):
             m = getattr(self.layer, name)
             wb = m._w_cache.get(m.weight)
             assert wb is not None
-            self.gemms.append((a11008 if name == "down_proj" else a4096, wb))
+            self.gemms.append((a11008 if name == "down_proj" else a4096, wb, m._w_cache.packed()))
         self._gemm = gemm_bf16_tn
         self.linear_flops = self.layer.linear_flops(tok)
         self.attn_flops = 4.0 * self.B * 32 * self.T * self.T * 128 / 2  # causal: half of the score matrix
@@ -365,8 +366,8 @@ class DecoderLayerMxint(Workload):
             self.out = self.layer(self.bufs[i % len(self.bufs)])
 
     def dominant_step(self, i):
-        for a, w in self.gemms:
-            self.out = self._gemm(a, w, None, self.torch.bfloat16)
+        for a, w, wp in self.gemms:  # as the modules' own forwards call it
+            self.out = self._gemm(a, w, None, self.torch.bfloat16, b_packed=wp)
 
     def work_per_step(self):
         return self.linear_flops + self.attn_flops

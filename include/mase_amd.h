@@ -29,6 +29,7 @@
  *   mase_gemm_mxfp4_skinny  nn/quantized/modules/linear.py:877-895 for at most 128 rows, MXFP4 weights
  *   mase_gemm_mxint8_skinny nn/quantized/modules/linear.py:972 for at most 128 rows, weights as int8 codes + scales
  *   mase_gemm_bf16_skinny   same call sites as mase_gemm_bf16_tn, for at most 128 rows of activations
+ *   mase_gemm_bf16_tn_packed, mase_gemm_bf16_pack_b   the same F.linear with the weight in fragment order
  *   mase_gemm_bf16_tn       nn/quantized/modules/linear.py:972 and :895 (the F.linear of LinearMXInt.forward /
  *                           LinearMXFP.forward on the quantize-dequantized operands)
  */
@@ -154,6 +155,17 @@ int mase_gemm_bf16_tn(const void* A, const void* B, const void* bias, void* C, s
 size_t mase_gemm_bf16_tn_splitk_workspace_bytes(size_t M, size_t N, size_t K);
 int mase_gemm_bf16_tn_splitk(const void* A, const void* B, const void* bias, void* C, size_t M, size_t N, size_t K,
                              int out_dtype, int bias_dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* The same product with B given as the fragment-ordered image written by mase_gemm_bf16_pack_b (a weight is packed
+ * once when it is loaded): B's fragments then go from the cache straight into registers instead of through LDS, which
+ * the kernel otherwise shares between the copies arriving and the fragment reads.  K % 128 == 0; the image takes
+ * mase_gemm_bf16_packed_bytes(N, K) = ceil(N/32)*32*K*2 bytes (below 4 GiB), 16-byte aligned.  Same results as
+ * mase_gemm_bf16_tn (the same products added in the same order).  Replaces the same F.linear
+ * (nn/quantized/modules/linear.py:972, :895). */
+size_t mase_gemm_bf16_packed_bytes(size_t N, size_t K);
+int mase_gemm_bf16_pack_b(const void* B, void* B_packed, size_t N, size_t K, void* stream);
+int mase_gemm_bf16_tn_packed(const void* A, const void* B_packed, const void* bias, void* C, size_t M, size_t N,
+                             size_t K, int out_dtype, int bias_dtype, void* stream);
 
 /* The same product for few rows of A (M <= 128, the token-by-token shape of serving): bound by streaming B once
  * from HBM.  The work is split over N and over K ranges; the partial results of the K ranges go through

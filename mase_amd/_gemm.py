@@ -11,8 +11,38 @@ SKINNY_MAX_ROWS = 128  # at most this many rows of activations take mase_gemm_bf
 OPERAND_BYTES_LIMIT = (1 << 32) - 1  # per-call operand size the GEMM entry points accept
 
 
-def gemm_bf16_tn(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dtype) -> Tensor:
-    """``a[M,K] @ b[N,K].T + bias`` with bf16 operands and fp32 accumulation; result in ``out_dtype``."""
+PACKED_B_K_MULTIPLE = 128
+
+
+def gemm_bf16_packed_b_supported(N: int, K: int) -> bool:
+    return K % PACKED_B_K_MULTIPLE == 0 and (N + 31) // 32 * 32 * K * 2 <= OPERAND_BYTES_LIMIT
+
+
+def gemm_bf16_takes_packed_b(M: int, N: int, K: int) -> bool:
+    """whether ``gemm_bf16_tn`` would run the tiled kernel on a fragment-ordered B for this shape (not the
+    weight-streaming kernel of few rows, not the K-range form of a few hundred rows)"""
+    if M <= SKINNY_MAX_ROWS or not gemm_bf16_packed_b_supported(N, K):
+        return False
+    return 2 * M * K > OPERAND_BYTES_LIMIT or _lib.load().mase_gemm_bf16_tn_splitk_workspace_bytes(M, N, K) == 0
+
+
+def gemm_bf16_pack_b(b: Tensor) -> Tensor:
+    """fragment-ordered image of ``b[N,K]`` (bf16) for ``gemm_bf16_tn(..., b_packed=...)``: ``mase_gemm_bf16_pack_b``"""
+    _lib.require_device(b, "gemm_bf16_pack_b")
+    lib = _lib.load()
+    assert b.dtype == torch.bfloat16 and b.dim() == 2
+    b = b.contiguous()
+    N, K = b.shape
+    nbytes = lib.mase_gemm_bf16_packed_bytes(N, K)
+    assert nbytes > 0, "K must be a multiple of 16"
+    out = torch.empty(nbytes, dtype=torch.uint8, device=b.device)
+    _lib.check(lib.mase_gemm_bf16_pack_b(b.data_ptr(), out.data_ptr(), N, K, _lib.stream_ptr(b)), "mase_gemm_bf16_pack_b")
+    return out
+
+
+def gemm_bf16_tn(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dtype, b_packed: Tensor | None = None) -> Tensor:
+    """``a[M,K] @ b[N,K].T + bias`` with bf16 operands and fp32 accumulation; result in ``out_dtype``.
+    ``b_packed``: the image of ``gemm_bf16_pack_b(b)``, used by the tiled kernel when the shape takes that kernel."""
     _lib.require_device(a, "gemm_bf16_tn")
     lib = _lib.load()
     assert a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16
@@ -53,14 +83,15 @@ def gemm_bf16_tn(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dty
         return out
     # the kernel addresses an operand with 32-bit byte offsets: activations beyond 4 GiB go in row chunks
     rows_per_call = max(1, min(M, (OPERAND_BYTES_LIMIT // (2 * K)) // 256 * 256 or 1))
+    packed = b_packed is not None and gemm_bf16_packed_b_supported(N, K)
     for r0 in range(0, M, rows_per_call):
         r1 = min(M, r0 + rows_per_call)
-        rc = lib.mase_gemm_bf16_tn(
-            a[r0:r1].data_ptr(), b.data_ptr(), bias.data_ptr() if bias is not None else None, out[r0:r1].data_ptr(),
-            r1 - r0, N, K, _lib.DTYPE_CODE[out_dtype], _lib.DTYPE_CODE[bias.dtype] if bias is not None else 0,
-            _lib.stream_ptr(a),
-        )
-        _lib.check(rc, "mase_gemm_bf16_tn")
+        args = (bias.data_ptr() if bias is not None else None, out[r0:r1].data_ptr(), r1 - r0, N, K,
+                _lib.DTYPE_CODE[out_dtype], _lib.DTYPE_CODE[bias.dtype] if bias is not None else 0, _lib.stream_ptr(a))
+        if packed:
+            _lib.check(lib.mase_gemm_bf16_tn_packed(a[r0:r1].data_ptr(), b_packed.data_ptr(), *args), "mase_gemm_bf16_tn_packed")
+        else:
+            _lib.check(lib.mase_gemm_bf16_tn(a[r0:r1].data_ptr(), b.data_ptr(), *args), "mase_gemm_bf16_tn")
     return out
 
 

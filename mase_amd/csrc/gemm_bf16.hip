@@ -24,6 +24,8 @@
 // copied while the epilogue of the current one runs and its stores drain behind the next main loop.
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace mase {
 namespace {
 
@@ -85,9 +87,20 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8) | ((N >> 4) << 14));
 }
 
+// One wavefront-wide 1 KB load HBM/L2 -> registers (16 bytes per lane), issued from inline assembly for the same
+// reason as the async copies: the compiler does not know of it, so nothing waits for it except wait_vmcnt.  The
+// destination must not be touched before the wait that covers it.
+__device__ __forceinline__ void load_16_untracked(bf16x8_t& dst, uint32_t off, const unsigned char* base) {
+  asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst) : "v"(off), "s"(base) : "memory");
+}
+
 // STREAM: K holds at least S tiles, so the copy stream is never more than one output tile ahead and advances
 // without branches; the other instantiation (K = one tile) advances it with the general, branching step.
-template <int OUT_DT, bool STREAM>
+// BPACK (with STREAM, an even number of K tiles): B is the fragment-ordered image of mase_gemm_bf16_pack_b and its
+// fragments go from L2 straight into registers, one K tile ahead of the MFMAs that use them; only A passes through
+// LDS.  That halves the LDS traffic (the copies landing in LDS while the wavefronts read their fragments is what
+// holds the plain kernel back) at the price of every B fragment being fetched by the two wavefronts that share it.
+template <int OUT_DT, bool STREAM, bool BPACK = false>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int tid = threadIdx.x;
@@ -142,7 +155,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
       const int r = (wave + 4 * j) * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ ((r >> 1) & 7);  // chunk that belongs at LDS position lane&7 of row r
       ga[j] = (uint32_t)((size_t)min(m0 + r, p.M - 1) * ldb) + chunk * 16 + k0;
-      gb[j] = (uint32_t)((size_t)min(n0 + r, p.N - 1) * ldb) + chunk * 16 + k0;
+      if constexpr (!BPACK) gb[j] = (uint32_t)((size_t)min(n0 + r, p.N - 1) * ldb) + chunk * 16 + k0;
     }
   };
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;
@@ -152,6 +165,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   int c_kt = 0, c_ord = 0, c_stage = 0;
   // copy number c (0..15) of the current K tile: row group c/2 of A (even c) or B (odd c)
   auto issue_copy = [&](int c) __attribute__((always_inline)) {
+    if constexpr (BPACK) {
+      if (c & 1) return;  // B does not pass through LDS
+    }
     const uint32_t st = lds_base + (uint32_t)(c_stage * kStageBytes) + (c & 1) * kTileBytes;
     const int j = c >> 1;
     async_copy_16(((c & 1) ? p.B : p.A) + (size_t)c_kt * kRowBytes, (c & 1) ? gb[j] : ga[j], st + (wave + 4 * j) * 1024);
@@ -304,12 +320,77 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // stream is advanced by a caller-supplied, branch-free step.
   // The epilogue's stores count in vmcnt like the copies, so the first hand-over of an output tile also waits
   // for the previous tile's stores to be acknowledged.
-  bf16x8_t fr[4][8];
-  wait_vmcnt<kCopies>();  // K tile 0 landed; K tile 1 may still be in flight
+  bf16x8_t fr[4][BPACK ? 4 : 8];
+  // BPACK: B fragments of two K tiles (the one in use and the one being loaded): [buffer][K step][column tile].
+  // Image layout: 1 KB blocks [column tile of 32][K step of 16][lane][8 bf16], lane l = column l % 32, K 8*(l/32)..+8.
+  bf16x8_t fb[BPACK ? 2 : 1][4][4];
+  uint32_t boff[4];          // this lane's byte offset of K step 0 of its four column tiles
+  const unsigned char* b_kbase = p.B;  // image address of K tile 0 of the K range of the output tile being loaded
+  int b_kt = 0;              // K tile (within the range) whose fragments the current iteration loads
+  auto set_b_tile = [&](int ord) __attribute__((always_inline)) {
+    int m0, n0, ks;
+    tile_origin(ord, m0, n0, ks);
+    int lane = lane_id;
+    asm volatile("" : "+v"(lane));
+    const int nt_last = (p.N + 31) / 32 - 1;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      boff[j] = (uint32_t)((size_t)min((n0 + wn * 128) / 32 + j, nt_last) * (size_t)(p.K / 16) * 1024u) + (uint32_t)lane * 16u;
+    b_kbase = p.B + (size_t)ks * (size_t)(p.kc / 16) * 1024u;
+    b_kt = 0;
+  };
+  if constexpr (BPACK) {
+    set_b_tile(0);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) load_16_untracked(fb[0][i >> 2][i & 3], boff[i & 3], b_kbase + (size_t)(i >> 2) * 1024);
+    b_kt = 1;
+    wait_vmcnt<0>();
+  } else {
+    wait_vmcnt<kCopies>();  // K tile 0 landed; K tile 1 may still be in flight
+  }
   asm volatile("s_barrier" ::: "memory");
 #pragma unroll
-  for (int f = 0; f < 8; ++f) fr[0][f] = load_frag(0, 0, f);
+  for (int f = 0; f < (BPACK ? 4 : 8); ++f) fr[0][f] = load_frag(0, 0, f);
   int stage = 0;
+  // BPACK form of the K iteration.  vmcnt holds, oldest first: at the start the 16 B loads of this K tile and the 8 A
+  // copies of the next; steps 0 and 1 add the 16 B loads of the next K tile (second half of the slots, the first half
+  // carries the LDS reads), the hand-over needs the A copies (all but the youngest 16), steps 2 and 3 add the A
+  // copies of the K tile after next.  Stores of an epilogue in between only make the waits conservative.
+  auto k_iteration_b = [&](auto&& advance, auto bufc) __attribute__((always_inline)) {
+    constexpr int NB = decltype(bufc)::value;
+    wait_vmcnt<kCopies / 2>();
+    const unsigned char* bsrc = b_kbase + (size_t)b_kt * 4096;
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) {
+#pragma unroll
+      for (int t = 0; t < 16; ++t) {
+        acc[t >> 2][t & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[s][t >> 2], fb[NB][s][t & 3],
+                                                                     acc[t >> 2][t & 3], 0, 0, 0);
+        if (s == 0) {
+          if (t < 4) fr[1][t] = load_frag(stage, 1, t);
+          if (t >= 8) load_16_untracked(fb[NB ^ 1][(t - 8) >> 2][t & 3], boff[t & 3], bsrc + (size_t)((t - 8) >> 2) * 1024);
+        } else if (s == 1) {
+          if (t < 4) fr[2][t] = load_frag(stage, 2, t);
+          else if (t < 8) fr[3][t - 4] = load_frag(stage, 3, t - 4);
+          else load_16_untracked(fb[NB ^ 1][t >> 2][t & 3], boff[t & 3], bsrc + (size_t)(t >> 2) * 1024);
+        } else if (s == 2) {
+          if (t < 4) fr[0][t] = load_frag(stage ^ 1, 0, t);
+          if ((t & 3) == 3) issue_copy((t >> 2) * 2);
+        } else {
+          if ((t & 3) == 3) issue_copy(8 + (t >> 2) * 2);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (s == 1) {
+        wait_vmcnt<16>();
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    advance();
+    stage ^= 1;
+    ++b_kt;
+  };
   auto k_iteration = [&](auto&& advance) __attribute__((always_inline)) {
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
@@ -340,7 +421,20 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     stage ^= 1;
   };
   for (int ord = 0; ord < n_my; ++ord) {
-    if constexpr (STREAM) {
+    if constexpr (BPACK) {
+      // two K tiles per trip (the fragment buffers alternate); the copy stream as in the plain form below, the B
+      // stream one K tile ahead: it moves on to the next output tile before the last K tile of this one
+#pragma unroll 1
+      for (int kt = 0; kt < nk - S; kt += 2) {
+        k_iteration_b(step_within_tile, std::integral_constant<int, 0>{});
+        k_iteration_b(step_within_tile, std::integral_constant<int, 1>{});
+      }
+      set_copy_tile(ord + 1);
+      c_kt = 0;
+      k_iteration_b(step_within_tile, std::integral_constant<int, 0>{});
+      set_b_tile(ord + 1);
+      k_iteration_b(step_within_tile, std::integral_constant<int, 1>{});
+    } else if constexpr (STREAM) {
       // the copy stream stands at K tile S of this output tile (or, if nk == S, at K tile 0 of the next)
 #pragma unroll 1
       for (int kt = 0; kt < nk - S; ++kt) k_iteration(step_within_tile);
@@ -371,7 +465,7 @@ int persistent_grid_bf16(int total_tiles) {
 }
 
 // launch of the persistent kernel for the work items of p (tiles x K ranges), output dtype out_dtype
-int launch_gemm_bf16(const GemmParams& p, int out_dtype, hipStream_t st) {
+int launch_gemm_bf16(const GemmParams& p, int out_dtype, hipStream_t st, bool bpack = false) {
   const size_t lds_bytes = (size_t)kLdsBytes;
   const int nwg = persistent_grid_bf16(p.tiles_m * p.tiles_n * p.splits);
   if (nwg <= 0) return MASE_ERR_LAUNCH;
@@ -388,7 +482,24 @@ int launch_gemm_bf16(const GemmParams& p, int out_dtype, hipStream_t st) {
     }                                                                                                             \
     hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, STREAM_>), grid, block, lds_bytes, st, p);                       \
   } while (0)
-  if (stream_fits) {
+  if (bpack) {
+    if (!stream_fits || ((p.kc / BK) & 1) != 0) return MASE_ERR_SHAPE;
+#define MASE_GEMM_LAUNCH_B(DT_)                                                                                   \
+  do {                                                                                                            \
+    static bool attr_set = false;                                                                                 \
+    const void* k = (const void*)gemm_bf16_tn_kernel<DT_, true, true>;                                            \
+    if (!attr_set) {                                                                                              \
+      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)       \
+        return MASE_ERR_LAUNCH;                                                                                   \
+      attr_set = true;                                                                                            \
+    }                                                                                                             \
+    hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, true, true>), grid, block, lds_bytes, st, p);                    \
+  } while (0)
+    if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH_B(MASE_DT_F32);
+    else if (out_dtype == MASE_DT_BF16) MASE_GEMM_LAUNCH_B(MASE_DT_BF16);
+    else MASE_GEMM_LAUNCH_B(MASE_DT_F16);
+#undef MASE_GEMM_LAUNCH_B
+  } else if (stream_fits) {
     if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH(MASE_DT_F32, true);
     else if (out_dtype == MASE_DT_BF16) MASE_GEMM_LAUNCH(MASE_DT_BF16, true);
     else MASE_GEMM_LAUNCH(MASE_DT_F16, true);
@@ -414,6 +525,22 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
   if constexpr (OUT_DT == MASE_DT_F32) ((float*)C)[i] = s;
   else if constexpr (OUT_DT == MASE_DT_BF16) ((uint16_t*)C)[i] = (uint16_t)f32_to_bf16_bits(s);
   else ((uint16_t*)C)[i] = (uint16_t)f32_to_f16_bits(s);
+}
+
+// B[N, K] row-major -> fragment-ordered image: 1 KB blocks [column tile of 32][K step of 16][lane][8 bf16]; lane l
+// of a block holds B[tile*32 + l%32][step*16 + 8*(l/32) .. +8], rows beyond N are zero
+__global__ __launch_bounds__(256) void gemm_pack_b_kernel(const uint4* __restrict__ B, uint4* __restrict__ out, int N,
+                                                          int K, size_t granules) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= granules) return;
+  const int lane = (int)(g & 63);
+  const size_t blk = g >> 6;
+  const int steps = K / 16;
+  const int nt = (int)(blk / (size_t)steps), ks = (int)(blk % (size_t)steps);
+  const int row = nt * 32 + (lane & 31);
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (row < N) v = B[((size_t)row * K + (size_t)ks * 16 + 8 * (lane >> 5)) / 8];
+  out[g] = v;
 }
 
 // K ranges for a product whose output tiles alone would leave most CUs idle: as many as fill the machine once, each a
@@ -506,4 +633,47 @@ extern "C" int mase_gemm_bf16_tn_splitk(const void* A, const void* B, const void
   else
     hipLaunchKernelGGL(gemm_splitk_reduce_kernel<MASE_DT_F16>, grid, block, 0, st, P, C, bias, bias_dtype, mn, (int)N, splits);
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+extern "C" size_t mase_gemm_bf16_packed_bytes(size_t N, size_t K) {
+  if (N == 0 || K == 0 || (K % 16) != 0) return 0;
+  return ((N + 31) / 32) * 32 * K * 2;
+}
+
+extern "C" int mase_gemm_bf16_pack_b(const void* B, void* B_packed, size_t N, size_t K, void* stream) {
+  using namespace mase;
+  if (N == 0 || K == 0) return MASE_OK;
+  if (B == nullptr || B_packed == nullptr) return MASE_ERR_NULL;
+  if ((K % 16) != 0 || N > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
+  if (!aligned16(B) || !aligned16(B_packed)) return MASE_ERR_ALIGN;
+  const size_t granules = mase_gemm_bf16_packed_bytes(N, K) / 16;
+  hipLaunchKernelGGL(gemm_pack_b_kernel, dim3(blocks_for(granules, (size_t)256)), dim3(256), 0, (hipStream_t)stream,
+                     (const uint4*)B, (uint4*)B_packed, (int)N, (int)K, granules);
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+extern "C" int mase_gemm_bf16_tn_packed(const void* A, const void* B_packed, const void* bias, void* C, size_t M,
+                                        size_t N, size_t K, int out_dtype, int bias_dtype, void* stream) {
+  using namespace mase;
+  if (M == 0 || N == 0) return MASE_OK;
+  if (A == nullptr || B_packed == nullptr || C == nullptr) return MASE_ERR_NULL;
+  if (K == 0 || (K % (2 * BK)) != 0 || M > (1u << 30) || N > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
+  if ((unsigned long long)M * K * 2 > 0xFFFFFFFFull || (unsigned long long)mase_gemm_bf16_packed_bytes(N, K) > 0xFFFFFFFFull)
+    return MASE_ERR_SHAPE;
+  if (!aligned16(A) || !aligned16(B_packed)) return MASE_ERR_ALIGN;
+  if (out_dtype < 0 || out_dtype > 2 || (bias != nullptr && (bias_dtype < 0 || bias_dtype > 2))) return MASE_ERR_DTYPE;
+  GemmParams p;
+  p.A = (const unsigned char*)A;
+  p.B = (const unsigned char*)B_packed;
+  p.bias = bias;
+  p.C = C;
+  p.M = (int)M;
+  p.N = (int)N;
+  p.K = (int)K;
+  p.bias_dtype = bias_dtype;
+  p.tiles_m = (int)((M + BM - 1) / BM);
+  p.tiles_n = (int)((N + BN - 1) / BN);
+  p.splits = 1;
+  p.kc = (int)K;
+  return launch_gemm_bf16(p, out_dtype, (hipStream_t)stream, true);
 }

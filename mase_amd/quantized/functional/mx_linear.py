@@ -13,9 +13,9 @@ import torch
 from torch import Tensor
 from torch.nn import functional as F
 
-from ..._gemm import (MXFP_HW_FORMATS, MXFP_K_MULTIPLE, SKINNY_MAX_ROWS, gemm_bf16_tn, gemm_mxfp4_skinny,
-                      gemm_mxfp4_skinny_supported, gemm_mxfp_scaled, gemm_mxint8_skinny, gemm_mxint8_skinny_supported,
-                      mxfp_pack)
+from ..._gemm import (MXFP_HW_FORMATS, MXFP_K_MULTIPLE, SKINNY_MAX_ROWS, gemm_bf16_pack_b, gemm_bf16_packed_b_supported,
+                      gemm_bf16_takes_packed_b, gemm_bf16_tn, gemm_mxfp4_skinny, gemm_mxfp4_skinny_supported,
+                      gemm_mxfp_scaled, gemm_mxint8_skinny, gemm_mxint8_skinny_supported, mxfp_pack)
 
 
 class WeightCache:
@@ -33,10 +33,12 @@ class WeightCache:
     def __init__(self):
         self._key = None
         self._w = None
+        self._packed = None
 
     def invalidate(self):
         self._key = None
         self._w = None
+        self._packed = None
 
     def get(self, weight: Tensor):
         key = (weight.data_ptr(), weight._version, weight.dtype, weight.device, tuple(weight.shape))
@@ -48,8 +50,19 @@ class WeightCache:
                 wb = w.to(torch.bfloat16).contiguous()
                 if not torch.equal(wb.to(w.dtype), w):
                     wb = None
-            self._key, self._w = key, wb
+            self._key, self._w, self._packed = key, wb, None
         return self._w
+
+    def packed(self):
+        """The fragment-ordered copy of the image returned by the last ``get`` (for ``gemm_bf16_tn(b_packed=...)``),
+        built on first use: another 2 bytes per weight, spent only by modules that see batches large enough for the
+        tiled kernel.  None while a HIP graph is being captured and the copy does not exist yet (it must not be
+        allocated from the graph's pool)."""
+        if self._packed is None and self._w is not None and gemm_bf16_packed_b_supported(*self._w.shape):
+            if torch.cuda.is_current_stream_capturing():
+                return None
+            self._packed = gemm_bf16_pack_b(self._w)
+        return self._packed
 
 
 class _SharedActivation:
@@ -97,7 +110,8 @@ def mx_linear(x: Tensor, weight: Tensor, bias: Tensor | None, quantize_to_bf16, 
         xq = _shared_activation.get(x, quantizer_key, lambda: quantize_to_bf16(x.reshape(-1, x.shape[-1])))
     else:
         xq = quantize_to_bf16(x.reshape(-1, x.shape[-1]))
-    y = gemm_bf16_tn(xq, wb, bias, x.dtype)
+    wp = cache.packed() if gemm_bf16_takes_packed_b(xq.shape[0], wb.shape[0], wb.shape[1]) else None
+    y = gemm_bf16_tn(xq, wb, bias, x.dtype, b_packed=wp)
     return y.reshape(*lead, weight.shape[0])
 
 

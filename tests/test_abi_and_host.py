@@ -64,6 +64,14 @@ def test_entry_points_reject_bad_arguments_without_a_gpu(lib):
     assert lib.mase_gemm_bf16_tn_splitk(p, p, None, p, 4, 4, 96, 0, 0, None, 0, None) == -2
     assert lib.mase_gemm_bf16_tn_splitk(p, None, None, p, 4, 4, 64, 0, 0, None, 0, None) == -1
     assert lib.mase_gemm_bf16_tn_splitk_workspace_bytes(0, 4, 64) == 0
+    # mase_gemm_bf16_tn_packed(A, B_packed, bias, C, M, N, K, out_dtype, bias_dtype, stream) and the packer
+    assert lib.mase_gemm_bf16_tn_packed(p, p, None, p, 256, 256, 192, 0, 0, None) == -2   # K in pairs of 64-element tiles
+    assert lib.mase_gemm_bf16_tn_packed(p, None, None, p, 256, 256, 128, 0, 0, None) == -1
+    assert lib.mase_gemm_bf16_tn_packed(p, p, None, p, 256, 256, 128, 4, 0, None) == -4
+    assert lib.mase_gemm_bf16_tn_packed(p, p, None, p, 0, 256, 128, 0, 0, None) == 0
+    assert lib.mase_gemm_bf16_pack_b(p, p, 64, 24, None) == -2
+    assert lib.mase_gemm_bf16_pack_b(None, p, 64, 32, None) == -1
+    assert lib.mase_gemm_bf16_packed_bytes(33, 64) == 64 * 64 * 2 and lib.mase_gemm_bf16_packed_bytes(32, 24) == 0
     # mase_gemm_mxint8_skinny(A, codes, scales, bias, C, M, N, K, out_dtype, bias_dtype, workspace, workspace_bytes, stream)
     assert lib.mase_gemm_mxint8_skinny(p, p, p, None, p, 4, 4, 192, 0, 0, p, 4096, None) == -2    # K in whole 128-chunks
     assert lib.mase_gemm_mxint8_skinny(p, p, p, None, p, 129, 4, 128, 0, 0, p, 4096, None) == -2

@@ -187,3 +187,28 @@ def test_gemm_a_few_hundred_rows_cuts_k_into_work_items(dev, M):
         assert torch.equal(got, gemm_bf16_tn(a, b, None, torch.float32))
     assert lib.mase_gemm_bf16_tn_splitk_workspace_bytes(4096, 4096, 4096) == 0      # 256 tiles: nothing to split
     assert lib.mase_gemm_bf16_tn_splitk_workspace_bytes(512, 4096, 4096) > 0
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (512, 768, 256), (300, 200, 384), (4096, 4096, 1024), (2048, 8448, 512),
+                                   (4100, 4200, 640), (16384, 1024, 4096), (1000, 33, 128)])
+def test_gemm_with_the_weight_in_fragment_order_is_the_same_product(dev, M, N, K):
+    """mase_gemm_bf16_tn_packed against mase_gemm_bf16_tn on the same operands: the same products in the same order,
+    so bit-identical (random operands; the bias and every output dtype), one to several output tiles per work-group,
+    ragged M and N, 1 to 32 pairs of K tiles"""
+    from mase_amd._gemm import gemm_bf16_pack_b, gemm_bf16_packed_b_supported, gemm_bf16_tn
+
+    g = torch.Generator().manual_seed(M + N + K)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
+    b = (torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+    bias = torch.randn(N, generator=g).to(dev)
+    print(f"packed-B gemm M={M} N={N} K={K}", flush=True)
+    assert gemm_bf16_packed_b_supported(N, K) == (K % 128 == 0)
+    bp = gemm_bf16_pack_b(b)
+    assert bp.numel() == (N + 31) // 32 * 32 * K * 2
+    for dt, bs in ((torch.float32, None), (torch.bfloat16, bias), (torch.float16, bias.to(torch.float16))):
+        want = gemm_bf16_tn(a, b, bs, dt)
+        got = gemm_bf16_tn(a, b, bs, dt, b_packed=bp)
+        assert torch.equal(got, want), (dt, float((got.float() - want.float()).abs().max()))
+    if K % 128 == 0 and M > 512:
+        ref = (a.float() @ b.float().t())
+        assert float((gemm_bf16_tn(a, b, None, torch.float32, b_packed=bp) - ref).abs().max() / ref.abs().max()) < 1e-5
