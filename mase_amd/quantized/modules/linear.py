@@ -9,7 +9,8 @@ import torch
 from torch.nn import functional as F
 
 from ...quantizers import _ops, mxfp_quantizer, mxint_quantizer
-from ..functional.linear import linearBlockFP, linearInteger, linearMinifloatDenorm, linearMinifloatIEEE
+from ..functional.linear import (QuantizedParamCache, linearBlockFP, linearInteger, linearMinifloatDenorm,
+                                 linearMinifloatIEEE)
 from ..functional.mx_linear import (PackedMXFPWeight, PackedMXIntWeight, WeightCache, mx_linear, mxfp_linear_native,
                                     mxint_decode_applies, mxint_linear_decode)
 
@@ -19,6 +20,12 @@ class _LinearBase(torch.nn.Linear):
         super().__init__(in_features, out_features, bias, device, dtype)
         self.bypass = False
         self.pruning_masks = None
+        # the reference quantizes weight and bias on every forward; between inference forwards they do not change
+        self._param_cache = QuantizedParamCache()
+
+    def invalidate_weight_cache(self):
+        """Forget the cached quantized parameters (needed only after an in-place edit through ``weight.data``)."""
+        self._param_cache.invalidate()
 
 
 class LinearInteger(_LinearBase):
@@ -35,7 +42,7 @@ class LinearInteger(_LinearBase):
     def forward(self, x):
         if self.bypass:
             return F.linear(x, self.weight, self.bias)
-        return linearInteger(x, self.weight, self.bias, self.config, self.out_config)
+        return linearInteger(x, self.weight, self.bias, self.config, self.out_config, param_cache=self._param_cache)
 
 
 class _ConfigLinear(_LinearBase):
@@ -51,7 +58,7 @@ class _ConfigLinear(_LinearBase):
     def forward(self, x):
         if self.bypass:
             return F.linear(x, self.weight, self.bias)
-        return type(self)._functional(x, self.weight, self.bias, self.config)
+        return type(self)._functional(x, self.weight, self.bias, self.config, param_cache=self._param_cache)
 
 
 class LinearMinifloatDenorm(_ConfigLinear):

@@ -306,3 +306,40 @@ def test_quantize_module_transform_pass(dev):
         quantize_module_transform_pass(MLP().to(dev), {"by": "layer"})
     assert set(quantized_module_map) >= {"linear_mxint", "linear_mxfp", "linear_block_fp", "linear_integer",
                                          "linear_fixed", "linear_minifloat_ieee", "linear_minifloat_denorm"}
+
+
+def test_quantized_parameters_are_kept_between_inference_forwards(dev):
+    """LinearBlockFP / Integer / Minifloat*: the module keeps the quantized weight and bias (and the weight's bf16 and
+    fragment-ordered copies) between forwards under no_grad; results are those of the functional form, which
+    quantizes them on every call, and a changed parameter is picked up"""
+    import mase_amd.quantized.functional.linear as FL
+    from mase_amd.quantized import LinearBlockFP, LinearInteger, LinearMinifloatDenorm, LinearMinifloatIEEE
+
+    g = torch.Generator().manual_seed(6)
+    bfp = {f"{k}_{s}": v for k in ("weight", "data_in", "bias")
+           for s, v in (("width", 8), ("exponent_width", 8), ("exponent_bias", None), ("block_size", [16]))}
+    icfg = {"weight_width": 8, "weight_frac_width": 6, "data_in_width": 8, "data_in_frac_width": 4, "bias_width": 8,
+            "bias_frac_width": 5}
+    mcfg = {f"{k}_{s}": v for k in ("weight", "data_in", "bias") for s, v in (("width", 8), ("exponent_width", 4), ("exponent_bias", None))}
+    cases = [(LinearBlockFP, FL.linearBlockFP, bfp), (LinearInteger, FL.linearInteger, icfg),
+             (LinearMinifloatDenorm, FL.linearMinifloatDenorm, mcfg), (LinearMinifloatIEEE, FL.linearMinifloatIEEE, mcfg)]
+    for dtype in (torch.float32, torch.bfloat16):
+        for cls, fn, cfg in cases:
+            m = cls(256, 512, device=dev, dtype=dtype, config=dict(cfg))
+            m.load_state_dict({"weight": (torch.randn(512, 256, generator=g) * 0.1).to(dtype), "bias": torch.randn(512, generator=g).to(dtype)})
+            for rows in (8, 300, 4096):  # weight-streaming kernel, K-range form, tiled kernel on the fragment-ordered copy
+                x = torch.randn(rows, 256, generator=g).to(dtype).to(dev)
+                with torch.no_grad():
+                    want = fn(x, m.weight, m.bias, dict(cfg))
+                    assert torch.equal(m(x), want) and torch.equal(m(x), want), (cls.__name__, dtype, rows)
+            assert m._param_cache.qw is not None and m._param_cache.packed() is not None
+            with torch.no_grad():
+                m.weight.mul_(0.5)
+                want = fn(x, m.weight, m.bias, dict(cfg))
+                assert torch.equal(m(x), want), (cls.__name__, "after an in-place update")
+                m.weight.data.add_(0.25)           # an edit the version counter does not see
+                m.invalidate_weight_cache()
+                assert torch.equal(m(x), fn(x, m.weight, m.bias, dict(cfg)))
+            y = m(x[:4].clone().requires_grad_(True))  # gradients recorded: nothing cached is used, autograd works
+            y.sum().backward()
+            assert m.weight.grad is not None
