@@ -12,6 +12,7 @@
 // bit is cleared), and everything below that binade, which becomes a signed zero.
 #pragma once
 #include "common.hpp"
+#include "minifloat_mx.hpp"
 
 namespace mase {
 
@@ -59,6 +60,44 @@ inline Pk16Format make_pk16_format(int F, int round_mode) {
   f.exp_lsb2 = (1u << MB) * one;
   f.exp_mask2 = (0x7FFFu & ~((1u << MB) - 1u)) * one;
   return f;
+}
+
+// Everything pk16_cast needs for format m on elements of dtype DT, and the domain it covers: an element e is handled
+// iff e == 0 or lo_thr <= |e| < hi_thr (bit patterns); `sub`: the binade below the format's normal range can be taken
+// in line (pk16_cast<MB, true>), which moves the lower end of the domain down to T's own smallest normal.  Returns
+// false when the packed form does not apply.
+// A format with more fraction bits than T has mantissa bits (F > MB) rounds nothing inside its normal range; its
+// largest value, 2^top * (2 - 2^-F), is not a value of T and rounds to 2^(top+1) (T's infinity when top is T's last
+// binade) when the result is stored, so that is what elements beyond the range become.
+struct Pk16CastParams {
+  Pk16Format f;
+  Pk16Range r;
+  uint32_t lo_thr, hi_thr;
+  bool sub;
+};
+
+template <int DT>
+inline bool make_pk16_cast_params(const MinifloatMxFmt& m, Pk16CastParams& q) {
+  constexpr int MB = (DT == MASE_DT_BF16) ? 7 : 10, EB = (DT == MASE_DT_BF16) ? 127 : 15;
+  constexpr int kMaxField = (DT == MASE_DT_BF16) ? 254 : 30;
+  const int top = m.e_hi - m.bias + EB;      // exponent field (in T) of the format's largest binade
+  const int bottom = 1 - m.bias + EB;        // and of its smallest normal binade
+  if (top > kMaxField || top < 1) return false;
+  const bool wide = m.F > MB;
+  const int F = wide ? MB : m.F;
+  const uint32_t one = 0x00010001u;
+  q.f = make_pk16_format<MB>(F, m.round_mode);
+  q.r.odd_k2 = (((m.bias - EB) & 1) ? (1u << MB) : 0u) * one;
+  q.r.max2 = (wide ? ((uint32_t)(top + 1) << MB)
+                   : (((uint32_t)top << MB) | ((uint32_t)m.frac_hi << q.f.drop))) * one;
+  q.lo_thr = (uint32_t)(bottom < 1 ? 1 : bottom) << MB;
+  q.r.lo_thr2 = q.lo_thr * one;
+  q.r.sub_thr2 = ((uint32_t)(bottom - 1 < 1 ? 1 : bottom - 1) << MB) * one;
+  // Inf/NaN inputs, and for a format with inf/nan codes every element of its top ordinary binade
+  q.hi_thr = m.is_finite ? ((uint32_t)(kMaxField + 1) << MB) : ((uint32_t)top << MB);
+  // in-line handling of the binade below the normal range when ordinary data reaches it and it exists in T
+  q.sub = !wide && m.bias < 12 && q.lo_thr > (2u << MB) && m.F >= 1;
+  return true;
 }
 
 // One register (two elements).  lo_acc / hi_acc collect min(|x| - 1) (a zero wraps to 0xFFFF) and max(|x|) for the

@@ -468,22 +468,15 @@ struct MinifloatRun {
 struct MinifloatMxRun {
   const void* in; void* out; size_t numel; int out_dtype; MinifloatMxFmt m; hipStream_t st;
   // parameters of the packed 16-bit kernel, or false when the format does not fit it
-  template <int DT> bool pk16_params(MinifloatPk16Params& q) const {
-    constexpr int MB = (DT == MASE_DT_BF16) ? 7 : 10, EB = (DT == MASE_DT_BF16) ? 127 : 15;
-    constexpr int kMaxField = (DT == MASE_DT_BF16) ? 254 : 30;
-    const int top = m.e_hi - m.bias + EB;      // exponent field (in T) of the format's largest binade
-    const int bottom = 1 - m.bias + EB;        // and of its smallest normal binade
-    if (m.F > MB || top > kMaxField || top < 1) return false;
-    const uint32_t one = 0x00010001u;
-    q.f = make_pk16_format<MB>(m.F, m.round_mode);
-    q.r.odd_k2 = (((m.bias - EB) & 1) ? (1u << MB) : 0u) * one;
-    q.r.max2 = (((uint32_t)top << MB) | ((uint32_t)m.frac_hi << q.f.drop)) * one;
-    q.lo_thr = (uint32_t)(bottom < 1 ? 1 : bottom) << MB;
-    q.r.lo_thr2 = q.lo_thr * one;
-    q.r.sub_thr2 = ((uint32_t)(bottom - 1 < 1 ? 1 : bottom - 1) << MB) * one;
-    // Inf/NaN inputs, and for a format with inf/nan codes every element of its top ordinary binade
-    q.hi_thr = m.is_finite ? ((uint32_t)(kMaxField + 1) << MB) : ((uint32_t)top << MB);
+  template <int DT> bool pk16_params(MinifloatPk16Params& q, bool& sub) const {
+    Pk16CastParams c;
+    if (!make_pk16_cast_params<DT>(m, c)) return false;
+    q.f = c.f;
+    q.r = c.r;
+    q.lo_thr = c.lo_thr;
+    q.hi_thr = c.hi_thr;
     q.m = m;
+    sub = c.sub;
     return true;
   }
   template <int DTI> int run() {
@@ -492,10 +485,9 @@ struct MinifloatMxRun {
     op.m = m;
     if constexpr (DTI != MASE_DT_F32) {
       MinifloatPk16Params q;
-      if (out_dtype == DTI && aligned16(in) && aligned16(out) && numel >= 8 && pk16_params<DTI>(q)) {
+      bool sub = false;
+      if (out_dtype == DTI && aligned16(in) && aligned16(out) && numel >= 8 && pk16_params<DTI>(q, sub)) {
         const size_t n8 = numel / 8;
-        // in-line handling of the binade below the normal range when ordinary data reaches it and it exists in T
-        const bool sub = m.bias < 12 && q.lo_thr > (2u << ((DTI == MASE_DT_BF16) ? 7 : 10)) && m.F >= 1;
         const dim3 grid(blocks_for(n8, kEwThreads)), block(kEwThreads);
         if (sub) hipLaunchKernelGGL((minifloat_mx_pk16_kernel<DTI, true>), grid, block, 0, st, (const uint4*)in, (uint4*)out, n8, q);
         else hipLaunchKernelGGL((minifloat_mx_pk16_kernel<DTI, false>), grid, block, 0, st, (const uint4*)in, (uint4*)out, n8, q);

@@ -233,7 +233,7 @@ def test_minifloat_denorm_ieee(Q, dev, dtype, cfg):
 
 
 # ------------------------------------------------------------------ bit-level minifloat and MXFP
-MF_FORMATS = [(4, 3), (5, 2), (2, 1), (2, 3), (3, 2), (1, 2), (5, 10), (8, 7), (3, 4)]
+MF_FORMATS = [(4, 3), (5, 2), (2, 1), (2, 3), (3, 2), (1, 2), (5, 10), (8, 7), (3, 4), (5, 8), (4, 9), (8, 6)]
 
 
 @pytest.mark.parametrize("fmt", MF_FORMATS)
