@@ -273,7 +273,7 @@ class MxfpLinear(Workload):
 
     def setup(self, torch, dev, n_buffers):
         from mase_amd.quantized import LinearMXFP
-        from mase_amd._gemm import gemm_mxfp_scaled, mxfp_pack
+        from mase_amd._gemm import gemm_mxfp4_scaled_tiled, mxfp_pack_tiled
 
         self.torch = torch
         self.m = LinearMXFP(self.K, self.N, bias=False, device=dev, dtype=torch.bfloat16, config=dict(self.cfg))
@@ -281,15 +281,15 @@ class MxfpLinear(Workload):
         assert self.m._w_packed.valid_for(self.m.weight)
         x = self.make_x(torch, self.M).to(dev)
         self.bufs = [x.roll(i, dims=0).contiguous() for i in range(max(n_buffers, 2))]
-        self.xc, self.xs = mxfp_pack(self.bufs[0], 4, 3)
-        self._gemm = gemm_mxfp_scaled
+        self.xt, self.xs = mxfp_pack_tiled(self.bufs[0], 4, 3)
+        self._gemm = gemm_mxfp4_scaled_tiled
 
     def step(self, i):
         self.out = self.m(self.bufs[i % len(self.bufs)])
 
     def dominant_step(self, i):
         p = self.m._w_packed
-        self.out = self._gemm(self.xc, self.xs, (4, 3), p.codes, p.scales, p.fmt, None, self.torch.bfloat16)
+        self.out = self._gemm(self.xt, self.xs, (4, 3), p.tiled(self.K), p.scales, None, self.torch.bfloat16)
 
     def work_per_step(self):
         return 2.0 * self.M * self.N * self.K

@@ -24,7 +24,8 @@
  *   mase_silu_mul_minifloat nn/quantized/modules/llama/mlp.py:60-62 (silu_minifloat(gate) * up)
  *   mase_attn_softmax_mx    nn/quantized/modules/llama/attention.py:363-392 (scores -> quantized probabilities)
  *   mase_mx_unpack          nn/quantizers/mxint/fake.py:59-80, nn/quantizers/mxfp/fake.py:75-104 (compose_*)
- *   mase_mxfp_pack, mase_gemm_mxfp_scaled   nn/quantized/modules/linear.py:877-895 (LinearMXFP.forward on
+ *   mase_mxfp_pack(_tiled), mase_mxfp_tile_codes, mase_gemm_mxfp_scaled, mase_gemm_mxfp4_scaled_tiled
+ *                           nn/quantized/modules/linear.py:877-895 (LinearMXFP.forward on
  *                           formats the block-scaled matrix instruction supports)
  *   mase_gemm_mxfp4_skinny  nn/quantized/modules/linear.py:877-895 for at most 128 rows, MXFP4 weights
  *   mase_gemm_mxint8_skinny nn/quantized/modules/linear.py:972 for at most 128 rows, weights as int8 codes + scales
@@ -213,6 +214,25 @@ int mase_mxfp_pack(const void* in, uint8_t* codes, uint8_t* scales, size_t numel
 int mase_gemm_mxfp_scaled(const void* A, const void* A_scales, int a_format, const void* B, const void* B_scales,
                           int b_format, const void* bias, void* C, size_t M, size_t N, size_t K, int out_dtype,
                           int bias_dtype, void* stream);
+
+/* The same product with both code matrices as tile images: for a [rows, K] code matrix of 8-bit (4-bit) codes the image
+ * is [row tile of 256][K tile of 128][row in tile][128 (64) bytes], the 16-byte chunks of each row segment exchanged by
+ * chunk ^= (row >> 1) & 7 (chunk ^= (row >> 2) & 3), rows past the end repeating the last one: the bytes one K tile of
+ * one row tile occupies in the kernel's LDS stage, contiguous, so that every copy reads one 1 KB run.  Scales stay
+ * row-major.  mase_mxfp_tiled_bytes: size of an image (0 for K % 128 != 0 or bits other than 4, 8).
+ * mase_mxfp_tile_codes: image of a row-major code matrix (done once for a weight).  mase_mxfp_pack_tiled: mase_mxfp_pack
+ * for a [rows, K] matrix of e4m3 / e5m2 activations writing the image directly (tiled_codes holds
+ * mase_mxfp_tiled_bytes(rows, K, 8) bytes; rows past the end are left unwritten and only ever feed output rows that are
+ * not stored).  mase_gemm_mxfp4_scaled_tiled: A e4m3 / e5m2 image, B e2m1 image; result bit-identical to
+ * mase_gemm_mxfp_scaled on the row-major forms; both images must be below 2^32 bytes.  Same contraction of
+ * LinearMXFP.forward (nn/quantized/modules/linear.py:877-895). */
+size_t mase_mxfp_tiled_bytes(size_t rows, size_t K, int bits);
+int mase_mxfp_tile_codes(const void* codes, void* tiled, size_t rows, size_t K, int bits, void* stream);
+int mase_mxfp_pack_tiled(const void* in, uint8_t* tiled_codes, uint8_t* scales, size_t rows, size_t K, int in_dtype,
+                         int exp_bits, int frac_bits, const uint32_t* log2_tab, void* stream);
+int mase_gemm_mxfp4_scaled_tiled(const void* A_tiled, const void* A_scales, int a_format, const void* B_tiled,
+                                 const void* B_scales, const void* bias, void* C, size_t M, size_t N, size_t K,
+                                 int out_dtype, int bias_dtype, void* stream);
 
 /* Attention probabilities of the MX-quantized Llama attention in one pass: for scores [batch, heads, q_len, kv_len]
  * (dense, dtype) and an optional additive mask [batch, 1, q_len, kv_len] of the same dtype (rows mask_row_stride

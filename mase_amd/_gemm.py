@@ -176,6 +176,77 @@ def gemm_mxfp_scaled(a_codes: Tensor, a_scales: Tensor, a_fmt, b_codes: Tensor, 
     return out
 
 
+def gemm_mxfp4_tiled_supported(M: int, N: int, K: int, a_fmt, b_fmt) -> bool:
+    """Whether ``gemm_mxfp4_scaled_tiled`` takes the product: 8-bit activations, e2m1 weights, whole K tiles and a weight
+    image below 2^32 bytes (the activations are cut into row ranges that fit)."""
+    return (tuple(a_fmt) in ((4, 3), (5, 2)) and tuple(b_fmt) == (2, 1) and K > 0 and K % MXFP_K_MULTIPLE == 0
+            and M > 0 and -(-N // 256) * 256 * K // 2 < (1 << 32) and 256 * K < (1 << 32))
+
+
+def mxfp_tile_codes(codes: Tensor, K: int, bits: int) -> Tensor:
+    """The tile image of a row-major code matrix ``[rows, K * bits / 8]`` (``mase_mxfp_tile_codes``): what the tiled
+    block-scaled GEMM copies from.  Done once for a weight."""
+    _lib.require_device(codes, "mxfp_tile_codes")
+    lib = _lib.load()
+    codes = codes.contiguous()
+    rows = codes.shape[0]
+    assert codes.dtype == torch.uint8 and codes.shape == (rows, K * bits // 8)
+    nbytes = lib.mase_mxfp_tiled_bytes(rows, K, bits)
+    assert nbytes > 0, "K must be a multiple of 128 and bits 4 or 8"
+    tiled = torch.empty(nbytes, dtype=torch.uint8, device=codes.device)
+    _lib.check(lib.mase_mxfp_tile_codes(codes.data_ptr(), tiled.data_ptr(), rows, K, bits, _lib.stream_ptr(codes)),
+               "mase_mxfp_tile_codes")
+    return tiled
+
+
+def mxfp_pack_tiled(x: Tensor, exp_bits: int, frac_bits: int):
+    """``mxfp_pack`` of a 2-D ``x`` [rows, K] to e4m3 / e5m2 with the codes written as the tile image (flat uint8 of
+    ``mase_mxfp_tiled_bytes(rows, K, 8)`` bytes; the rows that pad the last tile are left unwritten).  Returns
+    ``(tiled codes, scales uint8 [rows, K/32])``."""
+    from ._tables import log2_table
+
+    _lib.require_device(x, "mxfp_pack_tiled")
+    lib = _lib.load()
+    assert x.dim() == 2 and (exp_bits, frac_bits) in ((4, 3), (5, 2))
+    x = x.contiguous()
+    rows, K = x.shape
+    nbytes = lib.mase_mxfp_tiled_bytes(rows, K, 8)
+    assert nbytes > 0, "K must be a multiple of 128"
+    tiled = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    scales = torch.empty(rows, K // 32, dtype=torch.uint8, device=x.device)
+    tab = log2_table(torch.float32, x.device)
+    rc = lib.mase_mxfp_pack_tiled(x.data_ptr(), tiled.data_ptr(), scales.data_ptr(), rows, K, _lib.dtype_code(x),
+                                  exp_bits, frac_bits, tab.data_ptr(), _lib.stream_ptr(x))
+    _lib.check(rc, "mase_mxfp_pack_tiled")
+    return tiled, scales
+
+
+def gemm_mxfp4_scaled_tiled(a_tiled: Tensor, a_scales: Tensor, a_fmt, b_tiled: Tensor, b_scales: Tensor,
+                            bias: Tensor | None, out_dtype: torch.dtype) -> Tensor:
+    """``gemm_mxfp_scaled`` for e4m3 / e5m2 activations and e2m1 weights with both code matrices as tile images
+    (``mxfp_pack_tiled`` / ``mxfp_tile_codes``); the same bits come out."""
+    _lib.require_device(a_tiled, "gemm_mxfp4_scaled_tiled")
+    lib = _lib.load()
+    M, K = a_scales.shape[0], a_scales.shape[1] * 32
+    N = b_scales.shape[0]
+    assert gemm_mxfp4_tiled_supported(M, N, K, a_fmt, (2, 1)) and b_scales.shape[1] * 32 == K
+    assert a_tiled.numel() == lib.mase_mxfp_tiled_bytes(M, K, 8) and b_tiled.numel() == lib.mase_mxfp_tiled_bytes(N, K, 4)
+    out = torch.empty((M, N), dtype=out_dtype, device=a_tiled.device)
+    if bias is not None:
+        bias = bias.contiguous()
+    rows_per_call = max(256, (OPERAND_BYTES_LIMIT // K) // 256 * 256)  # whole row tiles, image below 2^32 bytes per call
+    for r0 in range(0, M, rows_per_call):
+        r1 = min(M, r0 + rows_per_call)
+        rc = lib.mase_gemm_mxfp4_scaled_tiled(
+            a_tiled.data_ptr() + r0 * K, a_scales[r0:r1].data_ptr(), MXFP_HW_FORMATS[tuple(a_fmt)], b_tiled.data_ptr(),
+            b_scales.data_ptr(), bias.data_ptr() if bias is not None else None, out[r0:r1].data_ptr(), r1 - r0, N, K,
+            _lib.DTYPE_CODE[out_dtype], _lib.DTYPE_CODE[bias.dtype] if bias is not None else 0,
+            _lib.stream_ptr(a_tiled),
+        )
+        _lib.check(rc, "mase_gemm_mxfp4_scaled_tiled")
+    return out
+
+
 def gemm_mxfp4_skinny_supported(M: int, N: int, K: int, b_fmt) -> bool:
     return 0 < M <= SKINNY_MAX_ROWS and K % 128 == 0 and tuple(b_fmt) == (2, 1) and N * K // 2 < (1 << 32)
 

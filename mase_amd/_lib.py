@@ -59,6 +59,12 @@ SIGNATURES = {
     "mase_gemm_mxfp4_skinny": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t,
                                        c_size_t, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "mase_mxfp_pack": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "mase_mxfp_tiled_bytes": (c_size_t, [c_size_t, c_size_t, c_int]),
+    "mase_mxfp_tile_codes": (c_int, [c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_void_p]),
+    "mase_mxfp_pack_tiled": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_int, c_int, c_void_p,
+                                     c_void_p]),
+    "mase_gemm_mxfp4_scaled_tiled": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
+                                             c_size_t, c_size_t, c_int, c_int, c_void_p]),
     "mase_gemm_mxfp_scaled": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_int, c_int, c_void_p]),
     "mase_copy_bytes": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "mase_isclose_zero_threshold_bits": (c_uint32, [c_int]),

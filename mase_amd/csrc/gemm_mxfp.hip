@@ -97,7 +97,11 @@ struct MxGemmGeom {
 // in flight while the epilogue of the current one runs, and its stores drain behind the next main loop.
 // STREAM: K holds at least S tiles, so the copy stream is never more than one output tile ahead and advances
 // without branches; the other instantiation (short K) advances it with the general, branching step.
-template <int B_BITS, int CBSZ, int BLGP, int OUT_DT, bool STREAM>
+// TILED: both code matrices come as the images of mase_mxfp_tile_codes / mase_mxfp_pack_tiled, in which the 32 KB (A) or
+// 16 KB (4-bit B) that one K tile of one 256-row tile occupies in an LDS stage lie contiguous and already swizzled, so a
+// wavefront's copy reads one 1 KB run instead of 8 or 16 row segments a whole row apart (K bytes: a stride that keeps
+// hitting the same L2 channels).  The LDS contents, and with them the result, are those of the row-major form.
+template <int B_BITS, int CBSZ, int BLGP, int OUT_DT, bool STREAM, bool TILED = false>
 __global__ __launch_bounds__(kThreadsG) void gemm_mxfp_kernel(MxGemmParams p) {
   using G = MxGemmGeom<B_BITS>;
   constexpr int RA = G::RA, RB = G::RB, kTileA = G::kTileA, kTileB = G::kTileB, kStage = G::kStage, S = G::S;
@@ -156,11 +160,14 @@ __global__ __launch_bounds__(kThreadsG) void gemm_mxfp_kernel(MxGemmParams p) {
 #pragma unroll
     for (int j = 0; j < kCopiesA; ++j) {  // 8 rows of 128 B per copy
       const int r = (wave + 4 * j) * 8 + (lane >> 3);
-      ga[j] = (uint32_t)((size_t)min(m0 + r, p.M - 1) * lda) + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
+      if constexpr (TILED) ga[j] = (uint32_t)(m0 / BM) * (uint32_t)(nk * kTileA) + (wave + 4 * j) * 1024 + lane * 16;
+      else ga[j] = (uint32_t)((size_t)min(m0 + r, p.M - 1) * lda) + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
     }
 #pragma unroll
     for (int j = 0; j < kCopiesB; ++j) {
-      if constexpr (RB == 128) {
+      if constexpr (TILED) {
+        gb[j] = (uint32_t)(n0 / BN) * (uint32_t)(nk * kTileB) + (wave + 4 * j) * 1024 + lane * 16;
+      } else if constexpr (RB == 128) {
         const int r = (wave + 4 * j) * 8 + (lane >> 3);
         gb[j] = (uint32_t)((size_t)min(n0 + r, p.N - 1) * ldbb) + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
       } else {  // 16 rows of 64 B per copy
@@ -185,10 +192,10 @@ __global__ __launch_bounds__(kThreadsG) void gemm_mxfp_kernel(MxGemmParams p) {
   auto issue_copy = [&](int c) __attribute__((always_inline)) {
     const uint32_t st = lds_base + (uint32_t)(c_stage * kStage);
     if (c < kCopiesA) {
-      async_copy<16>(p.A + (size_t)c_kt * RA, ga[c], st + (wave + 4 * c) * 1024);
+      async_copy<16>(p.A + (size_t)c_kt * (TILED ? kTileA : RA), ga[c], st + (wave + 4 * c) * 1024);
     } else if (c < kCopiesA + kCopiesB) {
       const int j = c - kCopiesA;
-      async_copy<16>(p.B + (size_t)c_kt * RB, gb[j], st + kTileA + (wave + 4 * j) * 1024);
+      async_copy<16>(p.B + (size_t)c_kt * (TILED ? kTileB : RB), gb[j], st + kTileA + (wave + 4 * j) * 1024);
     } else if (c == kCopiesA + kCopiesB) {
       async_copy<4>(p.SA + (size_t)c_kt * 4, gsa, st + kTileA + kTileB + wave * 256);
     } else {
@@ -434,7 +441,7 @@ int persistent_grid(int total_tiles) {
   return total_tiles < n_cu ? total_tiles : n_cu;
 }
 
-template <int B_BITS, int CBSZ, int BLGP>
+template <int B_BITS, int CBSZ, int BLGP, bool TILED = false>
 int launch_mx_gemm(const MxGemmParams& p, int out_dtype, hipStream_t st) {
   const size_t lds_bytes = (size_t)MxGemmGeom<B_BITS>::kLdsBytes;
   const int nwg = persistent_grid(p.tiles_m * p.tiles_n);
@@ -444,13 +451,14 @@ int launch_mx_gemm(const MxGemmParams& p, int out_dtype, hipStream_t st) {
 #define MASE_MX_LAUNCH(DT_, STREAM_)                                                                              \
   do {                                                                                                            \
     static bool attr_set = false;                                                                                 \
-    const void* k = (const void*)gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, DT_, STREAM_>;                              \
+    const void* k = (const void*)gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, DT_, STREAM_, TILED>;                       \
     if (!attr_set) {                                                                                              \
       if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)       \
         return MASE_ERR_LAUNCH;                                                                                   \
       attr_set = true;                                                                                            \
     }                                                                                                             \
-    hipLaunchKernelGGL((gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, DT_, STREAM_>), grid, block, lds_bytes, st, p);      \
+    hipLaunchKernelGGL((gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, DT_, STREAM_, TILED>), grid, block, lds_bytes, st,   \
+                       p);                                                                                        \
   } while (0)
   if (stream) {
     if (out_dtype == MASE_DT_F32) MASE_MX_LAUNCH(MASE_DT_F32, true);
@@ -465,8 +473,86 @@ int launch_mx_gemm(const MxGemmParams& p, int out_dtype, hipStream_t st) {
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
 
+// One thread per 16-byte granule of the image: tile (row tile, K tile), row r of the tile, chunk position cl; the
+// source chunk is cl ^ swizzle(r), the source row clamped to the last one as the row-major kernel clamps it.
+template <int BITS>
+__global__ __launch_bounds__(256) void mxfp_tile_codes_kernel(const unsigned char* __restrict__ codes,
+                                                              uint4* __restrict__ tiled, int rows, int K,
+                                                              size_t granules) {
+  constexpr int kRowBytes = BK * BITS / 8;  // 128 or 64
+  constexpr int kChunks = kRowBytes / 16;   // 8 or 4
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= granules) return;
+  const int nk = K / BK;
+  const size_t tile = g / (size_t)(BM * kChunks);
+  const int within = (int)(g % (size_t)(BM * kChunks));
+  const int r = within / kChunks, cl = within % kChunks;
+  const int tm = (int)(tile / (size_t)nk), kt = (int)(tile % (size_t)nk);
+  const int sw = (BITS == 8) ? ((r >> 1) & 7) : ((r >> 2) & 3);
+  const size_t row = (size_t)min(tm * BM + r, rows - 1);
+  const unsigned char* src = codes + row * ((size_t)K * BITS / 8) + (size_t)kt * kRowBytes + ((cl ^ sw) << 4);
+  tiled[g] = *(const uint4*)src;
+}
+
 }  // namespace
 }  // namespace mase
+
+extern "C" size_t mase_mxfp_tiled_bytes(size_t rows, size_t K, int bits) {
+  if (rows == 0 || K == 0 || (K % mase::BK) != 0 || (bits != 4 && bits != 8)) return 0;
+  return ((rows + mase::BM - 1) / mase::BM) * mase::BM * (K * (size_t)bits / 8);
+}
+
+extern "C" int mase_mxfp_tile_codes(const void* codes, void* tiled, size_t rows, size_t K, int bits, void* stream) {
+  using namespace mase;
+  static_assert(BM == BN, "one image geometry for both operands");
+  if (rows == 0 || K == 0) return MASE_OK;
+  if (codes == nullptr || tiled == nullptr) return MASE_ERR_NULL;
+  if (bits != 4 && bits != 8) return MASE_ERR_PARAM;
+  if ((K % BK) != 0 || rows > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
+  if (!aligned16(codes) || !aligned16(tiled)) return MASE_ERR_ALIGN;
+  const size_t granules = mase_mxfp_tiled_bytes(rows, K, bits) / 16;
+  const dim3 grid(blocks_for(granules, (size_t)256)), block(256);
+  if (bits == 8)
+    hipLaunchKernelGGL(mxfp_tile_codes_kernel<8>, grid, block, 0, (hipStream_t)stream, (const unsigned char*)codes,
+                       (uint4*)tiled, (int)rows, (int)K, granules);
+  else
+    hipLaunchKernelGGL(mxfp_tile_codes_kernel<4>, grid, block, 0, (hipStream_t)stream, (const unsigned char*)codes,
+                       (uint4*)tiled, (int)rows, (int)K, granules);
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+extern "C" int mase_gemm_mxfp4_scaled_tiled(const void* A_tiled, const void* A_scales, int a_format, const void* B_tiled,
+                                            const void* B_scales, const void* bias, void* C, size_t M, size_t N,
+                                            size_t K, int out_dtype, int bias_dtype, void* stream) {
+  using namespace mase;
+  if (M == 0 || N == 0) return MASE_OK;
+  if (A_tiled == nullptr || B_tiled == nullptr || A_scales == nullptr || B_scales == nullptr || C == nullptr)
+    return MASE_ERR_NULL;
+  if (K == 0 || (K % BK) != 0 || M > (1u << 30) || N > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
+  // the kernel addresses each image with a 32-bit byte offset from its base
+  if ((unsigned long long)mase_mxfp_tiled_bytes(M, K, 8) > 0xFFFFFFFFull ||
+      (unsigned long long)mase_mxfp_tiled_bytes(N, K, 4) > 0xFFFFFFFFull)
+    return MASE_ERR_SHAPE;
+  if (!aligned16(A_tiled) || !aligned16(B_tiled) || (((uintptr_t)A_scales) & 3u) != 0 || (((uintptr_t)B_scales) & 3u) != 0)
+    return MASE_ERR_ALIGN;
+  if (out_dtype < 0 || out_dtype > 2 || (bias != nullptr && (bias_dtype < 0 || bias_dtype > 2))) return MASE_ERR_DTYPE;
+  if (a_format != 0 && a_format != 1) return MASE_ERR_PARAM;
+  MxGemmParams p;
+  p.A = (const unsigned char*)A_tiled;
+  p.B = (const unsigned char*)B_tiled;
+  p.SA = (const unsigned char*)A_scales;
+  p.SB = (const unsigned char*)B_scales;
+  p.bias = bias;
+  p.C = C;
+  p.M = (int)M;
+  p.N = (int)N;
+  p.K = (int)K;
+  p.bias_dtype = bias_dtype;
+  p.tiles_m = (int)((M + BM - 1) / BM);
+  p.tiles_n = (int)((N + BN - 1) / BN);
+  hipStream_t st = (hipStream_t)stream;
+  return a_format == 0 ? launch_mx_gemm<4, 0, 4, true>(p, out_dtype, st) : launch_mx_gemm<4, 1, 4, true>(p, out_dtype, st);
+}
 
 // a_format / b_format: 0 = e4m3 (8-bit), 1 = e5m2 (8-bit), 4 = e2m1 (4-bit, two codes per byte); A must be 8-bit.
 extern "C" int mase_gemm_mxfp_scaled(const void* A, const void* A_scales, int a_format, const void* B,

@@ -296,9 +296,14 @@ __device__ __forceinline__ bool code_is_reserved(uint32_t c) {
   return false;
 }
 
-template <int DTI, int E, int F>
+// TILED (8-bit codes only): the codes of a [rows, K] matrix go to the image the tiled block-scaled GEMM copies from,
+// [row tile of 256][K tile of 128][row][128 B] with the 16-byte chunks of a row segment exchanged by
+// chunk ^= (row >> 1) & 7 (the GEMM's LDS swizzle); k8 = K / 8 lanes per row.  Scales stay row-major.
+template <int DTI, int E, int F, bool TILED = false>
 __global__ __launch_bounds__(64) void mxfp_pack_kernel(const void* __restrict__ in, uint8_t* __restrict__ codes,
-                                                       uint8_t* __restrict__ scales, size_t n8, MxfpParams p) {
+                                                       uint8_t* __restrict__ scales, size_t n8, MxfpParams p,
+                                                       uint32_t k8) {
+  static_assert(!TILED || E + F + 1 == 8, "the tiled image is written for 8-bit codes");
   using TI = DTypeTraits<DTI>;
   const size_t idx = (size_t)blockIdx.x * 64 + threadIdx.x;  // 8 elements per lane, 4 lanes per block of 32
   const bool live = idx < n8;
@@ -347,7 +352,16 @@ __global__ __launch_bounds__(64) void mxfp_pack_kernel(const void* __restrict__ 
     uint2 w;
     w.x = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
     w.y = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
-    ((uint2*)codes)[idx] = w;
+    if constexpr (TILED) {
+      const size_t m = idx / k8;
+      const uint32_t k0 = (uint32_t)(idx - m * k8) * 8u;  // byte (= element) position in the row
+      const uint32_t r = (uint32_t)m & 255u, kin = k0 & 127u;
+      const size_t tile = (m >> 8) * (size_t)(k8 >> 4) + (k0 >> 7);
+      const uint32_t at = r * 128u + ((((kin >> 4) ^ ((r >> 1) & 7u)) << 4) | (kin & 15u));
+      *(uint2*)(codes + tile * 32768 + at) = w;
+    } else {
+      ((uint2*)codes)[idx] = w;
+    }
   }
 }
 
@@ -356,9 +370,23 @@ int launch_mxfp_pack(const void* in, uint8_t* codes, uint8_t* scales, size_t num
                      hipStream_t st) {
   const size_t n8 = numel / 8;
   const dim3 grid(blocks_for(n8, 64)), block(64);
-  if (E == 4 && F == 3) hipLaunchKernelGGL((mxfp_pack_kernel<DTI, 4, 3>), grid, block, 0, st, in, codes, scales, n8, p);
-  else if (E == 5 && F == 2) hipLaunchKernelGGL((mxfp_pack_kernel<DTI, 5, 2>), grid, block, 0, st, in, codes, scales, n8, p);
-  else if (E == 2 && F == 1) hipLaunchKernelGGL((mxfp_pack_kernel<DTI, 2, 1>), grid, block, 0, st, in, codes, scales, n8, p);
+  if (E == 4 && F == 3) hipLaunchKernelGGL((mxfp_pack_kernel<DTI, 4, 3>), grid, block, 0, st, in, codes, scales, n8, p, 0u);
+  else if (E == 5 && F == 2) hipLaunchKernelGGL((mxfp_pack_kernel<DTI, 5, 2>), grid, block, 0, st, in, codes, scales, n8, p, 0u);
+  else if (E == 2 && F == 1) hipLaunchKernelGGL((mxfp_pack_kernel<DTI, 2, 1>), grid, block, 0, st, in, codes, scales, n8, p, 0u);
+  else return MASE_ERR_PARAM;
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+template <int DTI>
+int launch_mxfp_pack_tiled(const void* in, uint8_t* codes, uint8_t* scales, size_t rows, size_t K, int E, int F,
+                           const MxfpParams& p, hipStream_t st) {
+  const size_t n8 = rows * K / 8;
+  const dim3 grid(blocks_for(n8, 64)), block(64);
+  const uint32_t k8 = (uint32_t)(K / 8);
+  if (E == 4 && F == 3)
+    hipLaunchKernelGGL((mxfp_pack_kernel<DTI, 4, 3, true>), grid, block, 0, st, in, codes, scales, n8, p, k8);
+  else if (E == 5 && F == 2)
+    hipLaunchKernelGGL((mxfp_pack_kernel<DTI, 5, 2, true>), grid, block, 0, st, in, codes, scales, n8, p, k8);
   else return MASE_ERR_PARAM;
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
@@ -433,6 +461,33 @@ extern "C" int mase_mxfp_pack(const void* in, uint8_t* codes, uint8_t* scales, s
     case MASE_DT_F32: return launch_mxfp_pack<MASE_DT_F32>(in, codes, scales, numel, exp_bits, frac_bits, p, st);
     case MASE_DT_BF16: return launch_mxfp_pack<MASE_DT_BF16>(in, codes, scales, numel, exp_bits, frac_bits, p, st);
     case MASE_DT_F16: return launch_mxfp_pack<MASE_DT_F16>(in, codes, scales, numel, exp_bits, frac_bits, p, st);
+    default: return MASE_ERR_DTYPE;
+  }
+}
+
+extern "C" int mase_mxfp_pack_tiled(const void* in, uint8_t* tiled_codes, uint8_t* scales, size_t rows, size_t K,
+                                    int in_dtype, int exp_bits, int frac_bits, const uint32_t* log2_tab, void* stream) {
+  using namespace mase;
+  if (rows == 0 || K == 0) return MASE_OK;
+  if (in == nullptr || tiled_codes == nullptr || scales == nullptr || log2_tab == nullptr) return MASE_ERR_NULL;
+  if (K % 128 != 0 || rows > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
+  if (!aligned16(in) || (((uintptr_t)tiled_codes) & 15u) != 0) return MASE_ERR_ALIGN;
+  if (!((exp_bits == 4 && frac_bits == 3) || (exp_bits == 5 && frac_bits == 2))) return MASE_ERR_PARAM;
+  MxfpParams p;
+  p.m.E = exp_bits;
+  p.m.F = frac_bits;
+  p.m.bias = (1 << (exp_bits - 1)) - 1;
+  p.m.e_hi = (1 << exp_bits) - 1;
+  p.m.frac_hi = (1 << frac_bits) - 1;
+  p.m.is_finite = 1;
+  p.m.round_mode = 0;
+  p.el_emax = p.m.e_hi - p.m.bias;
+  p.tab = log2_tab;
+  hipStream_t st = (hipStream_t)stream;
+  switch (in_dtype) {
+    case MASE_DT_F32: return launch_mxfp_pack_tiled<MASE_DT_F32>(in, tiled_codes, scales, rows, K, exp_bits, frac_bits, p, st);
+    case MASE_DT_BF16: return launch_mxfp_pack_tiled<MASE_DT_BF16>(in, tiled_codes, scales, rows, K, exp_bits, frac_bits, p, st);
+    case MASE_DT_F16: return launch_mxfp_pack_tiled<MASE_DT_F16>(in, tiled_codes, scales, rows, K, exp_bits, frac_bits, p, st);
     default: return MASE_ERR_DTYPE;
   }
 }

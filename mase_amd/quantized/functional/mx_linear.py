@@ -14,7 +14,8 @@ from torch import Tensor
 from torch.nn import functional as F
 
 from ..._gemm import (MXFP_HW_FORMATS, MXFP_K_MULTIPLE, SKINNY_MAX_ROWS, gemm_bf16_pack_b, gemm_bf16_packed_b_supported,
-                      gemm_bf16_takes_packed_b, gemm_bf16_tn, gemm_mxfp4_skinny, gemm_mxfp4_skinny_supported,
+                      gemm_bf16_takes_packed_b, gemm_bf16_tn, gemm_mxfp4_scaled_tiled, gemm_mxfp4_skinny, gemm_mxfp4_skinny_supported,
+                      gemm_mxfp4_tiled_supported, mxfp_pack_tiled, mxfp_tile_codes,
                       gemm_mxfp_scaled, gemm_mxint8_skinny, gemm_mxint8_skinny_supported, mxfp_pack)
 
 
@@ -136,10 +137,22 @@ class PackedMXFPWeight:
         self.codes = None
         self.scales = None
         self.fmt = None
+        self._tiled = None
 
     def invalidate(self):
         self._key = None
-        self.codes = self.scales = self.fmt = None
+        self.codes = self.scales = self.fmt = self._tiled = None
+
+    def tiled(self, K: int):
+        """The e2m1 codes as the tile image the tiled GEMM copies from (``mxfp_tile_codes``), made on the first forward
+        that takes that kernel: another 0.5 bytes per weight.  None while a HIP graph is being captured before the
+        image exists (it must not come from the graph's memory pool)."""
+        if self._tiled is not None and self._tiled[0] is self.codes:
+            return self._tiled[1]
+        if self.codes is None or torch.cuda.is_current_stream_capturing():
+            return None
+        self._tiled = (self.codes, mxfp_tile_codes(self.codes, K, 4))
+        return self._tiled[1]
 
     @staticmethod
     def eligible(weight: Tensor, block_size: int, fmt) -> bool:
@@ -241,6 +254,14 @@ def mxfp_linear_native(x: Tensor, packed: PackedMXFPWeight, bias: Tensor | None,
     weight; accumulation is fp32 and the result is written in x's dtype."""
     lead = x.shape[:-1]
     x2 = x.reshape(-1, x.shape[-1])
+    M, K = x2.shape
+    N = packed.scales.shape[0]
+    if (not gemm_mxfp4_skinny_supported(M, N, K, packed.fmt) and gemm_mxfp4_tiled_supported(M, N, K, act_fmt, packed.fmt)
+            and (w_tiled := packed.tiled(K)) is not None):
+        # both code matrices as tile images (the activations' written directly by the quantizer): same bits, 7 % faster
+        xt, xs = mxfp_pack_tiled(x2, *act_fmt)
+        y = gemm_mxfp4_scaled_tiled(xt, xs, act_fmt, w_tiled, packed.scales, bias, x.dtype)
+        return y.reshape(*lead, N)
     xc, xs = mxfp_pack(x2, *act_fmt)
     if gemm_mxfp4_skinny_supported(x2.shape[0], packed.scales.shape[0], x2.shape[1], packed.fmt):
         # decode-sized batch with MXFP4 weights: bound by streaming the weight codes once (0.53 bytes per weight)

@@ -72,6 +72,23 @@ def test_entry_points_reject_bad_arguments_without_a_gpu(lib):
     assert lib.mase_gemm_bf16_pack_b(p, p, 64, 24, None) == -2
     assert lib.mase_gemm_bf16_pack_b(None, p, 64, 32, None) == -1
     assert lib.mase_gemm_bf16_packed_bytes(33, 64) == 64 * 64 * 2 and lib.mase_gemm_bf16_packed_bytes(32, 24) == 0
+    # mase_gemm_mxfp4_scaled_tiled(A_tiled, A_scales, a_format, B_tiled, B_scales, bias, C, M, N, K, out_dtype,
+    # bias_dtype, stream), the image maker and the activation quantizer that writes the image
+    assert lib.mase_gemm_mxfp4_scaled_tiled(p, p, 0, p, p, None, p, 256, 256, 192, 0, 0, None) == -2  # K % 128
+    assert lib.mase_gemm_mxfp4_scaled_tiled(p, p, 0, None, p, None, p, 256, 256, 512, 0, 0, None) == -1
+    assert lib.mase_gemm_mxfp4_scaled_tiled(p, p, 0, p, p, None, p, 256, 256, 512, 3, 0, None) == -4
+    assert lib.mase_gemm_mxfp4_scaled_tiled(p, p, 4, p, p, None, p, 256, 256, 512, 0, 0, None) == -5  # A must be 8-bit
+    assert lib.mase_gemm_mxfp4_scaled_tiled(p, p, 0, p, p, None, p, 1 << 20, 256, 1 << 13, 0, 0, None) == -2  # image >= 2^32
+    assert lib.mase_gemm_mxfp4_scaled_tiled(p, p, 0, p, p, None, p, 0, 256, 512, 0, 0, None) == 0
+    assert lib.mase_mxfp_tile_codes(p, p, 64, 96, 4, None) == -2
+    assert lib.mase_mxfp_tile_codes(p, p, 64, 128, 6, None) == -5
+    assert lib.mase_mxfp_tile_codes(None, p, 64, 128, 4, None) == -1
+    assert lib.mase_mxfp_tiled_bytes(257, 128, 4) == 512 * 64 and lib.mase_mxfp_tiled_bytes(257, 128, 8) == 512 * 128
+    assert lib.mase_mxfp_tiled_bytes(256, 96, 8) == 0 and lib.mase_mxfp_tiled_bytes(256, 128, 6) == 0
+    assert lib.mase_mxfp_pack_tiled(p, p, p, 4, 96, 0, 4, 3, p, None) == -2
+    assert lib.mase_mxfp_pack_tiled(p, p, p, 4, 128, 0, 2, 1, p, None) == -5   # 8-bit element formats only
+    assert lib.mase_mxfp_pack_tiled(p, p, p, 4, 128, 7, 4, 3, p, None) == -4
+    assert lib.mase_mxfp_pack_tiled(p, None, p, 4, 128, 0, 4, 3, p, None) == -1
     # mase_gemm_mxint8_skinny(A, codes, scales, bias, C, M, N, K, out_dtype, bias_dtype, workspace, workspace_bytes, stream)
     assert lib.mase_gemm_mxint8_skinny(p, p, p, None, p, 4, 4, 192, 0, 0, p, 4096, None) == -2    # K in whole 128-chunks
     assert lib.mase_gemm_mxint8_skinny(p, p, p, None, p, 129, 4, 128, 0, 0, p, 4096, None) == -2

@@ -166,3 +166,70 @@ def test_gemm_mxfp4_few_rows_streams_the_weight_codes(dev, afmt, M):
     da, db = decode_ocp(ac, asc, afmt), decode_ocp(bc, bsc, (2, 1))
     if torch.equal(da.float(), ai) and torch.equal(db.float(), bi):
         assert torch.equal(gemm_mxfp4_skinny(ac, asc, afmt, bc, bsc, None, torch.float32).cpu().double(), da @ db.t())
+
+
+def tile_image(codes: torch.Tensor, bits: int) -> torch.Tensor:
+    """The tile image of a row-major code matrix, spelled out with indices: [row tile of 256][K tile of 128][row]
+    [128 or 64 bytes], 16-byte chunk c of a row segment at position c ^ swizzle(row), rows past the end repeating the last."""
+    codes = codes.cpu()
+    rows, row_bytes = codes.shape
+    seg = 128 * bits // 8
+    nk = row_bytes // seg
+    tiles = -(-rows // 256)
+    r = torch.arange(tiles * 256).clamp(max=rows - 1)
+    src = codes[r].reshape(tiles, 256, nk, seg // 16, 16)
+    rr = torch.arange(256)
+    sw = ((rr >> 1) & 7) if bits == 8 else ((rr >> 2) & 3)
+    pos = torch.arange(seg // 16)[None, :] ^ sw[:, None]              # [256, chunks]: position -> source chunk
+    img = src[:, rr[:, None], :, pos, :]                                # [256, chunks, tiles, nk, 16]
+    return img.permute(2, 3, 0, 1, 4).reshape(-1).contiguous()
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("rows,K", [(256, 128), (300, 384), (1, 256), (777, 1024)])
+def test_mxfp_tile_codes_is_the_stated_permutation(dev, bits, rows, K):
+    from mase_amd._gemm import mxfp_tile_codes
+
+    g = torch.Generator().manual_seed(rows + K + bits)
+    codes = torch.randint(0, 256, (rows, K * bits // 8), generator=g, dtype=torch.uint8)
+    got = mxfp_tile_codes(codes.to(dev), K, bits).cpu()
+    assert torch.equal(got, tile_image(codes, bits))
+
+
+@pytest.mark.parametrize("fmt", [(4, 3), (5, 2)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,K", [(256, 128), (300, 384), (3, 1024)])
+def test_mxfp_pack_tiled_writes_the_image_of_the_row_major_codes(dev, fmt, dtype, rows, K):
+    from mase_amd._gemm import mxfp_pack, mxfp_pack_tiled
+
+    rng = np.random.default_rng(rows + K)
+    x = adversarial(rng, (rows, K), dtype, block=32)
+    x = torch.where(x.float().abs() < 1e4, x, torch.zeros_like(x)).to(dev)
+    codes, scales = mxfp_pack(x, *fmt)
+    tiled, tscales = mxfp_pack_tiled(x, *fmt)
+    assert torch.equal(scales, tscales)
+    want = tile_image(codes, 8).reshape(-1, K // 128, 256, 128)
+    got = tiled.cpu().reshape(-1, K // 128, 256, 128)
+    live = torch.arange(want.shape[0] * 256).reshape(-1, 256) < rows   # padding rows are left unwritten
+    assert torch.equal(got.permute(0, 2, 1, 3)[live], want.permute(0, 2, 1, 3)[live])
+
+
+@pytest.mark.parametrize("afmt", [(4, 3), (5, 2)])
+@pytest.mark.parametrize("out_dtype,with_bias", [(torch.bfloat16, False), (torch.float32, True), (torch.float16, True)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 200, 384), (512, 768, 1024), (129, 33, 256), (1024, 512, 2048)])
+def test_gemm_mxfp4_on_tile_images_is_the_same_product(dev, afmt, out_dtype, with_bias, M, N, K):
+    from mase_amd._gemm import gemm_mxfp4_scaled_tiled, gemm_mxfp_scaled, mxfp_pack, mxfp_pack_tiled, mxfp_tile_codes
+
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+    bias = torch.randn(N, generator=g).to(out_dtype).to(dev) if with_bias else None
+    xc, xs = mxfp_pack(x, *afmt)
+    wc, ws = mxfp_pack(w, 2, 1)
+    want = gemm_mxfp_scaled(xc, xs, afmt, wc, ws, (2, 1), bias, out_dtype)
+    xt, xts = mxfp_pack_tiled(x, *afmt)
+    got = gemm_mxfp4_scaled_tiled(xt, xts, afmt, mxfp_tile_codes(wc, K, 4), ws, bias, out_dtype)
+    assert torch.equal(got, want)
+    # the activation image made from the row-major codes gives the same product as the one the quantizer writes
+    got2 = gemm_mxfp4_scaled_tiled(mxfp_tile_codes(xc, K, 8), xs, afmt, mxfp_tile_codes(wc, K, 4), ws, bias, out_dtype)
+    assert torch.equal(got2, want)
