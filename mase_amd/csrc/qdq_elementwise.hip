@@ -265,6 +265,8 @@ struct MinifloatOp {
 // inside the clamp range (fp16 always; bf16 when e_lo >= -20), 1 = fp32 add, 2 = add and round to bf16.
 // Non-finite elements take the stepwise evaluation with the table read from memory.
 // ---------------------------------------------------------------------------------------------
+constexpr int kValueItems = 2;
+
 template <int DT, bool IEEE, int EPS>
 __global__ __launch_bounds__(kEwThreads) void minifloat_value_kernel(const void* __restrict__ in, void* __restrict__ out,
                                                                      size_t n8, MinifloatOp<DT, IEEE> op) {
@@ -274,19 +276,30 @@ __global__ __launch_bounds__(kEwThreads) void minifloat_value_kernel(const void*
   const int E_l = 95 + ((lane - 95) & 63);
   const uint32_t thr = op.tab[(IEEE ? kLog2TabHalf : 0) + 149 + (E_l - 127)];
   const uint32_t delta = IEEE ? (0x800000u - thr) : (0x7FFFFFu - thr);
-  const size_t t = (size_t)blockIdx.x * kEwThreads + threadIdx.x;
-  const bool live = t < n8;
-  const size_t item = live ? t : n8 - 1;  // every lane takes part in the register permutes
-  float x[8], y[8];
-  load8<DT, true>(in, item, n8, x);
+  // kValueItems items per lane, 64 items apart, all loaded before the first is worked on: with one item per lane the
+  // wavefronts a CU can hold keep too few bytes in flight once an item takes ~140 instructions
+  const size_t t0 = (size_t)blockIdx.x * (kEwThreads * kValueItems) + threadIdx.x;
+  float xs[kValueItems][8];
+#pragma unroll
+  for (int u = 0; u < kValueItems; ++u) {
+    const size_t t = t0 + (size_t)u * kEwThreads;
+    load8<DT, true>(in, t < n8 ? t : n8 - 1, n8, xs[u]);  // every lane takes part in the register permutes
+  }
   // clamp bounds of the exponent in place, and the constants that turn (e + 127) << 23 into the rounding constant
   // and into the upper bound of |y| (mb >= 1 for the denorm flavour, checked by the launcher)
   const uint32_t lo_f = (uint32_t)(op.e_lo_i + 127) << 23, hi_f = ((uint32_t)(op.e_hi_i + 127) << 23) | 0x7FFFFFu;
-  const uint32_t k_magic = ((uint32_t)(23 - op.mb) << 23) + 0x400000u;
-  const uint32_t k_cap = IEEE ? (0x800000u - (0x800000u >> op.mb))                    // (2 - 2^-mb) * 2^e
+  uint32_t k_magic = ((uint32_t)(23 - op.mb) << 23) + 0x400000u;
+  uint32_t k_cap = IEEE ? (0x800000u - (0x800000u >> op.mb))                    // (2 - 2^-mb) * 2^e
                               : (0x800000u - (0x1000000u >> op.mb)) - 0x800000u;      // (2 - 2^(1-mb)) * 2^(e-1)
-  [[maybe_unused]] const float c_sub = bits2f(lo_f + k_magic + 0x800000u);
   [[maybe_unused]] const float cap_sub = op.mb == 0 ? 0.0f : bits2f(lo_f + (0x800000u - (0x1000000u >> op.mb)));
+  // one scalar each: left visible, the sums would be taken apart again into two vector additions per element
+  asm volatile("" : "+s"(k_magic), "+s"(k_cap));
+#pragma unroll
+  for (int u = 0; u < kValueItems; ++u) {
+  const size_t t = t0 + (size_t)u * kEwThreads;
+  const bool live = t < n8;
+  float* x = xs[u];
+  float y[8];
   uint32_t worst = 0;
   uint32_t lbs[8], ds[8];
   // all eight permutes are issued before the first result is needed
@@ -297,19 +310,22 @@ __global__ __launch_bounds__(kEwThreads) void minifloat_value_kernel(const void*
     if constexpr (EPS == 1) lb = f2bits(bits2f(ab) + 1e-9f);
     if constexpr (EPS == 2) lb = f2bits(TR::round(bits2f(ab) + 1e-9f));
     lbs[j] = lb;
-    ds[j] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((lb >> 21) & 0xFCu), (int)delta);
+    // the permute takes its source lane from address bits 7:2 and ignores the rest: (lb >> 23) mod 64
+    ds[j] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(lb >> 21), (int)delta);
   }
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const uint32_t xb = f2bits(x[j]);
-    const uint32_t ab = xb & 0x7FFFFFFFu;
+    const uint32_t lb = lbs[j], d = ds[j];
+    const uint32_t ab = (EPS == 0) ? lb : (xb & 0x7FFFFFFFu);
     const float val = bits2f(ab);
     worst = max(worst, ab);
-    const uint32_t lb = lbs[j], d = ds[j];
     // e clamped, kept in place as the exponent field: ebs = (e + 127) << 23
+    // (the ieee flavour clamps at e_lo + 1 instead: an element with e == e_lo is rounded on the grid of e_lo + 1)
+    const uint32_t kraw = lb + d;
     uint32_t c;
-    asm("v_med3_u32 %0, %1, %2, %3" : "=v"(c) : "v"(lb + d), "s"(lo_f), "v"(hi_f));  // one scalar operand at most
+    asm("v_med3_u32 %0, %1, %2, %3" : "=v"(c) : "v"(kraw), "s"(IEEE ? lo_f + 0x800000u : lo_f), "v"(hi_f));  // one scalar operand at most
     const uint32_t ebs = c & 0x7F800000u;
     // rounding to the grid 2^(e-mb) by adding and subtracting 1.5 * 2^(23+e-mb) (exact while |x| < 2^(22+e-mb);
     // beyond that the result only has to stay at or above the upper clamp bound, which it does)
@@ -317,15 +333,18 @@ __global__ __launch_bounds__(kEwThreads) void minifloat_value_kernel(const void*
     if constexpr (!IEEE) {
       const float C = bits2f(ebs + k_magic);
       const float r = (val + C) - C;
-      yabs = fminf(r, bits2f(ebs + k_cap));  // qmax * 2^(e-mb)
+      // r >= +0: the order of the bit patterns is the order of the values, and an integer minimum needs no
+      // canonicalizing move of the bound first
+      yabs = bits2f(min(f2bits(r), ebs + k_cap));  // qmax * 2^(e-mb)
     } else {
       // e == e_lo: grid 2^(e-mb+1), range [0, qmax * 2^(e-mb+1)];  otherwise [2^e, (2^(mb+1) - 1) * 2^(e-mb)]
-      const bool sub = c < lo_f + 0x800000u;
-      const float C = sub ? c_sub : bits2f(ebs + k_magic);
-      const float lo = sub ? 0.0f : bits2f(ebs);
-      const float hi = sub ? cap_sub : bits2f(ebs + k_cap);
+      const bool sub = kraw < lo_f + 0x800000u;
+      const float C = bits2f(ebs + k_magic);
+      const uint32_t lo = sub ? 0u : ebs;
+      const uint32_t hi = sub ? f2bits(cap_sub) : ebs + k_cap;
       const float r = (val + C) - C;
-      yabs = __builtin_amdgcn_fmed3f(r, lo, hi);
+      // r, lo, hi >= +0: clamped as bit patterns (same order as the values, no canonicalizing moves)
+      yabs = bits2f(min(max(f2bits(r), lo), hi));
     }
     const uint32_t yb = (f2bits(yabs) & 0x7FFFFFFFu) | (xb & 0x80000000u);
     // isclose(x, 0): the element passes through, and both zeros become +0 (x + 0.0).  A bitwise select: a
@@ -336,10 +355,15 @@ __global__ __launch_bounds__(kEwThreads) void minifloat_value_kernel(const void*
   }
   if (__builtin_expect(worst >= 0x7F800000u, 0)) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
-      if ((f2bits(x[j]) & 0x7FFFFFFFu) >= 0x7F800000u) y[j] = op.stepwise_from_memory(x[j]);
+    for (int j = 0; j < 8; ++j) {
+      // an opaque copy: terms of the rare path must not be shared with (and so computed on) the common path
+      float xj = x[j];
+      asm volatile("" : "+v"(xj));
+      if ((f2bits(xj) & 0x7FFFFFFFu) >= 0x7F800000u) y[j] = op.stepwise_from_memory(xj);
+    }
   }
-  if (live) store8<DT, true>(out, item, n8, y);
+  if (live) store8<DT, true>(out, t, n8, y);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -446,12 +470,12 @@ struct MinifloatRun {
     op.fast_ok = sig <= sig_T && op.e_hi_i <= max_e && op.e_lo_i - op.mb >= min_step &&
                  op.qmax == (float)((1 << op.mb) - 1) && op.neg_bias == (float)(-bias) && bias < 256;
     // value-level kernel on the 16-byte-aligned vector part, the general kernel on what is left
-    const bool window = op.e_lo_i >= -32 && op.e_hi_i <= 31 && op.mb <= 16 && (IEEE || op.mb >= 1);
+    const bool window = op.e_lo_i >= -32 && op.e_hi_i <= 31 && op.mb <= 16 && (IEEE ? op.e_hi_i > op.e_lo_i : op.mb >= 1);
     size_t done = 0;
     if (op.fast_ok && window && aligned16(in) && aligned16(out) && numel >= 8) {
       const size_t n8 = numel / 8;
       const int eps = (DT == MASE_DT_F16) ? 0 : (DT == MASE_DT_F32 ? 1 : (op.e_lo_i >= -20 ? 0 : 2));
-      const dim3 grid(blocks_for(n8, kEwThreads)), block(kEwThreads);
+      const dim3 grid(blocks_for(n8, kEwThreads * kValueItems)), block(kEwThreads);
       if (eps == 0) hipLaunchKernelGGL((minifloat_value_kernel<DT, IEEE, 0>), grid, block, 0, st, in, out, n8, op);
       else if (eps == 1) hipLaunchKernelGGL((minifloat_value_kernel<DT, IEEE, 1>), grid, block, 0, st, in, out, n8, op);
       else hipLaunchKernelGGL((minifloat_value_kernel<DT, IEEE, 2>), grid, block, 0, st, in, out, n8, op);
