@@ -400,9 +400,19 @@ __global__ __launch_bounds__(kEwThreads) void minifloat_mx_pk16_kernel(const uin
                                                                        uint4* __restrict__ out, size_t n8,
                                                                        MinifloatPk16Params p) {
   constexpr int MB = (DT == MASE_DT_BF16) ? 7 : 10;
-  const size_t i = (size_t)blockIdx.x * kEwThreads + threadIdx.x;
+  // kValueItems items per lane, 64 items apart, all loaded first (more bytes in flight per wavefront)
+  const size_t i0 = (size_t)blockIdx.x * (kEwThreads * kValueItems) + threadIdx.x;
+  uint4 vs[kValueItems];
+#pragma unroll
+  for (int u = 0; u < kValueItems; ++u) {
+    const size_t i = i0 + (size_t)u * kEwThreads;
+    vs[u] = i < n8 ? load_nt(in + i) : make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int u = 0; u < kValueItems; ++u) {
+  const size_t i = i0 + (size_t)u * kEwThreads;
   if (i >= n8) return;
-  const uint4 v = load_nt(in + i);
+  const uint4 v = vs[u];
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};
   uint32_t r[4];
   u16x2 lo_acc = as_u16x2(0xFFFFFFFFu), hi_acc = as_u16x2(0u);
@@ -419,6 +429,7 @@ __global__ __launch_bounds__(kEwThreads) void minifloat_mx_pk16_kernel(const uin
     o = DTypeTraits<DT>::pack(y);
   }
   store_nt(out + i, o);
+  }
 }
 
 template <typename MakeOp>
@@ -512,7 +523,7 @@ struct MinifloatMxRun {
       bool sub = false;
       if (out_dtype == DTI && aligned16(in) && aligned16(out) && numel >= 8 && pk16_params<DTI>(q, sub)) {
         const size_t n8 = numel / 8;
-        const dim3 grid(blocks_for(n8, kEwThreads)), block(kEwThreads);
+        const dim3 grid(blocks_for(n8, kEwThreads * kValueItems)), block(kEwThreads);
         if (sub) hipLaunchKernelGGL((minifloat_mx_pk16_kernel<DTI, true>), grid, block, 0, st, (const uint4*)in, (uint4*)out, n8, q);
         else hipLaunchKernelGGL((minifloat_mx_pk16_kernel<DTI, false>), grid, block, 0, st, (const uint4*)in, (uint4*)out, n8, q);
         if (hipGetLastError() != hipSuccess) return MASE_ERR_LAUNCH;

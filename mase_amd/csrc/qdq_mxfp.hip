@@ -118,16 +118,28 @@ struct MxfpPk16Params {
   int parity0;        // (format bias - T bias) & 1
 };
 
+constexpr int kPk16Items = 2;
+
 template <int DT, int LPB, bool SUBN>
 __global__ __launch_bounds__(kVecThreads) void mxfp_qdq_pk16_kernel(const uint4* __restrict__ in, uint4* __restrict__ out,
                                                                     size_t n_vec, MxfpParams p, MxfpPk16Params q) {
   using TR = DTypeTraits<DT>;
   constexpr int MB = (DT == MASE_DT_BF16) ? 7 : 10;
-  const size_t idx = (size_t)blockIdx.x * kVecThreads + threadIdx.x;
-  const bool live = idx < n_vec;  // whole blocks are live or dead together: n_vec is a multiple of LPB
   WaveLog2 meta;
   meta.init(p.tab, kLog2TabHalf);
-  const uint4 raw = live ? load_nt(in + idx) : make_uint4(0, 0, 0, 0);
+  // kPk16Items vectors per lane, a work-group's width apart, all loaded first (more bytes in flight per wavefront)
+  const size_t idx0 = (size_t)blockIdx.x * (kVecThreads * kPk16Items) + threadIdx.x;
+  uint4 raws[kPk16Items];
+#pragma unroll
+  for (int u = 0; u < kPk16Items; ++u) {
+    const size_t idx = idx0 + (size_t)u * kVecThreads;
+    raws[u] = idx < n_vec ? load_nt(in + idx) : make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int u = 0; u < kPk16Items; ++u) {
+  const size_t idx = idx0 + (size_t)u * kVecThreads;
+  const bool live = idx < n_vec;  // whole blocks are live or dead together: n_vec is a multiple of LPB
+  const uint4 raw = raws[u];
   const uint32_t m = group_max_u32<LPB>(vec_flushed_absmax<DT>(raw));
   int sh = 0;
   const int state = mxfp_block_scale(m, p, sh, meta);
@@ -160,6 +172,7 @@ __global__ __launch_bounds__(kVecThreads) void mxfp_qdq_pk16_kernel(const uint4*
     o = TR::pack(z);
   }
   if (live) store_nt(out + idx, o);
+  }
 }
 
 template <int DTI, int DTO>
@@ -206,12 +219,13 @@ int launch_mxfp(const void* in, void* out, uint8_t* codes, uint8_t* scales, size
         q.parity0 = (p.m.bias - EB) & 1;
         const uint4* src = (const uint4*)in;
         uint4* dst = (uint4*)out;
+        const dim3 grid_pk(blocks_for(n_vec, (size_t)kVecThreads * kPk16Items));
 #define MASE_MXFP_PK(LPB_)                                                                                          \
   do {                                                                                                              \
     if (p.m.E >= 4)                                                                                                 \
-      hipLaunchKernelGGL((mxfp_qdq_pk16_kernel<DTI, LPB_, false>), grid, block, 0, st, src, dst, n_vec, p, q);      \
+      hipLaunchKernelGGL((mxfp_qdq_pk16_kernel<DTI, LPB_, false>), grid_pk, block, 0, st, src, dst, n_vec, p, q);   \
     else                                                                                                            \
-      hipLaunchKernelGGL((mxfp_qdq_pk16_kernel<DTI, LPB_, true>), grid, block, 0, st, src, dst, n_vec, p, q);       \
+      hipLaunchKernelGGL((mxfp_qdq_pk16_kernel<DTI, LPB_, true>), grid_pk, block, 0, st, src, dst, n_vec, p, q);    \
   } while (0)
         switch (lpb) {
           case 1: MASE_MXFP_PK(1); break;
