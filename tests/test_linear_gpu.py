@@ -173,6 +173,15 @@ def test_linear_mxfp_native_path_shapes_bias_and_invalidation(dev, dtype, wfmt):
     e = rel_err(y, ref)
     print(f"LinearMXFP native {dtype} w=e{wfmt[0]}m{wfmt[1]}: rel err {e:.3e}")
     assert e < (TOL if dtype != torch.float32 else 2e-3)
+    if wfmt == (2, 1):
+        # 600 rows of e2m1 weights take the kernel that reads tile images; same bits as the row-major kernel
+        from mase_amd._gemm import gemm_mxfp_scaled, mxfp_pack
+
+        pk = m._w_packed
+        assert pk._tiled is not None and pk._tiled[0] is pk.codes
+        xc, xs = mxfp_pack(x.to(dev).reshape(-1, 1024), 4, 3)
+        y_rm = gemm_mxfp_scaled(xc, xs, (4, 3), pk.codes, pk.scales, pk.fmt, m.bias.data, dtype)
+        assert torch.equal(y.reshape(-1, 768), y_rm)
     # same module with the matrix instruction switched off: the two paths agree to the same bound
     m2 = LinearMXFP(1024, 768, bias=True, device=dev, dtype=dtype, config=dict(cfg, native_mx=False))
     m2.load_state_dict({"weight": w, "bias": b})
