@@ -51,6 +51,11 @@ def make_mxint_input(torch, seed=0):
 
 class Workload:
     name = ""
+    # Defaults of --steps / --warmup.  The timed region has to last tens of milliseconds for the clocks and the memory
+    # system to reach their steady state: 200 steps of a 45 us kernel (9 ms) read 5.7-5.9 TB/s where 1000 steps after
+    # 300 warm-up steps read 6.5 TB/s.  Workloads with long steps override these.
+    default_steps = 2000
+    default_warmup = 300
     metric = ""
     unit = ""
     dtype = ""
@@ -182,6 +187,7 @@ class CopyBytes(Workload):
 
 class MxintLinear(Workload):
     name = "mxint_linear"
+    default_steps, default_warmup = 1000, 100
     metric = "MXINT8 Linear forward throughput (2*M*N*K flop per step; activation quantization included in the step)"
     unit = "TFLOP/s"
     dtype = "bf16"
@@ -246,6 +252,7 @@ class MxintLinear(Workload):
 
 class MxfpLinear(Workload):
     name = "mxfp_linear"
+    default_steps, default_warmup = 300, 50
     metric = ("MXFP8 x MXFP4 Linear forward throughput (2*M*N*K flop per step; activation quantization to packed "
               "codes included in the step)")
     unit = "TFLOP/s"
@@ -316,6 +323,7 @@ class MxfpLinear(Workload):
 
 class DecoderLayerMxint(Workload):
     name = "decoder_layer"
+    default_steps, default_warmup = 100, 10
     metric = ("Llama-style decoder layer forward with MXINT8 Linears (flop per step = 7 Linears + causal attention; "
               "RMSNorm, rotary embedding and the SwiGLU product run as one-pass kernels, attention as the library's "
               "scaled_dot_product_attention, all inside the step)")
@@ -483,6 +491,7 @@ class MxfpQdq(_ElementwiseQdq):
 class MxintClipSearch(_ElementwiseQdq):
     """mxint_quantizer(quantile_search=True): 11 candidate scales per block of 32, the weight-loading path of LinearMXInt
     with config["clip_search"]"""
+    default_steps, default_warmup = 1000, 100
     name, unit, kernel = "mxint_clip_search", "GB/s", "mxint_clip_search_kernel"
     fn_name, args = "mxint_quantizer", (32, 4, -1, 8, True)
     oracle_name, oracle_args = "mxint_quantizer", (32, 4, -1, 8, True)
@@ -506,6 +515,7 @@ class MinifloatMxQdq(_ElementwiseQdq):
 class AttnProb(Workload):
     """score -> probability chain of the MX-quantized Llama attention (scale, causal mask, minifloat cast e5m8,
     fp32 softmax, MXINT8 blocks of 32) on [4,32,2048,2048]"""
+    default_steps, default_warmup = 300, 50
     name = "attn_prob"
     unit = "GB/s"
     kernel = "attn_prob_kernel"
@@ -683,8 +693,8 @@ def load_traffic(name):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=None, help="timed steps (default: the workload's own)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed warm-up steps (default: the workload's own)")
     ap.add_argument("--workload", default="bfp_qdq", choices=sorted(WORKLOADS))
     ap.add_argument("--buffers", type=int, default=4)
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f32", "f16"],
@@ -705,6 +715,10 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     w = WORKLOADS[a.workload]()
+    if a.steps is None:
+        a.steps = w.default_steps
+    if a.warmup is None:
+        a.warmup = w.default_warmup
     if hasattr(w, "torch_dtype"):
         w.torch_dtype = {"bf16": torch.bfloat16, "f32": torch.float32, "f16": torch.float16}[a.dtype]
     w.setup(torch, dev, a.buffers)
