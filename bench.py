@@ -4,8 +4,11 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident in HBM.
+Without --workload the five headline configurations run one after the other and the ONE JSON line carries config 2
+as its headline fields (--steps / --warmup apply to it) and all five under "configs", each with its whole-step
+throughput, the dominant kernel's roofline fraction and its CPU baseline.
 Workloads (the headline configurations):
-    bfp_qdq      config 2 (default): block-FP quantize-dequantize, bf16 [8,2048,4096], width 8, exp 8, block [1,16]
+    bfp_qdq      config 2 (headline): block-FP quantize-dequantize, bf16 [8,2048,4096], width 8, exp 8, block [1,16]
     mxint_qdq    config 1: MXINT8 quantize-dequantize, fp32 [4096,4096], block 32
     mxint_linear config 3: MXINT8 Linear forward, 4096x4096x4096, fp32 in/out
     mxfp_linear  config 4: MXFP4(e2m1) weights x MXFP8(e4m3) activations Linear, M=8192 K=8192 N=28672
@@ -682,12 +685,96 @@ WORKLOADS = {w.name: w for w in (MxintClipSearch, BfpQdq, MxintQdq, MxintLinear,
 
 
 def load_traffic(name):
-    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE), if a summary is committed."""
-    path = os.path.join(ROOT, "profiles", f"traffic_{name}.json")
+    """HBM bytes per launch of the dominant kernel, measured beforehand with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE,
+    two separate runs) and committed as a summary; None when there is none.  It is not measured by this run."""
+    rel = os.path.join("profiles", f"traffic_{name}.json")
+    path = os.path.join(ROOT, rel)
     if os.path.exists(path):
         with open(path) as f:
-            return json.load(f).get("traffic_bytes_per_launch")
-    return None
+            return json.load(f).get("traffic_bytes_per_launch"), rel
+    return None, None
+
+
+HEADLINE = ("bfp_qdq", "mxint_qdq", "mxint_linear", "mxfp_linear", "decoder_layer")  # configs 2, 1, 3, 4, 5
+SETTLE_SECONDS = 0.06  # untimed run-in before the warm-up steps, so that clocks and memory system are at steady state
+
+
+def measure(torch, dev, name, steps, warmup, a):
+    """One workload: W warm-up steps, K wall-clock-timed steps bracketed by synchronisation, K event-timed launches
+    of the dominant kernel, the CPU baseline leg.  Returns the fields of a bench line for it."""
+    w = WORKLOADS[name]()
+    steps = w.default_steps if steps is None else steps
+    warmup = w.default_warmup if warmup is None else warmup
+    if hasattr(w, "torch_dtype"):
+        w.torch_dtype = {"bf16": torch.bfloat16, "f32": torch.float32, "f16": torch.float16}[a.dtype]
+    w.setup(torch, dev, a.buffers)
+    # run-in (not counted as steps): short timed regions otherwise read the ramp of the clocks, not the kernel
+    t0 = time.perf_counter()
+    settle = 0
+    while time.perf_counter() - t0 < SETTLE_SECONDS:
+        w.step(settle)
+        settle += 1
+        if settle % 16 == 0:
+            torch.cuda.synchronize()
+    for i in range(warmup):
+        w.step(i)
+    torch.cuda.synchronize()
+
+    # whole-job timing: wall clock bracketed by synchronisation
+    t0 = time.perf_counter()
+    for i in range(steps):
+        w.step(i)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    # kernel timing: one HIP event pair on the launch stream (torch's current stream is the one handed to the
+    # C ABI) around K back-to-back launches; average launch duration = elapsed / K
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    dominant = getattr(w, "dominant_step", w.step)
+    e0.record()
+    for i in range(steps):
+        dominant(i)
+    e1.record()
+    torch.cuda.synchronize()
+    k_avg = e0.elapsed_time(e1) / steps
+
+    work = w.work_per_step()
+    scale = 1e9 if w.bound == "hbm" else 1e12
+    value = work * steps / wall / scale
+    dominant_work = w.dominant_work() if hasattr(w, "dominant_work") else work
+    achieved = dominant_work / (k_avg * 1e-3) / scale
+    peak = HBM_PEAK_GBS if w.bound == "hbm" else MFMA_PEAK_TFLOPS[getattr(w, "mfma_dtype", "bf16")]
+    traffic, traffic_src = load_traffic(w.name)
+    cpu = None if a.no_cpu else w.cpu_baseline(torch, a.cpu_seconds)
+    out = {
+        "workload": w.name,
+        "metric": w.metric,
+        "value": round(value, 2),
+        "unit": w.unit,
+        "steps": steps,
+        "warmup": warmup,
+        "settle_steps": settle,
+        "ms_per_step": round(wall / steps * 1e3, 5),
+        "whole_step_frac": round(value / peak, 4),
+        "dtype": w.dtype,
+        "config": w.config,
+        "roofline": {
+            "bound": w.bound,
+            "kernel": w.kernel,
+            "achieved": round(achieved, 2),
+            "peak": peak,
+            "unit": "GB/s" if w.bound == "hbm" else "TFLOP/s",
+            "frac": round(achieved / peak, 4),
+            "traffic": traffic,
+            "traffic_source": traffic_src,
+            "kernel_ms_avg": round(k_avg, 5),
+        },
+        "cpu_baseline": cpu,
+    }
+    del w
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    return out
 
 
 def main():
@@ -695,12 +782,14 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default: the workload's own)")
     ap.add_argument("--warmup", type=int, default=None, help="untimed warm-up steps (default: the workload's own)")
-    ap.add_argument("--workload", default="bfp_qdq", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="all", choices=["all"] + sorted(WORKLOADS),
+                    help="all (default): the five headline configurations, config 2 as the headline of the line")
     ap.add_argument("--buffers", type=int, default=4)
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f32", "f16"],
                     help="tensor dtype of the secondary workloads (the headline ones fix theirs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--cpu-seconds", type=float, default=None,
+                    help="budget of each CPU baseline leg (default 15 for one workload, 6 each for all)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); multi-GPU sharding is a design note, not code",
@@ -714,68 +803,39 @@ def main():
         sys.exit(3)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    w = WORKLOADS[a.workload]()
-    if a.steps is None:
-        a.steps = w.default_steps
-    if a.warmup is None:
-        a.warmup = w.default_warmup
-    if hasattr(w, "torch_dtype"):
-        w.torch_dtype = {"bf16": torch.bfloat16, "f32": torch.float32, "f16": torch.float16}[a.dtype]
-    w.setup(torch, dev, a.buffers)
-    for i in range(a.warmup):
-        w.step(i)
-    torch.cuda.synchronize()
-
-    # whole-job timing: wall clock bracketed by synchronisation
-    t0 = time.perf_counter()
-    for i in range(a.steps):
-        w.step(i)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-
-    # kernel timing: one HIP event pair on the launch stream (torch's current stream is the one handed to the
-    # C ABI) around K back-to-back launches; average launch duration = elapsed / K
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    dominant = getattr(w, "dominant_step", w.step)
-    e0.record()
-    for i in range(a.steps):
-        dominant(i)
-    e1.record()
-    torch.cuda.synchronize()
-    k_avg = e0.elapsed_time(e1) / a.steps
-
-    work = w.work_per_step()
-    scale = 1e9 if w.bound == "hbm" else 1e12
-    value = work * a.steps / wall / scale
-    dominant_work = w.dominant_work() if hasattr(w, "dominant_work") else work
-    achieved = dominant_work / (k_avg * 1e-3) / scale
-    peak = HBM_PEAK_GBS if w.bound == "hbm" else MFMA_PEAK_TFLOPS[getattr(w, "mfma_dtype", "bf16")]
+    if a.cpu_seconds is None:
+        a.cpu_seconds = 6.0 if a.workload == "all" else 15.0
+    names = HEADLINE if a.workload == "all" else (a.workload,)
+    results = []
+    for i, name in enumerate(names):
+        # --steps / --warmup apply to the headline workload; the other configurations of `all` run their own counts
+        # (stated in their entries), sized so that each timed region lasts tens of milliseconds
+        r = measure(torch, dev, name, a.steps if i == 0 else None, a.warmup if i == 0 else None, a)
+        print(f"bench.py: {name}: {r['value']} {r['unit']} whole step ({r['whole_step_frac']:.3f} of peak), dominant "
+              f"kernel {r['roofline']['frac']:.3f} of peak", file=sys.stderr, flush=True)
+        results.append(r)
+    head = results[0]
     out = {
-        "metric": w.metric,
-        "value": round(value, 2),
-        "unit": w.unit,
+        "metric": head["metric"],
+        "value": head["value"],
+        "unit": head["unit"],
         "n_gpus": 1,
-        "steps": a.steps,
-        "warmup": a.warmup,
-        "ms_per_step": round(wall / a.steps * 1e3, 5),
+        "steps": head["steps"],
+        "warmup": head["warmup"],
+        "ms_per_step": head["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": w.dtype,
+        "dtype": head["dtype"],
         "data": "synthetic",
-        "config": w.config,
-        "roofline": {
-            "bound": w.bound,
-            "kernel": w.kernel,
-            "achieved": round(achieved, 2),
-            "peak": peak,
-            "unit": "GB/s" if w.bound == "hbm" else "TFLOP/s",
-            "frac": round(achieved / peak, 4),
-            "traffic": load_traffic(w.name),
-            "kernel_ms_avg": round(k_avg, 5),
-        },
-        "cpu_baseline": None if a.no_cpu else w.cpu_baseline(torch, a.cpu_seconds),
+        "config": head["config"],
+        "roofline": head["roofline"],
+        "cpu_baseline": head["cpu_baseline"],
+        "settle_steps": head["settle_steps"],
+        "whole_step_frac": head["whole_step_frac"],
     }
+    if a.workload == "all":
+        out["configs"] = results
     print(json.dumps(out))
 
 

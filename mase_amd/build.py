@@ -1,6 +1,6 @@
 """Builds ``mase_amd/lib/libmase_amd.so`` (the C-ABI library) from ``mase_amd/csrc/*.hip`` with hipcc for gfx950.
 
-Usage:  python -m mase_amd.build [-j N]
+Usage:  python -m mase_amd.build [-j N] [-i]
 The library is built in-tree so that it travels with the source tree; nothing is installed.
 """
 from __future__ import annotations
@@ -42,8 +42,16 @@ def sources() -> list[str]:
     return sorted(os.path.join(SRC_DIR, f) for f in os.listdir(SRC_DIR) if f.endswith(".hip"))
 
 
-def _compile(src: str, verbose: bool) -> str:
+def _headers_mtime() -> float:
+    hs = [os.path.join(SRC_DIR, f) for f in os.listdir(SRC_DIR) if f.endswith(".hpp")]
+    hs.append(os.path.join(os.path.dirname(PKG_DIR), "include", "mase_amd.h"))
+    return max(os.path.getmtime(h) for h in hs)
+
+
+def _compile(src: str, verbose: bool, incremental: bool = False) -> str:
     obj = os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + ".o")
+    if incremental and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), _headers_mtime()):
+        return obj
     cmd = [HIPCC, *COMMON_FLAGS, "-c", src, "-o", obj]
     if verbose:
         print(" ".join(cmd), flush=True)
@@ -57,11 +65,12 @@ def _compile(src: str, verbose: bool) -> str:
     return obj
 
 
-def build_library(jobs: int = 8, verbose: bool = True) -> str:
+def build_library(jobs: int = 8, verbose: bool = True, incremental: bool = False) -> str:
+    """compiles every source (``incremental``: only those newer than their object) and links the library"""
     os.makedirs(OBJ_DIR, exist_ok=True)
     srcs = sources()
     with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(srcs)))) as ex:
-        objs = list(ex.map(lambda s: _compile(s, verbose), srcs))
+        objs = list(ex.map(lambda s: _compile(s, verbose, incremental), srcs))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", LIB_PATH]
     if verbose:
         print(" ".join(cmd), flush=True)
@@ -75,8 +84,9 @@ def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("-j", type=int, default=8)
     ap.add_argument("-q", action="store_true")
+    ap.add_argument("-i", "--incremental", action="store_true", help="recompile only sources newer than their objects")
     a = ap.parse_args()
-    path = build_library(a.j, not a.q)
+    path = build_library(a.j, not a.q, a.incremental)
     print("built", path, os.path.getsize(path), "bytes")
 
 

@@ -7,8 +7,9 @@ kernels.  When the quantized operands are exactly representable in bf16 (at most
 block-FP widths up to 9, minifloat mantissas up to 7 or 8 bits) the contraction runs on the bf16 matrix-core kernel
 with fp32 accumulation (inference only: under ``torch.no_grad()`` or with no tensor requiring grad), which computes
 the same real-number dot products as ``F.linear`` on the dequantized operands; otherwise it is the library GEMM (``F.linear``) in the tensors' own dtype, the operation the reference
-performs at that point.  ``param_cache`` (keyword-only, not in the reference's signatures; the modules pass theirs) keeps the
-quantized parameters between inference calls instead of recomputing identical tensors.  One caveat of the bf16 form for fp32 tensors: block-FP and minifloat pass elements with
+performs at that point.  ``param_cache`` (keyword-only, not in the reference's signatures; the modules pass theirs when their config holds
+``cache_quantized_params=True``) keeps the quantized parameters between inference calls instead of recomputing
+identical tensors; without it weight and bias are quantized on every call, as in the reference.  One caveat of the bf16 form for fp32 tensors: block-FP and minifloat pass elements with
 |x| <= 1e-8 through unquantized, and those are rounded to bf16 (absolute error below 4e-11 per element).
 """
 from __future__ import annotations
@@ -20,6 +21,7 @@ from torch import Tensor
 from torch.nn import functional as F
 
 from ..._gemm import gemm_bf16_pack_b, gemm_bf16_packed_b_supported, gemm_bf16_takes_packed_b, gemm_bf16_tn
+from .mx_linear import _tensor_key as _observable_key
 
 from ...quantizers import (
     block_fp_quantizer,
@@ -31,7 +33,7 @@ from ...quantizers import (
 
 
 def _tensor_key(t: Tensor | None):
-    return None if t is None else (t.data_ptr(), t._version, t.dtype, t.device, tuple(t.shape))
+    return "absent" if t is None else _observable_key(t)
 
 
 class QuantizedParamCache:
@@ -76,7 +78,8 @@ class QuantizedParamCache:
 def _quantized_params(cache, weight, bias, spec, quantize_weight, quantize_bias):
     """(quantized weight, quantized bias, cache or None): from ``cache`` when it may be used, else freshly computed"""
     make = lambda: (quantize_weight(weight), quantize_bias(bias) if bias is not None else None)
-    if cache is not None and weight.is_cuda and weight.dim() == 2 and QuantizedParamCache.usable():
+    if (cache is not None and weight.is_cuda and weight.dim() == 2 and QuantizedParamCache.usable()
+            and _tensor_key(weight) is not None and _tensor_key(bias) is not None):  # None: an inference tensor
         qw, qb = cache.get(weight, bias, spec, make)
         return qw, qb, cache
     qw, qb = make()

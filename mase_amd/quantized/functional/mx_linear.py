@@ -7,8 +7,6 @@ fp32 accumulation, so the real-number dot products are those of the reference; o
 """
 from __future__ import annotations
 
-import weakref
-
 import torch
 from torch import Tensor
 from torch.nn import functional as F
@@ -29,6 +27,8 @@ class WeightCache:
     Changes are detected through the parameter's storage pointer, shape, dtype, device and version counter
     (``load_state_dict``, ``.to()``, ``weight.copy_()``, ``weight.data = ...`` all change one of them).  An in-place
     edit made through ``weight.data`` bypasses the version counter: call ``invalidate()`` after such an edit.
+    A parameter that is an inference tensor (created under ``torch.inference_mode()``) has no version counter: its
+    image is rebuilt on every call rather than trusted.
     """
 
     def __init__(self):
@@ -42,8 +42,8 @@ class WeightCache:
         self._packed = None
 
     def get(self, weight: Tensor):
-        key = (weight.data_ptr(), weight._version, weight.dtype, weight.device, tuple(weight.shape))
-        if key != self._key:
+        key = _tensor_key(weight)
+        if key is None or key != self._key:
             w = weight.detach()
             if w.dtype == torch.bfloat16:
                 wb = w.contiguous()
@@ -66,58 +66,50 @@ class WeightCache:
         return self._packed
 
 
-class _SharedActivation:
-    """The quantized form of the activation tensor most recently fed to an MX Linear, so that sibling projections of
-    the same tensor (q/k/v, gate/up) quantize it once.  A hit requires the very same tensor object, unmodified (same
-    version counter) and the same quantizer; the entry holds the tensor only weakly and is dropped when it dies.
-    The quantized copy itself (the size of the activation in bf16) stays allocated until the next miss.  Callers are
-    assumed to run their projections on one stream, and an in-place edit made through ``.data`` is not seen."""
-
-    def __init__(self):
-        self._ref = None
-        self._key = None
-        self._xq = None
-
-    def _drop(self, _ref=None):
-        self._ref = self._key = self._xq = None
-
-    def get(self, x: Tensor, quantizer_key, make):
-        key = (x._version, tuple(x.shape), x.dtype, quantizer_key)
-        if self._ref is not None and self._ref() is x and self._key == key:
-            return self._xq
-        xq = make()
-        try:
-            self._ref, self._key, self._xq = weakref.ref(x, self._drop), key, xq
-        except TypeError:
-            self._drop()
-        return xq
-
-
-_shared_activation = _SharedActivation()
+def _tensor_key(t: Tensor):
+    """identity of a parameter as far as it can be observed without reading it: storage pointer, version counter,
+    dtype, device, shape; None for an inference tensor (it has no version counter, so changes cannot be seen and
+    nothing derived from it is kept)"""
+    if t.is_inference():
+        return None
+    return (t.data_ptr(), t._version, t.dtype, t.device, tuple(t.shape))
 
 
 def mx_linear(x: Tensor, weight: Tensor, bias: Tensor | None, quantize_to_bf16, quantize_same_dtype,
-              cache: WeightCache, quantizer_key=None) -> Tensor:
+              cache: WeightCache, xq: Tensor | None = None) -> Tensor:
     """``F.linear(q(x), weight, bias)``.  ``quantize_to_bf16(x2d)`` returns q(x) as bf16 (exact);
     ``quantize_same_dtype(x)`` returns q(x) in x's dtype (used when the weight has no exact bf16 image).
-    ``quantizer_key`` identifies the activation quantizer (format and block size): with it, projections that are fed
-    the same tensor object share one quantized copy."""
+    ``xq``: q(x) as a bf16 matrix when the caller already has it (sibling projections of one tensor, see
+    ``project_shared``)."""
     wb = cache.get(weight) if x.is_cuda and weight.dim() == 2 else None
     if wb is None or x.dtype not in (torch.float32, torch.bfloat16, torch.float16):
         return F.linear(quantize_same_dtype(x), weight, bias)
     lead = x.shape[:-1]
-    # not while a HIP graph is being captured: a hit would leave the quantizer out of the graph
-    if quantizer_key is not None and not torch.is_grad_enabled() and not torch.cuda.is_current_stream_capturing():
-        xq = _shared_activation.get(x, quantizer_key, lambda: quantize_to_bf16(x.reshape(-1, x.shape[-1])))
-    else:
+    if xq is None:
         xq = quantize_to_bf16(x.reshape(-1, x.shape[-1]))
     wp = cache.packed() if gemm_bf16_takes_packed_b(xq.shape[0], wb.shape[0], wb.shape[1]) else None
     y = gemm_bf16_tn(xq, wb, bias, x.dtype, b_packed=wp)
     return y.reshape(*lead, weight.shape[0])
 
 
+def project_shared(x: Tensor, modules) -> list:
+    """``[m(x) for m in modules]`` for sibling projections of one tensor (query / key / value, gate / up): modules
+    that quantize ``x`` the same way (``activation_key``) receive one quantized copy instead of making their own.
+    The copy lives for the duration of this call only; nothing is remembered between calls."""
+    outs, key, prepared = [], None, None
+    for m in modules:
+        k = m.activation_key(x) if hasattr(m, "activation_key") else None
+        if k is None:
+            outs.append(m(x))
+            continue
+        if prepared is None or k != key:
+            key, prepared = k, m.prepare_activation(x)
+        outs.append(m(x, prepared=prepared))
+    return outs
+
+
 def _weight_key(weight: Tensor):
-    return (weight.data_ptr(), weight._version, weight.dtype, weight.device, tuple(weight.shape))
+    return _tensor_key(weight)
 
 
 class PackedMXFPWeight:
@@ -195,7 +187,7 @@ class PackedMXFPWeight:
         return bool(torch.equal(got, weight))
 
     def valid_for(self, weight: Tensor) -> bool:
-        return self.codes is not None and self._key == _weight_key(weight)
+        return self.codes is not None and self._key is not None and self._key == _weight_key(weight)
 
 
 class PackedMXIntWeight:
@@ -230,13 +222,15 @@ class PackedMXIntWeight:
         return bool(torch.equal(got, weight))
 
     def valid_for(self, weight: Tensor) -> bool:
-        return self.codes is not None and self._key == _weight_key(weight)
+        return self.codes is not None and self._key is not None and self._key == _weight_key(weight)
 
 
-def mxint_linear_decode(x: Tensor, packed: PackedMXIntWeight, bias: Tensor | None, quantize_to_bf16) -> Tensor:
+def mxint_linear_decode(x: Tensor, packed: PackedMXIntWeight, bias: Tensor | None, quantize_to_bf16,
+                        xq: Tensor | None = None) -> Tensor:
     """``F.linear(q(x), W, b)`` for at most 128 rows of activations with W as MXINT8 codes + scales"""
     lead = x.shape[:-1]
-    xq = quantize_to_bf16(x.reshape(-1, x.shape[-1]))
+    if xq is None:
+        xq = quantize_to_bf16(x.reshape(-1, x.shape[-1]))
     y = gemm_mxint8_skinny(xq, packed.codes, packed.scales, bias, x.dtype)
     return y.reshape(*lead, packed.codes.shape[0])
 
@@ -248,24 +242,39 @@ def mxint_decode_applies(x: Tensor, packed: PackedMXIntWeight, weight: Tensor) -
             and not torch.is_grad_enabled())
 
 
-def mxfp_linear_native(x: Tensor, packed: PackedMXFPWeight, bias: Tensor | None, act_fmt) -> Tensor:
-    """``F.linear(q(x), W, b)`` on the block-scaled matrix instruction: the activations are quantized straight to
-    element codes + scales (one pass over x, 1.03 bytes written per element) and contracted with the packed
-    weight; accumulation is fp32 and the result is written in x's dtype."""
-    lead = x.shape[:-1]
-    x2 = x.reshape(-1, x.shape[-1])
-    M, K = x2.shape
+def mxfp_native_layout(x: Tensor, packed: PackedMXFPWeight, act_fmt) -> str:
+    """which form of the packed activations the block-scaled contraction of ``x`` with this weight takes: "tiled"
+    (tile image, for the tiled kernel) or "rows" (row-major codes: the weight-streaming kernel of few rows and the
+    row-major tiled kernel)"""
+    M, K = (x.numel() // x.shape[-1] if x.numel() else 0), x.shape[-1]
     N = packed.scales.shape[0]
     if (not gemm_mxfp4_skinny_supported(M, N, K, packed.fmt) and gemm_mxfp4_tiled_supported(M, N, K, act_fmt, packed.fmt)
-            and (w_tiled := packed.tiled(K)) is not None):
+            and packed.tiled(K) is not None):
+        return "tiled"
+    return "rows"
+
+
+def mxfp_native_pack(x: Tensor, act_fmt, layout: str):
+    """(codes, scales) of the activations in the given layout: one pass over x, 1.03 bytes written per element"""
+    x2 = x.reshape(-1, x.shape[-1])
+    return mxfp_pack_tiled(x2, *act_fmt) if layout == "tiled" else mxfp_pack(x2, *act_fmt)
+
+
+def mxfp_linear_native(x: Tensor, packed: PackedMXFPWeight, bias: Tensor | None, act_fmt, prepared=None) -> Tensor:
+    """``F.linear(q(x), W, b)`` on the block-scaled matrix instruction: the activations are quantized straight to
+    element codes + scales and contracted with the packed weight; accumulation is fp32 and the result is written in
+    x's dtype.  ``prepared``: ``mxfp_native_pack(x, act_fmt, mxfp_native_layout(...))`` when the caller has it."""
+    lead = x.shape[:-1]
+    M, K = x.numel() // x.shape[-1], x.shape[-1]
+    N = packed.scales.shape[0]
+    layout = mxfp_native_layout(x, packed, act_fmt)
+    xc, xs = prepared if prepared is not None else mxfp_native_pack(x, act_fmt, layout)
+    if layout == "tiled":
         # both code matrices as tile images (the activations' written directly by the quantizer): same bits, 7 % faster
-        xt, xs = mxfp_pack_tiled(x2, *act_fmt)
-        y = gemm_mxfp4_scaled_tiled(xt, xs, act_fmt, w_tiled, packed.scales, bias, x.dtype)
-        return y.reshape(*lead, N)
-    xc, xs = mxfp_pack(x2, *act_fmt)
-    if gemm_mxfp4_skinny_supported(x2.shape[0], packed.scales.shape[0], x2.shape[1], packed.fmt):
+        y = gemm_mxfp4_scaled_tiled(xc, xs, act_fmt, packed.tiled(K), packed.scales, bias, x.dtype)
+    elif gemm_mxfp4_skinny_supported(M, N, K, packed.fmt):
         # decode-sized batch with MXFP4 weights: bound by streaming the weight codes once (0.53 bytes per weight)
         y = gemm_mxfp4_skinny(xc, xs, act_fmt, packed.codes, packed.scales, bias, x.dtype)
     else:
         y = gemm_mxfp_scaled(xc, xs, act_fmt, packed.codes, packed.scales, packed.fmt, bias, x.dtype)
-    return y.reshape(*lead, packed.codes.shape[0])
+    return y.reshape(*lead, N)

@@ -12,7 +12,7 @@ from ...quantizers import _ops, mxfp_quantizer, mxint_quantizer
 from ..functional.linear import (QuantizedParamCache, linearBlockFP, linearInteger, linearMinifloatDenorm,
                                  linearMinifloatIEEE)
 from ..functional.mx_linear import (PackedMXFPWeight, PackedMXIntWeight, WeightCache, mx_linear, mxfp_linear_native,
-                                    mxint_decode_applies, mxint_linear_decode)
+                                    mxfp_native_layout, mxfp_native_pack, mxint_decode_applies, mxint_linear_decode)
 
 
 class _LinearBase(torch.nn.Linear):
@@ -20,11 +20,19 @@ class _LinearBase(torch.nn.Linear):
         super().__init__(in_features, out_features, bias, device, dtype)
         self.bypass = False
         self.pruning_masks = None
-        # the reference quantizes weight and bias on every forward; between inference forwards they do not change
         self._param_cache = QuantizedParamCache()
 
+    def _cache_for(self, config):
+        """The reference quantizes weight and bias on every forward, and so does this module unless
+        ``config["cache_quantized_params"]`` (not a key of the reference, default False) is set: then the quantized
+        parameters are kept between inference forwards while the parameters are the same tensors at the same
+        version.  An edit made through ``weight.data`` is not seen by that test; ``invalidate_weight_cache()`` after
+        such an edit."""
+        return self._param_cache if config.get("cache_quantized_params", False) else None
+
     def invalidate_weight_cache(self):
-        """Forget the cached quantized parameters (needed only after an in-place edit through ``weight.data``)."""
+        """Forget the cached quantized parameters (needed only after an in-place edit through ``weight.data`` with
+        ``cache_quantized_params`` on)."""
         self._param_cache.invalidate()
 
 
@@ -42,7 +50,8 @@ class LinearInteger(_LinearBase):
     def forward(self, x):
         if self.bypass:
             return F.linear(x, self.weight, self.bias)
-        return linearInteger(x, self.weight, self.bias, self.config, self.out_config, param_cache=self._param_cache)
+        return linearInteger(x, self.weight, self.bias, self.config, self.out_config,
+                             param_cache=self._cache_for(self.config))
 
 
 class _ConfigLinear(_LinearBase):
@@ -58,7 +67,7 @@ class _ConfigLinear(_LinearBase):
     def forward(self, x):
         if self.bypass:
             return F.linear(x, self.weight, self.bias)
-        return type(self)._functional(x, self.weight, self.bias, self.config, param_cache=self._param_cache)
+        return type(self)._functional(x, self.weight, self.bias, self.config, param_cache=self._cache_for(self.config))
 
 
 class LinearMinifloatDenorm(_ConfigLinear):
@@ -166,22 +175,37 @@ class LinearMXInt(_LinearMX):
                                 quantile_search=self.clip_search)
             )
 
+    def _act_cfg(self):
+        return self.config.get("data_in_block_size"), self.config.get("data_in_width")
+
+    def activation_key(self, x):
+        """what identifies this module's quantized form of ``x`` (``project_shared``); None when the forward does not
+        go through the bf16 form of the quantized activations"""
+        bs, bits = self._act_cfg()
+        if (self.bypass or bs is None or bits is None or not x.is_cuda or x.numel() == 0
+                or x.dtype not in (torch.float32, torch.bfloat16, torch.float16)):
+            return None
+        if not mxint_decode_applies(x, self._w_codes, self.weight) and self._w_cache.get(self.weight) is None:
+            return None
+        return ("mxint", bs, bits)
+
+    def prepare_activation(self, x):
+        bs, bits = self._act_cfg()
+        return _ops.mxint_qdq(x.reshape(-1, x.shape[-1]), bs, bits, -1, 8, out_dtype=torch.bfloat16)
+
     @torch.no_grad()
-    def forward(self, x):
+    def forward(self, x, prepared=None):
         if self.bypass:
             return F.linear(x, self.weight, self.bias)
-        bs = self.config.get("data_in_block_size")
-        bits = self.config.get("data_in_width")
+        bs, bits = self._act_cfg()
         if bs is None or bits is None:
             return F.linear(x, self.weight, self.bias)
         if mxint_decode_applies(x, self._w_codes, self.weight):
-            return mxint_linear_decode(x, self._w_codes, self.bias,
-                                       lambda t: _ops.mxint_qdq(t, bs, bits, -1, 8, out_dtype=torch.bfloat16))
+            return mxint_linear_decode(x, self._w_codes, self.bias, self.prepare_activation, xq=prepared)
         return mx_linear(
-            x, self.weight, self.bias,
-            lambda t: _ops.mxint_qdq(t, bs, bits, -1, 8, out_dtype=torch.bfloat16),
+            x, self.weight, self.bias, self.prepare_activation,
             lambda t: mxint_quantizer(t, block_size=bs, element_bits=bits, block_dim=-1),
-            self._w_cache, ("mxint", bs, bits),
+            self._w_cache, xq=prepared,
         )
 
 
@@ -247,21 +271,45 @@ class LinearMXFP(_LinearMX):
                                element_frac_bits=b_frac_bits, block_dim=0)
             )
 
+    def _act_cfg(self):
+        return (self.config.get("data_in_block_size"), self.config.get("data_in_exponent_width"),
+                self.config.get("data_in_frac_width"))
+
+    def _native(self, x) -> bool:
+        bs, eb, fb = self._act_cfg()
+        return (bs == 32 and (eb, fb) in ((4, 3), (5, 2)) and x.is_cuda and x.dtype == self.weight.dtype
+                and x.numel() > 0 and self._w_packed.valid_for(self.weight))
+
+    def activation_key(self, x):
+        """see ``LinearMXInt.activation_key``; the block-scaled path shares the packed codes, in the layout the
+        contraction with this module's weight takes"""
+        bs, eb, fb = self._act_cfg()
+        if self.bypass or bs is None or eb is None or not x.is_cuda or x.numel() == 0:
+            return None
+        if self._native(x):
+            return ("mxfp-codes", eb, fb, mxfp_native_layout(x, self._w_packed, (eb, fb)))
+        if x.dtype not in (torch.float32, torch.bfloat16, torch.float16) or self._w_cache.get(self.weight) is None:
+            return None
+        return ("mxfp", bs, eb, fb)
+
+    def prepare_activation(self, x):
+        bs, eb, fb = self._act_cfg()
+        if self._native(x):
+            return mxfp_native_pack(x, (eb, fb), mxfp_native_layout(x, self._w_packed, (eb, fb)))
+        return _ops.mxfp_qdq(x.reshape(-1, x.shape[-1]), bs, eb, fb, -1, 8, out_dtype=torch.bfloat16)
+
     @torch.no_grad()
-    def forward(self, x):
+    def forward(self, x, prepared=None):
         if self.bypass:
             return F.linear(x, self.weight, self.bias)
-        bs = self.config.get("data_in_block_size")
-        eb = self.config.get("data_in_exponent_width")
-        fb = self.config.get("data_in_frac_width")
+        bs, eb, fb = self._act_cfg()
         if bs is None or eb is None:
             return F.linear(x, self.weight, self.bias)
-        if (bs == 32 and (eb, fb) in ((4, 3), (5, 2)) and x.is_cuda and x.dtype == self.weight.dtype
-                and x.numel() > 0 and self._w_packed.valid_for(self.weight)):
-            return mxfp_linear_native(x, self._w_packed, self.bias, (eb, fb))
+        if self._native(x):
+            return mxfp_linear_native(x, self._w_packed, self.bias, (eb, fb), prepared=prepared)
         return mx_linear(
             x, self.weight, self.bias,
             lambda t: _ops.mxfp_qdq(t, bs, eb, fb, -1, 8, out_dtype=torch.bfloat16),
             lambda t: mxfp_quantizer(t, block_size=bs, element_exp_bits=eb, element_frac_bits=fb, block_dim=-1),
-            self._w_cache, ("mxfp", bs, eb, fb),
+            self._w_cache, xq=prepared,
         )

@@ -29,6 +29,7 @@ from torch import Tensor, nn
 from ...quantizers import mxfp_quantizer, mxint_quantizer
 from ...quantizers import _ops
 from ...quantizers._ops import attn_softmax_mx, attn_softmax_mx_supported, minifloat_mx_qdq
+from ..functional.mx_linear import project_shared
 from ..functional.activations import kv_cache_mxfp, kv_cache_mxint, rope_minifloat, rotate_half, silu_minifloat, softmax_minifloat
 
 
@@ -177,10 +178,8 @@ class _LlamaAttentionMX(nn.Module):
 
     def _project(self, hidden_states, hidden_shape):
         """query / key / value states [batch, heads, seq, head_dim] (attention.py:157-159)"""
-        query_states = self.q_proj(hidden_states).view(hidden_shape).transpose(1, 2)
-        key_states = self.k_proj(hidden_states).view(hidden_shape).transpose(1, 2)
-        value_states = self.v_proj(hidden_states).view(hidden_shape).transpose(1, 2)
-        return query_states, key_states, value_states
+        q, k, v = project_shared(hidden_states, (self.q_proj, self.k_proj, self.v_proj))
+        return tuple(t.view(hidden_shape).transpose(1, 2) for t in (q, k, v))
 
     @classmethod
     def from_attention(cls, attention: nn.Module, q_config: dict = None):
@@ -222,7 +221,7 @@ class _LlamaMLPMX(nn.Module):
         self.bypass = self.q_config.get("bypass", False)
 
     def forward(self, x: Tensor) -> Tensor:
-        gate, up = self.gate_proj(x), self.up_proj(x)
+        gate, up = project_shared(x, (self.gate_proj, self.up_proj))
         if _ops.silu_mul_supported(gate, up):  # one pass: cast, SiLU and product
             cast = None if self.bypass else (self.q_config["data_in_exponent_width"], self.q_config["data_in_frac_width"],
                                              self.q_config.get("data_in_is_finite", True),

@@ -13,6 +13,7 @@ from __future__ import annotations
 import torch
 from torch import nn
 
+from ..functional.mx_linear import project_shared
 from .llama import LlamaRMSNormMinifloat, _LlamaAttentionMX, _LlamaMLPMX
 
 
@@ -40,10 +41,10 @@ class _Qwen3AttentionMX(_LlamaAttentionMX):
         self.k_norm = _HeadRMSNorm(self.head_dim, config.rms_norm_eps)
 
     def _project(self, hidden_states, hidden_shape):
-        query_states = self.q_norm(self.q_proj(hidden_states).view(hidden_shape)).transpose(1, 2)
-        key_states = self.k_norm(self.k_proj(hidden_states).view(hidden_shape)).transpose(1, 2)
-        value_states = self.v_proj(hidden_states).view(hidden_shape).transpose(1, 2)
-        return query_states, key_states, value_states
+        q, k, v = project_shared(hidden_states, (self.q_proj, self.k_proj, self.v_proj))
+        query_states = self.q_norm(q.view(hidden_shape)).transpose(1, 2)
+        key_states = self.k_norm(k.view(hidden_shape)).transpose(1, 2)
+        return query_states, key_states, v.view(hidden_shape).transpose(1, 2)
 
 
 class Qwen3AttentionMXFP(_Qwen3AttentionMX):

@@ -28,7 +28,7 @@ class _STE(torch.autograd.Function):
 
 
 def _ste(fn, x: Tensor, *args):
-    if torch.is_grad_enabled() and x.requires_grad:
+    if x.requires_grad and torch.is_grad_enabled():
         return _STE.apply(x, fn, args)
     return fn(x, *args)
 

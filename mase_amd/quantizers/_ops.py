@@ -15,6 +15,32 @@ from .. import _lib
 from .._tables import log2_table
 
 
+# ------------------------------------------------------------------------------------------------
+# Launch state bound once per (entry point, tensor dtype, device): the foreign function, the dtype code and the
+# address of the log2 table.  A 20 us kernel is launch-bound unless the host side of a call stays well below that, so
+# the common case (a contiguous, 16-byte aligned tensor on the device) skips every lookup that cannot change.
+# ------------------------------------------------------------------------------------------------
+_launch_state: dict = {}
+_raw_stream = torch._C._cuda_getCurrentRawStream
+
+
+def _state(name: str, dtype: torch.dtype, device: torch.device, tab_dtype=None):
+    key = (name, dtype, device)
+    st = _launch_state.get(key)
+    if st is None:
+        lib = _lib.load()
+        code = _lib.DTYPE_CODE.get(dtype)
+        if code is None:
+            raise _lib.MaseAmdError(f"mase_amd kernels support float32, bfloat16 and float16 tensors, got {dtype}")
+        tab = log2_table(tab_dtype or dtype, device)  # kept alive by the table cache
+        st = _launch_state[key] = (getattr(lib, name), code, tab.data_ptr(), device.index)
+    return st
+
+
+def _fast_reset():
+    _launch_state.clear()
+
+
 def _contig(x: Tensor) -> Tensor:
     x = x.contiguous()
     if x.data_ptr() % 16 != 0:  # views with odd storage offsets: realign so the 16-byte path applies
@@ -52,6 +78,21 @@ def mxint_qdq(x: Tensor, block_size: int, element_bits: int, block_dim: int, sca
               out_dtype: torch.dtype | None = None):
     """Returns the dequantized tensor (in ``out_dtype``, default the input dtype), or
     (dequantized, codes int8, scales uint8) when ``pack``."""
+    if not pack and x.is_cuda and (block_dim == -1 or block_dim == x.dim() - 1) and x.is_contiguous():
+        ptr = x.data_ptr()
+        if not ptr & 15:
+            n = x.numel()
+            assert n % block_size == 0, f"Input tensor size {n} is not divisible by block size {block_size}."
+            fn, code, tab, index = _state("mase_mxint_qdq", x.dtype, x.device)
+            if out_dtype is None:
+                out, ocode = torch.empty_like(x), code
+            else:
+                out, ocode = torch.empty_like(x, dtype=out_dtype), _lib.DTYPE_CODE[out_dtype]
+            rc = fn(ptr, out.data_ptr(), None, None, n, code, ocode, block_size, element_bits, scale_bits, tab,
+                    _raw_stream(index))
+            if rc:
+                _lib.check(rc, "mase_mxint_qdq")
+            return out
     _lib.require_device(x, "mxint_quantizer")
     lib = _lib.load()
     shape = tuple(x.shape)
@@ -339,7 +380,33 @@ def block_fp_geometry(shape: Sequence[int], block_size, skip_first_dim: bool):
     raise RuntimeError(f"Unsupported x.ndim = {nd}")
 
 
+_bfp_geometry_cache: dict = {}
+
+
 def block_fp_qdq(x: Tensor, width: int, exponent_width: int, exponent_bias, block_size, skip_first_dim: bool) -> Tensor:
+    if x.is_cuda and x.is_contiguous():
+        ptr = x.data_ptr()
+        shape = x.shape
+        gkey = (shape, tuple(block_size) if isinstance(block_size, (list, tuple)) else block_size, skip_first_dim,
+                x.dtype)
+        geom = _bfp_geometry_cache.get(gkey)
+        if geom is None:
+            batch, rows, cols, b0, b1, folded = block_fp_geometry(tuple(shape), block_size, skip_first_dim)
+            vec = 4 if x.dtype == torch.float32 else 8
+            single_pass = (b0 == 1 and b1 > 0 and (b1 & (b1 - 1)) == 0 and b1 <= 64 * vec and cols % b1 == 0
+                           and x.numel() % vec == 0 and x.numel() > 0)
+            if len(_bfp_geometry_cache) > 256:
+                _bfp_geometry_cache.clear()
+            geom = _bfp_geometry_cache[gkey] = (batch, rows, cols, b0, b1, int(folded), single_pass)
+        if geom[6] and not ptr & 15:
+            fn, code, tab, index = _state("mase_block_fp_qdq", x.dtype, x.device)
+            out = torch.empty_like(x)
+            bias = -1 if exponent_bias in (None, "none", "None") else int(exponent_bias)
+            rc = fn(ptr, out.data_ptr(), geom[0], geom[1], geom[2], geom[3], geom[4], code, width, exponent_width, bias,
+                    geom[5], tab, None, 0, _raw_stream(index))
+            if rc:
+                _lib.check(rc, "mase_block_fp_qdq")
+            return out
     _lib.require_device(x, "block_fp_quantizer")
     lib = _lib.load()
     batch, rows, cols, b0, b1, folded = block_fp_geometry(tuple(x.shape), block_size, skip_first_dim)

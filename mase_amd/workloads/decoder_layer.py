@@ -19,6 +19,7 @@ from torch import nn
 from torch.nn import functional as F
 
 from ..quantizers import _ops
+from ..quantized.functional.mx_linear import project_shared
 
 
 @dataclass
@@ -94,9 +95,9 @@ class DecoderLayer(nn.Module):
         cfg = self.cfg
         B, T, _ = x.shape
         h = self.input_layernorm(x)
-        q = self.q_proj(h).view(B, T, cfg.num_heads, cfg.head_dim).transpose(1, 2)
-        k = self.k_proj(h).view(B, T, cfg.num_heads, cfg.head_dim).transpose(1, 2)
-        v = self.v_proj(h).view(B, T, cfg.num_heads, cfg.head_dim).transpose(1, 2)
+        # sibling projections of one tensor: quantized Linears that treat it alike share one quantized copy
+        q, k, v = (t.view(B, T, cfg.num_heads, cfg.head_dim).transpose(1, 2)
+                   for t in project_shared(h, (self.q_proj, self.k_proj, self.v_proj)))
         cos, sin = rope_tables(T, cfg.head_dim, cfg.rope_theta, x.device, x.dtype)
         if q.is_cuda and _ops.rope_supported(q, cos, sin) and _ops.rope_supported(k, cos, sin):
             q, k = _ops.rope(q, cos, sin), _ops.rope(k, cos, sin)  # the same products and sum in one pass
@@ -107,7 +108,7 @@ class DecoderLayer(nn.Module):
         a = a.transpose(1, 2).reshape(B, T, cfg.num_heads * cfg.head_dim)
         x = x + self.o_proj(a)
         h = self.post_attention_layernorm(x)
-        gate, up = self.gate_proj(h), self.up_proj(h)
+        gate, up = project_shared(h, (self.gate_proj, self.up_proj))
         if gate.is_cuda and _ops.silu_mul_supported(gate, up):
             act = _ops.silu_mul_minifloat(gate, up)  # silu(gate) * up in one pass
         else:

@@ -190,11 +190,13 @@ def test_gemm_a_few_hundred_rows_cuts_k_into_work_items(dev, M):
 
 
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (512, 768, 256), (300, 200, 384), (4096, 4096, 1024), (2048, 8448, 512),
-                                   (4100, 4200, 640), (16384, 1024, 4096), (1000, 33, 128)])
+                                   (4100, 4200, 640), (16384, 1024, 4096), (1000, 33, 128),
+                                   (16384, 4096, 11008), (16384, 11008, 4096), (16131, 4096, 11008), (3000, 600, 11008)])
 def test_gemm_with_the_weight_in_fragment_order_is_the_same_product(dev, M, N, K):
     """mase_gemm_bf16_tn_packed against mase_gemm_bf16_tn on the same operands: the same products in the same order,
     so bit-identical (random operands; the bias and every output dtype), one to several output tiles per work-group,
-    ragged M and N, 1 to 32 pairs of K tiles"""
+    ragged M and N, 1 to 86 pairs of K tiles (K = 11008 and N = 11008 at 16384 rows are the decoder layer's
+    down / gate / up projections at batch 8 x seq 2048), and against an fp32 product"""
     from mase_amd._gemm import gemm_bf16_pack_b, gemm_bf16_packed_b_supported, gemm_bf16_tn
 
     g = torch.Generator().manual_seed(M + N + K)

@@ -317,10 +317,12 @@ def test_quantize_module_transform_pass(dev):
                                          "linear_fixed", "linear_minifloat_ieee", "linear_minifloat_denorm"}
 
 
-def test_quantized_parameters_are_kept_between_inference_forwards(dev):
-    """LinearBlockFP / Integer / Minifloat*: the module keeps the quantized weight and bias (and the weight's bf16 and
-    fragment-ordered copies) between forwards under no_grad; results are those of the functional form, which
-    quantizes them on every call, and a changed parameter is picked up"""
+def test_quantized_parameter_cache_modes(dev):
+    """LinearBlockFP / Integer / Minifloat*.  Default (the reference's behaviour): weight and bias are quantized on
+    every forward, so an edit made through ``weight.data`` (which no version counter sees) is picked up.  With
+    ``cache_quantized_params=True`` the module keeps the quantized weight and bias (and the weight's bf16 and
+    fragment-ordered copies) between forwards under no_grad: the same results, a versioned in-place update is picked
+    up, an edit through ``.data`` is served from the old parameters until ``invalidate_weight_cache()``."""
     import mase_amd.quantized.functional.linear as FL
     from mase_amd.quantized import LinearBlockFP, LinearInteger, LinearMinifloatDenorm, LinearMinifloatIEEE
 
@@ -334,21 +336,115 @@ def test_quantized_parameters_are_kept_between_inference_forwards(dev):
              (LinearMinifloatDenorm, FL.linearMinifloatDenorm, mcfg), (LinearMinifloatIEEE, FL.linearMinifloatIEEE, mcfg)]
     for dtype in (torch.float32, torch.bfloat16):
         for cls, fn, cfg in cases:
-            m = cls(256, 512, device=dev, dtype=dtype, config=dict(cfg))
-            m.load_state_dict({"weight": (torch.randn(512, 256, generator=g) * 0.1).to(dtype), "bias": torch.randn(512, generator=g).to(dtype)})
-            for rows in (8, 300, 4096):  # weight-streaming kernel, K-range form, tiled kernel on the fragment-ordered copy
+            for cached in (False, True):
+                mc = dict(cfg, cache_quantized_params=True) if cached else dict(cfg)
+                m = cls(256, 512, device=dev, dtype=dtype, config=mc)
+                m.load_state_dict({"weight": (torch.randn(512, 256, generator=g) * 0.1).to(dtype), "bias": torch.randn(512, generator=g).to(dtype)})
+                for rows in (8, 300, 4096):  # weight-streaming kernel, K-range form, tiled kernel
+                    x = torch.randn(rows, 256, generator=g).to(dtype).to(dev)
+                    with torch.no_grad():
+                        want = fn(x, m.weight, m.bias, dict(cfg))
+                        assert torch.equal(m(x), want) and torch.equal(m(x), want), (cls.__name__, dtype, rows, cached)
+                if cached:
+                    assert m._param_cache.qw is not None and m._param_cache.packed() is not None
+                else:
+                    assert m._param_cache.qw is None
+                with torch.no_grad():
+                    m.weight.mul_(0.5)
+                    want = fn(x, m.weight, m.bias, dict(cfg))
+                    assert torch.equal(m(x), want), (cls.__name__, "after an in-place update", cached)
+                    m.weight.data.add_(0.25)           # an edit the version counter does not see
+                    fresh = fn(x, m.weight, m.bias, dict(cfg))
+                    assert not torch.equal(fresh, want)
+                    if cached:
+                        assert torch.equal(m(x), want), "the opt-in cache serves the parameters it was built from"
+                        m.invalidate_weight_cache()
+                    assert torch.equal(m(x), fresh), (cls.__name__, "after an edit through .data", cached)
+                y = m(x[:4].clone().requires_grad_(True))  # gradients recorded: nothing cached is used, autograd works
+                y.sum().backward()
+                assert m.weight.grad is not None
+
+
+def test_mx_linears_under_inference_mode(dev):
+    """activations (and parameters) made under torch.inference_mode() carry no version counter; the forwards must not
+    depend on one: same results as under no_grad"""
+    from mase_amd.quantized import LinearMXFP, LinearMXInt
+    from mase_amd.workloads import DecoderLayer, DecoderLayerConfig
+    from mase_amd.passes import quantize_module_transform_pass
+
+    g = torch.Generator().manual_seed(16)
+    fcfg = {"weight_block_size": 32, "weight_exponent_width": 2, "weight_frac_width": 1,
+            "data_in_block_size": 32, "data_in_exponent_width": 4, "data_in_frac_width": 3}
+    w = torch.randn(512, 256, generator=g) * 0.05
+    for cls, cfg in ((LinearMXInt, MXINT_CFG), (LinearMXFP, fcfg), (LinearMXFP, dict(fcfg, native_mx=False))):
+        for dtype in (torch.float32, torch.bfloat16):
+            m = cls(256, 512, bias=False, device=dev, dtype=dtype, config=dict(cfg))
+            m.load_state_dict({"weight": w.to(dtype)})
+            for rows in (8, 600):
                 x = torch.randn(rows, 256, generator=g).to(dtype).to(dev)
                 with torch.no_grad():
-                    want = fn(x, m.weight, m.bias, dict(cfg))
-                    assert torch.equal(m(x), want) and torch.equal(m(x), want), (cls.__name__, dtype, rows)
-            assert m._param_cache.qw is not None and m._param_cache.packed() is not None
+                    want = m(x)
+                with torch.inference_mode():
+                    xi = x * 1.0                   # an inference tensor
+                    assert xi.is_inference()
+                    got = m(xi)
+                    got2 = m(xi)
+                assert torch.equal(got, want) and torch.equal(got2, want), (cls.__name__, dtype, rows)
+    # a module whose parameters are inference tensors themselves
+    with torch.inference_mode():
+        mi = LinearMXInt(256, 512, bias=False, device=dev, config=dict(MXINT_CFG))
+        mi.load_state_dict({"weight": w})
+        assert mi.weight.is_inference()
+        x = torch.randn(300, 256, generator=g).to(dev)
+        got = mi(x)
+    m = LinearMXInt(256, 512, bias=False, device=dev, config=dict(MXINT_CFG))
+    m.load_state_dict({"weight": w})
+    assert torch.equal(got, m(x))
+    # the decoder layer with its shared projections
+    cfg = DecoderLayerConfig(hidden_size=256, num_heads=4, head_dim=64, intermediate_size=512)
+    layer = DecoderLayer(cfg, device=dev, dtype=torch.bfloat16, seed=3)
+    layer, _ = quantize_module_transform_pass(layer, {"by": "type", "linear": {"config": dict(MXINT_CFG, name="mxint")}})
+    x = torch.randn(2, 160, 256, generator=g).bfloat16().to(dev)
+    with torch.no_grad():
+        want = layer(x)
+    with torch.inference_mode():
+        got = layer(x * 1.0)
+    assert torch.equal(got, want)
+
+
+def test_sibling_projections_share_one_quantized_activation(dev):
+    """project_shared(x, modules) == [m(x) for m in modules], bit for bit, for every path an MX Linear can take, for
+    modules that quantize differently (each gets its own copy) and for plain nn.Linear; nothing is kept afterwards, so
+    an in-place change of x between two calls is seen"""
+    from mase_amd.quantized import LinearMXFP, LinearMXInt
+    from mase_amd.quantized.functional.mx_linear import project_shared
+
+    g = torch.Generator().manual_seed(17)
+    fcfg = {"weight_block_size": 32, "weight_exponent_width": 2, "weight_frac_width": 1,
+            "data_in_block_size": 32, "data_in_exponent_width": 4, "data_in_frac_width": 3}
+
+    def make(cls, cfg, n_out, dtype):
+        m = cls(256, n_out, bias=False, device=dev, dtype=dtype, config=dict(cfg))
+        m.load_state_dict({"weight": (torch.randn(n_out, 256, generator=g) * 0.05).to(dtype)})
+        return m
+
+    for dtype in (torch.float32, torch.bfloat16):
+        mods = [make(LinearMXInt, MXINT_CFG, 512, dtype), make(LinearMXInt, MXINT_CFG, 128, dtype),
+                make(LinearMXInt, dict(MXINT_CFG, data_in_width=6), 256, dtype),
+                make(LinearMXInt, dict(MXINT_CFG, packed_decode=True), 256, dtype),
+                make(LinearMXFP, fcfg, 512, dtype), make(LinearMXFP, fcfg, 256, dtype),
+                make(LinearMXFP, dict(fcfg, native_mx=False), 256, dtype),
+                make(LinearMXInt, dict(MXINT_CFG, bypass=True), 64, dtype),
+                torch.nn.Linear(256, 64, bias=False, device=dev, dtype=dtype)]
+        for rows in (4, 200, 1500):
+            x = torch.randn(2, rows // 2, 256, generator=g).to(dtype).to(dev)
             with torch.no_grad():
-                m.weight.mul_(0.5)
-                want = fn(x, m.weight, m.bias, dict(cfg))
-                assert torch.equal(m(x), want), (cls.__name__, "after an in-place update")
-                m.weight.data.add_(0.25)           # an edit the version counter does not see
-                m.invalidate_weight_cache()
-                assert torch.equal(m(x), fn(x, m.weight, m.bias, dict(cfg)))
-            y = m(x[:4].clone().requires_grad_(True))  # gradients recorded: nothing cached is used, autograd works
-            y.sum().backward()
-            assert m.weight.grad is not None
+                want = [m(x) for m in mods]
+                got = project_shared(x, mods)
+                for a, b, m in zip(got, want, mods):
+                    assert torch.equal(a, b), (type(m).__name__, dtype, rows)
+                x.data.mul_(1.5)  # unseen by any version counter
+                want2 = [m(x) for m in mods]
+                for a, b, m in zip(project_shared(x, mods), want2, mods):
+                    assert torch.equal(a, b), (type(m).__name__, dtype, rows, "after an edit of x")
+                assert not torch.equal(want2[0], want[0])
