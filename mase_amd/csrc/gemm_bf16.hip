@@ -34,6 +34,7 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
 constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int S = 2;                              // LDS stages
+constexpr int kStagesB = 3;                       // stages of A alone (32 KB each) when B comes in fragment order
 constexpr int kGemmThreads = 256;
 constexpr int kRowBytes = BK * 2;                 // 128: one cache line per operand row per K tile
 constexpr int kTileBytes = BM * kRowBytes;        // 32 KB per operand per stage
@@ -98,8 +99,9 @@ __device__ __forceinline__ void load_16_untracked(bf16x8_t& dst, uint32_t off, c
 // without branches; the other instantiation (K = one tile) advances it with the general, branching step.
 // BPACK (with STREAM, an even number of K tiles): B is the fragment-ordered image of mase_gemm_bf16_pack_b and its
 // fragments go from L2 straight into registers, one K tile ahead of the MFMAs that use them; only A passes through
-// LDS.  That halves the LDS traffic (the copies landing in LDS while the wavefronts read their fragments is what
-// holds the plain kernel back) at the price of every B fragment being fetched by the two wavefronts that share it.
+// LDS, in three stages of 32 KB.  That halves the LDS traffic (the copies landing in LDS while the wavefronts read
+// their fragments is what holds the plain kernel back) at the price of every B fragment being fetched by the two
+// wavefronts that share it.
 template <int OUT_DT, bool STREAM, bool BPACK = false>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
@@ -162,22 +164,28 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // copy-stream position: K tile c_kt of this work-group's c_ord-th output tile goes to stage c_stage.  Past the
   // last tile the stream keeps re-copying K tiles into stages nobody reads any more, which keeps the main
   // loop free of branches around the copies and the vmcnt bookkeeping uniform.
+  // LDS stages: the plain form keeps S stages of A + B; the BPACK form keeps kStagesB stages of A alone (B never
+  // passes through LDS), which lets the A copies of a K tile be issued a whole K tile before the hand-over that
+  // waits for the K tile before it
+  constexpr int kStages = BPACK ? kStagesB : S;
+  constexpr int kStride = BPACK ? kTileBytes : kStageBytes;
+  auto next_of = [](int st) __attribute__((always_inline)) { return (st + 1 == kStages) ? 0 : st + 1; };
   int c_kt = 0, c_ord = 0, c_stage = 0;
   // copy number c (0..15) of the current K tile: row group c/2 of A (even c) or B (odd c)
   auto issue_copy = [&](int c) __attribute__((always_inline)) {
     if constexpr (BPACK) {
       if (c & 1) return;  // B does not pass through LDS
     }
-    const uint32_t st = lds_base + (uint32_t)(c_stage * kStageBytes) + (c & 1) * kTileBytes;
+    const uint32_t st = lds_base + (uint32_t)(c_stage * kStride) + (c & 1) * kTileBytes;
     const int j = c >> 1;
     async_copy_16(((c & 1) ? p.B : p.A) + (size_t)c_kt * kRowBytes, (c & 1) ? gb[j] : ga[j], st + (wave + 4 * j) * 1024);
   };
   auto step_within_tile = [&]() __attribute__((always_inline)) {
-    c_stage ^= 1;
+    c_stage = next_of(c_stage);
     ++c_kt;
   };
   auto advance_copy_stream = [&]() __attribute__((always_inline)) {
-    c_stage ^= 1;
+    c_stage = next_of(c_stage);
     if (c_ord >= n_my) return;  // past the end: stay on the final K tile
     if (++c_kt == nk) {
       if (++c_ord < n_my) {
@@ -212,7 +220,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   const int kgrp = lane >> 5;
   // fragment f (0..3: A row tile f, 4..7: B column tile f-4) of K step s of the K tile in `stage`
   auto load_frag = [&](int stage, int s, int f) __attribute__((always_inline)) -> bf16x8_t {
-    const unsigned char* st = lds + stage * kStageBytes + ((f < 4) ? (wm * 128) * kRowBytes : kTileBytes + (wn * 128) * kRowBytes);
+    const unsigned char* st = lds + stage * kStride + ((f < 4) ? (wm * 128) * kRowBytes : kTileBytes + (wn * 128) * kRowBytes);
     return __builtin_bit_cast(bf16x8_t, *(const uint4*)(st + lds_off((f & 3) * 32 + frag_row, s * 2 + kgrp)));
   };
 
@@ -352,14 +360,26 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
 #pragma unroll
   for (int f = 0; f < (BPACK ? 4 : 8); ++f) fr[0][f] = load_frag(0, 0, f);
   int stage = 0;
-  // BPACK form of the K iteration.  vmcnt holds, oldest first: at the start the 16 B loads of this K tile and the 8 A
-  // copies of the next; steps 0 and 1 add the 16 B loads of the next K tile (second half of the slots, the first half
-  // carries the LDS reads), the hand-over needs the A copies (all but the youngest 16), steps 2 and 3 add the A
-  // copies of the K tile after next.  Stores of an epilogue in between only make the waits conservative.
+  // BPACK form of the K iteration.  The wavefront has two kinds of loads in flight, the B fragment loads into
+  // registers and the A copies into LDS.  Each kind retires in order, but the two kinds do NOT retire in order with
+  // respect to each other: a younger register load can complete before an older LDS copy (with "all but the 16
+  // youngest" as the hand-over test, A tiles were read before they had landed, on shapes whose B image often misses the
+  // cache).  One counter covers both, so "at most n outstanding" proves that an A copy has landed only if at least
+  // n + 1 younger *A copies* would otherwise have to be pending with it.  Hence three stages of A: the 8 copies of the
+  // K tile after next are issued *before* the hand-over that needs the next K tile, and that hand-over waits for
+  // "at most 8 outstanding": the next K tile has landed (its copies are older than those 8), and so have the B loads
+  // unless fewer than 8 of the young copies are still in flight; the young copies themselves fly on across the barrier.
+  //   step 0: MFMAs on fr[0]; LDS reads of step 1; the 16 B loads of the next K tile (their registers were last read
+  //           one K tile ago)
+  //   step 1: MFMAs on fr[1]; LDS reads of steps 2 and 3; the 8 A copies of the K tile after next into the stage
+  //           vacated at the previous hand-over, one every other MFMA slot
+  //   step 2: MFMAs on fr[2]; then the hand-over: at most 8 loads outstanding, own LDS reads complete, barrier
+  //   step 3: MFMAs on fr[3]; LDS reads of step 0 of the next K tile
+  // Stores of an epilogue only make the wait of the next output tile's first hand-over conservative.
   auto k_iteration_b = [&](auto&& advance, auto bufc) __attribute__((always_inline)) {
     constexpr int NB = decltype(bufc)::value;
-    wait_vmcnt<kCopies / 2>();
     const unsigned char* bsrc = b_kbase + (size_t)b_kt * 4096;
+    const int stage_next = next_of(stage);
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
 #pragma unroll
@@ -368,27 +388,24 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
                                                                      acc[t >> 2][t & 3], 0, 0, 0);
         if (s == 0) {
           if (t < 4) fr[1][t] = load_frag(stage, 1, t);
-          if (t >= 8) load_16_untracked(fb[NB ^ 1][(t - 8) >> 2][t & 3], boff[t & 3], bsrc + (size_t)((t - 8) >> 2) * 1024);
+          load_16_untracked(fb[NB ^ 1][t >> 2][t & 3], boff[t & 3], bsrc + (size_t)(t >> 2) * 1024);
         } else if (s == 1) {
           if (t < 4) fr[2][t] = load_frag(stage, 2, t);
           else if (t < 8) fr[3][t - 4] = load_frag(stage, 3, t - 4);
-          else load_16_untracked(fb[NB ^ 1][t >> 2][t & 3], boff[t & 3], bsrc + (size_t)(t >> 2) * 1024);
-        } else if (s == 2) {
-          if (t < 4) fr[0][t] = load_frag(stage ^ 1, 0, t);
-          if ((t & 3) == 3) issue_copy((t >> 2) * 2);
-        } else {
-          if ((t & 3) == 3) issue_copy(8 + (t >> 2) * 2);
+          if (t & 1) issue_copy(t - 1);
+        } else if (s == 3) {
+          if (t < 4) fr[0][t] = load_frag(stage_next, 0, t);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
-      if (s == 1) {
-        wait_vmcnt<16>();
+      if (s == 2) {
+        wait_vmcnt<kWaveCopies>();
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
       }
     }
     advance();
-    stage ^= 1;
+    stage = stage_next;
     ++b_kt;
   };
   auto k_iteration = [&](auto&& advance) __attribute__((always_inline)) {
