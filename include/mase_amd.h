@@ -98,6 +98,19 @@ int mase_block_fp_qdq(const void* in, void* out, size_t batch, size_t rows, size
                       int zero_sign_mode, const uint32_t* log2_tab, void* workspace, size_t workspace_bytes,
                       void* stream);
 
+/* mase_block_fp_qdq for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same arguments and results, without the workspace.  It has no counterpart
+ * in the reference.  The per-tile maxima of the two-pass schedule live in a 4 MiB array inside the library's own
+ * device image (one copy per GPU, held until the process ends), so at most MASE_BLOCK_FP_STATIC_MAX_TILES
+ * tiles per call: MASE_ERR_WORKSPACE beyond that.  The call allocates and frees nothing; the first call on a device
+ * looks up the array's address (do it once outside any graph capture).  All calls on one GPU share the array:
+ * calls that may overlap on one GPU (different streams, different host threads) race on it and must be serialized by
+ * the caller.  The part of the array a call uses is cleared by a fill kernel on `stream` before it is used. */
+#define MASE_BLOCK_FP_STATIC_MAX_TILES (1u << 20)
+int mase_block_fp_qdq_static(const void* in, void* out, size_t batch, size_t rows, size_t cols, int tile_rows,
+                             int tile_cols, int dtype, int width, int exponent_width, int exponent_bias,
+                             int zero_sign_mode, const uint32_t* log2_tab, void* stream);
+
 /* Fixed point: clamp(round_or_floor(x * 2^frac_width)) / 2^frac_width. */
 int mase_integer_qdq(const void* in, void* out, size_t numel, int dtype, int width, int frac_width,
                      int is_signed, int use_floor, void* stream);

@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libm
 DT_F32, DT_BF16, DT_F16 = 0, 1, 2
 DTYPE_CODE = {torch.float32: DT_F32, torch.bfloat16: DT_BF16, torch.float16: DT_F16}
 LOG2_TABLE_WORDS = 576
+BLOCK_FP_STATIC_MAX_TILES = 1 << 20
 
 
 class MaseAmdError(RuntimeError):
@@ -29,6 +30,7 @@ SIGNATURES = {
     "mase_mxint_qdq": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mase_block_fp_workspace_bytes": (c_size_t, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int]),
     "mase_block_fp_qdq": (c_int, [c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "mase_block_fp_qdq_static": (c_int, [c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mase_integer_qdq": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "mase_minifloat_qdq": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mase_minifloat_mx_qdq": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),

@@ -23,6 +23,33 @@
 //                 workspace, pass 2 quantizes; both are coalesced along the last dimension.
 #include "common.hpp"
 
+#include <mutex>
+
+// ---- scratch of the entry point that allocates nothing (mase_block_fp_qdq_static): the per-tile maxima of the
+// two-pass schedule, held in the library's own device image.  Each GPU the library runs on keeps its own 4 MiB copy
+// until the process ends.  In host code the array's name is only a handle of the symbol, never a device address: the
+// address on a device comes from hipGetSymbolAddress, looked up once per device with that device current.
+static __device__ __align__(256) uint32_t scratch[MASE_BLOCK_FP_STATIC_MAX_TILES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+uint32_t* g_scratch_ptr[kMaxDevices];
+
+uint32_t* static_scratch_of_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) return nullptr;
+    g_scratch_ptr[dev] = (uint32_t*)ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+}  // namespace
+
+
 #ifndef MASE_RUN_THREADS
 #define MASE_RUN_THREADS 64
 #endif
@@ -304,4 +331,21 @@ extern "C" int mase_block_fp_qdq(const void* in, void* out, size_t batch, size_t
     default:
       return launch_bfp<MASE_DT_F16>(in, out, batch, rows, cols, tile_rows, tile_cols, p, workspace, workspace_bytes, st);
   }
+}
+
+extern "C" int mase_block_fp_qdq_static(const void* in, void* out, size_t batch, size_t rows, size_t cols, int tile_rows,
+                                        int tile_cols, int dtype, int width, int exponent_width, int exponent_bias,
+                                        int zero_sign_mode, const uint32_t* log2_tab, void* stream) {
+  using namespace mase;
+  if (batch == 0 || rows == 0 || cols == 0) return MASE_OK;
+  if (tile_rows <= 0 || tile_cols <= 0) return MASE_ERR_SHAPE;
+  const size_t tiles = batch * ((rows + tile_rows - 1) / tile_rows) * ((cols + tile_cols - 1) / tile_cols);
+  if (tiles > (size_t)MASE_BLOCK_FP_STATIC_MAX_TILES) return MASE_ERR_WORKSPACE;  // more tile maxima than the static scratch holds
+  uint32_t* ws = static_scratch_of_current_device();
+  if (ws == nullptr) return MASE_ERR_LAUNCH;
+  // the two-pass schedule clears the maxima it uses with a fill kernel before pass 1, so what an earlier call
+  // left in the scratch does not matter
+  return mase_block_fp_qdq(in, out, batch, rows, cols, tile_rows, tile_cols, dtype, width, exponent_width,
+                           exponent_bias, zero_sign_mode, log2_tab, ws,
+                           (size_t)MASE_BLOCK_FP_STATIC_MAX_TILES * sizeof(uint32_t), stream);
 }
