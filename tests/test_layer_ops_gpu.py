@@ -89,8 +89,11 @@ def test_rope_one_pass_is_bit_identical_to_the_tensor_operations(dev, dtype):
     assert not _ops.rope_supported(q[..., :40], cos[..., :40], sin[..., :40])   # head_dim not a multiple of 16
 
 
-def test_sibling_projections_share_one_quantized_activation(dev, monkeypatch):
+def test_project_shared_quantizes_once_per_quantizer(dev, monkeypatch):
+    """project_shared: one activation quantization for sibling projections with the same quantizer, one more for a
+    module with another format; separate module calls quantize every time (nothing is remembered between calls)"""
     from mase_amd.quantized import LinearMXInt
+    from mase_amd.quantized.functional.mx_linear import project_shared
     from mase_amd.quantizers import _ops
 
     cfg = {"weight_block_size": 32, "weight_width": 8, "data_in_block_size": 32, "data_in_width": 8}
@@ -100,22 +103,18 @@ def test_sibling_projections_share_one_quantized_activation(dev, monkeypatch):
         m = LinearMXInt(256, 128, bias=False, device=dev, dtype=torch.bfloat16, config=dict(cfg))
         m.load_state_dict({"weight": torch.randn(128, 256) * 0.05})
         mods.append(m)
+    other = LinearMXInt(256, 128, bias=False, device=dev, dtype=torch.bfloat16, config={**cfg, "data_in_width": 6})
+    other.load_state_dict({"weight": torch.randn(128, 256) * 0.05})
     calls = []
     real = _ops.mxint_qdq
     monkeypatch.setattr(_ops, "mxint_qdq", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
     x = torch.randn(300, 256, device=dev, dtype=torch.bfloat16)
-    ys = [m(x) for m in mods]
+    ys = project_shared(x, mods)
     assert len(calls) == 1                               # q/k/v style: one quantization for three projections
-    ref = [m(x.clone()) for m in mods]                   # other tensor objects: quantized again each time
+    ref = [m(x) for m in mods]                           # separate calls: quantized again each time
     assert len(calls) == 4
     for a, b in zip(ys, ref):
         assert torch.equal(a, b)
-    x.mul_(0.5)                                          # modified in place: the cached copy is stale
-    y2 = mods[0](x)
-    assert len(calls) == 5 and torch.equal(y2, mods[0](x.clone()))
-    other = LinearMXInt(256, 128, bias=False, device=dev, dtype=torch.bfloat16,
-                        config={**cfg, "data_in_width": 6})
-    other.load_state_dict({"weight": torch.randn(128, 256) * 0.05})
     n = len(calls)
-    other(x)                                             # another activation format: not shared
-    assert len(calls) == n + 1
+    project_shared(x, mods + [other])                    # another activation format gets its own copy
+    assert len(calls) == n + 2
