@@ -17,13 +17,20 @@ Pinning status (what fixes each function besides reading the source):
 
 * ``integer_quantizer``            closed form (exact rational arithmetic), exhaustive over bf16   -> pinned
 * ``mxint_quantizer``              closed form with torch's own ``log2().ceil()``, invariants       -> pinned
-* ``block_fp_quantizer``           closed form; blocking checked against a brute-force index map   -> pinned
-                                   except the per-op rounding order in bf16/fp16 for width > 9,
-                                   which only the reference could confirm             -> parity unpinned (that part)
-* ``minifloat_denorm/ieee``        closed form in fp32; bf16/fp16 per-op rounding      -> parity unpinned (low-precision part)
-* ``_minifloat_mx`` encode/decode  nearest-value brute force away from the documented quirks; the quirks
-  and ``mxfp_quantizer``           (``>> 8`` double rounding, lost carry in odd binades, truncating subnormals)
-                                   are source-defined                                   -> parity unpinned (quirk regions)
+* ``block_fp_quantizer``           blocking checked against a brute-force index map; element values: exact rational
+                                   closed form in fp32; in bf16 / fp16 an op-by-op model with every rounding to the
+                                   dtype written out (``oracle/scalar.py``: float64 arithmetic, where each single op is
+                                   exact, plus an explicit round-to-fp32-then-dtype), and the closed form with the one
+                                   rounding that matters; every finite 16-bit value as block maximum and as element,
+                                   exponents from the library's own ``log2`` in the dtype               -> pinned
+* ``minifloat_denorm/ieee``        exact closed form in fp32; in bf16 / fp16 the same explicit-rounding model over
+                                   every finite 16-bit input for (8,4), (8,5), (6,3)                     -> pinned
+* ``_minifloat_mx`` encode/decode  nearest-value brute force away from the documented quirks; invariants the format
+  and ``mxfp_quantizer``           fixes (codes fit 1+E+F bits, normal codes survive decode -> encode).  The quirks
+                                   themselves (``>> 8`` double rounding, lost carry in odd binades, truncating
+                                   subnormals, flushed values below 2^-bias) are defined by the source text alone: two
+                                   restatements of that text agree, nothing else can confirm the reading
+                                                                                        -> parity unpinned (quirk regions)
 
 * clip search (``quantile_search``)   quantile against exact rational interpolation; candidates against the scalar
                                    restatement; the choice against exact errors (first minimum, strict replace);
@@ -31,8 +38,9 @@ Pinning status (what fixes each function besides reading the source):
                                    library's summation order inside ``norm`` / ``sum`` and the uint8 power wrap,
                                    which are facts of the host library              -> parity unpinned (that part)
 
-``tests/golden/known_answers.json`` holds small vectors computed with the exact scalar restatement; the vectorised
-restatement (and the kernels) must reproduce them bit for bit.
+``tests/golden/known_answers.json`` holds small vectors computed with the exact scalar restatement (fp32 for all
+quantizers, bf16 for block floating point in the headline configuration's format); the vectorised restatement (and
+the kernels) must reproduce them bit for bit.
 
 The reference ships no golden vectors or value-asserting tests for this path, and running the reference
 to produce vectors was refused by the environment, so "parity unpinned" above means: restated from the

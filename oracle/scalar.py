@@ -149,3 +149,117 @@ def minifloat_representable(E: int, F: int, is_finite: bool):
         if not isinstance(v, str):
             vals.add(v)
     return sorted(vals)
+
+
+# ------------------------------------------------------------------------------------------------
+# Explicit-rounding model of the element-wise and block quantizers on 16-bit tensors.
+#
+# A torch op on a bf16 / fp16 tensor computes in fp32 and stores the result in the tensor dtype.  The functions below
+# evaluate the reference's op sequences (block_fp.py:55-80, minifloat.py:46-66, :158-180) in float64, where every
+# single op on fp32-representable operands is exact (sums: the smaller addend of a pair more than 29 binades apart
+# cannot move the fp32 rounding of the larger), and write every rounding out: ``store(v, fmt)`` = round to fp32, then
+# to the dtype, both to nearest even with gradual underflow and overflow to infinity, done with integer scaling, not
+# with a library conversion.  The two library-defined pieces are passed in by the caller: log2 as the library rounds
+# it in the dtype, and isclose(x, 0).
+# ------------------------------------------------------------------------------------------------
+import numpy as np
+
+FMT = {  # precision in bits (with the implicit one), exponent of the smallest subnormal step, largest finite value
+    "f32": (24, -149, float(np.finfo(np.float32).max)),
+    "bf16": (8, -133, 3.3895313892515355e38),
+    "f16": (11, -24, 65504.0),
+}
+EPS_F32 = float(np.float32(1e-9))  # the scalar 1e-9 as the fp32 computation sees it
+
+
+def round_to(v, fmt: str):
+    """round float64 values to the format: nearest even, subnormals, overflow to infinity; NaN and infinity pass"""
+    p, qmin, vmax = FMT[fmt]
+    v = np.asarray(v, dtype=np.float64)
+    out = v.copy()
+    fin = np.isfinite(v) & (v != 0)
+    m, e = np.frexp(v[fin])                      # |m| in [0.5, 1)
+    qe = np.maximum(e - p, qmin)                 # exponent of the rounding step at this magnitude
+    r = np.ldexp(np.rint(np.ldexp(v[fin], -qe)), qe)   # rint: nearest even on an exactly scaled value
+    r = np.where(np.abs(r) > vmax, np.copysign(np.inf, r), r)
+    out[fin] = r
+    return out
+
+
+def store(v, fmt: str):
+    """the result of one torch op on a tensor of the format: computed in fp32, stored in the format"""
+    return round_to(v, "f32") if fmt == "f32" else round_to(round_to(v, "f32"), fmt)
+
+
+def _pow2(e, fmt):
+    with np.errstate(over="ignore"):
+        return store(np.ldexp(1.0, e.astype(np.int64)), fmt)  # 2 ** e on a tensor of integers held in the format
+
+
+def _select(close, y, x, fmt):
+    """(~close) * y + close * x as tensor ops: products with 0.0 / 1.0, then a sum (keeps or loses the sign of zero
+    exactly as the float ops do)"""
+    with np.errstate(invalid="ignore"):
+        return store(store((~close).astype(np.float64) * y, fmt) + store(close.astype(np.float64) * x, fmt), fmt)
+
+
+def block_fp_model(x, bmax_log2_ceil, close, width: int, exponent_width: int, fmt: str, exponent_bias=None):
+    """op-by-op model of block_fp.py:55-80 for elements ``x`` whose block maximum has ceil(log2(max)) =
+    ``bmax_log2_ceil`` (as the library rounds it, float64 array of integers or +-inf), ``close`` = isclose(x, 0)"""
+    mb = width - 1
+    bias = (1 << (exponent_width - 1)) - 1 if exponent_bias is None else exponent_bias
+    e_lo, e_hi = float(-bias), float((1 << exponent_width) - 1 - bias)
+    m_hi = float(store(np.float64((1 << mb) - 1), fmt))   # a clamp bound is first converted to the dtype
+    x = np.asarray(x, dtype=np.float64)
+    with np.errstate(invalid="ignore", over="ignore", divide="ignore"):
+        sgn = np.sign(store(x + EPS_F32, fmt))
+        val = store(np.abs(x) + EPS_F32, fmt)
+        e = np.clip(bmax_log2_ceil, e_lo, e_hi)
+        p2 = _pow2(e, fmt)
+        man = store(val / p2, fmt)
+        q = np.clip(np.rint(store(man * float(1 << mb), fmt)), 0.0, m_hi)
+        man = store(q / float(1 << mb), fmt)
+        y = store(store(sgn * p2, fmt) * man, fmt)
+    return _select(close, y, x, fmt)
+
+
+def block_fp_closed_form(x, e, width: int, fmt: str):
+    """the closed form that holds when 2^e, v / 2^e and the final product are exact in the format (widths up to 9 in
+    bf16, 12 in fp16, exponents inside the format's normal range): one rounding, that of |x| + 1e-9"""
+    mb = width - 1
+    x = np.asarray(x, dtype=np.float64)
+    v = store(np.abs(x) + EPS_F32, fmt)
+    q = np.clip(np.rint(np.ldexp(v, (mb - e).astype(np.int64))), 0.0, float((1 << mb) - 1))
+    return np.copysign(np.ldexp(q, (e - mb).astype(np.int64)), x)
+
+
+def minifloat_model(x, log2_of, close, width: int, exponent_width: int, fmt: str, ieee: bool, exponent_bias=None):
+    """op-by-op model of minifloat.py:46-66 (denorm) / :158-180 (ieee).  ``log2_of(v)``: the library's log2 of a
+    float64 array of values of the format, evaluated in the format; ``close`` = isclose(|x|, 0)"""
+    mb = width - exponent_width - 1
+    bias = (1 << (exponent_width - 1)) - 1 if exponent_bias is None else exponent_bias
+    e_lo, e_hi = float(-bias), float((1 << exponent_width) - 1 - bias)
+    shift = float(1 << mb)
+    m_hi = float(store(np.float64((1 << mb) - 1), fmt))
+    x = np.asarray(x, dtype=np.float64)
+    with np.errstate(invalid="ignore", over="ignore", divide="ignore"):
+        sgn = np.sign(store(x + EPS_F32, fmt))
+        val = np.abs(x)
+        lg = log2_of(store(val + EPS_F32, fmt))
+        e = np.clip(np.floor(lg) if ieee else np.ceil(lg), e_lo, e_hi)
+        p2 = _pow2(e, fmt)
+        man = store(val / p2, fmt)
+        if not ieee:
+            q = np.clip(np.rint(store(man * shift, fmt)), 0.0, m_hi)
+            man = store(q / shift, fmt)
+        else:
+            normal = ~(e == -float(bias))     # isclose(e, -bias) on integers held exactly in the format
+            nf = normal.astype(np.float64)
+            qn = np.clip(np.rint(store(store(man * shift, fmt) - shift, fmt)), 0.0, m_hi)
+            qs = np.clip(np.rint(store(store(man * shift, fmt) / 2.0, fmt)), 0.0, m_hi)
+            q = store(store(nf * qn, fmt) + store((1.0 - nf) * qs, fmt), fmt)
+            mn = store(1.0 + store(q / shift, fmt), fmt)
+            ms = store(store(q / shift, fmt) * 2.0, fmt)
+            man = store(store(nf * mn, fmt) + store((1.0 - nf) * ms, fmt), fmt)
+        y = store(store(sgn * p2, fmt) * man, fmt)
+    return _select(close, y, x, fmt)

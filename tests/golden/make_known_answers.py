@@ -103,6 +103,40 @@ def main():
                 ys.append(frac_bits(v * Fraction(2) ** sh, negative_zero=(v == 0 and sgn == 1)))
             out["mxfp"].append({"block_size": 32, "exp_bits": E, "frac_bits": F, "scale_byte": sh + 127,
                                 "x": [bits(x) for x in xs], "y": ys})
+    # block floating point on bf16 tensors (the headline configuration: width 8, exponent width 8, blocks of 16, and a
+    # narrower one).  Values are bf16 bit patterns.  The only rounding to the dtype that changes a value is that of
+    # |x| + 1e-9 (S.store: fp32 sum, then bf16); 2^e, the scalings by powers of two and the final product are exact.
+    # Block maxima sit in the upper 70 % of their binade, where log2 rounded to bf16 cannot reach the next integer.
+    import numpy as np
+
+    def bf16_bits(v):
+        b = bits(v)
+        assert b & 0xFFFF == 0, v
+        return b >> 16
+
+    out["block_fp_bf16"] = []
+    for width in (8, 6):
+        for scale in (1.0, 50.0, 0.003):
+            while True:
+                xs = [float(S.round_to(np.float64(rng.gauss(0.0, 1.0) * scale), "bf16")) for _ in range(16)]
+                if scale == 50.0:
+                    xs[3], xs[7], xs[11] = 0.0, -0.0, float(S.round_to(np.float64(3e-9), "bf16"))
+                m = max(abs(x) for x in xs)
+                if 1.3 < m / 2.0 ** exact_floor_log2(m) < 1.95:
+                    break
+            e = exact_floor_log2(m) + 1
+            ys = []
+            for x in xs:
+                if abs(x) <= float(S.round_to(np.float64(1e-8), "bf16")):   # isclose(x, 0): passed through, -0 -> +0
+                    ys.append(bf16_bits(abs(x)) if x == 0 else bf16_bits(x))
+                    continue
+                v = Fraction(float(S.store(np.float64(abs(x)) + S.EPS_F32, "bf16")))
+                q = min(max(S.rne(v / Fraction(2) ** e * (1 << (width - 1))), 0), (1 << (width - 1)) - 1)
+                y = Fraction(q, 1 << (width - 1)) * Fraction(2) ** e
+                ys.append(bf16_bits(float(y)) | (0x8000 if x < 0 else 0))
+            out["block_fp_bf16"].append({"width": width, "exponent_width": 8, "block": 16,
+                                         "x": [bf16_bits(x) | 0 if not (x == 0 and str(x).startswith("-")) else 0x8000 for x in xs],
+                                         "y": ys})
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "known_answers.json")
     with open(path, "w") as f:
         json.dump(out, f, separators=(",", ":"))

@@ -312,6 +312,167 @@ def test_minifloat_denorm_ieee_closed_form_fp32(w, ew):
     assert n > 2000
 
 
+# ------------------------------------------------------------------ 16-bit tensors: explicit-rounding models
+_T16 = {"bf16": torch.bfloat16, "f16": torch.float16}
+
+
+def all_16bit_values(fmt, finite_only=True):
+    bits16 = torch.arange(0, 1 << 16, dtype=torch.int32).to(torch.int16)
+    t = bits16.view(_T16[fmt])
+    if finite_only:
+        t = t[torch.isfinite(t.float())]
+    return t
+
+
+def lib_log2(fmt):
+    return lambda v: torch.from_numpy(np.asarray(v)).to(_T16[fmt]).log2().double().numpy()
+
+
+def lib_close(t):
+    return torch.isclose(t, torch.tensor([0.0], dtype=t.dtype)).numpy()
+
+
+def same_values(got: torch.Tensor, want: np.ndarray):
+    """bit-level equality of a 16-bit tensor with float64 model values (signed zeros told apart, NaN == NaN)"""
+    g = got.double().numpy()
+    ok = ((g == want) & (np.signbit(g) == np.signbit(want))) | (np.isnan(g) & np.isnan(want))
+    return ok
+
+
+def test_explicit_rounding_helper_is_round_to_nearest_even():
+    """the model's own rounding routine against exact rational arithmetic (ties, subnormals, overflow)"""
+    rng = np.random.default_rng(5)
+    for fmt, (p, qmin, vmax) in S.FMT.items():
+        vals = list((rng.standard_normal(300) * np.exp(rng.uniform(-60, 40, 300))).astype(np.float64))
+        vals += [np.ldexp(1.0 + (2 * k + 1) * 2.0 ** -p, e) for k in range(4) for e in (-3, 0, 7)]       # exact ties
+        vals += [np.ldexp(float(k) + 0.5, qmin) for k in range(6)] + [np.ldexp(0.5, qmin), np.ldexp(0.25, qmin)]
+        vals += [vmax, np.nextafter(vmax, np.inf), vmax + np.ldexp(1.0, int(np.log2(vmax)) - p), vmax * 1.1]
+        got = S.round_to(np.array(vals), fmt)
+        for v, g in zip(vals, got):
+            fr = Fraction(float(v))
+            k = 0 if fr == 0 else (abs(fr).numerator.bit_length() - abs(fr).denominator.bit_length())
+            while Fraction(2) ** k > abs(fr):
+                k -= 1
+            while Fraction(2) ** (k + 1) <= abs(fr):
+                k += 1
+            qe = max(k + 1 - p, qmin)
+            want = Fraction(S.rne(fr / Fraction(2) ** qe)) * Fraction(2) ** qe
+            if abs(want) > Fraction(vmax):
+                assert np.isinf(g) and (g > 0) == (fr > 0), (fmt, v, g)
+            else:
+                assert Fraction(float(g)) == want, (fmt, v, g, float(want))
+
+
+@pytest.mark.parametrize("fmt", ["bf16", "f16"])
+@pytest.mark.parametrize("width", [8, 6, 9])
+def test_block_fp_16bit_every_value_as_block_maximum_and_as_element(fmt, width):
+    """block_fp_quantizer on bf16 / fp16 (width 8 on bf16 is the headline configuration): the oracle against (1) the
+    op-by-op model with every rounding to the dtype written out and (2), where it applies, the closed form with the
+    single rounding of |x| + 1e-9; exponents from the library's own log2 in the dtype.  Every finite 16-bit value
+    serves once as the maximum of a block and once as an element of blocks with a larger maximum."""
+    T = _T16[fmt]
+    vals = all_16bit_values(fmt)
+    n = vals.numel()
+    # (a) every value as block maximum: element 0 is the value, the others are fixed fractions of it
+    fr = torch.tensor([1.0, 0.5, -0.75, 0.3, -0.011, 0.99, 1e-3, -1.0, 0.0, 0.66, -0.2, 0.127, 0.9, -0.45, 2.0 ** -9, 0.07])
+    blocks_a = (vals.float()[:, None] * fr[None, :]).to(T)
+    # (b) every value as an element: 15 values per block, the block maximum a fixed larger value
+    cases = [blocks_a]
+    for mx in ((1.0, 200.0, 3e-4, 40000.0) if fmt == "f16" else (1.0, 200.0, 3e-4, 7e20, 1e-30)):
+        sel = vals[vals.float().abs() <= mx]
+        sel = sel[: sel.numel() // 15 * 15].reshape(-1, 15)
+        cases.append(torch.cat((torch.full((sel.shape[0], 1), mx).to(T), sel), dim=1))
+    checked = closed = 0
+    for blocks in cases:
+        got = O.block_fp_quantizer(blocks.clone(), width, 8, None, [16], True)
+        bmax = blocks.float().abs().amax(1, keepdim=True).to(T)
+        with np.errstate(divide="ignore"):
+            lg = np.ceil(lib_log2(fmt)(bmax.double().numpy()))               # -inf for an all-zero block
+        lg = np.broadcast_to(lg, blocks.shape).copy()
+        close = lib_close(blocks)
+        x = blocks.double().numpy()
+        lg[np.isneginf(lg)] = 0.0   # all-zero blocks: every element takes the isclose branch, the exponent is moot
+        want = S.block_fp_model(x, lg, close, width, 8, fmt)
+        ok = same_values(got, want)
+        assert ok.all(), (fmt, width, int((~ok).sum()), x[~ok][:4], got.double().numpy()[~ok][:4], want[~ok][:4])
+        checked += ok.size
+        # closed form: exponent inside the range where 2^e and the scalings are exact in the dtype
+        e = np.clip(lg, -127, 128)
+        lo, hi = ((-14 + width, 15) if fmt == "f16" else (-120, 120))
+        dom = (~close) & (e >= lo) & (e <= hi) & (np.abs(x) < np.ldexp(1.0, e.astype(np.int64) + 1))
+        cf = S.block_fp_closed_form(x[dom], e[dom], width, fmt)
+        g = got.double().numpy()[dom]
+        assert ((g == cf) | ((g == 0) & (cf == 0))).all(), (fmt, width)
+        closed += int(dom.sum())
+    assert checked > n * 17 and closed > n * 8, (checked, closed, n)
+
+
+@pytest.mark.parametrize("fmt", ["bf16", "f16"])
+@pytest.mark.parametrize("w,ew", [(8, 4), (8, 5), (6, 3)])
+def test_minifloat_denorm_ieee_16bit_exhaustive(fmt, w, ew):
+    """minifloat_denorm / ieee on bf16 and fp16 tensors, every finite 16-bit input: the oracle against the op-by-op
+    model in which each op's result is rounded to fp32 and then to the dtype explicitly (log2 and isclose are the
+    library's own, evaluated in the dtype)"""
+    vals = all_16bit_values(fmt)
+    x = vals.double().numpy()
+    close = lib_close(vals.abs())
+    for ieee, fn in ((False, O.minifloat_denorm_quantizer), (True, O.minifloat_ieee_quantizer)):
+        got = fn(vals.clone(), w, ew)
+        want = S.minifloat_model(x, lib_log2(fmt), close, w, ew, fmt, ieee)
+        ok = same_values(got, want)
+        assert ok.all(), (fmt, w, ew, ieee, int((~ok).sum()), x[~ok][:5], got.double().numpy()[~ok][:5], want[~ok][:5])
+        # the model reduces to the textbook value away from the library's log2 thresholds: spot-check in exact arithmetic
+        mb, bias = w - ew - 1, 2 ** (ew - 1) - 1
+        idx = np.flatnonzero(~close & (np.abs(x) > 2.0 ** (-bias + 1)) & (np.abs(x) < 2.0 ** (2 ** ew - 2 - bias)))[::97]
+        for i in idx:
+            a = abs(float(x[i]))
+            if not far_from_pow2(a, 0.02):
+                continue
+            kx, p2 = exact_log2_parts(a)
+            if ieee:
+                q = min(max(S.rne(Fraction(a) / Fraction(2) ** kx * 2 ** mb - 2 ** mb), 0), 2 ** mb - 1)
+                expect = (1 + Fraction(q, 2 ** mb)) * Fraction(2) ** kx
+            else:
+                e = kx if p2 else kx + 1
+                q = min(max(S.rne(Fraction(a) / Fraction(2) ** e * 2 ** mb), 0), 2 ** mb - 1)
+                expect = Fraction(q, 2 ** mb) * Fraction(2) ** e
+            assert Fraction(abs(float(want[i]))) == expect, (fmt, w, ew, ieee, a)
+
+
+@pytest.mark.parametrize("E,F", [(4, 3), (5, 2), (2, 1), (2, 3), (3, 2), (1, 2), (5, 8), (6, 9), (5, 10)])
+def test_minifloat_mx_invariants_fixed_by_the_format(E, F):
+    """what the format itself fixes, whatever the source-specific roundings do: every code fits in 1 + E + F bits, for
+    any input and rounding mode; every code with a non-zero exponent field decodes to a value that encodes back to
+    the same code (decode after encode is the identity on the format's normal values).  Codes with exponent field 0
+    are the source-specific part (values below 2^-bias are flushed, the negative-zero code becomes the zero code):
+    for those the vectorised restatement is held to the scalar one."""
+    from helpers import adversarial_fp32_bits, fp32_from_bits
+
+    rng = np.random.default_rng(E * 16 + F)
+    x = fp32_from_bits(adversarial_fp32_bits(rng, 40000, finite_only=False))
+    for finite in (True, False):
+        for mode in ("rn", "ru", "rd", "rz"):
+            codes = O.minifloat_mx_extract(x, E, F, finite, mode)
+            assert int(codes.to(torch.int32).max()) < (1 << (1 + E + F)) and int(codes.to(torch.int32).min()) >= 0
+    all_codes = torch.arange(0, 1 << (1 + E + F), dtype=torch.int32).to(torch.uint16)
+    for finite in (True, False):
+        dec = O.minifloat_mx_compose(all_codes.clone(), E, F, finite, torch.float32)
+        back = O.minifloat_mx_extract(dec, E, F, finite, "rn").to(torch.int32)
+        want = all_codes.to(torch.int32)
+        xe = (want >> F) & ((1 << E) - 1)
+        top = (1 << E) - 1
+        expect = want.clone()
+        for i in range(want.numel()):
+            v, sgn = S.minifloat_mx_decode(int(want[i]), E, F, finite)
+            if isinstance(v, str):
+                continue
+            expect[i] = S.minifloat_mx_encode(S.f32_bits(float(v)) | ((sgn << 31) if v == 0 else 0), E, F, finite, "rn")
+        finite_code = torch.tensor([not isinstance(S.minifloat_mx_decode(int(c), E, F, finite)[0], str) for c in want])
+        assert torch.equal(back[finite_code], expect[finite_code])
+        stable = finite_code & (xe > 0) & ((xe < top) | finite)
+        assert torch.equal(back[stable], want[stable]), "normal codes must survive decode -> encode"
+
+
 # ------------------------------------------------------------------ Linear glue
 def test_linear_forwards_are_f_linear_of_quantized_operands():
     torch.manual_seed(0)
