@@ -19,6 +19,8 @@
  *   mase_mxfp_qdq           nn/quantizers/mxfp/mxfp.py:187-230    (mxfp_quantizer, non-search branch)
  *   mase_mxint_clip_search  nn/quantizers/mxint/mxint.py:40-143 (quantile_search=True without calibration activations)
  *   mase_mxfp_clip_search   nn/quantizers/mxfp/mxfp.py:40-105   (quantile_search=True without calibration activations)
+ *   mase_mxint_clip_candidates, mase_mxfp_clip_candidates   the candidates of the same searches, for the form scored
+ *                           on calibration outputs (mxint.py:99-131, mxfp.py:65-93)
  *   mase_rope               nn/quantized/functional/rope.py:17-27 (_apply_rope)
  *   mase_rmsnorm_minifloat  nn/quantized/modules/llama/rms_norm.py:72-84 (LlamaRMSNormMinifloat.forward)
  *   mase_silu_mul_minifloat nn/quantized/modules/llama/mlp.py:60-62 (silu_minifloat(gate) * up)
@@ -135,7 +137,7 @@ int mase_mxfp_qdq(const void* in, void* out, uint8_t* codes, uint8_t* scales, si
  * interpolation, as the library's quantile) instead of the maximum; the candidate the reference's error measure
  * prefers is written to `out` (same dtype as `in`), its index 0..10 to `choice` (optional, one byte per block).
  * in: the tensor with block_dim moved last, flattened; ref: the tensor in its plain flattening (the reference
- * measures the error against that one; the same array when block_dim is the last dimension).  block_size must be 32;
+ * measures the error against that one; the same array when block_dim is the last dimension).  block_size 16, 32 or 64;
  * in / ref / out 16-byte aligned.  MXINT (nn/quantizers/mxint/mxint.py:40-143): error = L2 norm in `dtype`, first
  * minimum wins.  MXFP (nn/quantizers/mxfp/mxfp.py:40-105): the reference's score on the integer codes, strictly
  * smaller replaces.  Candidates whose errors differ only by the summation order of the 32 squares may swap with respect
@@ -144,6 +146,18 @@ int mase_mxint_clip_search(const void* in, const void* ref, void* out, uint8_t* 
                            int block_size, int element_bits, int scale_bits, const uint32_t* log2_tab, void* stream);
 int mase_mxfp_clip_search(const void* in, const void* ref, void* out, uint8_t* choice, size_t numel, int dtype,
                           int block_size, int exp_bits, int frac_bits, const uint32_t* log2_tab, void* stream);
+
+/* All eleven candidates of the clip search instead of the winner, for the search scored on calibration outputs
+ * (quantile_search=True with act_tensor: nn/quantizers/mxint/mxint.py:99-131, nn/quantizers/mxfp/mxfp.py:65-93, the
+ * clip_search_y option of the GPTQ pass, passes/module/transforms/gptq/run.py:194), whose error measure is a norm over
+ * batches of activations times the candidate and is evaluated with matrix products by the caller.  in: the tensor with
+ * block_dim moved last, flattened; cand: 11 * numel elements of dtype, cand[P * numel + i] = element i quantized with
+ * the scale of percentile P.  score (MXFP only, same shape): the values the reference multiplies with the activations,
+ * code / 2^(F-1) * 2^(scale - 127) on the integer codes with the power in uint8 arithmetic.  block_size 16, 32 or 64. */
+int mase_mxint_clip_candidates(const void* in, void* cand, size_t numel, int dtype, int block_size, int element_bits,
+                               int scale_bits, const uint32_t* log2_tab, void* stream);
+int mase_mxfp_clip_candidates(const void* in, void* cand, void* score, size_t numel, int dtype, int block_size,
+                              int exp_bits, int frac_bits, const uint32_t* log2_tab, void* stream);
 
 /* Dequantization of the packed outputs of mase_mxint_qdq (kind 0: p0 = element_bits, p1 unused; value = code *
  * 2^(scale - 134)) or mase_mxfp_qdq (kind 1: p0 = exp_bits, p1 = frac_bits; value = minifloat(code) * 2^(scale - 127),

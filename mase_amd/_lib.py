@@ -50,6 +50,8 @@ SIGNATURES = {
     "mase_silu_mul_minifloat": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "mase_mxint_clip_search": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mase_mxfp_clip_search": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "mase_mxint_clip_candidates": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "mase_mxfp_clip_candidates": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mase_gemm_bf16_packed_bytes": (c_size_t, [c_size_t, c_size_t]),
     "mase_gemm_bf16_pack_b": (c_int, [c_void_p, c_void_p, c_size_t, c_size_t, c_void_p]),
     "mase_gemm_bf16_tn_packed": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_int, c_int, c_void_p]),

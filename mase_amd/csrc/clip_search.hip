@@ -5,7 +5,7 @@
 // Per block of B elements the reference quantizes 11 times, with the block's scale taken from the 1.0, 0.995, 0.99,
 // 0.97, 0.95, 0.93, 0.90, 0.80, 0.70, 0.60 and 0.50 quantile of |x| instead of the maximum, and keeps the candidate with
 // the smallest error.  It does so with some thirty tensor passes over an [11, n_blocks, B] intermediate; here one
-// work-item owns one block: the 32 magnitudes are sorted in registers (bitonic network), the quantiles interpolated,
+// work-item owns one block: the B (16, 32 or 64) magnitudes are sorted in registers (bitonic network), the quantiles interpolated,
 // the candidates with distinct scales evaluated with the device functions of the plain quantizers, and the winner
 // written once.
 //
@@ -241,21 +241,148 @@ __global__ __launch_bounds__(64) void mxfp_clip_search_kernel(const void* __rest
   if (choice != nullptr) choice[blk] = (uint8_t)best;
 }
 
+// All eleven candidates of every block instead of the winner: what the search scored on calibration outputs needs
+// (nn/quantizers/mxint/mxint.py:99-131, nn/quantizers/mxfp/mxfp.py:65-93), where a candidate's error is a norm over whole
+// batches of activations times the candidate and is left to matrix products on the host side.  cand[P * numel + i]:
+// element i of the tensor quantized with the scale of percentile P.  MXFP also writes the values the reference
+// scores, code / 2^(F-1) * 2^(scale - 127) on the integer codes with the power in uint8 arithmetic (see above).
+template <int DT, int B>
+__global__ __launch_bounds__(64) void mxint_clip_candidates_kernel(const void* __restrict__ in, void* __restrict__ cand,
+                                                                   size_t n_blocks, MxintParams p) {
+  using TR = DTypeTraits<DT>;
+  constexpr int V = TR::kVec;
+  const size_t blk = (size_t)blockIdx.x * 64 + threadIdx.x;
+  if (blk >= n_blocks) return;
+  float x[B];
+  load_block<DT, B>(in, blk, x);
+  uint32_t s[B];
+#pragma unroll
+  for (int i = 0; i < B; ++i) s[i] = f2bits(x[i]) & 0x7FFFFFFFu;
+  sort_ascending<B>(s);
+  static_for<0, kCand>([&](auto pc) __attribute__((always_inline)) {
+    constexpr int P = decltype(pc)::value;
+    const uint32_t mbits = f2bits(TR::round(clip_quantile<B, P>(s)));
+    int k = 0, kc = 0;
+    const int state = block_exponent<DT>(mbits, p, k, kc);
+    float y[B];
+#pragma unroll
+    for (int i = 0; i < B; ++i) {
+      int code;
+      y[i] = TR::round(mxint_element<DT>(x[i], state, k, kc, p, code));
+    }
+    uint4* o = (uint4*)cand + ((size_t)P * n_blocks + blk) * (B / V);
+#pragma unroll
+    for (int j = 0; j < B / V; ++j) o[j] = TR::pack(y + j * V);
+  });
+}
+
+template <int DT, int B>
+__global__ __launch_bounds__(64) void mxfp_clip_candidates_kernel(const void* __restrict__ in, void* __restrict__ cand,
+                                                                  void* __restrict__ score, size_t n_blocks,
+                                                                  MxfpParams p) {
+  using TR = DTypeTraits<DT>;
+  constexpr int V = TR::kVec;
+  const size_t blk = (size_t)blockIdx.x * 64 + threadIdx.x;
+  if (blk >= n_blocks) return;
+  float t[B];
+  load_block<DT, B>(in, blk, t);
+  uint32_t s[B];
+#pragma unroll
+  for (int i = 0; i < B; ++i) {
+    t[i] = flush_subnormal(t[i]);
+    s[i] = f2bits(t[i]) & 0x7FFFFFFFu;
+  }
+  sort_ascending<B>(s);
+  const bool all_flushed = s[B - 1] == 0;
+  const float code_unit = pow2f(1 - p.m.F);  // 1 / 2^(F-1)
+  static_for<0, kCand>([&](auto pc) __attribute__((always_inline)) {
+    constexpr int P = decltype(pc)::value;
+    int sh = 0;
+    int state = mxfp_block_scale(f2bits(clip_quantile<B, P>(s)), p, sh);
+    // states as in the search kernel: 0 all flushed, 1 regular, 2 quantile not finite, 3 zero quantile in a block
+    // that is not all zero (scale byte 255, elements x / inf, value NaN)
+    state = all_flushed ? 0 : (state == 0 ? 3 : state);
+    const int sc = (state == 0) ? 0 : (state == 1 ? sh + 127 : 255);
+    const float unit = ((sc >= 127 && sc <= 134) ? (float)(1 << (sc - 127)) : 0.0f) * code_unit;
+    float y[B], q[B];
+#pragma unroll
+    for (int i = 0; i < B; ++i) {
+      uint32_t code;
+      if (state == 3) {
+        code = minifloat_mx_encode(bits2f(f2bits(t[i]) & 0x80000000u), p.m);
+        y[i] = qnan();
+      } else {
+        y[i] = mxfp_element(t[i], state, sh, p, code);
+      }
+      q[i] = TR::round((float)code * unit);
+    }
+    uint4* o = (uint4*)cand + ((size_t)P * n_blocks + blk) * (B / V);
+    uint4* oq = (uint4*)score + ((size_t)P * n_blocks + blk) * (B / V);
+#pragma unroll
+    for (int j = 0; j < B / V; ++j) {
+      o[j] = TR::pack(y + j * V);
+      oq[j] = TR::pack(q + j * V);
+    }
+  });
+}
+
 template <typename L>
-int clip_dispatch(int dtype, L&& launch) {
+int clip_dispatch_b(int block_size, L&& launch) {
+  switch (block_size) {
+    case 16: return launch(std::integral_constant<int, 16>{});
+    case 32: return launch(std::integral_constant<int, 32>{});
+    case 64: return launch(std::integral_constant<int, 64>{});
+    default: return MASE_ERR_PARAM;
+  }
+}
+
+// launch(dtype constant, block size constant)
+template <typename L>
+int clip_dispatch(int dtype, int block_size, L&& launch) {
   switch (dtype) {
-    case MASE_DT_F32: return launch(std::integral_constant<int, MASE_DT_F32>{});
-    case MASE_DT_BF16: return launch(std::integral_constant<int, MASE_DT_BF16>{});
-    case MASE_DT_F16: return launch(std::integral_constant<int, MASE_DT_F16>{});
+    case MASE_DT_F32:
+      return clip_dispatch_b(block_size, [&](auto b) { return launch(std::integral_constant<int, MASE_DT_F32>{}, b); });
+    case MASE_DT_BF16:
+      return clip_dispatch_b(block_size, [&](auto b) { return launch(std::integral_constant<int, MASE_DT_BF16>{}, b); });
+    case MASE_DT_F16:
+      return clip_dispatch_b(block_size, [&](auto b) { return launch(std::integral_constant<int, MASE_DT_F16>{}, b); });
     default: return MASE_ERR_DTYPE;
   }
+}
+
+MxintParams make_mxint_params(int element_bits, int scale_bits, int dtype, const uint32_t* log2_tab) {
+  MxintParams p;
+  p.qshift = element_bits - 1;
+  p.bias = (1 << (scale_bits - 1)) - 1;
+  p.scale_max = (1 << scale_bits) - 1;
+  p.lo = mase_round_scalar_to_dtype(-(double)(1 << (element_bits - 1)), dtype);
+  p.hi = mase_round_scalar_to_dtype((double)((1 << (element_bits - 1)) - 1), dtype);
+  p.tab = log2_tab;
+  return p;
+}
+
+bool make_mxfp_params(int exp_bits, int frac_bits, const uint32_t* log2_tab, MxfpParams& p) {
+  const int legal[6][2] = {{4, 3}, {5, 2}, {2, 3}, {3, 2}, {2, 1}, {1, 2}};  // nn/quantizers/mxfp/meta.py:41
+  bool ok = false;
+  for (auto& l : legal) ok = ok || (l[0] == exp_bits && l[1] == frac_bits);
+  if (!ok) return false;
+  p.m.E = exp_bits;
+  p.m.F = frac_bits;
+  p.m.bias = (1 << (exp_bits - 1)) - 1;
+  p.m.e_hi = (1 << exp_bits) - 1;
+  p.m.frac_hi = (1 << frac_bits) - 1;
+  p.m.is_finite = 1;
+  p.m.round_mode = 0;
+  p.el_emax = p.m.e_hi - p.m.bias;
+  p.tab = log2_tab;
+  return true;
 }
 
 int clip_args(const void* in, const void* ref, void* out, size_t numel, int dtype, int block_size,
               const uint32_t* log2_tab) {
   if (in == nullptr || ref == nullptr || out == nullptr || log2_tab == nullptr) return MASE_ERR_NULL;
-  if (block_size != 32) return MASE_ERR_PARAM;
-  if (numel % 32 != 0) return MASE_ERR_SHAPE;
+  if (block_size != 16 && block_size != 32 && block_size != 64) return MASE_ERR_PARAM;
+  if (numel % (size_t)block_size != 0) return MASE_ERR_SHAPE;
   if (dtype != MASE_DT_F32 && dtype != MASE_DT_BF16 && dtype != MASE_DT_F16) return MASE_ERR_DTYPE;
   if (!aligned16(in) || !aligned16(ref) || !aligned16(out)) return MASE_ERR_ALIGN;
   return MASE_OK;
@@ -271,18 +398,12 @@ extern "C" int mase_mxint_clip_search(const void* in, const void* ref, void* out
   if (numel == 0) return MASE_OK;
   if (int rc = clip_args(in, ref, out, numel, dtype, block_size, log2_tab)) return rc;
   if (element_bits < 2 || element_bits > 24 || scale_bits < 1 || scale_bits > 8) return MASE_ERR_PARAM;
-  MxintParams p;
-  p.qshift = element_bits - 1;
-  p.bias = (1 << (scale_bits - 1)) - 1;
-  p.scale_max = (1 << scale_bits) - 1;
-  p.lo = mase_round_scalar_to_dtype(-(double)(1 << (element_bits - 1)), dtype);
-  p.hi = mase_round_scalar_to_dtype((double)((1 << (element_bits - 1)) - 1), dtype);
-  p.tab = log2_tab;
-  const size_t n_blocks = numel / 32;
+  const MxintParams p = make_mxint_params(element_bits, scale_bits, dtype, log2_tab);
+  const size_t n_blocks = numel / (size_t)block_size;
   hipStream_t st = (hipStream_t)stream;
-  return clip_dispatch(dtype, [&](auto dt) {
-    constexpr int DT = decltype(dt)::value;
-    hipLaunchKernelGGL((mxint_clip_search_kernel<DT, 32>), dim3(blocks_for(n_blocks, 64)), dim3(64), 0, st, in, ref, out,
+  return clip_dispatch(dtype, block_size, [&](auto dt, auto bs) {
+    constexpr int DT = decltype(dt)::value, B = decltype(bs)::value;
+    hipLaunchKernelGGL((mxint_clip_search_kernel<DT, B>), dim3(blocks_for(n_blocks, 64)), dim3(64), 0, st, in, ref, out,
                        choice, n_blocks, p);
     return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
   });
@@ -294,26 +415,51 @@ extern "C" int mase_mxfp_clip_search(const void* in, const void* ref, void* out,
   using namespace mase;
   if (numel == 0) return MASE_OK;
   if (int rc = clip_args(in, ref, out, numel, dtype, block_size, log2_tab)) return rc;
-  const int legal[6][2] = {{4, 3}, {5, 2}, {2, 3}, {3, 2}, {2, 1}, {1, 2}};  // nn/quantizers/mxfp/meta.py:41
-  bool ok = false;
-  for (auto& l : legal) ok = ok || (l[0] == exp_bits && l[1] == frac_bits);
-  if (!ok) return MASE_ERR_PARAM;
   MxfpParams p;
-  p.m.E = exp_bits;
-  p.m.F = frac_bits;
-  p.m.bias = (1 << (exp_bits - 1)) - 1;
-  p.m.e_hi = (1 << exp_bits) - 1;
-  p.m.frac_hi = (1 << frac_bits) - 1;
-  p.m.is_finite = 1;
-  p.m.round_mode = 0;
-  p.el_emax = p.m.e_hi - p.m.bias;
-  p.tab = log2_tab;
-  const size_t n_blocks = numel / 32;
+  if (!make_mxfp_params(exp_bits, frac_bits, log2_tab, p)) return MASE_ERR_PARAM;
+  const size_t n_blocks = numel / (size_t)block_size;
   hipStream_t st = (hipStream_t)stream;
-  return clip_dispatch(dtype, [&](auto dt) {
-    constexpr int DT = decltype(dt)::value;
-    hipLaunchKernelGGL((mxfp_clip_search_kernel<DT, 32>), dim3(blocks_for(n_blocks, 64)), dim3(64), 0, st, in, ref, out,
+  return clip_dispatch(dtype, block_size, [&](auto dt, auto bs) {
+    constexpr int DT = decltype(dt)::value, B = decltype(bs)::value;
+    hipLaunchKernelGGL((mxfp_clip_search_kernel<DT, B>), dim3(blocks_for(n_blocks, 64)), dim3(64), 0, st, in, ref, out,
                        choice, n_blocks, p);
+    return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+  });
+}
+
+extern "C" int mase_mxint_clip_candidates(const void* in, void* cand, size_t numel, int dtype, int block_size,
+                                          int element_bits, int scale_bits, const uint32_t* log2_tab, void* stream) {
+  using namespace mase;
+  if (numel == 0) return MASE_OK;
+  if (int rc = clip_args(in, in, cand, numel, dtype, block_size, log2_tab)) return rc;
+  if (element_bits < 2 || element_bits > 24 || scale_bits < 1 || scale_bits > 8) return MASE_ERR_PARAM;
+  const MxintParams p = make_mxint_params(element_bits, scale_bits, dtype, log2_tab);
+  const size_t n_blocks = numel / (size_t)block_size;
+  hipStream_t st = (hipStream_t)stream;
+  return clip_dispatch(dtype, block_size, [&](auto dt, auto bs) {
+    constexpr int DT = decltype(dt)::value, B = decltype(bs)::value;
+    hipLaunchKernelGGL((mxint_clip_candidates_kernel<DT, B>), dim3(blocks_for(n_blocks, 64)), dim3(64), 0, st, in, cand,
+                       n_blocks, p);
+    return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+  });
+}
+
+extern "C" int mase_mxfp_clip_candidates(const void* in, void* cand, void* score, size_t numel, int dtype,
+                                         int block_size, int exp_bits, int frac_bits, const uint32_t* log2_tab,
+                                         void* stream) {
+  using namespace mase;
+  if (numel == 0) return MASE_OK;
+  if (score == nullptr) return MASE_ERR_NULL;
+  if (int rc = clip_args(in, in, cand, numel, dtype, block_size, log2_tab)) return rc;
+  if (!aligned16(score)) return MASE_ERR_ALIGN;
+  MxfpParams p;
+  if (!make_mxfp_params(exp_bits, frac_bits, log2_tab, p)) return MASE_ERR_PARAM;
+  const size_t n_blocks = numel / (size_t)block_size;
+  hipStream_t st = (hipStream_t)stream;
+  return clip_dispatch(dtype, block_size, [&](auto dt, auto bs) {
+    constexpr int DT = decltype(dt)::value, B = decltype(bs)::value;
+    hipLaunchKernelGGL((mxfp_clip_candidates_kernel<DT, B>), dim3(blocks_for(n_blocks, 64)), dim3(64), 0, st, in, cand,
+                       score, n_blocks, p);
     return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
   });
 }

@@ -13,8 +13,8 @@ device.  Weights are written back into the ``nn.Linear`` modules, so that the qu
 
 Differences from the reference's driver: calibration token ids are passed in (``gptq_config["calibration_data"]``, an
 integer tensor ``[nsamples, seqlen]`` or a list of ``[1, seqlen]`` tensors) instead of being downloaded by dataset
-name; ``clip_search_y`` (the search scored on calibration outputs, ``act_tensor``) and the per-layer checkpoint files
-are not built and raise ``NotImplementedError``.
+name; the per-layer checkpoint files are not built and raise ``NotImplementedError``.  ``clip_search_y`` scores the
+clip search of each column group on the group's calibration inputs (``mase_mx*_clip_candidates`` plus matrix products).
 """
 from __future__ import annotations
 
@@ -94,8 +94,6 @@ class GPTQ:
     def fasterquant(self, activation, fmt, weight_config, percdamp=0.01, cali_batch_size=32, layer_name=None,
                     quant_search=True):
         """gptq.py:39-122"""
-        if activation is not None:
-            raise NotImplementedError("GPTQ with the clip search scored on calibration outputs (clip_search_y) is not built")
         W = self.layer.weight.data.clone()
         Hinv, dead = self.inverse_factor(percdamp)
         W[:, dead] = 0
@@ -104,7 +102,10 @@ class GPTQ:
         for i1 in range(0, self.columns, blocksize):
             i2 = min(i1 + blocksize, self.columns)
             W1 = W[:, i1:i2].clone()
-            Q1 = quantize_tensor(W1, block_dim=1, fmt=fmt, config=weight_config, quantile_search=quant_search)
+            # clip_search_y: the group's search is scored on the layer's calibration inputs of these columns
+            act1 = None if activation is None else activation[:, :, i1:i2].clone()
+            Q1 = quantize_tensor(W1, block_dim=1, fmt=fmt, config=weight_config, quantile_search=quant_search,
+                                 act_tensor=act1, cali_batch_size=cali_batch_size)
             Q[:, i1:i2] = Q1
             if i2 < self.columns:
                 err = (W1 - Q1) / torch.diag(Hinv[i1:i2, i1:i2]).unsqueeze(0)
@@ -126,10 +127,13 @@ _SEQUENTIAL = (  # run.py:136-141
 
 @torch.no_grad()
 def gptq_decoder_layer(layer, run_layer, nsamples: int, fmt: str, weight_config: dict, quantile_search: bool = True,
-                       cali_batch_size: int = 32, sequential=_SEQUENTIAL, layer_name: str = ""):
+                       cali_batch_size: int = 32, sequential=_SEQUENTIAL, layer_name: str = "",
+                       clip_search_y: bool = False):
     """The per-layer body of run.py:150-214: for each group of projections in ``sequential``, run the layer over the
     ``nsamples`` calibration samples (``run_layer(j)`` runs sample j through ``layer``) with hooks that feed each
-    projection's inputs to its GPTQ object, then quantize those projections and write the weights back."""
+    projection's inputs to its GPTQ object, then quantize those projections and write the weights back.
+    ``clip_search_y``: the inputs of the group (its projections share them; recorded at the last one, run.py:173) are
+    kept as [nsamples, tokens, columns] and the clip search of every column group is scored on them."""
     full = find_qlayers(layer, layers=[nn.Linear])
     for names in sequential:
         subset = {n: full[n] for n in names if n in full}
@@ -143,14 +147,19 @@ def gptq_decoder_layer(layer, run_layer, nsamples: int, fmt: str, weight_config:
             return fn
 
         handles = [m.register_forward_hook(hook(n)) for n, m in subset.items()]
+        pre_act = []
+        if clip_search_y:
+            last = list(subset.values())[-1]
+            handles.append(last.register_forward_pre_hook(lambda _, inp: pre_act.append(inp[0])))
         try:
             for j in range(nsamples):
                 run_layer(j)
         finally:
             for h in handles:
                 h.remove()
+        activation = torch.cat(pre_act, dim=0) if clip_search_y else None
         for n, m in subset.items():
-            q = gptq[n].fasterquant(activation=None, fmt=fmt, weight_config=weight_config, percdamp=0.01,
+            q = gptq[n].fasterquant(activation=activation, fmt=fmt, weight_config=weight_config, percdamp=0.01,
                                     cali_batch_size=cali_batch_size, layer_name=f"{layer_name}.{n}",
                                     quant_search=quantile_search)
             assert q.shape == m.weight.shape
@@ -174,9 +183,9 @@ def run_gptq(network, gptq_config):
     """run.py:20-232 for a ``transformers`` causal LM with ``network.model.layers`` / ``embed_tokens`` / ``norm`` /
     ``rotary_emb``: GPTQ over every ``nn.Linear`` of every decoder layer, layer by layer, the inputs of layer i+1 being
     the outputs of the already quantized layer i.  Keys of ``gptq_config`` as in the reference (``device``, ``format``,
-    ``weight_config``, ``quantile_search``, ``cali_batch_size``, ``max_layers``) plus ``calibration_data``."""
-    if gptq_config.get("clip_search_y", False):
-        raise NotImplementedError("run_gptq: clip_search_y (the search scored on calibration outputs) is not built")
+    ``weight_config``, ``quantile_search``, ``clip_search_y``, ``cali_batch_size``, ``max_layers``) plus
+    ``calibration_data``."""
+    clip_search_y = gptq_config.get("clip_search_y", False)
     if gptq_config.get("checkpoint_dir") is not None:
         raise NotImplementedError("run_gptq: per-layer checkpoint files are not built")
     dev = gptq_config.get("device", "cuda:0")
@@ -236,7 +245,7 @@ def run_gptq(network, gptq_config):
             outs[j] = out[0] if isinstance(out, tuple) else out
 
         gptq_decoder_layer(layer, run_layer, nsamples, fmt, weight_config, quantile_search, cali_batch_size,
-                           layer_name=f"layers{i}")
+                           layer_name=f"layers{i}", clip_search_y=clip_search_y)
         for j in range(nsamples):  # run.py:197-205: the quantized layer's outputs feed the next layer
             run_layer(j)
         inps, outs = outs, inps

@@ -85,19 +85,15 @@ class MXFPMeta:
 # ---------------------------------------------------------------------------------------------
 # MXINT
 # ---------------------------------------------------------------------------------------------
-def _reject_calibration(act_tensor, name: str):
-    if act_tensor is not None:
-        raise NotImplementedError(
-            f"{name}: quantile_search with calibration activations (GPTQ) is outside the accelerated path"
-        )
-
-
 def mxint_quantizer_sim(tensor: Tensor, block_dim: int, mxint_meta: MXIntMeta, act_tensor: Tensor | None = None,
                         dtype: torch.dtype | None = None, quantile_search: bool = False,
                         cali_batch_size: int = 32) -> Tensor:
-    """mxint/mxint.py:14-171; the search branch (:40-143) without calibration activations."""
+    """mxint/mxint.py:14-171, both forms of the search branch (:40-143): scored on the weights themselves, or with
+    ``act_tensor`` [batches, tokens, block_size] on the products with calibration activations."""
     if quantile_search:
-        _reject_calibration(act_tensor, "mxint_quantizer_sim")
+        if act_tensor is not None:
+            return _ops.mxint_clip_search_calibrated(tensor, mxint_meta.block_size, mxint_meta.element_bits, block_dim,
+                                                     mxint_meta.scale_bits, act_tensor, cali_batch_size)
         return _ops.mxint_clip_search(tensor, mxint_meta.block_size, mxint_meta.element_bits, block_dim,
                                       mxint_meta.scale_bits)  # the search branch ignores `dtype` (mxint.py:143)
     out = _ops.mxint_qdq(tensor, mxint_meta.block_size, mxint_meta.element_bits, block_dim, mxint_meta.scale_bits)
@@ -126,11 +122,16 @@ def mxfp_quantizer_sim(tensor: Tensor, block_dim: int, mxfp_meta: MXFPMeta, act_
                        dtype: torch.dtype | None = None, quantile_search: bool = False,
                        cali_batch_size: int = 32) -> Tensor:
     """mxfp/mxfp.py:14-115 (finite elements, round-to-nearest as MXFPQuantize fixes them); the search branch
-    (:40-105) without calibration activations."""
+    (:40-105) scored on the weights themselves or, with ``act_tensor`` [batches, tokens, block_size], on the products
+    with calibration activations."""
     if not (mxfp_meta.element_is_finite and mxfp_meta.round_mode == "rn"):
         raise NotImplementedError("mxfp_quantizer_sim: only finite elements with round mode 'rn' are accelerated")
     if quantile_search:
-        _reject_calibration(act_tensor, "mxfp_quantizer_sim")
+        if act_tensor is not None:
+            out = _ops.mxfp_clip_search_calibrated(tensor, mxfp_meta.block_size, mxfp_meta.element_exp_bits,
+                                                   mxfp_meta.element_frac_bits, block_dim, mxfp_meta.scale_exp_bits,
+                                                   act_tensor, cali_batch_size)
+            return out.to(dtype or tensor.dtype)
         out = _ops.mxfp_clip_search(tensor, mxfp_meta.block_size, mxfp_meta.element_exp_bits,
                                     mxfp_meta.element_frac_bits, block_dim, mxfp_meta.scale_exp_bits)
         return out.to(dtype or tensor.dtype)

@@ -153,7 +153,7 @@ def mxfp_qdq(x: Tensor, block_size: int, exp_bits: int, frac_bits: int, block_di
     return (res, codes, scales) if pack else res
 
 
-CLIP_SEARCH_BLOCK = 32
+CLIP_SEARCH_BLOCKS = (16, 32, 64)
 
 
 def _clip_search(name: str, x: Tensor, block_size: int, block_dim: int, tab_dtype, params, return_choice: bool):
@@ -161,8 +161,8 @@ def _clip_search(name: str, x: Tensor, block_size: int, block_dim: int, tab_dtyp
     measured against the blocks of the plain flattening (mxint/mxint.py:41-45, :97; mxfp/mxfp.py:41-45, :94-97)"""
     _lib.require_device(x, name)
     lib = _lib.load()
-    if block_size != CLIP_SEARCH_BLOCK:
-        raise NotImplementedError(f"{name}: quantile_search=True is built for block_size {CLIP_SEARCH_BLOCK}, got {block_size}")
+    if block_size not in CLIP_SEARCH_BLOCKS:
+        raise NotImplementedError(f"{name}: quantile_search=True is built for block sizes {CLIP_SEARCH_BLOCKS}, got {block_size}")
     shape = tuple(x.shape)
     nd = len(shape)
     assert block_dim < nd and block_dim >= -nd
@@ -198,6 +198,105 @@ def mxfp_clip_search(x: Tensor, block_size: int, exp_bits: int, frac_bits: int, 
     )
     return _clip_search("mase_mxfp_clip_search", x, block_size, block_dim, torch.float32, (exp_bits, frac_bits),
                         return_choice)
+
+
+def _clip_candidates(name: str, x: Tensor, block_size: int, block_dim: int, tab_dtype, params, with_score: bool):
+    """the eleven candidates of the search as [11, n_blocks, B] (blocks along block_dim), and for MXFP the values the
+    reference scores (same shape)"""
+    _lib.require_device(x, name)
+    lib = _lib.load()
+    if block_size not in CLIP_SEARCH_BLOCKS:
+        raise NotImplementedError(f"{name}: quantile_search=True is built for block sizes {CLIP_SEARCH_BLOCKS}, got {block_size}")
+    nd = x.dim()
+    assert block_dim < nd and block_dim >= -nd
+    assert x.numel() % block_size == 0, f"Input tensor size {x.numel()} is not divisible by block size {block_size}."
+    flat = _to_block_last_flat(x, block_dim)
+    if flat.data_ptr() % 16:
+        flat = flat.clone()
+    n = flat.numel()
+    cand = torch.empty((11, n // block_size, block_size), dtype=x.dtype, device=x.device)
+    score = torch.empty_like(cand) if with_score else None
+    tab = log2_table(tab_dtype, x.device)
+    fn = getattr(lib, name)
+    args = [flat.data_ptr(), cand.data_ptr()] + ([score.data_ptr()] if with_score else [])
+    rc = fn(*args, n, _lib.dtype_code(x), block_size, *params, tab.data_ptr(), _lib.stream_ptr(x))
+    _lib.check(rc, name)
+    return cand, score
+
+
+def _calibration_view(act_tensor: Tensor, block_size: int) -> Tensor:
+    """The reference contracts the calibration activations [batches, tokens, B] with blocks of B weights; an
+    activation tensor whose last dimension is a multiple of B is viewed as [..., last/B, B] there and then fails in
+    the contraction (mxint.py:101-104, :121; mxfp.py:67-72, :86), so only last dimension == B is a usable input."""
+    if act_tensor.dim() != 3 or act_tensor.shape[-1] != block_size:
+        raise ValueError(f"act_tensor must be [batches, tokens, {block_size}] (the block size), got {tuple(act_tensor.shape)}")
+    return act_tensor
+
+
+_CAL_CHUNK_ELEMS = 1 << 28  # elements of the [11, a, s, rows] product held at a time
+
+
+def mxint_clip_search_calibrated(x: Tensor, block_size: int, element_bits: int, block_dim: int, scale_bits: int,
+                                 act_tensor: Tensor, cali_batch_size: int = 32, return_choice: bool = False):
+    """quantile_search=True with act_tensor (mxint/mxint.py:99-143): the candidate of each block of weights whose
+    product with the calibration activations is closest to the unquantized block's, the distance being the sum over
+    batches of ``cali_batch_size`` samples of the 2-norm over (sample, token).  The candidates come from
+    ``mase_mxint_clip_candidates``; the products and norms are the reference's tensor operations on the device, done
+    for groups of weight rows so that the [11, samples, tokens, rows] product stays bounded."""
+    act = _calibration_view(act_tensor, block_size)
+    shape = tuple(x.shape)
+    cand, _ = _clip_candidates("mase_mxint_clip_candidates", x, block_size, block_dim, x.dtype,
+                               (element_bits, scale_bits), False)
+    rows = x.contiguous().flatten().reshape(-1, block_size)          # blocks of the plain flattening (mxint.py:41-45)
+    H = rows.shape[0]
+    err = torch.zeros((11, H), device=x.device, dtype=x.dtype)
+    for b in range(0, act.shape[0], cali_batch_size):
+        act_b = act[b:b + cali_batch_size]
+        step = max(1, _CAL_CHUNK_ELEMS // max(1, 11 * act_b.shape[0] * act_b.shape[1]))
+        for h0 in range(0, H, step):
+            h1 = min(H, h0 + step)
+            out_orig = torch.matmul(act_b, rows[h0:h1].T)
+            out_q = torch.einsum("asb,phb->pash", act_b, cand[:, h0:h1].to(act.dtype))
+            err[:, h0:h1] += torch.norm(out_q - out_orig, p=2, dim=(1, 2))
+    pick = torch.argmin(err, dim=0)
+    chosen = cand[pick, torch.arange(H, device=x.device)]
+    out = _from_block_last_flat(chosen.reshape(-1), shape, block_dim).to(x.dtype)
+    return (out, pick.to(torch.uint8)) if return_choice else out
+
+
+def mxfp_clip_search_calibrated(x: Tensor, block_size: int, exp_bits: int, frac_bits: int, block_dim: int,
+                                scale_exp_bits: int, act_tensor: Tensor, cali_batch_size: int = 32,
+                                return_choice: bool = False):
+    """quantile_search=True with act_tensor (mxfp/mxfp.py:40-115): per percentile the reference multiplies the
+    activations with its score values (integer codes times the uint8 power, see ``mase_mxfp_clip_candidates``) and
+    with the unquantized blocks, takes the 2-norm of the difference over (sample, token) summed over the batches, and
+    replaces the incumbent on a strictly smaller error."""
+    assert scale_exp_bits in (8,), f"Invalid scale exponent bits: {scale_exp_bits}. Legal values are: (8,)."
+    assert (exp_bits, frac_bits) in _LEGAL_MXFP, (
+        f"Invalid element exp/frac bits: {(exp_bits, frac_bits)}. Legal values are: {_LEGAL_MXFP}."
+    )
+    act = _calibration_view(act_tensor, block_size)
+    shape = tuple(x.shape)
+    cand, score = _clip_candidates("mase_mxfp_clip_candidates", x, block_size, block_dim, torch.float32,
+                                   (exp_bits, frac_bits), True)
+    rows = x.contiguous().flatten().reshape(-1, block_size)
+    H = rows.shape[0]
+    best = torch.full([H], float("inf"), device=x.device, dtype=x.dtype)
+    pick = torch.zeros(H, dtype=torch.int64, device=x.device)
+    for p in range(11):
+        q = score[p].to(rows.dtype)
+        err = torch.zeros(H, device=x.device, dtype=x.dtype)
+        for b in range(0, act.shape[0], cali_batch_size):
+            act_b = act[b:b + cali_batch_size]
+            out_q = torch.matmul(act_b, q.T)
+            out_orig = torch.matmul(act_b, rows.T)
+            err += torch.norm(out_q - out_orig, p=2, dim=(0, 1))
+        better = err < best
+        best = torch.where(better, err, best)
+        pick = torch.where(better, torch.full_like(pick, p), pick)
+    chosen = cand[pick, torch.arange(H, device=x.device)]
+    out = _from_block_last_flat(chosen.reshape(-1), shape, block_dim)
+    return (out, pick.to(torch.uint8)) if return_choice else out
 
 
 def _cast_args(cast):

@@ -12,7 +12,7 @@ import math
 
 import torch
 
-from .quantizers import mxfp_quantizer, mxint_quantizer
+from .quantizers import mxfp_clip_search, mxfp_quantizer, mxint_clip_search, mxint_quantizer
 
 
 def hessian(batches):
@@ -45,8 +45,17 @@ def inverse_factor(H, percdamp=0.01):
     return torch.linalg.cholesky(H, upper=True), dead
 
 
-def quantize_group(W1, fmt, weight_config, quant_search):
-    """quantize_dispatch.py:36-82 with block_dim=1"""
+def quantize_group(W1, fmt, weight_config, quant_search, act_tensor=None, cali_batch_size=32):
+    """quantize_dispatch.py:36-82 with block_dim=1; ``act_tensor``: the calibration inputs of these columns, which
+    only the search branch looks at (mxint.py:99, mxfp.py:65)"""
+    if act_tensor is not None and quant_search:
+        bs = weight_config["weight_block_size"]
+        if fmt == "mxint":
+            return mxint_clip_search(W1, bs, weight_config["weight_width"], 1, act_tensor=act_tensor,
+                                     cali_batch_size=cali_batch_size)[0]
+        if fmt == "mxfp":
+            return mxfp_clip_search(W1, bs, weight_config["weight_exponent_width"], weight_config["weight_frac_width"], 1,
+                                    act_tensor=act_tensor, cali_batch_size=cali_batch_size)[0]
     if fmt == "mxint":
         return mxint_quantizer(W1, weight_config["weight_block_size"], weight_config["weight_width"], 1,
                                quantile_search=quant_search)
@@ -56,8 +65,8 @@ def quantize_group(W1, fmt, weight_config, quant_search):
     raise ValueError(fmt)
 
 
-def fasterquant(weight, H, fmt, weight_config, percdamp=0.01, quant_search=True):
-    """gptq.py:39-122 with activation=None"""
+def fasterquant(weight, H, fmt, weight_config, percdamp=0.01, quant_search=True, activation=None, cali_batch_size=32):
+    """gptq.py:39-122; ``activation`` [nsamples, tokens, columns]: the layer's calibration inputs (clip_search_y)"""
     W = weight.clone()
     Hinv, dead = inverse_factor(H, percdamp)
     W[:, dead] = 0
@@ -67,7 +76,8 @@ def fasterquant(weight, H, fmt, weight_config, percdamp=0.01, quant_search=True)
     for i1 in range(0, cols, bs):
         i2 = min(i1 + bs, cols)
         W1 = W[:, i1:i2].clone()
-        Q1 = quantize_group(W1, fmt, weight_config, quant_search)
+        act1 = None if activation is None else activation[:, :, i1:i2].clone()
+        Q1 = quantize_group(W1, fmt, weight_config, quant_search, act1, cali_batch_size)
         Hinv1 = Hinv[i1:i2, i1:i2]
         err = (W1 - Q1) / torch.diag(Hinv1).unsqueeze(0)
         Q[:, i1:i2] = Q1

@@ -86,8 +86,10 @@ def mxint_quantizer(
 CLIP_PERCENTILES = (1.0, 0.995, 0.99, 0.97, 0.95, 0.93, 0.90, 0.80, 0.70, 0.60, 0.50)  # mxint.py:47-51, mxfp.py:53
 
 
-def mxint_clip_search(x: Tensor, block_size: int, element_bits: int, block_dim: int = -1, scale_bits: int = 8):
-    """The search branch of mxint_quantizer_sim with act_tensor=None (mxint/mxint.py:40-143).
+def mxint_clip_search(x: Tensor, block_size: int, element_bits: int, block_dim: int = -1, scale_bits: int = 8,
+                      act_tensor: Tensor | None = None, cali_batch_size: int = 32):
+    """The search branch of mxint_quantizer_sim (mxint/mxint.py:40-143), scored on the weights (act_tensor=None, :97-98)
+    or on their products with calibration activations [batches, tokens, B] (:99-131).
 
     Returns (dequantized tensor, index of the chosen percentile per block, errors [11, n_blocks], candidates
     [11, n_blocks, B]).  The candidates are the blocks taken along block_dim; the error is measured against the blocks of the plain flattening (:41-45, :97),
@@ -108,8 +110,18 @@ def mxint_clip_search(x: Tensor, block_size: int, element_bits: int, block_dim: 
     scale = (scale + bias).clamp(min=0, max=2**scale_bits - 1)  # :81-82
     mant = mant.round().clamp(min=-(2 ** (element_bits - 1)), max=2 ** (element_bits - 1) - 1)  # :83-86
     cand = mant / 2 ** (element_bits - 1) * 2 ** (scale - bias)  # :88-90
-    err = torch.norm(cand - rows, p=2, dim=-1)  # :97
-    pick = torch.argmin(err, dim=0).reshape(-1)  # :98
+    if act_tensor is None:
+        err = torch.norm(cand - rows, p=2, dim=-1)  # :97
+        pick = torch.argmin(err, dim=0).reshape(-1)  # :98
+    else:
+        assert act_tensor.shape[-1] == B  # :101-104 views any other width to 4-D, which the contraction below rejects
+        err = torch.zeros([len(CLIP_PERCENTILES), rows.shape[0]], dtype=x.dtype)  # :107-111
+        for b in range(0, act_tensor.shape[0], cali_batch_size):  # :114-126
+            act_b = act_tensor[b:b + cali_batch_size]
+            out_orig = torch.matmul(act_b, rows.T)
+            out_q = torch.einsum("asb,phb->pash", act_b, cand.to(act_tensor.dtype))
+            err += torch.norm(out_q - out_orig, p=2, dim=(1, 2))
+        pick = torch.argmin(err, dim=0)  # :128
     chosen = cand[pick, torch.arange(cand.shape[1])]  # :132
     out = _restore_from_flat(chosen, shape, block_dim).to(x.dtype)  # :141-143
     return out, pick, err, cand
@@ -278,8 +290,10 @@ def mxfp_quantizer(
 
 
 def mxfp_clip_search(x: Tensor, block_size: int, element_exp_bits: int, element_frac_bits: int, block_dim: int = -1,
-                     scale_exp_bits: int = 8, dtype: torch.dtype | None = None):
-    """The search branch of mxfp_quantizer_sim with act_tensor=None (mxfp/mxfp.py:40-105).
+                     scale_exp_bits: int = 8, dtype: torch.dtype | None = None, act_tensor: Tensor | None = None,
+                     cali_batch_size: int = 32):
+    """The search branch of mxfp_quantizer_sim (mxfp/mxfp.py:40-105), scored on the weights (act_tensor=None, :94-97) or
+    on the products with calibration activations [batches, tokens, B] (:65-93).
 
     Returns (dequantized tensor, index of the chosen percentile per block, errors [11, n_blocks], candidates
     [11, n_blocks, B] dequantized).  The score of a
@@ -306,10 +320,19 @@ def mxfp_clip_search(x: Tensor, block_size: int, element_exp_bits: int, element_
         sc, el = mxfp_components(flat, B, element_exp_bits, element_frac_bits, scale_exp_bits, True, "rn", pct)
         q = el / 2 ** (element_frac_bits - 1) * 2 ** (sc - sc_bias)  # :58-62 (uint8 tensors: sc - bias and 2**() wrap)
         q = q.to(dtype=rows.dtype)  # :63
-        q -= rows  # :94
-        q.abs_()
-        q.pow_(2)
-        err = torch.sum(q, 1)  # :97
+        if act_tensor is not None:
+            assert act_tensor.shape[-1] == B  # :67-72 views any other width to 4-D, which makes the error's shape wrong
+            err = torch.zeros(rows.shape[0], dtype=x.dtype)  # :75-77
+            for b in range(0, act_tensor.shape[0], cali_batch_size):  # :80-90
+                act_b = act_tensor[b:b + cali_batch_size]
+                out_q = torch.matmul(act_b, q.T)
+                out_orig = torch.matmul(act_b, rows.T)
+                err += torch.norm(out_q - out_orig, p=2, dim=(0, 1))
+        else:
+            q -= rows  # :94
+            q.abs_()
+            q.pow_(2)
+            err = torch.sum(q, 1)  # :97
         errs.append(err)
         cands.append(compose(sc, el))
         better = err < best  # :99

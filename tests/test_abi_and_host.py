@@ -104,14 +104,26 @@ def test_entry_points_reject_bad_arguments_without_a_gpu(lib):
     assert lib.mase_gemm_mxfp4_skinny(p, p, 0, p, p, None, p, 4, 4, 128, 7, 0, p, 4096, None) == -4
     assert lib.mase_gemm_mxfp4_skinny_workspace_bytes(4, 4, 192) == 0
     # mase_mxint_clip_search(in, ref, out, choice, numel, dtype, block_size, element_bits, scale_bits, tab, stream)
-    assert lib.mase_mxint_clip_search(p, p, p, None, 64, 0, 16, 8, 8, p, None) == -5     # block size 32 only
+    assert lib.mase_mxint_clip_search(p, p, p, None, 64, 0, 8, 8, 8, p, None) == -5      # block sizes 16, 32, 64
     assert lib.mase_mxint_clip_search(p, p, p, None, 48, 0, 32, 8, 8, p, None) == -2
     assert lib.mase_mxint_clip_search(p, None, p, None, 64, 0, 32, 8, 8, p, None) == -1
     assert lib.mase_mxint_clip_search(p, p, p, None, 64, 0, 32, 1, 8, p, None) == -5
     assert lib.mase_mxint_clip_search(p, p, p, None, 64, 3, 32, 8, 8, p, None) == -4
     assert lib.mase_mxint_clip_search(p, p, p, None, 0, 0, 32, 8, 8, p, None) == 0
     assert lib.mase_mxfp_clip_search(p, p, p, None, 64, 0, 32, 3, 3, p, None) == -5      # illegal element format
-    assert lib.mase_mxfp_clip_search(p, p, p, None, 64, 0, 64, 4, 3, p, None) == -5
+    assert lib.mase_mxfp_clip_search(p, p, p, None, 64, 0, 128, 4, 3, p, None) == -5
+    # mase_mxint_clip_candidates(in, cand, numel, dtype, block_size, element_bits, scale_bits, tab, stream)
+    assert lib.mase_mxint_clip_candidates(p, p, 64, 0, 24, 8, 8, p, None) == -5
+    assert lib.mase_mxint_clip_candidates(p, None, 64, 0, 32, 8, 8, p, None) == -1
+    assert lib.mase_mxint_clip_candidates(p, p, 72, 0, 16, 8, 8, p, None) == -2
+    assert lib.mase_mxint_clip_candidates(p, p, 0, 0, 16, 8, 8, p, None) == 0
+    # mase_mxfp_clip_candidates(in, cand, score, numel, dtype, block_size, exp_bits, frac_bits, tab, stream)
+    assert lib.mase_mxfp_clip_candidates(p, p, None, 64, 0, 32, 2, 1, p, None) == -1
+    assert lib.mase_mxfp_clip_candidates(p, p, p, 64, 0, 32, 3, 3, p, None) == -5
+    assert lib.mase_mxfp_clip_candidates(p, p, p, 64, 5, 32, 2, 1, p, None) == -4
+    # mase_block_fp_qdq_static: the size limit is checked before anything touches a device
+    assert lib.mase_block_fp_qdq_static(p, p, 1, 1, (1 << 20) + 1, 1, 1, 1, 8, 8, -1, 0, p, None) == -7
+    assert lib.mase_block_fp_qdq_static(p, p, 0, 1, 16, 1, 16, 1, 8, 8, -1, 0, p, None) == 0
     assert lib.mase_mxfp_clip_search(p, p, None, None, 64, 0, 32, 4, 3, p, None) == -1
     assert lib.mase_mxfp_qdq(p, p, None, None, 64, 0, 0, 32, 3, 3, p, None) == -5  # illegal element format
     assert lib.mase_mxfp_qdq(p, p, None, None, 63, 0, 0, 32, 4, 3, p, None) == -2

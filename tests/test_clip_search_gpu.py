@@ -133,10 +133,10 @@ def test_quantizer_entry_points_take_the_search_branch(dev):
     meta = MXFPMeta(block_size=32, scale_exp_bits=8, element_exp_bits=2, element_frac_bits=1, element_is_finite=True,
                     round_mode="rn")
     assert_bits_equal(mxfp_quantizer_sim(big.to(dev), -1, meta, quantile_search=True), got, "sim entry point")
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(ValueError):   # calibration activations must be [batches, tokens, block size]
         mxint_quantizer_sim(xd, -1, MXIntMeta(block_size=32, scale_bits=8, element_bits=4), act_tensor=xd, quantile_search=True)
     with pytest.raises(NotImplementedError):
-        mxint_quantizer(xd, 16, 4, quantile_search=True)
+        mxint_quantizer(xd, 8, 4, quantile_search=True)
     # a view that does not start on a 16-byte boundary
     base = torch.randn(4 * 64 + 3, generator=torch.Generator().manual_seed(8)).to(torch.bfloat16)
     view = base[3:].view(4, 64)
@@ -186,3 +186,78 @@ def test_clip_search_on_a_weight_sized_tensor(dev):
     xf = x.float() * 1000
     got, choice = _ops.mxfp_clip_search(xf.to(dev), 32, 2, 1, -1, 8, return_choice=True)
     check_against_oracle(got.cpu(), choice, O.mxfp_clip_search(xf, 32, 2, 1), torch.float32, "mxfp4 f32 [1024,4096]", 0.9995)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B", [16, 64])
+def test_clip_search_block_sizes_16_and_64(dev, dtype, B):
+    """the search for the other block sizes the MX formats use: same checks as for 32"""
+    from mase_amd.quantizers import _ops
+
+    x = search_inputs(B, dtype, rows=48)
+    got, choice = _ops.mxint_clip_search(x.to(dev), B, 4, -1, 8, return_choice=True)
+    check_against_oracle(got.cpu(), choice, O.mxint_clip_search(x, B, 4), dtype, f"mxint4 B={B} {dtype}", 0.995)
+    xf = search_inputs(B + 1, dtype, rows=48, scale=10.0 * 2.0 ** 2)
+    got, choice = _ops.mxfp_clip_search(xf.to(dev), B, 2, 1, -1, 8, return_choice=True)
+    check_against_oracle(got.cpu(), choice, O.mxfp_clip_search(xf, B, 2, 1), dtype, f"mxfp4 B={B} {dtype}", 0.995)
+
+
+def _calibration_case(seed, rows, B, dtype, batches=5, tokens=24):
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(rows, B, generator=g) * 0.05
+    w[::5] *= torch.exp2(torch.randint(-3, 4, (B,), generator=g).float())
+    w[3, 0] *= 40                      # an outlier: clipping it pays when the activations of that column are small
+    act = torch.randn(batches, tokens, B, generator=g)
+    act[..., 0] *= 0.05
+    act[..., 1::7] *= 4
+    return w.to(dtype), act.to(dtype)
+
+
+def _check_calibrated(got, choice, ref, dtype, what, min_agree):
+    """the tensor written is the oracle's candidate of the reported index, bit for bit; the index is the oracle's except
+    where the two errors (norms of matrix products, whose summation order differs between the library's CPU and GPU
+    kernels) agree to within a few steps of the dtype"""
+    want, pick, err, cand = ref
+    nb = cand.shape[1]
+    choice = choice.cpu().long()
+    mine = cand[choice, torch.arange(nb)]
+    assert_bits_equal(got.cpu().reshape(mine.shape), mine.to(dtype), f"{what}: contents for the reported index")
+    agree = choice == pick
+    rate = float(agree.double().mean())
+    print(f"{what}: same candidate as the oracle in {rate:.4f} of {nb} rows; histogram {torch.bincount(pick, minlength=11).tolist()}")
+    assert rate >= min_agree, what
+    if not bool(agree.all()) and err.dim() == 2:
+        idx = (~agree).nonzero().flatten()
+        e_mine, e_ref = err[choice[idx], idx].double(), err[pick[idx], idx].double()
+        assert bool(((e_mine - e_ref).abs() <= e_ref.abs() * ULP[dtype] * 16).all()), what
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B", [32, 16, 64])
+def test_clip_search_scored_on_calibration_outputs(dev, dtype, B):
+    """quantile_search=True with act_tensor (mxint.py:99-131, mxfp.py:65-93) through the quantizer entry points, several
+    calibration batches (cali_batch_size smaller than the number of samples)"""
+    from mase_amd.quantizers import MXFPMeta, MXIntMeta, _ops, mxfp_quantizer_sim, mxint_quantizer_sim
+
+    w, act = _calibration_case(B, 96, B, dtype)
+    got, choice = _ops.mxint_clip_search_calibrated(w.to(dev), B, 4, 1, 8, act.to(dev), 2, return_choice=True)
+    ref = O.mxint_clip_search(w, B, 4, 1, act_tensor=act, cali_batch_size=2)
+    _check_calibrated(got, choice, ref, dtype, f"mxint4 calibrated B={B} {dtype}", 0.9 if dtype == torch.bfloat16 else 0.97)
+    assert int((ref[1] != 0).sum()) > 5       # the calibration data does move choices away from the plain maximum
+    plain = O.mxint_clip_search(w, B, 4, 1)
+    assert not torch.equal(plain[1], ref[1])  # and away from the search scored on the weights alone
+    sim = mxint_quantizer_sim(w.to(dev), 1, MXIntMeta(block_size=B, scale_bits=8, element_bits=4), act_tensor=act.to(dev),
+                              quantile_search=True, cali_batch_size=2)
+    assert torch.equal(sim, got)
+    wf = (w.float() * 500).to(dtype)
+    got, choice = _ops.mxfp_clip_search_calibrated(wf.to(dev), B, 2, 1, 1, 8, act.to(dev), 2, return_choice=True)
+    ref = O.mxfp_clip_search(wf, B, 2, 1, 1, act_tensor=act, cali_batch_size=2)
+    # the strict-replace rule compares each percentile's error with the running best: agreement of the final pick
+    want, pick = ref[0], ref[1]
+    ch = choice.cpu().long()
+    assert_bits_equal(got.cpu().reshape(-1, B), ref[3][ch, torch.arange(ch.numel())].to(dtype), "mxfp calibrated contents")
+    rate = float((ch == pick).double().mean())
+    print(f"mxfp4 calibrated B={B} {dtype}: same candidate in {rate:.4f}")
+    assert rate >= (0.85 if dtype == torch.bfloat16 else 0.95)
+    meta = MXFPMeta(block_size=B, scale_exp_bits=8, element_exp_bits=2, element_frac_bits=1, element_is_finite=True, round_mode="rn")
+    assert torch.equal(mxfp_quantizer_sim(wf.to(dev), 1, meta, act_tensor=act.to(dev), quantile_search=True, cali_batch_size=2), got)

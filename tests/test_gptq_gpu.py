@@ -65,8 +65,16 @@ def test_gptq_without_search_and_with_a_dead_column(dev):
     want = G.fasterquant(lin.weight.data.cpu(), H, "mxint", {"weight_block_size": 32, "weight_width": 8}, quant_search=False)
     assert bool((q[:, 7] == 0).all())
     assert float((q == want).float().mean()) > 0.97
-    with pytest.raises(NotImplementedError):
-        GPTQ(lin).fasterquant(torch.zeros(1, 1, 128, device=dev), "mxint", MXINT4)
+    # clip_search_y: the search of every column group scored on the layer's calibration inputs
+    gp = GPTQ(lin)
+    for x in xs:
+        gp.add_batch(x.to(dev))
+    act = torch.stack([x.reshape(-1, x.shape[-1]) for x in xs])
+    q_y = gp.fasterquant(act.to(dev), "mxint", MXINT4, cali_batch_size=2).cpu()
+    want_y = G.fasterquant(lin.weight.data.cpu(), H, "mxint", MXINT4, activation=act, cali_batch_size=2)
+    assert float((q_y[:, :32] == want_y[:, :32]).float().mean()) > 0.97   # the first column group sees identical inputs
+    assert float((q_y == want_y).float().mean()) > 0.9
+    assert G.proxy_loss(lin.weight.data.cpu(), q_y, H) < 1.1 * G.proxy_loss(lin.weight.data.cpu(), want_y, H)
 
 
 def test_run_gptq_on_a_small_causal_lm(dev):
@@ -121,5 +129,7 @@ def test_run_gptq_on_a_small_causal_lm(dev):
     assert torch.equal(swapped.model.layers[1].mlp.down_proj.weight, want)
     with pytest.raises(NotImplementedError):
         run_gptq(copy.deepcopy(base), {**gcfg, "calibration_data": None})
-    with pytest.raises(NotImplementedError):
-        run_gptq(copy.deepcopy(base), {**gcfg, "clip_search_y": True})
+    tuned_y = run_gptq(copy.deepcopy(base), {**gcfg, "clip_search_y": True, "cali_batch_size": 4})
+    e_y = float((hidden(tuned_y) - ref).pow(2).mean())
+    print(f"hidden-state MSE with clip_search_y: {e_y:.4e}")
+    assert e_y < e_plain

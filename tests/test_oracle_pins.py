@@ -585,6 +585,59 @@ def test_mxfp_clip_search_score_is_on_the_integer_codes():
 # ------------------------------------------------------------------------------------------------
 # GPTQ
 # ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("fmt", ["mxint", "mxfp"])
+def test_clip_search_scored_on_calibration_outputs_is_the_gram_matrix_form(fmt):
+    """quantile_search with act_tensor: the error of candidate p for weight row h is the sum over calibration batches of
+    sqrt(d^T G d), d = candidate - row (for MXFP: the scored values - row), G = the batch's Gram matrix of activations.
+    Evaluated in float64 from that formula, independently of the oracle's matmul / einsum / norm calls; the oracle's
+    pick must be the formula's minimum (first minimum for MXINT, strict replacement in percentile order for MXFP),
+    except where the two best errors agree to within float32 rounding."""
+    g = torch.Generator().manual_seed(31)
+    B, rows = 32, 64
+    w = torch.randn(rows, B, generator=g) * (0.05 if fmt == "mxint" else 30.0)
+    w[3, 0] *= 40
+    act = torch.randn(5, 24, B, generator=g)
+    act[..., 0] *= 0.05
+    bsz = 2
+    if fmt == "mxint":
+        out, pick, err, cand = O.mxint_clip_search(w, B, 4, 1, act_tensor=act, cali_batch_size=bsz)
+        scored = cand.double()
+    else:
+        out, pick, err, cand = O.mxfp_clip_search(w, B, 2, 1, 1, act_tensor=act, cali_batch_size=bsz)
+        # the scored values: integer codes times the uint8 power (recomputed here from the components)
+        flat = w.reshape(-1)
+        scored = []
+        for pct in O.CLIP_PERCENTILES:
+            sc, el = O.mxfp_components(flat, B, 2, 1, 8, True, "rn", pct)
+            e = sc.to(torch.int64) - 127
+            unit = torch.where((e >= 0) & (e <= 7), torch.exp2(e.double()), torch.zeros_like(e, dtype=torch.float64))
+            scored.append(el.double() / 2 ** (1 - 1) * unit)
+        scored = torch.stack(scored)
+    exact = torch.zeros(11, rows, dtype=torch.float64)
+    for b in range(0, act.shape[0], bsz):
+        a = act[b:b + bsz].double().reshape(-1, B)
+        G = a.T @ a
+        d = scored - w.double()[None]
+        exact += torch.sqrt(torch.einsum("phb,bc,phc->ph", d, G, d).clamp_min(0))
+    if fmt == "mxint":
+        want = exact.argmin(0)
+    else:
+        want = torch.zeros(rows, dtype=torch.int64)
+        best = torch.full((rows,), float("inf"), dtype=torch.float64)
+        for p in range(11):
+            better = exact[p] < best
+            best = torch.where(better, exact[p], best)
+            want = torch.where(better, torch.full_like(want, p), want)
+    differ = (want != pick).nonzero().flatten()
+    for h in differ.tolist():
+        a, b = float(exact[want[h], h]), float(exact[pick[h], h])
+        assert abs(a - b) <= 1e-5 * max(abs(a), 1e-30), (fmt, h, int(want[h]), int(pick[h]), a, b)
+    assert differ.numel() <= rows // 8
+    assert int((pick != 0).sum()) > 3
+    chosen = cand[pick, torch.arange(rows)]
+    assert torch.equal(out, chosen.reshape(out.shape).to(out.dtype))
+
+
 def _correlated_inputs(g, n, tokens, cols):
     mix = torch.randn(cols, cols, generator=g) * 0.3 + torch.eye(cols)
     return [torch.randn(2, tokens, cols, generator=g) @ mix for _ in range(n)]
