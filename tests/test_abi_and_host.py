@@ -229,8 +229,9 @@ def test_product_has_no_cpu_path():
                  lambda: Q.mxfp_quantizer(x, 32, 4, 3, quantile_search=True)):
         with pytest.raises(MaseAmdError):
             call()
-    with pytest.raises(NotImplementedError):  # the calibrated (GPTQ) search is not part of the path
-        Q.mxint_quantizer_sim(x, -1, Q.MXIntMeta(block_size=32, scale_bits=8, element_bits=8), act_tensor=x, quantile_search=True)
+    with pytest.raises(MaseAmdError):  # the search scored on calibration outputs runs on the device as well
+        Q.mxint_quantizer_sim(x, -1, Q.MXIntMeta(block_size=32, scale_bits=8, element_bits=8),
+                              act_tensor=x.reshape(1, 4, 32), quantile_search=True)
 
 
 def test_product_does_not_import_the_oracle():
