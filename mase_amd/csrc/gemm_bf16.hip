@@ -367,8 +367,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // cache).  One counter covers both, so "at most n outstanding" proves that an A copy has landed only if at least
   // n + 1 younger *A copies* would otherwise have to be pending with it.  Hence three stages of A: the 8 copies of the
   // K tile after next are issued *before* the hand-over that needs the next K tile, and that hand-over waits for
-  // "at most 8 outstanding": the next K tile has landed (its copies are older than those 8), and so have the B loads
-  // unless fewer than 8 of the young copies are still in flight; the young copies themselves fly on across the barrier.
+  // "at most 8 outstanding": the next K tile has landed (its copies are older than those 8); the young copies
+  // themselves fly on across the barrier.  The B fragments are proven the same way, by counting the register loads
+  // issued after them (see the waits at the head of each step).
   //   step 0: MFMAs on fr[0]; LDS reads of step 1; the 16 B loads of the next K tile (their registers were last read
   //           one K tile ago)
   //   step 1: MFMAs on fr[1]; LDS reads of steps 2 and 3; the 8 A copies of the K tile after next into the stage
@@ -382,6 +383,13 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     const int stage_next = next_of(stage);
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
+      // the B fragments of this step (register loads 4s+1 .. 4s+4 of the 16 issued one K tile ago) have landed once
+      // at most as many loads are outstanding as *register loads* were issued after them: the other 12 - 4s of their
+      // batch, plus, from step 1 on, the 16 of the next batch issued during step 0.  (Step 3 is covered by the
+      // hand-over's wait.)
+      if (s == 0) wait_vmcnt<12>();
+      else if (s == 1) wait_vmcnt<24>();
+      else if (s == 2) wait_vmcnt<20>();
 #pragma unroll
       for (int t = 0; t < 16; ++t) {
         acc[t >> 2][t & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[s][t >> 2], fb[NB][s][t & 3],

@@ -20,6 +20,9 @@
 #ifndef MASE_RUN_THREADS
 #define MASE_RUN_THREADS 64
 #endif
+#ifndef MASE_MXINT_NARROW_ITEMS
+#define MASE_MXINT_NARROW_ITEMS 1
+#endif
 
 namespace mase {
 namespace {
@@ -61,69 +64,82 @@ __device__ __forceinline__ void store_vec(void* out, size_t idx, const float* y,
   }
 }
 
-template <int DT, int DTO, int LPB, int SUB, int T>
+// ITEMS vectors per lane, a work-group's width apart, all loaded before the first is worked on: a wavefront then has
+// ITEMS KB in flight instead of one, which is what a latency-bound stream needs when the stores are narrower than the
+// loads (fp32 in, 16-bit out).
+template <int DT, int DTO, int LPB, int SUB, int T, int ITEMS>
 __global__ __launch_bounds__(T) void mxint_qdq_vec_kernel(const uint4* __restrict__ in, void* __restrict__ out,
                                                           int8_t* __restrict__ codes, uint8_t* __restrict__ scales,
                                                           size_t n_vec, MxintParams p) {
   using TR = DTypeTraits<DT>;
   constexpr int V = TR::kVec;
   constexpr int EPS = V / SUB;  // elements per sub-block held by this lane
-  const size_t idx = (size_t)blockIdx.x * T + threadIdx.x;
-  const bool live = idx < n_vec;  // whole blocks are live or dead together: n_vec is a multiple of LPB
-  const uint4 raw = live ? load_nt(in + idx) : make_uint4(0, 0, 0, 0);
+  const size_t idx0 = (size_t)blockIdx.x * (T * ITEMS) + threadIdx.x;
+  uint4 raws[ITEMS];
+#pragma unroll
+  for (int u = 0; u < ITEMS; ++u) {
+    const size_t i = idx0 + (size_t)u * T;
+    raws[u] = i < n_vec ? load_nt(in + i) : make_uint4(0, 0, 0, 0);
+  }
   WaveLog2 meta;
   meta.init(p.tab, 0);
-  float x[V], y[V];
-  int c[V];
-  TR::unpack(raw, x);
-  bool exact_bf16 = (DT == MASE_DT_BF16);  // 8-bit-significand inputs: results need no rounding to bf16
 #pragma unroll
-  for (int s = 0; s < SUB; ++s) {
-    uint32_t m;
-    if constexpr (SUB == 1) {
-      m = group_max_u32<LPB>(vec_absmax_bits<DT>(raw));
-    } else {
-      m = 0;
+  for (int u = 0; u < ITEMS; ++u) {
+    const size_t idx = idx0 + (size_t)u * T;
+    const bool live = idx < n_vec;  // whole blocks are live or dead together: n_vec is a multiple of LPB
+    const uint4 raw = raws[u];
+    float x[V], y[V];
+    int c[V];
+    TR::unpack(raw, x);
+    bool exact_bf16 = (DT == MASE_DT_BF16);  // 8-bit-significand inputs: results need no rounding to bf16
 #pragma unroll
-      for (int j = 0; j < EPS; ++j) m = max(m, f2bits(x[s * EPS + j]) & 0x7FFFFFFFu);
-    }
-    int k = 0, kc = 0;
-    const int state = block_exponent<DT>(m, p, k, kc, meta);
-    if (state == 0) {
-      const int up = p.qshift - k, dn = kc - p.qshift;
-      exact_bf16 = exact_bf16 && (dn >= -126);
-#pragma unroll
-      for (int j = 0; j < EPS; ++j) {
-        float r = fminf(fmaxf(rintf(ldexpf(x[s * EPS + j], up)), p.lo), p.hi);
-        c[s * EPS + j] = (int)r;
-        y[s * EPS + j] = ldexpf(r, dn);
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < EPS; ++j) y[s * EPS + j] = mxint_element<DT>(x[s * EPS + j], state, k, kc, p, c[s * EPS + j]);
-    }
-    if (codes != nullptr && live) {
-      int sb = (state == 0) ? min(max(kc - p.qshift + 134, 0), 255) : 255;
-      if constexpr (LPB > 1) {
-        if ((idx & (LPB - 1)) == 0) scales[idx / LPB] = (uint8_t)sb;
+    for (int s = 0; s < SUB; ++s) {
+      uint32_t m;
+      if constexpr (SUB == 1) {
+        m = group_max_u32<LPB>(vec_absmax_bits<DT>(raw));
       } else {
-        scales[idx * SUB + s] = (uint8_t)sb;
+        m = 0;
+#pragma unroll
+        for (int j = 0; j < EPS; ++j) m = max(m, f2bits(x[s * EPS + j]) & 0x7FFFFFFFu);
+      }
+      int k = 0, kc = 0;
+      const int state = block_exponent<DT>(m, p, k, kc, meta);
+      if (state == 0) {
+        const int up = p.qshift - k, dn = kc - p.qshift;
+        exact_bf16 = exact_bf16 && (dn >= -126);
+#pragma unroll
+        for (int j = 0; j < EPS; ++j) {
+          float r = fminf(fmaxf(rintf(ldexpf(x[s * EPS + j], up)), p.lo), p.hi);
+          c[s * EPS + j] = (int)r;
+          y[s * EPS + j] = ldexpf(r, dn);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < EPS; ++j) y[s * EPS + j] = mxint_element<DT>(x[s * EPS + j], state, k, kc, p, c[s * EPS + j]);
+      }
+      if (codes != nullptr && live) {
+        int sb = (state == 0) ? min(max(kc - p.qshift + 134, 0), 255) : 255;
+        if constexpr (LPB > 1) {
+          if ((idx & (LPB - 1)) == 0) scales[idx / LPB] = (uint8_t)sb;
+        } else {
+          scales[idx * SUB + s] = (uint8_t)sb;
+        }
       }
     }
-  }
-  if (!live) return;
-  store_vec<DTO, V>(out, idx, y, exact_bf16);
-  if (codes != nullptr) {
-    if constexpr (V == 4) {
-      ((uint32_t*)codes)[idx] = (uint32_t)(c[0] & 0xFF) | ((uint32_t)(c[1] & 0xFF) << 8) | ((uint32_t)(c[2] & 0xFF) << 16) |
-                                ((uint32_t)(c[3] & 0xFF) << 24);
-    } else {
-      uint2 w;
-      w.x = (uint32_t)(c[0] & 0xFF) | ((uint32_t)(c[1] & 0xFF) << 8) | ((uint32_t)(c[2] & 0xFF) << 16) |
-            ((uint32_t)(c[3] & 0xFF) << 24);
-      w.y = (uint32_t)(c[4] & 0xFF) | ((uint32_t)(c[5] & 0xFF) << 8) | ((uint32_t)(c[6] & 0xFF) << 16) |
-            ((uint32_t)(c[7] & 0xFF) << 24);
-      ((uint2*)codes)[idx] = w;
+    if (!live) continue;
+    store_vec<DTO, V>(out, idx, y, exact_bf16);
+    if (codes != nullptr) {
+      if constexpr (V == 4) {
+        ((uint32_t*)codes)[idx] = (uint32_t)(c[0] & 0xFF) | ((uint32_t)(c[1] & 0xFF) << 8) | ((uint32_t)(c[2] & 0xFF) << 16) |
+                                  ((uint32_t)(c[3] & 0xFF) << 24);
+      } else {
+        uint2 w;
+        w.x = (uint32_t)(c[0] & 0xFF) | ((uint32_t)(c[1] & 0xFF) << 8) | ((uint32_t)(c[2] & 0xFF) << 16) |
+              ((uint32_t)(c[3] & 0xFF) << 24);
+        w.y = (uint32_t)(c[4] & 0xFF) | ((uint32_t)(c[5] & 0xFF) << 8) | ((uint32_t)(c[6] & 0xFF) << 16) |
+              ((uint32_t)(c[7] & 0xFF) << 24);
+        ((uint2*)codes)[idx] = w;
+      }
     }
   }
 }
@@ -160,10 +176,12 @@ int launch_mxint(const void* in, void* out, int8_t* codes, uint8_t* scales, size
                       (codes == nullptr || (((uintptr_t)codes) & 7u) == 0);
   if (vec_ok) {
     size_t n_vec = numel / V;
-    dim3 grid(blocks_for(n_vec, kRunThreads)), block(kRunThreads);
+    // more than one vector per lane was measured slower for every dtype pair of this kernel (fp32 -> bf16 on 4096^2: 17.6, 18.5, 19.6 us with 1, 2, 4)
+    constexpr int kItems = (DT == MASE_DT_F32 && DTO != MASE_DT_F32) ? MASE_MXINT_NARROW_ITEMS : 1;
+    dim3 grid(blocks_for(n_vec, (size_t)kRunThreads * kItems)), block(kRunThreads);
 #define MASE_MXINT_CASE(LPB_, SUB_)                                                                               \
-  hipLaunchKernelGGL((mxint_qdq_vec_kernel<DT, DTO, LPB_, SUB_, kRunThreads>), grid, block, 0, st, (const uint4*)in, \
-                     out, codes, scales, n_vec, p)
+  hipLaunchKernelGGL((mxint_qdq_vec_kernel<DT, DTO, LPB_, SUB_, kRunThreads, kItems>), grid, block, 0, st,         \
+                     (const uint4*)in, out, codes, scales, n_vec, p)
     if (B >= V) {
       switch (B / V) {
         case 1: MASE_MXINT_CASE(1, 1); break;
