@@ -33,6 +33,7 @@
  *   mase_gemm_mxint8_skinny nn/quantized/modules/linear.py:972 for at most 128 rows, weights as int8 codes + scales
  *   mase_gemm_bf16_skinny   same call sites as mase_gemm_bf16_tn, for at most 128 rows of activations
  *   mase_gemm_bf16_tn_packed, mase_gemm_bf16_pack_b   the same F.linear with the weight in fragment order
+ *   mase_gemm_mxint8_tn_packed, mase_gemm_mxint8_pack_b   the same with the weight as MXINT8 codes in fragment order
  *   mase_gemm_bf16_tn       nn/quantized/modules/linear.py:972 and :895 (the F.linear of LinearMXInt.forward /
  *                           LinearMXFP.forward on the quantize-dequantized operands)
  */
@@ -194,6 +195,22 @@ size_t mase_gemm_bf16_packed_bytes(size_t N, size_t K);
 int mase_gemm_bf16_pack_b(const void* B, void* B_packed, size_t N, size_t K, void* stream);
 int mase_gemm_bf16_tn_packed(const void* A, const void* B_packed, const void* bias, void* C, size_t M, size_t N,
                              size_t K, int out_dtype, int bias_dtype, void* stream);
+
+/* The tiled product with B held as an MXINT8 weight in fragment order: the code image and the scale image written by
+ * mase_gemm_mxint8_pack_b from int8 codes [N, K] and scale bytes [N, K/32] (value = code * 2^(scale - 134): the packed
+ * outputs of mase_mxint_qdq with element_bits 8, block 32).  1.03 bytes per weight in memory and on the way in; the
+ * codes are widened to the same bf16 values in registers, so the result is that of mase_gemm_bf16_tn on the dequantized
+ * weight (the same products added in the same order) as long as every scale byte is at least 8 (weights of 2^-119 and
+ * less are taken as zero).  K % 128 == 0; images 16-byte / 2-byte aligned, the code image below 4 GiB.
+ * _code_bytes / _scale_bytes: sizes of the two images (0 when K % 128 != 0).  Replaces the F.linear of
+ * LinearMXInt.forward (nn/quantized/modules/linear.py:972) with the weight dequantized on the way into the matrix
+ * instruction instead of beforehand. */
+size_t mase_gemm_mxint8_packed_code_bytes(size_t N, size_t K);
+size_t mase_gemm_mxint8_packed_scale_bytes(size_t N, size_t K);
+int mase_gemm_mxint8_pack_b(const int8_t* codes, const uint8_t* scales, void* code_image, void* scale_image, size_t N,
+                            size_t K, void* stream);
+int mase_gemm_mxint8_tn_packed(const void* A, const void* code_image, const void* scale_image, const void* bias, void* C,
+                               size_t M, size_t N, size_t K, int out_dtype, int bias_dtype, void* stream);
 
 /* The same product for few rows of A (M <= 128, the token-by-token shape of serving): bound by streaming B once
  * from HBM.  The work is split over N and over K ranges; the partial results of the K ranges go through

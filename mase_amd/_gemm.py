@@ -95,6 +95,51 @@ def gemm_bf16_tn(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dty
     return out
 
 
+def gemm_mxint8_packed_supported(N: int, K: int) -> bool:
+    return K % PACKED_B_K_MULTIPLE == 0 and (N + 31) // 32 * 32 * K <= OPERAND_BYTES_LIMIT
+
+
+def gemm_mxint8_pack_b(codes: Tensor, scales: Tensor):
+    """fragment-ordered code and scale images of an MXINT8 weight (int8 codes [N,K], uint8 scales [N,K/32]) for
+    ``gemm_mxint8_tn_packed``: ``mase_gemm_mxint8_pack_b``"""
+    _lib.require_device(codes, "gemm_mxint8_pack_b")
+    lib = _lib.load()
+    assert codes.dtype == torch.int8 and scales.dtype == torch.uint8 and codes.dim() == 2
+    codes, scales = codes.contiguous(), scales.contiguous()
+    N, K = codes.shape
+    assert scales.shape == (N, K // 32) and gemm_mxint8_packed_supported(N, K)
+    img = torch.empty(lib.mase_gemm_mxint8_packed_code_bytes(N, K), dtype=torch.uint8, device=codes.device)
+    simg = torch.empty(lib.mase_gemm_mxint8_packed_scale_bytes(N, K), dtype=torch.uint8, device=codes.device)
+    _lib.check(lib.mase_gemm_mxint8_pack_b(codes.data_ptr(), scales.data_ptr(), img.data_ptr(), simg.data_ptr(), N, K,
+                                           _lib.stream_ptr(codes)), "mase_gemm_mxint8_pack_b")
+    return img, simg
+
+
+def gemm_mxint8_tn_packed(a: Tensor, code_image: Tensor, scale_image: Tensor, N: int, bias: Tensor | None,
+                          out_dtype: torch.dtype) -> Tensor:
+    """``a[M,K] @ dequant(weight)[N,K].T + bias`` on the tiled kernel with the weight as MXINT8 code / scale images
+    (``gemm_mxint8_pack_b``); bf16 activations, fp32 accumulation; the same values as ``gemm_bf16_tn`` on the
+    dequantized weight."""
+    _lib.require_device(a, "gemm_mxint8_tn_packed")
+    lib = _lib.load()
+    assert a.dtype == torch.bfloat16 and a.dim() == 2
+    a = a.contiguous()
+    M, K = a.shape
+    assert gemm_mxint8_packed_supported(N, K) and code_image.numel() == lib.mase_gemm_mxint8_packed_code_bytes(N, K)
+    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    if bias is not None:
+        bias = bias.contiguous()
+    rows_per_call = max(1, min(M, (OPERAND_BYTES_LIMIT // (2 * K)) // 256 * 256 or 1))
+    for r0 in range(0, M, rows_per_call):
+        r1 = min(M, r0 + rows_per_call)
+        rc = lib.mase_gemm_mxint8_tn_packed(
+            a[r0:r1].data_ptr(), code_image.data_ptr(), scale_image.data_ptr(), bias.data_ptr() if bias is not None else None,
+            out[r0:r1].data_ptr(), r1 - r0, N, K, _lib.DTYPE_CODE[out_dtype],
+            _lib.DTYPE_CODE[bias.dtype] if bias is not None else 0, _lib.stream_ptr(a))
+        _lib.check(rc, "mase_gemm_mxint8_tn_packed")
+    return out
+
+
 MXINT8_SKINNY_K_MULTIPLE = 128
 
 

@@ -50,6 +50,7 @@ constexpr int kLdsBytes = S * kStageBytes + 4 * kStgWave;
 struct GemmParams {
   const unsigned char* A;
   const unsigned char* B;
+  const unsigned char* Bs;  // BCODES: the scale image that goes with the code image in B
   const void* bias;
   void* C;
   int M, N, K;
@@ -95,6 +96,25 @@ __device__ __forceinline__ void load_16_untracked(bf16x8_t& dst, uint32_t off, c
   asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst) : "v"(off), "s"(base) : "memory");
 }
 
+// One wavefront-wide 512-byte / 128-byte load (8 / 2 bytes per lane) outside the compiler's tracking, as above.
+__device__ __forceinline__ void load_8_untracked(uint2& dst, uint32_t off, const unsigned char* base) {
+  asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(dst) : "v"(off), "s"(base) : "memory");
+}
+__device__ __forceinline__ void load_2_untracked(uint32_t& dst, uint32_t off, const unsigned char* base) {
+  asm volatile("global_load_ushort %0, %1, %2" : "=v"(dst) : "v"(off), "s"(base) : "memory");
+}
+
+// four codes (already offset by 128: unsigned bytes) -> two registers of two bf16 values each: (u - 128) * scale,
+// exact in fp32, at most 8 significant bits, so the upper halves are the values
+__device__ __forceinline__ void ucodes4_to_bf16(uint32_t u, float scale, float bias, uint32_t& lo, uint32_t& hi) {
+  const float f0 = __builtin_fmaf((float)(u & 0xFFu), scale, bias);
+  const float f1 = __builtin_fmaf((float)((u >> 8) & 0xFFu), scale, bias);
+  const float f2 = __builtin_fmaf((float)((u >> 16) & 0xFFu), scale, bias);
+  const float f3 = __builtin_fmaf((float)(u >> 24), scale, bias);
+  lo = __builtin_amdgcn_perm(f2bits(f1), f2bits(f0), 0x07060302u);
+  hi = __builtin_amdgcn_perm(f2bits(f3), f2bits(f2), 0x07060302u);
+}
+
 // STREAM: K holds at least S tiles, so the copy stream is never more than one output tile ahead and advances
 // without branches; the other instantiation (K = one tile) advances it with the general, branching step.
 // BPACK (with STREAM, an even number of K tiles): B is the fragment-ordered image of mase_gemm_bf16_pack_b and its
@@ -102,8 +122,13 @@ __device__ __forceinline__ void load_16_untracked(bf16x8_t& dst, uint32_t off, c
 // LDS, in three stages of 32 KB.  That halves the LDS traffic (the copies landing in LDS while the wavefronts read
 // their fragments is what holds the plain kernel back) at the price of every B fragment being fetched by the two
 // wavefronts that share it.
-template <int OUT_DT, bool STREAM, bool BPACK = false>
+// BCODES (with BPACK): B is an MXINT8 weight as codes + scale bytes in fragment order (mase_gemm_mxint8_pack_b): half
+// the bytes of the bf16 image in memory and on the way in; the codes are widened to the same bf16 operand values in
+// registers, one K step ahead of the MFMAs that use them (code + 128 as an unsigned byte -> v_cvt_f32_ubyte -> one fma
+// that removes the 128 and applies the block's power-of-two scale -> the upper half of the exact fp32 product).
+template <int OUT_DT, bool STREAM, bool BPACK = false, bool BCODES = false>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p) {
+  static_assert(!BCODES || BPACK, "codes come in fragment order");
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int tid = threadIdx.x;
   const int lane_id = tid & 63;
@@ -331,7 +356,14 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   bf16x8_t fr[4][BPACK ? 4 : 8];
   // BPACK: B fragments of two K tiles (the one in use and the one being loaded): [buffer][K step][column tile].
   // Image layout: 1 KB blocks [column tile of 32][K step of 16][lane][8 bf16], lane l = column l % 32, K 8*(l/32)..+8.
-  bf16x8_t fb[BPACK ? 2 : 1][4][4];
+  bf16x8_t fb[(BPACK && !BCODES) ? 2 : 1][(BPACK && !BCODES) ? 4 : 1][4];
+  // BCODES: the codes of two K tiles [buffer][K step][column tile] (8 per lane), their scale bytes [buffer][column
+  // tile] (the two blocks of 32 a K tile holds, for the lane's column) and the widened fragments of two K steps
+  uint2 fbc[BCODES ? 2 : 1][BCODES ? 4 : 1][4];
+  uint32_t fsc[BCODES ? 2 : 1][4];
+  uint4 fbq[2][4];
+  uint32_t soff[4];          // BCODES: this lane's byte offset of K tile 0 of its four column tiles in the scale image
+  const unsigned char* s_kbase = p.Bs;
   uint32_t boff[4];          // this lane's byte offset of K step 0 of its four column tiles
   const unsigned char* b_kbase = p.B;  // image address of K tile 0 of the K range of the output tile being loaded
   int b_kt = 0;              // K tile (within the range) whose fragments the current iteration loads
@@ -341,13 +373,42 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     int lane = lane_id;
     asm volatile("" : "+v"(lane));
     const int nt_last = (p.N + 31) / 32 - 1;
+    constexpr uint32_t kFragBytes = BCODES ? 512u : 1024u;  // one fragment of a wavefront: 8 codes or 8 bf16 per lane
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      boff[j] = (uint32_t)((size_t)min((n0 + wn * 128) / 32 + j, nt_last) * (size_t)(p.K / 16) * 1024u) + (uint32_t)lane * 16u;
-    b_kbase = p.B + (size_t)ks * (size_t)(p.kc / 16) * 1024u;
+    for (int j = 0; j < 4; ++j) {
+      const size_t ct = (size_t)min((n0 + wn * 128) / 32 + j, nt_last);
+      boff[j] = (uint32_t)(ct * (size_t)(p.K / 16) * kFragBytes) + (uint32_t)lane * (kFragBytes / 64u);
+      if constexpr (BCODES) soff[j] = (uint32_t)(ct * (size_t)(p.K / 64) * 64u) + (uint32_t)(lane & 31) * 2u;
+    }
+    b_kbase = p.B + (size_t)ks * (size_t)(p.kc / 16) * kFragBytes;
+    if constexpr (BCODES) s_kbase = p.Bs + (size_t)ks * (size_t)(p.kc / 64) * 64u;
     b_kt = 0;
   };
-  if constexpr (BPACK) {
+  // BCODES: widening of the fragment of column tile j, K step st of the K tile in code buffer `buf` into fragment set
+  // `set`; `half` 0 / 1 = the first / second four codes.  The scale byte of a step is byte st / 2 of the lane's two.
+  auto widen = [&](int set, int buf, int st, int j, int half) __attribute__((always_inline)) {
+    const uint32_t sb = (fsc[buf][j] >> (8 * (st >> 1))) & 0xFFu;
+    const float scale = bits2f(sb >= 8u ? (sb - 7u) << 23 : 0u);  // 2^(sb - 134)
+    const float bias = -128.0f * scale;
+    uint32_t lo, hi;
+    ucodes4_to_bf16(half ? fbc[buf][st][j].y : fbc[buf][st][j].x, scale, bias, lo, hi);
+    if (half) { fbq[set][j].z = lo; fbq[set][j].w = hi; }
+    else { fbq[set][j].x = lo; fbq[set][j].y = hi; }
+  };
+  if constexpr (BCODES) {
+    set_b_tile(0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) load_2_untracked(fsc[0][j], soff[j], s_kbase);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) load_8_untracked(fbc[0][i >> 2][i & 3], boff[i & 3], b_kbase + (size_t)(i >> 2) * 512);
+    b_kt = 1;
+    wait_vmcnt<0>();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      widen(0, 0, 0, j, 0);
+      widen(0, 0, 0, j, 1);
+    }
+  } else if constexpr (BPACK) {
     set_b_tile(0);
 #pragma unroll
     for (int i = 0; i < 16; ++i) load_16_untracked(fb[0][i >> 2][i & 3], boff[i & 3], b_kbase + (size_t)(i >> 2) * 1024);
@@ -416,6 +477,55 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     stage = stage_next;
     ++b_kt;
   };
+  // BCODES form: as the BPACK form, with 4 scale loads and 16 code loads per K tile (in that order, step 0) and the
+  // widening of K step s + 1 (of step 0 of the next K tile during step 3) spread over the MFMA slots of step s, two
+  // slots per half fragment.  A step's codes must have landed one step earlier than in the BPACK form; counting the
+  // register loads issued after them: codes of step 1 (loads 9-12 of the 20): 8 at the head of the K tile; step 2:
+  // 4 + 20 at the head of step 1; step 3: 20 at the head of step 2; step 0 of the next K tile and the scales: covered
+  // by the hand-over's 8.
+  auto k_iteration_c = [&](auto&& advance, auto bufc) __attribute__((always_inline)) {
+    constexpr int NB = decltype(bufc)::value;
+    const unsigned char* bsrc = b_kbase + (size_t)b_kt * 2048;
+    const unsigned char* ssrc = s_kbase + (size_t)b_kt * 64;
+    const int stage_next = next_of(stage);
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) {
+      if (s == 0) wait_vmcnt<8>();
+      else if (s == 1) wait_vmcnt<24>();
+      else if (s == 2) wait_vmcnt<20>();
+#pragma unroll
+      for (int t = 0; t < 16; ++t) {
+        acc[t >> 2][t & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            fr[s][t >> 2], __builtin_bit_cast(bf16x8_t, fbq[s & 1][t & 3]), acc[t >> 2][t & 3], 0, 0, 0);
+        if ((t & 1) == 0) {  // half fragment (t >> 2, (t >> 1) & 1) of the next step
+          if (s < 3) widen((s + 1) & 1, NB, s + 1, t >> 2, (t >> 1) & 1);
+          else widen(0, NB ^ 1, 0, t >> 2, (t >> 1) & 1);
+        }
+        if (s == 0) {
+          if (t < 4) {
+            fr[1][t] = load_frag(stage, 1, t);
+            load_2_untracked(fsc[NB ^ 1][t], soff[t], ssrc);
+          }
+          load_8_untracked(fbc[NB ^ 1][t >> 2][t & 3], boff[t & 3], bsrc + (size_t)(t >> 2) * 512);
+        } else if (s == 1) {
+          if (t < 4) fr[2][t] = load_frag(stage, 2, t);
+          else if (t < 8) fr[3][t - 4] = load_frag(stage, 3, t - 4);
+          if (t & 1) issue_copy(t - 1);
+        } else if (s == 3) {
+          if (t < 4) fr[0][t] = load_frag(stage_next, 0, t);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (s == 2) {
+        wait_vmcnt<kWaveCopies>();
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    advance();
+    stage = stage_next;
+    ++b_kt;
+  };
   auto k_iteration = [&](auto&& advance) __attribute__((always_inline)) {
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
@@ -449,16 +559,20 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     if constexpr (BPACK) {
       // two K tiles per trip (the fragment buffers alternate); the copy stream as in the plain form below, the B
       // stream one K tile ahead: it moves on to the next output tile before the last K tile of this one
+      auto iter = [&](auto bufc) __attribute__((always_inline)) {
+        if constexpr (BCODES) k_iteration_c(step_within_tile, bufc);
+        else k_iteration_b(step_within_tile, bufc);
+      };
 #pragma unroll 1
       for (int kt = 0; kt < nk - S; kt += 2) {
-        k_iteration_b(step_within_tile, std::integral_constant<int, 0>{});
-        k_iteration_b(step_within_tile, std::integral_constant<int, 1>{});
+        iter(std::integral_constant<int, 0>{});
+        iter(std::integral_constant<int, 1>{});
       }
       set_copy_tile(ord + 1);
       c_kt = 0;
-      k_iteration_b(step_within_tile, std::integral_constant<int, 0>{});
+      iter(std::integral_constant<int, 0>{});
       set_b_tile(ord + 1);
-      k_iteration_b(step_within_tile, std::integral_constant<int, 1>{});
+      iter(std::integral_constant<int, 1>{});
     } else if constexpr (STREAM) {
       // the copy stream stands at K tile S of this output tile (or, if nk == S, at K tile 0 of the next)
 #pragma unroll 1
@@ -490,7 +604,7 @@ int persistent_grid_bf16(int total_tiles) {
 }
 
 // launch of the persistent kernel for the work items of p (tiles x K ranges), output dtype out_dtype
-int launch_gemm_bf16(const GemmParams& p, int out_dtype, hipStream_t st, bool bpack = false) {
+int launch_gemm_bf16(const GemmParams& p, int out_dtype, hipStream_t st, bool bpack = false, bool bcodes = false) {
   const size_t lds_bytes = (size_t)kLdsBytes;
   const int nwg = persistent_grid_bf16(p.tiles_m * p.tiles_n * p.splits);
   if (nwg <= 0) return MASE_ERR_LAUNCH;
@@ -507,7 +621,24 @@ int launch_gemm_bf16(const GemmParams& p, int out_dtype, hipStream_t st, bool bp
     }                                                                                                             \
     hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, STREAM_>), grid, block, lds_bytes, st, p);                       \
   } while (0)
-  if (bpack) {
+  if (bpack && bcodes) {
+    if (!stream_fits || ((p.kc / BK) & 1) != 0) return MASE_ERR_SHAPE;
+#define MASE_GEMM_LAUNCH_C(DT_)                                                                                   \
+  do {                                                                                                            \
+    static bool attr_set = false;                                                                                 \
+    const void* k = (const void*)gemm_bf16_tn_kernel<DT_, true, true, true>;                                      \
+    if (!attr_set) {                                                                                              \
+      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)       \
+        return MASE_ERR_LAUNCH;                                                                                   \
+      attr_set = true;                                                                                            \
+    }                                                                                                             \
+    hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, true, true, true>), grid, block, lds_bytes, st, p);              \
+  } while (0)
+    if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH_C(MASE_DT_F32);
+    else if (out_dtype == MASE_DT_BF16) MASE_GEMM_LAUNCH_C(MASE_DT_BF16);
+    else MASE_GEMM_LAUNCH_C(MASE_DT_F16);
+#undef MASE_GEMM_LAUNCH_C
+  } else if (bpack) {
     if (!stream_fits || ((p.kc / BK) & 1) != 0) return MASE_ERR_SHAPE;
 #define MASE_GEMM_LAUNCH_B(DT_)                                                                                   \
   do {                                                                                                            \
@@ -568,6 +699,39 @@ __global__ __launch_bounds__(256) void gemm_pack_b_kernel(const uint4* __restric
   out[g] = v;
 }
 
+// MXINT8 weight [N, K] (int8 codes, one scale byte per 32 along K) -> fragment-ordered images for the BCODES kernel:
+// codes: 512-byte blocks [column tile of 32][K step of 16][lane][8 bytes], lane l of a block holding the codes of
+// column tile*32 + l%32 at K = step*16 + 8*(l/32) .. +8, each plus 128 (an unsigned byte); columns beyond N hold 128
+// (zero).  scales: 64-byte blocks [column tile][K tile of 64][column][2 bytes] (the scale bytes of the K tile's two
+// blocks of 32).
+__global__ __launch_bounds__(256) void gemm_pack_codes_kernel(const uint2* __restrict__ codes, const uint8_t* __restrict__ scales,
+                                                              uint2* __restrict__ img, uint16_t* __restrict__ simg, int N,
+                                                              int K, size_t granules) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= granules) return;
+  const int lane = (int)(g & 63);
+  const size_t blk = g >> 6;
+  const int steps = K / 16;
+  const int nt = (int)(blk / (size_t)steps), ks = (int)(blk % (size_t)steps);
+  const int row = nt * 32 + (lane & 31);
+  uint2 v = make_uint2(0x80808080u, 0x80808080u);
+  if (row < N) {
+    v = codes[((size_t)row * K + (size_t)ks * 16 + 8 * (lane >> 5)) / 8];
+    v.x ^= 0x80808080u;
+    v.y ^= 0x80808080u;
+  }
+  img[g] = v;
+  if ((ks & 3) == 0 && lane < 32) {  // one lane per column writes the K tile's two scale bytes
+    const int kt = ks >> 2;
+    uint16_t sc = 0;
+    if (row < N) {
+      const uint8_t* sp = scales + (size_t)row * (K / 32) + (size_t)kt * 2;
+      sc = (uint16_t)sp[0] | ((uint16_t)sp[1] << 8);
+    }
+    simg[((size_t)nt * (K / 64) + kt) * 32 + lane] = sc;
+  }
+}
+
 // K ranges for a product whose output tiles alone would leave most CUs idle: as many as fill the machine once, each a
 // whole number of K tiles and at least 4 of them; 1 when the tiles already fill three quarters of the CUs
 int splitk_ranges(size_t M, size_t N, size_t K) {
@@ -598,6 +762,7 @@ extern "C" int mase_gemm_bf16_tn(const void* A, const void* B, const void* bias,
   GemmParams p;
   p.A = (const unsigned char*)A;
   p.B = (const unsigned char*)B;
+  p.Bs = nullptr;
   p.bias = bias;
   p.C = C;
   p.M = (int)M;
@@ -635,6 +800,7 @@ extern "C" int mase_gemm_bf16_tn_splitk(const void* A, const void* B, const void
   GemmParams p;
   p.A = (const unsigned char*)A;
   p.B = (const unsigned char*)B;
+  p.Bs = nullptr;
   p.bias = nullptr;
   p.C = workspace;
   p.M = (int)M;
@@ -690,6 +856,7 @@ extern "C" int mase_gemm_bf16_tn_packed(const void* A, const void* B_packed, con
   GemmParams p;
   p.A = (const unsigned char*)A;
   p.B = (const unsigned char*)B_packed;
+  p.Bs = nullptr;
   p.bias = bias;
   p.C = C;
   p.M = (int)M;
@@ -701,4 +868,56 @@ extern "C" int mase_gemm_bf16_tn_packed(const void* A, const void* B_packed, con
   p.splits = 1;
   p.kc = (int)K;
   return launch_gemm_bf16(p, out_dtype, (hipStream_t)stream, true);
+}
+
+extern "C" size_t mase_gemm_mxint8_packed_code_bytes(size_t N, size_t K) {
+  if (N == 0 || K == 0 || (K % 128) != 0) return 0;
+  return ((N + 31) / 32) * 32 * K;
+}
+
+extern "C" size_t mase_gemm_mxint8_packed_scale_bytes(size_t N, size_t K) {
+  if (N == 0 || K == 0 || (K % 128) != 0) return 0;
+  return ((N + 31) / 32) * 32 * (K / 32);
+}
+
+extern "C" int mase_gemm_mxint8_pack_b(const int8_t* codes, const uint8_t* scales, void* code_image, void* scale_image,
+                                       size_t N, size_t K, void* stream) {
+  using namespace mase;
+  if (N == 0 || K == 0) return MASE_OK;
+  if (codes == nullptr || scales == nullptr || code_image == nullptr || scale_image == nullptr) return MASE_ERR_NULL;
+  if ((K % 128) != 0 || N > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
+  if ((((uintptr_t)codes) & 7u) != 0 || !aligned16(code_image) || (((uintptr_t)scale_image) & 1u) != 0) return MASE_ERR_ALIGN;
+  const size_t granules = mase_gemm_mxint8_packed_code_bytes(N, K) / 8;
+  hipLaunchKernelGGL(gemm_pack_codes_kernel, dim3(blocks_for(granules, (size_t)256)), dim3(256), 0, (hipStream_t)stream,
+                     (const uint2*)codes, scales, (uint2*)code_image, (uint16_t*)scale_image, (int)N, (int)K, granules);
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+extern "C" int mase_gemm_mxint8_tn_packed(const void* A, const void* code_image, const void* scale_image, const void* bias,
+                                          void* C, size_t M, size_t N, size_t K, int out_dtype, int bias_dtype,
+                                          void* stream) {
+  using namespace mase;
+  if (M == 0 || N == 0) return MASE_OK;
+  if (A == nullptr || code_image == nullptr || scale_image == nullptr || C == nullptr) return MASE_ERR_NULL;
+  if (K == 0 || (K % (2 * BK)) != 0 || M > (1u << 30) || N > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
+  if ((unsigned long long)M * K * 2 > 0xFFFFFFFFull ||
+      (unsigned long long)mase_gemm_mxint8_packed_code_bytes(N, K) > 0xFFFFFFFFull)
+    return MASE_ERR_SHAPE;
+  if (!aligned16(A) || !aligned16(code_image) || (((uintptr_t)scale_image) & 1u) != 0) return MASE_ERR_ALIGN;
+  if (out_dtype < 0 || out_dtype > 2 || (bias != nullptr && (bias_dtype < 0 || bias_dtype > 2))) return MASE_ERR_DTYPE;
+  GemmParams p;
+  p.A = (const unsigned char*)A;
+  p.B = (const unsigned char*)code_image;
+  p.Bs = (const unsigned char*)scale_image;
+  p.bias = bias;
+  p.C = C;
+  p.M = (int)M;
+  p.N = (int)N;
+  p.K = (int)K;
+  p.bias_dtype = bias_dtype;
+  p.tiles_m = (int)((M + BM - 1) / BM);
+  p.tiles_n = (int)((N + BN - 1) / BN);
+  p.splits = 1;
+  p.kc = (int)K;
+  return launch_gemm_bf16(p, out_dtype, (hipStream_t)stream, true, true);
 }

@@ -14,7 +14,8 @@ from torch.nn import functional as F
 from ..._gemm import (MXFP_HW_FORMATS, MXFP_K_MULTIPLE, SKINNY_MAX_ROWS, gemm_bf16_pack_b, gemm_bf16_packed_b_supported,
                       gemm_bf16_takes_packed_b, gemm_bf16_tn, gemm_mxfp4_scaled_tiled, gemm_mxfp4_skinny, gemm_mxfp4_skinny_supported,
                       gemm_mxfp4_tiled_supported, mxfp_pack_tiled, mxfp_tile_codes,
-                      gemm_mxfp_scaled, gemm_mxint8_skinny, gemm_mxint8_skinny_supported, mxfp_pack)
+                      gemm_mxfp_scaled, gemm_mxint8_pack_b, gemm_mxint8_packed_supported, gemm_mxint8_skinny,
+                      gemm_mxint8_skinny_supported, gemm_mxint8_tn_packed, mxfp_pack)
 
 
 class WeightCache:
@@ -223,6 +224,59 @@ class PackedMXIntWeight:
 
     def valid_for(self, weight: Tensor) -> bool:
         return self.codes is not None and self._key is not None and self._key == _weight_key(weight)
+
+
+class MXIntCodeImage:
+    """An MXINT8 weight as the fragment-ordered code and scale images of the tiled kernel that widens codes in
+    registers (``gemm_mxint8_tn_packed``): 1.03 bytes per weight, in place of the bf16 image and its fragment-ordered
+    copy (2 + 2 bytes per weight).  Valid only while the parameter is the tensor the codes were made for."""
+
+    def __init__(self):
+        self._key = None
+        self.codes = self.scales = None
+        self.n = 0
+
+    def invalidate(self):
+        self._key = None
+        self.codes = self.scales = None
+
+    @staticmethod
+    def eligible(weight: Tensor, block_size: int, element_bits: int) -> bool:
+        return (weight.is_cuda and weight.dim() == 2 and block_size == 32 and element_bits == 8
+                and gemm_mxint8_packed_supported(weight.shape[0], weight.shape[1])
+                and weight.dtype in (torch.float32, torch.bfloat16, torch.float16))
+
+    def set(self, codes: Tensor, scales: Tensor, weight: Tensor) -> bool:
+        """Build the images from row-major codes [N, K] and scale bytes [N, K/32].  False (nothing kept) when a block
+        scale is below 2^-126: the kernel takes such weights as zero."""
+        n, k = weight.shape
+        scales = scales.reshape(n, k // 32)
+        if bool((scales < 8).any()):
+            self.invalidate()
+            return False
+        self.codes, self.scales = gemm_mxint8_pack_b(codes.reshape(n, k), scales)
+        self.n = n
+        self._key = _weight_key(weight)
+        return True
+
+    def valid_for(self, weight: Tensor) -> bool:
+        return self.codes is not None and self._key is not None and self._key == _weight_key(weight)
+
+
+def mxint_linear_codes(x: Tensor, image: MXIntCodeImage, bias: Tensor | None, quantize_to_bf16,
+                       xq: Tensor | None = None) -> Tensor:
+    """``F.linear(q(x), W, b)`` on the tiled kernel with W as MXINT8 code / scale images"""
+    lead = x.shape[:-1]
+    if xq is None:
+        xq = quantize_to_bf16(x.reshape(-1, x.shape[-1]))
+    y = gemm_mxint8_tn_packed(xq, image.codes, image.scales, image.n, bias, x.dtype)
+    return y.reshape(*lead, image.n)
+
+
+def mxint_codes_apply(x: Tensor, image: MXIntCodeImage, weight: Tensor) -> bool:
+    rows = x.numel() // x.shape[-1] if x.numel() else 0
+    return (x.is_cuda and rows > SKINNY_MAX_ROWS and x.dtype in (torch.float32, torch.bfloat16, torch.float16)
+            and image.valid_for(weight) and not torch.is_grad_enabled())
 
 
 def mxint_linear_decode(x: Tensor, packed: PackedMXIntWeight, bias: Tensor | None, quantize_to_bf16,

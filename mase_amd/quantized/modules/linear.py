@@ -11,8 +11,9 @@ from torch.nn import functional as F
 from ...quantizers import _ops, mxfp_quantizer, mxint_quantizer
 from ..functional.linear import (QuantizedParamCache, linearBlockFP, linearInteger, linearMinifloatDenorm,
                                  linearMinifloatIEEE)
-from ..functional.mx_linear import (PackedMXFPWeight, PackedMXIntWeight, WeightCache, mx_linear, mxfp_linear_native,
-                                    mxfp_native_layout, mxfp_native_pack, mxint_decode_applies, mxint_linear_decode)
+from ..functional.mx_linear import (MXIntCodeImage, PackedMXFPWeight, PackedMXIntWeight, WeightCache, mx_linear,
+                                    mxfp_linear_native, mxfp_native_layout, mxfp_native_pack, mxint_codes_apply,
+                                    mxint_decode_applies, mxint_linear_codes, mxint_linear_decode)
 
 
 class _LinearBase(torch.nn.Linear):
@@ -130,22 +131,34 @@ class LinearMXInt(_LinearMX):
     """``config["packed_decode"]`` (default False; not a key of the reference) keeps the weight's MXINT8 codes and scale
     bytes next to the parameter (1.03 bytes per weight more) and lets forwards of at most 128 rows stream those instead
     of the bf16 image: the product of decode-sized batches is bound by the weight bytes, which this halves.  A packed
-    checkpoint (``mase_amd.quantized.packed``) hands the codes over without this key."""
+    checkpoint (``mase_amd.quantized.packed``) hands the codes over without this key.
+
+    ``config["weight_memory"] = "codes"`` (default ``"bf16"``; not a key of the reference) makes forwards of more than
+    128 rows run from the weight's MXINT8 codes as well: the tiled kernel takes them in fragment order (1.03 bytes per
+    weight, built when the state dict is loaded) and widens them to bf16 in registers on the way into the matrix
+    instruction, so neither the bf16 image of the weight nor its fragment-ordered copy (2 + 2 bytes per weight) is
+    built.  Same results bit for bit; the contraction runs 10-16 % slower."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, dtype=None,
                  config=None) -> None:
         super().__init__(in_features, out_features, bias, device, dtype, config)
         self._w_codes = PackedMXIntWeight()
+        self._w_image = MXIntCodeImage()
 
     def invalidate_weight_cache(self):
         super().invalidate_weight_cache()
         self._w_codes.invalidate()
+        self._w_image.invalidate()
+
+    def _codes_mode(self) -> bool:
+        return self.config.get("weight_memory", "bf16") == "codes"
 
     def weights_loaded_quantized(self, codes=None, scales=None):
         """``codes`` / ``scales``: the quantizer's codes and scale bytes of the weight when the caller has them (a packed
         checkpoint); kept for the decode path if they decode to exactly the weight."""
         super().weights_loaded_quantized()
         self._w_codes.invalidate()
+        self._w_image.invalidate()
         if codes is None or self.bypass or self.gptq:
             return
         if not PackedMXIntWeight.eligible(self.weight, self.config["weight_block_size"], self.config["weight_width"]):
@@ -153,15 +166,23 @@ class LinearMXInt(_LinearMX):
         self._w_codes.set(codes.to(self.weight.device), scales.to(self.weight.device), self.weight)
         if not self._w_codes.decodes_to(self.weight.data):
             self._w_codes.invalidate()
+        elif self._codes_mode() and MXIntCodeImage.eligible(self.weight, 32, 8):
+            self._w_image.set(self._w_codes.codes, self._w_codes.scales, self.weight)
 
     def _quantize_params(self):
         cfg = self.config
         self._w_codes.invalidate()
-        if (cfg.get("packed_decode", False) and not self.clip_search
-                and PackedMXIntWeight.eligible(self.weight, cfg["weight_block_size"], cfg["weight_width"])):
+        self._w_image.invalidate()
+        want_image = self._codes_mode() and MXIntCodeImage.eligible(self.weight, cfg["weight_block_size"], cfg["weight_width"])
+        want_codes = cfg.get("packed_decode", False) and PackedMXIntWeight.eligible(
+            self.weight, cfg["weight_block_size"], cfg["weight_width"])
+        if (want_image or want_codes) and not self.clip_search:
             deq, codes, scales = _ops.mxint_qdq(self.weight.data, 32, 8, 1, 8, pack=True)
             self.weight.data.copy_(deq)
-            self._w_codes.set(codes, scales, self.weight)
+            if want_codes:
+                self._w_codes.set(codes, scales, self.weight)
+            if want_image:
+                self._w_image.set(codes, scales, self.weight)
         else:
             self.weight.data.copy_(
                 mxint_quantizer(self.weight.data, block_size=cfg["weight_block_size"], element_bits=cfg["weight_width"],
@@ -185,7 +206,8 @@ class LinearMXInt(_LinearMX):
         if (self.bypass or bs is None or bits is None or not x.is_cuda or x.numel() == 0
                 or x.dtype not in (torch.float32, torch.bfloat16, torch.float16)):
             return None
-        if not mxint_decode_applies(x, self._w_codes, self.weight) and self._w_cache.get(self.weight) is None:
+        if (not mxint_decode_applies(x, self._w_codes, self.weight) and not mxint_codes_apply(x, self._w_image, self.weight)
+                and self._w_cache.get(self.weight) is None):
             return None
         return ("mxint", bs, bits)
 
@@ -202,6 +224,8 @@ class LinearMXInt(_LinearMX):
             return F.linear(x, self.weight, self.bias)
         if mxint_decode_applies(x, self._w_codes, self.weight):
             return mxint_linear_decode(x, self._w_codes, self.bias, self.prepare_activation, xq=prepared)
+        if mxint_codes_apply(x, self._w_image, self.weight):
+            return mxint_linear_codes(x, self._w_image, self.bias, self.prepare_activation, xq=prepared)
         return mx_linear(
             x, self.weight, self.bias, self.prepare_activation,
             lambda t: mxint_quantizer(t, block_size=bs, element_bits=bits, block_dim=-1),

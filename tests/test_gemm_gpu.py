@@ -217,3 +217,37 @@ def test_gemm_with_the_weight_in_fragment_order_is_the_same_product(dev, M, N, K
     if K % 128 == 0 and M > 512:
         ref = (a.float() @ b.float().t())
         assert float((gemm_bf16_tn(a, b, None, torch.float32, b_packed=bp) - ref).abs().max() / ref.abs().max()) < 1e-5
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (512, 768, 256), (300, 200, 384), (4096, 4096, 1024), (130, 4096, 512),
+                                   (4100, 4200, 640), (16384, 1024, 4096), (16384, 4096, 11008), (16131, 11008, 4096)])
+def test_gemm_with_the_weight_as_mxint8_codes_in_fragment_order(dev, M, N, K):
+    """mase_gemm_mxint8_tn_packed (weight as int8 codes + scale bytes, widened in registers) against mase_gemm_bf16_tn
+    on the dequantized weight: the operands the matrix instruction sees are the same bf16 values, so the results are
+    bit-identical, for every output dtype, with a bias, ragged M and N, several launches"""
+    from mase_amd._gemm import gemm_bf16_tn, gemm_mxint8_pack_b, gemm_mxint8_tn_packed
+    from mase_amd.quantizers import _ops
+
+    g = torch.Generator().manual_seed(M + N + K + 1)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
+    w = torch.randn(N, K, generator=g) * 0.05
+    w[::7] *= torch.exp2(torch.randint(-6, 7, (K,), generator=g).float())   # a wide range of block scales
+    w[3] = 0.0
+    bias = torch.randn(N, generator=g).to(dev)
+    print(f"mxint8-codes gemm M={M} N={N} K={K}", flush=True)
+    deq, codes, scales = _ops.mxint_qdq(w.to(dev), 32, 8, 1, 8, pack=True, out_dtype=torch.bfloat16)
+    img, simg = gemm_mxint8_pack_b(codes.view(N, K), scales.view(N, K // 32))
+    assert img.numel() == (N + 31) // 32 * 32 * K and simg.numel() == (N + 31) // 32 * 32 * (K // 32)
+    from mase_amd import _lib
+
+    # a few hundred rows: gemm_bf16_tn cuts K into ranges there and adds the partial sums in another order
+    split = _lib.load().mase_gemm_bf16_tn_splitk_workspace_bytes(M, N, K) > 0
+    for dt, bs in ((torch.float32, None), (torch.bfloat16, bias), (torch.float16, bias.to(torch.float16))):
+        want = gemm_bf16_tn(a, deq.view(N, K), bs, dt)
+        for rep in range(3 if M * N * K > (1 << 36) else 2):
+            got = gemm_mxint8_tn_packed(a, img, simg, N, bs, dt)
+            if split:
+                tol = 1e-5 if dt == torch.float32 else 1e-2
+                assert float((got.float() - want.float()).abs().max() / want.float().abs().max()) < tol, (dt, rep)
+            else:
+                assert torch.equal(got, want), (dt, rep, float((got.float() - want.float()).abs().max()))

@@ -448,3 +448,53 @@ def test_sibling_projections_share_one_quantized_activation(dev):
                 for a, b, m in zip(project_shared(x, mods), want2, mods):
                     assert torch.equal(a, b), (type(m).__name__, dtype, rows, "after an edit of x")
                 assert not torch.equal(want2[0], want[0])
+
+
+def test_linear_mxint_from_codes(dev):
+    """config["weight_memory"] = "codes": forwards of more than 128 rows run from the fragment-ordered MXINT8 code image
+    (widened to bf16 in registers); results are those of the default module bit for bit, neither the bf16 image nor its
+    fragment-ordered copy gets built, and a changed weight falls back to the reference's F.linear on the new values"""
+    from mase_amd.quantized import LinearMXInt
+
+    g = torch.Generator().manual_seed(21)
+    w = torch.randn(512, 256, generator=g) * 0.05
+    w[::5] *= torch.exp2(torch.randint(-5, 6, (256,), generator=g).float())
+    b = torch.randn(512, generator=g)
+    for dtype in (torch.float32, torch.bfloat16):
+        for extra in ({}, {"packed_decode": True}):
+            ref = LinearMXInt(256, 512, device=dev, dtype=dtype, config=dict(MXINT_CFG))
+            m = LinearMXInt(256, 512, device=dev, dtype=dtype, config=dict(MXINT_CFG, weight_memory="codes", **extra))
+            for mod in (ref, m):
+                mod.load_state_dict({"weight": w.to(dtype), "bias": b.to(dtype)})
+            assert torch.equal(m.weight, ref.weight)
+            assert m._w_image.valid_for(m.weight) and m._w_codes.valid_for(m.weight) == bool(extra)
+            assert m._w_image.codes.numel() == 512 * 256 and m._w_image.scales.numel() == 512 * 8
+            for rows in (300, 1500, 4096):
+                x = torch.randn(rows, 256, generator=g).to(dtype).to(dev)
+                got, want = m(x), ref(x)
+                if rows == 300:   # the default module cuts K into ranges for a few hundred rows: another summation order
+                    assert rel_err(got, want.cpu()) < (1e-5 if dtype == torch.float32 else 1e-2)
+                else:
+                    assert torch.equal(got, want), (dtype, rows)
+            assert m._w_cache._w is None and m._w_cache._packed is None, "the bf16 images must not have been built"
+            x8 = torch.randn(8, 256, generator=g).to(dtype).to(dev)
+            assert rel_err(m(x8), ref(x8).cpu()) < (1e-5 if dtype == torch.float32 else 1e-2)
+            with torch.no_grad():
+                m.weight.mul_(0.5)     # no longer the tensor the codes were made for
+                ref.weight.mul_(0.5)
+            x = torch.randn(600, 256, generator=g).to(dtype).to(dev)
+            assert not m._w_image.valid_for(m.weight)
+            assert rel_err(m(x), ref(x).cpu()) < (1e-5 if dtype == torch.float32 else 1e-2)
+    # a packed checkpoint hands the codes over: the image is built from them
+    from mase_amd.quantized.packed import load_packed_state_dict, packed_state_dict
+
+    src = LinearMXInt(256, 512, device=dev, dtype=torch.bfloat16, config=dict(MXINT_CFG))
+    src.load_state_dict({"weight": w.bfloat16(), "bias": b.bfloat16()})
+    dst = LinearMXInt(256, 512, device=dev, dtype=torch.bfloat16, config=dict(MXINT_CFG, weight_memory="codes"))
+    holder_src, holder_dst = nn.Sequential(src), nn.Sequential(dst)
+    packed = packed_state_dict(holder_src, {"0.weight": w.bfloat16()})   # codes of the weights the model was quantized from
+    assert "0.weight.mx_codes" in packed
+    load_packed_state_dict(holder_dst, packed)
+    assert dst._w_image.valid_for(dst.weight)
+    x = torch.randn(2048, 256, generator=g).bfloat16().to(dev)
+    assert torch.equal(dst(x), src(x))
