@@ -253,6 +253,32 @@ class MxintLinear(Workload):
                 "kind": "port", "sample": f"{n} full forwards (activation quantize-dequantize + fp32 F.linear), {dt*1e3:.0f} ms each"}
 
 
+class MxintLinearCodes(MxintLinear):
+    """config 3's operands with the weight kept as fragment-ordered MXINT8 codes (1.03 B per weight) that the tiled
+    kernel widens in registers: ``config["weight_memory"] = "codes"``"""
+    name = "mxint_linear_codes"
+    config = {"workload": MxintLinear.config["workload"] + "; weight_memory=codes"}
+
+    def setup(self, torch, dev, n_buffers):
+        from mase_amd.quantized import LinearMXInt
+        from mase_amd.quantizers import _ops
+        from mase_amd._gemm import gemm_mxint8_tn_packed
+
+        self.torch = torch
+        x, w, b = self.make(torch)
+        self.host = (x, w, b)
+        self.m = LinearMXInt(self.K, self.N, bias=True, device=dev, config=dict(self.cfg, weight_memory="codes"))
+        self.m.load_state_dict({"weight": w, "bias": b})
+        self.bufs = [x.to(dev).roll(i, dims=0).contiguous() for i in range(max(n_buffers, 4))]
+        self.xq = _ops.mxint_qdq(self.bufs[0], 32, 8, -1, 8, out_dtype=torch.bfloat16)
+        self.img = self.m._w_image
+        assert self.img.valid_for(self.m.weight)
+        self._gemm = gemm_mxint8_tn_packed
+
+    def dominant_step(self, i):
+        self.out = self._gemm(self.xq, self.img.codes, self.img.scales, self.img.n, self.m.bias, self.torch.float32)
+
+
 class MxfpLinear(Workload):
     name = "mxfp_linear"
     default_steps, default_warmup = 300, 50
@@ -679,7 +705,7 @@ class DecodeLinearMxfp4(Workload):
                 "kind": "port", "sample": f"{n} forwards with {n_rows} of the {self.N} output rows (fp32 on the CPU), {dt*1e3:.0f} ms each"}
 
 
-WORKLOADS = {w.name: w for w in (MxintClipSearch, BfpQdq, MxintQdq, MxintLinear, MxfpLinear, DecoderLayerMxint, CopyBytes, IntegerQdq,
+WORKLOADS = {w.name: w for w in (MxintClipSearch, BfpQdq, MxintQdq, MxintLinear, MxintLinearCodes, MxfpLinear, DecoderLayerMxint, CopyBytes, IntegerQdq,
                                  MinifloatDenormQdq, MinifloatIeeeQdq, MinifloatMxQdq, MxfpQdq, AttnProb, DecodeLinear,
                                  DecodeLinearPacked, DecodeLinearMxfp4)}
 

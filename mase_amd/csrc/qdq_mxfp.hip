@@ -9,6 +9,7 @@
 //   y_i  = minifloat_decode(c_i) * 2^sh, converted to the output dtype;  scale byte = sh + 127
 // An all-flushed block has scale byte 0 and decodes to +0.  A block holding Inf/NaN decodes to NaN in the
 // reference (its int32 conversion of log2 wraps to the largest scale, 0 * inf), and does here.
+#include <algorithm>
 #include "common.hpp"
 #include "minifloat_mx.hpp"
 #include "mxfp_core.hpp"
@@ -379,10 +380,235 @@ __global__ __launch_bounds__(64) void mxfp_pack_kernel(const void* __restrict__ 
   }
 }
 
+// The same packing for a 16-bit tensor and a wide-exponent element format (e4m3, e5m2) on the packed 16-bit cast:
+// the cast value's [exponent | kept mantissa bits] field, rebased from the tensor dtype's exponent bias at this block's
+// scale to the code's, IS the code, so codes come out two per register without the elements ever being widened.
+// One lane owns one block of 32 (four 16-byte vectors, 64 consecutive bytes): the block's scale and the cast's
+// per-block constants are computed once per 32 elements.
+// A block uses a reserved code iff one of its cast values reaches the format's top code (e4m3) or top binade (e5m2):
+// seen on the cast values' running maximum; such a block is rebased one exponent step higher, which halves every code
+// with exponent field >= 2 exactly.  A vector of 8 elements is encoded on the fp32 form instead where the
+// quantize-dequantize kernel would do so (block not regular, element subnormal in T or below the format's normal
+// range) and, in a re-expressed block, when it may hold a code with exponent field 1 (whose half is a rounded
+// subnormal); its codes are then halved as codes.
+// The row of block b (< 2^31) is b / kb by multiplication: row = mulhi(b, kb_magic) >> kb_shift with
+// kb_magic = ceil(2^(31 + l) / kb), kb_shift = l - 1, l = ceil(log2 kb) >= 2 (exact for 31-bit dividends).
+template <int DT, int E, int F, bool TILED>
+__global__ __launch_bounds__(kVecThreads) void mxfp_pack_pk16_kernel(const uint4* __restrict__ in,
+                                                                     uint8_t* __restrict__ codes,
+                                                                     uint8_t* __restrict__ scales, uint32_t n_blocks,
+                                                                     MxfpParams p, MxfpPk16Params q, uint32_t kb,
+                                                                     uint32_t kb_magic, uint32_t kb_shift) {
+  static_assert(E + F + 1 == 8 && E >= 4, "8-bit codes of a wide-exponent format");
+  using TR = DTypeTraits<DT>;
+  constexpr int MB = (DT == MASE_DT_BF16) ? 7 : 10, EB = (DT == MASE_DT_BF16) ? 127 : 15;
+  constexpr uint32_t one = 0x00010001u;
+  WaveLog2 meta;
+  meta.init(p.tab, kLog2TabHalf);
+  const uint32_t lane = threadIdx.x;
+  const uint32_t blk = blockIdx.x * (uint32_t)kVecThreads + lane;
+  const bool live = blk < n_blocks;
+  // Load v of a quad of lanes (4q .. 4q+3) reads the 64 bytes of block 4q + v, 16 per lane, so every load touches
+  // runs of 64 bytes; a 4 x 4 exchange inside the quad (two butterfly steps on quad permutes) then gives each lane
+  // the four vectors of its own block.  n_blocks is a multiple of 4 (the launcher's condition).
+  uint4 raw[4];
+  {
+    const uint32_t quad_blk = blk - (lane & 3u);
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+      raw[v] = live ? load_nt(in + (size_t)(quad_blk + v) * 4 + (lane & 3u)) : make_uint4(0, 0, 0, 0);
+    uint32_t t[4][4];  // [register][dword]
+#pragma unroll
+    for (int v = 0; v < 4; ++v) { t[v][0] = raw[v].x; t[v][1] = raw[v].y; t[v][2] = raw[v].z; t[v][3] = raw[v].w; }
+    const bool odd = (lane & 1u) != 0, upper = (lane & 2u) != 0;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+#pragma unroll
+      for (int r0 = 0; r0 < 4; r0 += 2) {  // lanes i, i^1 exchange registers (r0, r0+1)
+        const uint32_t got = dpp_mov<0xB1>(odd ? t[r0][d] : t[r0 + 1][d]);
+        t[r0][d] = odd ? got : t[r0][d];
+        t[r0 + 1][d] = odd ? t[r0 + 1][d] : got;
+      }
+#pragma unroll
+      for (int r0 = 0; r0 < 2; ++r0) {  // lanes i, i^2 exchange registers (r0, r0+2)
+        const uint32_t got = dpp_mov<0x4E>(upper ? t[r0][d] : t[r0 + 2][d]);
+        t[r0][d] = upper ? got : t[r0][d];
+        t[r0 + 2][d] = upper ? t[r0 + 2][d] : got;
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < 4; ++v) raw[v] = make_uint4(t[v][0], t[v][1], t[v][2], t[v][3]);
+  }
+  // block maximum: packed over the 16 registers, then as flushed fp32 bits
+  uint32_t pm = 0;
+#pragma unroll
+  for (int v = 0; v < 4; ++v)
+    pm = pk_max_u16(pm, pk_max_u16(pk_max_u16(raw[v].x & 0x7FFF7FFFu, raw[v].y & 0x7FFF7FFFu),
+                                   pk_max_u16(raw[v].z & 0x7FFF7FFFu, raw[v].w & 0x7FFF7FFFu)));
+  pm = max(pm & 0xFFFFu, pm >> 16);
+  uint32_t m;
+  if constexpr (DT == MASE_DT_BF16) m = pm << 16;
+  else m = f2bits(f16_bits_to_f32(pm));
+  if ((m & 0x7F800000u) == 0) m = 0;  // a subnormal maximum means every element is flushed
+  int sh = 0;
+  const int state = mxfp_block_scale(m, p, sh, meta);
+  const int botf = q.bot0 + sh;
+  const uint32_t topf = (uint32_t)min(max(q.top0 + sh, 1), 0xFF);
+  Pk16Range r;
+  r.odd_k2 = (((q.parity0 - sh) & 1) ? (1u << MB) : 0u) * one;
+  r.max2 = ((topf << MB) | q.maxfrac) * one;
+  const uint32_t lo_thr = (uint32_t)min(max(botf, 1), 0xFF) << MB;
+  r.lo_thr2 = lo_thr * one;
+  r.sub_thr2 = 0;
+  uint32_t y[4][4], lo[4];
+  u16x2 top_acc = as_u16x2(0u);
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    const uint32_t w[4] = {raw[v].x, raw[v].y, raw[v].z, raw[v].w};
+    u16x2 lo_acc = as_u16x2(0xFFFFFFFFu), hi_acc = as_u16x2(0u);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      y[v][j] = pk16_cast<MB, false>(w[j], q.f, r, lo_acc, hi_acc);
+      top_acc = __builtin_elementwise_max(top_acc, as_u16x2(y[v][j] & 0x7FFF7FFFu));
+    }
+    lo[v] = min((uint32_t)lo_acc.x, (uint32_t)lo_acc.y);
+  }
+  const uint32_t top_y = max((uint32_t)top_acc.x, (uint32_t)top_acc.y);
+  // the element that takes a reserved code lies in the block's top binade, so its cast value is valid unless the whole
+  // block is subnormal in T, and then every vector takes the fp32 form and reports from its codes
+  const bool top_reserved = top_y >= ((E == 4) ? ((topf << MB) | q.maxfrac) : (topf << MB));
+  uint32_t lowest = lo_thr;
+  if constexpr (DT == MASE_DT_BF16) lowest = max(lowest, (uint32_t)min(max(sh + 1, 1), 0xFF) << MB);
+  if (top_reserved) lowest += 1u << MB;
+  uint32_t cc[4][4];  // codes, two per register (one per 16-bit half)
+  uint32_t fp32_form = 0, flag = 0;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    if (__builtin_expect(state != 1 || lo[v] + 1u < lowest, 0)) {
+      float x[8], z[8];
+      uint32_t c[8];
+      TR::unpack(raw[v], x);
+      mxfp_elements<true, 8>(x, state, sh, p, c, z);  // the form that handles codes with exponent field 0 in line
+#pragma unroll
+      for (int j = 0; j < 8; ++j) flag |= code_is_reserved<E, F>(c[j]) ? 1u : 0u;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) cc[v][j] = c[2 * j] | (c[2 * j + 1] << 16);
+      fp32_form |= 1u << v;
+    }
+  }
+  const bool reserved = state == 1 && (top_reserved || flag != 0);
+  const uint32_t rebase2 = ((uint32_t)((sh + (reserved ? 1 : 0) + EB - p.m.bias) << F) & 0xFFFFu) * one;
+  const u16x2 drop2 = {(unsigned short)q.f.drop, (unsigned short)q.f.drop};
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    if (__builtin_expect((fp32_form >> v) & 1u, 0)) {
+      if (reserved) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t a = cc[v][j] & 0x007F007Fu;
+          const uint32_t small = neg_mask2(as_u32(as_u16x2(a) - as_u16x2((2u << F) * one)));  // exponent field < 2
+          const uint32_t h_big = as_u32(as_u16x2(a) - as_u16x2((1u << F) * one));
+          const uint32_t half = (a >> 1) & 0x003F003Fu;
+          const uint32_t h_small = half + (a & half & one);  // the value of such a code is the code: round half even
+          cc[v][j] = (small & h_small) | (~small & h_big) | (cc[v][j] & 0x00800080u);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t ya = y[v][j] & 0x7FFF7FFFu;
+        const uint32_t nz = neg_mask2(as_u32(as_u16x2(ya) + as_u16x2(0x7FFF7FFFu)));  // halves that are not zero
+        const uint32_t field = as_u32((as_u16x2(ya) >> drop2) - as_u16x2(rebase2));
+        cc[v][j] = (field & nz & 0x007F007Fu) | ((y[v][j] >> 8) & 0x00800080u);
+      }
+    }
+  }
+  const int sb = (state == 1) ? min(sh + 127 + (reserved ? 1 : 0), 254) : (state == 0 ? 0 : 255);
+  if (live) scales[blk] = (uint8_t)sb;
+  uint4 o[2];  // the block's 32 code bytes
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    o[h].x = __builtin_amdgcn_perm(cc[2 * h][1], cc[2 * h][0], 0x06040200u);
+    o[h].y = __builtin_amdgcn_perm(cc[2 * h][3], cc[2 * h][2], 0x06040200u);
+    o[h].z = __builtin_amdgcn_perm(cc[2 * h + 1][1], cc[2 * h + 1][0], 0x06040200u);
+    o[h].w = __builtin_amdgcn_perm(cc[2 * h + 1][3], cc[2 * h + 1][2], 0x06040200u);
+  }
+  // A quad's four blocks are one 128-byte run of codes (tiled image: one row of one K tile, whose 16-byte chunks are
+  // exchanged by chunk ^= swizzle of the row).  Store h of lane j writes chunk 4h + j of the quad, fetched from the
+  // lane that produced it (lane (4h + j) / 2, its vector (4h + j) % 2), so a quad writes runs of 64 bytes.
+  const uint32_t j = lane & 3u;
+  uint8_t* line;
+  uint32_t sw = 0;
+  if constexpr (TILED) {
+    const uint32_t quad_blk = blk - j;
+    const uint32_t mrow = __umulhi(quad_blk, kb_magic) >> kb_shift;
+    const uint32_t k0 = (quad_blk - mrow * kb) * 32u;  // byte (= element) position in the row: a multiple of 128
+    const uint32_t rr = mrow & 255u;
+    sw = (rr >> 1) & 7u;
+    line = codes + ((size_t)(mrow >> 8) * (kb >> 2) + (k0 >> 7)) * 32768 + rr * 128u;
+  } else {
+    line = codes + (size_t)(blk - j) * 32;
+  }
+  const bool second = (lane & 1u) != 0;
+  uint4 d0, d1;
+  {
+    const uint32_t a0 = dpp_mov<0x50>(o[0].x), b0 = dpp_mov<0x50>(o[1].x), a1 = dpp_mov<0x50>(o[0].y), b1 = dpp_mov<0x50>(o[1].y);
+    const uint32_t a2 = dpp_mov<0x50>(o[0].z), b2 = dpp_mov<0x50>(o[1].z), a3 = dpp_mov<0x50>(o[0].w), b3 = dpp_mov<0x50>(o[1].w);
+    d0 = make_uint4(second ? b0 : a0, second ? b1 : a1, second ? b2 : a2, second ? b3 : a3);  // from lane j / 2
+  }
+  {
+    const uint32_t a0 = dpp_mov<0xFA>(o[0].x), b0 = dpp_mov<0xFA>(o[1].x), a1 = dpp_mov<0xFA>(o[0].y), b1 = dpp_mov<0xFA>(o[1].y);
+    const uint32_t a2 = dpp_mov<0xFA>(o[0].z), b2 = dpp_mov<0xFA>(o[1].z), a3 = dpp_mov<0xFA>(o[0].w), b3 = dpp_mov<0xFA>(o[1].w);
+    d1 = make_uint4(second ? b0 : a0, second ? b1 : a1, second ? b2 : a2, second ? b3 : a3);  // from lane 2 + j / 2
+  }
+  if (live) {
+    *(uint4*)(line + ((j ^ sw) << 4)) = d0;
+    *(uint4*)(line + (((4u + j) ^ sw) << 4)) = d1;
+  }
+}
+
+template <int DT, bool TILED>
+bool launch_mxfp_pack_pk16(const void* in, uint8_t* codes, uint8_t* scales, size_t n8, int E, int F,
+                           const MxfpParams& p, uint32_t k8, hipStream_t st) {
+  if constexpr (DT == MASE_DT_F32) {
+    return false;
+  } else {
+    constexpr int MB = (DT == MASE_DT_BF16) ? 7 : 10, EB = (DT == MASE_DT_BF16) ? 127 : 15;
+    if (!((E == 4 && F == 3) || (E == 5 && F == 2)) || !aligned16(in) || !aligned16(codes)) return false;
+    const size_t n_blocks = n8 / 4;
+    const uint32_t kb = k8 / 4;
+    // quads of lanes read and write four consecutive blocks together
+    if (n_blocks == 0 || (n_blocks & 3) != 0 || n_blocks >= (1ull << 31) || (TILED && kb < 4)) return false;
+    MxfpPk16Params q;
+    q.f = make_pk16_format<MB>(p.m.F, 0);
+    q.top0 = p.m.e_hi - p.m.bias + EB;
+    q.bot0 = 1 - p.m.bias + EB;
+    q.maxfrac = (uint32_t)p.m.frac_hi << q.f.drop;
+    q.parity0 = (p.m.bias - EB) & 1;
+    uint32_t magic = 0, shift = 0;
+    if (TILED) {
+      uint32_t l = 0;
+      while ((1ull << l) < kb) ++l;
+      magic = (uint32_t)(((1ull << (31 + l)) + kb - 1) / kb);
+      shift = l - 1;
+    }
+    const dim3 grid(blocks_for(n_blocks, (size_t)kVecThreads)), block(kVecThreads);
+    if (E == 4)
+      hipLaunchKernelGGL((mxfp_pack_pk16_kernel<DT, 4, 3, TILED>), grid, block, 0, st, (const uint4*)in, codes, scales,
+                         (uint32_t)n_blocks, p, q, kb, magic, shift);
+    else
+      hipLaunchKernelGGL((mxfp_pack_pk16_kernel<DT, 5, 2, TILED>), grid, block, 0, st, (const uint4*)in, codes, scales,
+                         (uint32_t)n_blocks, p, q, kb, magic, shift);
+    return true;
+  }
+}
+
 template <int DTI>
 int launch_mxfp_pack(const void* in, uint8_t* codes, uint8_t* scales, size_t numel, int E, int F, const MxfpParams& p,
                      hipStream_t st) {
   const size_t n8 = numel / 8;
+  if (launch_mxfp_pack_pk16<DTI, false>(in, codes, scales, n8, E, F, p, 0u, st))
+    return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
   const dim3 grid(blocks_for(n8, 64)), block(64);
   if (E == 4 && F == 3) hipLaunchKernelGGL((mxfp_pack_kernel<DTI, 4, 3>), grid, block, 0, st, in, codes, scales, n8, p, 0u);
   else if (E == 5 && F == 2) hipLaunchKernelGGL((mxfp_pack_kernel<DTI, 5, 2>), grid, block, 0, st, in, codes, scales, n8, p, 0u);
@@ -397,6 +623,8 @@ int launch_mxfp_pack_tiled(const void* in, uint8_t* codes, uint8_t* scales, size
   const size_t n8 = rows * K / 8;
   const dim3 grid(blocks_for(n8, 64)), block(64);
   const uint32_t k8 = (uint32_t)(K / 8);
+  if (launch_mxfp_pack_pk16<DTI, true>(in, codes, scales, n8, E, F, p, k8, st))
+    return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
   if (E == 4 && F == 3)
     hipLaunchKernelGGL((mxfp_pack_kernel<DTI, 4, 3, true>), grid, block, 0, st, in, codes, scales, n8, p, k8);
   else if (E == 5 && F == 2)

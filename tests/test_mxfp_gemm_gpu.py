@@ -53,6 +53,45 @@ def test_mxfp_pack_decodes_to_the_quantizer_output(dev, fmt, dtype):
     assert bool(((got == 0) == (want == 0)).all()) or fmt == (5, 2)
 
 
+@pytest.mark.parametrize("fmt", [(4, 3), (5, 2)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mxfp_pack_of_16bit_tensors_is_the_fp32_packing_of_the_same_values(dev, fmt, dtype):
+    """16-bit tensors take the kernel that derives the codes from the packed 16-bit cast; fp32 tensors the one that
+    encodes on the fp32 bit fields.  Same values in, same codes and scale bytes out: adversarial values (powers of two
+    and their neighbours, zeros, subnormals of the dtype, huge spreads inside a block), plain normal data, blocks that
+    use the reserved codes and a block of non-finite values."""
+    from mase_amd._gemm import mxfp_pack, mxfp_pack_tiled, mxfp_tile_codes
+
+    rng = np.random.default_rng(100 + fmt[0])
+    g = torch.Generator().manual_seed(7)
+    parts = [adversarial(rng, (96, 512), dtype, block=32), torch.randn(700, 512, generator=g).to(dtype),
+             (torch.randn(64, 512, generator=g) * torch.exp2(torch.randint(-20, 12, (64, 512), generator=g).float())).to(dtype)]
+    x = torch.cat(parts)
+    x[5, :32] = torch.linspace(-1, 1, 32).to(dtype) * 479.0 / 256   # maximum on the top e4m3 code
+    x[6, 32:64] = torch.linspace(-1, 1, 32).to(dtype) * 7.5          # and one that rounds up to it
+    x[7, :32] = float("inf")
+    x[8, 64:96] = float("nan")
+    x[9, :64] = 0
+    x[10, :32] = torch.tensor(2.0 ** -14 if dtype == torch.float16 else 2.0 ** -120).to(dtype) / 3  # subnormal / tiny
+    xd = x.to(dev)
+    c16, s16 = mxfp_pack(xd, *fmt)
+    c32, s32 = mxfp_pack(xd.float(), *fmt)
+    assert torch.equal(s16, s32)
+    bad = (c16 != c32)
+    assert not bool(bad.any()), (int(bad.sum()), x[bad.cpu()][:8], c16[bad][:8], c32[bad][:8])
+    for rows, K in ((3, 96), (1, 32), (5, 160), (7, 128)):  # block counts that are and are not multiples of 4
+        xs = xd[:rows, :K].contiguous()
+        a, b = mxfp_pack(xs, *fmt)
+        c, d = mxfp_pack(xs.float(), *fmt)
+        assert torch.equal(a, c) and torch.equal(b, d), (rows, K)
+    t16, ts16 = mxfp_pack_tiled(xd, *fmt)
+    assert torch.equal(ts16, s32)
+    want = mxfp_tile_codes(c32, 512, 8).cpu().reshape(-1, 4, 256, 128).permute(0, 2, 1, 3)
+    got = t16.cpu().reshape(-1, 4, 256, 128).permute(0, 2, 1, 3)
+    live = torch.arange(want.shape[0] * 256).reshape(-1, 256) < x.shape[0]  # padding rows are left unwritten
+    assert torch.equal(got[live], want[live])
+
+
 @pytest.mark.parametrize("bfmt", [(2, 1), (4, 3), (5, 2)])
 @pytest.mark.parametrize("afmt", [(4, 3), (5, 2)])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 200, 384), (512, 768, 1024), (1, 33, 256)])
