@@ -34,7 +34,7 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
 constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int S = 2;                              // LDS stages
-constexpr int kStagesB = 3;                       // stages of A alone (32 KB each) when B comes in fragment order
+constexpr int kStagesB = 4;                       // stages of A alone (32 KB each) when B comes in fragment order
 constexpr int kGemmThreads = 256;
 constexpr int kRowBytes = BK * 2;                 // 128: one cache line per operand row per K tile
 constexpr int kTileBytes = BM * kRowBytes;        // 32 KB per operand per stage
@@ -119,7 +119,7 @@ __device__ __forceinline__ void ucodes4_to_bf16(uint32_t u, float scale, float b
 // without branches; the other instantiation (K = one tile) advances it with the general, branching step.
 // BPACK (with STREAM, an even number of K tiles): B is the fragment-ordered image of mase_gemm_bf16_pack_b and its
 // fragments go from L2 straight into registers, one K tile ahead of the MFMAs that use them; only A passes through
-// LDS, in three stages of 32 KB.  That halves the LDS traffic (the copies landing in LDS while the wavefronts read
+// LDS, in four stages of 32 KB.  That halves the LDS traffic (the copies landing in LDS while the wavefronts read
 // their fragments is what holds the plain kernel back) at the price of every B fragment being fetched by the two
 // wavefronts that share it.
 // BCODES (with BPACK): B is an MXINT8 weight as codes + scale bytes in fragment order (mase_gemm_mxint8_pack_b): half
@@ -234,8 +234,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   zero_acc();
 
   set_copy_tile(0);
+  // the copy stream leads the K loop by S tiles (BPACK: by kStagesB - 1)
 #pragma unroll
-  for (int t = 0; t < S; ++t) {
+  for (int t = 0; t < (BPACK ? kStagesB - 1 : S); ++t) {
 #pragma unroll
     for (int c = 0; c < kCopies; ++c) issue_copy(c);
     advance_copy_stream();
@@ -426,16 +427,16 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // respect to each other: a younger register load can complete before an older LDS copy (with "all but the 16
   // youngest" as the hand-over test, A tiles were read before they had landed, on shapes whose B image often misses the
   // cache).  One counter covers both, so "at most n outstanding" proves that an A copy has landed only if at least
-  // n + 1 younger *A copies* would otherwise have to be pending with it.  Hence three stages of A: the 8 copies of the
-  // K tile after next are issued *before* the hand-over that needs the next K tile, and that hand-over waits for
-  // "at most 8 outstanding": the next K tile has landed (its copies are older than those 8); the young copies
-  // themselves fly on across the barrier.  The B fragments are proven the same way, by counting the register loads
-  // issued after them (see the waits at the head of each step).
+  // n + 1 younger *A copies* would otherwise have to be pending with it.  Hence four stages of A: the copy stream runs
+  // three K tiles ahead, so when a hand-over needs the next K tile, the 16 copies of the two K tiles after it have
+  // been issued, and the hand-over waits for "at most 16 outstanding": the next K tile has landed (its copies are older
+  // than those 16), while the young copies and up to that many B loads fly on across the barrier.  The B fragments are
+  // proven the same way, by counting the register loads issued after them (see the waits at the head of each step).
   //   step 0: MFMAs on fr[0]; LDS reads of step 1; the 16 B loads of the next K tile (their registers were last read
   //           one K tile ago)
-  //   step 1: MFMAs on fr[1]; LDS reads of steps 2 and 3; the 8 A copies of the K tile after next into the stage
+  //   step 1: MFMAs on fr[1]; LDS reads of steps 2 and 3; the 8 A copies of the K tile three ahead into the stage
   //           vacated at the previous hand-over, one every other MFMA slot
-  //   step 2: MFMAs on fr[2]; then the hand-over: at most 8 loads outstanding, own LDS reads complete, barrier
+  //   step 2: MFMAs on fr[2]; then the hand-over: at most 16 loads outstanding, own LDS reads complete, barrier
   //   step 3: MFMAs on fr[3]; LDS reads of step 0 of the next K tile
   // Stores of an epilogue only make the wait of the next output tile's first hand-over conservative.
   auto k_iteration_b = [&](auto&& advance, auto bufc) __attribute__((always_inline)) {
@@ -468,7 +469,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
         __builtin_amdgcn_sched_barrier(0);
       }
       if (s == 2) {
-        wait_vmcnt<kWaveCopies>();
+        wait_vmcnt<(kStagesB - 2) * kWaveCopies>();
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -517,7 +518,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
         __builtin_amdgcn_sched_barrier(0);
       }
       if (s == 2) {
-        wait_vmcnt<kWaveCopies>();
+        wait_vmcnt<(kStagesB - 2) * kWaveCopies>();
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -559,20 +560,25 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     if constexpr (BPACK) {
       // two K tiles per trip (the fragment buffers alternate); the copy stream as in the plain form below, the B
       // stream one K tile ahead: it moves on to the next output tile before the last K tile of this one
-      auto iter = [&](auto bufc) __attribute__((always_inline)) {
-        if constexpr (BCODES) k_iteration_c(step_within_tile, bufc);
-        else k_iteration_b(step_within_tile, bufc);
+      auto iter = [&](auto bufc, auto&& advance) __attribute__((always_inline)) {
+        if constexpr (BCODES) k_iteration_c(advance, bufc);
+        else k_iteration_b(advance, bufc);
       };
+      // while the copy stream (kStagesB - 1 = 3 K tiles ahead) stays inside this output tile it advances without
+      // branches; over the last four K tiles (both, when there are only two) it takes the general step, which moves
+      // it on to the next output tile
+      int kt = 0;
 #pragma unroll 1
-      for (int kt = 0; kt < nk - S; kt += 2) {
-        iter(std::integral_constant<int, 0>{});
-        iter(std::integral_constant<int, 1>{});
+      for (; kt + 6 <= nk; kt += 2) {
+        iter(std::integral_constant<int, 0>{}, step_within_tile);
+        iter(std::integral_constant<int, 1>{}, step_within_tile);
       }
-      set_copy_tile(ord + 1);
-      c_kt = 0;
-      iter(std::integral_constant<int, 0>{});
-      set_b_tile(ord + 1);
-      iter(std::integral_constant<int, 1>{});
+#pragma unroll 1
+      for (; kt < nk; kt += 2) {
+        iter(std::integral_constant<int, 0>{}, advance_copy_stream);
+        if (kt + 2 >= nk) set_b_tile(ord + 1);
+        iter(std::integral_constant<int, 1>{}, advance_copy_stream);
+      }
     } else if constexpr (STREAM) {
       // the copy stream stands at K tile S of this output tile (or, if nk == S, at K tile 0 of the next)
 #pragma unroll 1
