@@ -13,13 +13,19 @@ device.  Weights are written back into the ``nn.Linear`` modules, so that the qu
 
 Differences from the reference's driver: calibration token ids are passed in (``gptq_config["calibration_data"]``, an
 integer tensor ``[nsamples, seqlen]`` or a list of ``[1, seqlen]`` tensors) instead of being downloaded by dataset
-name; the per-layer checkpoint files are not built and raise ``NotImplementedError``.  ``clip_search_y`` scores the
-clip search of each column group on the group's calibration inputs (``mase_mx*_clip_candidates`` plus matrix products).
+name.  ``clip_search_y`` scores the clip search of each column group on the group's calibration inputs
+(``mase_mx*_clip_candidates`` plus matrix products).  ``checkpoint_dir`` writes one safetensors file (and a JSON
+description) per finished decoder layer and resumes after the last layer found there, with the reference's file names
+(``checkpoint.py:9-135``); like the reference's driver, a resumed run calibrates its first layer on the inputs of
+layer 0 unless ``resume_propagate`` is set, which first runs those inputs through the layers that were loaded.
 """
 from __future__ import annotations
 
+import json
 import logging
 import math
+import os
+import re
 
 import torch
 from torch import Tensor, nn
@@ -178,6 +184,65 @@ def _calibration_batches(gptq_config):
     return [d if d.dim() == 2 else d.unsqueeze(0) for d in data]
 
 
+_CKPT_MODEL_NAME = "quantized_model"
+
+
+def _layer_file(checkpoint_dir: str, layer_idx: int) -> str:
+    return os.path.join(checkpoint_dir, f"{_CKPT_MODEL_NAME}_layer_{layer_idx}.safetensors")
+
+
+def save_layer_checkpoint(network, layer_idx: int, checkpoint_dir: str | None) -> None:
+    """checkpoint.py:9-72: the parameters of decoder layer ``layer_idx`` under their names relative to the layer, in
+    ``<dir>/quantized_model_layer_<i>.safetensors``, and a JSON description beside it"""
+    if checkpoint_dir is None:
+        return
+    from safetensors.torch import save_file
+
+    os.makedirs(checkpoint_dir, exist_ok=True)
+    prefix = f"model.layers.{layer_idx}."
+    tensors = {name[len(prefix):]: p.detach().cpu().contiguous() for name, p in network.named_parameters()
+               if name.startswith(prefix)}
+    if not tensors:
+        logging.warning(f"No parameters found for layer {layer_idx} with prefix {prefix}")
+        return
+    path = _layer_file(checkpoint_dir, layer_idx)
+    save_file(tensors, path)
+    meta = {"layer_idx": layer_idx, "total_layers": len(network.model.layers), "checkpoint_file": path,
+            "model_name": _CKPT_MODEL_NAME, "num_parameters": len(tensors), "parameter_names": list(tensors)}
+    with open(os.path.join(checkpoint_dir, f"{_CKPT_MODEL_NAME}_layer_{layer_idx}_metadata.json"), "w") as f:
+        json.dump(meta, f, indent=2)
+
+
+def detect_quantized_layers(checkpoint_dir: str | None) -> dict:
+    """checkpoint.py:75-91: {layer index: file} of the layer files present"""
+    found = {}
+    if checkpoint_dir is None or not os.path.isdir(checkpoint_dir):
+        return found
+    pat = re.compile(rf"^{_CKPT_MODEL_NAME}_layer_(\d+)\.safetensors$")
+    for fn in os.listdir(checkpoint_dir):
+        m = pat.match(fn)
+        if m:
+            found[int(m.group(1))] = os.path.join(checkpoint_dir, fn)
+    return found
+
+
+def auto_load_quantized_layers(network, checkpoint_dir: str | None) -> int:
+    """checkpoint.py:94-135: loads the layer files in ascending order of their index, stops at the first that fails,
+    returns the last index loaded (-1: none)"""
+    from safetensors.torch import load_file
+
+    last = -1
+    for idx, path in sorted(detect_quantized_layers(checkpoint_dir).items()):
+        try:
+            state = {f"model.layers.{idx}.{k}": v for k, v in load_file(path).items()}
+            network.load_state_dict(state, strict=False)
+        except Exception as e:  # a damaged file ends the resume, as in the reference
+            logging.warning(f"Failed to load layer {idx} ({e}), stopping auto-load")
+            break
+        last = idx
+    return last
+
+
 @torch.no_grad()
 def run_gptq(network, gptq_config):
     """run.py:20-232 for a ``transformers`` causal LM with ``network.model.layers`` / ``embed_tokens`` / ``norm`` /
@@ -186,8 +251,15 @@ def run_gptq(network, gptq_config):
     ``weight_config``, ``quantile_search``, ``clip_search_y``, ``cali_batch_size``, ``max_layers``) plus
     ``calibration_data``."""
     clip_search_y = gptq_config.get("clip_search_y", False)
-    if gptq_config.get("checkpoint_dir") is not None:
-        raise NotImplementedError("run_gptq: per-layer checkpoint files are not built")
+    checkpoint_dir = gptq_config.get("checkpoint_dir", None)
+    start_layer = 0
+    if checkpoint_dir is not None:  # run.py:64-74
+        start_layer = auto_load_quantized_layers(network, checkpoint_dir) + 1
+        if start_layer:
+            logging.info(f"Resuming GPTQ from layer {start_layer}")
+        if start_layer == len(network.model.layers):
+            logging.info("All layers already quantized, skipping GPTQ")
+            return network
     dev = gptq_config.get("device", "cuda:0")
     fmt = gptq_config["format"]
     weight_config = gptq_config["weight_config"]
@@ -233,9 +305,18 @@ def run_gptq(network, gptq_config):
     if position_ids is None:
         position_ids = torch.arange(seqlen, device=dev).unsqueeze(0)
 
-    end_layer = len(layers) if max_layers is None else min(max_layers, len(layers))
-    logging.info(f"GPTQ: quantizing layers 0 to {end_layer - 1} (of {len(layers)} total)")
-    for i in range(end_layer):
+    end_layer = len(layers) if max_layers is None else min(start_layer + max_layers, len(layers))
+    logging.info(f"GPTQ: quantizing layers {start_layer} to {end_layer - 1} (of {len(layers)} total)")
+    if start_layer and gptq_config.get("resume_propagate", False):
+        for i in range(start_layer):  # the loaded layers' outputs, not layer 0's inputs, feed the first new layer
+            layer = layers[i].to(dev)
+            for j in range(nsamples):
+                x = inps[j].unsqueeze(0)
+                cos, sin = rope(x, position_ids)
+                out = layer(x, attention_mask=attention_mask, position_embeddings=(cos, sin))
+                outs[j] = out[0] if isinstance(out, tuple) else out
+            inps, outs = outs, inps
+    for i in range(start_layer, end_layer):
         layer = layers[i].to(dev)
 
         def run_layer(j, layer=layer):
@@ -249,5 +330,6 @@ def run_gptq(network, gptq_config):
         for j in range(nsamples):  # run.py:197-205: the quantized layer's outputs feed the next layer
             run_layer(j)
         inps, outs = outs, inps
+        save_layer_checkpoint(network, i, checkpoint_dir)
     network.config.use_cache = use_cache
     return network

@@ -372,3 +372,37 @@ def test_layer_op_entry_points_reject_bad_arguments_without_a_gpu(lib):
     assert s(p, p, p, 63, 1, 0, 0, 1, 0, None) == -2
     assert s(p, p, p, 64, 3, 0, 0, 1, 0, None) == -4
     assert s(p, p, p, 64, 1, 4, 12, 1, 0, None) == -5
+
+
+def test_gptq_layer_checkpoint_files(tmp_path):
+    """the per-layer files of the GPTQ driver: names, contents, detection, loading in ascending order up to the first gap
+    or damaged file (host logic only)"""
+    import json
+
+    from safetensors.torch import load_file
+    from torch import nn
+
+    from mase_amd.passes.gptq import auto_load_quantized_layers, detect_quantized_layers, save_layer_checkpoint
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.model = nn.Module()
+            self.model.layers = nn.ModuleList([nn.Linear(4, 4) for _ in range(4)])
+
+    torch.manual_seed(0)
+    a, b = Net(), Net()
+    d = str(tmp_path / "ckpt")
+    assert detect_quantized_layers(d) == {} and auto_load_quantized_layers(b, d) == -1
+    for i in (0, 1, 3):
+        save_layer_checkpoint(a, i, d)
+    save_layer_checkpoint(a, 2, None)  # no directory: nothing is written
+    assert sorted(detect_quantized_layers(d)) == [0, 1, 3]
+    meta = json.load(open(f"{d}/quantized_model_layer_1_metadata.json"))
+    assert meta["layer_idx"] == 1 and meta["total_layers"] == 4 and meta["parameter_names"] == ["weight", "bias"]
+    assert torch.equal(load_file(f"{d}/quantized_model_layer_3.safetensors")["weight"], a.model.layers[3].weight)
+    with open(f"{d}/quantized_model_layer_1.safetensors", "wb") as f:
+        f.write(b"not a safetensors file")
+    assert auto_load_quantized_layers(b, d) == 0  # layer 1 is damaged: the resume stops there, as in the reference
+    assert torch.equal(b.model.layers[0].weight, a.model.layers[0].weight)
+    assert not torch.equal(b.model.layers[3].weight, a.model.layers[3].weight)

@@ -1,5 +1,6 @@
 """GPU tests of the GPTQ pre-pass: the per-layer algorithm against the CPU oracle, and the driver on a small causal LM."""
 import copy
+import os
 
 import pytest
 import torch
@@ -133,3 +134,48 @@ def test_run_gptq_on_a_small_causal_lm(dev):
     e_y = float((hidden(tuned_y) - ref).pow(2).mean())
     print(f"hidden-state MSE with clip_search_y: {e_y:.4e}")
     assert e_y < e_plain
+
+
+def test_run_gptq_layer_checkpoints_and_resume(dev, tmp_path):
+    """checkpoint_dir: one safetensors file + JSON description per finished layer, named as the reference names them;
+    a second run finds them, loads them and quantizes only what is left; when every layer is there it returns at once.
+    With resume_propagate the resumed run gives the weights of the uninterrupted run (the reference's driver, and the
+    default here, calibrates the first resumed layer on layer 0's inputs instead)."""
+    from safetensors.torch import load_file
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    from mase_amd.passes.gptq import detect_quantized_layers, run_gptq
+
+    torch.manual_seed(0)
+    cfg = LlamaConfig(hidden_size=128, intermediate_size=256, num_hidden_layers=3, num_attention_heads=4,
+                      num_key_value_heads=2, vocab_size=128, max_position_embeddings=128)
+    base = LlamaForCausalLM(cfg).to(dev).eval()
+    data = torch.randint(0, 128, (4, 32), generator=torch.Generator().manual_seed(1))
+    gcfg = {"model_name": "synthetic", "device": str(dev), "format": "mxint", "weight_config": MXINT4,
+            "calibration_data": data, "quantile_search": True}
+    full = run_gptq(copy.deepcopy(base), dict(gcfg))
+
+    d = str(tmp_path / "ckpt")
+    first = run_gptq(copy.deepcopy(base), {**gcfg, "checkpoint_dir": d, "max_layers": 2})
+    assert sorted(detect_quantized_layers(d)) == [0, 1]
+    assert sorted(os.listdir(d)) == ["quantized_model_layer_0.safetensors", "quantized_model_layer_0_metadata.json",
+                                     "quantized_model_layer_1.safetensors", "quantized_model_layer_1_metadata.json"]
+    saved = load_file(os.path.join(d, "quantized_model_layer_1.safetensors"))
+    assert set(saved) == {n for n, _ in base.model.layers[1].named_parameters()}
+    assert torch.equal(saved["mlp.down_proj.weight"], first.model.layers[1].mlp.down_proj.weight.cpu())
+    assert torch.equal(first.model.layers[1].mlp.down_proj.weight, full.model.layers[1].mlp.down_proj.weight)
+    assert torch.equal(first.model.layers[2].mlp.down_proj.weight, base.model.layers[2].mlp.down_proj.weight)
+
+    resumed = run_gptq(copy.deepcopy(base), {**gcfg, "checkpoint_dir": d, "resume_propagate": True})
+    assert sorted(detect_quantized_layers(d)) == [0, 1, 2]
+    for lr, lf in zip(resumed.model.layers, full.model.layers):
+        for (n, pr), (_, pf) in zip(lr.named_parameters(), lf.named_parameters()):
+            assert torch.equal(pr, pf), n
+    # everything is there now: nothing is computed (no calibration data is even looked at)
+    again = run_gptq(copy.deepcopy(base), {**gcfg, "checkpoint_dir": d, "calibration_data": None})
+    assert torch.equal(again.model.layers[2].mlp.down_proj.weight, full.model.layers[2].mlp.down_proj.weight)
+    # the reference's resume: layer 2 calibrated on the embedding outputs, so other weights than the straight run's
+    os.remove(os.path.join(d, "quantized_model_layer_2.safetensors"))
+    ref_style = run_gptq(copy.deepcopy(base), {**gcfg, "checkpoint_dir": d})
+    assert torch.equal(ref_style.model.layers[1].mlp.down_proj.weight, full.model.layers[1].mlp.down_proj.weight)
+    assert not torch.equal(ref_style.model.layers[2].mlp.down_proj.weight, full.model.layers[2].mlp.down_proj.weight)
