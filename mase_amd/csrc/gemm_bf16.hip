@@ -304,19 +304,20 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
             const int row = m0 + wm * 128 + i * 32 + q * 8 + kgrp * 4 + rl;
             if (row >= p.M) continue;
             const size_t o = (size_t)row * p.N + col0;
+            // streaming stores: the output is not read again by this kernel and should not displace operand panels
             if (vec_ok && col0 + 3 < p.N) {
               if constexpr (OUT_DT == MASE_DT_F32) {
-                *(float4*)((float*)Cs + o) = make_float4(v[0], v[1], v[2], v[3]);
+                store_nt((uint4*)((float*)Cs + o), make_uint4(f2bits(v[0]), f2bits(v[1]), f2bits(v[2]), f2bits(v[3])));
               } else if constexpr (OUT_DT == MASE_DT_BF16) {
                 uint2 w;
                 w.x = f32x2_to_bf16x2_bits(v[0], v[1]);
                 w.y = f32x2_to_bf16x2_bits(v[2], v[3]);
-                *(uint2*)((uint16_t*)Cs + o) = w;
+                store_nt((uint2*)((uint16_t*)Cs + o), w);
               } else {
                 uint2 w;
                 w.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
                 w.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
-                *(uint2*)((uint16_t*)Cs + o) = w;
+                store_nt((uint2*)((uint16_t*)Cs + o), w);
               }
             } else {
 #pragma unroll

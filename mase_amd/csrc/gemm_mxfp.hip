@@ -335,17 +335,17 @@ __global__ __launch_bounds__(kThreadsG) void gemm_mxfp_kernel(MxGemmParams p) {
         const size_t o = (size_t)row * p.N + col0;
         if (vec_ok && col0 + 3 < p.N) {
           if constexpr (OUT_DT == MASE_DT_F32) {
-            *(float4*)((float*)p.C + o) = make_float4(v[0], v[1], v[2], v[3]);
+            store_nt((uint4*)((float*)p.C + o), make_uint4(f2bits(v[0]), f2bits(v[1]), f2bits(v[2]), f2bits(v[3])));
           } else if constexpr (OUT_DT == MASE_DT_BF16) {
             uint2 w;
             w.x = f32x2_to_bf16x2_bits(v[0], v[1]);
             w.y = f32x2_to_bf16x2_bits(v[2], v[3]);
-            *(uint2*)((uint16_t*)p.C + o) = w;
+            store_nt((uint2*)((uint16_t*)p.C + o), w);
           } else {
             uint2 w;
             w.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
             w.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
-            *(uint2*)((uint16_t*)p.C + o) = w;
+            store_nt((uint2*)((uint16_t*)p.C + o), w);
           }
         } else {
 #pragma unroll
