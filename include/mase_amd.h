@@ -24,6 +24,8 @@
  *   mase_rope               nn/quantized/functional/rope.py:17-27 (_apply_rope)
  *   mase_rmsnorm_minifloat  nn/quantized/modules/llama/rms_norm.py:72-84 (LlamaRMSNormMinifloat.forward)
  *   mase_silu_mul_minifloat nn/quantized/modules/llama/mlp.py:60-62 (silu_minifloat(gate) * up)
+ *   mase_rmsnorm_mxint, mase_silu_mul_mxint   the two above followed by the consumer LinearMXInt's activation
+ *                           quantizer (nn/quantized/modules/linear.py:956-972) in the same pass
  *   mase_attn_softmax_mx    nn/quantized/modules/llama/attention.py:363-392 (scores -> quantized probabilities)
  *   mase_mx_unpack          nn/quantizers/mxint/fake.py:59-80, nn/quantizers/mxfp/fake.py:75-104 (compose_*)
  *   mase_mxfp_pack(_tiled), mase_mxfp_tile_codes, mase_gemm_mxfp_scaled, mase_gemm_mxfp4_scaled_tiled
@@ -307,6 +309,17 @@ int mase_rmsnorm_minifloat(const void* x, const void* weight, void* out, size_t 
  * (nn/quantized/modules/llama/mlp.py:60-62, nn/quantized/functional/silu.py:41-57). */
 int mase_silu_mul_minifloat(const void* gate, const void* up, void* out, size_t numel, int dtype, int exp_bits,
                             int frac_bits, int is_finite, int round_mode, void* stream);
+
+/* The same RMSNorm (casts off) and SwiGLU product (cast off) with the MXINT quantize-dequantize of the LinearMXInt that
+ * consumes the result applied to it before it is stored: out = mxint_quantizer(result, block 32 along the last
+ * dimension, element_bits), the arithmetic of mase_mxint_qdq on the result rounded to dtype, so out holds what that
+ * Linear's forward would compute from the stored result (nn/quantized/modules/linear.py:956-972 after
+ * models/llama/modeling_llama.py:79-93 / :219-236) and a pass over the tensor is saved.  cols % 32 == 0 (numel % 32 == 0),
+ * log2_tab as for mase_mxint_qdq in dtype. */
+int mase_rmsnorm_mxint(const void* x, const void* weight, void* out, size_t rows, size_t cols, int dtype, float eps,
+                       int element_bits, const uint32_t* log2_tab, void* stream);
+int mase_silu_mul_mxint(const void* gate, const void* up, void* out, size_t numel, int dtype, int element_bits,
+                        const uint32_t* log2_tab, void* stream);
 
 /* Rotary embedding out = x * cos + rotate_half(x) * sin for x [B, H, T, D] with the last dimension contiguous and
  * element strides (x_stride_b, x_stride_h, x_stride_t); out has the same strides; cos / sin tables [B or 1, T, D] with

@@ -5,10 +5,14 @@
 //   rope_minifloat applies to the small cos / sin tables and is done by the caller)
 //   SiLU(cast(gate)) * up (nn/quantized/modules/llama/mlp.py:60-62 with functional/silu.py:41-57; cast off: the plain
 //   SwiGLU product, models/llama/modeling_llama.py:219-236)
+// RMSNorm and the SwiGLU product can also hand their result on already MXINT-quantized (blocks of 32 along the last
+// dimension, the arithmetic of qdq_mxint's vector kernel on the values rounded to T): what the LinearMXInt that
+// consumes them would compute from the stored tensor in a pass of its own (nn/quantized/modules/linear.py:956-972).
 // Every intermediate is rounded to the tensor dtype T where the separate tensor operations would round it.  Both are
 // HBM-bound: the tensor is read once and written once, against 10-20 passes of the separate operations.
 #include "common.hpp"
 #include "minifloat_mx.hpp"
+#include "mxint_core.hpp"
 
 namespace mase {
 namespace {
@@ -28,7 +32,29 @@ struct RmsNormParams {
   int cols;  // multiple of 8, at most 8192
   float eps;
   CastSpec x_cast, w_cast;
+  MxintParams mx;  // MX instantiation only
 };
+
+// MXINT quantize-dequantize of the 8 values a lane has just produced (already rounded to T); a block of 32 is the 4
+// lanes of a group.  Every lane of the wavefront must take part (register permutes).
+template <int DT>
+__device__ __forceinline__ void mxint_block32(float* v, const MxintParams& q, const WaveLog2& meta) {
+  uint32_t mbits = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) mbits = max(mbits, f2bits(v[j]) & 0x7FFFFFFFu);
+  const uint32_t mx = group_max_u32<4>(mbits);
+  int k = 0, kc = 0;
+  const int state = block_exponent<DT>(mx, q, k, kc, meta);
+  if (state == 0) {
+    const int up = q.qshift - k, dn = kc - q.qshift;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = ldexpf(fminf(fmaxf(rintf(ldexpf(v[j], up)), q.lo), q.hi), dn);
+  } else {
+    int code;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = mxint_element<DT>(v[j], state, k, kc, q, code);
+  }
+}
 
 template <int DT>
 __device__ __forceinline__ void load_vec8(const void* base, size_t elem, float* x) {
@@ -62,13 +88,16 @@ __device__ __forceinline__ void cast8(float* v, const CastSpec& c) {
   for (int j = 0; j < 8; ++j) v[j] = DTypeTraits<DT>::round(y[j]);
 }
 
-// one wavefront per row; the row stays in registers (NCH chunks of 64 lanes x 8 elements)
-template <int DT, int NCH>
+// one wavefront per row; the row stays in registers (NCH chunks of 64 lanes x 8 elements).  MX: the output is the
+// MXINT quantize-dequantize of the normalised row (cols a multiple of 32)
+template <int DT, int NCH, bool MX = false>
 __global__ __launch_bounds__(kRowThreads) void rmsnorm_kernel(RmsNormParams p) {
   using TR = DTypeTraits<DT>;
   const int lane = (int)(threadIdx.x & 63);
   const size_t row = blockIdx.x;
   const size_t base = row * (size_t)p.cols;
+  WaveLog2 meta;
+  if constexpr (MX) meta.init(p.mx.tab, 0);
   float h[NCH][8];
   float ss = 0.0f;
 #pragma unroll
@@ -89,25 +118,37 @@ __global__ __launch_bounds__(kRowThreads) void rmsnorm_kernel(RmsNormParams p) {
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
     const int e0 = (c * 64 + lane) * 8;
-    if (e0 >= p.cols) continue;
+    const bool live = e0 < p.cols;
+    if constexpr (!MX) {
+      if (!live) continue;
+    }
     float w[8], y[8];
-    load_vec8<DT>(p.weight, (size_t)e0, w);
-    cast8<DT>(w, p.w_cast);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) w[j] = 0.0f;
+    if (live) {
+      load_vec8<DT>(p.weight, (size_t)e0, w);
+      cast8<DT>(w, p.w_cast);
+    }
 #pragma unroll
     for (int j = 0; j < 8; ++j) y[j] = w[j] * TR::round(h[c][j] * r);  // weight * hidden.to(dtype), rounded by the store
-    store_vec8<DT>(p.out, base + (size_t)e0, y);
+    if constexpr (MX) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) y[j] = TR::round(y[j]);
+      mxint_block32<DT>(y, p.mx, meta);
+    }
+    if (live) store_vec8<DT>(p.out, base + (size_t)e0, y);
   }
 }
 
-template <int DT>
+template <int DT, bool MX = false>
 int launch_rmsnorm(const RmsNormParams& p, hipStream_t st) {
   const int nch = (p.cols + 511) / 512;
   const dim3 grid((unsigned)p.rows), block(kRowThreads);
-  if (nch <= 1) hipLaunchKernelGGL((rmsnorm_kernel<DT, 1>), grid, block, 0, st, p);
-  else if (nch <= 2) hipLaunchKernelGGL((rmsnorm_kernel<DT, 2>), grid, block, 0, st, p);
-  else if (nch <= 4) hipLaunchKernelGGL((rmsnorm_kernel<DT, 4>), grid, block, 0, st, p);
-  else if (nch <= 8) hipLaunchKernelGGL((rmsnorm_kernel<DT, 8>), grid, block, 0, st, p);
-  else hipLaunchKernelGGL((rmsnorm_kernel<DT, 16>), grid, block, 0, st, p);
+  if (nch <= 1) hipLaunchKernelGGL((rmsnorm_kernel<DT, 1, MX>), grid, block, 0, st, p);
+  else if (nch <= 2) hipLaunchKernelGGL((rmsnorm_kernel<DT, 2, MX>), grid, block, 0, st, p);
+  else if (nch <= 4) hipLaunchKernelGGL((rmsnorm_kernel<DT, 4, MX>), grid, block, 0, st, p);
+  else if (nch <= 8) hipLaunchKernelGGL((rmsnorm_kernel<DT, 8, MX>), grid, block, 0, st, p);
+  else hipLaunchKernelGGL((rmsnorm_kernel<DT, 16, MX>), grid, block, 0, st, p);
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
 
@@ -117,23 +158,40 @@ struct SiluMulParams {
   void* out;
   size_t n8;
   CastSpec cast;
+  MxintParams mx;  // MX instantiation only
 };
 
 // silu(x) = x / (1 + exp(-x)) evaluated in fp32
 __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
 
-template <int DT>
+// MX: the output is the MXINT quantize-dequantize of the product (blocks of 32 consecutive elements: numel a multiple
+// of 32, so the 4 lanes of a block are live or dead together)
+template <int DT, bool MX = false>
 __global__ __launch_bounds__(kRowThreads) void silu_mul_kernel(SiluMulParams p) {
   using TR = DTypeTraits<DT>;
   const size_t i = (size_t)blockIdx.x * kRowThreads + threadIdx.x;
-  if (i >= p.n8) return;
+  const bool live = i < p.n8;
+  if constexpr (!MX) {
+    if (!live) return;
+  }
+  WaveLog2 meta;
+  if constexpr (MX) meta.init(p.mx.tab, 0);
   float g[8], u[8], y[8];
-  load_vec8<DT>(p.gate, i * 8, g);
-  load_vec8<DT>(p.up, i * 8, u);
-  cast8<DT>(g, p.cast);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) g[j] = u[j] = 0.0f;
+  if (live) {
+    load_vec8<DT>(p.gate, i * 8, g);
+    load_vec8<DT>(p.up, i * 8, u);
+    cast8<DT>(g, p.cast);
+  }
 #pragma unroll
   for (int j = 0; j < 8; ++j) y[j] = TR::round(silu_f32(g[j])) * u[j];
-  store_vec8<DT>(p.out, i * 8, y);
+  if constexpr (MX) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) y[j] = TR::round(y[j]);
+    mxint_block32<DT>(y, p.mx, meta);
+  }
+  if (live) store_vec8<DT>(p.out, i * 8, y);
 }
 
 struct RopeParams {
@@ -242,6 +300,69 @@ extern "C" int mase_silu_mul_minifloat(const void* gate, const void* up, void* o
     case MASE_DT_F32: hipLaunchKernelGGL((silu_mul_kernel<MASE_DT_F32>), grid, block, 0, st, p); break;
     case MASE_DT_BF16: hipLaunchKernelGGL((silu_mul_kernel<MASE_DT_BF16>), grid, block, 0, st, p); break;
     default: hipLaunchKernelGGL((silu_mul_kernel<MASE_DT_F16>), grid, block, 0, st, p); break;
+  }
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+namespace mase {
+namespace {
+bool fill_mxint(MxintParams& q, int element_bits, int dtype, const uint32_t* tab) {
+  if (element_bits < 2 || element_bits > 24 || tab == nullptr) return false;
+  q.qshift = element_bits - 1;
+  q.bias = 127;
+  q.scale_max = 255;
+  q.lo = mase_round_scalar_to_dtype(-(double)(1 << (element_bits - 1)), dtype);
+  q.hi = mase_round_scalar_to_dtype((double)((1 << (element_bits - 1)) - 1), dtype);
+  q.tab = tab;
+  return true;
+}
+}  // namespace
+}  // namespace mase
+
+extern "C" int mase_rmsnorm_mxint(const void* x, const void* weight, void* out, size_t rows, size_t cols, int dtype,
+                                  float eps, int element_bits, const uint32_t* log2_tab, void* stream) {
+  using namespace mase;
+  if (rows == 0 || cols == 0) return MASE_OK;
+  if (x == nullptr || weight == nullptr || out == nullptr || log2_tab == nullptr) return MASE_ERR_NULL;
+  if (cols % 32 != 0 || cols > 8192 || rows > 0x7FFFFFFFull) return MASE_ERR_SHAPE;
+  if (!aligned16(x) || !aligned16(weight) || !aligned16(out)) return MASE_ERR_ALIGN;
+  if (dtype < 0 || dtype > 2) return MASE_ERR_DTYPE;
+  RmsNormParams p{};
+  p.x = x;
+  p.weight = weight;
+  p.out = out;
+  p.rows = rows;
+  p.cols = (int)cols;
+  p.eps = eps;
+  if (!fill_mxint(p.mx, element_bits, dtype, log2_tab)) return MASE_ERR_PARAM;
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case MASE_DT_F32: return launch_rmsnorm<MASE_DT_F32, true>(p, st);
+    case MASE_DT_BF16: return launch_rmsnorm<MASE_DT_BF16, true>(p, st);
+    default: return launch_rmsnorm<MASE_DT_F16, true>(p, st);
+  }
+}
+
+extern "C" int mase_silu_mul_mxint(const void* gate, const void* up, void* out, size_t numel, int dtype,
+                                   int element_bits, const uint32_t* log2_tab, void* stream) {
+  using namespace mase;
+  if (numel == 0) return MASE_OK;
+  if (gate == nullptr || up == nullptr || out == nullptr || log2_tab == nullptr) return MASE_ERR_NULL;
+  if (numel % 32 != 0) return MASE_ERR_SHAPE;
+  if (!aligned16(gate) || !aligned16(up) || !aligned16(out)) return MASE_ERR_ALIGN;
+  if (dtype < 0 || dtype > 2) return MASE_ERR_DTYPE;
+  SiluMulParams p{};
+  p.gate = gate;
+  p.up = up;
+  p.out = out;
+  p.n8 = numel / 8;
+  if (!fill_mxint(p.mx, element_bits, dtype, log2_tab)) return MASE_ERR_PARAM;
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid(blocks_for(p.n8, (size_t)kRowThreads)), block(kRowThreads);
+  switch (dtype) {
+    case MASE_DT_F32: hipLaunchKernelGGL((silu_mul_kernel<MASE_DT_F32, true>), grid, block, 0, st, p); break;
+    case MASE_DT_BF16: hipLaunchKernelGGL((silu_mul_kernel<MASE_DT_BF16, true>), grid, block, 0, st, p); break;
+    default: hipLaunchKernelGGL((silu_mul_kernel<MASE_DT_F16, true>), grid, block, 0, st, p); break;
   }
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }

@@ -109,6 +109,23 @@ def project_shared(x: Tensor, modules) -> list:
     return outs
 
 
+def shared_mxint_width(x: Tensor, modules) -> int | None:
+    """The element width when every module would turn the bf16 tensor ``x`` into the same MXINT form with blocks of 32
+    on its way to the matrix cores (``activation_key``), else None.  A producer of ``x`` that can quantize what it
+    writes (``rmsnorm_mxint``, ``silu_mul_mxint``) then hands the modules that form directly:
+    ``m(xq, prepared=xq.reshape(-1, K))``: with ``prepared`` given, a module reads only the shape and dtype of its
+    first argument."""
+    if x.dtype != torch.bfloat16 or not modules:
+        return None
+    keys = {m.activation_key(x) if hasattr(m, "activation_key") else None for m in modules}
+    if len(keys) != 1:
+        return None
+    key = keys.pop()
+    if key is None or key[0] != "mxint" or key[1] != 32:
+        return None
+    return key[2]
+
+
 def _weight_key(weight: Tensor):
     return _tensor_key(weight)
 

@@ -351,6 +351,38 @@ def silu_mul_minifloat(gate: Tensor, up: Tensor, cast=None) -> Tensor:
     return out
 
 
+def rmsnorm_mxint(x: Tensor, weight: Tensor, eps: float, element_bits: int) -> Tensor:
+    """``mxint_quantizer(rmsnorm(x), block 32 along the last dimension, element_bits)`` in one pass
+    (``mase_rmsnorm_mxint``): the quantized activation the ``LinearMXInt`` modules after the norm would each compute
+    from the stored norm output.  The last dimension must be a multiple of 32."""
+    _lib.require_device(x, "rmsnorm_mxint")
+    lib = _lib.load()
+    assert rmsnorm_supported(x, weight) and x.shape[-1] % 32 == 0
+    xc = _contig(x)
+    w = weight.detach().contiguous()
+    out = torch.empty_like(xc)
+    cols = xc.shape[-1]
+    rc = lib.mase_rmsnorm_mxint(xc.data_ptr(), w.data_ptr(), out.data_ptr(), xc.numel() // cols, cols, _lib.dtype_code(xc),
+                                float(eps), int(element_bits), log2_table(xc.dtype, xc.device).data_ptr(),
+                                _lib.stream_ptr(xc))
+    _lib.check(rc, "mase_rmsnorm_mxint")
+    return out
+
+
+def silu_mul_mxint(gate: Tensor, up: Tensor, element_bits: int) -> Tensor:
+    """``mxint_quantizer(silu(gate) * up, block 32 along the last dimension, element_bits)`` in one pass
+    (``mase_silu_mul_mxint``); the last dimension must be a multiple of 32."""
+    _lib.require_device(gate, "silu_mul_mxint")
+    lib = _lib.load()
+    assert silu_mul_supported(gate, up) and gate.shape[-1] % 32 == 0
+    g, u = _contig(gate), _contig(up)
+    out = torch.empty_like(g)
+    rc = lib.mase_silu_mul_mxint(g.data_ptr(), u.data_ptr(), out.data_ptr(), g.numel(), _lib.dtype_code(g),
+                                 int(element_bits), log2_table(g.dtype, g.device).data_ptr(), _lib.stream_ptr(g))
+    _lib.check(rc, "mase_silu_mul_mxint")
+    return out
+
+
 def rope_supported(x: Tensor, cos: Tensor, sin: Tensor) -> bool:
     """x [B, H, T, D] (any strides with the last dimension contiguous), cos / sin [B or 1, T, D] or [T, D]"""
     if not (x.is_cuda and x.dim() == 4 and x.dtype in _lib.DTYPE_CODE and x.numel() > 0 and x.stride(3) == 1):

@@ -8,7 +8,9 @@ attention, ``:843-918`` layer with pre-norm residuals); no KV cache, no dropout,
 On the CPU everything except the seven Linears is ordinary torch, which is what lets the same class serve as the CPU
 reference once its Linears are swapped for reference ones; on the GPU (no gradient recorded) RMSNorm, the rotary
 embedding and the SwiGLU product run as one-pass kernels with the same arithmetic (``mase_rmsnorm_minifloat``,
-``mase_rope``, ``mase_silu_mul_minifloat`` with their casts off).
+``mase_rope``, ``mase_silu_mul_minifloat`` with their casts off); where the Linears that consume an RMSNorm or the
+SwiGLU product are MXINT Linears on the matrix-core path, those kernels write the quantized form the Linears would
+each compute (``mase_rmsnorm_mxint``, ``mase_silu_mul_mxint``), which saves a pass over the tensor.
 """
 from __future__ import annotations
 
@@ -19,7 +21,7 @@ from torch import nn
 from torch.nn import functional as F
 
 from ..quantizers import _ops
-from ..quantized.functional.mx_linear import project_shared
+from ..quantized.functional.mx_linear import project_shared, shared_mxint_width
 
 
 @dataclass
@@ -91,13 +93,28 @@ class DecoderLayer(nn.Module):
             w = getattr(self, name).weight
             w.copy_((torch.randn(w.shape, generator=g) * self.cfg.init_std).to(w.dtype))
 
+    # RMSNorm / the SwiGLU product write the quantized form MXINT Linears after them would compute (see
+    # _norm_then_project); False: every Linear receives the plain tensor and quantizes it itself
+    fuse_producers = True
+
+    def _norm_then_project(self, norm, x, modules):
+        """``[m(norm(x)) for m in modules]``.  Sibling projections of one tensor: quantized Linears that treat it alike
+        share one quantized copy, and when they are MXINT Linears on the matrix-core path the norm writes that copy
+        itself instead of a tensor each of them would read and quantize (same values: the quantizer's arithmetic on
+        the norm's rounded output)."""
+        if (self.fuse_producers and x.is_cuda and not torch.is_grad_enabled() and x.shape[-1] % 32 == 0
+                and _ops.rmsnorm_supported(x, norm.weight)):
+            bits = shared_mxint_width(x, modules)
+            if bits is not None:
+                hq = _ops.rmsnorm_mxint(x, norm.weight, norm.eps, bits)
+                return [m(hq, prepared=hq.reshape(-1, hq.shape[-1])) for m in modules]
+        return project_shared(norm(x), modules)
+
     def forward(self, x):
         cfg = self.cfg
         B, T, _ = x.shape
-        h = self.input_layernorm(x)
-        # sibling projections of one tensor: quantized Linears that treat it alike share one quantized copy
         q, k, v = (t.view(B, T, cfg.num_heads, cfg.head_dim).transpose(1, 2)
-                   for t in project_shared(h, (self.q_proj, self.k_proj, self.v_proj)))
+                   for t in self._norm_then_project(self.input_layernorm, x, (self.q_proj, self.k_proj, self.v_proj)))
         cos, sin = rope_tables(T, cfg.head_dim, cfg.rope_theta, x.device, x.dtype)
         if q.is_cuda and _ops.rope_supported(q, cos, sin) and _ops.rope_supported(k, cos, sin):
             q, k = _ops.rope(q, cos, sin), _ops.rope(k, cos, sin)  # the same products and sum in one pass
@@ -107,9 +124,12 @@ class DecoderLayer(nn.Module):
         a = self.attention_fn(q, k, v)
         a = a.transpose(1, 2).reshape(B, T, cfg.num_heads * cfg.head_dim)
         x = x + self.o_proj(a)
-        h = self.post_attention_layernorm(x)
-        gate, up = project_shared(h, (self.gate_proj, self.up_proj))
+        gate, up = self._norm_then_project(self.post_attention_layernorm, x, (self.gate_proj, self.up_proj))
         if gate.is_cuda and _ops.silu_mul_supported(gate, up):
+            bits = shared_mxint_width(gate, (self.down_proj,)) if self.fuse_producers and gate.shape[-1] % 32 == 0 else None
+            if bits is not None and not torch.is_grad_enabled():
+                actq = _ops.silu_mul_mxint(gate, up, bits)  # the product, already in down_proj's quantized form
+                return x + self.down_proj(actq, prepared=actq.reshape(-1, actq.shape[-1]))
             act = _ops.silu_mul_minifloat(gate, up)  # silu(gate) * up in one pass
         else:
             act = F.silu(gate) * up

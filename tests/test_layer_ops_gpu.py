@@ -118,3 +118,30 @@ def test_project_shared_quantizes_once_per_quantizer(dev, monkeypatch):
     n = len(calls)
     project_shared(x, mods + [other])                    # another activation format gets its own copy
     assert len(calls) == n + 2
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("bits", [8, 4])
+def test_norm_and_silu_product_written_in_the_consumers_mxint_form(dev, dtype, bits):
+    """mase_rmsnorm_mxint / mase_silu_mul_mxint: bit for bit the MXINT quantizer (checked against the oracle elsewhere)
+    applied to what the unquantized kernels store; rows of awkward lengths, blocks of zeros, huge and tiny blocks"""
+    from mase_amd.quantizers import _ops
+    from helpers import assert_bits_equal
+
+    g = torch.Generator().manual_seed(5 + bits)
+    for rows, cols in ((37, 4096), (5, 32), (3, 5120), (130, 96), (2, 8192)):
+        x = (torch.randn(rows, cols, generator=g) * 1.7).to(dtype)
+        x[0, :32] = 0
+        x[1 % rows, 32:64] *= 1e-3
+        w = (1.0 + 0.2 * torch.randn(cols, generator=g)).to(dtype)
+        w[:32] = 0  # a block of zeros after the norm
+        xd, wd = x.to(dev), w.to(dev)
+        want = _ops.mxint_qdq(_ops.rmsnorm_minifloat(xd, wd, 1e-6), 32, bits, -1, 8)
+        assert_bits_equal(_ops.rmsnorm_mxint(xd, wd, 1e-6, bits), want, f"rmsnorm_mxint {dtype} {rows}x{cols}")
+        gate = (torch.randn(rows, cols, generator=g) * 3).to(dtype)
+        up = torch.randn(rows, cols, generator=g).to(dtype)
+        gate[0, :8] = torch.tensor([0.0, -0.0, 30.0, -30.0, 88.0, -88.0, 1e-3, -1e-3]).to(dtype)
+        up[-1, -32:] *= 1e4 if dtype != torch.float16 else 50.0
+        gd, ud = gate.to(dev), up.to(dev)
+        want = _ops.mxint_qdq(_ops.silu_mul_minifloat(gd, ud), 32, bits, -1, 8)
+        assert_bits_equal(_ops.silu_mul_mxint(gd, ud, bits), want, f"silu_mul_mxint {dtype} {rows}x{cols}")
