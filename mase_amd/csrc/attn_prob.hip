@@ -17,6 +17,7 @@
 #include "minifloat_mx.hpp"
 #include "mxfp_core.hpp"
 #include "mxint_core.hpp"
+#include "pk16_cast.hpp"
 
 namespace mase {
 namespace {
@@ -35,6 +36,8 @@ struct AttnProbParams {
   float scaling;
   int cast_on;          // 0: softmax on the masked scores as they are
   MinifloatMxFmt cast;
+  int pk_on;            // 16-bit T: the cast runs on packed 16-bit patterns (pk16_cast.hpp) with these parameters
+  Pk16CastParams pk;
   int mx_kind;          // 0 none, 1 MXINT, 2 MXFP
   MxintParams qi;
   MxfpParams qf;
@@ -106,10 +109,40 @@ __global__ __launch_bounds__(kRowThreads) void attn_prob_kernel(AttnProbParams p
       s[j] = v;
     }
     if (p.cast_on) {
-      float y[8];
-      minifloat_mx_qdq8(s, y, p.cast);
+      bool done = false;
+      if constexpr (DT != MASE_DT_F32) {
+        if (p.pk_on) {  // the masked scores are values of T: cast their bit patterns two per register
+          constexpr int MB = (DT == MASE_DT_BF16) ? 7 : 10;
+          uint4 v;
+          if constexpr (DT == MASE_DT_BF16) {
+            v = make_uint4(pack_bf16_exact(s[0], s[1]), pack_bf16_exact(s[2], s[3]), pack_bf16_exact(s[4], s[5]),
+                           pack_bf16_exact(s[6], s[7]));
+          } else {
+            v = TR::pack(s);
+          }
+          const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+          uint32_t r[4];
+          u16x2 lo_acc = as_u16x2(0xFFFFFFFFu), hi_acc = as_u16x2(0u);
+          if (p.pk.sub) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) s[j] = TR::round(y[j]);
+            for (int j = 0; j < 4; ++j) r[j] = pk16_cast<MB, true>(w[j], p.pk.f, p.pk.r, lo_acc, hi_acc);
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) r[j] = pk16_cast<MB, false>(w[j], p.pk.f, p.pk.r, lo_acc, hi_acc);
+          }
+          const uint32_t lo = min((uint32_t)lo_acc.x, (uint32_t)lo_acc.y), hi = max((uint32_t)hi_acc.x, (uint32_t)hi_acc.y);
+          const uint32_t lowest = p.pk.sub ? (1u << MB) : p.pk.lo_thr;
+          // a lane with an element outside the packed form's domain takes the step-by-step cast below
+          done = !(lo + 1u < lowest || hi >= p.pk.hi_thr);
+          if (done) TR::unpack(make_uint4(r[0], r[1], r[2], r[3]), s);
+        }
+      }
+      if (!done) {
+        float y[8];
+        minifloat_mx_qdq8(s, y, p.cast);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s[j] = TR::round(y[j]);
+      }
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -228,6 +261,8 @@ extern "C" int mase_attn_softmax_mx(const void* scores, const void* mask, void* 
     p.cast.frac_hi = (1 << cast_frac_bits) - 1;
     p.cast.is_finite = cast_is_finite;
     p.cast.round_mode = cast_round_mode;
+    if (dtype == MASE_DT_BF16) p.pk_on = make_pk16_cast_params<MASE_DT_BF16>(p.cast, p.pk) ? 1 : 0;
+    else if (dtype == MASE_DT_F16) p.pk_on = make_pk16_cast_params<MASE_DT_F16>(p.cast, p.pk) ? 1 : 0;
   }
   p.mx_kind = mx_kind;
   if (mx_kind == 1) {
