@@ -110,12 +110,20 @@ class DecoderLayer(nn.Module):
                 return [m(hq, prepared=hq.reshape(-1, hq.shape[-1])) for m in modules]
         return project_shared(norm(x), modules)
 
+    def _rope_tables(self, T, device, dtype):
+        """the cos / sin tables of the rotary embedding depend on (sequence length, device, dtype) only: kept from one
+        forward to the next (a model computes them once per forward for all its layers)"""
+        key = (T, device, dtype)
+        if getattr(self, "_rope_key", None) != key:
+            self._rope_key, self._rope_val = key, rope_tables(T, self.cfg.head_dim, self.cfg.rope_theta, device, dtype)
+        return self._rope_val
+
     def forward(self, x):
         cfg = self.cfg
         B, T, _ = x.shape
         q, k, v = (t.view(B, T, cfg.num_heads, cfg.head_dim).transpose(1, 2)
                    for t in self._norm_then_project(self.input_layernorm, x, (self.q_proj, self.k_proj, self.v_proj)))
-        cos, sin = rope_tables(T, cfg.head_dim, cfg.rope_theta, x.device, x.dtype)
+        cos, sin = self._rope_tables(T, x.device, x.dtype)
         if q.is_cuda and _ops.rope_supported(q, cos, sin) and _ops.rope_supported(k, cos, sin):
             q, k = _ops.rope(q, cos, sin), _ops.rope(k, cos, sin)  # the same products and sum in one pass
         else:
