@@ -1,0 +1,7 @@
+// The MXFP clip-search kernels for blocks of 64: one translation unit per family and block size, see
+// clip_search_kernels.hpp.
+#include "clip_search_kernels.hpp"
+
+namespace mase {
+MASE_CLIP_DEFINE_MXFP(64)
+}  // namespace mase
