@@ -27,6 +27,7 @@
  *   mase_rmsnorm_mxint, mase_silu_mul_mxint   the two above followed by the consumer LinearMXInt's activation
  *                           quantizer (nn/quantized/modules/linear.py:956-972) in the same pass
  *   mase_attn_softmax_mx    nn/quantized/modules/llama/attention.py:363-392 (scores -> quantized probabilities)
+ *   mase_attention_causal   models/llama/modeling_llama.py:362-480 (the attention core on unquantized q, k, v)
  *   mase_mx_unpack          nn/quantizers/mxint/fake.py:59-80, nn/quantizers/mxfp/fake.py:75-104 (compose_*)
  *   mase_mxfp_pack(_tiled), mase_mxfp_tile_codes, mase_gemm_mxfp_scaled, mase_gemm_mxfp4_scaled_tiled
  *                           nn/quantized/modules/linear.py:877-895 (LinearMXFP.forward on
@@ -320,6 +321,19 @@ int mase_rmsnorm_mxint(const void* x, const void* weight, void* out, size_t rows
                        int element_bits, const uint32_t* log2_tab, void* stream);
 int mase_silu_mul_mxint(const void* gate, const void* up, void* out, size_t numel, int dtype, int element_bits,
                         const uint32_t* log2_tab, void* stream);
+
+/* Causal self-attention core out = softmax(q k^T * scaling + causal mask) v for bf16 q, k, v [batch, heads, tokens, 128]
+ * given by element strides of batch / head / token (last dimension contiguous, strides multiples of 8), out likewise;
+ * tokens % 128 == 0.  Scores and softmax statistics in fp32, probabilities rounded to bf16 before the product with v
+ * (as the tensor operations of the reference's Llama attention core do on unquantized operands,
+ * models/llama/modeling_llama.py:362-480); no [tokens, tokens] matrix is materialised.  workspace: at least
+ * mase_attention_causal_workspace_bytes bytes (v transposed), 16-byte aligned; 0 from that function = unsupported. */
+size_t mase_attention_causal_workspace_bytes(size_t batch, size_t heads, size_t tokens, size_t head_dim);
+int mase_attention_causal(const void* q, const void* k, const void* v, void* out, size_t batch, size_t heads,
+                          size_t tokens, size_t head_dim, size_t q_stride_b, size_t q_stride_h, size_t q_stride_t,
+                          size_t k_stride_b, size_t k_stride_h, size_t k_stride_t, size_t v_stride_b, size_t v_stride_h,
+                          size_t v_stride_t, size_t o_stride_b, size_t o_stride_h, size_t o_stride_t, int dtype,
+                          float scaling, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Rotary embedding out = x * cos + rotate_half(x) * sin for x [B, H, T, D] with the last dimension contiguous and
  * element strides (x_stride_b, x_stride_h, x_stride_t); out has the same strides; cos / sin tables [B or 1, T, D] with

@@ -1,0 +1,285 @@
+// Causal self-attention core of the decoder layer for gfx950: out = softmax(q k^T * scaling + causal mask) v, bf16
+// operands, head dimension 128, fp32 softmax statistics and accumulators, in one pass over the keys (no [T, T] score
+// matrix in memory).  Semantics of the reference's Llama attention core on unquantized q / k / v
+// (models/llama/modeling_llama.py:362-480: scores in the model dtype, fp32 softmax, probabilities cast back to the
+// model dtype before the product with v); here the probabilities are rounded to bf16 before that product too, and the
+// row sum divides once at the end, so results agree with the tensor operations to bf16 rounding, not bit for bit.
+//
+// One work-group (4 wavefronts) owns 128 queries of one (batch, head); a wavefront owns 32 of them.  Key blocks of 64
+// are streamed through LDS (K as [key][128 d], V transposed as [d][64 keys], both double-buffered with async copies).
+// Per key block a wavefront computes S^T = K Q^T with v_mfma_f32_32x32x16_bf16 (A = K rows from LDS, B = its Q
+// fragments, kept in registers for the whole kernel): a lane then holds, for ONE query (lane % 32), the scores of 32 of
+// the 64 keys in its accumulator registers, so the softmax statistics are in-lane but for one exchange with lane ^ 32.
+// exp2 of the scaled scores gives P^T, which is already laid out as the B operand of O^T += V^T P^T (the matrix
+// instruction's 8 contraction slots of lane group g at step s are accumulator registers 8 (s % 2) .. + 7 of score tile
+// s / 2, i.e. keys 32 (s / 2) + 8 (2 (s % 2) + j / 4) + 4 g + j % 4: the V^T fragments are read from LDS in the same
+// key order, two 8-byte pieces each).  Two work-groups fit a CU (66 KB of LDS, under 256 registers), so one
+// wavefront's exponentials overlap the other's matrix instructions.
+//
+// V^T is made by a transposing pre-pass into a caller workspace [batch * heads][128][T].
+#include "common.hpp"
+
+namespace mase {
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+constexpr int kQB = 128, kKB = 64, kHD = 128;
+constexpr int kKBytes = kKB * kHD * 2;       // 16 KB: 64 key rows of 256 bytes
+constexpr int kVGroup = 8 * 128 + 16;        // 8 rows (d) of 128 bytes (64 keys) + 16 bytes that stagger the groups' banks
+constexpr int kVBytes = 16 * kVGroup;
+constexpr int kAttnLds = 2 * kKBytes + 2 * kVBytes;
+
+// lane i's 16 bytes at base + off_i land at LDS address lds_addr + 16 * i; tracked by hand with at_wait_vmcnt
+__device__ __forceinline__ void at_async_copy_16(const unsigned char* base, uint32_t off, uint32_t lds_addr) {
+  const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_addr);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void at_wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8) | ((N >> 4) << 14));
+}
+
+struct AttnParams {
+  const unsigned char* q;
+  const unsigned char* k;
+  const unsigned char* vt;  // [batch * heads][128][T] bf16
+  unsigned char* out;
+  int BH, H, T;
+  size_t q_sb, q_sh, k_sb, k_sh, o_sb, o_sh;  // byte strides of batch and head
+  uint32_t q_st, k_st, o_st;                  // byte strides of a token
+  float c;                                    // scaling * log2(e)
+};
+
+__global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  const int l32 = lane & 31, g = lane >> 5;
+  // the query blocks with the most keys first
+  const int n_qb = p.T / kQB;
+  const int qb = n_qb - 1 - (int)blockIdx.x / p.BH;
+  const int bh = (int)blockIdx.x % p.BH;
+  const int b = bh / p.H, h = bh % p.H;
+  const unsigned char* qp = p.q + (size_t)b * p.q_sb + (size_t)h * p.q_sh;
+  const unsigned char* kp = p.k + (size_t)b * p.k_sb + (size_t)h * p.k_sh;
+  const unsigned char* vtp = p.vt + (size_t)bh * ((size_t)kHD * p.T * 2);
+  const int q0 = qb * kQB + wave * 32;  // this wavefront's first query
+  const int qi = q0 + l32;              // this lane's query
+
+  bf16x8_t qf[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) qf[s] = *(const bf16x8_t*)(qp + (size_t)qi * p.q_st + (s * 16 + g * 8) * 2);
+
+  // async copies of one key block: 4 of K (4 rows of 256 bytes each) and 4 of V^T (8 rows of 128 bytes) per wavefront.
+  // LDS position (row, 16-byte slot) holds the row's chunk slot ^ (row % 16) (K) / slot ^ (row % 8) (V^T), so that the
+  // fragment reads of 32 lanes (32 rows, same chunk) spread over the banks.
+  uint32_t koff[4], voff[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int krow = (wave * 4 + i) * 4 + (lane >> 4);
+    koff[i] = (uint32_t)krow * p.k_st + (uint32_t)(((lane & 15) ^ (krow & 15)) << 4);
+    const int d = (wave * 4 + i) * 8 + (lane >> 3);
+    voff[i] = (uint32_t)d * (uint32_t)(p.T * 2) + (uint32_t)(((lane & 7) ^ (d & 7)) << 4);
+  }
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;
+  auto issue = [&](int j) __attribute__((always_inline)) {
+    const unsigned char* kb = kp + (size_t)j * kKB * p.k_st;
+    const unsigned char* vb = vtp + (size_t)j * kKB * 2;
+    const uint32_t kdst = lds_base + (uint32_t)((j & 1) * kKBytes), vdst = lds_base + (uint32_t)(2 * kKBytes + (j & 1) * kVBytes);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      at_async_copy_16(kb, koff[i], kdst + (uint32_t)((wave * 4 + i) * 1024));
+      at_async_copy_16(vb, voff[i], vdst + (uint32_t)((wave * 4 + i) * kVGroup));
+    }
+  };
+
+  f32x16_t o[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[dt][r] = 0.0f;
+  float m = -__builtin_inff(), lsum = 0.0f;
+
+  const int nblk = 2 * qb + 2;  // key blocks that hold a key <= the block's last query
+  issue(0);
+  for (int j = 0; j < nblk; ++j) {
+    at_wait_vmcnt<0>();  // this wavefront's copies of block j have landed
+    asm volatile("s_barrier" ::: "memory");  // ... everyone's have, and everyone has finished with block j - 1's buffers
+    if (j + 1 < nblk) issue(j + 1);
+    const int key0 = j * kKB;
+    if (key0 > q0 + 31) continue;  // every key of the block lies after every query of this wavefront
+    const unsigned char* Kb = lds + (j & 1) * kKBytes;
+    const unsigned char* Vb = lds + 2 * kKBytes + (j & 1) * kVBytes;
+
+    f32x16_t sc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[t][r] = 0.0f;
+      const int row = t * 32 + l32;
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        const bf16x8_t kf = *(const bf16x8_t*)(Kb + row * 256 + (((2 * s + g) ^ (row & 15)) << 4));
+        sc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sc[t], 0, 0, 0);
+      }
+    }
+    // register r of tile t is key key0 + 32 t + 8 (r / 4) + 4 g + r % 4
+    if (key0 + kKB - 1 > q0) {  // the block reaches past this wavefront's first query: mask
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = key0 + 32 * t + 8 * (r >> 2) + 4 * g + (r & 3);
+          if (key > qi) sc[t][r] = -__builtin_inff();
+        }
+    }
+    float mx = m;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sc[t][r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));  // finite: key0 <= q0 <= this lane's query, so key0 itself is not masked
+    const float alpha = __builtin_amdgcn_exp2f((m - mx) * p.c);
+    m = mx;
+    const float mc = mx * p.c;
+    float psum = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        sc[t][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[t][r], p.c, -mc));
+        psum += sc[t][r];
+      }
+    lsum = lsum * alpha + psum;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int t = s >> 1, r0 = (s & 1) * 8;
+      uint4 pw;
+      pw.x = f32x2_to_bf16x2_bits(sc[t][r0 + 0], sc[t][r0 + 1]);
+      pw.y = f32x2_to_bf16x2_bits(sc[t][r0 + 2], sc[t][r0 + 3]);
+      pw.z = f32x2_to_bf16x2_bits(sc[t][r0 + 4], sc[t][r0 + 5]);
+      pw.w = f32x2_to_bf16x2_bits(sc[t][r0 + 6], sc[t][r0 + 7]);
+      const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pw);
+      const int kbyte = (32 * t + 16 * (s & 1) + 4 * g) * 2;  // first of this lane group's keys, then 8 keys further
+      const int gran = kbyte >> 4, half = (kbyte & 15);
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) {
+        const int d = dt * 32 + l32;
+        const unsigned char* vrow = Vb + (d >> 3) * kVGroup + (d & 7) * 128;
+        const uint2 v0 = *(const uint2*)(vrow + ((gran ^ (d & 7)) << 4) + half);
+        const uint2 v1 = *(const uint2*)(vrow + (((gran + 1) ^ (d & 7)) << 4) + half);
+        const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, make_uint4(v0.x, v0.y, v1.x, v1.y));
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, o[dt], 0, 0, 0);
+      }
+    }
+  }
+  at_wait_vmcnt<0>();
+  lsum += __shfl_xor(lsum, 32, 64);
+  const float inv = 1.0f / lsum;
+  // register r of tile dt is d = 32 dt + 8 (r / 4) + 4 g + r % 4: four consecutive d per group of four registers
+  unsigned char* op = p.out + (size_t)b * p.o_sb + (size_t)h * p.o_sh + (size_t)qi * p.o_st;
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int qq = 0; qq < 4; ++qq) {
+      uint2 w;
+      w.x = f32x2_to_bf16x2_bits(o[dt][4 * qq] * inv, o[dt][4 * qq + 1] * inv);
+      w.y = f32x2_to_bf16x2_bits(o[dt][4 * qq + 2] * inv, o[dt][4 * qq + 3] * inv);
+      *(uint2*)(op + (32 * dt + 8 * qq + 4 * g) * 2) = w;
+    }
+}
+
+// vt[bh][d][t] = v[b][t][h][d]: tiles of 64 tokens x 128 d through LDS (rows padded to 264 bytes)
+__global__ __launch_bounds__(256) void attn_transpose_v_kernel(const unsigned char* __restrict__ v, unsigned char* __restrict__ vt,
+                                                               int H, int T, size_t v_sb, size_t v_sh, uint32_t v_st) {
+  __shared__ __attribute__((aligned(16))) unsigned char tile[64 * 264];
+  const int bh = blockIdx.y, t0 = blockIdx.x * 64;
+  const int b = bh / H, h = bh % H;
+  const unsigned char* src = v + (size_t)b * v_sb + (size_t)h * v_sh + (size_t)t0 * v_st;
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {  // 1024 chunks of 16 bytes: token = chunk / 16, slot = chunk % 16
+    const int c = i * 256 + tid, tok = c >> 4, slot = c & 15;
+    *(uint4*)(tile + tok * 264 + slot * 16) = *(const uint4*)(src + (size_t)tok * v_st + slot * 16);
+  }
+  __syncthreads();
+  unsigned char* dst = vt + (size_t)bh * ((size_t)kHD * T * 2) + (size_t)t0 * 2;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {  // 1024 pieces of 8 tokens: d = piece / 8, token group = piece % 8
+    const int c = i * 256 + tid, d = c >> 3, tg = c & 7;
+    uint32_t w[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t lo = *(const uint16_t*)(tile + (tg * 8 + 2 * e) * 264 + d * 2);
+      const uint32_t hi = *(const uint16_t*)(tile + (tg * 8 + 2 * e + 1) * 264 + d * 2);
+      w[e] = lo | (hi << 16);
+    }
+    *(uint4*)(dst + (size_t)d * T * 2 + tg * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
+
+}  // namespace
+}  // namespace mase
+
+extern "C" size_t mase_attention_causal_workspace_bytes(size_t batch, size_t heads, size_t tokens, size_t head_dim) {
+  if (head_dim != 128 || tokens == 0 || tokens % 128 != 0) return 0;
+  return batch * heads * tokens * head_dim * 2;
+}
+
+extern "C" int mase_attention_causal(const void* q, const void* k, const void* v, void* out, size_t batch, size_t heads,
+                                     size_t tokens, size_t head_dim, size_t q_stride_b, size_t q_stride_h,
+                                     size_t q_stride_t, size_t k_stride_b, size_t k_stride_h, size_t k_stride_t,
+                                     size_t v_stride_b, size_t v_stride_h, size_t v_stride_t, size_t o_stride_b,
+                                     size_t o_stride_h, size_t o_stride_t, int dtype, float scaling, void* workspace,
+                                     size_t workspace_bytes, void* stream) {
+  using namespace mase;
+  if (batch == 0 || heads == 0 || tokens == 0) return MASE_OK;
+  if (q == nullptr || k == nullptr || v == nullptr || out == nullptr) return MASE_ERR_NULL;
+  if (dtype != MASE_DT_BF16) return MASE_ERR_DTYPE;
+  if (head_dim != 128 || tokens % 128 != 0 || tokens > (1u << 20) || batch * heads > (1u << 20)) return MASE_ERR_SHAPE;
+  // strides in elements; rows of 128 elements must be whole 16-byte chunks, a token stride must fit 32 bits in bytes
+  const size_t strides[12] = {q_stride_b, q_stride_h, q_stride_t, k_stride_b, k_stride_h, k_stride_t,
+                              v_stride_b, v_stride_h, v_stride_t, o_stride_b, o_stride_h, o_stride_t};
+  for (size_t s : strides)
+    if (s % 8 != 0) return MASE_ERR_ALIGN;
+  if (q_stride_t < 128 || k_stride_t < 128 || v_stride_t < 128 || o_stride_t < 128) return MASE_ERR_SHAPE;
+  if (k_stride_t * 2 * tokens > 0xFFFFFFFFull || q_stride_t * 2 > 0xFFFFFFFFull || o_stride_t * 2 > 0xFFFFFFFFull ||
+      v_stride_t * 2 > 0xFFFFFFFFull)
+    return MASE_ERR_SHAPE;
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return MASE_ERR_ALIGN;
+  const size_t need = mase_attention_causal_workspace_bytes(batch, heads, tokens, head_dim);
+  if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace)) return MASE_ERR_WORKSPACE;
+  hipStream_t st = (hipStream_t)stream;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)attn_causal_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLds) !=
+        hipSuccess)
+      return MASE_ERR_LAUNCH;
+    attr_set = true;
+  }
+  const int BH = (int)(batch * heads), T = (int)tokens;
+  hipLaunchKernelGGL(attn_transpose_v_kernel, dim3((unsigned)(T / 64), (unsigned)BH), dim3(256), 0, st,
+                     (const unsigned char*)v, (unsigned char*)workspace, (int)heads, T, v_stride_b * 2, v_stride_h * 2,
+                     (uint32_t)(v_stride_t * 2));
+  AttnParams p;
+  p.q = (const unsigned char*)q;
+  p.k = (const unsigned char*)k;
+  p.vt = (const unsigned char*)workspace;
+  p.out = (unsigned char*)out;
+  p.BH = BH;
+  p.H = (int)heads;
+  p.T = T;
+  p.q_sb = q_stride_b * 2; p.q_sh = q_stride_h * 2; p.q_st = (uint32_t)(q_stride_t * 2);
+  p.k_sb = k_stride_b * 2; p.k_sh = k_stride_h * 2; p.k_st = (uint32_t)(k_stride_t * 2);
+  p.o_sb = o_stride_b * 2; p.o_sh = o_stride_h * 2; p.o_st = (uint32_t)(o_stride_t * 2);
+  p.c = scaling * 1.4426950408889634f;
+  hipLaunchKernelGGL(attn_causal_fwd_kernel, dim3((unsigned)(BH * (T / kQB))), dim3(256), kAttnLds, st, p);
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}

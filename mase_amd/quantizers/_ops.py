@@ -383,6 +383,45 @@ def silu_mul_mxint(gate: Tensor, up: Tensor, element_bits: int) -> Tensor:
     return out
 
 
+def attention_causal_supported(q: Tensor, k: Tensor, v: Tensor) -> bool:
+    """q, k, v [batch, heads, tokens, 128] bf16 on one device, last dimension contiguous, strides multiples of 8,
+    tokens a multiple of 128, no gradient recorded"""
+    if not (q.is_cuda and q.dim() == 4 and q.dtype == torch.bfloat16 and q.shape == k.shape == v.shape):
+        return False
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+        return False
+    B, H, T, D = q.shape
+    if D != 128 or T == 0 or T % 128 != 0 or B * H == 0:
+        return False
+    for t in (q, k, v):
+        if t.dtype != torch.bfloat16 or t.device != q.device or t.stride(3) != 1 or t.data_ptr() % 16:
+            return False
+        if any(s % 8 for s in t.stride()[:3]) or t.stride(2) < 128 or t.stride(2) * 2 * T > 0xFFFFFFFF:
+            return False
+    return True
+
+
+def attention_causal(q: Tensor, k: Tensor, v: Tensor, scaling: float | None = None) -> Tensor:
+    """``softmax(q k^T * scaling + causal mask) v`` for bf16 [batch, heads, tokens, 128] operands in one pass over the keys
+    (``mase_attention_causal``).  Returned as [batch, heads, tokens, 128] over memory laid out [batch, tokens, heads,
+    128], so that ``out.transpose(1, 2).reshape(batch, tokens, heads * 128)`` is a view."""
+    _lib.require_device(q, "attention_causal")
+    lib = _lib.load()
+    assert attention_causal_supported(q, k, v)
+    B, H, T, D = q.shape
+    if scaling is None:
+        scaling = D ** -0.5
+    out = torch.empty((B, T, H, D), dtype=q.dtype, device=q.device).transpose(1, 2)
+    need = lib.mase_attention_causal_workspace_bytes(B, H, T, D)
+    ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+    rc = lib.mase_attention_causal(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, H, T, D,
+                                   q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+                                   v.stride(0), v.stride(1), v.stride(2), out.stride(0), out.stride(1), out.stride(2),
+                                   _lib.dtype_code(q), float(scaling), ws.data_ptr(), need, _lib.stream_ptr(q))
+    _lib.check(rc, "mase_attention_causal")
+    return out
+
+
 def rope_supported(x: Tensor, cos: Tensor, sin: Tensor) -> bool:
     """x [B, H, T, D] (any strides with the last dimension contiguous), cos / sin [B or 1, T, D] or [T, D]"""
     if not (x.is_cuda and x.dim() == 4 and x.dtype in _lib.DTYPE_CODE and x.numel() > 0 and x.stride(3) == 1):

@@ -6,8 +6,9 @@ Semantics follow the reference's Llama block (``chop/models/llama/modeling_llama
 185-216`` rotary embedding with ``rotate_half``, ``:219-236`` MLP ``down(silu(gate(x)) * up(x))``, ``:362-480``
 attention, ``:843-918`` layer with pre-norm residuals); no KV cache, no dropout, no attention bias.
 On the CPU everything except the seven Linears is ordinary torch, which is what lets the same class serve as the CPU
-reference once its Linears are swapped for reference ones; on the GPU (no gradient recorded) RMSNorm, the rotary
-embedding and the SwiGLU product run as one-pass kernels with the same arithmetic (``mase_rmsnorm_minifloat``,
+reference once its Linears are swapped for reference ones; on the GPU (no gradient recorded) the causal attention
+core runs as a one-pass kernel (``mase_attention_causal``: bf16, head dimension 128, sequence a multiple of 128;
+otherwise the library's), and RMSNorm, the rotary embedding and the SwiGLU product run as one-pass kernels with the same arithmetic (``mase_rmsnorm_minifloat``,
 ``mase_rope``, ``mase_silu_mul_minifloat`` with their casts off); where the Linears that consume an RMSNorm or the
 SwiGLU product are MXINT Linears on the matrix-core path, those kernels write the quantized form the Linears would
 each compute (``mase_rmsnorm_mxint``, ``mase_silu_mul_mxint``), which saves a pass over the tensor.
@@ -63,6 +64,14 @@ def rope_tables(seq_len: int, head_dim: int, theta: float, device, dtype):
     return emb.cos().to(dtype), emb.sin().to(dtype)
 
 
+def causal_attention(q, k, v):
+    """softmax(q k^T / sqrt(d) + causal mask) v: the one-pass kernel of this package where it applies (bf16, head
+    dimension 128, a multiple of 128 tokens, no gradient), the library's scaled_dot_product_attention otherwise"""
+    if q.is_cuda and _ops.attention_causal_supported(q, k, v):
+        return _ops.attention_causal(q, k, v)
+    return F.scaled_dot_product_attention(q, k, v, is_causal=True)
+
+
 class DecoderLayer(nn.Module):
     def __init__(self, cfg: DecoderLayerConfig = DecoderLayerConfig(), device=None, dtype=None, seed: int | None = None):
         super().__init__()
@@ -78,9 +87,9 @@ class DecoderLayer(nn.Module):
         self.gate_proj = nn.Linear(H, I, **kw)
         self.up_proj = nn.Linear(H, I, **kw)
         self.down_proj = nn.Linear(I, H, **kw)
-        # the attention core is a plain torch library call; tests replace it to keep both sides of a comparison on
-        # the same implementation (the library's CPU and GPU kernels differ by a few bf16 ulps)
-        self.attention_fn = lambda q, k, v: F.scaled_dot_product_attention(q, k, v, is_causal=True)
+        # the attention core; tests replace it to keep both sides of a comparison on the same implementation (the
+        # library's CPU and GPU kernels and the kernel of this package differ by a few bf16 ulps)
+        self.attention_fn = causal_attention
         if seed is not None:
             self.reset_parameters_seeded(seed)
 

@@ -97,6 +97,11 @@ def test_decoder_layer_mxint_matches_cpu_reference(dev, shape, widths):
         del gpu.attention_fn
         gpu.attention_fn = lambda q, k, v: torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)
         e_lib = rel_err(gpu(x.to(dev)), ref)
+        # (d) free-running layer with its own default attention (the kernel of this package where the shape allows)
+        from mase_amd.workloads.decoder_layer import causal_attention
+        gpu.attention_fn = causal_attention
+        e_own = rel_err(gpu(x.to(dev)), ref)
+        assert e_own < 3e-2, e_own
     print(f"decoder layer MXINT8 {shape} widths {widths}: rel err {e:.3e} (same attention kernel), {e_lib:.3e} (GPU attention kernel)")
     assert y.dtype == torch.bfloat16 and y.shape == x.shape
     assert e < 1e-2

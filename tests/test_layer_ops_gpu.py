@@ -145,3 +145,40 @@ def test_norm_and_silu_product_written_in_the_consumers_mxint_form(dev, dtype, b
         gd, ud = gate.to(dev), up.to(dev)
         want = _ops.mxint_qdq(_ops.silu_mul_minifloat(gd, ud), 32, bits, -1, 8)
         assert_bits_equal(_ops.silu_mul_mxint(gd, ud, bits), want, f"silu_mul_mxint {dtype} {rows}x{cols}")
+
+
+@pytest.mark.parametrize("B,H,T", [(1, 1, 128), (2, 3, 256), (1, 2, 640), (1, 4, 2048)])
+@pytest.mark.parametrize("layout", ["bthd", "bhtd"])
+def test_causal_attention_one_pass(dev, B, H, T, layout):
+    """mase_attention_causal against the tensor operations in fp32 (masked scores, softmax, product with v) on the same
+    bf16 operands: bound 1e-2 of the output range (the probabilities are rounded to bf16 before the second product and
+    the output is bf16); the library's own kernel is held to the same bound for comparison.  Operands as strided views
+    of [batch, tokens, heads, 128] memory (what the projections produce) and contiguous [batch, heads, tokens, 128]."""
+    from mase_amd.quantizers import _ops
+
+    g = torch.Generator().manual_seed(B * 1000 + T)
+    mk = lambda scale: (torch.randn(B, T, H, 128, generator=g) * scale).bfloat16().to(dev)
+    q, k, v = mk(1.5), mk(1.0), mk(2.0)
+    if layout == "bthd":
+        q, k, v = (t.transpose(1, 2) for t in (q, k, v))
+    else:
+        q, k, v = (t.transpose(1, 2).contiguous() for t in (q, k, v))
+    assert _ops.attention_causal_supported(q, k, v)
+    for scaling in (None, 0.05):
+        sc = 128 ** -0.5 if scaling is None else scaling
+        s = (q.float() @ k.float().transpose(-1, -2)) * sc
+        s = s.masked_fill(torch.triu(torch.ones(T, T, dtype=torch.bool, device=dev), 1), float("-inf"))
+        ref = torch.softmax(s, -1) @ v.float()
+        got = _ops.attention_causal(q, k, v, scaling)
+        assert got.shape == (B, H, T, 128) and got.dtype == torch.bfloat16
+        assert got.transpose(1, 2).reshape(B, T, H * 128).data_ptr() == got.data_ptr()  # [B, T, H*128] is a view
+        e = float((got.float() - ref).abs().max() / ref.abs().max())
+        lib = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, scale=sc)
+        e_lib = float((lib.float() - ref).abs().max() / ref.abs().max())
+        print(f"causal attention {B}x{H}x{T} {layout} scale {sc:.3f}: err {e:.2e} (library kernel {e_lib:.2e})")
+        assert e < 1e-2
+        # the first query attends to the first key only: its output row is v[0]
+        assert torch.equal(got[:, :, 0], v[:, :, 0])
+    assert not _ops.attention_causal_supported(q[:, :, :100], k[:, :, :100], v[:, :, :100])
+    assert not _ops.attention_causal_supported(q.float(), k.float(), v.float())
+    assert not _ops.attention_causal_supported(q[..., :64], k[..., :64], v[..., :64])
