@@ -354,8 +354,8 @@ class DecoderLayerMxint(Workload):
     name = "decoder_layer"
     default_steps, default_warmup = 100, 10
     metric = ("Llama-style decoder layer forward with MXINT8 Linears (flop per step = 7 Linears + causal attention; "
-              "RMSNorm, rotary embedding and the SwiGLU product run as one-pass kernels, attention as the library's "
-              "scaled_dot_product_attention, all inside the step)")
+              "RMSNorm, rotary embedding, the SwiGLU product and causal attention run as one-pass kernels of this "
+              "library, all inside the step)")
     unit = "TFLOP/s"
     dtype = "bf16"
     bound = "mfma"

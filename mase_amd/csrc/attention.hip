@@ -12,11 +12,12 @@
 // the 64 keys in its accumulator registers, so the softmax statistics are in-lane but for one exchange with lane ^ 32.
 // exp2 of the scaled scores gives P^T, which is already laid out as the B operand of O^T += V^T P^T (the matrix
 // instruction's 8 contraction slots of lane group g at step s are accumulator registers 8 (s % 2) .. + 7 of score tile
-// s / 2, i.e. keys 32 (s / 2) + 8 (2 (s % 2) + j / 4) + 4 g + j % 4: the V^T fragments are read from LDS in the same
-// key order, two 8-byte pieces each).  Two work-groups fit a CU (66 KB of LDS, under 256 registers), so one
-// wavefront's exponentials overlap the other's matrix instructions.
+// s / 2, i.e. keys 16 s + 4 g + 8 (j / 4) + j % 4).  Two work-groups fit a CU (64 KB of LDS, under 256 registers),
+// so one wavefront's exponentials overlap the other's matrix instructions.
 //
-// V^T is made by a transposing pre-pass into a caller workspace [batch * heads][128][T].
+// V^T is made by a transposing pre-pass into a caller workspace [batch * heads][128][T] whose key axis is permuted
+// inside every group of 16 keys (order 0-3, 8-11, 4-7, 12-15), so that the 8 keys of a lane's contraction slots are one
+// 16-byte chunk (chunk 2 s + g of the 64-key row) and the V^T fragments are read like the K fragments.
 #include "common.hpp"
 
 namespace mase {
@@ -28,8 +29,22 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 
 constexpr int kQB = 128, kKB = 64, kHD = 128;
 constexpr int kKBytes = kKB * kHD * 2;       // 16 KB: 64 key rows of 256 bytes
-constexpr int kVGroup = 8 * 128 + 16;        // 8 rows (d) of 128 bytes (64 keys) + 16 bytes that stagger the groups' banks
+constexpr int kVGroup = 8 * 128;             // 8 rows (d) of 128 bytes (64 keys): one async copy of a wavefront
 constexpr int kVBytes = 16 * kVGroup;
+constexpr float kGrow = 8.0f;                // see the softmax reference point in the kernel
+
+// 16-byte slot of V^T row d that holds the row's chunk c is c ^ v_swizzle(d): distinct over any 8 consecutive rows, and
+// over the even and the odd rows of any 16 (rows are 128 bytes, so two rows span 64 four-byte banks)
+// max of a lane's value and lane ^ 32's, without a trip through the LDS queue (which would wait for the fragment reads
+// in flight)
+__device__ __forceinline__ float max_with_other_half(float v) {
+  const unsigned u = __builtin_bit_cast(unsigned, v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const unsigned a = r[0], b = r[1];  // (a bit cast applied to r[1] directly reads element 0)
+  return fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
+}
+
+__device__ __forceinline__ int v_swizzle(int d) { return (d & 7) ^ ((d >> 3) & 1); }
 constexpr int kAttnLds = 2 * kKBytes + 2 * kVBytes;
 
 // lane i's 16 bytes at base + off_i land at LDS address lds_addr + 16 * i; tracked by hand with at_wait_vmcnt
@@ -58,10 +73,19 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
   const int l32 = lane & 31, g = lane >> 5;
-  // the query blocks with the most keys first
+  // Work-groups are handed to the 8 XCDs in turn (blockIdx % 8), each XCD with an L2 of its own.  All query blocks of
+  // one (batch, head) go to one XCD, one after the other and the ones with the most keys first: they run at the same
+  // time and walk the keys from the start together, so K and V^T come from HBM once and from that L2 afterwards.
   const int n_qb = p.T / kQB;
-  const int qb = n_qb - 1 - (int)blockIdx.x / p.BH;
-  const int bh = (int)blockIdx.x % p.BH;
+  int bh, qb;
+  if (p.BH % 8 == 0) {
+    const int xcd = (int)blockIdx.x & 7, slot = (int)blockIdx.x >> 3;
+    bh = (slot / n_qb) * 8 + xcd;
+    qb = n_qb - 1 - slot % n_qb;
+  } else {
+    bh = (int)blockIdx.x / n_qb;
+    qb = n_qb - 1 - (int)blockIdx.x % n_qb;
+  }
   const int b = bh / p.H, h = bh % p.H;
   const unsigned char* qp = p.q + (size_t)b * p.q_sb + (size_t)h * p.q_sh;
   const unsigned char* kp = p.k + (size_t)b * p.k_sb + (size_t)h * p.k_sh;
@@ -74,7 +98,7 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
   for (int s = 0; s < 8; ++s) qf[s] = *(const bf16x8_t*)(qp + (size_t)qi * p.q_st + (s * 16 + g * 8) * 2);
 
   // async copies of one key block: 4 of K (4 rows of 256 bytes each) and 4 of V^T (8 rows of 128 bytes) per wavefront.
-  // LDS position (row, 16-byte slot) holds the row's chunk slot ^ (row % 16) (K) / slot ^ (row % 8) (V^T), so that the
+  // LDS position (row, 16-byte slot) holds the row's chunk slot ^ (row % 16) (K) / slot ^ v_swizzle(row) (V^T), so that the
   // fragment reads of 32 lanes (32 rows, same chunk) spread over the banks.
   uint32_t koff[4], voff[4];
 #pragma unroll
@@ -82,7 +106,7 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
     const int krow = (wave * 4 + i) * 4 + (lane >> 4);
     koff[i] = (uint32_t)krow * p.k_st + (uint32_t)(((lane & 15) ^ (krow & 15)) << 4);
     const int d = (wave * 4 + i) * 8 + (lane >> 3);
-    voff[i] = (uint32_t)d * (uint32_t)(p.T * 2) + (uint32_t)(((lane & 7) ^ (d & 7)) << 4);
+    voff[i] = (uint32_t)d * (uint32_t)(p.T * 2) + (uint32_t)(((lane & 7) ^ v_swizzle(d)) << 4);
   }
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;
   auto issue = [&](int j) __attribute__((always_inline)) {
@@ -114,18 +138,39 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
     const unsigned char* Kb = lds + (j & 1) * kKBytes;
     const unsigned char* Vb = lds + 2 * kKBytes + (j & 1) * kVBytes;
 
+    // every fragment read of a phase is issued before the phase's first matrix instruction, in the order the
+    // instructions take them, so a wavefront waits one LDS latency per phase, not one per instruction
+    bf16x8_t kf[16];
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int row = t * 32 + l32;
+        kf[2 * s + t] = *(const bf16x8_t*)(Kb + row * 256 + (((2 * s + g) ^ (row & 15)) << 4));
+      }
+    __builtin_amdgcn_sched_barrier(0);
     f32x16_t sc[2];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) sc[t][r] = 0.0f;
-      const int row = t * 32 + l32;
 #pragma unroll
-      for (int s = 0; s < 8; ++s) {
-        const bf16x8_t kf = *(const bf16x8_t*)(Kb + row * 256 + (((2 * s + g) ^ (row & 15)) << 4));
-        sc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sc[t], 0, 0, 0);
+    for (int s = 0; s < 8; ++s)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) sc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[2 * s + t], qf[s], sc[t], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    // V^T fragments of the first two steps of the second product: their latency passes behind the exponentials
+    bf16x8_t vf[2][4];
+    auto read_v = [&](int s, bf16x8_t* dst) __attribute__((always_inline)) {
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) {
+        const int d = dt * 32 + l32;
+        dst[dt] = *(const bf16x8_t*)(Vb + d * 128 + (((2 * s + g) ^ v_swizzle(d)) << 4));
       }
-    }
+    };
+    read_v(0, vf[0]);
+    read_v(1, vf[1]);
+    __builtin_amdgcn_sched_barrier(0);
     // register r of tile t is key key0 + 32 t + 8 (r / 4) + 4 g + r % 4
     if (key0 + kKB - 1 > q0) {  // the block reaches past this wavefront's first query: mask
 #pragma unroll
@@ -136,16 +181,28 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
           if (key > qi) sc[t][r] = -__builtin_inff();
         }
     }
-    float mx = m;
+    float mx = sc[0][0];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sc[t][r]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));  // finite: key0 <= q0 <= this lane's query, so key0 itself is not masked
-    const float alpha = __builtin_amdgcn_exp2f((m - mx) * p.c);
-    m = mx;
-    const float mc = mx * p.c;
+    mx = max_with_other_half(mx);  // finite: key0 <= q0 <= this lane's query, so key0 itself is not masked
+    // The reference point m of the exponentials moves only when some query of the wavefront has met a score more than
+    // kGrow (in the exponent's unit) above it: probabilities then reach 2^kGrow instead of 1, which fp32 sums and the
+    // bf16 rounding (relative) do not mind, and most key blocks skip the rescaling of the 64 accumulator registers.
+    if (__builtin_amdgcn_ballot_w64((mx - m) * p.c > kGrow) != 0) {
+      const float mn = fmaxf(m, mx);
+      const float alpha = __builtin_amdgcn_exp2f((m - mn) * p.c);
+      m = mn;
+      lsum *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+    }
+    const float mc = m * p.c;
     float psum = 0.0f;
+    uint4 pw[4];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -153,31 +210,23 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
         sc[t][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[t][r], p.c, -mc));
         psum += sc[t][r];
       }
-    lsum = lsum * alpha + psum;
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+    lsum += psum;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int t = s >> 1, r0 = (s & 1) * 8;
-      uint4 pw;
-      pw.x = f32x2_to_bf16x2_bits(sc[t][r0 + 0], sc[t][r0 + 1]);
-      pw.y = f32x2_to_bf16x2_bits(sc[t][r0 + 2], sc[t][r0 + 3]);
-      pw.z = f32x2_to_bf16x2_bits(sc[t][r0 + 4], sc[t][r0 + 5]);
-      pw.w = f32x2_to_bf16x2_bits(sc[t][r0 + 6], sc[t][r0 + 7]);
-      const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pw);
-      const int kbyte = (32 * t + 16 * (s & 1) + 4 * g) * 2;  // first of this lane group's keys, then 8 keys further
-      const int gran = kbyte >> 4, half = (kbyte & 15);
+      pw[s].x = f32x2_to_bf16x2_bits(sc[t][r0 + 0], sc[t][r0 + 1]);
+      pw[s].y = f32x2_to_bf16x2_bits(sc[t][r0 + 2], sc[t][r0 + 3]);
+      pw[s].z = f32x2_to_bf16x2_bits(sc[t][r0 + 4], sc[t][r0 + 5]);
+      pw[s].w = f32x2_to_bf16x2_bits(sc[t][r0 + 6], sc[t][r0 + 7]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt) {
-        const int d = dt * 32 + l32;
-        const unsigned char* vrow = Vb + (d >> 3) * kVGroup + (d & 7) * 128;
-        const uint2 v0 = *(const uint2*)(vrow + ((gran ^ (d & 7)) << 4) + half);
-        const uint2 v1 = *(const uint2*)(vrow + (((gran + 1) ^ (d & 7)) << 4) + half);
-        const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, make_uint4(v0.x, v0.y, v1.x, v1.y));
-        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, o[dt], 0, 0, 0);
-      }
+    for (int s = 0; s < 4; ++s) {
+      const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pw[s]);
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[s & 1][dt], pf, o[dt], 0, 0, 0);
+      if (s < 2) read_v(s + 2, vf[s & 1]);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
   at_wait_vmcnt<0>();
@@ -196,7 +245,8 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
     }
 }
 
-// vt[bh][d][t] = v[b][t][h][d]: tiles of 64 tokens x 128 d through LDS (rows padded to 264 bytes)
+// vt[bh][d][perm(t)] = v[b][t][h][d], perm swapping the middle two quads of every 16 tokens: tiles of 64 tokens x 128 d
+// through LDS (rows padded to 264 bytes)
 __global__ __launch_bounds__(256) void attn_transpose_v_kernel(const unsigned char* __restrict__ v, unsigned char* __restrict__ vt,
                                                                int H, int T, size_t v_sb, size_t v_sh, uint32_t v_st) {
   __shared__ __attribute__((aligned(16))) unsigned char tile[64 * 264];
@@ -212,13 +262,15 @@ __global__ __launch_bounds__(256) void attn_transpose_v_kernel(const unsigned ch
   __syncthreads();
   unsigned char* dst = vt + (size_t)bh * ((size_t)kHD * T * 2) + (size_t)t0 * 2;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {  // 1024 pieces of 8 tokens: d = piece / 8, token group = piece % 8
+  for (int i = 0; i < 4; ++i) {  // 1024 chunks of 8 tokens: d = chunk / 8; chunk % 8 = 2 (group of 16) + half
     const int c = i * 256 + tid, d = c >> 3, tg = c & 7;
+    const int tok0 = (tg >> 1) * 16 + (tg & 1) * 4;  // tokens tok0 .. + 3 and tok0 + 8 .. + 11
     uint32_t w[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const uint32_t lo = *(const uint16_t*)(tile + (tg * 8 + 2 * e) * 264 + d * 2);
-      const uint32_t hi = *(const uint16_t*)(tile + (tg * 8 + 2 * e + 1) * 264 + d * 2);
+      const int tok = tok0 + (e >> 1) * 8 + (e & 1) * 2;
+      const uint32_t lo = *(const uint16_t*)(tile + tok * 264 + d * 2);
+      const uint32_t hi = *(const uint16_t*)(tile + (tok + 1) * 264 + d * 2);
       w[e] = lo | (hi << 16);
     }
     *(uint4*)(dst + (size_t)d * T * 2 + tg * 16) = make_uint4(w[0], w[1], w[2], w[3]);
@@ -243,6 +295,7 @@ extern "C" int mase_attention_causal(const void* q, const void* k, const void* v
   if (batch == 0 || heads == 0 || tokens == 0) return MASE_OK;
   if (q == nullptr || k == nullptr || v == nullptr || out == nullptr) return MASE_ERR_NULL;
   if (dtype != MASE_DT_BF16) return MASE_ERR_DTYPE;
+  if (!(scaling > 0.0f) || !(scaling < 3.0e38f)) return MASE_ERR_PARAM;  // the running maximum is taken before scaling
   if (head_dim != 128 || tokens % 128 != 0 || tokens > (1u << 20) || batch * heads > (1u << 20)) return MASE_ERR_SHAPE;
   // strides in elements; rows of 128 elements must be whole 16-byte chunks, a token stride must fit 32 bits in bytes
   const size_t strides[12] = {q_stride_b, q_stride_h, q_stride_t, k_stride_b, k_stride_h, k_stride_t,
