@@ -188,6 +188,55 @@ class CopyBytes(Workload):
         return 2.0 * self.nbytes
 
 
+class _MfmaIssueRate(Workload):
+    """calibration: v_mfma_f32_32x32x16_bf16 on register operands with nothing else running, two wavefronts per SIMD on
+    every CU.  The rate depends on the operand values (the part holds the instruction back when operand bits vary), so
+    it is measured for zeros and for uniform values; the second is the ceiling of a bf16 GEMM on real data."""
+    default_steps, default_warmup = 40, 10
+    unit = "TFLOP/s"
+    dtype = "bf16"
+    bound = "mfma"
+    kernel = "probe_mfma_bf16_kernel"
+    operands = 0
+    iters = 4096      # x 8 instructions per wavefront
+    work_groups = 256
+
+    def setup(self, torch, dev, n_buffers):
+        from mase_amd import _lib
+
+        self.lib = _lib.load()
+        self._lib = _lib
+        self.out = torch.empty(self.work_groups * 512 + 4, dtype=torch.float32, device=dev)
+        self.metric = "matrix-core issue rate of v_mfma_f32_32x32x16_bf16 on register operands (no memory traffic)"
+        self.config = {"workload": f"{self.work_groups} work-groups x 8 wavefronts x {8 * self.iters} instructions, operands: "
+                                   + ("zeros" if self.operands == 0 else "uniform in [-2, 2)")}
+
+    def step(self, i):
+        self._lib.check(self.lib.mase_probe_mfma_bf16(self.out.data_ptr(), self.out.numel() * 4, self.work_groups, 2, self.iters,
+                                                      self.operands, self._lib.stream_ptr(self.out)), "probe")
+
+    def work_per_step(self):
+        return float(self.work_groups * 8 * 8 * self.iters) * 2.0 * 32 * 32 * 16
+
+    def extra(self, torch):
+        """shader clock during the last launch, from the kernel's own two counters (first wavefront's loop)"""
+        cyc, ticks = self.out[-4:].view(torch.int64).tolist()
+        rate_khz = int(self.lib.mase_constant_rate_counter_khz())
+        secs = ticks / (rate_khz * 1e3)
+        return {"shader_clock_ghz_in_loop": round(cyc / secs / 1e9, 3), "cycles_per_instruction_of_first_wavefront": round(cyc / (8.0 * self.iters), 2),
+                "constant_rate_counter_khz": rate_khz}
+
+
+class MfmaRateZeros(_MfmaIssueRate):
+    name = "mfma_rate_zeros"
+    operands = 0
+
+
+class MfmaRateRandom(_MfmaIssueRate):
+    name = "mfma_rate_random"
+    operands = 2
+
+
 class MxintLinear(Workload):
     name = "mxint_linear"
     default_steps, default_warmup = 1000, 100
@@ -707,7 +756,7 @@ class DecodeLinearMxfp4(Workload):
 
 WORKLOADS = {w.name: w for w in (MxintClipSearch, BfpQdq, MxintQdq, MxintLinear, MxintLinearCodes, MxfpLinear, DecoderLayerMxint, CopyBytes, IntegerQdq,
                                  MinifloatDenormQdq, MinifloatIeeeQdq, MinifloatMxQdq, MxfpQdq, AttnProb, DecodeLinear,
-                                 DecodeLinearPacked, DecodeLinearMxfp4)}
+                                 DecodeLinearPacked, DecodeLinearMxfp4, MfmaRateZeros, MfmaRateRandom)}
 
 
 def load_traffic(name):
@@ -797,6 +846,8 @@ def measure(torch, dev, name, steps, warmup, a):
         },
         "cpu_baseline": cpu,
     }
+    if hasattr(w, "extra"):
+        out["extra"] = w.extra(torch)
     del w
     torch.cuda.synchronize()
     torch.cuda.empty_cache()
@@ -860,6 +911,8 @@ def main():
         "settle_steps": head["settle_steps"],
         "whole_step_frac": head["whole_step_frac"],
     }
+    if "extra" in head:
+        out["extra"] = head["extra"]
     if a.workload == "all":
         out["configs"] = results
     print(json.dumps(out))

@@ -348,6 +348,18 @@ int mase_rope(const void* x, const void* cos, const void* sin, void* out, size_t
  * it is the calibration kernel for the achievable-bandwidth ceiling and for scaling hardware byte counters. */
 int mase_copy_bytes(const void* in, void* out, size_t bytes, void* stream);
 
+/* Issue rate of v_mfma_f32_32x32x16_bf16 with nothing else running: work_groups x (4 x wavefronts_per_simd) wavefronts,
+ * each issuing 8 * iters instructions on register operands.  operands: 0 zeros, 1 small integers, 2 uniform values in
+ * [-2, 2).  No counterpart in the reference: it measures the matrix-core rate this GPU sustains for a given kind of
+ * operand values (the power management of the part holds the instruction back when operand bits vary), the ceiling
+ * the GEMM kernels are to be read against.  out (16-byte aligned): work_groups * 256 * wavefronts_per_simd floats of
+ * scratch followed by two int64 the kernel writes: the duration of the first wavefront's loop in shader-clock cycles
+ * and in ticks of the constant-rate counter (hipDeviceAttributeWallClockRate). */
+int mase_probe_mfma_bf16(void* out, size_t out_bytes, int work_groups, int wavefronts_per_simd, int iters, int operands,
+                         void* stream);
+/* rate of that constant-rate counter on the current device in kHz; 0 when the runtime cannot tell */
+int mase_constant_rate_counter_khz(void);
+
 /* test/diagnostic helpers (host only, no device work) */
 uint32_t mase_isclose_zero_threshold_bits(int dtype); /* largest |x| (fp32 bits) that isclose(x, 0) accepts */
 float mase_round_scalar_to_dtype(double v, int dtype); /* how a clamp bound is represented in dtype */

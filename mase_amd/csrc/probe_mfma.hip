@@ -1,0 +1,87 @@
+// Measurement aid, no counterpart in the reference: the rate at which the matrix cores of this GPU accept
+// v_mfma_f32_32x32x16_bf16 when nothing else runs (no memory traffic, no LDS, operands held in registers), as a
+// function of the operand VALUES.  The rate depends on them: with zero or small-integer operands the instruction
+// issues close to its nominal 32 cycles, with operands whose mantissa and exponent bits vary it is held back by the
+// power management of the part.  That second figure, not the published peak, is what a GEMM on real data can approach.
+#include "common.hpp"
+
+namespace mase {
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ uint32_t probe_hash(uint32_t x) {
+  x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16;
+  return x;
+}
+
+// operands: 0 zeros, 1 small integers, 2 uniform in [-2, 2) with full mantissas.  Each wavefront issues 8 * iters
+// instructions on two accumulator chains; out receives one float per lane so that nothing is optimised away, and after
+// those the first wavefront's loop duration on the shader-clock counter and on the constant-rate counter (two int64).
+__global__ __launch_bounds__(512) void probe_mfma_bf16_kernel(float* out, int iters, int operands) {
+  const int lane = threadIdx.x & 63;
+  bf16x8_t a[4], b[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t h1 = probe_hash(threadIdx.x * 64 + s * 8 + i + blockIdx.x * 7919), h2 = probe_hash(h1 + 12345);
+      float va = 0.0f, vb = 0.0f;
+      if (operands == 1) { va = (float)((lane + i) & 7); vb = (float)((lane - i) & 3); }
+      if (operands == 2) {
+        va = (float)(int)(h1 >> 8) * (1.0f / 4194304.0f) - 2.0f;
+        vb = (float)(int)(h2 >> 8) * (1.0f / 4194304.0f) - 2.0f;
+      }
+      a[s][i] = (__bf16)va;
+      b[s][i] = (__bf16)vb;
+    }
+  f32x16_t acc[2];
+#pragma unroll
+  for (int c = 0; c < 2; ++c)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[c][r] = 0.0f;
+  const long long c0 = __builtin_readcyclecounter(), w0 = wall_clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s], b[s], acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(s + 1) & 3], b[s], acc[1], 0, 0, 0);
+    }
+  }
+  float r = 0.0f;
+#pragma unroll
+  for (int c = 0; c < 2; ++c)
+#pragma unroll
+    for (int k = 0; k < 16; ++k) r += acc[c][k];
+  const long long c1 = __builtin_readcyclecounter(), w1 = wall_clock64();
+  out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = r;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    long long* t = (long long*)(out + (size_t)gridDim.x * blockDim.x);
+    t[0] = c1 - c0;
+    t[1] = w1 - w0;
+  }
+}
+
+}  // namespace
+}  // namespace mase
+
+extern "C" int mase_probe_mfma_bf16(void* out, size_t out_bytes, int work_groups, int wavefronts_per_simd, int iters,
+                                    int operands, void* stream) {
+  using namespace mase;
+  if (out == nullptr) return MASE_ERR_NULL;
+  if (work_groups < 1 || work_groups > 65536 || (wavefronts_per_simd != 1 && wavefronts_per_simd != 2) || iters < 1 ||
+      operands < 0 || operands > 2)
+    return MASE_ERR_PARAM;
+  const int threads = 256 * wavefronts_per_simd;
+  if (out_bytes < (size_t)work_groups * threads * sizeof(float) + 16 || !aligned16(out)) return MASE_ERR_WORKSPACE;
+  hipLaunchKernelGGL(probe_mfma_bf16_kernel, dim3((unsigned)work_groups), dim3((unsigned)threads), 0, (hipStream_t)stream,
+                     (float*)out, iters, operands);
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+extern "C" int mase_constant_rate_counter_khz(void) {
+  int dev = 0, khz = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess) return 0;
+  return khz;
+}
