@@ -88,12 +88,16 @@ __device__ __forceinline__ void cast8(float* v, const CastSpec& c) {
   for (int j = 0; j < 8; ++j) v[j] = DTypeTraits<DT>::round(y[j]);
 }
 
-// one wavefront per row; the row stays in registers (NCH chunks of 64 lanes x 8 elements).  MX: the output is the
-// MXINT quantize-dequantize of the normalised row (cols a multiple of 32)
-template <int DT, int NCH, bool MX = false>
-__global__ __launch_bounds__(kRowThreads) void rmsnorm_kernel(RmsNormParams p) {
+// WPR wavefronts per row (one work-group); the row stays in registers (NCH chunks of 64 lanes x 8 elements per
+// wavefront, chunk c of wavefront w at element ((c * WPR + w) * 64 + lane) * 8).  Rows of more than 1536 elements are
+// spread over 4 wavefronts: 16 or 32 elements per lane instead of 64 keep the register count low enough for 8
+// wavefronts per SIMD, which is what hides the one load - compute - store round trip of each wavefront.  MX: the
+// output is the MXINT quantize-dequantize of the normalised row (cols a multiple of 32)
+template <int DT, int NCH, bool MX = false, int WPR = 1>
+__global__ __launch_bounds__(kRowThreads * WPR) void rmsnorm_kernel(RmsNormParams p) {
   using TR = DTypeTraits<DT>;
   const int lane = (int)(threadIdx.x & 63);
+  const int wave = (int)(threadIdx.x >> 6);
   const size_t row = blockIdx.x;
   const size_t base = row * (size_t)p.cols;
   WaveLog2 meta;
@@ -102,7 +106,7 @@ __global__ __launch_bounds__(kRowThreads) void rmsnorm_kernel(RmsNormParams p) {
   float ss = 0.0f;
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
-    const int e0 = (c * 64 + lane) * 8;
+    const int e0 = ((c * WPR + wave) * 64 + lane) * 8;
 #pragma unroll
     for (int j = 0; j < 8; ++j) h[c][j] = 0.0f;
     if (e0 < p.cols) {
@@ -114,10 +118,18 @@ __global__ __launch_bounds__(kRowThreads) void rmsnorm_kernel(RmsNormParams p) {
   }
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) ss += __shfl_xor(ss, o, 64);
+  if constexpr (WPR > 1) {
+    __shared__ float part[WPR];
+    if (lane == 0) part[wave] = ss;
+    __syncthreads();
+    ss = 0.0f;
+#pragma unroll
+    for (int w = 0; w < WPR; ++w) ss += part[w];  // the same order in every wavefront
+  }
   const float r = rsqrtf(ss / (float)p.cols + p.eps);
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
-    const int e0 = (c * 64 + lane) * 8;
+    const int e0 = ((c * WPR + wave) * 64 + lane) * 8;
     const bool live = e0 < p.cols;
     if constexpr (!MX) {
       if (!live) continue;
@@ -140,16 +152,20 @@ __global__ __launch_bounds__(kRowThreads) void rmsnorm_kernel(RmsNormParams p) {
   }
 }
 
+template <int DT, bool MX, int WPR>
+int launch_rmsnorm_wpr(const RmsNormParams& p, int nch, hipStream_t st) {
+  const dim3 grid((unsigned)p.rows), block(kRowThreads * WPR);
+  if (nch <= 1) hipLaunchKernelGGL((rmsnorm_kernel<DT, 1, MX, WPR>), grid, block, 0, st, p);
+  else if (nch <= 2) hipLaunchKernelGGL((rmsnorm_kernel<DT, 2, MX, WPR>), grid, block, 0, st, p);
+  else hipLaunchKernelGGL((rmsnorm_kernel<DT, 4, MX, WPR>), grid, block, 0, st, p);
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
 template <int DT, bool MX = false>
 int launch_rmsnorm(const RmsNormParams& p, hipStream_t st) {
-  const int nch = (p.cols + 511) / 512;
-  const dim3 grid((unsigned)p.rows), block(kRowThreads);
-  if (nch <= 1) hipLaunchKernelGGL((rmsnorm_kernel<DT, 1, MX>), grid, block, 0, st, p);
-  else if (nch <= 2) hipLaunchKernelGGL((rmsnorm_kernel<DT, 2, MX>), grid, block, 0, st, p);
-  else if (nch <= 4) hipLaunchKernelGGL((rmsnorm_kernel<DT, 4, MX>), grid, block, 0, st, p);
-  else if (nch <= 8) hipLaunchKernelGGL((rmsnorm_kernel<DT, 8, MX>), grid, block, 0, st, p);
-  else hipLaunchKernelGGL((rmsnorm_kernel<DT, 16, MX>), grid, block, 0, st, p);
-  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+  const int nch = (p.cols + 511) / 512;  // chunks of 64 lanes x 8 elements in a row (cols <= 8192: at most 16)
+  if (nch <= 3) return launch_rmsnorm_wpr<DT, MX, 1>(p, nch, st);
+  return launch_rmsnorm_wpr<DT, MX, 4>(p, (nch + 3) / 4, st);
 }
 
 struct SiluMulParams {
