@@ -52,6 +52,7 @@ struct GemmParams {
   const unsigned char* B;
   const unsigned char* Bs;  // BCODES: the scale image that goes with the code image in B
   const void* bias;
+  const void* residual;  // RES instantiation: [M, N] in the output dtype, added to the rounded output
   void* C;
   int M, N, K;
   int bias_dtype;
@@ -126,8 +127,9 @@ __device__ __forceinline__ void ucodes4_to_bf16(uint32_t u, float scale, float b
 // the bytes of the bf16 image in memory and on the way in; the codes are widened to the same bf16 operand values in
 // registers, one K step ahead of the MFMAs that use them (code + 128 as an unsigned byte -> v_cvt_f32_ubyte -> one fma
 // that removes the 128 and applies the block's power-of-two scale -> the upper half of the exact fp32 product).
-template <int OUT_DT, bool STREAM, bool BPACK = false, bool BCODES = false>
+template <int OUT_DT, bool STREAM, bool BPACK = false, bool BCODES = false, bool RES = false>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p) {
+  static_assert(!RES || OUT_DT != MASE_DT_F32, "the residual epilogue holds a tile of 16-bit values in registers");
   static_assert(!BCODES || BPACK, "codes come in fragment order");
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int tid = threadIdx.x;
@@ -282,6 +284,27 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
       // inside the K loop, where that would also wait for every async copy in flight.
       wait_vmcnt<0>();
     }
+    // RES: out = round(round(A B^T + bias) + residual), the two roundings of a Linear followed by a residual add.
+    // The lane's 64 pieces of 4 residual values (the ones it stores below) are all requested before the first band
+    // and completed by one wait, so the tile pays one memory latency, not one per band.
+    uint2 rv[RES ? 64 : 1];
+    if constexpr (RES) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int jh = 0; jh < 2; ++jh)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+              const int row = m0 + wm * 128 + i * 32 + q * 8 + kgrp * 4 + rl0 + 2 * u;
+              const int col0 = n0 + wn * 128 + jh * 64 + c4;
+              uint2 r = make_uint2(0u, 0u);
+              if (row < p.M && col0 + 3 < p.N) r = *(const uint2*)((const uint16_t*)p.residual + (size_t)row * p.N + col0);
+              rv[((i * 4 + q) * 2 + jh) * 2 + u] = r;
+            }
+      wait_vmcnt<0>();
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
@@ -312,11 +335,23 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
                 uint2 w;
                 w.x = f32x2_to_bf16x2_bits(v[0], v[1]);
                 w.y = f32x2_to_bf16x2_bits(v[2], v[3]);
+                if constexpr (RES) {
+                  const uint2 r = rv[((i * 4 + q) * 2 + jh) * 2 + u];
+                  w.x = f32x2_to_bf16x2_bits(bits2f(w.x << 16) + bits2f(r.x << 16), bits2f(w.x & 0xFFFF0000u) + bits2f(r.x & 0xFFFF0000u));
+                  w.y = f32x2_to_bf16x2_bits(bits2f(w.y << 16) + bits2f(r.y << 16), bits2f(w.y & 0xFFFF0000u) + bits2f(r.y & 0xFFFF0000u));
+                }
                 store_nt((uint2*)((uint16_t*)Cs + o), w);
               } else {
                 uint2 w;
                 w.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
                 w.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
+                if constexpr (RES) {
+                  const uint2 r = rv[((i * 4 + q) * 2 + jh) * 2 + u];
+                  w.x = f32_to_f16_bits(f16_bits_to_f32(w.x & 0xFFFFu) + f16_bits_to_f32(r.x & 0xFFFFu)) |
+                        (f32_to_f16_bits(f16_bits_to_f32(w.x >> 16) + f16_bits_to_f32(r.x >> 16)) << 16);
+                  w.y = f32_to_f16_bits(f16_bits_to_f32(w.y & 0xFFFFu) + f16_bits_to_f32(r.y & 0xFFFFu)) |
+                        (f32_to_f16_bits(f16_bits_to_f32(w.y >> 16) + f16_bits_to_f32(r.y >> 16)) << 16);
+                }
                 store_nt((uint2*)((uint16_t*)Cs + o), w);
               }
             } else {
@@ -658,9 +693,25 @@ int launch_gemm_bf16(const GemmParams& p, int out_dtype, hipStream_t st, bool bp
     }                                                                                                             \
     hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, true, true>), grid, block, lds_bytes, st, p);                    \
   } while (0)
-    if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH_B(MASE_DT_F32);
+#define MASE_GEMM_LAUNCH_R(DT_)                                                                                   \
+  do {                                                                                                            \
+    static bool attr_set = false;                                                                                 \
+    const void* k = (const void*)gemm_bf16_tn_kernel<DT_, true, true, false, true>;                               \
+    if (!attr_set) {                                                                                              \
+      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)       \
+        return MASE_ERR_LAUNCH;                                                                                   \
+      attr_set = true;                                                                                            \
+    }                                                                                                             \
+    hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, true, true, false, true>), grid, block, lds_bytes, st, p);       \
+  } while (0)
+    if (p.residual != nullptr) {
+      if (out_dtype == MASE_DT_BF16) MASE_GEMM_LAUNCH_R(MASE_DT_BF16);
+      else if (out_dtype == MASE_DT_F16) MASE_GEMM_LAUNCH_R(MASE_DT_F16);
+      else return MASE_ERR_DTYPE;
+    } else if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH_B(MASE_DT_F32);
     else if (out_dtype == MASE_DT_BF16) MASE_GEMM_LAUNCH_B(MASE_DT_BF16);
     else MASE_GEMM_LAUNCH_B(MASE_DT_F16);
+#undef MASE_GEMM_LAUNCH_R
 #undef MASE_GEMM_LAUNCH_B
   } else if (stream_fits) {
     if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH(MASE_DT_F32, true);
@@ -771,6 +822,7 @@ extern "C" int mase_gemm_bf16_tn(const void* A, const void* B, const void* bias,
   p.B = (const unsigned char*)B;
   p.Bs = nullptr;
   p.bias = bias;
+  p.residual = nullptr;
   p.C = C;
   p.M = (int)M;
   p.N = (int)N;
@@ -809,6 +861,7 @@ extern "C" int mase_gemm_bf16_tn_splitk(const void* A, const void* B, const void
   p.B = (const unsigned char*)B;
   p.Bs = nullptr;
   p.bias = nullptr;
+  p.residual = nullptr;
   p.C = workspace;
   p.M = (int)M;
   p.N = (int)N;
@@ -865,6 +918,37 @@ extern "C" int mase_gemm_bf16_tn_packed(const void* A, const void* B_packed, con
   p.B = (const unsigned char*)B_packed;
   p.Bs = nullptr;
   p.bias = bias;
+  p.residual = nullptr;
+  p.C = C;
+  p.M = (int)M;
+  p.N = (int)N;
+  p.K = (int)K;
+  p.bias_dtype = bias_dtype;
+  p.tiles_m = (int)((M + BM - 1) / BM);
+  p.tiles_n = (int)((N + BN - 1) / BN);
+  p.splits = 1;
+  p.kc = (int)K;
+  return launch_gemm_bf16(p, out_dtype, (hipStream_t)stream, true);
+}
+
+extern "C" int mase_gemm_bf16_tn_packed_residual(const void* A, const void* B_packed, const void* bias, const void* residual,
+                                                 void* C, size_t M, size_t N, size_t K, int out_dtype, int bias_dtype,
+                                                 void* stream) {
+  using namespace mase;
+  if (M == 0 || N == 0) return MASE_OK;
+  if (A == nullptr || B_packed == nullptr || C == nullptr || residual == nullptr) return MASE_ERR_NULL;
+  if (K == 0 || (K % (2 * BK)) != 0 || (N % 4) != 0 || M > (1u << 30) || N > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
+  if ((unsigned long long)M * K * 2 > 0xFFFFFFFFull || (unsigned long long)mase_gemm_bf16_packed_bytes(N, K) > 0xFFFFFFFFull)
+    return MASE_ERR_SHAPE;
+  if (!aligned16(A) || !aligned16(B_packed) || !aligned16(C) || (((uintptr_t)residual) & 7u) != 0) return MASE_ERR_ALIGN;
+  if ((out_dtype != MASE_DT_BF16 && out_dtype != MASE_DT_F16) || (bias != nullptr && (bias_dtype < 0 || bias_dtype > 2)))
+    return MASE_ERR_DTYPE;
+  GemmParams p;
+  p.A = (const unsigned char*)A;
+  p.B = (const unsigned char*)B_packed;
+  p.Bs = nullptr;
+  p.bias = bias;
+  p.residual = residual;
   p.C = C;
   p.M = (int)M;
   p.N = (int)N;
@@ -917,6 +1001,7 @@ extern "C" int mase_gemm_mxint8_tn_packed(const void* A, const void* code_image,
   p.B = (const unsigned char*)code_image;
   p.Bs = (const unsigned char*)scale_image;
   p.bias = bias;
+  p.residual = nullptr;
   p.C = C;
   p.M = (int)M;
   p.N = (int)N;
