@@ -200,6 +200,10 @@ class _MfmaIssueRate(Workload):
     operands = 0
     iters = 4096      # x 8 instructions per wavefront
     work_groups = 256
+    entry = "mase_probe_mfma_bf16"
+    instruction = "v_mfma_f32_32x32x16_bf16"
+    flop_per_instruction = 2.0 * 32 * 32 * 16
+    nominal_cycles = 32
 
     def setup(self, torch, dev, n_buffers):
         from mase_amd import _lib
@@ -207,16 +211,19 @@ class _MfmaIssueRate(Workload):
         self.lib = _lib.load()
         self._lib = _lib
         self.out = torch.empty(self.work_groups * 512 + 4, dtype=torch.float32, device=dev)
-        self.metric = "matrix-core issue rate of v_mfma_f32_32x32x16_bf16 on register operands (no memory traffic)"
+        self.metric = f"matrix-core issue rate of {self.instruction} on register operands (no memory traffic)"
         self.config = {"workload": f"{self.work_groups} work-groups x 8 wavefronts x {8 * self.iters} instructions, operands: "
-                                   + ("zeros" if self.operands == 0 else "uniform in [-2, 2)")}
+                                   + ("zeros" if self.operands == 0 else self.random_kind)}
+        self.fn = getattr(self.lib, self.entry)
+
+    random_kind = "uniform in [-2, 2)"
 
     def step(self, i):
-        self._lib.check(self.lib.mase_probe_mfma_bf16(self.out.data_ptr(), self.out.numel() * 4, self.work_groups, 2, self.iters,
-                                                      self.operands, self._lib.stream_ptr(self.out)), "probe")
+        self._lib.check(self.fn(self.out.data_ptr(), self.out.numel() * 4, self.work_groups, 2, self.iters,
+                                self.operands, self._lib.stream_ptr(self.out)), "probe")
 
     def work_per_step(self):
-        return float(self.work_groups * 8 * 8 * self.iters) * 2.0 * 32 * 32 * 16
+        return float(self.work_groups * 8 * 8 * self.iters) * self.flop_per_instruction
 
     def extra(self, torch):
         """shader clock during the last launch, from the kernel's own two counters (first wavefront's loop)"""
@@ -234,6 +241,28 @@ class MfmaRateZeros(_MfmaIssueRate):
 
 class MfmaRateRandom(_MfmaIssueRate):
     name = "mfma_rate_random"
+    operands = 2
+
+
+class _MfmaF8F4Rate(_MfmaIssueRate):
+    kernel = "probe_mfma_f8f4_kernel"
+    entry = "mase_probe_mfma_f8f4"
+    instruction = "v_mfma_scale_f32_32x32x64_f8f6f4 (e4m3 x e2m1, scales of 1)"
+    flop_per_instruction = 2.0 * 32 * 32 * 64
+    nominal_cycles = 64
+    mfma_dtype = "fp8"
+    dtype = "mxfp8 x mxfp4"
+    iters = 2048
+    random_kind = "random codes"
+
+
+class MfmaF8F4RateZeros(_MfmaF8F4Rate):
+    name = "mfma_f8f4_rate_zeros"
+    operands = 0
+
+
+class MfmaF8F4RateRandom(_MfmaF8F4Rate):
+    name = "mfma_f8f4_rate_random"
     operands = 2
 
 
@@ -756,7 +785,8 @@ class DecodeLinearMxfp4(Workload):
 
 WORKLOADS = {w.name: w for w in (MxintClipSearch, BfpQdq, MxintQdq, MxintLinear, MxintLinearCodes, MxfpLinear, DecoderLayerMxint, CopyBytes, IntegerQdq,
                                  MinifloatDenormQdq, MinifloatIeeeQdq, MinifloatMxQdq, MxfpQdq, AttnProb, DecodeLinear,
-                                 DecodeLinearPacked, DecodeLinearMxfp4, MfmaRateZeros, MfmaRateRandom)}
+                                 DecodeLinearPacked, DecodeLinearMxfp4, MfmaRateZeros, MfmaRateRandom, MfmaF8F4RateZeros,
+                                 MfmaF8F4RateRandom)}
 
 
 def load_traffic(name):

@@ -364,6 +364,10 @@ int mase_copy_bytes(const void* in, void* out, size_t bytes, void* stream);
  * and in ticks of the constant-rate counter (hipDeviceAttributeWallClockRate). */
 int mase_probe_mfma_bf16(void* out, size_t out_bytes, int work_groups, int wavefronts_per_simd, int iters, int operands,
                          void* stream);
+/* the same for v_mfma_scale_f32_32x32x64_f8f6f4 with e4m3 codes in A and e2m1 codes in B, scales of 1 (the
+ * instruction of the MXFP8 x MXFP4 Linear); operands: 0 zero codes, 2 random codes */
+int mase_probe_mfma_f8f4(void* out, size_t out_bytes, int work_groups, int wavefronts_per_simd, int iters, int operands,
+                         void* stream);
 /* rate of that constant-rate counter on the current device in kHz; 0 when the runtime cannot tell */
 int mase_constant_rate_counter_khz(void);
 

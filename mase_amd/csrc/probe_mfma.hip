@@ -63,6 +63,46 @@ __global__ __launch_bounds__(512) void probe_mfma_bf16_kernel(float* out, int it
   }
 }
 
+// The same for v_mfma_scale_f32_32x32x64_f8f6f4 with e4m3 codes in A and e2m1 codes in B (the instruction of the
+// MXFP8 x MXFP4 Linear), scales of 1.  operands: 0 zero codes, 2 random codes (the e4m3 NaN code excluded).
+typedef int i32x8_t __attribute__((ext_vector_type(8)));
+__global__ __launch_bounds__(512) void probe_mfma_f8f4_kernel(float* out, int iters, int operands) {
+  i32x8_t a[4], b[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t h1 = probe_hash(threadIdx.x * 64 + s * 8 + i + blockIdx.x * 7919), h2 = probe_hash(h1 + 12345);
+      a[s][i] = operands == 2 ? (int)(h1 & 0xBFBFBFBFu) : 0;          // exponent field below 1000: never the NaN code
+      b[s][i] = (operands == 2 && i < 4) ? (int)h2 : 0;                // 64 e2m1 codes in the first four registers
+    }
+  f32x16_t acc[2];
+#pragma unroll
+  for (int c = 0; c < 2; ++c)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[c][r] = 0.0f;
+  const long long c0 = __builtin_readcyclecounter(), w0 = wall_clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      acc[0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[s], b[s], acc[0], 0, 4, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+      acc[1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[(s + 1) & 3], b[s], acc[1], 0, 4, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+    }
+  }
+  float r = 0.0f;
+#pragma unroll
+  for (int c = 0; c < 2; ++c)
+#pragma unroll
+    for (int k = 0; k < 16; ++k) r += acc[c][k];
+  const long long c1 = __builtin_readcyclecounter(), w1 = wall_clock64();
+  out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = r;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    long long* t = (long long*)(out + (size_t)gridDim.x * blockDim.x);
+    t[0] = c1 - c0;
+    t[1] = w1 - w0;
+  }
+}
+
 }  // namespace
 }  // namespace mase
 
@@ -76,6 +116,20 @@ extern "C" int mase_probe_mfma_bf16(void* out, size_t out_bytes, int work_groups
   const int threads = 256 * wavefronts_per_simd;
   if (out_bytes < (size_t)work_groups * threads * sizeof(float) + 16 || !aligned16(out)) return MASE_ERR_WORKSPACE;
   hipLaunchKernelGGL(probe_mfma_bf16_kernel, dim3((unsigned)work_groups), dim3((unsigned)threads), 0, (hipStream_t)stream,
+                     (float*)out, iters, operands);
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+extern "C" int mase_probe_mfma_f8f4(void* out, size_t out_bytes, int work_groups, int wavefronts_per_simd, int iters,
+                                    int operands, void* stream) {
+  using namespace mase;
+  if (out == nullptr) return MASE_ERR_NULL;
+  if (work_groups < 1 || work_groups > 65536 || (wavefronts_per_simd != 1 && wavefronts_per_simd != 2) || iters < 1 ||
+      (operands != 0 && operands != 2))
+    return MASE_ERR_PARAM;
+  const int threads = 256 * wavefronts_per_simd;
+  if (out_bytes < (size_t)work_groups * threads * sizeof(float) + 16 || !aligned16(out)) return MASE_ERR_WORKSPACE;
+  hipLaunchKernelGGL(probe_mfma_f8f4_kernel, dim3((unsigned)work_groups), dim3((unsigned)threads), 0, (hipStream_t)stream,
                      (float*)out, iters, operands);
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
