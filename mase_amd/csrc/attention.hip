@@ -31,6 +31,7 @@ constexpr int kQB = 128, kKB = 64, kHD = 128;
 constexpr int kKBytes = kKB * kHD * 2;       // 16 KB: 64 key rows of 256 bytes
 constexpr int kVGroup = 8 * 128;             // 8 rows (d) of 128 bytes (64 keys): one async copy of a wavefront
 constexpr int kVBytes = 16 * kVGroup;
+constexpr int kKRing = 5;                    // K fragment pairs in flight or in use: reads run 4 contraction steps ahead
 constexpr float kGrow = 8.0f;                // see the softmax reference point in the kernel
 
 // 16-byte slot of V^T row d that holds the row's chunk c is c ^ v_swizzle(d): distinct over any 8 consecutive rows, and
@@ -109,15 +110,19 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
     voff[i] = (uint32_t)d * (uint32_t)(p.T * 2) + (uint32_t)(((lane & 7) ^ v_swizzle(d)) << 4);
   }
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;
-  auto issue = [&](int j) __attribute__((always_inline)) {
-    const unsigned char* kb = kp + (size_t)j * kKB * p.k_st;
-    const unsigned char* vb = vtp + (size_t)j * kKB * 2;
-    const uint32_t kdst = lds_base + (uint32_t)((j & 1) * kKBytes), vdst = lds_base + (uint32_t)(2 * kKBytes + (j & 1) * kVBytes);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      at_async_copy_16(kb, koff[i], kdst + (uint32_t)((wave * 4 + i) * 1024));
-      at_async_copy_16(vb, voff[i], vdst + (uint32_t)((wave * 4 + i) * kVGroup));
+  // copy c (0..7) of key block j: 0-3 K, 4-7 V^T
+  auto issue_one = [&](int j, int c) __attribute__((always_inline)) {
+    const int i = c & 3;
+    if (c < 4) {
+      at_async_copy_16(kp + (size_t)j * kKB * p.k_st, koff[i], lds_base + (uint32_t)((j & 1) * kKBytes + (wave * 4 + i) * 1024));
+    } else {
+      at_async_copy_16(vtp + (size_t)j * kKB * 2, voff[i],
+                       lds_base + (uint32_t)(2 * kKBytes + (j & 1) * kVBytes + (wave * 4 + i) * kVGroup));
     }
+  };
+  auto issue = [&](int j) __attribute__((always_inline)) {
+#pragma unroll
+    for (int c = 0; c < 8; ++c) issue_one(j, c);
   };
 
   f32x16_t o[4];
@@ -132,33 +137,41 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
   for (int j = 0; j < nblk; ++j) {
     at_wait_vmcnt<0>();  // this wavefront's copies of block j have landed
     asm volatile("s_barrier" ::: "memory");  // ... everyone's have, and everyone has finished with block j - 1's buffers
-    if (j + 1 < nblk) issue(j + 1);
+    const bool more = j + 1 < nblk;
     const int key0 = j * kKB;
-    if (key0 > q0 + 31) continue;  // every key of the block lies after every query of this wavefront
+    const bool skip = key0 > q0 + 31;  // every key of the block lies after every query of this wavefront
+    if (skip && more) issue(j + 1);
+    if (skip) continue;
     const unsigned char* Kb = lds + (j & 1) * kKBytes;
     const unsigned char* Vb = lds + 2 * kKBytes + (j & 1) * kVBytes;
 
-    // every fragment read of a phase is issued before the phase's first matrix instruction, in the order the
-    // instructions take them, so a wavefront waits one LDS latency per phase, not one per instruction
-    bf16x8_t kf[16];
-#pragma unroll
-    for (int s = 0; s < 8; ++s)
+    // S^T = K Q^T: the K fragments are read kKRing - 1 contraction steps ahead of the matrix instructions that take them,
+    // and the wavefront's 8 copies of the next key block go out between those instructions (issued in one run they
+    // hold the wavefront for as long as the address path takes to accept them)
+    bf16x8_t kf[kKRing][2];  // ring: step s uses kf[s % kKRing]
+    auto read_k = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
         const int row = t * 32 + l32;
-        kf[2 * s + t] = *(const bf16x8_t*)(Kb + row * 256 + (((2 * s + g) ^ (row & 15)) << 4));
+        kf[s % kKRing][t] = *(const bf16x8_t*)(Kb + row * 256 + (((2 * s + g) ^ (row & 15)) << 4));
       }
-    __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll
+    for (int s = 0; s < kKRing - 1; ++s) read_k(s);
     f32x16_t sc[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) sc[t][r] = 0.0f;
-#pragma unroll
-    for (int s = 0; s < 8; ++s)
-#pragma unroll
-      for (int t = 0; t < 2; ++t) sc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[2 * s + t], qf[s], sc[t], 0, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) sc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s % kKRing][t], qf[s], sc[t], 0, 0, 0);
+      if (s + kKRing - 1 < 8) read_k(s + kKRing - 1);
+      if (more) issue_one(j + 1, s);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     // V^T fragments of the first two steps of the second product: their latency passes behind the exponentials
     bf16x8_t vf[2][4];
     auto read_v = [&](int s, bf16x8_t* dst) __attribute__((always_inline)) {
