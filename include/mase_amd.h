@@ -341,6 +341,16 @@ int mase_attention_causal(const void* q, const void* k, const void* v, void* out
                           size_t k_stride_b, size_t k_stride_h, size_t k_stride_t, size_t v_stride_b, size_t v_stride_h,
                           size_t v_stride_t, size_t o_stride_b, size_t o_stride_h, size_t o_stride_t, int dtype,
                           float scaling, void* workspace, size_t workspace_bytes, void* stream);
+/* The same with the result written as its MXINT quantize-dequantize (blocks of 32 along the head dimension, element_bits
+ * wide, E8M0 scales; log2_tab as for mase_mxint_qdq in bf16): what the LinearMXInt that reads the
+ * [batch, tokens, heads * 128] result would compute from it in a pass of its own (nn/quantized/modules/linear.py:956-972),
+ * bit for bit. */
+int mase_attention_causal_mxint(const void* q, const void* k, const void* v, void* out, size_t batch, size_t heads,
+                                size_t tokens, size_t head_dim, size_t q_stride_b, size_t q_stride_h, size_t q_stride_t,
+                                size_t k_stride_b, size_t k_stride_h, size_t k_stride_t, size_t v_stride_b,
+                                size_t v_stride_h, size_t v_stride_t, size_t o_stride_b, size_t o_stride_h,
+                                size_t o_stride_t, int dtype, float scaling, int element_bits, const uint32_t* log2_tab,
+                                void* workspace, size_t workspace_bytes, void* stream);
 
 /* Rotary embedding out = x * cos + rotate_half(x) * sin for x [B, H, T, D] with the last dimension contiguous and
  * element strides (x_stride_b, x_stride_h, x_stride_t); out has the same strides; cos / sin tables [B or 1, T, D] with

@@ -19,6 +19,7 @@
 // inside every group of 16 keys (order 0-3, 8-11, 4-7, 12-15), so that the 8 keys of a lane's contraction slots are one
 // 16-byte chunk (chunk 2 s + g of the 64-key row) and the V^T fragments are read like the K fragments.
 #include "common.hpp"
+#include "mxint_core.hpp"
 
 namespace mase {
 namespace {
@@ -45,6 +46,12 @@ __device__ __forceinline__ float max_with_other_half(float v) {
   return fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
 }
 
+__device__ __forceinline__ uint32_t umax_with_other_half(uint32_t v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  const unsigned a = r[0], b = r[1];
+  return max(a, b);
+}
+
 __device__ __forceinline__ int v_swizzle(int d) { return (d & 7) ^ ((d >> 3) & 1); }
 constexpr int kAttnLds = 2 * kKBytes + 2 * kVBytes;
 
@@ -67,8 +74,14 @@ struct AttnParams {
   size_t q_sb, q_sh, k_sb, k_sh, o_sb, o_sh;  // byte strides of batch and head
   uint32_t q_st, k_st, o_st;                  // byte strides of a token
   float c;                                    // scaling * log2(e)
+  MxintParams mx;                             // MX instantiation only
 };
 
+// MX: the output is written as the MXINT quantize-dequantize of the bf16 result, blocks of 32 along the head dimension
+// (what a LinearMXInt reading the [batch, tokens, heads * 128] result would compute in a pass of its own,
+// nn/quantized/modules/linear.py:956-972): the 32 values of a block are the 16 accumulator registers of one d tile in
+// lane l and in lane l ^ 32.
+template <bool MX>
 __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int lane = threadIdx.x & 63;
@@ -248,14 +261,38 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
   // register r of tile dt is d = 32 dt + 8 (r / 4) + 4 g + r % 4: four consecutive d per group of four registers
   unsigned char* op = p.out + (size_t)b * p.o_sb + (size_t)h * p.o_sh + (size_t)qi * p.o_st;
 #pragma unroll
-  for (int dt = 0; dt < 4; ++dt)
+  for (int dt = 0; dt < 4; ++dt) {
+    float y[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) y[r] = o[dt][r] * inv;
+    if constexpr (MX) {
+      uint32_t mbits = 0;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        y[r] = DTypeTraits<MASE_DT_BF16>::round(y[r]);  // the quantizer reads the stored bf16 value
+        mbits = max(mbits, f2bits(y[r]) & 0x7FFFFFFFu);
+      }
+      mbits = umax_with_other_half(mbits);
+      int k = 0, kc = 0;
+      const int state = block_exponent<MASE_DT_BF16>(mbits, p.mx, k, kc);
+      if (state == 0) {
+        const int up = p.mx.qshift - k, dn = kc - p.mx.qshift;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) y[r] = ldexpf(fminf(fmaxf(rintf(ldexpf(y[r], up)), p.mx.lo), p.mx.hi), dn);
+      } else {
+        int code;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) y[r] = mxint_element<MASE_DT_BF16>(y[r], state, k, kc, p.mx, code);
+      }
+    }
 #pragma unroll
     for (int qq = 0; qq < 4; ++qq) {
       uint2 w;
-      w.x = f32x2_to_bf16x2_bits(o[dt][4 * qq] * inv, o[dt][4 * qq + 1] * inv);
-      w.y = f32x2_to_bf16x2_bits(o[dt][4 * qq + 2] * inv, o[dt][4 * qq + 3] * inv);
+      w.x = f32x2_to_bf16x2_bits(y[4 * qq], y[4 * qq + 1]);
+      w.y = f32x2_to_bf16x2_bits(y[4 * qq + 2], y[4 * qq + 3]);
       *(uint2*)(op + (32 * dt + 8 * qq + 4 * g) * 2) = w;
     }
+  }
 }
 
 // vt[bh][d][perm(t)] = v[b][t][h][d], perm swapping the middle two quads of every 16 tokens: tiles of 64 tokens x 128 d
@@ -298,13 +335,14 @@ extern "C" size_t mase_attention_causal_workspace_bytes(size_t batch, size_t hea
   return batch * heads * tokens * head_dim * 2;
 }
 
-extern "C" int mase_attention_causal(const void* q, const void* k, const void* v, void* out, size_t batch, size_t heads,
-                                     size_t tokens, size_t head_dim, size_t q_stride_b, size_t q_stride_h,
-                                     size_t q_stride_t, size_t k_stride_b, size_t k_stride_h, size_t k_stride_t,
-                                     size_t v_stride_b, size_t v_stride_h, size_t v_stride_t, size_t o_stride_b,
-                                     size_t o_stride_h, size_t o_stride_t, int dtype, float scaling, void* workspace,
-                                     size_t workspace_bytes, void* stream) {
-  using namespace mase;
+namespace mase {
+namespace {
+int attention_causal_impl(const void* q, const void* k, const void* v, void* out, size_t batch, size_t heads,
+                          size_t tokens, size_t head_dim, size_t q_stride_b, size_t q_stride_h,
+                          size_t q_stride_t, size_t k_stride_b, size_t k_stride_h, size_t k_stride_t,
+                          size_t v_stride_b, size_t v_stride_h, size_t v_stride_t, size_t o_stride_b,
+                          size_t o_stride_h, size_t o_stride_t, int dtype, float scaling, int element_bits,
+                          const uint32_t* log2_tab, void* workspace, size_t workspace_bytes, void* stream) {
   if (batch == 0 || heads == 0 || tokens == 0) return MASE_OK;
   if (q == nullptr || k == nullptr || v == nullptr || out == nullptr) return MASE_ERR_NULL;
   if (dtype != MASE_DT_BF16) return MASE_ERR_DTYPE;
@@ -323,10 +361,13 @@ extern "C" int mase_attention_causal(const void* q, const void* k, const void* v
   const size_t need = mase_attention_causal_workspace_bytes(batch, heads, tokens, head_dim);
   if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace)) return MASE_ERR_WORKSPACE;
   hipStream_t st = (hipStream_t)stream;
+  const bool mx = element_bits != 0;
   static bool attr_set = false;
   if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)attn_causal_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLds) !=
-        hipSuccess)
+    if (hipFuncSetAttribute((const void*)attn_causal_fwd_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLds) !=
+            hipSuccess ||
+        hipFuncSetAttribute((const void*)attn_causal_fwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLds) !=
+            hipSuccess)
       return MASE_ERR_LAUNCH;
     attr_set = true;
   }
@@ -346,6 +387,45 @@ extern "C" int mase_attention_causal(const void* q, const void* k, const void* v
   p.k_sb = k_stride_b * 2; p.k_sh = k_stride_h * 2; p.k_st = (uint32_t)(k_stride_t * 2);
   p.o_sb = o_stride_b * 2; p.o_sh = o_stride_h * 2; p.o_st = (uint32_t)(o_stride_t * 2);
   p.c = scaling * 1.4426950408889634f;
-  hipLaunchKernelGGL(attn_causal_fwd_kernel, dim3((unsigned)(BH * (T / kQB))), dim3(256), kAttnLds, st, p);
+  if (mx) {
+    if (element_bits < 2 || element_bits > 24 || log2_tab == nullptr) return MASE_ERR_PARAM;
+    p.mx.qshift = element_bits - 1;
+    p.mx.bias = 127;
+    p.mx.scale_max = 255;
+    p.mx.lo = mase_round_scalar_to_dtype(-(double)(1 << (element_bits - 1)), dtype);
+    p.mx.hi = mase_round_scalar_to_dtype((double)((1 << (element_bits - 1)) - 1), dtype);
+    p.mx.tab = log2_tab;
+    hipLaunchKernelGGL(attn_causal_fwd_kernel<true>, dim3((unsigned)(BH * (T / kQB))), dim3(256), kAttnLds, st, p);
+  } else {
+    p.mx = MxintParams{};
+    hipLaunchKernelGGL(attn_causal_fwd_kernel<false>, dim3((unsigned)(BH * (T / kQB))), dim3(256), kAttnLds, st, p);
+  }
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+}  // namespace
+}  // namespace mase
+
+extern "C" int mase_attention_causal(const void* q, const void* k, const void* v, void* out, size_t batch, size_t heads,
+                                     size_t tokens, size_t head_dim, size_t q_stride_b, size_t q_stride_h,
+                                     size_t q_stride_t, size_t k_stride_b, size_t k_stride_h, size_t k_stride_t,
+                                     size_t v_stride_b, size_t v_stride_h, size_t v_stride_t, size_t o_stride_b,
+                                     size_t o_stride_h, size_t o_stride_t, int dtype, float scaling, void* workspace,
+                                     size_t workspace_bytes, void* stream) {
+  return mase::attention_causal_impl(q, k, v, out, batch, heads, tokens, head_dim, q_stride_b, q_stride_h, q_stride_t,
+                                     k_stride_b, k_stride_h, k_stride_t, v_stride_b, v_stride_h, v_stride_t, o_stride_b,
+                                     o_stride_h, o_stride_t, dtype, scaling, 0, nullptr, workspace, workspace_bytes, stream);
+}
+
+extern "C" int mase_attention_causal_mxint(const void* q, const void* k, const void* v, void* out, size_t batch,
+                                           size_t heads, size_t tokens, size_t head_dim, size_t q_stride_b,
+                                           size_t q_stride_h, size_t q_stride_t, size_t k_stride_b, size_t k_stride_h,
+                                           size_t k_stride_t, size_t v_stride_b, size_t v_stride_h, size_t v_stride_t,
+                                           size_t o_stride_b, size_t o_stride_h, size_t o_stride_t, int dtype,
+                                           float scaling, int element_bits, const uint32_t* log2_tab, void* workspace,
+                                           size_t workspace_bytes, void* stream) {
+  if (element_bits == 0) return MASE_ERR_PARAM;
+  return mase::attention_causal_impl(q, k, v, out, batch, heads, tokens, head_dim, q_stride_b, q_stride_h, q_stride_t,
+                                     k_stride_b, k_stride_h, k_stride_t, v_stride_b, v_stride_h, v_stride_t, o_stride_b,
+                                     o_stride_h, o_stride_t, dtype, scaling, element_bits, log2_tab, workspace,
+                                     workspace_bytes, stream);
 }

@@ -401,10 +401,12 @@ def attention_causal_supported(q: Tensor, k: Tensor, v: Tensor) -> bool:
     return True
 
 
-def attention_causal(q: Tensor, k: Tensor, v: Tensor, scaling: float | None = None) -> Tensor:
+def attention_causal(q: Tensor, k: Tensor, v: Tensor, scaling: float | None = None, mxint_bits: int | None = None) -> Tensor:
     """``softmax(q k^T * scaling + causal mask) v`` for bf16 [batch, heads, tokens, 128] operands in one pass over the keys
     (``mase_attention_causal``).  Returned as [batch, heads, tokens, 128] over memory laid out [batch, tokens, heads,
-    128], so that ``out.transpose(1, 2).reshape(batch, tokens, heads * 128)`` is a view."""
+    128], so that ``out.transpose(1, 2).reshape(batch, tokens, heads * 128)`` is a view.  ``mxint_bits``: the result is
+    written as ``mxint_quantizer(result, block 32 along the head dimension, mxint_bits)``, the form a ``LinearMXInt``
+    that reads it would compute itself (``mase_attention_causal_mxint``)."""
     _lib.require_device(q, "attention_causal")
     lib = _lib.load()
     assert attention_causal_supported(q, k, v)
@@ -414,10 +416,15 @@ def attention_causal(q: Tensor, k: Tensor, v: Tensor, scaling: float | None = No
     out = torch.empty((B, T, H, D), dtype=q.dtype, device=q.device).transpose(1, 2)
     need = lib.mase_attention_causal_workspace_bytes(B, H, T, D)
     ws = torch.empty(need, dtype=torch.uint8, device=q.device)
-    rc = lib.mase_attention_causal(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, H, T, D,
-                                   q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
-                                   v.stride(0), v.stride(1), v.stride(2), out.stride(0), out.stride(1), out.stride(2),
-                                   _lib.dtype_code(q), float(scaling), ws.data_ptr(), need, _lib.stream_ptr(q))
+    args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, H, T, D,
+            q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+            v.stride(0), v.stride(1), v.stride(2), out.stride(0), out.stride(1), out.stride(2),
+            _lib.dtype_code(q), float(scaling))
+    if mxint_bits is None:
+        rc = lib.mase_attention_causal(*args, ws.data_ptr(), need, _lib.stream_ptr(q))
+    else:
+        rc = lib.mase_attention_causal_mxint(*args, int(mxint_bits), log2_table(q.dtype, q.device).data_ptr(), ws.data_ptr(), need,
+                                             _lib.stream_ptr(q))
     _lib.check(rc, "mase_attention_causal")
     return out
 

@@ -65,11 +65,13 @@ def rope_tables(seq_len: int, head_dim: int, theta: float, device, dtype):
     return emb.cos().to(dtype), emb.sin().to(dtype)
 
 
-def causal_attention(q, k, v):
+def causal_attention(q, k, v, mxint_bits=None):
     """softmax(q k^T / sqrt(d) + causal mask) v: the one-pass kernel of this package where it applies (bf16, head
-    dimension 128, a multiple of 128 tokens, no gradient), the library's scaled_dot_product_attention otherwise"""
+    dimension 128, a multiple of 128 tokens, no gradient), the library's scaled_dot_product_attention otherwise.
+    ``mxint_bits`` (only where the kernel applies): the result in the MXINT form of the Linear that reads it."""
     if q.is_cuda and _ops.attention_causal_supported(q, k, v):
-        return _ops.attention_causal(q, k, v)
+        return _ops.attention_causal(q, k, v, mxint_bits=mxint_bits)
+    assert mxint_bits is None
     return F.scaled_dot_product_attention(q, k, v, is_causal=True)
 
 
@@ -145,9 +147,17 @@ class DecoderLayer(nn.Module):
         else:
             q = q * cos + rotate_half(q) * sin
             k = k * cos + rotate_half(k) * sin
-        a = self.attention_fn(q, k, v)
-        a = a.transpose(1, 2).reshape(B, T, cfg.num_heads * cfg.head_dim)
-        x = self._project_add(self.o_proj, a, x)
+        bits = None
+        if (self.fuse_producers and self.attention_fn is causal_attention and q.is_cuda and not torch.is_grad_enabled()
+                and _ops.attention_causal_supported(q, k, v)):
+            bits = shared_mxint_width(x, (self.o_proj,))  # o_proj's input: same dtype and device as x, head_dim % 32 == 0
+        if bits is not None:
+            a = causal_attention(q, k, v, mxint_bits=bits).transpose(1, 2).reshape(B, T, cfg.num_heads * cfg.head_dim)
+            x = self._project_add(self.o_proj, a, x, prepared=a.reshape(-1, a.shape[-1]))
+        else:
+            a = self.attention_fn(q, k, v)
+            a = a.transpose(1, 2).reshape(B, T, cfg.num_heads * cfg.head_dim)
+            x = self._project_add(self.o_proj, a, x)
         gate, up = self._norm_then_project(self.post_attention_layernorm, x, (self.gate_proj, self.up_proj))
         if gate.is_cuda and _ops.silu_mul_supported(gate, up):
             bits = shared_mxint_width(gate, (self.down_proj,)) if self.fuse_producers and gate.shape[-1] % 32 == 0 else None

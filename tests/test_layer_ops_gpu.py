@@ -154,6 +154,7 @@ def test_causal_attention_one_pass(dev, B, H, T, layout):
     bf16 operands: bound 1e-2 of the output range (the probabilities are rounded to bf16 before the second product and
     the output is bf16); the library's own kernel is held to the same bound for comparison.  Operands as strided views
     of [batch, tokens, heads, 128] memory (what the projections produce) and contiguous [batch, heads, tokens, 128]."""
+    from helpers import assert_bits_equal
     from mase_amd.quantizers import _ops
 
     g = torch.Generator().manual_seed(B * 1000 + T)
@@ -179,6 +180,11 @@ def test_causal_attention_one_pass(dev, B, H, T, layout):
         assert e < 1e-2
         # the first query attends to the first key only: its output row is v[0]
         assert torch.equal(got[:, :, 0], v[:, :, 0])
+        # the MXINT output form: the quantizer's result on the stored bf16 output (oracle on the CPU), bit for bit
+        for bits in (8, 4):
+            gq = _ops.attention_causal(q, k, v, scaling, mxint_bits=bits).transpose(1, 2).reshape(B, T, H * 128)
+            want = O.mxint_quantizer(got.transpose(1, 2).reshape(B, T, H * 128).cpu(), 32, bits, block_dim=-1)
+            assert_bits_equal(gq, want, f"attention output as MXINT{bits}")
     assert not _ops.attention_causal_supported(q[:, :, :100], k[:, :, :100], v[:, :, :100])
     assert not _ops.attention_causal_supported(q.float(), k.float(), v.float())
     assert not _ops.attention_causal_supported(q[..., :64], k[..., :64], v[..., :64])
