@@ -333,14 +333,13 @@ int mase_silu_mul_mxint(const void* gate, const void* up, void* out, size_t nume
  * given by element strides of batch / head / token (last dimension contiguous, strides multiples of 8), out likewise;
  * tokens % 128 == 0.  Scores and softmax statistics in fp32, probabilities rounded to bf16 before the product with v
  * (as the tensor operations of the reference's Llama attention core do on unquantized operands,
- * models/llama/modeling_llama.py:362-480); no [tokens, tokens] matrix is materialised.  workspace: at least
- * mase_attention_causal_workspace_bytes bytes (v transposed), 16-byte aligned; 0 from that function = unsupported. */
-size_t mase_attention_causal_workspace_bytes(size_t batch, size_t heads, size_t tokens, size_t head_dim);
+ * models/llama/modeling_llama.py:362-480); no [tokens, tokens] matrix is materialised and no workspace is needed.
+ * MASE_ERR_SHAPE for another head dimension or token count, MASE_ERR_DTYPE for another dtype. */
 int mase_attention_causal(const void* q, const void* k, const void* v, void* out, size_t batch, size_t heads,
                           size_t tokens, size_t head_dim, size_t q_stride_b, size_t q_stride_h, size_t q_stride_t,
                           size_t k_stride_b, size_t k_stride_h, size_t k_stride_t, size_t v_stride_b, size_t v_stride_h,
                           size_t v_stride_t, size_t o_stride_b, size_t o_stride_h, size_t o_stride_t, int dtype,
-                          float scaling, void* workspace, size_t workspace_bytes, void* stream);
+                          float scaling, void* stream);
 /* The same with the result written as its MXINT quantize-dequantize (blocks of 32 along the head dimension, element_bits
  * wide, E8M0 scales; log2_tab as for mase_mxint_qdq in bf16): what the LinearMXInt that reads the
  * [batch, tokens, heads * 128] result would compute from it in a pass of its own (nn/quantized/modules/linear.py:956-972),
@@ -350,7 +349,7 @@ int mase_attention_causal_mxint(const void* q, const void* k, const void* v, voi
                                 size_t k_stride_b, size_t k_stride_h, size_t k_stride_t, size_t v_stride_b,
                                 size_t v_stride_h, size_t v_stride_t, size_t o_stride_b, size_t o_stride_h,
                                 size_t o_stride_t, int dtype, float scaling, int element_bits, const uint32_t* log2_tab,
-                                void* workspace, size_t workspace_bytes, void* stream);
+                                void* stream);
 
 /* Rotary embedding out = x * cos + rotate_half(x) * sin for x [B, H, T, D] with the last dimension contiguous and
  * element strides (x_stride_b, x_stride_h, x_stride_t); out has the same strides; cos / sin tables [B or 1, T, D] with

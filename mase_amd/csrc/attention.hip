@@ -6,7 +6,7 @@
 // row sum divides once at the end, so results agree with the tensor operations to bf16 rounding, not bit for bit.
 //
 // One work-group (4 wavefronts) owns 128 queries of one (batch, head); a wavefront owns 32 of them.  Key blocks of 64
-// are streamed through LDS (K as [key][128 d], V transposed as [d][64 keys], both double-buffered with async copies).
+// are streamed through LDS (K and V as [key][128 d] rows, both double-buffered with async copies).
 // Per key block a wavefront computes S^T = K Q^T with v_mfma_f32_32x32x16_bf16 (A = K rows from LDS, B = its Q
 // fragments, kept in registers for the whole kernel): a lane then holds, for ONE query (lane % 32), the scores of 32 of
 // the 64 keys in its accumulator registers, so the softmax statistics are in-lane but for one exchange with lane ^ 32.
@@ -15,9 +15,8 @@
 // s / 2, i.e. keys 16 s + 4 g + 8 (j / 4) + j % 4).  Two work-groups fit a CU (64 KB of LDS, under 256 registers),
 // so one wavefront's exponentials overlap the other's matrix instructions.
 //
-// V^T is made by a transposing pre-pass into a caller workspace [batch * heads][128][T] whose key axis is permuted
-// inside every group of 16 keys (order 0-3, 8-11, 4-7, 12-15), so that the 8 keys of a lane's contraction slots are one
-// 16-byte chunk (chunk 2 s + g of the 64-key row) and the V^T fragments are read like the K fragments.
+// The V^T fragments of the second product (lane = d, 8 keys each) are made from V's rows by the transposing LDS read
+// ds_read_b64_tr_b16, so V needs no transposed copy in memory.
 #include "common.hpp"
 #include "mxint_core.hpp"
 
@@ -27,16 +26,16 @@ namespace {
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef __attribute__((address_space(3))) void* lptr_t;
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef short s16x8_t __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4_t lds_s16x4_t;
 
 constexpr int kQB = 128, kKB = 64, kHD = 128;
 constexpr int kKBytes = kKB * kHD * 2;       // 16 KB: 64 key rows of 256 bytes
-constexpr int kVGroup = 8 * 128;             // 8 rows (d) of 128 bytes (64 keys): one async copy of a wavefront
-constexpr int kVBytes = 16 * kVGroup;
+constexpr int kVBytes = kKBytes;             // V like K: 64 key rows of 256 bytes
 constexpr int kKRing = 5;                    // K fragment pairs in flight or in use: reads run 4 contraction steps ahead
 constexpr float kGrow = 8.0f;                // see the softmax reference point in the kernel
 
-// 16-byte slot of V^T row d that holds the row's chunk c is c ^ v_swizzle(d): distinct over any 8 consecutive rows, and
-// over the even and the odd rows of any 16 (rows are 128 bytes, so two rows span 64 four-byte banks)
 // max of a lane's value and lane ^ 32's, without a trip through the LDS queue (which would wait for the fragment reads
 // in flight)
 __device__ __forceinline__ float max_with_other_half(float v) {
@@ -52,7 +51,6 @@ __device__ __forceinline__ uint32_t umax_with_other_half(uint32_t v) {
   return max(a, b);
 }
 
-__device__ __forceinline__ int v_swizzle(int d) { return (d & 7) ^ ((d >> 3) & 1); }
 constexpr int kAttnLds = 2 * kKBytes + 2 * kVBytes;
 
 // lane i's 16 bytes at base + off_i land at LDS address lds_addr + 16 * i; tracked by hand with at_wait_vmcnt
@@ -68,11 +66,11 @@ __device__ __forceinline__ void at_wait_vmcnt() {
 struct AttnParams {
   const unsigned char* q;
   const unsigned char* k;
-  const unsigned char* vt;  // [batch * heads][128][T] bf16
+  const unsigned char* v;
   unsigned char* out;
   int BH, H, T;
-  size_t q_sb, q_sh, k_sb, k_sh, o_sb, o_sh;  // byte strides of batch and head
-  uint32_t q_st, k_st, o_st;                  // byte strides of a token
+  size_t q_sb, q_sh, k_sb, k_sh, v_sb, v_sh, o_sb, o_sh;  // byte strides of batch and head
+  uint32_t q_st, k_st, v_st, o_st;                        // byte strides of a token
   float c;                                    // scaling * log2(e)
   MxintParams mx;                             // MX instantiation only
 };
@@ -89,7 +87,7 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
   const int l32 = lane & 31, g = lane >> 5;
   // Work-groups are handed to the 8 XCDs in turn (blockIdx % 8), each XCD with an L2 of its own.  All query blocks of
   // one (batch, head) go to one XCD, one after the other and the ones with the most keys first: they run at the same
-  // time and walk the keys from the start together, so K and V^T come from HBM once and from that L2 afterwards.
+  // time and walk the keys from the start together, so K and V come from HBM once and from that L2 afterwards.
   const int n_qb = p.T / kQB;
   int bh, qb;
   if (p.BH % 8 == 0) {
@@ -103,7 +101,7 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
   const int b = bh / p.H, h = bh % p.H;
   const unsigned char* qp = p.q + (size_t)b * p.q_sb + (size_t)h * p.q_sh;
   const unsigned char* kp = p.k + (size_t)b * p.k_sb + (size_t)h * p.k_sh;
-  const unsigned char* vtp = p.vt + (size_t)bh * ((size_t)kHD * p.T * 2);
+  const unsigned char* vp = p.v + (size_t)b * p.v_sb + (size_t)h * p.v_sh;
   const int q0 = qb * kQB + wave * 32;  // this wavefront's first query
   const int qi = q0 + l32;              // this lane's query
 
@@ -111,26 +109,25 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
 #pragma unroll
   for (int s = 0; s < 8; ++s) qf[s] = *(const bf16x8_t*)(qp + (size_t)qi * p.q_st + (s * 16 + g * 8) * 2);
 
-  // async copies of one key block: 4 of K (4 rows of 256 bytes each) and 4 of V^T (8 rows of 128 bytes) per wavefront.
-  // LDS position (row, 16-byte slot) holds the row's chunk slot ^ (row % 16) (K) / slot ^ v_swizzle(row) (V^T), so that the
+  // async copies of one key block: 4 of K and 4 of V (4 rows of 256 bytes each) per wavefront.
+  // LDS position (row, 16-byte slot) holds the row's chunk slot ^ (row % 16), so that the
   // fragment reads of 32 lanes (32 rows, same chunk) spread over the banks.
   uint32_t koff[4], voff[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int krow = (wave * 4 + i) * 4 + (lane >> 4);
     koff[i] = (uint32_t)krow * p.k_st + (uint32_t)(((lane & 15) ^ (krow & 15)) << 4);
-    const int d = (wave * 4 + i) * 8 + (lane >> 3);
-    voff[i] = (uint32_t)d * (uint32_t)(p.T * 2) + (uint32_t)(((lane & 7) ^ v_swizzle(d)) << 4);
+    voff[i] = (uint32_t)krow * p.v_st + (uint32_t)(((lane & 15) ^ (krow & 15)) << 4);
   }
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;
-  // copy c (0..7) of key block j: 0-3 K, 4-7 V^T
+  // copy c (0..7) of key block j: 0-3 K, 4-7 V
   auto issue_one = [&](int j, int c) __attribute__((always_inline)) {
     const int i = c & 3;
     if (c < 4) {
       at_async_copy_16(kp + (size_t)j * kKB * p.k_st, koff[i], lds_base + (uint32_t)((j & 1) * kKBytes + (wave * 4 + i) * 1024));
     } else {
-      at_async_copy_16(vtp + (size_t)j * kKB * 2, voff[i],
-                       lds_base + (uint32_t)(2 * kKBytes + (j & 1) * kVBytes + (wave * 4 + i) * kVGroup));
+      at_async_copy_16(vp + (size_t)j * kKB * p.v_st, voff[i],
+                       lds_base + (uint32_t)(2 * kKBytes + (j & 1) * kVBytes + (wave * 4 + i) * 1024));
     }
   };
   auto issue = [&](int j) __attribute__((always_inline)) {
@@ -161,6 +158,28 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
     // S^T = K Q^T: the K fragments are read kKRing - 1 contraction steps ahead of the matrix instructions that take them,
     // and the wavefront's 8 copies of the next key block go out between those instructions (issued in one run they
     // hold the wavefront for as long as the address path takes to accept them)
+    // V fragments (A operand of O^T += V^T P^T: lane = d, 8 keys) come from V's natural [key][d] rows by transposing
+    // reads: in a group of 16 lanes, lane 4 e + a points at 4 consecutive d (8 bytes) of key row e, and lane i
+    // receives element i % 4 of the windows of lanes i / 4, 4 + i / 4, 8 + i / 4, 12 + i / 4: with the windows at
+    // d = c0 + 4 a of keys k0 + e, lane i gets d = c0 + i of keys k0 .. k0 + 3.  Two reads (keys k0 .., k0 + 8 ..) make a
+    // fragment.  The reads of steps 0 and 1 go out between the matrix instructions of the first product, those of
+    // steps 2 and 3 between the exponentials.
+    bf16x8_t vf[4][4];
+    auto read_v_one = [&](int s, int dt) __attribute__((always_inline)) {
+      const int dbyte = (dt * 32 + (l32 & 16) + 4 * (lane & 3)) * 2;
+      const int row0 = 16 * s + 4 * g + ((lane & 15) >> 2), row1 = row0 + 8;
+      const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (lds_s16x4_t*)(lptr_t)(Vb + row0 * 256 + (((dbyte >> 4) ^ (row0 & 15)) << 4) + (dbyte & 8)));
+      const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (lds_s16x4_t*)(lptr_t)(Vb + row1 * 256 + (((dbyte >> 4) ^ (row1 & 15)) << 4) + (dbyte & 8)));
+      s16x8_t both;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        both[e] = lo[e];
+        both[4 + e] = hi[e];
+      }
+      vf[s][dt] = __builtin_bit_cast(bf16x8_t, both);
+    };
     bf16x8_t kf[kKRing][2];  // ring: step s uses kf[s % kKRing]
     auto read_k = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
@@ -182,21 +201,10 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
 #pragma unroll
       for (int t = 0; t < 2; ++t) sc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s % kKRing][t], qf[s], sc[t], 0, 0, 0);
       if (s + kKRing - 1 < 8) read_k(s + kKRing - 1);
+      read_v_one(s >> 2, s & 3);
       if (more) issue_one(j + 1, s);
       __builtin_amdgcn_sched_barrier(0);
     }
-    // V^T fragments of the first two steps of the second product: their latency passes behind the exponentials
-    bf16x8_t vf[2][4];
-    auto read_v = [&](int s, bf16x8_t* dst) __attribute__((always_inline)) {
-#pragma unroll
-      for (int dt = 0; dt < 4; ++dt) {
-        const int d = dt * 32 + l32;
-        dst[dt] = *(const bf16x8_t*)(Vb + d * 128 + (((2 * s + g) ^ v_swizzle(d)) << 4));
-      }
-    };
-    read_v(0, vf[0]);
-    read_v(1, vf[1]);
-    __builtin_amdgcn_sched_barrier(0);
     // register r of tile t is key key0 + 32 t + 8 (r / 4) + 4 g + r % 4
     if (key0 + kKB - 1 > q0) {  // the block reaches past this wavefront's first query: mask
 #pragma unroll
@@ -235,6 +243,10 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
       for (int r = 0; r < 16; ++r) {
         sc[t][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[t][r], p.c, -mc));
         psum += sc[t][r];
+        if ((r & 3) == 3) {
+          read_v_one(2 + t, r >> 2);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
     lsum += psum;
 #pragma unroll
@@ -250,8 +262,7 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
     for (int s = 0; s < 4; ++s) {
       const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pw[s]);
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[s & 1][dt], pf, o[dt], 0, 0, 0);
-      if (s < 2) read_v(s + 2, vf[s & 1]);
+      for (int dt = 0; dt < 4; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[s][dt], pf, o[dt], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -295,45 +306,8 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
   }
 }
 
-// vt[bh][d][perm(t)] = v[b][t][h][d], perm swapping the middle two quads of every 16 tokens: tiles of 64 tokens x 128 d
-// through LDS (rows padded to 264 bytes)
-__global__ __launch_bounds__(256) void attn_transpose_v_kernel(const unsigned char* __restrict__ v, unsigned char* __restrict__ vt,
-                                                               int H, int T, size_t v_sb, size_t v_sh, uint32_t v_st) {
-  __shared__ __attribute__((aligned(16))) unsigned char tile[64 * 264];
-  const int bh = blockIdx.y, t0 = blockIdx.x * 64;
-  const int b = bh / H, h = bh % H;
-  const unsigned char* src = v + (size_t)b * v_sb + (size_t)h * v_sh + (size_t)t0 * v_st;
-  const int tid = threadIdx.x;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {  // 1024 chunks of 16 bytes: token = chunk / 16, slot = chunk % 16
-    const int c = i * 256 + tid, tok = c >> 4, slot = c & 15;
-    *(uint4*)(tile + tok * 264 + slot * 16) = *(const uint4*)(src + (size_t)tok * v_st + slot * 16);
-  }
-  __syncthreads();
-  unsigned char* dst = vt + (size_t)bh * ((size_t)kHD * T * 2) + (size_t)t0 * 2;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {  // 1024 chunks of 8 tokens: d = chunk / 8; chunk % 8 = 2 (group of 16) + half
-    const int c = i * 256 + tid, d = c >> 3, tg = c & 7;
-    const int tok0 = (tg >> 1) * 16 + (tg & 1) * 4;  // tokens tok0 .. + 3 and tok0 + 8 .. + 11
-    uint32_t w[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int tok = tok0 + (e >> 1) * 8 + (e & 1) * 2;
-      const uint32_t lo = *(const uint16_t*)(tile + tok * 264 + d * 2);
-      const uint32_t hi = *(const uint16_t*)(tile + (tok + 1) * 264 + d * 2);
-      w[e] = lo | (hi << 16);
-    }
-    *(uint4*)(dst + (size_t)d * T * 2 + tg * 16) = make_uint4(w[0], w[1], w[2], w[3]);
-  }
-}
-
 }  // namespace
 }  // namespace mase
-
-extern "C" size_t mase_attention_causal_workspace_bytes(size_t batch, size_t heads, size_t tokens, size_t head_dim) {
-  if (head_dim != 128 || tokens == 0 || tokens % 128 != 0) return 0;
-  return batch * heads * tokens * head_dim * 2;
-}
 
 namespace mase {
 namespace {
@@ -342,7 +316,7 @@ int attention_causal_impl(const void* q, const void* k, const void* v, void* out
                           size_t q_stride_t, size_t k_stride_b, size_t k_stride_h, size_t k_stride_t,
                           size_t v_stride_b, size_t v_stride_h, size_t v_stride_t, size_t o_stride_b,
                           size_t o_stride_h, size_t o_stride_t, int dtype, float scaling, int element_bits,
-                          const uint32_t* log2_tab, void* workspace, size_t workspace_bytes, void* stream) {
+                          const uint32_t* log2_tab, void* stream) {
   if (batch == 0 || heads == 0 || tokens == 0) return MASE_OK;
   if (q == nullptr || k == nullptr || v == nullptr || out == nullptr) return MASE_ERR_NULL;
   if (dtype != MASE_DT_BF16) return MASE_ERR_DTYPE;
@@ -358,8 +332,6 @@ int attention_causal_impl(const void* q, const void* k, const void* v, void* out
       v_stride_t * 2 > 0xFFFFFFFFull)
     return MASE_ERR_SHAPE;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return MASE_ERR_ALIGN;
-  const size_t need = mase_attention_causal_workspace_bytes(batch, heads, tokens, head_dim);
-  if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace)) return MASE_ERR_WORKSPACE;
   hipStream_t st = (hipStream_t)stream;
   const bool mx = element_bits != 0;
   static bool attr_set = false;
@@ -372,13 +344,11 @@ int attention_causal_impl(const void* q, const void* k, const void* v, void* out
     attr_set = true;
   }
   const int BH = (int)(batch * heads), T = (int)tokens;
-  hipLaunchKernelGGL(attn_transpose_v_kernel, dim3((unsigned)(T / 64), (unsigned)BH), dim3(256), 0, st,
-                     (const unsigned char*)v, (unsigned char*)workspace, (int)heads, T, v_stride_b * 2, v_stride_h * 2,
-                     (uint32_t)(v_stride_t * 2));
   AttnParams p;
   p.q = (const unsigned char*)q;
   p.k = (const unsigned char*)k;
-  p.vt = (const unsigned char*)workspace;
+  p.v = (const unsigned char*)v;
+  p.v_sb = v_stride_b * 2; p.v_sh = v_stride_h * 2; p.v_st = (uint32_t)(v_stride_t * 2);
   p.out = (unsigned char*)out;
   p.BH = BH;
   p.H = (int)heads;
@@ -409,11 +379,10 @@ extern "C" int mase_attention_causal(const void* q, const void* k, const void* v
                                      size_t tokens, size_t head_dim, size_t q_stride_b, size_t q_stride_h,
                                      size_t q_stride_t, size_t k_stride_b, size_t k_stride_h, size_t k_stride_t,
                                      size_t v_stride_b, size_t v_stride_h, size_t v_stride_t, size_t o_stride_b,
-                                     size_t o_stride_h, size_t o_stride_t, int dtype, float scaling, void* workspace,
-                                     size_t workspace_bytes, void* stream) {
+                                     size_t o_stride_h, size_t o_stride_t, int dtype, float scaling, void* stream) {
   return mase::attention_causal_impl(q, k, v, out, batch, heads, tokens, head_dim, q_stride_b, q_stride_h, q_stride_t,
                                      k_stride_b, k_stride_h, k_stride_t, v_stride_b, v_stride_h, v_stride_t, o_stride_b,
-                                     o_stride_h, o_stride_t, dtype, scaling, 0, nullptr, workspace, workspace_bytes, stream);
+                                     o_stride_h, o_stride_t, dtype, scaling, 0, nullptr, stream);
 }
 
 extern "C" int mase_attention_causal_mxint(const void* q, const void* k, const void* v, void* out, size_t batch,
@@ -421,11 +390,9 @@ extern "C" int mase_attention_causal_mxint(const void* q, const void* k, const v
                                            size_t q_stride_h, size_t q_stride_t, size_t k_stride_b, size_t k_stride_h,
                                            size_t k_stride_t, size_t v_stride_b, size_t v_stride_h, size_t v_stride_t,
                                            size_t o_stride_b, size_t o_stride_h, size_t o_stride_t, int dtype,
-                                           float scaling, int element_bits, const uint32_t* log2_tab, void* workspace,
-                                           size_t workspace_bytes, void* stream) {
+                                           float scaling, int element_bits, const uint32_t* log2_tab, void* stream) {
   if (element_bits == 0) return MASE_ERR_PARAM;
   return mase::attention_causal_impl(q, k, v, out, batch, heads, tokens, head_dim, q_stride_b, q_stride_h, q_stride_t,
                                      k_stride_b, k_stride_h, k_stride_t, v_stride_b, v_stride_h, v_stride_t, o_stride_b,
-                                     o_stride_h, o_stride_t, dtype, scaling, element_bits, log2_tab, workspace,
-                                     workspace_bytes, stream);
+                                     o_stride_h, o_stride_t, dtype, scaling, element_bits, log2_tab, stream);
 }

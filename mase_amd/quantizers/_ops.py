@@ -414,17 +414,14 @@ def attention_causal(q: Tensor, k: Tensor, v: Tensor, scaling: float | None = No
     if scaling is None:
         scaling = D ** -0.5
     out = torch.empty((B, T, H, D), dtype=q.dtype, device=q.device).transpose(1, 2)
-    need = lib.mase_attention_causal_workspace_bytes(B, H, T, D)
-    ws = torch.empty(need, dtype=torch.uint8, device=q.device)
     args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, H, T, D,
             q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
             v.stride(0), v.stride(1), v.stride(2), out.stride(0), out.stride(1), out.stride(2),
             _lib.dtype_code(q), float(scaling))
     if mxint_bits is None:
-        rc = lib.mase_attention_causal(*args, ws.data_ptr(), need, _lib.stream_ptr(q))
+        rc = lib.mase_attention_causal(*args, _lib.stream_ptr(q))
     else:
-        rc = lib.mase_attention_causal_mxint(*args, int(mxint_bits), log2_table(q.dtype, q.device).data_ptr(), ws.data_ptr(), need,
-                                             _lib.stream_ptr(q))
+        rc = lib.mase_attention_causal_mxint(*args, int(mxint_bits), log2_table(q.dtype, q.device).data_ptr(), _lib.stream_ptr(q))
     _lib.check(rc, "mase_attention_causal")
     return out
 
