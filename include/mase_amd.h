@@ -340,15 +340,20 @@ int mase_attention_causal(const void* q, const void* k, const void* v, void* out
                           size_t k_stride_b, size_t k_stride_h, size_t k_stride_t, size_t v_stride_b, size_t v_stride_h,
                           size_t v_stride_t, size_t o_stride_b, size_t o_stride_h, size_t o_stride_t, int dtype,
                           float scaling, void* stream);
-/* The same with the result written as its MXINT quantize-dequantize (blocks of 32 along the head dimension, element_bits
- * wide, E8M0 scales; log2_tab as for mase_mxint_qdq in bf16): what the LinearMXInt that reads the
- * [batch, tokens, heads * 128] result would compute from it in a pass of its own (nn/quantized/modules/linear.py:956-972),
- * bit for bit. */
-int mase_attention_causal_mxint(const void* q, const void* k, const void* v, void* out, size_t batch, size_t heads,
+/* The same with work of the neighbouring operations folded in, each part optional:
+ *   q_cos / q_sin (both or neither; bf16 tables [batch or 1, tokens, 128] with element strides cs_stride_b (0 for a
+ *   table shared by the batch) and cs_stride_t, multiples of 8): q is given BEFORE its rotary embedding, which is
+ *   applied as q is loaded with the roundings of mase_rope (nn/quantized/functional/rope.py:17-27);
+ *   element_bits != 0: the result is written as its MXINT quantize-dequantize (blocks of 32 along the head dimension,
+ *   E8M0 scales; log2_tab as for mase_mxint_qdq in bf16): what the LinearMXInt that reads the
+ *   [batch, tokens, heads * 128] result would compute from it in a pass of its own
+ *   (nn/quantized/modules/linear.py:956-972), bit for bit. */
+int mase_attention_causal_fused(const void* q, const void* k, const void* v, void* out, size_t batch, size_t heads,
                                 size_t tokens, size_t head_dim, size_t q_stride_b, size_t q_stride_h, size_t q_stride_t,
                                 size_t k_stride_b, size_t k_stride_h, size_t k_stride_t, size_t v_stride_b,
                                 size_t v_stride_h, size_t v_stride_t, size_t o_stride_b, size_t o_stride_h,
-                                size_t o_stride_t, int dtype, float scaling, int element_bits, const uint32_t* log2_tab,
+                                size_t o_stride_t, int dtype, float scaling, const void* q_cos, const void* q_sin,
+                                size_t cs_stride_b, size_t cs_stride_t, int element_bits, const uint32_t* log2_tab,
                                 void* stream);
 
 /* Rotary embedding out = x * cos + rotate_half(x) * sin for x [B, H, T, D] with the last dimension contiguous and

@@ -52,8 +52,8 @@ SIGNATURES = {
     "mase_constant_rate_counter_khz": (c_int, []),
     "mase_probe_mfma_f8f4": (c_int, [c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p]),
     "mase_probe_mfma_bf16": (c_int, [c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p]),
-    "mase_attention_causal_mxint": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p] + [c_size_t] * 16 + [c_int, c_float, c_int, c_void_p,
-                                            c_void_p]),
+    "mase_attention_causal_fused": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p] + [c_size_t] * 16 + [c_int, c_float, c_void_p, c_void_p,
+                                            c_size_t, c_size_t, c_int, c_void_p, c_void_p]),
     "mase_rmsnorm_mxint": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_float, c_int, c_void_p, c_void_p]),
     "mase_silu_mul_mxint": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_void_p, c_void_p]),
     "mase_mxint_clip_search": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),

@@ -73,13 +73,20 @@ struct AttnParams {
   uint32_t q_st, k_st, v_st, o_st;                        // byte strides of a token
   float c;                                    // scaling * log2(e)
   MxintParams mx;                             // MX instantiation only
+  const unsigned char* q_cos;                 // ROPE instantiation only: tables [batch or 1][tokens][128] bf16
+  const unsigned char* q_sin;
+  size_t cs_sb;                               // byte strides of the tables: batch (0 for a shared table), token
+  uint32_t cs_st;
 };
 
 // MX: the output is written as the MXINT quantize-dequantize of the bf16 result, blocks of 32 along the head dimension
 // (what a LinearMXInt reading the [batch, tokens, heads * 128] result would compute in a pass of its own,
 // nn/quantized/modules/linear.py:956-972): the 32 values of a block are the 16 accumulator registers of one d tile in
 // lane l and in lane l ^ 32.
-template <bool MX>
+// ROPE: q is given before its rotary embedding, which is applied as the fragments are loaded: x cos + rotate_half(x) sin
+// with the two products and the sum rounded to bf16 one by one, as mase_rope rounds them
+// (nn/quantized/functional/rope.py:17-27); the partner element d +- 64 lies in the same lane's fragment s +- 4.
+template <bool MX, bool ROPE>
 __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int lane = threadIdx.x & 63;
@@ -108,6 +115,25 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
   bf16x8_t qf[8];
 #pragma unroll
   for (int s = 0; s < 8; ++s) qf[s] = *(const bf16x8_t*)(qp + (size_t)qi * p.q_st + (s * 16 + g * 8) * 2);
+  if constexpr (ROPE) {
+    const unsigned char* cp = p.q_cos + (size_t)b * p.cs_sb + (size_t)qi * p.cs_st;
+    const unsigned char* sp = p.q_sin + (size_t)b * p.cs_sb + (size_t)qi * p.cs_st;
+    bf16x8_t rq[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const bf16x8_t cs = *(const bf16x8_t*)(cp + (s * 16 + g * 8) * 2), sn = *(const bf16x8_t*)(sp + (s * 16 + g * 8) * 2);
+      const bf16x8_t other = qf[s ^ 4];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        using TR = DTypeTraits<MASE_DT_BF16>;
+        const float x = (float)qf[s][e], xp = (float)other[e];
+        const float rot = (s < 4) ? -xp : xp;
+        rq[s][e] = __builtin_bit_cast(__bf16, (uint16_t)f32_to_bf16_bits(TR::round(x * (float)cs[e]) + TR::round(rot * (float)sn[e])));
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < 8; ++s) qf[s] = rq[s];
+  }
 
   // async copies of one key block: 4 of K and 4 of V (4 rows of 256 bytes each) per wavefront.
   // LDS position (row, 16-byte slot) holds the row's chunk slot ^ (row % 16), so that the
@@ -315,7 +341,8 @@ int attention_causal_impl(const void* q, const void* k, const void* v, void* out
                           size_t tokens, size_t head_dim, size_t q_stride_b, size_t q_stride_h,
                           size_t q_stride_t, size_t k_stride_b, size_t k_stride_h, size_t k_stride_t,
                           size_t v_stride_b, size_t v_stride_h, size_t v_stride_t, size_t o_stride_b,
-                          size_t o_stride_h, size_t o_stride_t, int dtype, float scaling, int element_bits,
+                          size_t o_stride_h, size_t o_stride_t, int dtype, float scaling, const void* q_cos,
+                          const void* q_sin, size_t cs_stride_b, size_t cs_stride_t, int element_bits,
                           const uint32_t* log2_tab, void* stream) {
   if (batch == 0 || heads == 0 || tokens == 0) return MASE_OK;
   if (q == nullptr || k == nullptr || v == nullptr || out == nullptr) return MASE_ERR_NULL;
@@ -333,14 +360,18 @@ int attention_causal_impl(const void* q, const void* k, const void* v, void* out
     return MASE_ERR_SHAPE;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return MASE_ERR_ALIGN;
   hipStream_t st = (hipStream_t)stream;
-  const bool mx = element_bits != 0;
+  const bool mx = element_bits != 0, rope = q_cos != nullptr || q_sin != nullptr;
+  if (rope) {
+    if (q_cos == nullptr || q_sin == nullptr) return MASE_ERR_NULL;
+    if (!aligned16(q_cos) || !aligned16(q_sin) || cs_stride_b % 8 != 0 || cs_stride_t % 8 != 0) return MASE_ERR_ALIGN;
+    if (cs_stride_t < 128 || cs_stride_t * 2 > 0xFFFFFFFFull) return MASE_ERR_SHAPE;
+  }
+  const void* kernels[4] = {(const void*)attn_causal_fwd_kernel<false, false>, (const void*)attn_causal_fwd_kernel<true, false>,
+                            (const void*)attn_causal_fwd_kernel<false, true>, (const void*)attn_causal_fwd_kernel<true, true>};
   static bool attr_set = false;
   if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)attn_causal_fwd_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLds) !=
-            hipSuccess ||
-        hipFuncSetAttribute((const void*)attn_causal_fwd_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLds) !=
-            hipSuccess)
-      return MASE_ERR_LAUNCH;
+    for (const void* kfn : kernels)
+      if (hipFuncSetAttribute(kfn, hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLds) != hipSuccess) return MASE_ERR_LAUNCH;
     attr_set = true;
   }
   const int BH = (int)(batch * heads), T = (int)tokens;
@@ -365,11 +396,18 @@ int attention_causal_impl(const void* q, const void* k, const void* v, void* out
     p.mx.lo = mase_round_scalar_to_dtype(-(double)(1 << (element_bits - 1)), dtype);
     p.mx.hi = mase_round_scalar_to_dtype((double)((1 << (element_bits - 1)) - 1), dtype);
     p.mx.tab = log2_tab;
-    hipLaunchKernelGGL(attn_causal_fwd_kernel<true>, dim3((unsigned)(BH * (T / kQB))), dim3(256), kAttnLds, st, p);
   } else {
     p.mx = MxintParams{};
-    hipLaunchKernelGGL(attn_causal_fwd_kernel<false>, dim3((unsigned)(BH * (T / kQB))), dim3(256), kAttnLds, st, p);
   }
+  p.q_cos = (const unsigned char*)q_cos;
+  p.q_sin = (const unsigned char*)q_sin;
+  p.cs_sb = cs_stride_b * 2;
+  p.cs_st = (uint32_t)(cs_stride_t * 2);
+  const dim3 grid((unsigned)(BH * (T / kQB))), block(256);
+  if (mx && rope) hipLaunchKernelGGL((attn_causal_fwd_kernel<true, true>), grid, block, kAttnLds, st, p);
+  else if (mx) hipLaunchKernelGGL((attn_causal_fwd_kernel<true, false>), grid, block, kAttnLds, st, p);
+  else if (rope) hipLaunchKernelGGL((attn_causal_fwd_kernel<false, true>), grid, block, kAttnLds, st, p);
+  else hipLaunchKernelGGL((attn_causal_fwd_kernel<false, false>), grid, block, kAttnLds, st, p);
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
 }  // namespace
@@ -382,17 +420,18 @@ extern "C" int mase_attention_causal(const void* q, const void* k, const void* v
                                      size_t o_stride_h, size_t o_stride_t, int dtype, float scaling, void* stream) {
   return mase::attention_causal_impl(q, k, v, out, batch, heads, tokens, head_dim, q_stride_b, q_stride_h, q_stride_t,
                                      k_stride_b, k_stride_h, k_stride_t, v_stride_b, v_stride_h, v_stride_t, o_stride_b,
-                                     o_stride_h, o_stride_t, dtype, scaling, 0, nullptr, stream);
+                                     o_stride_h, o_stride_t, dtype, scaling, nullptr, nullptr, 0, 0, 0, nullptr, stream);
 }
 
-extern "C" int mase_attention_causal_mxint(const void* q, const void* k, const void* v, void* out, size_t batch,
+extern "C" int mase_attention_causal_fused(const void* q, const void* k, const void* v, void* out, size_t batch,
                                            size_t heads, size_t tokens, size_t head_dim, size_t q_stride_b,
                                            size_t q_stride_h, size_t q_stride_t, size_t k_stride_b, size_t k_stride_h,
                                            size_t k_stride_t, size_t v_stride_b, size_t v_stride_h, size_t v_stride_t,
                                            size_t o_stride_b, size_t o_stride_h, size_t o_stride_t, int dtype,
-                                           float scaling, int element_bits, const uint32_t* log2_tab, void* stream) {
-  if (element_bits == 0) return MASE_ERR_PARAM;
+                                           float scaling, const void* q_cos, const void* q_sin, size_t cs_stride_b,
+                                           size_t cs_stride_t, int element_bits, const uint32_t* log2_tab, void* stream) {
   return mase::attention_causal_impl(q, k, v, out, batch, heads, tokens, head_dim, q_stride_b, q_stride_h, q_stride_t,
                                      k_stride_b, k_stride_h, k_stride_t, v_stride_b, v_stride_h, v_stride_t, o_stride_b,
-                                     o_stride_h, o_stride_t, dtype, scaling, element_bits, log2_tab, stream);
+                                     o_stride_h, o_stride_t, dtype, scaling, q_cos, q_sin, cs_stride_b, cs_stride_t,
+                                     element_bits, log2_tab, stream);
 }

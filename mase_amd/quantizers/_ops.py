@@ -401,12 +401,15 @@ def attention_causal_supported(q: Tensor, k: Tensor, v: Tensor) -> bool:
     return True
 
 
-def attention_causal(q: Tensor, k: Tensor, v: Tensor, scaling: float | None = None, mxint_bits: int | None = None) -> Tensor:
+def attention_causal(q: Tensor, k: Tensor, v: Tensor, scaling: float | None = None, mxint_bits: int | None = None,
+                     q_rope: tuple[Tensor, Tensor] | None = None) -> Tensor:
     """``softmax(q k^T * scaling + causal mask) v`` for bf16 [batch, heads, tokens, 128] operands in one pass over the keys
     (``mase_attention_causal``).  Returned as [batch, heads, tokens, 128] over memory laid out [batch, tokens, heads,
     128], so that ``out.transpose(1, 2).reshape(batch, tokens, heads * 128)`` is a view.  ``mxint_bits``: the result is
     written as ``mxint_quantizer(result, block 32 along the head dimension, mxint_bits)``, the form a ``LinearMXInt``
-    that reads it would compute itself (``mase_attention_causal_mxint``)."""
+    that reads it would compute itself.  ``q_rope = (cos, sin)``: ``q`` is given before its rotary embedding, which the
+    kernel applies as it loads ``q`` (the values of ``rope(q, cos, sin)``; the tables must satisfy ``rope_supported``).
+    Both through ``mase_attention_causal_fused``."""
     _lib.require_device(q, "attention_causal")
     lib = _lib.load()
     assert attention_causal_supported(q, k, v)
@@ -418,10 +421,20 @@ def attention_causal(q: Tensor, k: Tensor, v: Tensor, scaling: float | None = No
             q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
             v.stride(0), v.stride(1), v.stride(2), out.stride(0), out.stride(1), out.stride(2),
             _lib.dtype_code(q), float(scaling))
-    if mxint_bits is None:
+    if mxint_bits is None and q_rope is None:
         rc = lib.mase_attention_causal(*args, _lib.stream_ptr(q))
     else:
-        rc = lib.mase_attention_causal_mxint(*args, int(mxint_bits), log2_table(q.dtype, q.device).data_ptr(), _lib.stream_ptr(q))
+        cos = sin = None
+        cs_b = cs_t = 0
+        if q_rope is not None:
+            cos, sin = q_rope
+            assert rope_supported(q, cos, sin)
+            cs_b = cos.stride(0) if cos.dim() == 3 and cos.shape[0] == B and B > 1 else 0
+            cs_t = cos.stride(-2)
+        tab = log2_table(q.dtype, q.device).data_ptr() if mxint_bits is not None else None
+        rc = lib.mase_attention_causal_fused(*args, cos.data_ptr() if cos is not None else None,
+                                             sin.data_ptr() if sin is not None else None, cs_b, cs_t,
+                                             int(mxint_bits or 0), tab, _lib.stream_ptr(q))
     _lib.check(rc, "mase_attention_causal")
     return out
 

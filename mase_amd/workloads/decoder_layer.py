@@ -65,13 +65,14 @@ def rope_tables(seq_len: int, head_dim: int, theta: float, device, dtype):
     return emb.cos().to(dtype), emb.sin().to(dtype)
 
 
-def causal_attention(q, k, v, mxint_bits=None):
+def causal_attention(q, k, v, mxint_bits=None, q_rope=None):
     """softmax(q k^T / sqrt(d) + causal mask) v: the one-pass kernel of this package where it applies (bf16, head
     dimension 128, a multiple of 128 tokens, no gradient), the library's scaled_dot_product_attention otherwise.
-    ``mxint_bits`` (only where the kernel applies): the result in the MXINT form of the Linear that reads it."""
+    Only where the kernel applies: ``mxint_bits``, the result in the MXINT form of the Linear that reads it;
+    ``q_rope = (cos, sin)``, q handed over before its rotary embedding, which the kernel applies on load."""
     if q.is_cuda and _ops.attention_causal_supported(q, k, v):
-        return _ops.attention_causal(q, k, v, mxint_bits=mxint_bits)
-    assert mxint_bits is None
+        return _ops.attention_causal(q, k, v, mxint_bits=mxint_bits, q_rope=q_rope)
+    assert mxint_bits is None and q_rope is None
     return F.scaled_dot_product_attention(q, k, v, is_causal=True)
 
 
@@ -142,22 +143,25 @@ class DecoderLayer(nn.Module):
         q, k, v = (t.view(B, T, cfg.num_heads, cfg.head_dim).transpose(1, 2)
                    for t in self._norm_then_project(self.input_layernorm, x, (self.q_proj, self.k_proj, self.v_proj)))
         cos, sin = self._rope_tables(T, x.device, x.dtype)
-        if q.is_cuda and _ops.rope_supported(q, cos, sin) and _ops.rope_supported(k, cos, sin):
-            q, k = _ops.rope(q, cos, sin), _ops.rope(k, cos, sin)  # the same products and sum in one pass
+        own_kernel = (self.fuse_producers and self.attention_fn is causal_attention and q.is_cuda
+                      and not torch.is_grad_enabled() and _ops.attention_causal_supported(q, k, v))
+        rope_ok = q.is_cuda and _ops.rope_supported(q, cos, sin) and _ops.rope_supported(k, cos, sin)
+        q_rope = (cos, sin) if own_kernel and rope_ok else None  # the attention kernel rotates q as it loads it
+        if rope_ok:
+            k = _ops.rope(k, cos, sin)  # the same products and sum in one pass
+            if q_rope is None:
+                q = _ops.rope(q, cos, sin)
         else:
             q = q * cos + rotate_half(q) * sin
             k = k * cos + rotate_half(k) * sin
-        bits = None
-        if (self.fuse_producers and self.attention_fn is causal_attention and q.is_cuda and not torch.is_grad_enabled()
-                and _ops.attention_causal_supported(q, k, v)):
-            bits = shared_mxint_width(x, (self.o_proj,))  # o_proj's input: same dtype and device as x, head_dim % 32 == 0
-        if bits is not None:
-            a = causal_attention(q, k, v, mxint_bits=bits).transpose(1, 2).reshape(B, T, cfg.num_heads * cfg.head_dim)
-            x = self._project_add(self.o_proj, a, x, prepared=a.reshape(-1, a.shape[-1]))
+        # o_proj's input has x's dtype and device and a last dimension that is a multiple of 32
+        bits = shared_mxint_width(x, (self.o_proj,)) if own_kernel else None
+        if own_kernel:
+            a = causal_attention(q, k, v, mxint_bits=bits, q_rope=q_rope)
         else:
             a = self.attention_fn(q, k, v)
-            a = a.transpose(1, 2).reshape(B, T, cfg.num_heads * cfg.head_dim)
-            x = self._project_add(self.o_proj, a, x)
+        a = a.transpose(1, 2).reshape(B, T, cfg.num_heads * cfg.head_dim)
+        x = self._project_add(self.o_proj, a, x, prepared=a.reshape(-1, a.shape[-1]) if bits is not None else None)
         gate, up = self._norm_then_project(self.post_attention_layernorm, x, (self.gate_proj, self.up_proj))
         if gate.is_cuda and _ops.silu_mul_supported(gate, up):
             bits = shared_mxint_width(gate, (self.down_proj,)) if self.fuse_producers and gate.shape[-1] % 32 == 0 else None

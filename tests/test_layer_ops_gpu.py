@@ -187,6 +187,17 @@ def test_causal_attention_one_pass(dev, B, H, T, layout):
             gq = _ops.attention_causal(q, k, v, scaling, mxint_bits=bits).transpose(1, 2).reshape(B, T, H * 128)
             want = O.mxint_quantizer(got.transpose(1, 2).reshape(B, T, H * 128).cpu(), 32, bits, block_dim=-1)
             assert_bits_equal(gq, want, f"attention output as MXINT{bits}")
+    # q handed over before its rotary embedding: the kernel's rotation on load gives the values of rope() followed by
+    # the plain call, with and without the MXINT output form; tables shared by the batch and per batch item
+    ang = torch.rand(T, 64, generator=g) * 6.28
+    emb = torch.cat((ang, ang), -1)
+    cos, sin = emb.cos().bfloat16().to(dev), emb.sin().bfloat16().to(dev)
+    for tables in ((cos, sin), (cos[None].expand(B, T, 128).contiguous(), sin[None].expand(B, T, 128).contiguous() * 0.5)):
+        assert _ops.rope_supported(q, *tables)
+        want = _ops.attention_causal(_ops.rope(q, *tables), k, v)
+        assert torch.equal(_ops.attention_causal(q, k, v, q_rope=tables), want)
+        assert torch.equal(_ops.attention_causal(q, k, v, mxint_bits=8, q_rope=tables),
+                           _ops.attention_causal(_ops.rope(q, *tables), k, v, mxint_bits=8))
     assert not _ops.attention_causal_supported(q[:, :, :100], k[:, :, :100], v[:, :, :100])
     assert not _ops.attention_causal_supported(q.float(), k.float(), v.float())
     assert not _ops.attention_causal_supported(q[..., :64], k[..., :64], v[..., :64])
