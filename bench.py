@@ -673,6 +673,54 @@ class AttnProb(Workload):
                 "kind": "port", "sample": f"{n} passes of the separate tensor operations over 2 heads [1,2,2048,2048], {dt*1e3:.0f} ms each"}
 
 
+class AttentionCausal(Workload):
+    """the decoder layer's attention core on its own: causal softmax(q k^T / sqrt(d)) v, bf16, batch 8 x 32 heads x 2048
+    tokens x 128, operands as strided views of [batch, tokens, heads, 128] memory (what the projections produce)"""
+    name = "attention_causal"
+    default_steps, default_warmup = 200, 20
+    unit = "TFLOP/s"
+    dtype = "bf16"
+    bound = "mfma"
+    kernel = "attn_causal_fwd_kernel"
+    shape = (8, 32, 2048, 128)
+
+    def setup(self, torch, dev, n_buffers):
+        from mase_amd.quantizers import _ops
+
+        self._ops = _ops
+        B, H, T, D = self.shape
+        g = torch.Generator(device=dev).manual_seed(7)
+        mk = lambda: torch.randn(B, T, H, D, device=dev, generator=g).bfloat16().transpose(1, 2)
+        self.sets = [(mk(), mk(), mk()) for _ in range(2)]
+        self.metric = "causal attention core throughput (4 * batch * heads * tokens^2 * 128 / 2 flop per step: the unmasked half)"
+        self.config = {"workload": f"q, k, v bf16 {list(self.shape)} N(0,1) seed 7, scaling 128^-0.5, causal"}
+
+    def step(self, i):
+        q, k, v = self.sets[i % 2]
+        self.out = self._ops.attention_causal(q, k, v)
+
+    def work_per_step(self):
+        B, H, T, D = self.shape
+        return 4.0 * B * H * T * T * D / 2
+
+    def cpu_baseline(self, torch, budget_s):
+        B, H, T, D = self.shape
+        q, k, v = (t[:1, :2].float().cpu() for t in self.sets[0])  # 2 heads of one batch item
+        mask = torch.triu(torch.ones(T, T, dtype=torch.bool), 1)
+        t0 = time.perf_counter()
+        n = 0
+        while True:
+            s = (q @ k.transpose(-1, -2)) * D ** -0.5
+            torch.softmax(s.masked_fill(mask, float("-inf")), -1) @ v
+            n += 1
+            if time.perf_counter() - t0 > budget_s or n >= 20:
+                break
+        dt = (time.perf_counter() - t0) / n
+        return {"value": 4.0 * 2 * T * T * D / 2 / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+                "sample": f"{n} passes of the tensor operations (fp32, full score matrix) over 2 heads, {dt*1e3:.0f} ms each; "
+                          "flop counted as for the GPU (the unmasked half)"}
+
+
 class DecodeLinear(Workload):
     """LinearMXInt forward for a handful of tokens: bound by streaming the weight once"""
     name = "decode_linear"
@@ -785,7 +833,7 @@ class DecodeLinearMxfp4(Workload):
 
 WORKLOADS = {w.name: w for w in (MxintClipSearch, BfpQdq, MxintQdq, MxintLinear, MxintLinearCodes, MxfpLinear, DecoderLayerMxint, CopyBytes, IntegerQdq,
                                  MinifloatDenormQdq, MinifloatIeeeQdq, MinifloatMxQdq, MxfpQdq, AttnProb, DecodeLinear,
-                                 DecodeLinearPacked, DecodeLinearMxfp4, MfmaRateZeros, MfmaRateRandom, MfmaF8F4RateZeros,
+                                 DecodeLinearPacked, DecodeLinearMxfp4, AttentionCausal, MfmaRateZeros, MfmaRateRandom, MfmaF8F4RateZeros,
                                  MfmaF8F4RateRandom)}
 
 
