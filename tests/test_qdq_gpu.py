@@ -87,6 +87,30 @@ def test_mxint_fp32_power_of_two_neighbourhood(Q, dev):
     assert_bits_equal(got, want, "mxint fp32 pow2 neighbourhood")
 
 
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16], ids=_ID.get)
+@pytest.mark.parametrize("block,bits", [(32, 8), (8, 8), (16, 4), (64, 8), (128, 12), (512, 8), (1024, 8), (4, 8)])
+def test_mxint_fp32_in_16bit_out(dev, out_dtype, block, bits):
+    """The activation quantizer of an MX Linear on fp32 inputs writes its result in a 16-bit dtype directly
+    (``mxint_qdq(..., out_dtype=)``): the oracle's fp32 result converted to that dtype, bit for bit, for blocks that take
+    the wide kernel (8 elements per lane) and blocks that do not, a ragged tail, the log2 corrections next to powers of
+    two, non-finite blocks and values that overflow fp16"""
+    from mase_amd.quantizers import _ops
+
+    rng = np.random.default_rng(77 + block + bits)
+    x = adversarial(rng, (96, 3072), torch.float32, block=block if 3072 % block == 0 else 32).reshape(-1)
+    k = torch.arange(-100, 100, dtype=torch.int32)
+    edge = torch.cat([torch.ldexp(torch.tensor(1.0 + m * 2.0 ** -23, dtype=torch.float64), k) for m in (0, 1, 2, 5, 9)]).float()
+    x[: edge.numel()] = edge
+    x[5000] = float("inf")
+    x[9000] = float("nan")
+    x[12000] = 7.0e4   # finite in fp32 and bf16, infinite in fp16
+    n = (x.numel() // block) * block - block * 3  # not a multiple of the work-group's 512 elements
+    x = x[:n].contiguous()
+    want = O.mxint_quantizer(x, block, bits).to(out_dtype)
+    got = _ops.mxint_qdq(x.to(dev), block, bits, -1, 8, out_dtype=out_dtype)
+    assert_bits_equal(got, want, f"mxint fp32 -> {out_dtype} B={block} b={bits}")
+
+
 def test_mxint_nonfinite_blocks(Q, dev):
     x = torch.randn(8, 32)
     x[1, 3] = float("inf")
