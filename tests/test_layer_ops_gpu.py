@@ -20,7 +20,7 @@ def close_in_ulps(got, want, dtype, n_ulp, frac_equal):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("cols", [8, 256, 4096, 5120, 8192])
+@pytest.mark.parametrize("cols", [8, 256, 1536, 1600, 2048, 4096, 5120, 8192])
 def test_rmsnorm_one_pass(dev, dtype, cols):
     from mase_amd.quantizers import _ops
 
@@ -129,7 +129,7 @@ def test_norm_and_silu_product_written_in_the_consumers_mxint_form(dev, dtype, b
     from helpers import assert_bits_equal
 
     g = torch.Generator().manual_seed(5 + bits)
-    for rows, cols in ((37, 4096), (5, 32), (3, 5120), (130, 96), (2, 8192)):
+    for rows, cols in ((37, 4096), (5, 32), (3, 5120), (130, 96), (2, 8192), (9, 1536), (7, 1600), (4, 2048)):
         x = (torch.randn(rows, cols, generator=g) * 1.7).to(dtype)
         x[0, :32] = 0
         x[1 % rows, 32:64] *= 1e-3
