@@ -69,6 +69,7 @@ struct AttnParams {
   const unsigned char* v;
   unsigned char* out;
   int BH, H, T;
+  int rounds, bh_lanes;  // persistent form: work items per work-group, (batch, head) pairs an XCD works on side by side
   size_t q_sb, q_sh, k_sb, k_sh, v_sb, v_sh, o_sb, o_sh;  // byte strides of batch and head
   uint32_t q_st, k_st, v_st, o_st;                        // byte strides of a token
   float c;                                    // scaling * log2(e)
@@ -93,11 +94,23 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
   const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
   const int l32 = lane & 31, g = lane >> 5;
   // Work-groups are handed to the 8 XCDs in turn (blockIdx % 8), each XCD with an L2 of its own.  All query blocks of
-  // one (batch, head) go to one XCD, one after the other and the ones with the most keys first: they run at the same
-  // time and walk the keys from the start together, so K and V come from HBM once and from that L2 afterwards.
+  // one (batch, head) go to one XCD and run at the same time, walking the keys from the start together, so K and V come
+  // from HBM once and from that L2 afterwards.
+  // Persistent form (rounds > 0; the host picks it when the counts divide): two work-groups per CU for the whole
+  // launch, each taking `rounds` items; an XCD's work-groups cover bh_lanes (batch, head) pairs x all query blocks per
+  // round, and a work-group alternates between query block n - 1 - i and query block i, so that all of them have the
+  // same number of key blocks to go through and finish together.  Otherwise one item per work-group, the query blocks
+  // with the most keys first.
   const int n_qb = p.T / kQB;
+  const int n_items = p.rounds > 0 ? p.rounds : 1;
+  for (int item = 0; item < n_items; ++item) {
   int bh, qb;
-  if (p.BH % 8 == 0) {
+  if (p.rounds > 0) {
+    const int xcd = (int)blockIdx.x & 7, wl = (int)blockIdx.x >> 3;
+    const int qidx = wl % n_qb;
+    bh = (wl / n_qb + p.bh_lanes * item) * 8 + xcd;
+    qb = (item & 1) ? qidx : n_qb - 1 - qidx;
+  } else if (p.BH % 8 == 0) {
     const int xcd = (int)blockIdx.x & 7, slot = (int)blockIdx.x >> 3;
     bh = (slot / n_qb) * 8 + xcd;
     qb = n_qb - 1 - slot % n_qb;
@@ -109,6 +122,14 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
   const unsigned char* qp = p.q + (size_t)b * p.q_sb + (size_t)h * p.q_sh;
   const unsigned char* kp = p.k + (size_t)b * p.k_sb + (size_t)h * p.k_sh;
   const unsigned char* vp = p.v + (size_t)b * p.v_sb + (size_t)h * p.v_sh;
+  // persistent form: the first key block of the work-group's next item is fetched during the last key block of this one
+  const bool has_next = item + 1 < n_items;
+  const unsigned char *kp_next = kp, *vp_next = vp;
+  if (has_next) {
+    const int bhn = bh + p.bh_lanes * 8, bn = bhn / p.H, hn = bhn % p.H;
+    kp_next = p.k + (size_t)bn * p.k_sb + (size_t)hn * p.k_sh;
+    vp_next = p.v + (size_t)bn * p.v_sb + (size_t)hn * p.v_sh;
+  }
   const int q0 = qb * kQB + wave * 32;  // this wavefront's first query
   const int qi = q0 + l32;              // this lane's query
 
@@ -146,13 +167,17 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
     voff[i] = (uint32_t)krow * p.v_st + (uint32_t)(((lane & 15) ^ (krow & 15)) << 4);
   }
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;
-  // copy c (0..7) of key block j: 0-3 K, 4-7 V
+  const int nblk = 2 * qb + 2;  // key blocks that hold a key <= the block's last query (even: the last one uses stage 1)
+  // copy c (0..7) of key block j: 0-3 K, 4-7 V; j == nblk stands for key block 0 of the next item (stage 0 again)
   auto issue_one = [&](int j, int c) __attribute__((always_inline)) {
     const int i = c & 3;
+    const bool nxt = j == nblk;
+    const size_t blk = nxt ? 0 : (size_t)j;
     if (c < 4) {
-      at_async_copy_16(kp + (size_t)j * kKB * p.k_st, koff[i], lds_base + (uint32_t)((j & 1) * kKBytes + (wave * 4 + i) * 1024));
+      at_async_copy_16((nxt ? kp_next : kp) + blk * kKB * p.k_st, koff[i],
+                       lds_base + (uint32_t)((j & 1) * kKBytes + (wave * 4 + i) * 1024));
     } else {
-      at_async_copy_16(vp + (size_t)j * kKB * p.v_st, voff[i],
+      at_async_copy_16((nxt ? vp_next : vp) + blk * kKB * p.v_st, voff[i],
                        lds_base + (uint32_t)(2 * kKBytes + (j & 1) * kVBytes + (wave * 4 + i) * 1024));
     }
   };
@@ -168,12 +193,11 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
     for (int r = 0; r < 16; ++r) o[dt][r] = 0.0f;
   float m = -__builtin_inff(), lsum = 0.0f;
 
-  const int nblk = 2 * qb + 2;  // key blocks that hold a key <= the block's last query
-  issue(0);
+  if (item == 0) issue(0);  // later items: fetched by the item before
   for (int j = 0; j < nblk; ++j) {
     at_wait_vmcnt<0>();  // this wavefront's copies of block j have landed
     asm volatile("s_barrier" ::: "memory");  // ... everyone's have, and everyone has finished with block j - 1's buffers
-    const bool more = j + 1 < nblk;
+    const bool more = j + 1 < nblk || has_next;
     const int key0 = j * kKB;
     const bool skip = key0 > q0 + 31;  // every key of the block lies after every query of this wavefront
     if (skip && more) issue(j + 1);
@@ -292,7 +316,7 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
       __builtin_amdgcn_sched_barrier(0);
     }
   }
-  at_wait_vmcnt<0>();
+  if (!has_next) at_wait_vmcnt<0>();  // no copy may be in flight towards LDS when the work-group retires
   lsum += __shfl_xor(lsum, 32, 64);
   const float inv = 1.0f / lsum;
   // register r of tile dt is d = 32 dt + 8 (r / 4) + 4 g + r % 4: four consecutive d per group of four registers
@@ -330,6 +354,7 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
       *(uint2*)(op + (32 * dt + 8 * qq + 4 * g) * 2) = w;
     }
   }
+  }  // items
 }
 
 }  // namespace
@@ -399,11 +424,33 @@ int attention_causal_impl(const void* q, const void* k, const void* v, void* out
   } else {
     p.mx = MxintParams{};
   }
+  // persistent form when the work divides evenly over two work-groups per CU (see the kernel)
+  p.rounds = 0;
+  p.bh_lanes = 0;
+  unsigned n_wg = (unsigned)(BH * (T / kQB));
+  {
+    static int n_cu = 0;
+    if (n_cu == 0) {
+      int dev = 0;
+      hipDeviceProp_t prop;
+      if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return MASE_ERR_LAUNCH;
+      n_cu = prop.multiProcessorCount;
+    }
+    const int n_qb = T / kQB, wg_per_xcd = 2 * n_cu / 8;
+    if (BH % 8 == 0 && n_cu % 8 == 0 && n_qb <= wg_per_xcd && wg_per_xcd % n_qb == 0) {
+      const int lanes = wg_per_xcd / n_qb, per_xcd = BH / 8;
+      if (per_xcd % lanes == 0 && per_xcd / lanes >= 2) {
+        p.rounds = per_xcd / lanes;
+        p.bh_lanes = lanes;
+        n_wg = (unsigned)(8 * wg_per_xcd);
+      }
+    }
+  }
   p.q_cos = (const unsigned char*)q_cos;
   p.q_sin = (const unsigned char*)q_sin;
   p.cs_sb = cs_stride_b * 2;
   p.cs_st = (uint32_t)(cs_stride_t * 2);
-  const dim3 grid((unsigned)(BH * (T / kQB))), block(256);
+  const dim3 grid(n_wg), block(256);
   if (mx && rope) hipLaunchKernelGGL((attn_causal_fwd_kernel<true, true>), grid, block, kAttnLds, st, p);
   else if (mx) hipLaunchKernelGGL((attn_causal_fwd_kernel<true, false>), grid, block, kAttnLds, st, p);
   else if (rope) hipLaunchKernelGGL((attn_causal_fwd_kernel<false, true>), grid, block, kAttnLds, st, p);

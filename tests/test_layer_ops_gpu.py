@@ -147,7 +147,9 @@ def test_norm_and_silu_product_written_in_the_consumers_mxint_form(dev, dtype, b
         assert_bits_equal(_ops.silu_mul_mxint(gd, ud, bits), want, f"silu_mul_mxint {dtype} {rows}x{cols}")
 
 
-@pytest.mark.parametrize("B,H,T", [(1, 1, 128), (2, 3, 256), (1, 2, 640), (1, 4, 2048), (2, 4, 384), (1, 16, 256)])
+# the last two: enough (batch, head) pairs per XCD for the persistent form of the kernel (2 and 4 items per work-group)
+@pytest.mark.parametrize("B,H,T", [(1, 1, 128), (2, 3, 256), (1, 2, 640), (1, 4, 2048), (2, 4, 384), (1, 16, 256), (8, 64, 256),
+                                   (2, 64, 1024)])
 @pytest.mark.parametrize("layout", ["bthd", "bhtd"])
 def test_causal_attention_one_pass(dev, B, H, T, layout):
     """mase_attention_causal against the tensor operations in fp32 (masked scores, softmax, product with v) on the same
