@@ -198,13 +198,6 @@ size_t mase_gemm_bf16_packed_bytes(size_t N, size_t K);
 int mase_gemm_bf16_pack_b(const void* B, void* B_packed, size_t N, size_t K, void* stream);
 int mase_gemm_bf16_tn_packed(const void* A, const void* B_packed, const void* bias, void* C, size_t M, size_t N,
                              size_t K, int out_dtype, int bias_dtype, void* stream);
-/* C = round(round(A B^T + bias) + residual): the Linear above followed by the residual addition of a pre-norm block
- * (hidden = residual + linear(x), models/llama/modeling_llama.py:901, :908), both roundings to out_dtype kept, so the
- * result is bit for bit that of the two operations.  residual: [M, N] contiguous in out_dtype (bf16 or f16 only),
- * 8-byte aligned; N % 4 == 0; C 16-byte aligned. */
-int mase_gemm_bf16_tn_packed_residual(const void* A, const void* B_packed, const void* bias, const void* residual,
-                                      void* C, size_t M, size_t N, size_t K, int out_dtype, int bias_dtype,
-                                      void* stream);
 
 /* The tiled product with B held as an MXINT8 weight in fragment order: the code image and the scale image written by
  * mase_gemm_mxint8_pack_b from int8 codes [N, K] and scale bytes [N, K/32] (value = code * 2^(scale - 134): the packed

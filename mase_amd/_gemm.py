@@ -40,21 +40,9 @@ def gemm_bf16_pack_b(b: Tensor) -> Tensor:
     return out
 
 
-def gemm_bf16_tn(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dtype, b_packed: Tensor | None = None,
-                 residual: Tensor | None = None) -> Tensor:
+def gemm_bf16_tn(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dtype, b_packed: Tensor | None = None) -> Tensor:
     """``a[M,K] @ b[N,K].T + bias`` with bf16 operands and fp32 accumulation; result in ``out_dtype``.
-    ``b_packed``: the image of ``gemm_bf16_pack_b(b)``, used by the tiled kernel when the shape takes that kernel.
-    ``residual`` ([M,N], ``out_dtype``): the result is ``residual + (product rounded to out_dtype)``, added in the
-    kernel's epilogue on the tiled fragment-ordered path with a 16-bit output, by a tensor addition otherwise (the same
-    values either way)."""
-    if residual is not None:
-        residual = residual.reshape(-1, residual.shape[-1])
-        fused = (b_packed is not None and out_dtype in (torch.bfloat16, torch.float16) and residual.dtype == out_dtype
-                 and residual.shape == (a.shape[0], b.shape[0]) and b.shape[0] % 4 == 0
-                 and gemm_bf16_takes_packed_b(a.shape[0], b.shape[0], a.shape[1]))
-        if not fused:
-            return gemm_bf16_tn(a, b, bias, out_dtype, b_packed=b_packed) + residual
-        residual = residual.contiguous()
+    ``b_packed``: the image of ``gemm_bf16_pack_b(b)``, used by the tiled kernel when the shape takes that kernel."""
     _lib.require_device(a, "gemm_bf16_tn")
     lib = _lib.load()
     assert a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16
@@ -100,10 +88,7 @@ def gemm_bf16_tn(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dty
         r1 = min(M, r0 + rows_per_call)
         args = (bias.data_ptr() if bias is not None else None, out[r0:r1].data_ptr(), r1 - r0, N, K,
                 _lib.DTYPE_CODE[out_dtype], _lib.DTYPE_CODE[bias.dtype] if bias is not None else 0, _lib.stream_ptr(a))
-        if packed and residual is not None:
-            _lib.check(lib.mase_gemm_bf16_tn_packed_residual(a[r0:r1].data_ptr(), b_packed.data_ptr(), args[0], residual[r0:r1].data_ptr(),
-                                                             *args[1:]), "mase_gemm_bf16_tn_packed_residual")
-        elif packed:
+        if packed:
             _lib.check(lib.mase_gemm_bf16_tn_packed(a[r0:r1].data_ptr(), b_packed.data_ptr(), *args), "mase_gemm_bf16_tn_packed")
         else:
             _lib.check(lib.mase_gemm_bf16_tn(a[r0:r1].data_ptr(), b.data_ptr(), *args), "mase_gemm_bf16_tn")

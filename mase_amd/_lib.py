@@ -63,8 +63,6 @@ SIGNATURES = {
     "mase_gemm_bf16_packed_bytes": (c_size_t, [c_size_t, c_size_t]),
     "mase_gemm_bf16_pack_b": (c_int, [c_void_p, c_void_p, c_size_t, c_size_t, c_void_p]),
     "mase_gemm_bf16_tn_packed": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_int, c_int, c_void_p]),
-    "mase_gemm_bf16_tn_packed_residual": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_int,
-                                                  c_int, c_void_p]),
     "mase_gemm_mxint8_packed_code_bytes": (c_size_t, [c_size_t, c_size_t]),
     "mase_gemm_mxint8_packed_scale_bytes": (c_size_t, [c_size_t, c_size_t]),
     "mase_gemm_mxint8_pack_b": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_void_p]),

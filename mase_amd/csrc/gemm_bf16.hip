@@ -52,7 +52,6 @@ struct GemmParams {
   const unsigned char* B;
   const unsigned char* Bs;  // BCODES: the scale image that goes with the code image in B
   const void* bias;
-  const void* residual;  // RES instantiation: [M, N] in the output dtype, added to the rounded output
   void* C;
   int M, N, K;
   int bias_dtype;
@@ -105,31 +104,23 @@ __device__ __forceinline__ void load_2_untracked(uint32_t& dst, uint32_t off, co
   asm volatile("global_load_ushort %0, %1, %2" : "=v"(dst) : "v"(off), "s"(base) : "memory");
 }
 
-// four codes (already offset by 128: unsigned bytes) -> two registers of two bf16 values each: (u - 128) * scale,
-// exact in fp32, at most 8 significant bits, so the upper halves are the values
-__device__ __forceinline__ void ucodes4_to_bf16(uint32_t u, float scale, float bias, uint32_t& lo, uint32_t& hi) {
-  const float f0 = __builtin_fmaf((float)(u & 0xFFu), scale, bias);
-  const float f1 = __builtin_fmaf((float)((u >> 8) & 0xFFu), scale, bias);
-  const float f2 = __builtin_fmaf((float)((u >> 16) & 0xFFu), scale, bias);
-  const float f3 = __builtin_fmaf((float)(u >> 24), scale, bias);
-  lo = __builtin_amdgcn_perm(f2bits(f1), f2bits(f0), 0x07060302u);
-  hi = __builtin_amdgcn_perm(f2bits(f3), f2bits(f2), 0x07060302u);
-}
-
 // STREAM: K holds at least S tiles, so the copy stream is never more than one output tile ahead and advances
 // without branches; the other instantiation (K = one tile) advances it with the general, branching step.
 // BPACK (with STREAM, an even number of K tiles): B is the fragment-ordered image of mase_gemm_bf16_pack_b and its
 // fragments go from L2 straight into registers, one K tile ahead of the MFMAs that use them; only A passes through
-// LDS, in four stages of 32 KB.  That halves the LDS traffic (the copies landing in LDS while the wavefronts read
-// their fragments is what holds the plain kernel back) at the price of every B fragment being fetched by the two
-// wavefronts that share it.
+// LDS, in four stages of 32 KB (the copies landing in LDS while the wavefronts read their fragments is what holds the
+// plain kernel back).  The four wavefronts then split the 256 x 256 tile 1 x 4 (each 256 rows x 64 columns: 8 x 2 MFMA
+// tiles) instead of 2 x 2 (128 x 128: 4 x 4), so that no two wavefronts load the same B fragments: the CU's
+// vector-memory path carries 32 KB of B per K tile next to A's 32 KB (64 KB with the 2 x 2 split, measured 5 % slower),
+// at the price of each wavefront reading all of A from LDS.  That path, not the matrix pipe, is what the K loop waits
+// for.
 // BCODES (with BPACK): B is an MXINT8 weight as codes + scale bytes in fragment order (mase_gemm_mxint8_pack_b): half
 // the bytes of the bf16 image in memory and on the way in; the codes are widened to the same bf16 operand values in
 // registers, one K step ahead of the MFMAs that use them (code + 128 as an unsigned byte -> v_cvt_f32_ubyte -> one fma
 // that removes the 128 and applies the block's power-of-two scale -> the upper half of the exact fp32 product).
-template <int OUT_DT, bool STREAM, bool BPACK = false, bool BCODES = false, bool RES = false>
+template <int OUT_DT, bool STREAM, bool BPACK = false, bool BCODES = false>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p) {
-  static_assert(!RES || OUT_DT != MASE_DT_F32, "the residual epilogue holds a tile of 16-bit values in registers");
+  constexpr int NI = BPACK ? 8 : 4, NJ = BPACK ? 2 : 4;  // MFMA tiles of a wavefront: rows x columns
   static_assert(!BCODES || BPACK, "codes come in fragment order");
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int tid = threadIdx.x;
@@ -137,6 +128,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   const int lane = lane_id;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
+  const int row_base = BPACK ? 0 : wm * 128, col_base = BPACK ? wave * 64 : wn * 128;  // the wavefront's part of the tile
   const int nk = p.kc / BK;
 
   // ---- this work-group's output tiles.  Work-groups are dealt to the 8 XCDs round-robin; when the counts
@@ -224,12 +216,12 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     }
   };
 
-  f32x16_t acc[4][4];
+  f32x16_t acc[NI][NJ];
   auto zero_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < NI; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < NJ; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
   };
@@ -247,9 +239,15 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   const int frag_row = lane & 31;
   const int kgrp = lane >> 5;
   // fragment f (0..3: A row tile f, 4..7: B column tile f-4) of K step s of the K tile in `stage`
+  // (BPACK: f = 0..7, A row tile f of the whole tile)
   auto load_frag = [&](int stage, int s, int f) __attribute__((always_inline)) -> bf16x8_t {
-    const unsigned char* st = lds + stage * kStride + ((f < 4) ? (wm * 128) * kRowBytes : kTileBytes + (wn * 128) * kRowBytes);
-    return __builtin_bit_cast(bf16x8_t, *(const uint4*)(st + lds_off((f & 3) * 32 + frag_row, s * 2 + kgrp)));
+    if constexpr (BPACK) {
+      const unsigned char* st = lds + stage * kStride;
+      return __builtin_bit_cast(bf16x8_t, *(const uint4*)(st + lds_off(f * 32 + frag_row, s * 2 + kgrp)));
+    } else {
+      const unsigned char* st = lds + stage * kStride + ((f < 4) ? (wm * 128) * kRowBytes : kTileBytes + (wn * 128) * kRowBytes);
+      return __builtin_bit_cast(bf16x8_t, *(const uint4*)(st + lds_off((f & 3) * 32 + frag_row, s * 2 + kgrp)));
+    }
   };
 
   // ---- epilogue of one output tile: accumulators -> bands of 8 rows x 64 columns through the wavefront's own
@@ -270,13 +268,18 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     float* stg = (float*)(lds + S * kStageBytes + wave * kStgWave) + kgrp * (4 * kStgStride);
     const int c4 = (lane & 15) * 4;          // columns within the 64-column band
     const int rl0 = (lane & 31) >> 4;        // this lane reads rows rl0 and rl0 + 2 of its half-wave's 4
-    float bv[2][4] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+    constexpr int NJH = NJ / 2;  // 64-column bands across the wavefront's columns
+    float bv[NJH][4];
+#pragma unroll
+    for (int jh = 0; jh < NJH; ++jh)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bv[jh][e] = 0.0f;
     if (p.bias != nullptr) {
 #pragma unroll
-      for (int jh = 0; jh < 2; ++jh)
+      for (int jh = 0; jh < NJH; ++jh)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const int col = n0 + wn * 128 + jh * 64 + c4 + e;
+          const int col = n0 + col_base + jh * 64 + c4 + e;
           if (col < p.N) bv[jh][e] = load_bias(p.bias, p.bias_dtype, col);
         }
       // The bias loads are the only vector-memory loads the compiler itself tracks in this kernel.  Completing
@@ -284,33 +287,12 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
       // inside the K loop, where that would also wait for every async copy in flight.
       wait_vmcnt<0>();
     }
-    // RES: out = round(round(A B^T + bias) + residual), the two roundings of a Linear followed by a residual add.
-    // The lane's 64 pieces of 4 residual values (the ones it stores below) are all requested before the first band
-    // and completed by one wait, so the tile pays one memory latency, not one per band.
-    uint2 rv[RES ? 64 : 1];
-    if constexpr (RES) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-#pragma unroll
-          for (int jh = 0; jh < 2; ++jh)
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-              const int row = m0 + wm * 128 + i * 32 + q * 8 + kgrp * 4 + rl0 + 2 * u;
-              const int col0 = n0 + wn * 128 + jh * 64 + c4;
-              uint2 r = make_uint2(0u, 0u);
-              if (row < p.M && col0 + 3 < p.N) r = *(const uint2*)((const uint16_t*)p.residual + (size_t)row * p.N + col0);
-              rv[((i * 4 + q) * 2 + jh) * 2 + u] = r;
-            }
-      wait_vmcnt<0>();
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < NI; ++i) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
 #pragma unroll
-        for (int jh = 0; jh < 2; ++jh) {
+        for (int jh = 0; jh < NJH; ++jh) {
 #pragma unroll
           for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
@@ -318,13 +300,13 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
               stg[rr * kStgStride + jj * 32 + frag_row] = acc[i][jh * 2 + jj][q * 4 + rr];
           asm volatile("" ::: "memory");  // lanes exchange data through LDS: no value may be carried across
           __builtin_amdgcn_sched_barrier(0);  // bands stay in program order: bounded register use
-          const int col0 = n0 + wn * 128 + jh * 64 + c4;
+          const int col0 = n0 + col_base + jh * 64 + c4;
 #pragma unroll
           for (int u = 0; u < 2; ++u) {
             const int rl = rl0 + 2 * u;
             const float4 v4 = *(const float4*)(stg + rl * kStgStride + c4);
             const float v[4] = {v4.x + bv[jh][0], v4.y + bv[jh][1], v4.z + bv[jh][2], v4.w + bv[jh][3]};
-            const int row = m0 + wm * 128 + i * 32 + q * 8 + kgrp * 4 + rl;
+            const int row = m0 + row_base + i * 32 + q * 8 + kgrp * 4 + rl;
             if (row >= p.M) continue;
             const size_t o = (size_t)row * p.N + col0;
             // streaming stores: the output is not read again by this kernel and should not displace operand panels
@@ -335,23 +317,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
                 uint2 w;
                 w.x = f32x2_to_bf16x2_bits(v[0], v[1]);
                 w.y = f32x2_to_bf16x2_bits(v[2], v[3]);
-                if constexpr (RES) {
-                  const uint2 r = rv[((i * 4 + q) * 2 + jh) * 2 + u];
-                  w.x = f32x2_to_bf16x2_bits(bits2f(w.x << 16) + bits2f(r.x << 16), bits2f(w.x & 0xFFFF0000u) + bits2f(r.x & 0xFFFF0000u));
-                  w.y = f32x2_to_bf16x2_bits(bits2f(w.y << 16) + bits2f(r.y << 16), bits2f(w.y & 0xFFFF0000u) + bits2f(r.y & 0xFFFF0000u));
-                }
                 store_nt((uint2*)((uint16_t*)Cs + o), w);
               } else {
                 uint2 w;
                 w.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
                 w.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
-                if constexpr (RES) {
-                  const uint2 r = rv[((i * 4 + q) * 2 + jh) * 2 + u];
-                  w.x = f32_to_f16_bits(f16_bits_to_f32(w.x & 0xFFFFu) + f16_bits_to_f32(r.x & 0xFFFFu)) |
-                        (f32_to_f16_bits(f16_bits_to_f32(w.x >> 16) + f16_bits_to_f32(r.x >> 16)) << 16);
-                  w.y = f32_to_f16_bits(f16_bits_to_f32(w.y & 0xFFFFu) + f16_bits_to_f32(r.y & 0xFFFFu)) |
-                        (f32_to_f16_bits(f16_bits_to_f32(w.y >> 16) + f16_bits_to_f32(r.y >> 16)) << 16);
-                }
                 store_nt((uint2*)((uint16_t*)Cs + o), w);
               }
             } else {
@@ -390,16 +360,16 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // stream is advanced by a caller-supplied, branch-free step.
   // The epilogue's stores count in vmcnt like the copies, so the first hand-over of an output tile also waits
   // for the previous tile's stores to be acknowledged.
-  bf16x8_t fr[4][BPACK ? 4 : 8];
+  bf16x8_t fr[4][8];
   // BPACK: B fragments of two K tiles (the one in use and the one being loaded): [buffer][K step][column tile].
   // Image layout: 1 KB blocks [column tile of 32][K step of 16][lane][8 bf16], lane l = column l % 32, K 8*(l/32)..+8.
-  bf16x8_t fb[(BPACK && !BCODES) ? 2 : 1][(BPACK && !BCODES) ? 4 : 1][4];
+  bf16x8_t fb[(BPACK && !BCODES) ? 2 : 1][(BPACK && !BCODES) ? 4 : 1][NJ];
   // BCODES: the codes of two K tiles [buffer][K step][column tile] (8 per lane), their scale bytes [buffer][column
   // tile] (the two blocks of 32 a K tile holds, for the lane's column) and the widened fragments of two K steps
-  uint2 fbc[BCODES ? 2 : 1][BCODES ? 4 : 1][4];
-  uint32_t fsc[BCODES ? 2 : 1][4];
-  uint4 fbq[2][4];
-  uint32_t soff[4];          // BCODES: this lane's byte offset of K tile 0 of its four column tiles in the scale image
+  uint2 fbc[BCODES ? 2 : 1][BCODES ? 4 : 1][2];
+  uint32_t fsc[BCODES ? 2 : 1][2];
+  uint4 fbq[2][2];
+  uint32_t soff[2];          // BCODES: this lane's byte offset of K tile 0 of its four column tiles in the scale image
   const unsigned char* s_kbase = p.Bs;
   uint32_t boff[4];          // this lane's byte offset of K step 0 of its four column tiles
   const unsigned char* b_kbase = p.B;  // image address of K tile 0 of the K range of the output tile being loaded
@@ -412,8 +382,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     const int nt_last = (p.N + 31) / 32 - 1;
     constexpr uint32_t kFragBytes = BCODES ? 512u : 1024u;  // one fragment of a wavefront: 8 codes or 8 bf16 per lane
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const size_t ct = (size_t)min((n0 + wn * 128) / 32 + j, nt_last);
+    for (int j = 0; j < NJ; ++j) {
+      const size_t ct = (size_t)min((n0 + col_base) / 32 + j, nt_last);
       boff[j] = (uint32_t)(ct * (size_t)(p.K / 16) * kFragBytes) + (uint32_t)lane * (kFragBytes / 64u);
       if constexpr (BCODES) soff[j] = (uint32_t)(ct * (size_t)(p.K / 64) * 64u) + (uint32_t)(lane & 31) * 2u;
     }
@@ -423,32 +393,45 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   };
   // BCODES: widening of the fragment of column tile j, K step st of the K tile in code buffer `buf` into fragment set
   // `set`; `half` 0 / 1 = the first / second four codes.  The scale byte of a step is byte st / 2 of the lane's two.
-  auto widen = [&](int set, int buf, int st, int j, int half) __attribute__((always_inline)) {
-    const uint32_t sb = (fsc[buf][j] >> (8 * (st >> 1))) & 0xFFu;
-    const float scale = bits2f(sb >= 8u ? (sb - 7u) << 23 : 0u);  // 2^(sb - 134)
-    const float bias = -128.0f * scale;
-    uint32_t lo, hi;
-    ucodes4_to_bf16(half ? fbc[buf][st][j].y : fbc[buf][st][j].x, scale, bias, lo, hi);
-    if (half) { fbq[set][j].z = lo; fbq[set][j].w = hi; }
-    else { fbq[set][j].x = lo; fbq[set][j].y = hi; }
+  // The widening is issued in pieces small enough to hide between two MFMAs (which leave room for about seven VALU
+  // instructions): set_scale puts the scale of block `blk` (0 / 1) of column tile j of the K tile in buffer `buf`, and
+  // the -128 * scale that removes the code offset, into wsc / wbs; widen_quarter makes register q (0..3: two codes) of
+  // the fragment of column tile j, K step st ((code - 128) * scale is exact in fp32 and has at most 8 significant
+  // bits, so the upper half of the fp32 value is the bf16 value).
+  float wsc[2], wbs[2];
+  auto set_scale = [&](int buf, int blk, int j) __attribute__((always_inline)) {
+    const uint32_t sb = (fsc[buf][j] >> (8 * blk)) & 0xFFu;
+    wsc[j] = bits2f(sb >= 8u ? (sb - 7u) << 23 : 0u);  // 2^(sb - 134)
+    wbs[j] = -128.0f * wsc[j];
+  };
+  auto widen_quarter = [&](int set, int buf, int st, int j, int q) __attribute__((always_inline)) {
+    const uint32_t u = (q & 2) ? fbc[buf][st][j].y : fbc[buf][st][j].x;
+    const float f0 = __builtin_fmaf((float)((q & 1) ? (u >> 16) & 0xFFu : u & 0xFFu), wsc[j], wbs[j]);
+    const float f1 = __builtin_fmaf((float)((q & 1) ? u >> 24 : (u >> 8) & 0xFFu), wsc[j], wbs[j]);
+    const uint32_t r = __builtin_amdgcn_perm(f2bits(f1), f2bits(f0), 0x07060302u);  // the upper halves: two bf16
+    if (q == 0) fbq[set][j].x = r;
+    else if (q == 1) fbq[set][j].y = r;
+    else if (q == 2) fbq[set][j].z = r;
+    else fbq[set][j].w = r;
   };
   if constexpr (BCODES) {
     set_b_tile(0);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) load_2_untracked(fsc[0][j], soff[j], s_kbase);
+    for (int j = 0; j < 2; ++j) load_2_untracked(fsc[0][j], soff[j], s_kbase);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) load_8_untracked(fbc[0][i >> 2][i & 3], boff[i & 3], b_kbase + (size_t)(i >> 2) * 512);
+    for (int i = 0; i < 8; ++i) load_8_untracked(fbc[0][i >> 1][i & 1], boff[i & 1], b_kbase + (size_t)(i >> 1) * 512);
     b_kt = 1;
     wait_vmcnt<0>();
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      widen(0, 0, 0, j, 0);
-      widen(0, 0, 0, j, 1);
+    for (int j = 0; j < 2; ++j) {
+      set_scale(0, 0, j);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) widen_quarter(0, 0, 0, j, q);
     }
   } else if constexpr (BPACK) {
     set_b_tile(0);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) load_16_untracked(fb[0][i >> 2][i & 3], boff[i & 3], b_kbase + (size_t)(i >> 2) * 1024);
+    for (int i = 0; i < 4 * NJ; ++i) load_16_untracked(fb[0][i / NJ][i % NJ], boff[i % NJ], b_kbase + (size_t)(i / NJ) * 1024);
     b_kt = 1;
     wait_vmcnt<0>();
   } else {
@@ -456,7 +439,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   }
   asm volatile("s_barrier" ::: "memory");
 #pragma unroll
-  for (int f = 0; f < (BPACK ? 4 : 8); ++f) fr[0][f] = load_frag(0, 0, f);
+  for (int f = 0; f < 8; ++f) fr[0][f] = load_frag(0, 0, f);
   int stage = 0;
   // BPACK form of the K iteration.  The wavefront has two kinds of loads in flight, the B fragment loads into
   // registers and the A copies into LDS.  Each kind retires in order, but the two kinds do NOT retire in order with
@@ -467,40 +450,42 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // three K tiles ahead, so when a hand-over needs the next K tile, the 16 copies of the two K tiles after it have
   // been issued, and the hand-over waits for "at most 16 outstanding": the next K tile has landed (its copies are older
   // than those 16), while the young copies and up to that many B loads fly on across the barrier.  The B fragments are
-  // proven the same way, by counting the register loads issued after them (see the waits at the head of each step).
-  //   step 0: MFMAs on fr[0]; LDS reads of step 1; the 16 B loads of the next K tile (their registers were last read
-  //           one K tile ago)
-  //   step 1: MFMAs on fr[1]; LDS reads of steps 2 and 3; the 8 A copies of the K tile three ahead into the stage
+  // proven the same way, by counting the *register loads* issued after them: at the head of step s the two fragments
+  // of the step (loads 2s+1, 2s+2 of the 8 issued one K tile ago) have landed once at most 6 / 12 / 10 / 8 loads are
+  // outstanding (the rest of their batch, plus from step 1 on the 8 of the next batch issued during step 0).
+  // Per step 16 MFMAs, MFMA t on (A row tile t / 2, B column tile t % 2):
+  //   step 0: MFMAs on fr[0]; LDS reads of step 1 (8) and the 8 B loads of the next K tile (their registers were last
+  //           read one K tile ago), one each per MFMA slot 0..7
+  //   step 1: MFMAs on fr[1]; LDS reads of steps 2 and 3 (16); the 8 A copies of the K tile three ahead into the stage
   //           vacated at the previous hand-over, one every other MFMA slot
   //   step 2: MFMAs on fr[2]; then the hand-over: at most 16 loads outstanding, own LDS reads complete, barrier
-  //   step 3: MFMAs on fr[3]; LDS reads of step 0 of the next K tile
-  // Stores of an epilogue only make the wait of the next output tile's first hand-over conservative.
+  //   step 3: MFMAs on fr[3]; LDS reads of step 0 of the next K tile (8)
+  // Stores of an epilogue only make the waits of the next output tile's first K tile conservative.
   auto k_iteration_b = [&](auto&& advance, auto bufc) __attribute__((always_inline)) {
     constexpr int NB = decltype(bufc)::value;
     const unsigned char* bsrc = b_kbase + (size_t)b_kt * 4096;
     const int stage_next = next_of(stage);
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
-      // the B fragments of this step (register loads 4s+1 .. 4s+4 of the 16 issued one K tile ago) have landed once
-      // at most as many loads are outstanding as *register loads* were issued after them: the other 12 - 4s of their
-      // batch, plus, from step 1 on, the 16 of the next batch issued during step 0.  (Step 3 is covered by the
-      // hand-over's wait.)
-      if (s == 0) wait_vmcnt<12>();
-      else if (s == 1) wait_vmcnt<24>();
-      else if (s == 2) wait_vmcnt<20>();
+      if (s == 0) wait_vmcnt<6>();
+      else if (s == 1) wait_vmcnt<12>();
+      else if (s == 2) wait_vmcnt<10>();
+      else wait_vmcnt<8>();
 #pragma unroll
       for (int t = 0; t < 16; ++t) {
-        acc[t >> 2][t & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[s][t >> 2], fb[NB][s][t & 3],
-                                                                     acc[t >> 2][t & 3], 0, 0, 0);
+        acc[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[s][t >> 1], fb[NB][s][t & 1],
+                                                                     acc[t >> 1][t & 1], 0, 0, 0);
         if (s == 0) {
-          if (t < 4) fr[1][t] = load_frag(stage, 1, t);
-          load_16_untracked(fb[NB ^ 1][t >> 2][t & 3], boff[t & 3], bsrc + (size_t)(t >> 2) * 1024);
+          if (t < 8) {
+            fr[1][t] = load_frag(stage, 1, t);
+            load_16_untracked(fb[NB ^ 1][t >> 1][t & 1], boff[t & 1], bsrc + (size_t)(t >> 1) * 1024);
+          }
         } else if (s == 1) {
-          if (t < 4) fr[2][t] = load_frag(stage, 2, t);
-          else if (t < 8) fr[3][t - 4] = load_frag(stage, 3, t - 4);
+          if (t < 8) fr[2][t] = load_frag(stage, 2, t);
+          else fr[3][t - 8] = load_frag(stage, 3, t - 8);
           if (t & 1) issue_copy(t - 1);
         } else if (s == 3) {
-          if (t < 4) fr[0][t] = load_frag(stage_next, 0, t);
+          if (t < 8) fr[0][t] = load_frag(stage_next, 0, t);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -514,12 +499,13 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     stage = stage_next;
     ++b_kt;
   };
-  // BCODES form: as the BPACK form, with 4 scale loads and 16 code loads per K tile (in that order, step 0) and the
-  // widening of K step s + 1 (of step 0 of the next K tile during step 3) spread over the MFMA slots of step s, two
-  // slots per half fragment.  A step's codes must have landed one step earlier than in the BPACK form; counting the
-  // register loads issued after them: codes of step 1 (loads 9-12 of the 20): 8 at the head of the K tile; step 2:
-  // 4 + 20 at the head of step 1; step 3: 20 at the head of step 2; step 0 of the next K tile and the scales: covered
-  // by the hand-over's 8.
+  // BCODES form: as the BPACK form, with 2 scale loads and 8 code loads per K tile (step 0, slots 0..7: the scale of
+  // column tile t first in slots 0 and 1, then the codes of K step t / 2, column tile t % 2) and the widening of K
+  // step s + 1 (of step 0 of the next K tile during step 3) spread over the MFMA slots of step s, two codes at a
+  // time.  A step's codes must have landed one step earlier than in the BPACK form; counting the register loads issued after them (batch order S0 C0 S1 C1 C2 .. C7): codes of step 1 (C2, C3):
+  // 4 at the head of the K tile; step 2 (C4, C5): 2 + the 10 of the next batch at the head of step 1; step 3: 10 at
+  // the head of step 2; scales and codes of step 0 of the next K tile (S0 .. C1 of the batch issued during step 0):
+  // 6 at the head of step 3.
   auto k_iteration_c = [&](auto&& advance, auto bufc) __attribute__((always_inline)) {
     constexpr int NB = decltype(bufc)::value;
     const unsigned char* bsrc = b_kbase + (size_t)b_kt * 2048;
@@ -527,29 +513,34 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     const int stage_next = next_of(stage);
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
-      if (s == 0) wait_vmcnt<8>();
-      else if (s == 1) wait_vmcnt<24>();
-      else if (s == 2) wait_vmcnt<20>();
+      if (s == 0) wait_vmcnt<4>();
+      else if (s == 1) wait_vmcnt<12>();
+      else if (s == 2) wait_vmcnt<10>();
+      else wait_vmcnt<6>();
 #pragma unroll
       for (int t = 0; t < 16; ++t) {
-        acc[t >> 2][t & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            fr[s][t >> 2], __builtin_bit_cast(bf16x8_t, fbq[s & 1][t & 3]), acc[t >> 2][t & 3], 0, 0, 0);
-        if ((t & 1) == 0) {  // half fragment (t >> 2, (t >> 1) & 1) of the next step
-          if (s < 3) widen((s + 1) & 1, NB, s + 1, t >> 2, (t >> 1) & 1);
-          else widen(0, NB ^ 1, 0, t >> 2, (t >> 1) & 1);
+        acc[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            fr[s][t >> 1], __builtin_bit_cast(bf16x8_t, fbq[s & 1][t & 1]), acc[t >> 1][t & 1], 0, 0, 0);
+        // slots 0, 1 of the steps after which the block of 32 changes: the scales the next step's codes take; slots
+        // 2, 4, .., 14, 15: quarter u = 0..7 (column tile u / 4, register u % 4) of the next step's fragments
+        if ((s & 1) && t < 2) set_scale(s == 1 ? NB : NB ^ 1, s == 1 ? 1 : 0, t);
+        const int u = (t == 15) ? 7 : ((t >= 2 && !(t & 1)) ? (t - 2) >> 1 : -1);
+        if (u >= 0) {
+          if (s < 3) widen_quarter((s + 1) & 1, NB, s + 1, u >> 2, u & 3);
+          else widen_quarter(0, NB ^ 1, 0, u >> 2, u & 3);
         }
         if (s == 0) {
-          if (t < 4) {
+          if (t < 8) {
             fr[1][t] = load_frag(stage, 1, t);
-            load_2_untracked(fsc[NB ^ 1][t], soff[t], ssrc);
+            if (t < 2) load_2_untracked(fsc[NB ^ 1][t], soff[t], ssrc);
+            load_8_untracked(fbc[NB ^ 1][t >> 1][t & 1], boff[t & 1], bsrc + (size_t)(t >> 1) * 512);
           }
-          load_8_untracked(fbc[NB ^ 1][t >> 2][t & 3], boff[t & 3], bsrc + (size_t)(t >> 2) * 512);
         } else if (s == 1) {
-          if (t < 4) fr[2][t] = load_frag(stage, 2, t);
-          else if (t < 8) fr[3][t - 4] = load_frag(stage, 3, t - 4);
+          if (t < 8) fr[2][t] = load_frag(stage, 2, t);
+          else fr[3][t - 8] = load_frag(stage, 3, t - 8);
           if (t & 1) issue_copy(t - 1);
         } else if (s == 3) {
-          if (t < 4) fr[0][t] = load_frag(stage_next, 0, t);
+          if (t < 8) fr[0][t] = load_frag(stage_next, 0, t);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -693,25 +684,9 @@ int launch_gemm_bf16(const GemmParams& p, int out_dtype, hipStream_t st, bool bp
     }                                                                                                             \
     hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, true, true>), grid, block, lds_bytes, st, p);                    \
   } while (0)
-#define MASE_GEMM_LAUNCH_R(DT_)                                                                                   \
-  do {                                                                                                            \
-    static bool attr_set = false;                                                                                 \
-    const void* k = (const void*)gemm_bf16_tn_kernel<DT_, true, true, false, true>;                               \
-    if (!attr_set) {                                                                                              \
-      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)       \
-        return MASE_ERR_LAUNCH;                                                                                   \
-      attr_set = true;                                                                                            \
-    }                                                                                                             \
-    hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, true, true, false, true>), grid, block, lds_bytes, st, p);       \
-  } while (0)
-    if (p.residual != nullptr) {
-      if (out_dtype == MASE_DT_BF16) MASE_GEMM_LAUNCH_R(MASE_DT_BF16);
-      else if (out_dtype == MASE_DT_F16) MASE_GEMM_LAUNCH_R(MASE_DT_F16);
-      else return MASE_ERR_DTYPE;
-    } else if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH_B(MASE_DT_F32);
+    if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH_B(MASE_DT_F32);
     else if (out_dtype == MASE_DT_BF16) MASE_GEMM_LAUNCH_B(MASE_DT_BF16);
     else MASE_GEMM_LAUNCH_B(MASE_DT_F16);
-#undef MASE_GEMM_LAUNCH_R
 #undef MASE_GEMM_LAUNCH_B
   } else if (stream_fits) {
     if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH(MASE_DT_F32, true);
@@ -822,7 +797,6 @@ extern "C" int mase_gemm_bf16_tn(const void* A, const void* B, const void* bias,
   p.B = (const unsigned char*)B;
   p.Bs = nullptr;
   p.bias = bias;
-  p.residual = nullptr;
   p.C = C;
   p.M = (int)M;
   p.N = (int)N;
@@ -861,7 +835,6 @@ extern "C" int mase_gemm_bf16_tn_splitk(const void* A, const void* B, const void
   p.B = (const unsigned char*)B;
   p.Bs = nullptr;
   p.bias = nullptr;
-  p.residual = nullptr;
   p.C = workspace;
   p.M = (int)M;
   p.N = (int)N;
@@ -918,37 +891,6 @@ extern "C" int mase_gemm_bf16_tn_packed(const void* A, const void* B_packed, con
   p.B = (const unsigned char*)B_packed;
   p.Bs = nullptr;
   p.bias = bias;
-  p.residual = nullptr;
-  p.C = C;
-  p.M = (int)M;
-  p.N = (int)N;
-  p.K = (int)K;
-  p.bias_dtype = bias_dtype;
-  p.tiles_m = (int)((M + BM - 1) / BM);
-  p.tiles_n = (int)((N + BN - 1) / BN);
-  p.splits = 1;
-  p.kc = (int)K;
-  return launch_gemm_bf16(p, out_dtype, (hipStream_t)stream, true);
-}
-
-extern "C" int mase_gemm_bf16_tn_packed_residual(const void* A, const void* B_packed, const void* bias, const void* residual,
-                                                 void* C, size_t M, size_t N, size_t K, int out_dtype, int bias_dtype,
-                                                 void* stream) {
-  using namespace mase;
-  if (M == 0 || N == 0) return MASE_OK;
-  if (A == nullptr || B_packed == nullptr || C == nullptr || residual == nullptr) return MASE_ERR_NULL;
-  if (K == 0 || (K % (2 * BK)) != 0 || (N % 4) != 0 || M > (1u << 30) || N > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
-  if ((unsigned long long)M * K * 2 > 0xFFFFFFFFull || (unsigned long long)mase_gemm_bf16_packed_bytes(N, K) > 0xFFFFFFFFull)
-    return MASE_ERR_SHAPE;
-  if (!aligned16(A) || !aligned16(B_packed) || !aligned16(C) || (((uintptr_t)residual) & 7u) != 0) return MASE_ERR_ALIGN;
-  if ((out_dtype != MASE_DT_BF16 && out_dtype != MASE_DT_F16) || (bias != nullptr && (bias_dtype < 0 || bias_dtype > 2)))
-    return MASE_ERR_DTYPE;
-  GemmParams p;
-  p.A = (const unsigned char*)A;
-  p.B = (const unsigned char*)B_packed;
-  p.Bs = nullptr;
-  p.bias = bias;
-  p.residual = residual;
   p.C = C;
   p.M = (int)M;
   p.N = (int)N;
@@ -1001,7 +943,6 @@ extern "C" int mase_gemm_mxint8_tn_packed(const void* A, const void* code_image,
   p.B = (const unsigned char*)code_image;
   p.Bs = (const unsigned char*)scale_image;
   p.bias = bias;
-  p.residual = nullptr;
   p.C = C;
   p.M = (int)M;
   p.N = (int)N;

@@ -77,21 +77,19 @@ def _tensor_key(t: Tensor):
 
 
 def mx_linear(x: Tensor, weight: Tensor, bias: Tensor | None, quantize_to_bf16, quantize_same_dtype,
-              cache: WeightCache, xq: Tensor | None = None, residual: Tensor | None = None) -> Tensor:
+              cache: WeightCache, xq: Tensor | None = None) -> Tensor:
     """``F.linear(q(x), weight, bias)``.  ``quantize_to_bf16(x2d)`` returns q(x) as bf16 (exact);
     ``quantize_same_dtype(x)`` returns q(x) in x's dtype (used when the weight has no exact bf16 image).
     ``xq``: q(x) as a bf16 matrix when the caller already has it (sibling projections of one tensor, see
-    ``project_shared``).  ``residual``: the result is ``residual + F.linear(...)`` (the values of the two operations),
-    added in the GEMM's epilogue where that kernel runs."""
+    ``project_shared``)."""
     wb = cache.get(weight) if x.is_cuda and weight.dim() == 2 else None
     if wb is None or x.dtype not in (torch.float32, torch.bfloat16, torch.float16):
-        y = F.linear(quantize_same_dtype(x), weight, bias)
-        return y if residual is None else residual + y
+        return F.linear(quantize_same_dtype(x), weight, bias)
     lead = x.shape[:-1]
     if xq is None:
         xq = quantize_to_bf16(x.reshape(-1, x.shape[-1]))
     wp = cache.packed() if gemm_bf16_takes_packed_b(xq.shape[0], wb.shape[0], wb.shape[1]) else None
-    y = gemm_bf16_tn(xq, wb, bias, x.dtype, b_packed=wp, residual=residual)
+    y = gemm_bf16_tn(xq, wb, bias, x.dtype, b_packed=wp)
     return y.reshape(*lead, weight.shape[0])
 
 

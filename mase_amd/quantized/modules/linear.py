@@ -216,15 +216,7 @@ class LinearMXInt(_LinearMX):
         return _ops.mxint_qdq(x.reshape(-1, x.shape[-1]), bs, bits, -1, 8, out_dtype=torch.bfloat16)
 
     @torch.no_grad()
-    def forward(self, x, prepared=None, residual=None):
-        """``prepared``, ``residual``: not arguments of the reference's forward.  ``prepared`` is this module's quantized
-        form of ``x`` when the caller already holds it; with ``residual`` the result is ``residual + forward(x)``, the
-        sum of a pre-norm block (models/llama/modeling_llama.py:901, :908), added in the GEMM's epilogue on the tiled
-        path and by a tensor addition elsewhere, with the same values."""
-        if residual is not None:
-            if (self.bypass or None in self._act_cfg() or mxint_decode_applies(x, self._w_codes, self.weight)
-                    or mxint_codes_apply(x, self._w_image, self.weight)):
-                return residual + self.forward(x, prepared=prepared)
+    def forward(self, x, prepared=None):
         if self.bypass:
             return F.linear(x, self.weight, self.bias)
         bs, bits = self._act_cfg()
@@ -237,7 +229,7 @@ class LinearMXInt(_LinearMX):
         return mx_linear(
             x, self.weight, self.bias, self.prepare_activation,
             lambda t: mxint_quantizer(t, block_size=bs, element_bits=bits, block_dim=-1),
-            self._w_cache, xq=prepared, residual=residual,
+            self._w_cache, xq=prepared,
         )
 
 

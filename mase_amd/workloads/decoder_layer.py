@@ -23,7 +23,6 @@ from torch.nn import functional as F
 
 from ..quantizers import _ops
 from ..quantized.functional.mx_linear import project_shared, shared_mxint_width
-from ..quantized.modules.linear import LinearMXInt
 
 
 @dataclass
@@ -123,12 +122,6 @@ class DecoderLayer(nn.Module):
                 return [m(hq, prepared=hq.reshape(-1, hq.shape[-1])) for m in modules]
         return project_shared(norm(x), modules)
 
-    def _project_add(self, module, x, residual, prepared=None):
-        """``residual + module(x)``; an MXINT Linear adds the residual in its GEMM's epilogue (the same two roundings)"""
-        if self.fuse_producers and isinstance(module, LinearMXInt) and not torch.is_grad_enabled():
-            return module(x, prepared=prepared, residual=residual)
-        return residual + (module(x) if prepared is None else module(x, prepared=prepared))
-
     def _rope_tables(self, T, device, dtype):
         """the cos / sin tables of the rotary embedding depend on (sequence length, device, dtype) only: kept from one
         forward to the next (a model computes them once per forward for all its layers)"""
@@ -161,17 +154,17 @@ class DecoderLayer(nn.Module):
         else:
             a = self.attention_fn(q, k, v)
         a = a.transpose(1, 2).reshape(B, T, cfg.num_heads * cfg.head_dim)
-        x = self._project_add(self.o_proj, a, x, prepared=a.reshape(-1, a.shape[-1]) if bits is not None else None)
+        x = x + (self.o_proj(a, prepared=a.reshape(-1, a.shape[-1])) if bits is not None else self.o_proj(a))
         gate, up = self._norm_then_project(self.post_attention_layernorm, x, (self.gate_proj, self.up_proj))
         if gate.is_cuda and _ops.silu_mul_supported(gate, up):
             bits = shared_mxint_width(gate, (self.down_proj,)) if self.fuse_producers and gate.shape[-1] % 32 == 0 else None
             if bits is not None and not torch.is_grad_enabled():
                 actq = _ops.silu_mul_mxint(gate, up, bits)  # the product, already in down_proj's quantized form
-                return self._project_add(self.down_proj, actq, x, prepared=actq.reshape(-1, actq.shape[-1]))
+                return x + self.down_proj(actq, prepared=actq.reshape(-1, actq.shape[-1]))
             act = _ops.silu_mul_minifloat(gate, up)  # silu(gate) * up in one pass
         else:
             act = F.silu(gate) * up
-        return self._project_add(self.down_proj, act, x)
+        return x + self.down_proj(act)
 
     def linear_flops(self, tokens: int) -> float:
         H, D, I = self.cfg.hidden_size, self.cfg.num_heads * self.cfg.head_dim, self.cfg.intermediate_size

@@ -219,34 +219,6 @@ def test_gemm_with_the_weight_in_fragment_order_is_the_same_product(dev, M, N, K
         assert float((gemm_bf16_tn(a, b, None, torch.float32, b_packed=bp) - ref).abs().max() / ref.abs().max()) < 1e-5
 
 
-@pytest.mark.parametrize("M,N,K", [(4096, 4096, 1024), (4100, 4200, 640), (16384, 4096, 4096), (16131, 4096, 11008), (1000, 36, 128),
-                                   (300, 200, 384)])
-def test_gemm_with_the_residual_added_in_the_epilogue(dev, M, N, K):
-    """residual + Linear in one kernel (mase_gemm_bf16_tn_packed_residual) against the product rounded to the output
-    dtype followed by a tensor addition: bit-identical, bf16 and fp16, with and without bias, ragged M and N (N a
-    multiple of 4), several launches; shapes that do not take the tiled fragment-ordered kernel (few rows, K not a
-    multiple of 128) and fp32 outputs fall back to the tensor addition inside the wrapper and give the same values"""
-    from mase_amd._gemm import gemm_bf16_pack_b, gemm_bf16_packed_b_supported, gemm_bf16_takes_packed_b, gemm_bf16_tn
-
-    g = torch.Generator().manual_seed(M + N + K + 5)
-    a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
-    b = (torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16).to(dev)
-    bias = torch.randn(N, generator=g).to(dev)
-    print(f"residual gemm M={M} N={N} K={K} tiled={gemm_bf16_takes_packed_b(M, N, K)}", flush=True)
-    bp = gemm_bf16_pack_b(b) if gemm_bf16_packed_b_supported(N, K) else None
-    for dt, bs in ((torch.bfloat16, bias), (torch.float16, None), (torch.float32, bias)):
-        r = (torch.randn(M, N, generator=g) * 3).to(dt).to(dev)
-        want = gemm_bf16_tn(a, b, bs, dt, b_packed=bp) + r
-        for rep in range(3):
-            got = gemm_bf16_tn(a, b, bs, dt, b_packed=bp, residual=r)
-            assert got.dtype == dt and torch.equal(got, want), (dt, rep, float((got.float() - want.float()).abs().max()))
-    # a residual handed over with leading dimensions (a [B, T, N] hidden state)
-    r3 = (torch.randn(2, M // 2, N, generator=g)).to(torch.bfloat16).to(dev) if M % 2 == 0 else None
-    if r3 is not None:
-        assert torch.equal(gemm_bf16_tn(a, b, None, torch.bfloat16, b_packed=bp, residual=r3),
-                           gemm_bf16_tn(a, b, None, torch.bfloat16, b_packed=bp) + r3.reshape(M, N))
-
-
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (512, 768, 256), (300, 200, 384), (4096, 4096, 1024), (130, 4096, 512),
                                    (4100, 4200, 640), (16384, 1024, 4096), (16384, 4096, 11008), (16131, 11008, 4096)])
 def test_gemm_with_the_weight_as_mxint8_codes_in_fragment_order(dev, M, N, K):
