@@ -7,8 +7,8 @@
 // products as the reference's fp32 GEMM on the quantize-dequantized operands; only the summation order
 // differs.
 //
-// Schedule: 256x256 output tile (4 wavefronts, 2x2, 128x128 each = 4x4 MFMA tiles, 256 accumulator registers
-// per lane), K tile 64 so that every operand row of a tile is one full 128-byte cache line (64-byte rows made
+// Schedule: 256x256 output tile (4 wavefronts, 2x2, 128x128 each = 4x4 MFMA tiles, or 1x4, 256x64 each = 8x2 MFMA
+// tiles, when B comes in fragment order; 256 accumulator registers per lane either way), K tile 64 so that every operand row of a tile is one full 128-byte cache line (64-byte rows made
 // the L1 fetch every line twice and bound the loop), two LDS stages of 64 KB.  Operand tiles go from HBM/L2
 // straight into LDS with global_load_lds_dwordx4 (no staging registers, no ds_write).  A wavefront-wide copy
 // deposits 64 consecutive 16-byte chunks = 8 LDS rows of 128 B, so the bank-conflict swizzle is applied on
@@ -41,10 +41,11 @@ constexpr int kTileBytes = BM * kRowBytes;        // 32 KB per operand per stage
 constexpr int kStageBytes = 2 * kTileBytes;       // A then B
 constexpr int kWaveCopies = kTileBytes / 1024 / 4;  // copies per wavefront per operand per K tile = 8
 constexpr int kCopies = 2 * kWaveCopies;          // async copies one wavefront issues per K tile = 16
-constexpr int kSteps = BK / 16;                   // MFMA K steps per K tile = 4                   // MFMA K steps per K tile = 4
-// epilogue staging, separate from the stages: per wavefront 8 rows x 64 columns of fp32, row stride 68 floats
-constexpr int kStgStride = 68;
-constexpr int kStgWave = 8 * kStgStride * 4;
+constexpr int kSteps = BK / 16;                   // MFMA K steps per K tile = 4
+// epilogue staging, separate from the stages: per wavefront 32 rows of 128 bytes, row stride 144 bytes (16-byte
+// accesses of 16 consecutive rows at one column offset then fall on 64 different banks)
+constexpr int kStgRow = 144;
+constexpr int kStgWave = 32 * kStgRow;
 constexpr int kLdsBytes = S * kStageBytes + 4 * kStgWave;
 
 struct GemmParams {
@@ -81,6 +82,17 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 __device__ __forceinline__ void async_copy_16(const unsigned char* base, uint32_t off, uint32_t lds_addr) {
   const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_addr);
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
+}
+
+// The lane number, computed where it is needed (two instructions) instead of being kept: the code between output tiles
+// then holds no value across the K loop that the register allocator would spill.  A reload from scratch memory is a
+// vector-memory load the compiler tracks, and it guards such a load with s_waitcnt vmcnt(0), which also waits for
+// every async copy and fragment load in flight.  The asm statement keeps the terms derived from the lane number from
+// being hoisted out of their place and into the K loop's live registers.
+__device__ __forceinline__ int lane_now() {
+  int lane;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
+  return lane;
 }
 
 template <int N>
@@ -169,8 +181,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     int m0, n0, ks;
     tile_origin(ord, m0, n0, ks);
     const uint32_t k0 = (uint32_t)ks * (uint32_t)p.kc * 2u;  // byte offset of the item's K range inside a row
-    int lane = lane_id;
-    asm volatile("" : "+v"(lane));  // keeps the lane-derived terms below out of the K loop's live registers
+    const int lane = lane_now();
 #pragma unroll
     for (int j = 0; j < kWaveCopies; ++j) {
       const int r = (wave + 4 * j) * 8 + (lane >> 3);
@@ -236,8 +247,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     advance_copy_stream();
   }
 
-  const int frag_row = lane & 31;
-  const int kgrp = lane >> 5;
+  // The lane's row and K group within a fragment, which every LDS read of the K loop is addressed with.  Set again
+  // from the lane number after each epilogue rather than kept across it: what lives across the epilogue's register
+  // demand gets spilled (see lane_now).
+  int frag_row = lane & 31;
+  int kgrp = lane >> 5;
   // fragment f (0..3: A row tile f, 4..7: B column tile f-4) of K step s of the K tile in `stage`
   // (BPACK: f = 0..7, A row tile f of the whole tile)
   auto load_frag = [&](int stage, int s, int f) __attribute__((always_inline)) -> bf16x8_t {
@@ -250,92 +264,126 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     }
   };
 
-  // ---- epilogue of one output tile: accumulators -> bands of 8 rows x 64 columns through the wavefront's own
-  // staging rows -> 16 bytes of consecutive columns per lane (bias added, converted) -> global.
-  // acc[i][j][r] is C[row, col] with row = i*32 + (r/4)*8 + kgrp*4 + r%4, col = j*32 + lane%32: lanes 0-31 hold
-  // rows q*8+0..3 and lanes 32-63 rows q*8+4..7 of each band.  Each half-wave writes its 4 rows and reads the
-  // same 4 rows back, so no lane depends on LDS writes of the other half-wave or of another wavefront: no
-  // barrier and no wait for write completion is needed (the LDS executes one half-wave's accesses in order).
-  const bool vec_ok = ((p.N & 3) == 0) && ((((uintptr_t)p.C) & 15u) == 0);
+  // ---- epilogue of one output tile.  The MFMAs take the B fragment as their first operand, so the accumulators hold
+  // the tile transposed: acc[i][j][q*4 + rr] is C[row, col] with row = i*32 + lane%32 and
+  // col = j*32 + q*8 + (lane/32)*4 + rr, i.e. a lane holds runs of four consecutive columns of one row.  Bias is added
+  // and the value converted in registers; the runs then pass through the wavefront's own staging rows (32 rows of 128
+  // bytes: 64 columns of a 16-bit output, 32 of an fp32 one), from which every lane takes 16 consecutive bytes, so that
+  // a store instruction writes 8 rows of 128 contiguous bytes.  Only lanes of one wavefront exchange data (its LDS
+  // accesses execute in order, and the writes are waited for before the reads are issued): no barrier.
   auto epilogue = [&](int ord) __attribute__((always_inline)) {
     int m0, n0, ks;
     tile_origin(ord, m0, n0, ks);
     // partial tiles of K range ks go to slice ks of C (fp32, no bias: the caller's reduction adds it)
     unsigned char* const Cs = (unsigned char*)p.C + (size_t)ks * (size_t)p.M * (size_t)p.N * sizeof(float);
-    int lane = lane_id;
-    asm volatile("" : "+v"(lane));  // keeps the lane-derived terms below out of the K loop's live registers
-    const int frag_row = lane & 31, kgrp = lane >> 5;
-    float* stg = (float*)(lds + S * kStageBytes + wave * kStgWave) + kgrp * (4 * kStgStride);
-    const int c4 = (lane & 15) * 4;          // columns within the 64-column band
-    const int rl0 = (lane & 31) >> 4;        // this lane reads rows rl0 and rl0 + 2 of its half-wave's 4
-    constexpr int NJH = NJ / 2;  // 64-column bands across the wavefront's columns
-    float bv[NJH][4];
+    const int lane = lane_now();
+    const int r32 = lane & 31, kgrp = lane >> 5;
+    const int rrow = lane >> 3, chunk = lane & 7;  // read side: row rrow + 8 * pass, 16-byte piece `chunk` of it
+    unsigned char* const stg = lds + S * kStageBytes + wave * kStgWave;
+    unsigned char* const stg_w = stg + r32 * kStgRow;
+    const unsigned char* const stg_r = stg + rrow * kStgRow + chunk * 16;
+    constexpr int kEsz = (OUT_DT == MASE_DT_F32) ? 4 : 2;
+    constexpr int kVec = 16 / kEsz;  // elements per 16-byte piece
+    const bool vec_ok = ((p.N & (kVec - 1)) == 0) && ((((uintptr_t)p.C) & 15u) == 0);
+    // the wavefront's whole part of the tile lies inside C and takes 16-byte stores (wavefront-uniform)
+    const bool interior = vec_ok && m0 + row_base + NI * 32 <= p.M && n0 + col_base + NJ * 32 <= p.N;
+    const size_t row_step = (size_t)p.N * kEsz;  // bytes from one output row to the next
+    // where this lane's piece of row 0 of the wavefront's first band goes
+    unsigned char* const lane_c = Cs + ((size_t)(m0 + row_base + rrow) * p.N + (size_t)(n0 + col_base + chunk * kVec)) * kEsz;
+    float bv[NJ][4][4];  // bias of the lane's columns
 #pragma unroll
-    for (int jh = 0; jh < NJH; ++jh)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) bv[jh][e] = 0.0f;
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) bv[j][q][rr] = 0.0f;
     if (p.bias != nullptr) {
+      auto fill = [&](auto dtc) __attribute__((always_inline)) {  // the dtype is decided once, not per element
 #pragma unroll
-      for (int jh = 0; jh < NJH; ++jh)
+        for (int j = 0; j < NJ; ++j)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int col = n0 + col_base + jh * 64 + c4 + e;
-          if (col < p.N) bv[jh][e] = load_bias(p.bias, p.bias_dtype, col);
-        }
+          for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+              const int col = n0 + col_base + j * 32 + q * 8 + kgrp * 4 + rr;
+              if (col < p.N) bv[j][q][rr] = load_bias(p.bias, decltype(dtc)::value, col);
+            }
+      };
+      if (p.bias_dtype == MASE_DT_F32) fill(std::integral_constant<int, MASE_DT_F32>{});
+      else if (p.bias_dtype == MASE_DT_BF16) fill(std::integral_constant<int, MASE_DT_BF16>{});
+      else fill(std::integral_constant<int, MASE_DT_F16>{});
       // The bias loads are the only vector-memory loads the compiler itself tracks in this kernel.  Completing
       // them here, with a wait it can see, keeps it from guarding their registers with s_waitcnt vmcnt(0)
       // inside the K loop, where that would also wait for every async copy in flight.
       wait_vmcnt<0>();
     }
+    // one band: kBandTiles MFMA tiles of row tile i side by side = 128 bytes of output per row
+    constexpr int kBandTiles = (OUT_DT == MASE_DT_F32) ? 1 : 2;
+    constexpr int kBandsPerRowTile = NJ / kBandTiles;
+    constexpr int kBands = NI * kBandsPerRowTile;
+    auto stage_band = [&](int b) __attribute__((always_inline)) {
+      const int i = b / kBandsPerRowTile, jb = b % kBandsPerRowTile;
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
+      for (int jj = 0; jj < kBandTiles; ++jj) {
+        const int j = jb * kBandTiles + jj;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
+        for (int q = 0; q < 4; ++q) {
+          const float v[4] = {acc[i][j][q * 4 + 0] + bv[j][q][0], acc[i][j][q * 4 + 1] + bv[j][q][1],
+                              acc[i][j][q * 4 + 2] + bv[j][q][2], acc[i][j][q * 4 + 3] + bv[j][q][3]};
+          unsigned char* const dst = stg_w + (jj * 32 + q * 8 + kgrp * 4) * kEsz;
+          if constexpr (OUT_DT == MASE_DT_F32) {
+            *(uint4*)dst = make_uint4(f2bits(v[0]), f2bits(v[1]), f2bits(v[2]), f2bits(v[3]));
+          } else if constexpr (OUT_DT == MASE_DT_BF16) {
+            *(uint2*)dst = make_uint2(f32x2_to_bf16x2_bits(v[0], v[1]), f32x2_to_bf16x2_bits(v[2], v[3]));
+          } else {
+            *(uint2*)dst = make_uint2(f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16),
+                                      f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16));
+          }
+        }
+      }
+    };
+    // (Staging band b + 1 between the issue of band b's reads and their use was measured: no gain, more registers.)
 #pragma unroll
-        for (int jh = 0; jh < NJH; ++jh) {
+    for (int b = 0; b < kBands; ++b) {
+      const int i = b / kBandsPerRowTile, jb = b % kBandsPerRowTile;
+      stage_band(b);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the band is in LDS before any lane reads it
+      uint4 w[4];
 #pragma unroll
-          for (int jj = 0; jj < 2; ++jj)
+      for (int ps = 0; ps < 4; ++ps) w[ps] = *(const uint4*)(stg_r + ps * 8 * kStgRow);
+      // streaming stores: the output is not read again by this kernel and should not displace operand panels
+      unsigned char* const dst0 = lane_c + (size_t)(i * 32) * row_step + jb * 128;
+      if (__builtin_expect(interior, 1)) {
 #pragma unroll
-            for (int rr = 0; rr < 4; ++rr)
-              stg[rr * kStgStride + jj * 32 + frag_row] = acc[i][jh * 2 + jj][q * 4 + rr];
-          asm volatile("" ::: "memory");  // lanes exchange data through LDS: no value may be carried across
-          __builtin_amdgcn_sched_barrier(0);  // bands stay in program order: bounded register use
-          const int col0 = n0 + col_base + jh * 64 + c4;
+        for (int ps = 0; ps < 4; ++ps) store_nt((uint4*)(dst0 + (size_t)(ps * 8) * row_step), w[ps]);
+      } else {
+        const int col0 = n0 + col_base + jb * kBandTiles * 32 + chunk * kVec;
 #pragma unroll
-          for (int u = 0; u < 2; ++u) {
-            const int rl = rl0 + 2 * u;
-            const float4 v4 = *(const float4*)(stg + rl * kStgStride + c4);
-            const float v[4] = {v4.x + bv[jh][0], v4.y + bv[jh][1], v4.z + bv[jh][2], v4.w + bv[jh][3]};
-            const int row = m0 + row_base + i * 32 + q * 8 + kgrp * 4 + rl;
-            if (row >= p.M) continue;
-            const size_t o = (size_t)row * p.N + col0;
-            // streaming stores: the output is not read again by this kernel and should not displace operand panels
-            if (vec_ok && col0 + 3 < p.N) {
+        for (int ps = 0; ps < 4; ++ps) {
+          const int row = m0 + row_base + i * 32 + ps * 8 + rrow;
+          unsigned char* const dst = dst0 + (size_t)(ps * 8) * row_step;
+          if (row >= p.M) continue;
+          if (vec_ok && col0 + kVec - 1 < p.N) {
+            store_nt((uint4*)dst, w[ps]);
+          } else {
+            // element by element, the 16 bytes shifted down as they go (a rolled loop: this path is rare and is
+            // kept small so that the code between two K loops stays short)
+            uint32_t x0 = w[ps].x, x1 = w[ps].y, x2 = w[ps].z, x3 = w[ps].w;
+#pragma unroll 1
+            for (int e = 0; e < kVec && col0 + e < p.N; ++e) {
               if constexpr (OUT_DT == MASE_DT_F32) {
-                store_nt((uint4*)((float*)Cs + o), make_uint4(f2bits(v[0]), f2bits(v[1]), f2bits(v[2]), f2bits(v[3])));
-              } else if constexpr (OUT_DT == MASE_DT_BF16) {
-                uint2 w;
-                w.x = f32x2_to_bf16x2_bits(v[0], v[1]);
-                w.y = f32x2_to_bf16x2_bits(v[2], v[3]);
-                store_nt((uint2*)((uint16_t*)Cs + o), w);
+                ((uint32_t*)dst)[e] = x0;
+                x0 = x1, x1 = x2, x2 = x3;
               } else {
-                uint2 w;
-                w.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
-                w.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
-                store_nt((uint2*)((uint16_t*)Cs + o), w);
-              }
-            } else {
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                if (col0 + e >= p.N) continue;
-                if constexpr (OUT_DT == MASE_DT_F32) ((float*)Cs)[o + e] = v[e];
-                else if constexpr (OUT_DT == MASE_DT_BF16) ((uint16_t*)Cs)[o + e] = (uint16_t)f32_to_bf16_bits(v[e]);
-                else ((uint16_t*)Cs)[o + e] = (uint16_t)f32_to_f16_bits(v[e]);
+                ((uint16_t*)dst)[e] = (uint16_t)x0;
+                x0 = (x0 >> 16) | (x1 << 16), x1 = (x1 >> 16) | (x2 << 16), x2 = (x2 >> 16) | (x3 << 16), x3 >>= 16;
               }
             }
           }
         }
       }
+      asm volatile("" ::: "memory");      // lanes exchange data through LDS: no value may be carried across
+      __builtin_amdgcn_sched_barrier(0);  // bands stay in program order: bounded register use
     }
   };
 
@@ -377,8 +425,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   auto set_b_tile = [&](int ord) __attribute__((always_inline)) {
     int m0, n0, ks;
     tile_origin(ord, m0, n0, ks);
-    int lane = lane_id;
-    asm volatile("" : "+v"(lane));
+    const int lane = lane_now();
     const int nt_last = (p.N + 31) / 32 - 1;
     constexpr uint32_t kFragBytes = BCODES ? 512u : 1024u;  // one fragment of a wavefront: 8 codes or 8 bf16 per lane
 #pragma unroll
@@ -473,7 +520,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
       else wait_vmcnt<8>();
 #pragma unroll
       for (int t = 0; t < 16; ++t) {
-        acc[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[s][t >> 1], fb[NB][s][t & 1],
+        acc[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[NB][s][t & 1], fr[s][t >> 1],
                                                                      acc[t >> 1][t & 1], 0, 0, 0);
         if (s == 0) {
           if (t < 8) {
@@ -520,7 +567,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
 #pragma unroll
       for (int t = 0; t < 16; ++t) {
         acc[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            fr[s][t >> 1], __builtin_bit_cast(bf16x8_t, fbq[s & 1][t & 1]), acc[t >> 1][t & 1], 0, 0, 0);
+            __builtin_bit_cast(bf16x8_t, fbq[s & 1][t & 1]), fr[s][t >> 1], acc[t >> 1][t & 1], 0, 0, 0);
         // slots 0, 1 of the steps after which the block of 32 changes: the scales the next step's codes take; slots
         // 2, 4, .., 14, 15: quarter u = 0..7 (column tile u / 4, register u % 4) of the next step's fragments
         if ((s & 1) && t < 2) set_scale(s == 1 ? NB : NB ^ 1, s == 1 ? 1 : 0, t);
@@ -559,7 +606,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     for (int s = 0; s < kSteps; ++s) {
 #pragma unroll
       for (int t = 0; t < 16; ++t) {
-        acc[t >> 2][t & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[s][t >> 2], fr[s][4 + (t & 3)],
+        acc[t >> 2][t & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[s][4 + (t & 3)], fr[s][t >> 2],
                                                                      acc[t >> 2][t & 3], 0, 0, 0);
         if (s == 0) {
           if (t < 8) fr[1][t] = load_frag(stage, 1, t);
@@ -620,6 +667,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     }
     epilogue(ord);
     zero_acc();
+    {
+      const int l = lane_now();
+      frag_row = l & 31;
+      kgrp = l >> 5;
+    }
   }
   wait_vmcnt<0>();  // no copy may still be in flight towards LDS when the work-group retires
 }
