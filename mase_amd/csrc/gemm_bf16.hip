@@ -95,6 +95,14 @@ __device__ __forceinline__ int lane_now() {
   return lane;
 }
 
+// An accumulator value moved to an ordinary register at the place of the call.  Left to itself the compiler copies all
+// 256 accumulators out of their registers at once when it reaches the epilogue, and spills what that displaces.
+__device__ __forceinline__ float acc_read(float a) {
+  float v;
+  asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+  return v;
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   // gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14 ; leave the others at max
@@ -328,8 +336,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
         const int j = jb * kBandTiles + jj;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const float v[4] = {acc[i][j][q * 4 + 0] + bv[j][q][0], acc[i][j][q * 4 + 1] + bv[j][q][1],
-                              acc[i][j][q * 4 + 2] + bv[j][q][2], acc[i][j][q * 4 + 3] + bv[j][q][3]};
+          const float v[4] = {acc_read(acc[i][j][q * 4 + 0]) + bv[j][q][0], acc_read(acc[i][j][q * 4 + 1]) + bv[j][q][1],
+                              acc_read(acc[i][j][q * 4 + 2]) + bv[j][q][2], acc_read(acc[i][j][q * 4 + 3]) + bv[j][q][3]};
           unsigned char* const dst = stg_w + (jj * 32 + q * 8 + kgrp * 4) * kEsz;
           if constexpr (OUT_DT == MASE_DT_F32) {
             *(uint4*)dst = make_uint4(f2bits(v[0]), f2bits(v[1]), f2bits(v[2]), f2bits(v[3]));

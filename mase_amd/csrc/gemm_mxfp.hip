@@ -22,6 +22,8 @@
 // half-waves (the byte select of the instruction is an immediate).
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace mase {
 namespace {
 
@@ -62,6 +64,14 @@ __device__ __forceinline__ void wait_vmcnt_n() {
   __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8) | ((N >> 4) << 14));
 }
 
+// An accumulator value moved to an ordinary register at the place of the call.  Left to itself the compiler copies all
+// 256 accumulators out of their registers at once when it reaches the epilogue, and spills what that displaces.
+__device__ __forceinline__ float acc_read(float a) {
+  float v;
+  asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+  return v;
+}
+
 __device__ __forceinline__ float load_bias_v(const void* bias, int dt, int col) {
   if (dt == MASE_DT_F32) return ((const float*)bias)[col];
   if (dt == MASE_DT_BF16) return bits2f((uint32_t)((const uint16_t*)bias)[col] << 16);
@@ -84,11 +94,10 @@ struct MxGemmGeom {
   static constexpr int kStage = kTileA + kTileB + 2 * 1024;  // + one scale dword per row for A and for B
   static constexpr int S = (kStage <= 53 * 1024) ? 3 : 2;
   // epilogue staging, separate from the stages (copies of the next tile are in flight during the epilogue):
-  // per wavefront two buffers of 8 rows x 32 columns of fp32 (4 rows per half-wave).  Row stride 32 floats is
-  // conflict-free both for the half-wave row writes and for the 16-lane phases of the 16-byte reads.
-  static constexpr int kStgStride = 32;
-  static constexpr int kStgBuf = 8 * kStgStride;       // floats per buffer
-  static constexpr int kStgWave = 2 * kStgBuf * 4;     // bytes per wavefront
+  // per wavefront 16 rows of 128 bytes, row stride 144 bytes (16-byte accesses of 16 consecutive rows at one column
+  // offset then fall on 64 different banks); three stages of the 4-bit form leave room for no more
+  static constexpr int kStgRow = 144;
+  static constexpr int kStgWave = 16 * kStgRow;        // bytes per wavefront
   static constexpr int kLdsBytes = S * kStage + 4 * kStgWave;
 };
 
@@ -274,90 +283,163 @@ __global__ __launch_bounds__(kThreadsG) void gemm_mxfp_kernel(MxGemmParams p) {
     } else {
       b[4] = 0; b[5] = 0; b[6] = 0; b[7] = 0;
     }
+    // B's fragment goes in as the first operand (formats and scales swapped with it): the accumulators then hold the
+    // tile transposed, which is the layout the epilogue wants
     if (s == 0)
-      acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], CBSZ, BLGP, 0, sa[i], 0, sb[j]);
+      acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b, a, acc[i][j], BLGP, CBSZ, 0, sb[j], 0, sa[i]);
     else
-      acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], CBSZ, BLGP, 2, sa[i], 2, sb[j]);
+      acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b, a, acc[i][j], BLGP, CBSZ, 2, sb[j], 2, sa[i]);
   };
 
-  // ---- epilogue of one output tile: accumulators -> bands of 8 rows x 32 columns through the wavefront's own
-  // staging rows -> 16 bytes of consecutive columns per lane (bias added, converted) -> global.
-  // In the accumulator layout lanes 0-31 hold rows q*8+0..3 and lanes 32-63 rows q*8+4..7 of each 32-row MFMA
-  // tile (one column per lane); each half-wave writes its 4 rows and reads the same 4 rows back, so no lane
-  // depends on LDS writes of the other half-wave or of another wavefront: no barrier and no wait for write
-  // completion is needed (the LDS executes one half-wave's accesses in order).  Two staging buffers alternate:
-  // the writes of band b+1 are issued while the read of band b is still in flight.
-  const bool vec_ok = ((p.N & 3) == 0) && ((((uintptr_t)p.C) & 15u) == 0);
+  // ---- epilogue of one output tile (the scheme of gemm_bf16.hip).  acc[i][j][q*4 + rr] is C[row, col] with
+  // row = i*32 + lane%32 and col = j*32 + q*8 + (lane/32)*4 + rr: a lane holds runs of four consecutive columns of one
+  // row.  The runs pass through the wavefront's own staging rows, 16 rows of 128 bytes at a time (the lanes of rows
+  // 0-15 of the MFMA tile, then those of rows 16-31), from which every lane takes 16 consecutive bytes.  Only lanes of
+  // one wavefront exchange data (its LDS accesses execute in order, and the writes are waited for before the reads are
+  // issued): no barrier.
+  //   without bias: the values are converted to the output type before staging, so a row of the staging area is 64
+  //     columns of a 16-bit output and a store instruction writes 8 rows of 128 contiguous bytes.  (No "+ 0" stands in
+  //     for the bias: an accumulator that started at +0 never holds -0, so there is nothing for it to normalise.)
+  //   with bias: staged as fp32, 32 columns per row; bias added and the value converted after the read-back, where a
+  //     lane's columns are the same for every band (16 bias registers instead of 64).
   auto epilogue = [&](int ord) __attribute__((always_inline)) {
     int m0, n0;
     tile_origin(ord, m0, n0);
     int lane = lane_id;
     asm volatile("" : "+v"(lane));  // keeps the lane-derived terms below out of the K loop's live registers
-    const int frag_row = lane & 31, kgrp = lane >> 5;
-    float* stg = (float*)(lds + S * kStage + wave * G::kStgWave) + kgrp * (4 * G::kStgStride);
-    const int c4 = (lane & 7) * 4;           // columns within the 32-column band
-    const int rl = (lane & 31) >> 3;         // the row of its half-wave's 4 that this lane reads back
-    float bv[4][4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) bv[j][e] = 0.0f;
-    if (p.bias != nullptr) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int col = n0 + wn * 128 + j * 32 + c4 + e;
-          if (col < p.N) bv[j][e] = load_bias_v(p.bias, p.bias_dtype, col);
+    const int r32 = lane & 31, kgrp = lane >> 5;
+    const int rrow = lane >> 3, chunk = lane & 7;  // read side: row rrow + 8 * pass, 16-byte piece `chunk` of it
+    unsigned char* const stg = lds + S * kStage + wave * G::kStgWave;
+    unsigned char* const stg_w = stg + (r32 & 15) * G::kStgRow;
+    const unsigned char* const stg_r = stg + rrow * G::kStgRow + chunk * 16;
+    constexpr int kEsz = (OUT_DT == MASE_DT_F32) ? 4 : 2;
+    const size_t row_step = (size_t)p.N * kEsz;  // bytes from one output row to the next
+    unsigned char* const wave_c = (unsigned char*)p.C + ((size_t)(m0 + wm * 128) * p.N + (size_t)(n0 + wn * 128)) * kEsz;
+    // `n` consecutive elements (16 or 8 bytes in x0..x3) to row `row`, columns col0.. of C, in one store where that is
+    // possible, else element by element, the bytes shifted down as they go (a rolled loop: rare, and kept small so that
+    // the code between two K loops stays short)
+    auto store_piece = [&](auto nc, int row, int col0, uint32_t x0, uint32_t x1, uint32_t x2, uint32_t x3)
+                           __attribute__((always_inline)) {
+      constexpr int n = decltype(nc)::value;
+      if (row >= p.M) return;
+      unsigned char* const dst = (unsigned char*)p.C + ((size_t)row * p.N + (size_t)col0) * kEsz;
+      if ((p.N & (n - 1)) == 0 && ((((uintptr_t)p.C) & 15u) == 0) && col0 + n - 1 < p.N) {
+        if constexpr (n * kEsz == 16) store_nt((uint4*)dst, make_uint4(x0, x1, x2, x3));
+        else store_nt((uint2*)dst, make_uint2(x0, x1));
+      } else {
+#pragma unroll 1
+        for (int e = 0; e < n && col0 + e < p.N; ++e) {
+          if constexpr (OUT_DT == MASE_DT_F32) {
+            ((uint32_t*)dst)[e] = x0;
+            x0 = x1, x1 = x2, x2 = x3;
+          } else {
+            ((uint16_t*)dst)[e] = (uint16_t)x0;
+            x0 = (x0 >> 16) | (x1 << 16), x1 = (x1 >> 16) | (x2 << 16), x2 = (x2 >> 16) | (x3 << 16), x3 >>= 16;
+          }
         }
+      }
+    };
+    if (p.bias == nullptr) {
+      constexpr int kVec = 16 / kEsz;  // elements per 16-byte piece
+      // the wavefront's whole part of the tile lies inside C and takes 16-byte stores (wavefront-uniform)
+      const bool interior = ((p.N & (kVec - 1)) == 0) && ((((uintptr_t)p.C) & 15u) == 0) &&
+                            m0 + wm * 128 + 128 <= p.M && n0 + wn * 128 + 128 <= p.N;
+      unsigned char* const lane_c = wave_c + (size_t)rrow * row_step + chunk * 16;
+      // one band: kBandTiles MFMA tiles of row tile i side by side = 128 bytes of output per row, 16 rows at a time
+      constexpr int kBandTiles = (OUT_DT == MASE_DT_F32) ? 1 : 2;
+      constexpr int kBandsPerRowTile = 4 / kBandTiles;
+#pragma unroll
+      for (int b = 0; b < 4 * kBandsPerRowTile * 2; ++b) {
+        const int i = b / (kBandsPerRowTile * 2), jb = (b >> 1) % kBandsPerRowTile, half = b & 1;
+        if ((r32 >> 4) == half) {
+#pragma unroll
+          for (int jj = 0; jj < kBandTiles; ++jj) {
+            const int j = jb * kBandTiles + jj;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const float v[4] = {acc_read(acc[i][j][q * 4 + 0]), acc_read(acc[i][j][q * 4 + 1]),
+                                  acc_read(acc[i][j][q * 4 + 2]), acc_read(acc[i][j][q * 4 + 3])};
+              unsigned char* const dst = stg_w + (jj * 32 + q * 8 + kgrp * 4) * kEsz;
+              if constexpr (OUT_DT == MASE_DT_F32) {
+                *(uint4*)dst = make_uint4(f2bits(v[0]), f2bits(v[1]), f2bits(v[2]), f2bits(v[3]));
+              } else if constexpr (OUT_DT == MASE_DT_BF16) {
+                *(uint2*)dst = make_uint2(f32x2_to_bf16x2_bits(v[0], v[1]), f32x2_to_bf16x2_bits(v[2], v[3]));
+              } else {
+                *(uint2*)dst = make_uint2(f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16),
+                                          f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16));
+              }
+            }
+          }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the band is in LDS before any lane reads it
+        uint4 w[2];
+#pragma unroll
+        for (int ps = 0; ps < 2; ++ps) w[ps] = *(const uint4*)(stg_r + ps * 8 * G::kStgRow);
+        // streaming stores: the output is not read again by this kernel and should not displace operand panels
+        if (__builtin_expect(interior, 1)) {
+          unsigned char* const dst0 = lane_c + (size_t)(i * 32 + half * 16) * row_step + jb * 128;
+#pragma unroll
+          for (int ps = 0; ps < 2; ++ps) store_nt((uint4*)(dst0 + (size_t)(ps * 8) * row_step), w[ps]);
+        } else {
+#pragma unroll
+          for (int ps = 0; ps < 2; ++ps)
+            store_piece(std::integral_constant<int, kVec>{}, m0 + wm * 128 + i * 32 + half * 16 + ps * 8 + rrow,
+                        n0 + wn * 128 + jb * kBandTiles * 32 + chunk * kVec, w[ps].x, w[ps].y, w[ps].z, w[ps].w);
+        }
+        asm volatile("" ::: "memory");      // lanes exchange data through LDS: no value may be carried across
+        __builtin_amdgcn_sched_barrier(0);  // bands stay in program order: bounded register use
+      }
+    } else {
+      float bv[4][4];  // bias of the four columns this lane reads back, per column tile
+      auto fill = [&](auto dtc) __attribute__((always_inline)) {  // the dtype is decided once, not per element
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int col = n0 + wn * 128 + j * 32 + chunk * 4 + e;
+            bv[j][e] = col < p.N ? load_bias_v(p.bias, decltype(dtc)::value, col) : 0.0f;
+          }
+      };
+      if (p.bias_dtype == MASE_DT_F32) fill(std::integral_constant<int, MASE_DT_F32>{});
+      else if (p.bias_dtype == MASE_DT_BF16) fill(std::integral_constant<int, MASE_DT_BF16>{});
+      else fill(std::integral_constant<int, MASE_DT_F16>{});
       // The bias loads are the only vector-memory loads the compiler itself tracks in this kernel.  Completing
       // them here, with a wait it can see, keeps it from guarding their registers with s_waitcnt vmcnt(0)
       // inside the K loop, where that would also wait for every async copy in flight.
       wait_vmcnt_n<0>();
-    }
-    auto write_band = [&](int band) __attribute__((always_inline)) {  // band = (i*4 + q)*4 + j
-      const int i = band >> 4, q = (band >> 2) & 3, j = band & 3;
-      float* b = stg + (band & 1) * G::kStgBuf;
 #pragma unroll
-      for (int rr = 0; rr < 4; ++rr) b[rr * G::kStgStride + frag_row] = acc[i][j][q * 4 + rr];
-    };
-    write_band(0);
+      for (int b = 0; b < 32; ++b) {  // band: MFMA tile (i, j), 16 rows at a time
+        const int i = b >> 3, j = (b >> 1) & 3, half = b & 1;
+        if ((r32 >> 4) == half) {
 #pragma unroll
-    for (int band = 0; band < 64; ++band) {
-      const int i = band >> 4, q = (band >> 2) & 3, j = band & 3;
-      asm volatile("" ::: "memory");  // lanes exchange data through LDS: no value may be carried across
-      const float4 v4 = *(const float4*)(stg + (band & 1) * G::kStgBuf + rl * G::kStgStride + c4);
-      if (band + 1 < 64) write_band(band + 1);
-      const float v[4] = {v4.x + bv[j][0], v4.y + bv[j][1], v4.z + bv[j][2], v4.w + bv[j][3]};
-      const int row = m0 + wm * 128 + i * 32 + q * 8 + kgrp * 4 + rl;
-      const int col0 = n0 + wn * 128 + j * 32 + c4;
-      if (row < p.M) {
-        const size_t o = (size_t)row * p.N + col0;
-        if (vec_ok && col0 + 3 < p.N) {
+          for (int q = 0; q < 4; ++q)
+            *(uint4*)(stg_w + (q * 8 + kgrp * 4) * 4) =
+                make_uint4(f2bits(acc_read(acc[i][j][q * 4 + 0])), f2bits(acc_read(acc[i][j][q * 4 + 1])),
+                           f2bits(acc_read(acc[i][j][q * 4 + 2])), f2bits(acc_read(acc[i][j][q * 4 + 3])));
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the band is in LDS before any lane reads it
+        uint4 w[2];
+#pragma unroll
+        for (int ps = 0; ps < 2; ++ps) w[ps] = *(const uint4*)(stg_r + ps * 8 * G::kStgRow);
+#pragma unroll
+        for (int ps = 0; ps < 2; ++ps) {
+          const float v[4] = {bits2f(w[ps].x) + bv[j][0], bits2f(w[ps].y) + bv[j][1], bits2f(w[ps].z) + bv[j][2],
+                              bits2f(w[ps].w) + bv[j][3]};
+          const int row = m0 + wm * 128 + i * 32 + half * 16 + ps * 8 + rrow;
+          const int col0 = n0 + wn * 128 + j * 32 + chunk * 4;
           if constexpr (OUT_DT == MASE_DT_F32) {
-            store_nt((uint4*)((float*)p.C + o), make_uint4(f2bits(v[0]), f2bits(v[1]), f2bits(v[2]), f2bits(v[3])));
+            store_piece(std::integral_constant<int, 4>{}, row, col0, f2bits(v[0]), f2bits(v[1]), f2bits(v[2]), f2bits(v[3]));
           } else if constexpr (OUT_DT == MASE_DT_BF16) {
-            uint2 w;
-            w.x = f32x2_to_bf16x2_bits(v[0], v[1]);
-            w.y = f32x2_to_bf16x2_bits(v[2], v[3]);
-            store_nt((uint2*)((uint16_t*)p.C + o), w);
+            store_piece(std::integral_constant<int, 4>{}, row, col0, f32x2_to_bf16x2_bits(v[0], v[1]),
+                        f32x2_to_bf16x2_bits(v[2], v[3]), 0u, 0u);
           } else {
-            uint2 w;
-            w.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
-            w.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
-            store_nt((uint2*)((uint16_t*)p.C + o), w);
-          }
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            if (col0 + e >= p.N) continue;
-            if constexpr (OUT_DT == MASE_DT_F32) ((float*)p.C)[o + e] = v[e];
-            else if constexpr (OUT_DT == MASE_DT_BF16) ((uint16_t*)p.C)[o + e] = (uint16_t)f32_to_bf16_bits(v[e]);
-            else ((uint16_t*)p.C)[o + e] = (uint16_t)f32_to_f16_bits(v[e]);
+            store_piece(std::integral_constant<int, 4>{}, row, col0, f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16),
+                        f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16), 0u, 0u);
           }
         }
+        asm volatile("" ::: "memory");      // lanes exchange data through LDS: no value may be carried across
+        __builtin_amdgcn_sched_barrier(0);  // bands stay in program order: bounded register use
       }
-      __builtin_amdgcn_sched_barrier(0);  // bands stay in program order: bounded register use
     }
   };
 
