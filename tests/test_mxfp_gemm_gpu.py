@@ -123,6 +123,15 @@ def test_gemm_mxfp_scaled_against_decoded_operands(dev, afmt, bfmt, M, N, K):
     want = ref + bias.double()
     d = (yb.cpu().double() - want).abs()
     assert bool((d <= want.abs() * 2.0 ** -8 + ref.abs().max() * 5e-4).all())  # bf16 rounding of the output
+    # the epilogue's forms agree bit for bit: a 16-bit output is the fp32 output rounded once, with or without a bias
+    # (which is added in fp32 before the rounding)
+    for dt in (torch.bfloat16, torch.float16):
+        assert torch.equal(gemm_mxfp_scaled(ac, asc, afmt, bc, bsc, bfmt, None, dt), y.to(dt)), dt
+    yf = gemm_mxfp_scaled(ac, asc, afmt, bc, bsc, bfmt, bias.to(dev), torch.float32)
+    assert torch.equal(yf, y + bias.to(dev))
+    assert torch.equal(yb, yf.to(torch.bfloat16))
+    assert torch.equal(gemm_mxfp_scaled(ac, asc, afmt, bc, bsc, bfmt, bias.to(dev).half(), torch.float16),
+                       (y + bias.to(dev).half().float()).half())
 
 
 def test_gemm_mxfp_exact_small_integers(dev):
