@@ -26,6 +26,7 @@
  *   mase_silu_mul_minifloat nn/quantized/modules/llama/mlp.py:60-62 (silu_minifloat(gate) * up)
  *   mase_rmsnorm_mxint, mase_silu_mul_mxint   the two above followed by the consumer LinearMXInt's activation
  *                           quantizer (nn/quantized/modules/linear.py:956-972) in the same pass
+ *   mase_add_rmsnorm_mxint  models/llama/modeling_llama.py:901-905 (residual addition, then the norm as above)
  *   mase_attn_softmax_mx    nn/quantized/modules/llama/attention.py:363-392 (scores -> quantized probabilities)
  *   mase_attention_causal   models/llama/modeling_llama.py:362-480 (the attention core on unquantized q, k, v)
  *   mase_mx_unpack          nn/quantizers/mxint/fake.py:59-80, nn/quantizers/mxfp/fake.py:75-104 (compose_*)
@@ -321,6 +322,14 @@ int mase_rmsnorm_mxint(const void* x, const void* weight, void* out, size_t rows
                        int element_bits, const uint32_t* log2_tab, void* stream);
 int mase_silu_mul_mxint(const void* gate, const void* up, void* out, size_t numel, int dtype, int element_bits,
                         const uint32_t* log2_tab, void* stream);
+
+/* The residual addition of a pre-norm block followed by mase_rmsnorm_mxint, in one pass: sum_out = x + residual (rounded
+ * to dtype, as the tensor addition rounds it) and out = mxint_quantizer(rmsnorm(sum_out)) as above
+ * (models/llama/modeling_llama.py:901-905: hidden = residual + hidden; residual = hidden;
+ * hidden = post_attention_layernorm(hidden)).  x, residual, sum_out, out: [rows, cols] contiguous; sum_out may be x or
+ * residual. */
+int mase_add_rmsnorm_mxint(const void* x, const void* residual, const void* weight, void* sum_out, void* out, size_t rows,
+                           size_t cols, int dtype, float eps, int element_bits, const uint32_t* log2_tab, void* stream);
 
 /* Causal self-attention core out = softmax(q k^T * scaling + causal mask) v for bf16 q, k, v [batch, heads, tokens, 128]
  * given by element strides of batch / head / token (last dimension contiguous, strides multiples of 8), out likewise;

@@ -55,6 +55,8 @@ SIGNATURES = {
     "mase_attention_causal_fused": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p] + [c_size_t] * 16 + [c_int, c_float, c_void_p, c_void_p,
                                             c_size_t, c_size_t, c_int, c_void_p, c_void_p]),
     "mase_rmsnorm_mxint": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_float, c_int, c_void_p, c_void_p]),
+    "mase_add_rmsnorm_mxint": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_float, c_int,
+                                      c_void_p, c_void_p]),
     "mase_silu_mul_mxint": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_void_p, c_void_p]),
     "mase_mxint_clip_search": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mase_mxfp_clip_search": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),

@@ -28,6 +28,8 @@ struct RmsNormParams {
   const void* x;
   const void* weight;
   void* out;
+  const void* residual;  // when set: the row normalised is x + residual, rounded to the dtype and also stored to sum_out
+  void* sum_out;
   size_t rows;
   int cols;  // multiple of 8, at most 8192
   float eps;
@@ -92,7 +94,8 @@ __device__ __forceinline__ void cast8(float* v, const CastSpec& c) {
 // wavefront, chunk c of wavefront w at element ((c * WPR + w) * 64 + lane) * 8).  Rows of more than 1536 elements are
 // spread over 4 wavefronts: 16 or 32 elements per lane instead of 64 keep the register count low enough for 8
 // wavefronts per SIMD, which is what hides the one load - compute - store round trip of each wavefront.  MX: the
-// output is the MXINT quantize-dequantize of the normalised row (cols a multiple of 32)
+// output is the MXINT quantize-dequantize of the normalised row (cols a multiple of 32).  The weight chunks are requested
+// together with the row's, so that their latency passes during the reduction instead of after it.
 template <int DT, int NCH, bool MX = false, int WPR = 1>
 __global__ __launch_bounds__(kRowThreads * WPR) void rmsnorm_kernel(RmsNormParams p) {
   using TR = DTypeTraits<DT>;
@@ -102,15 +105,23 @@ __global__ __launch_bounds__(kRowThreads * WPR) void rmsnorm_kernel(RmsNormParam
   const size_t base = row * (size_t)p.cols;
   WaveLog2 meta;
   if constexpr (MX) meta.init(p.mx.tab, 0);
-  float h[NCH][8];
+  float h[NCH][8], wv[NCH][8];
   float ss = 0.0f;
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
     const int e0 = ((c * WPR + wave) * 64 + lane) * 8;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) h[c][j] = 0.0f;
+    for (int j = 0; j < 8; ++j) h[c][j] = 0.0f, wv[c][j] = 0.0f;
     if (e0 < p.cols) {
       load_vec8<DT>(p.x, base + (size_t)e0, h[c]);
+      load_vec8<DT>(p.weight, (size_t)e0, wv[c]);
+      if (p.residual != nullptr) {
+        float res[8];
+        load_vec8<DT>(p.residual, base + (size_t)e0, res);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) h[c][j] = TR::round(h[c][j] + res[j]);
+        store_vec8<DT>(p.sum_out, base + (size_t)e0, h[c]);
+      }
       cast8<DT>(h[c], p.x_cast);
     }
 #pragma unroll
@@ -134,15 +145,10 @@ __global__ __launch_bounds__(kRowThreads * WPR) void rmsnorm_kernel(RmsNormParam
     if constexpr (!MX) {
       if (!live) continue;
     }
-    float w[8], y[8];
+    float y[8];
+    if (live) cast8<DT>(wv[c], p.w_cast);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) w[j] = 0.0f;
-    if (live) {
-      load_vec8<DT>(p.weight, (size_t)e0, w);
-      cast8<DT>(w, p.w_cast);
-    }
-#pragma unroll
-    for (int j = 0; j < 8; ++j) y[j] = w[j] * TR::round(h[c][j] * r);  // weight * hidden.to(dtype), rounded by the store
+    for (int j = 0; j < 8; ++j) y[j] = wv[c][j] * TR::round(h[c][j] * r);  // weight * hidden.to(dtype), rounded by the store
     if constexpr (MX) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) y[j] = TR::round(y[j]);
@@ -345,6 +351,34 @@ extern "C" int mase_rmsnorm_mxint(const void* x, const void* weight, void* out, 
   if (dtype < 0 || dtype > 2) return MASE_ERR_DTYPE;
   RmsNormParams p{};
   p.x = x;
+  p.weight = weight;
+  p.out = out;
+  p.rows = rows;
+  p.cols = (int)cols;
+  p.eps = eps;
+  if (!fill_mxint(p.mx, element_bits, dtype, log2_tab)) return MASE_ERR_PARAM;
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case MASE_DT_F32: return launch_rmsnorm<MASE_DT_F32, true>(p, st);
+    case MASE_DT_BF16: return launch_rmsnorm<MASE_DT_BF16, true>(p, st);
+    default: return launch_rmsnorm<MASE_DT_F16, true>(p, st);
+  }
+}
+
+extern "C" int mase_add_rmsnorm_mxint(const void* x, const void* residual, const void* weight, void* sum_out, void* out,
+                                      size_t rows, size_t cols, int dtype, float eps, int element_bits,
+                                      const uint32_t* log2_tab, void* stream) {
+  using namespace mase;
+  if (rows == 0 || cols == 0) return MASE_OK;
+  if (x == nullptr || residual == nullptr || weight == nullptr || sum_out == nullptr || out == nullptr || log2_tab == nullptr)
+    return MASE_ERR_NULL;
+  if (cols % 32 != 0 || cols > 8192 || rows > 0x7FFFFFFFull) return MASE_ERR_SHAPE;
+  if (!aligned16(x) || !aligned16(residual) || !aligned16(weight) || !aligned16(sum_out) || !aligned16(out)) return MASE_ERR_ALIGN;
+  if (dtype < 0 || dtype > 2) return MASE_ERR_DTYPE;
+  RmsNormParams p{};
+  p.x = x;
+  p.residual = residual;
+  p.sum_out = sum_out;
   p.weight = weight;
   p.out = out;
   p.rows = rows;

@@ -369,6 +369,24 @@ def rmsnorm_mxint(x: Tensor, weight: Tensor, eps: float, element_bits: int) -> T
     return out
 
 
+def add_rmsnorm_mxint(x: Tensor, residual: Tensor, weight: Tensor, eps: float, element_bits: int):
+    """``s = x + residual`` and ``rmsnorm_mxint(s, weight, eps, element_bits)`` in one pass (``mase_add_rmsnorm_mxint``);
+    returns ``(s, quantized norm)``.  Same shapes and dtype for ``x`` and ``residual``."""
+    _lib.require_device(x, "add_rmsnorm_mxint")
+    lib = _lib.load()
+    assert rmsnorm_supported(x, weight) and x.shape[-1] % 32 == 0
+    assert residual.shape == x.shape and residual.dtype == x.dtype and residual.device == x.device
+    xc, rc_ = _contig(x), _contig(residual)
+    w = weight.detach().contiguous()
+    s, out = torch.empty_like(xc), torch.empty_like(xc)
+    cols = xc.shape[-1]
+    rc = lib.mase_add_rmsnorm_mxint(xc.data_ptr(), rc_.data_ptr(), w.data_ptr(), s.data_ptr(), out.data_ptr(),
+                                    xc.numel() // cols, cols, _lib.dtype_code(xc), float(eps), int(element_bits),
+                                    log2_table(xc.dtype, xc.device).data_ptr(), _lib.stream_ptr(xc))
+    _lib.check(rc, "mase_add_rmsnorm_mxint")
+    return s, out
+
+
 def silu_mul_mxint(gate: Tensor, up: Tensor, element_bits: int) -> Tensor:
     """``mxint_quantizer(silu(gate) * up, block 32 along the last dimension, element_bits)`` in one pass
     (``mase_silu_mul_mxint``); the last dimension must be a multiple of 32."""

@@ -109,18 +109,24 @@ class DecoderLayer(nn.Module):
     # _norm_then_project); False: every Linear receives the plain tensor and quantizes it itself
     fuse_producers = True
 
-    def _norm_then_project(self, norm, x, modules):
-        """``[m(norm(x)) for m in modules]``.  Sibling projections of one tensor: quantized Linears that treat it alike
+    def _norm_then_project(self, norm, x, modules, addend=None):
+        """``x, [m(norm(x)) for m in modules]`` with ``x + addend`` for ``x`` when an addend is given (the residual
+        addition that precedes the norm).  Sibling projections of one tensor: quantized Linears that treat it alike
         share one quantized copy, and when they are MXINT Linears on the matrix-core path the norm writes that copy
         itself instead of a tensor each of them would read and quantize (same values: the quantizer's arithmetic on
-        the norm's rounded output)."""
+        the norm's rounded output); the addition then happens in the norm's pass as well."""
         if (self.fuse_producers and x.is_cuda and not torch.is_grad_enabled() and x.shape[-1] % 32 == 0
                 and _ops.rmsnorm_supported(x, norm.weight)):
             bits = shared_mxint_width(x, modules)
             if bits is not None:
-                hq = _ops.rmsnorm_mxint(x, norm.weight, norm.eps, bits)
-                return [m(hq, prepared=hq.reshape(-1, hq.shape[-1])) for m in modules]
-        return project_shared(norm(x), modules)
+                if addend is not None and addend.shape == x.shape and addend.dtype == x.dtype:
+                    x, hq = _ops.add_rmsnorm_mxint(x, addend, norm.weight, norm.eps, bits)
+                else:
+                    x = x if addend is None else x + addend
+                    hq = _ops.rmsnorm_mxint(x, norm.weight, norm.eps, bits)
+                return x, [m(hq, prepared=hq.reshape(-1, hq.shape[-1])) for m in modules]
+        x = x if addend is None else x + addend
+        return x, project_shared(norm(x), modules)
 
     def _rope_tables(self, T, device, dtype):
         """the cos / sin tables of the rotary embedding depend on (sequence length, device, dtype) only: kept from one
@@ -134,7 +140,7 @@ class DecoderLayer(nn.Module):
         cfg = self.cfg
         B, T, _ = x.shape
         q, k, v = (t.view(B, T, cfg.num_heads, cfg.head_dim).transpose(1, 2)
-                   for t in self._norm_then_project(self.input_layernorm, x, (self.q_proj, self.k_proj, self.v_proj)))
+                   for t in self._norm_then_project(self.input_layernorm, x, (self.q_proj, self.k_proj, self.v_proj))[1])
         cos, sin = self._rope_tables(T, x.device, x.dtype)
         own_kernel = (self.fuse_producers and self.attention_fn is causal_attention and q.is_cuda
                       and not torch.is_grad_enabled() and _ops.attention_causal_supported(q, k, v))
@@ -154,8 +160,8 @@ class DecoderLayer(nn.Module):
         else:
             a = self.attention_fn(q, k, v)
         a = a.transpose(1, 2).reshape(B, T, cfg.num_heads * cfg.head_dim)
-        x = x + (self.o_proj(a, prepared=a.reshape(-1, a.shape[-1])) if bits is not None else self.o_proj(a))
-        gate, up = self._norm_then_project(self.post_attention_layernorm, x, (self.gate_proj, self.up_proj))
+        o = self.o_proj(a, prepared=a.reshape(-1, a.shape[-1])) if bits is not None else self.o_proj(a)
+        x, (gate, up) = self._norm_then_project(self.post_attention_layernorm, x, (self.gate_proj, self.up_proj), addend=o)
         if gate.is_cuda and _ops.silu_mul_supported(gate, up):
             bits = shared_mxint_width(gate, (self.down_proj,)) if self.fuse_producers and gate.shape[-1] % 32 == 0 else None
             if bits is not None and not torch.is_grad_enabled():

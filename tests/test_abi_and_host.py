@@ -358,6 +358,14 @@ def test_layer_op_entry_points_reject_bad_arguments_without_a_gpu(lib):
     assert r(p, p, p, 4, 64, 4, 1e-6, 0, 0, 1, 0, 0, 0, 1, 0, None) == -4
     assert r(p, p, p, 4, 64, 1, 1e-6, 9, 3, 1, 0, 0, 0, 1, 0, None) == -5      # cast format
     assert r(p, p, p, 4, 64, 1, 1e-6, 4, 3, 1, 0, 4, 3, 1, 7, None) == -5      # rounding mode
+    # mase_add_rmsnorm_mxint(x, residual, weight, sum_out, out, rows, cols, dtype, eps, element_bits, log2_tab, stream)
+    ar = lib.mase_add_rmsnorm_mxint
+    assert ar(p, p, p, p, p, 0, 64, 1, 1e-6, 8, p, None) == 0
+    assert ar(p, None, p, p, p, 4, 64, 1, 1e-6, 8, p, None) == -1    # no residual
+    assert ar(p, p, p, None, p, 4, 64, 1, 1e-6, 8, p, None) == -1    # nowhere to put the sum
+    assert ar(p, p, p, p, p, 4, 48, 1, 1e-6, 8, p, None) == -2       # whole blocks of 32
+    assert ar(p, p, p, p, p, 4, 64, 3, 1e-6, 8, p, None) == -4
+    assert ar(p, p, p, p, p, 4, 64, 1, 1e-6, 1, p, None) == -5       # element width
     # mase_rope(x, cos, sin, out, B, H, T, D, xs_b, xs_h, xs_t, cs_b, cs_t, dtype, stream)
     ro = lib.mase_rope
     assert ro(p, p, p, p, 0, 2, 4, 64, 512, 64, 128, 0, 64, 1, None) == 0

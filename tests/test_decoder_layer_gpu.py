@@ -110,7 +110,7 @@ def test_decoder_layer_mxint_matches_cpu_reference(dev, shape, widths):
 
 def test_decoder_layer_producers_write_the_quantized_form(dev, monkeypatch):
     """RMSNorm and the SwiGLU product hand the MXINT Linears their quantized activations directly
-    (rmsnorm_mxint / silu_mul_mxint): the layer's output is bit for bit that of the layer whose Linears quantize the
+    (rmsnorm_mxint / add_rmsnorm_mxint / silu_mul_mxint): the layer's output is bit for bit that of the layer whose Linears quantize the
     stored tensors themselves, and the separate quantizer runs only for o_proj"""
     from mase_amd.quantizers import _ops
     from mase_amd.workloads import DecoderLayerConfig, decoder_layer
@@ -118,17 +118,19 @@ def test_decoder_layer_producers_write_the_quantized_form(dev, monkeypatch):
     cfg = DecoderLayerConfig(hidden_size=1024, num_heads=8, head_dim=128, intermediate_size=2752)
     _, gpu = build_pair(dev, cfg, 41)
     x = torch.randn(2, 300, cfg.hidden_size, generator=torch.Generator().manual_seed(5)).bfloat16().to(dev)
-    calls = {"qdq": 0, "norm": 0, "silu": 0}
-    real = {"qdq": _ops.mxint_qdq, "norm": _ops.rmsnorm_mxint, "silu": _ops.silu_mul_mxint}
+    calls = {"qdq": 0, "norm": 0, "addnorm": 0, "silu": 0}
+    real = {"qdq": _ops.mxint_qdq, "norm": _ops.rmsnorm_mxint, "addnorm": _ops.add_rmsnorm_mxint, "silu": _ops.silu_mul_mxint}
     monkeypatch.setattr(_ops, "mxint_qdq", lambda *a, **k: (calls.__setitem__("qdq", calls["qdq"] + 1), real["qdq"](*a, **k))[1])
     monkeypatch.setattr(_ops, "rmsnorm_mxint", lambda *a, **k: (calls.__setitem__("norm", calls["norm"] + 1), real["norm"](*a, **k))[1])
+    monkeypatch.setattr(_ops, "add_rmsnorm_mxint",
+                        lambda *a, **k: (calls.__setitem__("addnorm", calls["addnorm"] + 1), real["addnorm"](*a, **k))[1])
     monkeypatch.setattr(_ops, "silu_mul_mxint", lambda *a, **k: (calls.__setitem__("silu", calls["silu"] + 1), real["silu"](*a, **k))[1])
     with torch.no_grad():
         fused = gpu(x)
-    assert calls == {"qdq": 1, "norm": 2, "silu": 1}
+    assert calls == {"qdq": 1, "norm": 1, "addnorm": 1, "silu": 1}  # the second norm also takes the residual addition
     monkeypatch.setattr(decoder_layer, "shared_mxint_width", lambda *a, **k: None)
-    calls.update(qdq=0, norm=0, silu=0)
+    calls.update(qdq=0, norm=0, addnorm=0, silu=0)
     with torch.no_grad():
         plain = gpu(x)
-    assert calls == {"qdq": 4, "norm": 0, "silu": 0}
+    assert calls == {"qdq": 4, "norm": 0, "addnorm": 0, "silu": 0}
     assert torch.equal(fused.view(torch.int16), plain.view(torch.int16))

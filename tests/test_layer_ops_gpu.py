@@ -138,6 +138,11 @@ def test_norm_and_silu_product_written_in_the_consumers_mxint_form(dev, dtype, b
         xd, wd = x.to(dev), w.to(dev)
         want = _ops.mxint_qdq(_ops.rmsnorm_minifloat(xd, wd, 1e-6), 32, bits, -1, 8)
         assert_bits_equal(_ops.rmsnorm_mxint(xd, wd, 1e-6, bits), want, f"rmsnorm_mxint {dtype} {rows}x{cols}")
+        # the residual addition in the same pass: the sum as the tensor addition rounds it, and the norm of that sum
+        rd = (torch.randn(rows, cols, generator=g) * 0.9).to(dtype).to(dev)
+        ssum, hq = _ops.add_rmsnorm_mxint(xd, rd, wd, 1e-6, bits)
+        assert_bits_equal(ssum, xd + rd, f"add_rmsnorm_mxint sum {dtype} {rows}x{cols}")
+        assert_bits_equal(hq, _ops.rmsnorm_mxint(xd + rd, wd, 1e-6, bits), f"add_rmsnorm_mxint norm {dtype} {rows}x{cols}")
         gate = (torch.randn(rows, cols, generator=g) * 3).to(dtype)
         up = torch.randn(rows, cols, generator=g).to(dtype)
         gate[0, :8] = torch.tensor([0.0, -0.0, 30.0, -30.0, 88.0, -88.0, 1e-3, -1e-3]).to(dtype)
