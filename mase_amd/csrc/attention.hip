@@ -157,14 +157,17 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
   }
 
   // async copies of one key block: 4 of K and 4 of V (4 rows of 256 bytes each) per wavefront.
-  // LDS position (row, 16-byte slot) holds the row's chunk slot ^ (row % 16), so that the
-  // fragment reads of 32 lanes (32 rows, same chunk) spread over the banks.
+  // K: LDS position (row, 16-byte slot) holds the row's chunk slot ^ (row % 16), so that the fragment reads of 16 lanes
+  // (16 rows, same chunk) spread over the banks.  V: chunk slot ^ 4 * (row % 4): one pass of a transposing read takes
+  // 32 bytes (two chunks) of each of 4 consecutive rows for each of two 16-lane groups 32 bytes apart, and with the
+  // rows 4 chunks apart those 16 chunks are all different (with K's swizzle rows 2 e and 2 e + 1 shared a pair of
+  // chunks: two lanes per bank, measured as bank conflicts in 60 % of the LDS's active cycles).
   uint32_t koff[4], voff[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int krow = (wave * 4 + i) * 4 + (lane >> 4);
     koff[i] = (uint32_t)krow * p.k_st + (uint32_t)(((lane & 15) ^ (krow & 15)) << 4);
-    voff[i] = (uint32_t)krow * p.v_st + (uint32_t)(((lane & 15) ^ (krow & 15)) << 4);
+    voff[i] = (uint32_t)krow * p.v_st + (uint32_t)(((lane & 15) ^ ((krow & 3) << 2)) << 4);
   }
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lptr_t)lds;
   const int nblk = 2 * qb + 2;  // key blocks that hold a key <= the block's last query (even: the last one uses stage 1)
@@ -219,9 +222,9 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
       const int dbyte = (dt * 32 + (l32 & 16) + 4 * (lane & 3)) * 2;
       const int row0 = 16 * s + 4 * g + ((lane & 15) >> 2), row1 = row0 + 8;
       const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (lds_s16x4_t*)(lptr_t)(Vb + row0 * 256 + (((dbyte >> 4) ^ (row0 & 15)) << 4) + (dbyte & 8)));
+          (lds_s16x4_t*)(lptr_t)(Vb + row0 * 256 + (((dbyte >> 4) ^ ((row0 & 3) << 2)) << 4) + (dbyte & 8)));
       const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (lds_s16x4_t*)(lptr_t)(Vb + row1 * 256 + (((dbyte >> 4) ^ (row1 & 15)) << 4) + (dbyte & 8)));
+          (lds_s16x4_t*)(lptr_t)(Vb + row1 * 256 + (((dbyte >> 4) ^ ((row1 & 3) << 2)) << 4) + (dbyte & 8)));
       s16x8_t both;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
