@@ -227,35 +227,37 @@ struct RopeParams {
 };
 
 // out = R(R(x * cos) + R(rotate_half(x) * sin)), rotate_half(x) = cat(-x[D/2:], x[:D/2]); each lane takes 8 elements
-// of one (b, h, t) row and reads the 8 partner elements half a row away
+// of the lower half of one (b, h, t) row and the 8 elements half a row away, which are each other's partners, so
+// every element is read once.  Grid: x over the (head, vector) pairs of one token (heads of a token lie next to each
+// other in a projection's output), y and z the token (b * T + t = z * 32768 + y: uniform per work-group, so the
+// divisions by T are scalar).
 template <int DT>
 __global__ __launch_bounds__(256) void rope_kernel(RopeParams p) {
   using TR = DTypeTraits<DT>;
-  const int vec_per_row = p.D / 8;
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  const size_t total = (size_t)p.B * p.H * p.T * vec_per_row;
-  if (i >= total) return;
-  const int v = (int)(i % vec_per_row);
-  size_t r = i / vec_per_row;
-  const int h = (int)(r % p.H);
-  r /= p.H;
-  const int t = (int)(r % p.T);
-  const int b = (int)(r / p.T);
+  const uint32_t half_vecs = (uint32_t)p.D / 16;  // 8-element vectors in half a row
+  const uint32_t hv = blockIdx.x * 256u + threadIdx.x;
+  if (hv >= (uint32_t)p.H * half_vecs) return;
+  const uint32_t token = blockIdx.z * 32768u + blockIdx.y;
+  if (token >= (uint32_t)p.B * (uint32_t)p.T) return;
+  const uint32_t b = token / (uint32_t)p.T, t = token - b * (uint32_t)p.T;
+  const uint32_t h = hv / half_vecs, v = hv - h * half_vecs;
   const size_t row = (size_t)b * p.xs_b + (size_t)h * p.xs_h + (size_t)t * p.xs_t;
   const size_t crow = (size_t)b * p.cs_b + (size_t)t * p.cs_t;
-  const int d0 = v * 8, half = p.D / 2;
-  const bool low = d0 < half;
-  float x[8], xp[8], c[8], sn[8], y[8];
-  load_vec8<DT>(p.x, row + d0, x);
-  load_vec8<DT>(p.x, row + (low ? d0 + half : d0 - half), xp);
-  load_vec8<DT>(p.cos, crow + d0, c);
-  load_vec8<DT>(p.sin, crow + d0, sn);
+  const int d0 = (int)v * 8, half = p.D / 2;
+  float xl[8], xh[8], cl[8], ch[8], sl[8], sh[8], yl[8], yh[8];
+  load_vec8<DT>(p.x, row + d0, xl);
+  load_vec8<DT>(p.x, row + d0 + half, xh);
+  load_vec8<DT>(p.cos, crow + d0, cl);
+  load_vec8<DT>(p.cos, crow + d0 + half, ch);
+  load_vec8<DT>(p.sin, crow + d0, sl);
+  load_vec8<DT>(p.sin, crow + d0 + half, sh);
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    const float rot = low ? -xp[j] : xp[j];
-    y[j] = TR::round(x[j] * c[j]) + TR::round(rot * sn[j]);
+    yl[j] = TR::round(xl[j] * cl[j]) + TR::round(-xh[j] * sl[j]);
+    yh[j] = TR::round(xh[j] * ch[j]) + TR::round(xl[j] * sh[j]);
   }
-  store_vec8<DT>(p.out, row + d0, y);
+  store_vec8<DT>(p.out, row + d0, yl);
+  store_vec8<DT>(p.out, row + d0 + half, yh);
 }
 
 bool fill_cast(CastSpec& c, int exp_bits, int frac_bits, int is_finite, int round_mode) {
@@ -423,7 +425,7 @@ extern "C" int mase_rope(const void* x, const void* cos, const void* sin, void* 
   using namespace mase;
   if (B == 0 || H == 0 || T == 0 || D == 0) return MASE_OK;
   if (x == nullptr || cos == nullptr || sin == nullptr || out == nullptr) return MASE_ERR_NULL;
-  if (D % 16 != 0 || D > 4096 || B * H * T > 0x7FFFFFFFull) return MASE_ERR_SHAPE;
+  if (D % 16 != 0 || D > 4096 || B * H * T > 0x7FFFFFFFull || B * T > 65535ull * 32768ull) return MASE_ERR_SHAPE;
   if ((x_stride_b | x_stride_h | x_stride_t | cs_stride_b | cs_stride_t) % 8 != 0) return MASE_ERR_SHAPE;
   if (!aligned16(x) || !aligned16(cos) || !aligned16(sin) || !aligned16(out)) return MASE_ERR_ALIGN;
   if (dtype < 0 || dtype > 2) return MASE_ERR_DTYPE;
@@ -442,8 +444,9 @@ extern "C" int mase_rope(const void* x, const void* cos, const void* sin, void* 
   p.cs_b = cs_stride_b;
   p.cs_t = cs_stride_t;
   hipStream_t st = (hipStream_t)stream;
-  const size_t total = B * H * T * (D / 8);
-  const dim3 grid(blocks_for(total, (size_t)256)), block(256);
+  const size_t tokens = B * T;  // < 2^31 (checked above)
+  const dim3 grid(blocks_for(H * (D / 16), (size_t)256), (unsigned)(tokens < 32768 ? tokens : 32768),
+                  (unsigned)((tokens + 32767) / 32768)), block(256);
   switch (dtype) {
     case MASE_DT_F32: hipLaunchKernelGGL((rope_kernel<MASE_DT_F32>), grid, block, 0, st, p); break;
     case MASE_DT_BF16: hipLaunchKernelGGL((rope_kernel<MASE_DT_BF16>), grid, block, 0, st, p); break;
