@@ -181,8 +181,8 @@ __device__ __forceinline__ void codes4_to_bf16(uint32_t c, float scale, float bi
   const float f1 = __builtin_fmaf((float)((u >> 8) & 0xFFu), scale, bias);
   const float f2 = __builtin_fmaf((float)((u >> 16) & 0xFFu), scale, bias);
   const float f3 = __builtin_fmaf((float)(u >> 24), scale, bias);
-  lo = (f2bits(f0) >> 16) | (f2bits(f1) & 0xFFFF0000u);
-  hi = (f2bits(f2) >> 16) | (f2bits(f3) & 0xFFFF0000u);
+  lo = __builtin_amdgcn_perm(f2bits(f1), f2bits(f0), 0x07060302u);  // the upper halves: two bf16 values
+  hi = __builtin_amdgcn_perm(f2bits(f3), f2bits(f2), 0x07060302u);
 }
 
 template <int XC>
@@ -242,14 +242,19 @@ __global__ __launch_bounds__(kSqThreads) void gemm_skinny_mxint8_partial_kernel(
     sk_wait_vmcnt<(S - 1) * G::kCopies>();  // chunk c has landed; the later ones may be in flight
     const unsigned char* st = ring + (c % S) * G::kStageBytes;
     const uint32_t sc4 = *(const uint32_t*)(st + G::kCodeBytes + r * 4);  // the row's 4 scale bytes of this chunk
+    float scale4[4], bias4[4];  // 2^(byte - 134) and the -128 * scale that removes the code offset, per block of 32
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const uint32_t sb = (sc4 >> (8 * b)) & 0xFFu;
+      scale4[b] = bits2f(sb >= 8u ? (sb - 7u) << 23 : 0u);
+      bias4[b] = -128.0f * scale4[b];
+    }
 #pragma unroll
     for (int step = 0; step < 8; ++step) {
       // 8 codes of row r at K offset step*16 + g*8, and the 8 values of A row r at the same K offset
       const uint2 cw = *(const uint2*)(st + r * 128 + ((step ^ ((r >> 1) & 7)) << 4) + g * 8);
       const uint4 xv = *(const uint4*)(st + G::kCodeBytes + G::kScaleBytes + arow * 256 + (((2 * step + g) ^ (arow & 15)) << 4));
-      const uint32_t sb = (sc4 >> (8 * (step >> 1))) & 0xFFu;
-      const float scale = bits2f(sb >= 8u ? (sb - 7u) << 23 : 0u);  // 2^(sb - 134)
-      const float bias = -128.0f * scale;
+      const float scale = scale4[step >> 1], bias = bias4[step >> 1];
       uint4 wv;
       codes4_to_bf16(cw.x, scale, bias, wv.x, wv.y);
       codes4_to_bf16(cw.y, scale, bias, wv.z, wv.w);
