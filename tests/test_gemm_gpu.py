@@ -219,6 +219,39 @@ def test_gemm_with_the_weight_in_fragment_order_is_the_same_product(dev, M, N, K
         assert float((gemm_bf16_tn(a, b, None, torch.float32, b_packed=bp) - ref).abs().max() / ref.abs().max()) < 1e-5
 
 
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16, torch.float16])
+def test_gemm_output_not_on_a_16_byte_boundary(dev, dt):
+    """the epilogue's element-by-element stores on full tiles: C handed over 4 bytes past a 16-byte boundary (the C ABI
+    asks for no alignment of C), the same values as in an aligned C"""
+    from mase_amd import _lib
+    from mase_amd._gemm import gemm_bf16_pack_b, gemm_bf16_tn
+
+    lib = _lib.load()
+    M, N, K = 512, 520, 256  # two tile columns in full and a ragged third; N a multiple of 8
+    g = torch.Generator().manual_seed(7)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
+    b = (torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+    bias = torch.randn(N, generator=g).to(dev)
+    bp = gemm_bf16_pack_b(b)
+    want = gemm_bf16_tn(a, b, bias, dt, b_packed=bp)
+    shift = 4 // want.element_size()
+    buf = torch.zeros(M * N + 16, dtype=dt, device=dev)
+    c = buf[shift: shift + M * N]
+    assert c.data_ptr() % 16 == 4
+    code = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}[dt]
+    for packed in (True, False):
+        buf.zero_()
+        if packed:
+            rc = lib.mase_gemm_bf16_tn_packed(a.data_ptr(), bp.data_ptr(), bias.data_ptr(), c.data_ptr(), M, N, K, code, 0,
+                                              _lib.stream_ptr(a))
+        else:
+            rc = lib.mase_gemm_bf16_tn(a.data_ptr(), b.data_ptr(), bias.data_ptr(), c.data_ptr(), M, N, K, code, 0,
+                                       _lib.stream_ptr(a))
+        assert rc == 0
+        assert torch.equal(c.view(M, N), want), packed
+        assert float(buf[:shift].abs().max()) == 0 and float(buf[shift + M * N:].abs().max()) == 0  # nothing outside C
+
+
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (512, 768, 256), (300, 200, 384), (4096, 4096, 1024), (130, 4096, 512),
                                    (4100, 4200, 640), (16384, 1024, 4096), (16384, 4096, 11008), (16131, 11008, 4096)])
 def test_gemm_with_the_weight_as_mxint8_codes_in_fragment_order(dev, M, N, K):
