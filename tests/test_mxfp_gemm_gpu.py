@@ -134,6 +134,33 @@ def test_gemm_mxfp_scaled_against_decoded_operands(dev, afmt, bfmt, M, N, K):
                        (y + bias.to(dev).half().float()).half())
 
 
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_gemm_mxfp_output_not_on_a_16_byte_boundary(dev, dt, with_bias):
+    """the epilogue's element-by-element stores on full tiles: C handed over 4 bytes past a 16-byte boundary (the C ABI
+    asks for no alignment of C), the same values as in an aligned C and nothing written outside it"""
+    from mase_amd import _lib
+    from mase_amd._gemm import MXFP_HW_FORMATS, gemm_mxfp_scaled, mxfp_pack
+
+    lib = _lib.load()
+    M, N, K = 512, 520, 256
+    g = torch.Generator().manual_seed(11)
+    ac, asc = mxfp_pack(torch.randn(M, K, generator=g).to(dev), 4, 3)
+    bc, bsc = mxfp_pack((torch.randn(N, K, generator=g) * 0.02).to(dev), 2, 1)
+    bias = torch.randn(N, generator=g).to(dev) if with_bias else None
+    want = gemm_mxfp_scaled(ac, asc, (4, 3), bc, bsc, (2, 1), bias, dt)
+    shift = 4 // want.element_size()
+    buf = torch.zeros(M * N + 16, dtype=dt, device=dev)
+    c = buf[shift: shift + M * N]
+    assert c.data_ptr() % 16 == 4
+    rc = lib.mase_gemm_mxfp_scaled(ac.data_ptr(), asc.data_ptr(), MXFP_HW_FORMATS[(4, 3)], bc.data_ptr(), bsc.data_ptr(),
+                                   MXFP_HW_FORMATS[(2, 1)], bias.data_ptr() if with_bias else None, c.data_ptr(), M, N, K,
+                                   _lib.DTYPE_CODE[dt], 0, _lib.stream_ptr(ac))
+    assert rc == 0
+    assert torch.equal(c.view(M, N), want)
+    assert float(buf[:shift].abs().max()) == 0 and float(buf[shift + M * N:].abs().max()) == 0
+
+
 def test_gemm_mxfp_exact_small_integers(dev):
     """e2m1 x e4m3 with unit scales and values that both formats hold exactly: every product is a multiple of 32
     below 2^11, so neither the 12-bit alignment inside the instruction nor fp32 accumulation rounds anything"""
