@@ -102,6 +102,11 @@ __device__ __forceinline__ float acc_read(float a) {
   asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
   return v;
 }
+// The compiler separates a matrix instruction from a read of its result by the wait states the part requires, but it does
+// not look inside acc_read's assembly.  An epilogue therefore starts with this: more wait states than the longest
+// matrix instruction needs (19), issued after the K loop's last matrix instruction and, both being volatile assembly,
+// before the first acc_read.
+__device__ __forceinline__ void acc_read_fence() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -282,6 +287,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   auto epilogue = [&](int ord) __attribute__((always_inline)) {
     int m0, n0, ks;
     tile_origin(ord, m0, n0, ks);
+    acc_read_fence();
     // partial tiles of K range ks go to slice ks of C (fp32, no bias: the caller's reduction adds it)
     unsigned char* const Cs = (unsigned char*)p.C + (size_t)ks * (size_t)p.M * (size_t)p.N * sizeof(float);
     const int lane = lane_now();

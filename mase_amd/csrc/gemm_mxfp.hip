@@ -71,6 +71,11 @@ __device__ __forceinline__ float acc_read(float a) {
   asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
   return v;
 }
+// The compiler separates a matrix instruction from a read of its result by the wait states the part requires, but it does
+// not look inside acc_read's assembly.  An epilogue therefore starts with this: more wait states than the longest
+// matrix instruction needs (19), issued after the K loop's last matrix instruction and, both being volatile assembly,
+// before the first acc_read.
+__device__ __forceinline__ void acc_read_fence() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 
 __device__ __forceinline__ float load_bias_v(const void* bias, int dt, int col) {
   if (dt == MASE_DT_F32) return ((const float*)bias)[col];
@@ -305,6 +310,7 @@ __global__ __launch_bounds__(kThreadsG) void gemm_mxfp_kernel(MxGemmParams p) {
   auto epilogue = [&](int ord) __attribute__((always_inline)) {
     int m0, n0;
     tile_origin(ord, m0, n0);
+    acc_read_fence();
     int lane = lane_id;
     asm volatile("" : "+v"(lane));  // keeps the lane-derived terms below out of the K loop's live registers
     const int r32 = lane & 31, kgrp = lane >> 5;
