@@ -289,35 +289,38 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
     }
     const float mc = m * p.c;
     float psum = 0.0f;
-    uint4 pw[4];
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        sc[t][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[t][r], p.c, -mc));
-        psum += sc[t][r];
-        if ((r & 3) == 3) {
-          read_v_one(2 + t, r >> 2);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-    lsum += psum;
+    // Contraction step s of O^T += V^T P^T takes the probabilities of 8 keys per lane: registers 8 (s % 2) .. + 8 of
+    // score tile s / 2.  Each step's matrix instructions are issued as soon as its 8 exponentials are done, so the
+    // matrix pipe works on step s while the wavefront computes the exponentials of step s + 1.  The V fragments of steps
+    // 2 and 3 are read between the exponentials of steps 0, 1 and of step 2.
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int t = s >> 1, r0 = (s & 1) * 8;
-      pw[s].x = f32x2_to_bf16x2_bits(sc[t][r0 + 0], sc[t][r0 + 1]);
-      pw[s].y = f32x2_to_bf16x2_bits(sc[t][r0 + 2], sc[t][r0 + 3]);
-      pw[s].z = f32x2_to_bf16x2_bits(sc[t][r0 + 4], sc[t][r0 + 5]);
-      pw[s].w = f32x2_to_bf16x2_bits(sc[t][r0 + 6], sc[t][r0 + 7]);
-    }
-    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pw[s]);
+      for (int r = r0; r < r0 + 8; ++r) {
+        sc[t][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[t][r], p.c, -mc));
+        psum += sc[t][r];
+        if (t == 0 && (r & 3) == 3) {
+          read_v_one(2, r >> 2);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (s == 2 && (r & 1) == 1) {
+          read_v_one(3, r >> 1);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      uint4 pw;
+      pw.x = f32x2_to_bf16x2_bits(sc[t][r0 + 0], sc[t][r0 + 1]);
+      pw.y = f32x2_to_bf16x2_bits(sc[t][r0 + 2], sc[t][r0 + 3]);
+      pw.z = f32x2_to_bf16x2_bits(sc[t][r0 + 4], sc[t][r0 + 5]);
+      pw.w = f32x2_to_bf16x2_bits(sc[t][r0 + 6], sc[t][r0 + 7]);
+      const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pw);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[s][dt], pf, o[dt], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
+    lsum += psum;
   }
   if (!has_next) at_wait_vmcnt<0>();  // no copy may be in flight towards LDS when the work-group retires
   lsum += __shfl_xor(lsum, 32, 64);
