@@ -290,25 +290,23 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
     const float mc = m * p.c;
     float psum = 0.0f;
     // Contraction step s of O^T += V^T P^T takes the probabilities of 8 keys per lane: registers 8 (s % 2) .. + 8 of
-    // score tile s / 2.  Each step's matrix instructions are issued as soon as its 8 exponentials are done, so the
-    // matrix pipe works on step s while the wavefront computes the exponentials of step s + 1.  The V fragments of steps
-    // 2 and 3 are read between the exponentials of steps 0, 1 and of step 2.
+    // score tile s / 2.  A wavefront that issues matrix instructions back to back waits at each for the pipe to take it,
+    // so the 4 of step s are issued one at a time with two exponentials of step s + 1 after each (about what fits under
+    // one of them); only step 0's exponentials and step 3's matrix instructions have nothing to share the time with.
+    // The V fragments of steps 2 and 3 are read between the exponentials of steps 0, 1 and of step 2.
+    auto exp_one = [&](int s, int r) __attribute__((always_inline)) {  // r: 0..7 within step s
+      const int t = s >> 1, rr = (s & 1) * 8 + r;
+      sc[t][rr] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[t][rr], p.c, -mc));
+      psum += sc[t][rr];
+      if (t == 0 && (rr & 3) == 3) read_v_one(2, rr >> 2);
+      if (s == 2 && (rr & 1) == 1) read_v_one(3, rr >> 1);
+    };
+#pragma unroll
+    for (int r = 0; r < 8; ++r) exp_one(0, r);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int t = s >> 1, r0 = (s & 1) * 8;
-#pragma unroll
-      for (int r = r0; r < r0 + 8; ++r) {
-        sc[t][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[t][r], p.c, -mc));
-        psum += sc[t][r];
-        if (t == 0 && (r & 3) == 3) {
-          read_v_one(2, r >> 2);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        if (s == 2 && (r & 1) == 1) {
-          read_v_one(3, r >> 1);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
       uint4 pw;
       pw.x = f32x2_to_bf16x2_bits(sc[t][r0 + 0], sc[t][r0 + 1]);
       pw.y = f32x2_to_bf16x2_bits(sc[t][r0 + 2], sc[t][r0 + 3]);
@@ -317,8 +315,14 @@ __global__ __launch_bounds__(256, 2) void attn_causal_fwd_kernel(AttnParams p) {
       const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pw);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[s][dt], pf, o[dt], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
+      for (int dt = 0; dt < 4; ++dt) {
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[s][dt], pf, o[dt], 0, 0, 0);
+        if (s < 3) {
+          exp_one(s + 1, 2 * dt);
+          exp_one(s + 1, 2 * dt + 1);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
     lsum += psum;
   }
