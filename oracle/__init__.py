@@ -25,12 +25,17 @@ Pinning status (what fixes each function besides reading the source):
                                    exponents from the library's own ``log2`` in the dtype               -> pinned
 * ``minifloat_denorm/ieee``        exact closed form in fp32; in bf16 / fp16 the same explicit-rounding model over
                                    every finite 16-bit input for (8,4), (8,5), (6,3)                     -> pinned
-* ``_minifloat_mx`` encode/decode  nearest-value brute force away from the documented quirks; invariants the format
-  and ``mxfp_quantizer``           fixes (codes fit 1+E+F bits, normal codes survive decode -> encode).  The quirks
-                                   themselves (``>> 8`` double rounding, lost carry in odd binades, truncating
-                                   subnormals, flushed values below 2^-bias) are defined by the source text alone: two
-                                   restatements of that text agree, nothing else can confirm the reading
-                                                                                        -> parity unpinned (quirk regions)
+* ``_minifloat_mx`` encode/decode  what the bit-field text computes, stated as a function of the input VALUE in exact
+  and ``mxfp_quantizer``           arithmetic (carry out of the fraction: 2^(e+1) in even exponent fields, 2^e in odd
+                                   ones; exponent field 0: truncation to the subnormal grid, zero for fraction 0;
+                                   zero below 2^-bias; saturation; the 8-bit truncation before rounding), compared
+                                   over every 16-bit high-half fp32 pattern, the same with non-zero low halves and a
+                                   dense grid of ties, all six legal element formats x both ``is_finite`` x four
+                                   rounding modes; plausible misreadings (ADD for the OR, rounded subnormals, rounding
+                                   before truncation, gradual underflow) are each shown to fail that comparison
+                                   (``tests/test_minifloat_mx_value_pins.py``); format invariants (codes fit 1+E+F
+                                   bits, normal codes survive decode -> encode); the MXFP scale by exact arithmetic
+                                                                                        -> pinned
 
 * clip search (``quantile_search``)   quantile against exact rational interpolation; candidates against the scalar
                                    restatement; the choice against exact errors (first minimum, strict replace);

@@ -235,7 +235,8 @@ def test_minifloat_mx_is_nearest_value_away_from_the_quirks(E, F):
 
 
 def test_minifloat_mx_documented_quirks():
-    """The source-specific behaviours, asserted as such (parity unpinned: no reference execution backs them)."""
+    """The source-specific behaviours on hand-picked points (their value-domain closed form is swept exhaustively in
+    test_minifloat_mx_value_pins.py)."""
     q = lambda v, E, F: O.minifloat_quantizer_sim(torch.tensor([v], dtype=torch.float32), E, F, True, "rn").item()
     assert q(500.0, 4, 3) == 256.0     # [496,512): fraction rounds to 2^F, exponent field 15 is odd -> carry lost
     assert q(480.0, 4, 3) == 480.0     # all-finite e4m3 tops out at 480, not 448
