@@ -169,20 +169,21 @@ class CopyBytes(Workload):
     unit = "GB/s"
     dtype = "u8"
     kernel = "copy_bytes_kernel"
-    config = {"workload": "mase_copy_bytes of 134217728 bytes (calibration: achievable HBM ceiling, counter scale)"}
+    config = {"workload": "plain streaming copy of 134217728 bytes (calibration: achievable HBM ceiling, counter scale)"}
     nbytes = 134217728
 
     def setup(self, torch, dev, n_buffers):
+        import bench_support
         from mase_amd import _lib
 
-        self.lib = _lib.load()
+        self.lib = bench_support.load()
         self._lib = _lib
         self.bufs = [torch.randint(0, 255, (self.nbytes,), dtype=torch.uint8, device=dev) for _ in range(max(n_buffers, 4))]
         self.outs = [torch.empty(self.nbytes, dtype=torch.uint8, device=dev) for _ in range(2)]
 
     def step(self, i):
         src, dst = self.bufs[i % len(self.bufs)], self.outs[i % 2]
-        self._lib.check(self.lib.mase_copy_bytes(src.data_ptr(), dst.data_ptr(), self.nbytes, self._lib.stream_ptr(src)), "copy")
+        self._lib.check(self.lib.bench_copy_bytes(src.data_ptr(), dst.data_ptr(), self.nbytes, self._lib.stream_ptr(src)), "copy")
 
     def work_per_step(self):
         return 2.0 * self.nbytes
@@ -200,15 +201,16 @@ class _MfmaIssueRate(Workload):
     operands = 0
     iters = 4096      # x 8 instructions per wavefront
     work_groups = 256
-    entry = "mase_probe_mfma_bf16"
+    entry = "bench_probe_mfma_bf16"
     instruction = "v_mfma_f32_32x32x16_bf16"
     flop_per_instruction = 2.0 * 32 * 32 * 16
     nominal_cycles = 32
 
     def setup(self, torch, dev, n_buffers):
+        import bench_support
         from mase_amd import _lib
 
-        self.lib = _lib.load()
+        self.lib = bench_support.load()
         self._lib = _lib
         self.out = torch.empty(self.work_groups * 512 + 4, dtype=torch.float32, device=dev)
         self.metric = f"matrix-core issue rate of {self.instruction} on register operands (no memory traffic)"
@@ -228,7 +230,7 @@ class _MfmaIssueRate(Workload):
     def extra(self, torch):
         """shader clock during the last launch, from the kernel's own two counters (first wavefront's loop)"""
         cyc, ticks = self.out[-4:].view(torch.int64).tolist()
-        rate_khz = int(self.lib.mase_constant_rate_counter_khz())
+        rate_khz = int(self.lib.bench_constant_rate_counter_khz())
         secs = ticks / (rate_khz * 1e3)
         return {"shader_clock_ghz_in_loop": round(cyc / secs / 1e9, 3), "cycles_per_instruction_of_first_wavefront": round(cyc / (8.0 * self.iters), 2),
                 "constant_rate_counter_khz": rate_khz}
@@ -246,7 +248,7 @@ class MfmaRateRandom(_MfmaIssueRate):
 
 class _MfmaF8F4Rate(_MfmaIssueRate):
     kernel = "probe_mfma_f8f4_kernel"
-    entry = "mase_probe_mfma_f8f4"
+    entry = "bench_probe_mfma_f8f4"
     instruction = "v_mfma_scale_f32_32x32x64_f8f6f4 (e4m3 x e2m1, scales of 1)"
     flop_per_instruction = 2.0 * 32 * 32 * 64
     nominal_cycles = 64

@@ -1,9 +1,17 @@
-// Measurement aid, no counterpart in the reference: the rate at which the matrix cores of this GPU accept
+// Calibration kernels of the benchmark (bench.py), built into bench_support/libmase_bench.so: NOT part of the product
+// library or its C ABI, and without counterpart in the reference.
+//   bench_copy_bytes               plain streaming copy: the achievable-bandwidth ceiling and the scale of the hardware
+//                                  byte counters
+//   bench_probe_mfma_bf16 / _f8f4  issue rate of the matrix instruction on register operands, nothing else running
+//   bench_constant_rate_counter_khz
+// Status codes: 0 ok, negative = the product library's error codes (include/mase_amd.h).
+//
+// The matrix-core probe: the rate at which the matrix cores of this GPU accept
 // v_mfma_f32_32x32x16_bf16 when nothing else runs (no memory traffic, no LDS, operands held in registers), as a
 // function of the operand VALUES.  The rate depends on them: with zero or small-integer operands the instruction
 // issues close to its nominal 32 cycles, with operands whose mantissa and exponent bits vary it is held back by the
 // power management of the part.  That second figure, not the published peak, is what a GEMM on real data can approach.
-#include "common.hpp"
+#include "../mase_amd/csrc/common.hpp"
 
 namespace mase {
 namespace {
@@ -103,14 +111,40 @@ __global__ __launch_bounds__(512) void probe_mfma_f8f4_kernel(float* out, int it
   }
 }
 
+__global__ __launch_bounds__(64) void copy_bytes_kernel(const uint4* __restrict__ in, uint4* __restrict__ out, size_t n) {
+  size_t i = (size_t)blockIdx.x * 64 + threadIdx.x;
+  if (i < n) store_nt(out + i, load_nt(in + i));
+}
+
+// each wavefront issues 8 * iters matrix instructions; the bound keeps a mistaken argument from occupying the GPU for
+// minutes (2^20 iterations are about a tenth of a second)
+constexpr int kMaxProbeIters = 1 << 20;
+
 }  // namespace
 }  // namespace mase
 
-extern "C" int mase_probe_mfma_bf16(void* out, size_t out_bytes, int work_groups, int wavefronts_per_simd, int iters,
+// `bytes` a multiple of 16, pointers 16-byte aligned
+extern "C" int bench_copy_bytes(const void* in, void* out, size_t bytes, void* stream) {
+  using namespace mase;
+  if (bytes == 0) return MASE_OK;
+  if (in == nullptr || out == nullptr) return MASE_ERR_NULL;
+  if ((bytes & 15u) != 0) return MASE_ERR_SHAPE;
+  if (!aligned16(in) || !aligned16(out)) return MASE_ERR_ALIGN;
+  const size_t n = bytes / 16;
+  hipLaunchKernelGGL(copy_bytes_kernel, dim3(blocks_for(n, 64)), dim3(64), 0, (hipStream_t)stream, (const uint4*)in,
+                     (uint4*)out, n);
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+// work_groups x (4 x wavefronts_per_simd) wavefronts, each issuing 8 * iters instructions (1 <= iters <= 2^20) on
+// register operands.  out (16-byte aligned): work_groups * 256 * wavefronts_per_simd floats of scratch followed by two
+// int64 the kernel writes: the duration of the first wavefront's loop in shader-clock cycles and in ticks of the
+// constant-rate counter.
+extern "C" int bench_probe_mfma_bf16(void* out, size_t out_bytes, int work_groups, int wavefronts_per_simd, int iters,
                                     int operands, void* stream) {
   using namespace mase;
   if (out == nullptr) return MASE_ERR_NULL;
-  if (work_groups < 1 || work_groups > 65536 || (wavefronts_per_simd != 1 && wavefronts_per_simd != 2) || iters < 1 ||
+  if (work_groups < 1 || work_groups > 65536 || (wavefronts_per_simd != 1 && wavefronts_per_simd != 2) || iters < 1 || iters > kMaxProbeIters ||
       operands < 0 || operands > 2)
     return MASE_ERR_PARAM;
   const int threads = 256 * wavefronts_per_simd;
@@ -120,11 +154,11 @@ extern "C" int mase_probe_mfma_bf16(void* out, size_t out_bytes, int work_groups
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
 
-extern "C" int mase_probe_mfma_f8f4(void* out, size_t out_bytes, int work_groups, int wavefronts_per_simd, int iters,
+extern "C" int bench_probe_mfma_f8f4(void* out, size_t out_bytes, int work_groups, int wavefronts_per_simd, int iters,
                                     int operands, void* stream) {
   using namespace mase;
   if (out == nullptr) return MASE_ERR_NULL;
-  if (work_groups < 1 || work_groups > 65536 || (wavefronts_per_simd != 1 && wavefronts_per_simd != 2) || iters < 1 ||
+  if (work_groups < 1 || work_groups > 65536 || (wavefronts_per_simd != 1 && wavefronts_per_simd != 2) || iters < 1 || iters > kMaxProbeIters ||
       (operands != 0 && operands != 2))
     return MASE_ERR_PARAM;
   const int threads = 256 * wavefronts_per_simd;
@@ -134,7 +168,8 @@ extern "C" int mase_probe_mfma_f8f4(void* out, size_t out_bytes, int work_groups
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
 
-extern "C" int mase_constant_rate_counter_khz(void) {
+// rate of the constant-rate counter on the current device in kHz; 0 when the runtime cannot tell
+extern "C" int bench_constant_rate_counter_khz(void) {
   int dev = 0, khz = 0;
   if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess) return 0;
   return khz;

@@ -367,26 +367,6 @@ int mase_rope(const void* x, const void* cos, const void* sin, void* out, size_t
               size_t x_stride_b, size_t x_stride_h, size_t x_stride_t, size_t cs_stride_b, size_t cs_stride_t, int dtype,
               void* stream);
 
-/* Plain streaming copy of `bytes` (multiple of 16, 16-byte aligned pointers).  No counterpart in the reference:
- * it is the calibration kernel for the achievable-bandwidth ceiling and for scaling hardware byte counters. */
-int mase_copy_bytes(const void* in, void* out, size_t bytes, void* stream);
-
-/* Issue rate of v_mfma_f32_32x32x16_bf16 with nothing else running: work_groups x (4 x wavefronts_per_simd) wavefronts,
- * each issuing 8 * iters instructions on register operands.  operands: 0 zeros, 1 small integers, 2 uniform values in
- * [-2, 2).  No counterpart in the reference: it measures the matrix-core rate this GPU sustains for a given kind of
- * operand values (the power management of the part holds the instruction back when operand bits vary), the ceiling
- * the GEMM kernels are to be read against.  out (16-byte aligned): work_groups * 256 * wavefronts_per_simd floats of
- * scratch followed by two int64 the kernel writes: the duration of the first wavefront's loop in shader-clock cycles
- * and in ticks of the constant-rate counter (hipDeviceAttributeWallClockRate). */
-int mase_probe_mfma_bf16(void* out, size_t out_bytes, int work_groups, int wavefronts_per_simd, int iters, int operands,
-                         void* stream);
-/* the same for v_mfma_scale_f32_32x32x64_f8f6f4 with e4m3 codes in A and e2m1 codes in B, scales of 1 (the
- * instruction of the MXFP8 x MXFP4 Linear); operands: 0 zero codes, 2 random codes */
-int mase_probe_mfma_f8f4(void* out, size_t out_bytes, int work_groups, int wavefronts_per_simd, int iters, int operands,
-                         void* stream);
-/* rate of that constant-rate counter on the current device in kHz; 0 when the runtime cannot tell */
-int mase_constant_rate_counter_khz(void);
-
 /* test/diagnostic helpers (host only, no device work) */
 uint32_t mase_isclose_zero_threshold_bits(int dtype); /* largest |x| (fp32 bits) that isclose(x, 0) accepts */
 float mase_round_scalar_to_dtype(double v, int dtype); /* how a clamp bound is represented in dtype */

@@ -49,9 +49,6 @@ SIGNATURES = {
                                        c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "mase_silu_mul_minifloat": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "mase_attention_causal": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p] + [c_size_t] * 16 + [c_int, c_float, c_void_p]),
-    "mase_constant_rate_counter_khz": (c_int, []),
-    "mase_probe_mfma_f8f4": (c_int, [c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p]),
-    "mase_probe_mfma_bf16": (c_int, [c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p]),
     "mase_attention_causal_fused": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p] + [c_size_t] * 16 + [c_int, c_float, c_void_p, c_void_p,
                                             c_size_t, c_size_t, c_int, c_void_p, c_void_p]),
     "mase_rmsnorm_mxint": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_float, c_int, c_void_p, c_void_p]),
@@ -85,7 +82,6 @@ SIGNATURES = {
     "mase_gemm_mxfp4_scaled_tiled": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
                                              c_size_t, c_size_t, c_int, c_int, c_void_p]),
     "mase_gemm_mxfp_scaled": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_int, c_int, c_void_p]),
-    "mase_copy_bytes": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "mase_isclose_zero_threshold_bits": (c_uint32, [c_int]),
     "mase_round_scalar_to_dtype": (c_float, [c_double, c_int]),
 }

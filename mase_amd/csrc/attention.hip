@@ -56,7 +56,7 @@ constexpr int kAttnLds = 2 * kKBytes + 2 * kVBytes;
 // lane i's 16 bytes at base + off_i land at LDS address lds_addr + 16 * i; tracked by hand with at_wait_vmcnt
 __device__ __forceinline__ void at_async_copy_16(const unsigned char* base, uint32_t off, uint32_t lds_addr) {
   const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_addr);
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory", "m0");
 }
 template <int N>
 __device__ __forceinline__ void at_wait_vmcnt() {
@@ -390,8 +390,9 @@ int attention_causal_impl(const void* q, const void* k, const void* v, void* out
   for (size_t s : strides)
     if (s % 8 != 0) return MASE_ERR_ALIGN;
   if (q_stride_t < 128 || k_stride_t < 128 || v_stride_t < 128 || o_stride_t < 128) return MASE_ERR_SHAPE;
-  if (k_stride_t * 2 * tokens > 0xFFFFFFFFull || q_stride_t * 2 > 0xFFFFFFFFull || o_stride_t * 2 > 0xFFFFFFFFull ||
-      v_stride_t * 2 > 0xFFFFFFFFull)
+  // 32-bit lane offsets: a key block's rows (up to 63 token strides) for k and v, one token stride for q and the output
+  if (k_stride_t * 2 * tokens > 0xFFFFFFFFull || v_stride_t * 2 * tokens > 0xFFFFFFFFull ||
+      q_stride_t * 2 > 0xFFFFFFFFull || o_stride_t * 2 > 0xFFFFFFFFull)
     return MASE_ERR_SHAPE;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return MASE_ERR_ALIGN;
   hipStream_t st = (hipStream_t)stream;
@@ -403,11 +404,11 @@ int attention_causal_impl(const void* q, const void* k, const void* v, void* out
   }
   const void* kernels[4] = {(const void*)attn_causal_fwd_kernel<false, false>, (const void*)attn_causal_fwd_kernel<true, false>,
                             (const void*)attn_causal_fwd_kernel<false, true>, (const void*)attn_causal_fwd_kernel<true, true>};
-  static bool attr_set = false;
-  if (!attr_set) {
+  static std::atomic<uint64_t> attr_done{0};
+  if (!device_setup_done(attr_done)) {
     for (const void* kfn : kernels)
       if (hipFuncSetAttribute(kfn, hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLds) != hipSuccess) return MASE_ERR_LAUNCH;
-    attr_set = true;
+    mark_device_setup_done(attr_done);
   }
   const int BH = (int)(batch * heads), T = (int)tokens;
   AttnParams p;
@@ -439,13 +440,8 @@ int attention_causal_impl(const void* q, const void* k, const void* v, void* out
   p.bh_lanes = 0;
   unsigned n_wg = (unsigned)(BH * (T / kQB));
   {
-    static int n_cu = 0;
-    if (n_cu == 0) {
-      int dev = 0;
-      hipDeviceProp_t prop;
-      if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return MASE_ERR_LAUNCH;
-      n_cu = prop.multiProcessorCount;
-    }
+    const int n_cu = device_cu_count();  // of the device the call runs on
+    if (n_cu <= 0) return MASE_ERR_LAUNCH;
     const int n_qb = T / kQB, wg_per_xcd = 2 * n_cu / 8;
     if (BH % 8 == 0 && n_cu % 8 == 0 && n_qb <= wg_per_xcd && wg_per_xcd % n_qb == 0) {
       const int lanes = wg_per_xcd / n_qb, per_xcd = BH / 8;

@@ -19,23 +19,6 @@ float host_round_f16(float f) { return (float)(_Float16)f; }
 
 }  // namespace
 
-// plain streaming copy: the calibration kernel for bandwidth ceilings and for scaling HBM byte counters
-__global__ __launch_bounds__(64) void copy_bytes_kernel(const uint4* __restrict__ in, uint4* __restrict__ out, size_t n) {
-  size_t i = (size_t)blockIdx.x * 64 + threadIdx.x;
-  if (i < n) mase::store_nt(out + i, mase::load_nt(in + i));
-}
-
-extern "C" int mase_copy_bytes(const void* in, void* out, size_t bytes, void* stream) {
-  if (bytes == 0) return MASE_OK;
-  if (in == nullptr || out == nullptr) return MASE_ERR_NULL;
-  if ((bytes & 15u) != 0) return MASE_ERR_SHAPE;
-  if (!mase::aligned16(in) || !mase::aligned16(out)) return MASE_ERR_ALIGN;
-  size_t n = bytes / 16;
-  hipLaunchKernelGGL(copy_bytes_kernel, dim3(mase::blocks_for(n, 64)), dim3(64), 0, (hipStream_t)stream, (const uint4*)in,
-                     (uint4*)out, n);
-  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
-}
-
 extern "C" int mase_abi_version(void) { return 1; }
 
 extern "C" const char* mase_error_string(int code) {

@@ -8,6 +8,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/mase_amd.h"
 
 namespace mase {
@@ -263,5 +265,40 @@ static inline unsigned blocks_for(size_t items, size_t per_block) {
 }
 
 static inline bool aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
+
+// ---------------------------------------------------------------------------------------------
+// host side: per-device facts looked up once, safely from several host threads
+// ---------------------------------------------------------------------------------------------
+// number of compute units of the current device (0 on error); cached per device index
+inline int device_cu_count() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  std::atomic<int>& slot = cached[dev & 63];
+  int n = slot.load(std::memory_order_relaxed);
+  if (n > 0 && dev < 64) return n;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+  if (dev < 64) slot.store(n, std::memory_order_relaxed);
+  return n;
+}
+
+// One bit per device index in a call site's record `done`: whether its once-per-device set-up (a kernel attribute
+// belongs to the (kernel, device) pair) has run on the current device.  Two threads may both run an idempotent set-up
+// the first time; none reads the bit as set before the set-up has finished.
+inline bool device_setup_done(const std::atomic<uint64_t>& done) {
+  int dev = 0;
+  return hipGetDevice(&dev) == hipSuccess && dev < 64 && (done.load(std::memory_order_acquire) >> dev & 1) != 0;
+}
+inline void mark_device_setup_done(std::atomic<uint64_t>& done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) == hipSuccess && dev < 64) done.fetch_or(1ull << dev, std::memory_order_release);
+}
+// raises one kernel's dynamic-LDS limit once per device
+inline bool set_dynamic_lds_once(std::atomic<uint64_t>& done, const void* kernel, int bytes) {
+  if (device_setup_done(done)) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
+  mark_device_setup_done(done);
+  return true;
+}
 
 }  // namespace mase

@@ -81,7 +81,7 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 // kernel uses M0.
 __device__ __forceinline__ void async_copy_16(const unsigned char* base, uint32_t off, uint32_t lds_addr) {
   const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_addr);
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory", "m0");
 }
 
 // The lane number, computed where it is needed (two instructions) instead of being kept: the code between output tiles
@@ -692,13 +692,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
 
 // number of work-groups of the persistent kernel: one per CU (each takes the whole LDS of its CU)
 int persistent_grid_bf16(int total_tiles) {
-  static int n_cu = 0;
-  if (n_cu == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return -1;
-    n_cu = prop.multiProcessorCount;
-  }
+  const int n_cu = device_cu_count();
+  if (n_cu <= 0) return -1;
   return total_tiles < n_cu ? total_tiles : n_cu;
 }
 
@@ -711,26 +706,18 @@ int launch_gemm_bf16(const GemmParams& p, int out_dtype, hipStream_t st, bool bp
   const bool stream_fits = p.kc / BK >= S;
 #define MASE_GEMM_LAUNCH(DT_, STREAM_)                                                                            \
   do {                                                                                                            \
-    static bool attr_set = false;                                                                                 \
+    static std::atomic<uint64_t> attr_done{0};                                                                    \
     const void* k = (const void*)gemm_bf16_tn_kernel<DT_, STREAM_>;                                               \
-    if (!attr_set) {                                                                                              \
-      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)       \
-        return MASE_ERR_LAUNCH;                                                                                   \
-      attr_set = true;                                                                                            \
-    }                                                                                                             \
+    if (!set_dynamic_lds_once(attr_done, k, (int)lds_bytes)) return MASE_ERR_LAUNCH;                              \
     hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, STREAM_>), grid, block, lds_bytes, st, p);                       \
   } while (0)
   if (bpack && bcodes) {
     if (!stream_fits || ((p.kc / BK) & 1) != 0) return MASE_ERR_SHAPE;
 #define MASE_GEMM_LAUNCH_C(DT_)                                                                                   \
   do {                                                                                                            \
-    static bool attr_set = false;                                                                                 \
+    static std::atomic<uint64_t> attr_done{0};                                                                    \
     const void* k = (const void*)gemm_bf16_tn_kernel<DT_, true, true, true>;                                      \
-    if (!attr_set) {                                                                                              \
-      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)       \
-        return MASE_ERR_LAUNCH;                                                                                   \
-      attr_set = true;                                                                                            \
-    }                                                                                                             \
+    if (!set_dynamic_lds_once(attr_done, k, (int)lds_bytes)) return MASE_ERR_LAUNCH;                              \
     hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, true, true, true>), grid, block, lds_bytes, st, p);              \
   } while (0)
     if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH_C(MASE_DT_F32);
@@ -741,13 +728,9 @@ int launch_gemm_bf16(const GemmParams& p, int out_dtype, hipStream_t st, bool bp
     if (!stream_fits || ((p.kc / BK) & 1) != 0) return MASE_ERR_SHAPE;
 #define MASE_GEMM_LAUNCH_B(DT_)                                                                                   \
   do {                                                                                                            \
-    static bool attr_set = false;                                                                                 \
+    static std::atomic<uint64_t> attr_done{0};                                                                    \
     const void* k = (const void*)gemm_bf16_tn_kernel<DT_, true, true>;                                            \
-    if (!attr_set) {                                                                                              \
-      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)       \
-        return MASE_ERR_LAUNCH;                                                                                   \
-      attr_set = true;                                                                                            \
-    }                                                                                                             \
+    if (!set_dynamic_lds_once(attr_done, k, (int)lds_bytes)) return MASE_ERR_LAUNCH;                              \
     hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, true, true>), grid, block, lds_bytes, st, p);                    \
   } while (0)
     if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH_B(MASE_DT_F32);

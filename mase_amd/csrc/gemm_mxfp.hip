@@ -54,9 +54,9 @@ template <int BYTES>
 __device__ __forceinline__ void async_copy(const unsigned char* base, uint32_t off, uint32_t lds_addr) {
   const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_addr);
   if constexpr (BYTES == 16)
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory", "m0");
   else
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory", "m0");
 }
 
 template <int N>
@@ -519,13 +519,8 @@ __global__ __launch_bounds__(kThreadsG) void gemm_mxfp_kernel(MxGemmParams p) {
 
 // number of work-groups of the persistent kernel: one per CU (each takes the whole LDS of its CU)
 int persistent_grid(int total_tiles) {
-  static int n_cu = 0;
-  if (n_cu == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return -1;
-    n_cu = prop.multiProcessorCount;
-  }
+  const int n_cu = device_cu_count();
+  if (n_cu <= 0) return -1;
   return total_tiles < n_cu ? total_tiles : n_cu;
 }
 
@@ -538,13 +533,9 @@ int launch_mx_gemm(const MxGemmParams& p, int out_dtype, hipStream_t st) {
   const bool stream = p.K / BK >= MxGemmGeom<B_BITS>::S;
 #define MASE_MX_LAUNCH(DT_, STREAM_)                                                                              \
   do {                                                                                                            \
-    static bool attr_set = false;                                                                                 \
+    static std::atomic<uint64_t> attr_done{0};                                                                    \
     const void* k = (const void*)gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, DT_, STREAM_, TILED>;                       \
-    if (!attr_set) {                                                                                              \
-      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)       \
-        return MASE_ERR_LAUNCH;                                                                                   \
-      attr_set = true;                                                                                            \
-    }                                                                                                             \
+    if (!set_dynamic_lds_once(attr_done, k, (int)lds_bytes)) return MASE_ERR_LAUNCH;                              \
     hipLaunchKernelGGL((gemm_mxfp_kernel<B_BITS, CBSZ, BLGP, DT_, STREAM_, TILED>), grid, block, lds_bytes, st,   \
                        p);                                                                                        \
   } while (0)

@@ -45,7 +45,7 @@ __device__ __forceinline__ int sk_lds_off(int row, int chunk) { return row * 128
 // reasons given in gemm_bf16.hip); M0 = LDS address, nothing else in this kernel uses M0
 __device__ __forceinline__ void sk_async_copy(const unsigned char* base, uint32_t off, uint32_t lds_addr) {
   const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_addr);
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory", "m0");
 }
 
 template <int N>
@@ -171,7 +171,7 @@ struct SkinnyQParams {
 
 __device__ __forceinline__ void sk_async_copy4(const unsigned char* base, uint32_t off, uint32_t lds_addr) {
   const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_addr);
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory", "m0");
 }
 
 // four codes of one dword -> two registers of two bf16 values each (code * scale, exact)
@@ -577,14 +577,8 @@ int skinny_splits(int M, int N, int K, int n_cu) {
 }
 
 int skinny_cu_count() {
-  static int n_cu = 0;
-  if (n_cu == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return -1;
-    n_cu = prop.multiProcessorCount;
-  }
-  return n_cu;
+  const int n_cu = device_cu_count();
+  return n_cu > 0 ? n_cu : -1;
 }
 
 }  // namespace
@@ -614,15 +608,15 @@ extern "C" int mase_gemm_bf16_skinny(const void* A, const void* B, const void* b
   const size_t need = (size_t)splits * M * N * sizeof(float);
   if (workspace == nullptr || workspace_bytes < need || (((uintptr_t)workspace) & 15u) != 0) return MASE_ERR_WORKSPACE;
   hipStream_t st = (hipStream_t)stream;
-  static bool attr_set = false;
-  if (!attr_set) {
+  static std::atomic<uint64_t> attr_done{0};
+  if (!device_setup_done(attr_done)) {
     const void* ks[4] = {(const void*)gemm_skinny_partial_kernel<1>, (const void*)gemm_skinny_partial_kernel<2>,
                          (const void*)gemm_skinny_partial_kernel<3>, (const void*)gemm_skinny_partial_kernel<4>};
     const int sz[4] = {SkGeom<1>::kLdsBytes, SkGeom<2>::kLdsBytes, SkGeom<3>::kLdsBytes, SkGeom<4>::kLdsBytes};
     for (int i = 0; i < 4; ++i)
       if (hipFuncSetAttribute(ks[i], hipFuncAttributeMaxDynamicSharedMemorySize, sz[i]) != hipSuccess)
         return MASE_ERR_LAUNCH;
-    attr_set = true;
+    mark_device_setup_done(attr_done);
   }
   const dim3 grid((unsigned)(((N + 31) / 32 + 3) / 4), (unsigned)splits), block(kSkinnyThreads);
   SkinnyParams p;
@@ -680,15 +674,15 @@ extern "C" int mase_gemm_mxint8_skinny(const void* A, const int8_t* B_codes, con
   const size_t need = (size_t)splits * M * N * sizeof(float);
   if (workspace == nullptr || workspace_bytes < need || (((uintptr_t)workspace) & 15u) != 0) return MASE_ERR_WORKSPACE;
   hipStream_t st = (hipStream_t)stream;
-  static bool attr_set = false;
-  if (!attr_set) {
+  static std::atomic<uint64_t> attr_done{0};
+  if (!device_setup_done(attr_done)) {
     const void* ks[4] = {(const void*)gemm_skinny_mxint8_partial_kernel<1>, (const void*)gemm_skinny_mxint8_partial_kernel<2>,
                          (const void*)gemm_skinny_mxint8_partial_kernel<3>, (const void*)gemm_skinny_mxint8_partial_kernel<4>};
     const int sz[4] = {SqGeom<1>::kLdsBytes, SqGeom<2>::kLdsBytes, SqGeom<3>::kLdsBytes, SqGeom<4>::kLdsBytes};
     for (int i = 0; i < 4; ++i)
       if (hipFuncSetAttribute(ks[i], hipFuncAttributeMaxDynamicSharedMemorySize, sz[i]) != hipSuccess)
         return MASE_ERR_LAUNCH;
-    attr_set = true;
+    mark_device_setup_done(attr_done);
   }
   const dim3 grid((unsigned)(((N + 31) / 32 + kSqWaves - 1) / kSqWaves), (unsigned)splits), block(kSqThreads);
   SkinnyQParams p;
@@ -761,8 +755,8 @@ extern "C" int mase_gemm_mxfp4_skinny(const void* A_codes, const void* A_scales,
   const size_t need = (size_t)splits * M * N * sizeof(float);
   if (workspace == nullptr || workspace_bytes < need || (((uintptr_t)workspace) & 15u) != 0) return MASE_ERR_WORKSPACE;
   hipStream_t st = (hipStream_t)stream;
-  static bool attr_set = false;
-  if (!attr_set) {
+  static std::atomic<uint64_t> attr_done{0};
+  if (!device_setup_done(attr_done)) {
     const void* sl[8] = {(const void*)gemm_skinny_mxfp4_slab_kernel<1, 0>, (const void*)gemm_skinny_mxfp4_slab_kernel<2, 0>,
                          (const void*)gemm_skinny_mxfp4_slab_kernel<3, 0>, (const void*)gemm_skinny_mxfp4_slab_kernel<4, 0>,
                          (const void*)gemm_skinny_mxfp4_slab_kernel<1, 1>, (const void*)gemm_skinny_mxfp4_slab_kernel<2, 1>,
@@ -778,7 +772,7 @@ extern "C" int mase_gemm_mxfp4_skinny(const void* A_codes, const void* A_scales,
     for (int i = 0; i < 8; ++i)
       if (hipFuncSetAttribute(ks[i], hipFuncAttributeMaxDynamicSharedMemorySize, sz[i & 3]) != hipSuccess)
         return MASE_ERR_LAUNCH;
-    attr_set = true;
+    mark_device_setup_done(attr_done);
   }
   const dim3 grid((unsigned)(((N + 31) / 32 + 3) / 4), (unsigned)splits), block(kSkinnyThreads);
   SkinnyFParams p;

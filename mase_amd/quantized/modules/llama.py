@@ -90,8 +90,10 @@ def _fused_probabilities(kind, module, scores, key_states, attention_mask, scali
                          softmax_bypass, softmax_config):
     """scores -> scaled, masked, minifloat-cast, softmax, MX-quantized probabilities in one kernel when the operands
     allow it (device tensors, key length a multiple of 32 up to 8192, blocks of 32, no dropout); else None and the
-    caller runs the separate passes.  ``module.fused_probabilities = False`` switches it off."""
-    if not getattr(module, "fused_probabilities", True) or not scores.is_cuda:
+    caller runs the separate passes.  Opt-in (``module.fused_probabilities = True``): the kernel evaluates the
+    exponentials with the hardware ``exp2`` and about one probability in a hundred lands on the neighbouring code, while
+    the separate passes are the reference's own tensor operations on the device."""
+    if not getattr(module, "fused_probabilities", False) or not scores.is_cuda:
         return None
     if dropout != 0.0 and module.training:
         return None

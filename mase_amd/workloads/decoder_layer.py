@@ -57,11 +57,15 @@ def rotate_half(x):
 
 
 def rope_tables(seq_len: int, head_dim: int, theta: float, device, dtype):
-    inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32, device=device) / head_dim))
-    t = torch.arange(seq_len, dtype=torch.float32, device=device)
+    """cos / sin tables of the rotary embedding, evaluated on the host whatever ``device`` is: the host's and the
+    device's ``cos`` / ``sin`` differ in the last fp32 place for some arguments, which moves about one table entry in
+    a thousand to the neighbouring 16-bit value; with the host's tables a GPU layer and a CPU layer rotate with
+    identical factors"""
+    inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+    t = torch.arange(seq_len, dtype=torch.float32)
     freqs = torch.outer(t, inv_freq)
     emb = torch.cat((freqs, freqs), dim=-1)
-    return emb.cos().to(dtype), emb.sin().to(dtype)
+    return emb.cos().to(dtype).to(device), emb.sin().to(dtype).to(device)
 
 
 def causal_attention(q, k, v, mxint_bits=None, q_rope=None):

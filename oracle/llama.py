@@ -58,6 +58,23 @@ def head_rms_norm(x, weight, eps):
     return weight * x.to(dt)
 
 
+def eager_causal_attention(q, k, v, exact: bool = False):
+    """The attention core of the reference's unquantized Llama block on [batch, heads, tokens, head_dim] operands
+    (``chop/models/llama/modeling_llama.py:430-446``): ``matmul(q, k^T) / sqrt(head_dim)`` in the model dtype, the
+    additive causal mask, softmax in fp32, the probabilities cast back to the model dtype, ``matmul`` with v.
+    ``exact``: the same function evaluated in fp32 throughout with one rounding of the result (what the reference's
+    chain of roundings approximates); the distance between the two is the reference's own rounding noise."""
+    T, d = q.shape[-2], q.shape[-1]
+    dt = q.dtype
+    if exact:
+        q, k, v = q.float(), k.float(), v.float()
+    w = torch.matmul(q, k.transpose(2, 3)) / d ** 0.5
+    mask = torch.full((T, T), torch.finfo(w.dtype).min, dtype=w.dtype).triu(1)
+    w = w + mask
+    w = F.softmax(w, dim=-1, dtype=torch.float32).to(q.dtype)
+    return torch.matmul(w, v).to(dt)
+
+
 def attention_forward(kind, weights, hidden_states, cos, sin, attention_mask, n_heads, n_kv_heads, q_config,
                       past=None, qk_norm_eps=None):
     """weights: dict with q_proj/k_proj/v_proj/o_proj ``.weight`` (and optional ``.bias``) tensors.

@@ -7,13 +7,17 @@ so it is checked on a slice that is: the first 256 activation rows against the f
 the full-size operands (rows are independent in both quantizers and in the product), plus size-independent
 properties of the full-size result (finite, row slices agree with the sliced computation).
 Configuration 5 (decoder layer, batch 8 x seq 2048) runs at full size on the GPU; each of its seven Linears is checked
-on the first and the last 256 tokens against the oracle's forward of exactly the rows the GPU Linear was fed."""
+on the first and the last 256 tokens against the oracle's forward of exactly the rows the GPU Linear was fed; the
+attention kernel is checked inside the layer on two (batch, head) pairs against the tensor operations in fp32 at the
+full 2048 tokens; and the layer output rows of the first and last 256 tokens are compared with the CPU layer (oracle
+Linears) continued from the attention output the GPU produced for those tokens."""
 import pytest
 import torch
 
 import bench
 import oracle as O
 from oracle import linear as OL
+from oracle import llama as OLL
 from helpers import assert_bits_equal
 
 pytestmark = pytest.mark.gpu
@@ -112,15 +116,34 @@ def test_config5_decoder_layer_full_size_linear_slices(dev):
 
     hooks = [getattr(layer, n).register_forward_hook(hook(n)) for n in names]
     x = torch.randn(w.B, w.T, 4096, generator=torch.Generator().manual_seed(4)).bfloat16()
-    with torch.no_grad():
-        # the Linears are checked on the plain tensors they receive when each quantizes its own input; the layer as the
-        # benchmark runs it (RMSNorm and the SwiGLU product writing the quantized form) must give the same bits
-        layer.fuse_producers = False
-        y = layer(x.to(dev))
-        for h in hooks:
-            h.remove()
-        layer.fuse_producers = True
-        y_fused = layer(x.to(dev))
+    from mase_amd.quantizers import _ops
+
+    PAIRS = ((0, 0), (w.B - 1, 31))
+    attn_seen = []  # per call of the attention kernel: its options and, for PAIRS, operand and result slices
+    real_attention = _ops.attention_causal
+
+    def recording_attention(q, k, v, scaling=None, mxint_bits=None, q_rope=None):
+        out = real_attention(q, k, v, scaling, mxint_bits=mxint_bits, q_rope=q_rope)
+        sl = lambda t: [t[b:b + 1, h:h + 1] for b, h in PAIRS]
+        attn_seen.append(dict(mxint_bits=mxint_bits, q_rope=q_rope, q=sl(q), k=sl(k), v=sl(v), out=[t.clone() for t in sl(out)]))
+        return out
+
+    _ops.attention_causal = recording_attention
+    try:
+        with torch.no_grad():
+            layer.fuse_producers = False  # every Linear quantizes its own input; q rotated before the attention call
+            y = layer(x.to(dev))
+            for h in hooks:
+                h.remove()
+            layer.fuse_producers = True
+            y_fused = layer(x.to(dev))
+    finally:
+        _ops.attention_causal = real_attention
+    _check_config5_attention(attn_seen, w.T, dev)
+    _check_config5_rows_after_attention(w, x, y_fused, seen["o_proj"][0], S)
+    # the Linears are checked on the plain tensors they receive when each quantizes its own input; the layer as the
+    # benchmark runs it (RMSNorm, the SwiGLU product and the attention kernel writing the quantized form) must give the
+    # same bits
     assert torch.equal(y_fused.view(torch.int16), y.view(torch.int16))
     assert y.shape == x.shape and y.dtype == torch.bfloat16 and bool(torch.isfinite(y).all())
     assert len(seen) == 7
@@ -142,3 +165,54 @@ def test_config5_decoder_layer_full_size_linear_slices(dev):
               flush=True)
         assert e < 1e-2, n
         assert n_diff <= out.numel() * 1e-4 and (n_diff == 0 or int(step.max()) == 1), n
+
+
+def _check_config5_attention(attn_seen, T, dev):
+    """The two forwards of the layer called the attention kernel once each: plain (q rotated by rope() before the call)
+    and fused (q rotated on load, result in o_proj's MXINT8 form).  For each recorded (batch, head) pair, at the full
+    2048 tokens: the plain result against softmax(q k^T / sqrt(128) + causal mask) v in fp32 on the same bf16 operands,
+    bound 1e-2 of the result's range; the fused result bit for bit equal to the MXINT8 quantizer (CPU oracle) applied to
+    the plain kernel's result on the rotated q."""
+    from mase_amd.quantizers import _ops
+
+    assert len(attn_seen) == 2
+    plain, fused = attn_seen
+    assert plain["mxint_bits"] is None and plain["q_rope"] is None
+    assert fused["mxint_bits"] == 8 and fused["q_rope"] is not None
+    cos, sin = fused["q_rope"]
+    for i in range(len(plain["q"])):
+        q, k, v = plain["q"][i], plain["k"][i], plain["v"][i]
+        s = (q.float() @ k.float().transpose(-1, -2)) * 128 ** -0.5
+        s = s.masked_fill(torch.triu(torch.ones(T, T, dtype=torch.bool, device=dev), 1), float("-inf"))
+        ref = torch.softmax(s, -1) @ v.float()
+        e = float((plain["out"][i].float() - ref).abs().max() / ref.abs().max())
+        print(f"config 5 attention kernel inside the layer, pair {i}, {T} tokens: err {e:.3e} of the range vs fp32", flush=True)
+        assert e < 1e-2
+        # the fused call received q before its rotation: rope() of it is the q of the plain call
+        assert torch.equal(_ops.rope(fused["q"][i], cos, sin), q)
+        assert torch.equal(fused["k"][i], k) and torch.equal(fused["v"][i], v)
+        want = O.mxint_quantizer(plain["out"][i].transpose(1, 2).reshape(1, T, 128).cpu(), 32, 8, block_dim=-1)
+        assert_bits_equal(fused["out"][i].transpose(1, 2).reshape(1, T, 128), want, f"config 5 fused attention output, pair {i}")
+
+
+def _check_config5_rows_after_attention(w, x, y_gpu, attn_rows, S):
+    """Everything after the attention core is row-wise: the CPU layer (oracle Linears, torch's RMSNorm / SiLU
+    arithmetic) continued from the attention output the GPU layer produced for the first and last S tokens must give
+    the GPU layer's output rows for those tokens: max|y - y_ref| / max|y_ref| <= 1e-2."""
+    from test_decoder_layer_gpu import swap_in_oracle
+
+    cpu = swap_in_oracle(w.build(torch, None), w.cfg)
+    tok = w.B * w.T
+    xr = x.reshape(tok, -1)
+    xr = torch.cat((xr[:S], xr[-S:]))
+    with torch.no_grad():
+        h = xr + cpu.o_proj(attn_rows)
+        n = cpu.post_attention_layernorm(h)
+        ref = h + cpu.down_proj(torch.nn.functional.silu(cpu.gate_proj(n)) * cpu.up_proj(n))
+    yr = y_gpu.reshape(tok, -1)
+    got = torch.cat((yr[:S], yr[-S:])).cpu()
+    e = rel_err(got, ref)
+    n_diff = int((got.view(torch.int16) != ref.view(torch.int16)).sum())
+    print(f"config 5 layer output rows (first / last {S} tokens) vs the CPU layer continued from the GPU's attention "
+          f"output: rel err {e:.3e}, {n_diff} of {got.numel()} elements not bit-identical", flush=True)
+    assert e < 1e-2

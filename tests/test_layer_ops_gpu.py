@@ -199,7 +199,12 @@ def test_causal_attention_one_pass(dev, B, H, T, layout):
     ang = torch.rand(T, 64, generator=g) * 6.28
     emb = torch.cat((ang, ang), -1)
     cos, sin = emb.cos().bfloat16().to(dev), emb.sin().bfloat16().to(dev)
-    for tables in ((cos, sin), (cos[None].expand(B, T, 128).contiguous(), sin[None].expand(B, T, 128).contiguous() * 0.5)):
+    # per batch item: different angles for every item, so that a wrong batch stride of the tables shows
+    ang_b = ang[None] * (1.0 + 0.37 * torch.arange(B)[:, None, None])
+    emb_b = torch.cat((ang_b, ang_b), -1)
+    per_item = (emb_b.cos().bfloat16().to(dev), (emb_b.sin() * 0.5).bfloat16().to(dev))
+    assert B == 1 or not torch.equal(per_item[0][0], per_item[0][1])
+    for tables in ((cos, sin), per_item):
         assert _ops.rope_supported(q, *tables)
         want = _ops.attention_causal(_ops.rope(q, *tables), k, v)
         assert torch.equal(_ops.attention_causal(q, k, v, q_rope=tables), want)

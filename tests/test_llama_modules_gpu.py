@@ -296,8 +296,9 @@ def test_attention_module_one_pass_and_separate_passes_agree(dev):
     cos, sin = (t.to(dev) for t in rope_tables(B, S, CFG.head_dim, torch.bfloat16))
     mask = causal_mask(B, S, S, torch.bfloat16).to(dev)
     with torch.no_grad():
+        m.fused_probabilities = True
         y1, w1 = m(x, (cos, sin), mask)
-        m.fused_probabilities = False
+        m.fused_probabilities = False  # the default
         y0, w0 = m(x, (cos, sin), mask)
     assert float((w1.float() - w0.float()).abs().max()) <= 2 ** -7
     assert float((w1 == w0).float().mean()) > 0.99
