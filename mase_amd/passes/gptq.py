@@ -1,335 +1,271 @@
-"""GPTQ weight optimisation in front of the quantize pass, with the contract of the reference's
-``chop/passes/module/transforms/gptq/`` (``gptq.py:16-128`` the algorithm, ``quantize_dispatch.py:36-82`` the quantizer
-dispatch, ``utils.py:7-18`` the layer search, ``run.py:20-232`` the driver over a causal LM's decoder layers).
+"""Second-order weight rounding (GPTQ) in front of the quantize pass.
 
-The algorithm per ``nn.Linear``: accumulate H = 2/n * sum x x^T over the calibration inputs, damp its diagonal, take
-the upper Cholesky factor U of H^-1, then walk the columns in groups of ``weight_block_size``: quantize the group
-(``quantile_search`` clip search of the MX quantizers, one MX block per row and group), divide the quantization error
-by U's diagonal and subtract its product with U's off-diagonal rows from the columns still to come.  The quantizer
-calls are the device kernels of this package (``mase_mxint_clip_search`` / ``mase_mxfp_clip_search`` or the plain
-quantize-dequantize kernels); the Hessian, its factorisations and the rank-32 updates are library calls on the same
-device.  Weights are written back into the ``nn.Linear`` modules, so that the quantize pass that follows finds them
-(its ``LinearMX*`` replacements are configured with ``gptq=True`` and do not quantize again).
+Contract kept from the reference (``chop/passes/module/transforms/gptq/run.py:20-60``, called from
+``passes/module/transforms/quantize/quantize.py:134-138``): ``run_gptq(network, gptq_config)`` takes a causal LM with
+``network.model.layers`` and the keys ``device``, ``format`` ("mxint" | "mxfp"), ``weight_config`` (the MASE weight
+keys), ``quantile_search``, ``clip_search_y``, ``cali_batch_size``, ``max_layers``; it rewrites the weights of the
+``nn.Linear`` modules of the decoder layers in place and returns the network, whose modules the quantize pass then
+swaps for ``LinearMX*`` configured with ``gptq=True`` (they do not quantize the weights again).  Calibration token ids
+come in as ``gptq_config["calibration_data"]`` (``[samples, tokens]`` integers, or a list of ``[1, tokens]``): there
+is no dataset download here.
 
-Differences from the reference's driver: calibration token ids are passed in (``gptq_config["calibration_data"]``, an
-integer tensor ``[nsamples, seqlen]`` or a list of ``[1, seqlen]`` tensors) instead of being downloaded by dataset
-name.  ``clip_search_y`` scores the clip search of each column group on the group's calibration inputs
-(``mase_mx*_clip_candidates`` plus matrix products).  ``checkpoint_dir`` writes one safetensors file (and a JSON
-description) per finished decoder layer and resumes after the last layer found there, with the reference's file names
-(``checkpoint.py:9-135``); like the reference's driver, a resumed run calibrates its first layer on the inputs of
-layer 0 unless ``resume_propagate`` is set, which first runs those inputs through the layers that were loaded.
+What is computed (the algorithm of ``gptq/gptq.py:16-128`` for block formats): for a Linear with weight W [out, in] and
+calibration inputs X, with G = sum x x^T, damped by 1 % of its mean diagonal, and U the upper Cholesky factor of
+G^-1, the input columns are walked in groups of ``weight_block_size``; a group is quantized as a whole (one MX block
+per row, optionally with the clip search), its error divided by U's diagonal and fed forward into the columns not yet
+quantized through U's rows.  The scale of G does not matter (the damping is relative and U's scale cancels in
+``error / diag(U) @ U``), so G is kept as the plain sum.
+
+How it is organised here:
+
+* One Gram matrix per distinct input tensor.  Projections that read the same tensor (q / k / v; gate / up) are hooked
+  together, the hook recognises the shared tensor and its Gram matrix is accumulated once, with one ``addmm_`` per
+  sample, and factored once.
+* The feed-forward of the error is blocked on two levels: inside a panel of ``PANEL_GROUPS`` column groups the update
+  reaches the rest of the panel only; the columns behind the panel receive the panel's accumulated errors in one
+  ``addmm_`` ([out, panel] x [panel, rest]).  Same sums, fewer and larger products.
+* The working copy of W is fp32 whatever the weight dtype; each group is handed to the quantizer in the weight's
+  dtype, which is what the modules' own quantizer would see.
+* The quantizers are this package's device kernels (``mase_mx*_clip_search``, ``mase_mx*_qdq``, and with
+  ``clip_search_y`` the candidate kernels scored on the group's calibration inputs).
+* The first decoder layer's inputs are recorded by a forward pre-hook that stops the forward; every later call of a
+  layer replays the keyword arguments recorded there (mask, positions, rotary tables), whatever the model passes.
 """
 from __future__ import annotations
 
-import json
 import logging
-import math
-import os
-import re
+from typing import Callable, Sequence
 
 import torch
 from torch import Tensor, nn
 
 from ..quantizers import MXFPMeta, MXIntMeta, mxfp_quantizer_sim, mxint_quantizer_sim
 
+log = logging.getLogger(__name__)
 
-def quantize_tensor(input: Tensor, block_dim: int, fmt: str, config: dict, quantile_search: bool,
-                    act_tensor: Tensor | None = None, dtype: torch.dtype | None = None,
-                    cali_batch_size: int = 32) -> Tensor:
-    """quantize_dispatch.py:36-82"""
-    if fmt == "mxfp":
-        meta = MXFPMeta(block_size=config["weight_block_size"], scale_exp_bits=8,
-                        element_exp_bits=config["weight_exponent_width"], element_frac_bits=config["weight_frac_width"],
-                        element_is_finite=True, round_mode="rn")
-        return mxfp_quantizer_sim(input, block_dim=block_dim, mxfp_meta=meta, act_tensor=act_tensor, dtype=dtype,
-                                  quantile_search=quantile_search, cali_batch_size=cali_batch_size)
-    if fmt == "mxint":
-        meta = MXIntMeta(block_size=config["weight_block_size"], scale_bits=8, element_bits=config["weight_width"])
-        return mxint_quantizer_sim(input, block_dim=block_dim, mxint_meta=meta, act_tensor=act_tensor, dtype=dtype,
-                                   quantile_search=quantile_search, cali_batch_size=cali_batch_size)
-    raise ValueError(f"Unsupported GPTQ format: {fmt}. Use 'mxfp' or 'mxint'.")
+PANEL_GROUPS = 4       # column groups per panel of the blocked error feed-forward
+RELATIVE_DAMPING = 0.01
 
-
-def find_qlayers(module, layers=(nn.Linear,), name=""):
-    """utils.py:7-18: {dotted name: module} of the sub-modules whose type is one of ``layers``"""
-    if type(module) in tuple(layers):
-        return {name: module}
-    found = {}
-    for child_name, child in module.named_children():
-        found.update(find_qlayers(child, layers=layers, name=f"{name}.{child_name}" if name != "" else child_name))
-    return found
-
-
-class GPTQ:
-    """gptq.py:16-128"""
-
-    def __init__(self, layer):
-        self.layer = layer
-        self.dev = layer.weight.device
-        self.rows, self.columns = layer.weight.shape
-        self.H = torch.zeros((self.columns, self.columns), device=self.dev)
-        self.nsamples = 0
-
-    def add_batch(self, inp, out=None):
-        """gptq.py:27-37: running mean of 2 * x x^T over the samples seen"""
-        if inp.dim() == 2:
-            inp = inp.unsqueeze(0)
-        n = inp.shape[0]
-        if inp.dim() == 3:
-            inp = inp.reshape(-1, inp.shape[-1])
-        inp = inp.t()
-        self.H *= self.nsamples / (self.nsamples + n)
-        self.nsamples += n
-        inp = math.sqrt(2 / self.nsamples) * inp.float()
-        self.H += inp.matmul(inp.t())
-
-    def inverse_factor(self, percdamp: float = 0.01):
-        """gptq.py:65-78: columns that never fired are pinned, the diagonal damped by ``percdamp`` of its mean, and the
-        upper Cholesky factor of H^-1 returned; consumes ``self.H``"""
-        H = self.H
-        del self.H
-        dead = torch.diag(H) == 0
-        H[dead, dead] = 1
-        damp = percdamp * torch.mean(torch.diag(H))
-        diag = torch.arange(self.columns, device=self.dev)
-        H[diag, diag] += damp
-        H = torch.linalg.cholesky(H)
-        H = torch.cholesky_inverse(H)
-        return torch.linalg.cholesky(H, upper=True), dead
-
-    def fasterquant(self, activation, fmt, weight_config, percdamp=0.01, cali_batch_size=32, layer_name=None,
-                    quant_search=True):
-        """gptq.py:39-122"""
-        W = self.layer.weight.data.clone()
-        Hinv, dead = self.inverse_factor(percdamp)
-        W[:, dead] = 0
-        Q = torch.zeros_like(W)
-        blocksize = weight_config["weight_block_size"]
-        for i1 in range(0, self.columns, blocksize):
-            i2 = min(i1 + blocksize, self.columns)
-            W1 = W[:, i1:i2].clone()
-            # clip_search_y: the group's search is scored on the layer's calibration inputs of these columns
-            act1 = None if activation is None else activation[:, :, i1:i2].clone()
-            Q1 = quantize_tensor(W1, block_dim=1, fmt=fmt, config=weight_config, quantile_search=quant_search,
-                                 act_tensor=act1, cali_batch_size=cali_batch_size)
-            Q[:, i1:i2] = Q1
-            if i2 < self.columns:
-                err = (W1 - Q1) / torch.diag(Hinv[i1:i2, i1:i2]).unsqueeze(0)
-                W[:, i2:] -= err.matmul(Hinv[i1:i2, i2:])
-        assert Q.shape == W.shape, f"Shape mismatch: {Q.shape} != {W.shape}"
-        return Q
-
-    def free(self):
-        self.H = None
-
-
-_SEQUENTIAL = (  # run.py:136-141
-    ("self_attn.k_proj", "self_attn.v_proj", "self_attn.q_proj"),
+# projections of a decoder layer in the order they are rounded; members of one entry read the same tensor, and an
+# entry sees the outputs of the already rounded entries before it
+PROJECTION_GROUPS = (
+    ("self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj"),
     ("self_attn.o_proj",),
-    ("mlp.up_proj", "mlp.gate_proj"),
+    ("mlp.gate_proj", "mlp.up_proj"),
     ("mlp.down_proj",),
 )
 
 
+def group_quantizer(fmt: str, weight_config: dict, search: bool, cali_batch_size: int = 32) -> Callable:
+    """``f(w_group [out, block], calibration [samples, tokens, block] | None) -> quantize-dequantize of the group``, one
+    MX block per row (the dispatch of ``gptq/quantize_dispatch.py:36-82`` on the weight keys of the MASE config)"""
+    block = weight_config["weight_block_size"]
+    if fmt == "mxint":
+        meta = MXIntMeta(block_size=block, scale_bits=8, element_bits=weight_config["weight_width"])
+        sim = mxint_quantizer_sim
+        kw = {"mxint_meta": meta}
+    elif fmt == "mxfp":
+        meta = MXFPMeta(block_size=block, scale_exp_bits=8, element_exp_bits=weight_config["weight_exponent_width"],
+                        element_frac_bits=weight_config["weight_frac_width"], element_is_finite=True, round_mode="rn")
+        sim = mxfp_quantizer_sim
+        kw = {"mxfp_meta": meta}
+    else:
+        raise ValueError(f"gptq: format {fmt!r} is not one of 'mxint', 'mxfp'")
+
+    def quantize(w_group: Tensor, calibration: Tensor | None = None) -> Tensor:
+        return sim(w_group, block_dim=1, act_tensor=calibration if search else None, quantile_search=search,
+                   cali_batch_size=cali_batch_size, **kw)
+
+    return quantize
+
+
+class InputGram:
+    """sum of x x^T over the rows of every tensor handed to ``update`` (fp32, on the tensor's device), and optionally
+    the tensors themselves for a clip search scored on calibration inputs"""
+
+    def __init__(self, keep_inputs: bool = False):
+        self.matrix: Tensor | None = None
+        self.rows_seen = 0
+        self.inputs: list[Tensor] | None = [] if keep_inputs else None
+
+    def update(self, x: Tensor) -> None:
+        rows = x.detach().reshape(-1, x.shape[-1]).float()
+        if self.matrix is None:
+            self.matrix = torch.zeros(rows.shape[1], rows.shape[1], dtype=torch.float32, device=rows.device)
+        self.matrix.addmm_(rows.t(), rows)
+        self.rows_seen += rows.shape[0]
+        if self.inputs is not None:
+            self.inputs.append(x.detach().reshape(1, -1, x.shape[-1]) if x.dim() <= 2 else x.detach())
+
+    def calibration(self) -> Tensor | None:
+        return None if self.inputs is None else torch.cat(self.inputs, dim=0)
+
+
+def inverse_cholesky_upper(gram: Tensor, relative_damping: float = RELATIVE_DAMPING):
+    """(U, dead): U upper triangular with U^T U = (G + damping)^-1 where input columns that never fired (``dead``) are
+    given a unit diagonal first"""
+    G = gram.clone()
+    d = torch.diagonal(G)
+    dead = d == 0
+    d[dead] = 1.0
+    d += relative_damping * d.mean()
+    L = torch.linalg.cholesky(G)
+    return torch.linalg.cholesky(torch.cholesky_inverse(L), upper=True), dead
+
+
+def round_weight(weight: Tensor, gram: Tensor, group_size: int, quantize: Callable, calibration: Tensor | None = None,
+                 relative_damping: float = RELATIVE_DAMPING, panel_groups: int = PANEL_GROUPS) -> Tensor:
+    """The rounded weight, in ``weight``'s dtype.  ``quantize(w_group, calibration_group)`` rounds one column group;
+    ``calibration`` [samples, tokens, in] is sliced to the group's columns for it."""
+    out_features, in_features = weight.shape
+    U, dead = inverse_cholesky_upper(gram, relative_damping)
+    W = weight.detach().float().clone()
+    W[:, dead] = 0.0
+    Q = torch.empty_like(weight)
+    inv_diag = 1.0 / torch.diagonal(U)
+    panel = group_size * panel_groups
+    for p0 in range(0, in_features, panel):
+        p1 = min(p0 + panel, in_features)
+        scaled_err = torch.empty(out_features, p1 - p0, dtype=torch.float32, device=W.device)
+        for c0 in range(p0, p1, group_size):
+            c1 = min(c0 + group_size, p1)
+            cal = None if calibration is None else calibration[:, :, c0:c1].contiguous()
+            q = quantize(W[:, c0:c1].to(weight.dtype).contiguous(), cal)
+            Q[:, c0:c1] = q
+            e = (W[:, c0:c1] - q.float()) * inv_diag[c0:c1]
+            scaled_err[:, c0 - p0:c1 - p0] = e
+            if c1 < p1:  # the rest of this panel sees the group's error now
+                W[:, c1:p1].addmm_(e, U[c0:c1, c1:p1], alpha=-1.0)
+        if p1 < in_features:  # everything behind the panel sees the panel's errors in one product
+            W[:, p1:].addmm_(scaled_err, U[p0:p1, p1:], alpha=-1.0)
+    return Q
+
+
+def linear_modules(module: nn.Module) -> dict[str, nn.Linear]:
+    """{dotted name: module} of the plain ``nn.Linear`` sub-modules (subclasses, e.g. already swapped ones, excluded)"""
+    return {name: m for name, m in module.named_modules() if type(m) is nn.Linear}
+
+
 @torch.no_grad()
-def gptq_decoder_layer(layer, run_layer, nsamples: int, fmt: str, weight_config: dict, quantile_search: bool = True,
-                       cali_batch_size: int = 32, sequential=_SEQUENTIAL, layer_name: str = "",
-                       clip_search_y: bool = False):
-    """The per-layer body of run.py:150-214: for each group of projections in ``sequential``, run the layer over the
-    ``nsamples`` calibration samples (``run_layer(j)`` runs sample j through ``layer``) with hooks that feed each
-    projection's inputs to its GPTQ object, then quantize those projections and write the weights back.
-    ``clip_search_y``: the inputs of the group (its projections share them; recorded at the last one, run.py:173) are
-    kept as [nsamples, tokens, columns] and the clip search of every column group is scored on them."""
-    full = find_qlayers(layer, layers=[nn.Linear])
-    for names in sequential:
-        subset = {n: full[n] for n in names if n in full}
-        if not subset:
+def round_decoder_layer(layer: nn.Module, forward_sample: Callable[[int], object], n_samples: int, quantize: Callable,
+                        group_size: int, score_on_inputs: bool = False,
+                        projection_groups: Sequence[Sequence[str]] = PROJECTION_GROUPS) -> list[str]:
+    """Rounds the Linears of one decoder layer, one entry of ``projection_groups`` after the other: run the layer over
+    the calibration samples (``forward_sample(j)``) with pre-hooks collecting the Gram matrix of each distinct input
+    tensor of the entry, then rewrite the entry's weights.  Linears not named in ``projection_groups`` are left alone.
+    Returns the names rewritten."""
+    found = linear_modules(layer)
+    done = []
+    for entry in projection_groups:
+        members = [(n, found[n]) for n in entry if n in found]
+        if not members:
             continue
-        gptq = {n: GPTQ(m) for n, m in subset.items()}
+        gram_of: dict[str, InputGram] = {}
+        # within one forward: id of an input tensor -> (the tensor, kept alive so that the id stays its own; its Gram)
+        accounted: dict[int, tuple[Tensor, InputGram]] = {}
 
-        def hook(name):
-            def fn(_, inp, out):
-                gptq[name].add_batch(inp[0].data, out.data)
-            return fn
+        def collect(name):
+            def pre_hook(_module, args):
+                x = args[0]
+                hit = accounted.get(id(x))
+                if hit is None:  # the first member to read this tensor in this forward accumulates it
+                    gram = gram_of.setdefault(name, InputGram(keep_inputs=score_on_inputs))
+                    gram.update(x)
+                    accounted[id(x)] = (x, gram)
+                elif gram_of.setdefault(name, hit[1]) is not hit[1]:
+                    raise RuntimeError(f"gptq: {name} shares its input with a sibling in some calibration samples only")
+            return pre_hook
 
-        handles = [m.register_forward_hook(hook(n)) for n, m in subset.items()]
-        pre_act = []
-        if clip_search_y:
-            last = list(subset.values())[-1]
-            handles.append(last.register_forward_pre_hook(lambda _, inp: pre_act.append(inp[0])))
+        handles = [m.register_forward_pre_hook(collect(n)) for n, m in members]
         try:
-            for j in range(nsamples):
-                run_layer(j)
+            for j in range(n_samples):
+                accounted.clear()
+                forward_sample(j)
         finally:
             for h in handles:
                 h.remove()
-        activation = torch.cat(pre_act, dim=0) if clip_search_y else None
-        for n, m in subset.items():
-            q = gptq[n].fasterquant(activation=activation, fmt=fmt, weight_config=weight_config, percdamp=0.01,
-                                    cali_batch_size=cali_batch_size, layer_name=f"{layer_name}.{n}",
-                                    quant_search=quantile_search)
-            assert q.shape == m.weight.shape
-            m.weight.data.copy_(q)
-            gptq[n].free()
+        accounted.clear()
+        for name, m in members:
+            gram = gram_of[name]
+            cal = gram.calibration() if score_on_inputs else None
+            m.weight.data.copy_(round_weight(m.weight.data, gram.matrix, group_size, quantize, cal))
+            done.append(name)
+    return done
 
 
-def _calibration_batches(gptq_config):
+class _StopForward(Exception):
+    """raised by the recording hook once the first decoder layer's inputs are known"""
+
+
+def _samples(gptq_config) -> list[Tensor]:
     data = gptq_config.get("calibration_data")
     if data is None:
         raise NotImplementedError(
-            "run_gptq: pass the calibration token ids as gptq_config['calibration_data'] ([nsamples, seqlen] or a list "
-            "of [1, seqlen] tensors); loading a dataset by name needs a network connection and is not built")
+            "run_gptq: pass the calibration token ids as gptq_config['calibration_data'] ([samples, tokens] or a list "
+            "of [1, tokens] tensors); loading a dataset by name needs a network connection and is not built")
     if isinstance(data, Tensor):
-        return [row.unsqueeze(0) for row in data]
-    return [d if d.dim() == 2 else d.unsqueeze(0) for d in data]
-
-
-_CKPT_MODEL_NAME = "quantized_model"
-
-
-def _layer_file(checkpoint_dir: str, layer_idx: int) -> str:
-    return os.path.join(checkpoint_dir, f"{_CKPT_MODEL_NAME}_layer_{layer_idx}.safetensors")
-
-
-def save_layer_checkpoint(network, layer_idx: int, checkpoint_dir: str | None) -> None:
-    """checkpoint.py:9-72: the parameters of decoder layer ``layer_idx`` under their names relative to the layer, in
-    ``<dir>/quantized_model_layer_<i>.safetensors``, and a JSON description beside it"""
-    if checkpoint_dir is None:
-        return
-    from safetensors.torch import save_file
-
-    os.makedirs(checkpoint_dir, exist_ok=True)
-    prefix = f"model.layers.{layer_idx}."
-    tensors = {name[len(prefix):]: p.detach().cpu().contiguous() for name, p in network.named_parameters()
-               if name.startswith(prefix)}
-    if not tensors:
-        logging.warning(f"No parameters found for layer {layer_idx} with prefix {prefix}")
-        return
-    path = _layer_file(checkpoint_dir, layer_idx)
-    save_file(tensors, path)
-    meta = {"layer_idx": layer_idx, "total_layers": len(network.model.layers), "checkpoint_file": path,
-            "model_name": _CKPT_MODEL_NAME, "num_parameters": len(tensors), "parameter_names": list(tensors)}
-    with open(os.path.join(checkpoint_dir, f"{_CKPT_MODEL_NAME}_layer_{layer_idx}_metadata.json"), "w") as f:
-        json.dump(meta, f, indent=2)
-
-
-def detect_quantized_layers(checkpoint_dir: str | None) -> dict:
-    """checkpoint.py:75-91: {layer index: file} of the layer files present"""
-    found = {}
-    if checkpoint_dir is None or not os.path.isdir(checkpoint_dir):
-        return found
-    pat = re.compile(rf"^{_CKPT_MODEL_NAME}_layer_(\d+)\.safetensors$")
-    for fn in os.listdir(checkpoint_dir):
-        m = pat.match(fn)
-        if m:
-            found[int(m.group(1))] = os.path.join(checkpoint_dir, fn)
-    return found
-
-
-def auto_load_quantized_layers(network, checkpoint_dir: str | None) -> int:
-    """checkpoint.py:94-135: loads the layer files in ascending order of their index, stops at the first that fails,
-    returns the last index loaded (-1: none)"""
-    from safetensors.torch import load_file
-
-    last = -1
-    for idx, path in sorted(detect_quantized_layers(checkpoint_dir).items()):
-        try:
-            state = {f"model.layers.{idx}.{k}": v for k, v in load_file(path).items()}
-            network.load_state_dict(state, strict=False)
-        except Exception as e:  # a damaged file ends the resume, as in the reference
-            logging.warning(f"Failed to load layer {idx} ({e}), stopping auto-load")
-            break
-        last = idx
-    return last
+        return [row.reshape(1, -1) for row in data]
+    return [d.reshape(1, -1) for d in data]
 
 
 @torch.no_grad()
 def run_gptq(network, gptq_config):
-    """run.py:20-232 for a ``transformers`` causal LM with ``network.model.layers`` / ``embed_tokens`` / ``norm`` /
-    ``rotary_emb``: GPTQ over every ``nn.Linear`` of every decoder layer, layer by layer, the inputs of layer i+1 being
-    the outputs of the already quantized layer i.  Keys of ``gptq_config`` as in the reference (``device``, ``format``,
-    ``weight_config``, ``quantile_search``, ``clip_search_y``, ``cali_batch_size``, ``max_layers``) plus
-    ``calibration_data``."""
-    clip_search_y = gptq_config.get("clip_search_y", False)
-    checkpoint_dir = gptq_config.get("checkpoint_dir", None)
-    start_layer = 0
-    if checkpoint_dir is not None:  # run.py:64-74
-        start_layer = auto_load_quantized_layers(network, checkpoint_dir) + 1
-        if start_layer:
-            logging.info(f"Resuming GPTQ from layer {start_layer}")
-        if start_layer == len(network.model.layers):
-            logging.info("All layers already quantized, skipping GPTQ")
-            return network
-    dev = gptq_config.get("device", "cuda:0")
-    fmt = gptq_config["format"]
+    """See the module docstring.  Decoder layers are processed in order; layer i + 1 is calibrated on the outputs of the
+    already rounded layer i."""
+    dev = torch.device(gptq_config.get("device", "cuda:0"))
     weight_config = gptq_config["weight_config"]
-    quantile_search = gptq_config.get("quantile_search", True)
-    cali_batch_size = gptq_config.get("cali_batch_size", 32)
-    max_layers = gptq_config.get("max_layers", None)
-    batches = _calibration_batches(gptq_config)
-    nsamples = len(batches)
-    seqlen = batches[0].shape[-1]
+    score_on_inputs = bool(gptq_config.get("clip_search_y", False))
+    quantize = group_quantizer(gptq_config["format"], weight_config, bool(gptq_config.get("quantile_search", True)),
+                               gptq_config.get("cali_batch_size", 32))
+    samples = _samples(gptq_config)
+    decoder = network.model.layers
+    n_layers = len(decoder) if gptq_config.get("max_layers") is None else min(len(decoder), gptq_config["max_layers"])
 
-    use_cache = network.config.use_cache
-    network.config.use_cache = False
-    layers = network.model.layers
-    network.model.embed_tokens = network.model.embed_tokens.to(dev)
-    network.model.norm = network.model.norm.to(dev)
-    rope = network.model.rotary_emb.to(dev)
-    layers[0] = layers[0].to(dev)
-    dtype = next(iter(network.parameters())).dtype
-    inps = torch.zeros((nsamples, seqlen, network.config.hidden_size), dtype=dtype, device=dev)
-    cache = {"i": 0, "attention_mask": None, "position_ids": None}
+    # what the first decoder layer receives for every sample: positional hidden states + keyword arguments
+    hidden, call_kwargs = [], {}
 
-    class Catcher(nn.Module):  # run.py:108-118: records what the first decoder layer receives
-        def __init__(self, module):
-            super().__init__()
-            self.module = module
+    def record(_module, args, kwargs):
+        hidden.append(args[0] if args else kwargs["hidden_states"])
+        call_kwargs.clear()
+        call_kwargs.update({k: v for k, v in kwargs.items() if k != "hidden_states"})
+        raise _StopForward
 
-        def forward(self, inp, **kwargs):
-            inps[cache["i"]] = inp
-            cache["i"] += 1
-            cache["attention_mask"] = kwargs.get("attention_mask")
-            cache["position_ids"] = kwargs.get("position_ids")
-            raise ValueError
+    cache_setting = getattr(network.config, "use_cache", None)
+    if cache_setting is not None:
+        network.config.use_cache = False
+    network.to(dev)
+    handle = decoder[0].register_forward_pre_hook(record, with_kwargs=True)
+    try:
+        for ids in samples:
+            try:
+                network(ids.to(dev))
+            except _StopForward:
+                pass
+    finally:
+        handle.remove()
+    if len(hidden) != len(samples):
+        raise RuntimeError("gptq: the first decoder layer was not reached for every calibration sample")
+    call_kwargs.pop("past_key_values", None)
+    call_kwargs.pop("past_key_value", None)
+    if "use_cache" in call_kwargs:
+        call_kwargs["use_cache"] = False
 
-    layers[0] = Catcher(layers[0])
-    for batch in batches:
-        try:
-            network(batch.to(dev))
-        except ValueError:
-            pass
-    layers[0] = layers[0].module
-    outs = torch.zeros_like(inps)
-    attention_mask, position_ids = cache["attention_mask"], cache["position_ids"]
-    if position_ids is None:
-        position_ids = torch.arange(seqlen, device=dev).unsqueeze(0)
+    log.info("gptq: %d decoder layers, %d calibration samples of %d tokens, format %s", n_layers, len(samples),
+             samples[0].shape[-1], gptq_config["format"])
+    for index in range(n_layers):
+        layer = decoder[index]
+        outputs: list = [None] * len(samples)
 
-    end_layer = len(layers) if max_layers is None else min(start_layer + max_layers, len(layers))
-    logging.info(f"GPTQ: quantizing layers {start_layer} to {end_layer - 1} (of {len(layers)} total)")
-    if start_layer and gptq_config.get("resume_propagate", False):
-        for i in range(start_layer):  # the loaded layers' outputs, not layer 0's inputs, feed the first new layer
-            layer = layers[i].to(dev)
-            for j in range(nsamples):
-                x = inps[j].unsqueeze(0)
-                cos, sin = rope(x, position_ids)
-                out = layer(x, attention_mask=attention_mask, position_embeddings=(cos, sin))
-                outs[j] = out[0] if isinstance(out, tuple) else out
-            inps, outs = outs, inps
-    for i in range(start_layer, end_layer):
-        layer = layers[i].to(dev)
+        def forward_sample(j, layer=layer, outputs=outputs):
+            y = layer(hidden[j], **call_kwargs)
+            outputs[j] = y[0] if isinstance(y, (tuple, list)) else y
 
-        def run_layer(j, layer=layer):
-            x = inps[j].unsqueeze(0)
-            cos, sin = rope(x, position_ids)
-            out = layer(x, attention_mask=attention_mask, position_embeddings=(cos, sin))
-            outs[j] = out[0] if isinstance(out, tuple) else out
-
-        gptq_decoder_layer(layer, run_layer, nsamples, fmt, weight_config, quantile_search, cali_batch_size,
-                           layer_name=f"layers{i}", clip_search_y=clip_search_y)
-        for j in range(nsamples):  # run.py:197-205: the quantized layer's outputs feed the next layer
-            run_layer(j)
-        inps, outs = outs, inps
-        save_layer_checkpoint(network, i, checkpoint_dir)
-    network.config.use_cache = use_cache
+        names = round_decoder_layer(layer, forward_sample, len(samples), quantize, weight_config["weight_block_size"],
+                                    score_on_inputs)
+        for j in range(len(samples)):  # the rounded layer's outputs are the next layer's calibration inputs
+            forward_sample(j)
+        hidden = outputs
+        log.info("gptq: layer %d rounded (%s)", index, ", ".join(names))
+    if cache_setting is not None:
+        network.config.use_cache = cache_setting
     return network
