@@ -382,35 +382,82 @@ def test_layer_op_entry_points_reject_bad_arguments_without_a_gpu(lib):
     assert s(p, p, p, 64, 1, 4, 12, 1, 0, None) == -5
 
 
-def test_gptq_layer_checkpoint_files(tmp_path):
-    """the per-layer files of the GPTQ driver: names, contents, detection, loading in ascending order up to the first gap
-    or damaged file (host logic only)"""
-    import json
-
-    from safetensors.torch import load_file
+def test_gptq_host_logic_with_a_toy_quantizer():
+    """The parts of the GPTQ pass that run on any device, with a stand-in quantizer (round to a grid of 1/4): the
+    Cholesky factor satisfies U^T U = (G + damping)^-1; with a diagonal Gram matrix the result is plain rounding; with
+    correlated inputs the output error on the calibration inputs tr(E G E^T) is below plain rounding's; the blocked
+    feed-forward equals the group-by-group one; a dead input column comes out as zeros; and projections that read one
+    tensor share one Gram matrix, fed once per sample."""
     from torch import nn
 
-    from mase_amd.passes.gptq import auto_load_quantized_layers, detect_quantized_layers, save_layer_checkpoint
+    from mase_amd.passes import gptq as GP
 
-    class Net(nn.Module):
+    g = torch.Generator().manual_seed(11)
+    grid = lambda w, cal=None: torch.round(w * 4) / 4
+    x = torch.randn(512, 64, generator=g) @ (torch.randn(64, 64, generator=g) * 0.4 + torch.eye(64))
+    x[:, 5] = 0.0
+    gram = GP.InputGram()
+    gram.update(x[:256].reshape(2, 128, 64))
+    gram.update(x[256:])
+    assert gram.rows_seen == 512
+    G = (x.double().t() @ x.double()).float()
+    assert float((gram.matrix - G).abs().max() / G.abs().max()) < 1e-5
+    U, dead = GP.inverse_cholesky_upper(gram.matrix)
+    assert dead.tolist() == [i == 5 for i in range(64)]
+    Gd = G.double().clone()
+    Gd[5, 5] = 1.0
+    Gd += 0.01 * torch.diagonal(Gd).mean() * torch.eye(64, dtype=torch.float64)
+    assert float(((U.double().t() @ U.double()) @ Gd - torch.eye(64, dtype=torch.float64)).abs().max()) < 1e-3
+    assert bool((torch.tril(U, -1) == 0).all())
+
+    w = torch.randn(24, 64, generator=g)
+    loss = lambda q: float((((w - q).double() @ G.double()) * (w - q).double()).sum())
+    q = GP.round_weight(w, gram.matrix, 8, grid)
+    assert bool((q[:, 5] == 0).all())
+    assert torch.equal(q * 4, torch.round(q * 4))              # on the quantizer's grid
+    live = [0, 1, 2, 3, 4, 6, 7]
+    assert torch.equal(q[:, live], grid(w[:, live]))           # the first group has seen no feed-forward
+    assert loss(q) < 0.8 * loss(grid(w))
+    q1 = GP.round_weight(w, gram.matrix, 8, grid, panel_groups=1)
+    q8 = GP.round_weight(w, gram.matrix, 8, grid, panel_groups=8)
+    assert float((q == q1).float().mean()) > 0.995 and float((q == q8).float().mean()) > 0.995
+    diag = torch.diag(torch.rand(64, generator=g) + 0.5)
+    assert torch.equal(GP.round_weight(w, diag, 8, grid), grid(w))   # uncorrelated inputs: nothing to feed forward
+
+    class Block(nn.Module):
         def __init__(self):
             super().__init__()
-            self.model = nn.Module()
-            self.model.layers = nn.ModuleList([nn.Linear(4, 4) for _ in range(4)])
+            self.self_attn = nn.Module()
+            self.mlp = nn.Module()
+            for name in ("q_proj", "k_proj", "v_proj", "o_proj"):
+                setattr(self.self_attn, name, nn.Linear(16, 16, bias=False))
+            self.mlp.gate_proj, self.mlp.up_proj, self.mlp.down_proj = (nn.Linear(16, 32, bias=False), nn.Linear(16, 32, bias=False),
+                                                                        nn.Linear(32, 16, bias=False))
+            self.other = nn.Linear(16, 16)  # not named in PROJECTION_GROUPS: left alone
 
-    torch.manual_seed(0)
-    a, b = Net(), Net()
-    d = str(tmp_path / "ckpt")
-    assert detect_quantized_layers(d) == {} and auto_load_quantized_layers(b, d) == -1
-    for i in (0, 1, 3):
-        save_layer_checkpoint(a, i, d)
-    save_layer_checkpoint(a, 2, None)  # no directory: nothing is written
-    assert sorted(detect_quantized_layers(d)) == [0, 1, 3]
-    meta = json.load(open(f"{d}/quantized_model_layer_1_metadata.json"))
-    assert meta["layer_idx"] == 1 and meta["total_layers"] == 4 and meta["parameter_names"] == ["weight", "bias"]
-    assert torch.equal(load_file(f"{d}/quantized_model_layer_3.safetensors")["weight"], a.model.layers[3].weight)
-    with open(f"{d}/quantized_model_layer_1.safetensors", "wb") as f:
-        f.write(b"not a safetensors file")
-    assert auto_load_quantized_layers(b, d) == 0  # layer 1 is damaged: the resume stops there, as in the reference
-    assert torch.equal(b.model.layers[0].weight, a.model.layers[0].weight)
-    assert not torch.equal(b.model.layers[3].weight, a.model.layers[3].weight)
+        def forward(self, h):
+            a = self.self_attn
+            h = h + a.o_proj(a.q_proj(h) * torch.sigmoid(a.k_proj(h)) + a.v_proj(h))
+            m = self.mlp
+            return self.other(h + m.down_proj(torch.sigmoid(m.gate_proj(h)) * m.up_proj(h)))
+
+    torch.manual_seed(3)
+    blk = Block()
+    before = {n: m.weight.detach().clone() for n, m in GP.linear_modules(blk).items()}
+    xs = [torch.randn(1, 40, 16, generator=g) for _ in range(3)]
+    fed = []
+    real = GP.InputGram.update
+    GP.InputGram.update = lambda self, t: (fed.append(tuple(t.shape)), real(self, t))[1]
+    try:
+        names = GP.round_decoder_layer(blk, lambda j: blk(xs[j]), 3, grid, 8)
+    finally:
+        GP.InputGram.update = real
+    assert names == ["self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj", "self_attn.o_proj", "mlp.gate_proj",
+                     "mlp.up_proj", "mlp.down_proj"]
+    assert len(fed) == 4 * 3   # four distinct input tensors per forward (q/k/v share one, gate/up share one) x 3 samples
+    after = GP.linear_modules(blk)
+    for n in names:
+        assert not torch.equal(after[n].weight, before[n]) and torch.equal(after[n].weight * 4, torch.round(after[n].weight * 4)), n
+    assert torch.equal(after["other"].weight, before["other"])
+    with pytest.raises(ValueError):
+        GP.group_quantizer("int8", {"weight_block_size": 32}, True)
