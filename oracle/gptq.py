@@ -2,9 +2,12 @@
 TEST INFRASTRUCTURE ONLY, like the rest of this package.
 
 Pinned by: the Hessian against a direct double-precision sum; U^T U against the inverse of the damped Hessian; with
-uncorrelated inputs (diagonal H) the result is the plain clip-search quantization; with correlated inputs the proxy
-loss tr((W-Q) H (W-Q)^T) is below that of plain quantization (a wrong sign or a transposed factor raises it).  The
-reference holds no vectors or tests for this path: its exact output is otherwise **parity unpinned**.
+groups of one column the walk equals optimal-brain-surgeon rounding column by column evaluated in float64 with an
+explicit inverse per column (no factor involved), exactly; with uncorrelated inputs (diagonal H) the result is the
+plain clip-search quantization; with correlated inputs the proxy loss tr((W-Q) H (W-Q)^T) is below that of plain
+quantization.  What remains source text alone is the reference's simplification inside a group of more than one
+column (the error divided by the diagonal of the factor's block, gptq.py:111-117, where the column-by-column walk
+would solve with the block); the reference holds no vectors or tests for this path.
 """
 from __future__ import annotations
 

@@ -681,3 +681,32 @@ def test_gptq_feedback_lowers_the_proxy_loss(fmt, cfg):
     H2[5, :] = 0
     H2[:, 5] = 0
     assert bool((G.fasterquant(W, H2, fmt, cfg)[:, 5] == 0).all())
+
+
+@pytest.mark.parametrize("fmt,cfg", [("mxint", {"weight_block_size": 1, "weight_width": 4}),
+                                     ("mxint", {"weight_block_size": 1, "weight_width": 8})])
+def test_gptq_with_groups_of_one_column_is_the_textbook_column_update(fmt, cfg):
+    """With one column per group nothing of the group-wise simplification is left (inside a group the reference
+    divides by the diagonal of the factor's block instead of solving with the block, gptq.py:111-117), and the walk must
+    be optimal-brain-surgeon rounding column by column: with H_c the damped Hessian restricted to the columns not yet
+    rounded, the error of column c divided by (H_c^-1)[0, 0] is fed into the others through (H_c^-1)[0, 1:].  That is
+    evaluated here in float64 with an explicit inverse per column, no Cholesky factor involved."""
+    from oracle import gptq as G
+
+    g = torch.Generator().manual_seed(8)
+    cols = 7
+    W = torch.randn(6, cols, generator=g)
+    X = torch.randn(50, cols, generator=g) @ (torch.randn(cols, cols, generator=g) * 0.5 + torch.eye(cols))
+    H = G.hessian([X])
+    got = G.fasterquant(W, H, fmt, cfg, quant_search=False)
+    Hd = H.double() + 0.01 * torch.diagonal(H).double().mean() * torch.eye(cols, dtype=torch.float64)
+    Wd = W.double().clone()
+    want = torch.zeros_like(Wd)
+    for c in range(cols):
+        inv = torch.linalg.inv(Hd[c:, c:])
+        q = O.mxint_quantizer(Wd[:, c:c + 1].float(), 1, cfg["weight_width"], 1).double()
+        want[:, c:c + 1] = q
+        Wd[:, c + 1:] -= (Wd[:, c:c + 1] - q) / inv[0, 0] @ inv[0:1, 1:]
+    assert float((got.double() - want).abs().max()) == 0.0
+    # and a wrong sign of the feed-forward, or the factor transposed, does not give this result
+    assert not torch.equal(got, O.mxint_quantizer(W, 1, cfg["weight_width"], 1))
