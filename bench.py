@@ -851,12 +851,14 @@ def load_traffic(name):
 
 
 HEADLINE = ("bfp_qdq", "mxint_qdq", "mxint_linear", "mxfp_linear", "decoder_layer")  # configs 2, 1, 3, 4, 5
+REGIONS = 5             # timed regions per workload; the median is reported
 SETTLE_SECONDS = 0.06  # untimed run-in before the warm-up steps, so that clocks and memory system are at steady state
 
 
 def measure(torch, dev, name, steps, warmup, a):
-    """One workload: W warm-up steps, K wall-clock-timed steps bracketed by synchronisation, K event-timed launches
-    of the dominant kernel, the CPU baseline leg.  Returns the fields of a bench line for it."""
+    """One workload: W warm-up steps, REGIONS regions of K wall-clock-timed steps each bracketed by synchronisation
+    (median reported), as many event-timed regions of K launches of the dominant kernel, the CPU baseline leg.
+    Returns the fields of a bench line for it."""
     w = WORKLOADS[name]()
     steps = w.default_steps if steps is None else steps
     warmup = w.default_warmup if warmup is None else warmup
@@ -875,23 +877,33 @@ def measure(torch, dev, name, steps, warmup, a):
         w.step(i)
     torch.cuda.synchronize()
 
-    # whole-job timing: wall clock bracketed by synchronisation
-    t0 = time.perf_counter()
-    for i in range(steps):
-        w.step(i)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    # whole-job timing: REGIONS regions of exactly `steps` steps each, every region bracketed by synchronisation and
+    # timed on the wall clock; the median region is reported (a region of 20 steps of a 40 us kernel lasts under a
+    # millisecond, and a single such reading moves by several per cent)
+    walls = []
+    for _ in range(REGIONS):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            w.step(i)
+        torch.cuda.synchronize()
+        walls.append(time.perf_counter() - t0)
+    wall = sorted(walls)[REGIONS // 2]
 
-    # kernel timing: one HIP event pair on the launch stream (torch's current stream is the one handed to the
-    # C ABI) around K back-to-back launches; average launch duration = elapsed / K
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    # kernel timing: a HIP event pair on the launch stream (torch's current stream is the one handed to the C ABI)
+    # around `steps` back-to-back launches of the dominant kernel; average launch duration = elapsed / steps; the
+    # median of REGIONS such regions
     dominant = getattr(w, "dominant_step", w.step)
-    e0.record()
-    for i in range(steps):
-        dominant(i)
-    e1.record()
-    torch.cuda.synchronize()
-    k_avg = e0.elapsed_time(e1) / steps
+    k_regions = []
+    for _ in range(REGIONS):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(steps):
+            dominant(i)
+        e1.record()
+        torch.cuda.synchronize()
+        k_regions.append(e0.elapsed_time(e1) / steps)
+    k_avg = sorted(k_regions)[REGIONS // 2]
 
     work = w.work_per_step()
     scale = 1e9 if w.bound == "hbm" else 1e12
@@ -910,6 +922,8 @@ def measure(torch, dev, name, steps, warmup, a):
         "warmup": warmup,
         "settle_steps": settle,
         "ms_per_step": round(wall / steps * 1e3, 5),
+        "timed_regions": REGIONS,
+        "ms_per_step_regions": [round(t / steps * 1e3, 5) for t in walls],
         "whole_step_frac": round(value / peak, 4),
         "dtype": w.dtype,
         "config": w.config,
@@ -926,6 +940,13 @@ def measure(torch, dev, name, steps, warmup, a):
         },
         "cpu_baseline": cpu,
     }
+    # where the dominant kernel is the whole step, its average launch cannot take longer than a step
+    if not hasattr(w, "dominant_step"):
+        ok = k_avg <= wall / steps * 1e3 * 1.01
+        out["consistency"] = {"kernel_ms_avg_le_ms_per_step": bool(ok)}
+        if not ok:
+            out["warning"] = (f"dominant kernel average {k_avg:.5f} ms exceeds the whole step {wall / steps * 1e3:.5f} ms: the "
+                              "timed regions are too short to resolve; rerun with more --steps")
     if hasattr(w, "extra"):
         out["extra"] = w.extra(torch)
     del w
@@ -989,8 +1010,13 @@ def main():
         "roofline": head["roofline"],
         "cpu_baseline": head["cpu_baseline"],
         "settle_steps": head["settle_steps"],
+        "timed_regions": head["timed_regions"],
+        "ms_per_step_regions": head["ms_per_step_regions"],
         "whole_step_frac": head["whole_step_frac"],
     }
+    for key in ("consistency", "warning"):
+        if key in head:
+            out[key] = head[key]
     if "extra" in head:
         out["extra"] = head["extra"]
     if a.workload == "all":

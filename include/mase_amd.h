@@ -180,6 +180,20 @@ int mase_mx_unpack(const uint8_t* codes, const uint8_t* scales, void* out, size_
 int mase_gemm_bf16_tn(const void* A, const void* B, const void* bias, void* C, size_t M, size_t N, size_t K,
                       int out_dtype, int bias_dtype, void* stream);
 
+/* batch_outer x batch_inner independent products C[o][i] = A[o][i] (M x K) * B[o][i] (N x K)^T, bf16 operands, fp32
+ * accumulation, output in out_dtype, on the same tiled kernel: the batched contractions of the quantized attention
+ * modules (torch.matmul of the quantized query with the keys and of the quantized probabilities with the values,
+ * nn/quantized/modules/llama/attention.py:398-457) and of bmm_mx* / matmul_mx* on batched operands
+ * (nn/quantized/functional/matmul.py:437-512), whose quantized operands are exact in bf16.  All strides in elements:
+ * lda / ldb / ldc of a row of A / B / C, and per operand the strides of the outer and the inner batch index (a head
+ * of [batch, tokens, heads, d] memory is row stride heads * d, inner stride d, outer stride tokens * heads * d).
+ * K % 64 == 0; operand strides multiples of 8 and output strides multiples of 16 bytes; pointers 16-byte aligned;
+ * M * lda and N * ldb below 2^31 elements. */
+int mase_gemm_bf16_tn_batched(const void* A, const void* B, void* C, size_t batch_outer, size_t batch_inner, size_t M,
+                              size_t N, size_t K, size_t lda, size_t ldb, size_t ldc, size_t a_stride_outer,
+                              size_t a_stride_inner, size_t b_stride_outer, size_t b_stride_inner, size_t c_stride_outer,
+                              size_t c_stride_inner, int out_dtype, void* stream);
+
 /* The same product for shapes whose 256x256 output tiles alone would leave most CUs idle (a few hundred rows of A):
  * K is cut into ranges, every (tile, range) pair is a work item of the same kernel and writes an fp32 partial tile into
  * `workspace` (at least mase_gemm_bf16_tn_splitk_workspace_bytes(M, N, K) bytes, 16-byte aligned), and a second kernel

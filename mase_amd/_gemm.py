@@ -95,6 +95,121 @@ def gemm_bf16_tn(a: Tensor, b: Tensor, bias: Tensor | None, out_dtype: torch.dty
     return out
 
 
+def _batch_strides(t: Tensor):
+    """the leading dimensions of a [..., rows, cols] tensor as at most two nested indices: (outer count, inner count,
+    outer stride, inner stride) with outer count 1 when one index does; None when they need more than two"""
+    merged = []
+    for n, st in zip(t.shape[:-2], t.stride()[:-2]):
+        if n == 1:
+            continue
+        if merged and merged[-1][1] == st * n:  # contiguous with respect to the dimension before it: one index
+            merged[-1] = (merged[-1][0] * n, st)
+        else:
+            merged.append((n, st))
+    if len(merged) > 2:
+        return None
+    while len(merged) < 2:
+        merged.insert(0, (1, 0))
+    return merged[0][0], merged[1][0], merged[0][1], merged[1][1]
+
+
+def _common_batch_split(tensors):
+    """(outer count, inner count, [(outer stride, inner stride) per tensor]) such that every tensor's leading
+    dimensions are addressed by the same two nested indices; None when there is no such pair"""
+    parts = [_batch_strides(t) for t in tensors]
+    if any(p is None for p in parts):
+        return None
+    two_level = {p[:2] for p in parts if p[0] > 1}
+    if len(two_level) > 1:
+        return None
+    count = parts[0][0] * parts[0][1]
+    n_outer, n_inner = two_level.pop() if two_level else (1, count)
+    strides = []
+    for no, ni, so, si in parts:
+        if no * ni != count:
+            return None
+        # a tensor that needs one index only: the outer index advances it by n_inner inner steps
+        strides.append((so, si) if no > 1 else (si * n_inner, si))
+    return n_outer, n_inner, strides
+
+
+def gemm_bf16_tn_batched_supported(a: Tensor, b: Tensor) -> bool:
+    """a [..., M, K] and b [..., N, K] bf16 device tensors with equal leading shapes, last dimension contiguous, K a
+    multiple of 64, strides multiples of 8, leading dimensions expressible as two nested indices common to both"""
+    if not (a.is_cuda and a.device == b.device and a.dtype == b.dtype == torch.bfloat16 and a.dim() == b.dim() >= 3):
+        return False
+    if a.shape[:-2] != b.shape[:-2] or a.shape[-1] != b.shape[-1] or a.numel() == 0 or b.numel() == 0:
+        return False
+    if torch.is_grad_enabled() and (a.requires_grad or b.requires_grad):
+        return False
+    K = a.shape[-1]
+    if K % GEMM_K_MULTIPLE:
+        return False
+    for t in (a, b):
+        if t.stride(-1) != 1 or t.stride(-2) < K or any(st % 8 for st in t.stride()[:-1]) or t.data_ptr() % 16:
+            return False
+        if t.shape[-2] * t.stride(-2) * 2 > OPERAND_BYTES_LIMIT:
+            return False
+    return _common_batch_split((a, b)) is not None
+
+
+def gemm_bf16_tn_batched(a: Tensor, b: Tensor, out_dtype: torch.dtype | None = None, out: Tensor | None = None) -> Tensor:
+    """``a[..., M, K] @ b[..., N, K]^T`` for every index of the leading dimensions: bf16 operands (strided views are
+    taken as they are), fp32 accumulation, one rounding to ``out_dtype`` (``mase_gemm_bf16_tn_batched``).  ``out``: a
+    [..., M, N] tensor to write into (last dimension contiguous, e.g. a transposed view of [batch, M, heads, N]
+    memory); without it the result is contiguous."""
+    _lib.require_device(a, "gemm_bf16_tn_batched")
+    lib = _lib.load()
+    assert gemm_bf16_tn_batched_supported(a, b)
+    lead = tuple(a.shape[:-2])
+    M, K, N = a.shape[-2], a.shape[-1], b.shape[-2]
+    if out is None:
+        out = torch.empty(lead + (M, N), dtype=out_dtype or a.dtype, device=a.device)
+        if (N * out.element_size()) % 16:  # rows of whole 16-byte pieces: pad the row stride
+            pad = 16 // out.element_size()
+            out = torch.empty(lead + (M, (N + pad - 1) // pad * pad), dtype=out.dtype, device=a.device)[..., :N]
+    assert tuple(out.shape) == lead + (M, N) and out.stride(-1) == 1 and out.device == a.device
+    esz = out.element_size()
+    split = _common_batch_split((a, b, out))
+    if split is None or out.data_ptr() % 16 or any((st * esz) % 16 for st in out.stride()[:-1]):
+        raise _lib.MaseAmdError("gemm_bf16_tn_batched: the output's layout does not fit the operands' (strides of whole "
+                                "16-byte pieces, leading dimensions addressed by the same two nested indices)")
+    n_outer, n_inner, ((a_so, a_si), (b_so, b_si), (c_so, c_si)) = split
+    rc = lib.mase_gemm_bf16_tn_batched(a.data_ptr(), b.data_ptr(), out.data_ptr(), n_outer, n_inner, M, N, K, a.stride(-2),
+                                       b.stride(-2), out.stride(-2), a_so, a_si, b_so, b_si, c_so, c_si,
+                                       _lib.DTYPE_CODE[out.dtype], _lib.stream_ptr(a))
+    _lib.check(rc, "mase_gemm_bf16_tn_batched")
+    return out
+
+
+def matmul_bf16(x: Tensor, y: Tensor, out: Tensor | None = None, out_dtype: torch.dtype | None = None) -> Tensor | None:
+    """``torch.matmul(x, y)`` for bf16 device tensors x [..., M, K], y [..., K, N] with equal leading dimensions on the
+    batched matrix-core kernel of this package (fp32 accumulation, one rounding to ``out_dtype``, bf16 unless given), or None when the operands do
+    not fit it (the caller then uses the library's).  y is copied into [..., N, K] rows once (the kernel contracts
+    rows with rows); a contraction length that is not a multiple of 64 is padded with zeros in that copy and in a copy
+    of x.  ``out``: as in ``gemm_bf16_tn_batched``."""
+    if not (x.is_cuda and x.dtype == y.dtype == torch.bfloat16 and x.dim() == y.dim() >= 3 and x.shape[:-2] == y.shape[:-2]
+            and x.shape[-1] == y.shape[-2] and x.numel() > 0 and y.numel() > 0):
+        return None
+    if torch.is_grad_enabled() and (x.requires_grad or y.requires_grad):
+        return None
+    K = x.shape[-1]
+    pad = -K % GEMM_K_MULTIPLE
+    if y.stride(-2) == 1 and not pad and y.stride(-1) >= K:  # already rows of K (a transposed view)
+        yt = y.transpose(-1, -2)
+    else:
+        yt = torch.zeros(y.shape[:-2] + (y.shape[-1], K + pad), dtype=y.dtype, device=y.device) if pad else \
+            torch.empty(y.shape[:-2] + (y.shape[-1], K), dtype=y.dtype, device=y.device)
+        yt[..., :K].copy_(y.transpose(-1, -2))
+    if pad:
+        x = torch.nn.functional.pad(x, (0, pad))
+    elif x.stride(-1) != 1 or any(st % 8 for st in x.stride()[:-1]) or x.data_ptr() % 16:
+        x = x.contiguous()
+    if not gemm_bf16_tn_batched_supported(x, yt):
+        return None
+    return gemm_bf16_tn_batched(x, yt, out_dtype=out_dtype, out=out)
+
+
 def gemm_mxint8_packed_supported(N: int, K: int) -> bool:
     return K % PACKED_B_K_MULTIPLE == 0 and (N + 31) // 32 * 32 * K <= OPERAND_BYTES_LIMIT
 

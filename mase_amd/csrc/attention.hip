@@ -54,9 +54,12 @@ __device__ __forceinline__ uint32_t umax_with_other_half(uint32_t v) {
 constexpr int kAttnLds = 2 * kKBytes + 2 * kVBytes;
 
 // lane i's 16 bytes at base + off_i land at LDS address lds_addr + 16 * i; tracked by hand with at_wait_vmcnt
+// (m0 is written inside the statement and not listed as clobbered: the compiler keeps no value in m0 across
+// statements on this target, it reloads m0 before each use of its own, and rejects the name in a clobber list as a
+// reserved register)
 __device__ __forceinline__ void at_async_copy_16(const unsigned char* base, uint32_t off, uint32_t lds_addr) {
   const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_addr);
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
 }
 template <int N>
 __device__ __forceinline__ void at_wait_vmcnt() {

@@ -59,6 +59,11 @@ struct GemmParams {
   int tiles_m, tiles_n;
   int splits, kc;  // K is cut into `splits` ranges of kc elements; a work item is one output tile over one range and
                    // (when splits > 1) writes an fp32 partial tile into slice `range` of C, laid out [splits, M, N]
+  // BATCHED instantiation only: `batches` independent products, product index = outer * batch_inner + inner; byte
+  // strides of the two index parts per operand, and byte strides of an operand row / an output row
+  int batches = 1, batch_inner = 1;
+  size_t a_so = 0, a_si = 0, b_so = 0, b_si = 0, c_so = 0, c_si = 0;
+  size_t lda = 0, ldb = 0, ldc = 0;
 };
 
 __device__ __forceinline__ int lds_off(int row, int chunk) {
@@ -79,9 +84,12 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 // copies it knows to be in flight (s_waitcnt vmcnt(0) before each ds_read), which would serialize the
 // pipeline; completion is tracked by hand with wait_vmcnt.  M0 carries the LDS base; nothing else in this
 // kernel uses M0.
+// (m0 is written inside the statement and not listed as clobbered: the compiler keeps no value in m0 across
+// statements on this target, it reloads m0 before each use of its own, and rejects the name in a clobber list as a
+// reserved register)
 __device__ __forceinline__ void async_copy_16(const unsigned char* base, uint32_t off, uint32_t lds_addr) {
   const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_addr);
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
 }
 
 // The lane number, computed where it is needed (two instructions) instead of being kept: the code between output tiles
@@ -143,10 +151,14 @@ __device__ __forceinline__ void load_2_untracked(uint32_t& dst, uint32_t off, co
 // the bytes of the bf16 image in memory and on the way in; the codes are widened to the same bf16 operand values in
 // registers, one K step ahead of the MFMAs that use them (code + 128 as an unsigned byte -> v_cvt_f32_ubyte -> one fma
 // that removes the 128 and applies the block's power-of-two scale -> the upper half of the exact fp32 product).
-template <int OUT_DT, bool STREAM, bool BPACK = false, bool BCODES = false>
+// BATCHED (plain form only): the work items are the output tiles of `batches` independent products with strided
+// operands (the score and value products of an attention block, torch.bmm): an item's operand bases and its output
+// base follow from its product index; rows of A, B and C have the strides lda, ldb, ldc.
+template <int OUT_DT, bool STREAM, bool BPACK = false, bool BCODES = false, bool BATCHED = false>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p) {
   constexpr int NI = BPACK ? 8 : 4, NJ = BPACK ? 2 : 4;  // MFMA tiles of a wavefront: rows x columns
   static_assert(!BCODES || BPACK, "codes come in fragment order");
+  static_assert(!BATCHED || !BPACK, "the batched form takes row-major operands");
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int tid = threadIdx.x;
   const int lane_id = tid & 63;
@@ -160,7 +172,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // divide, XCD x owns the contiguous tile range [x*total/8, (x+1)*total/8) and its work-groups walk it
   // together (at any time they hold neighbouring tiles, which share operand rows in that XCD's L2).
   const int tiles_mn = p.tiles_m * p.tiles_n;
-  const int total = tiles_mn * p.splits;
+  const int total = tiles_mn * (BATCHED ? p.batches : p.splits);
   const int nwg = (int)gridDim.x;
   int t_first, t_step, t_end;
   if ((total & 7) == 0 && (nwg & 7) == 0) {
@@ -177,6 +189,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   if (n_my == 0) return;
   constexpr int GROUP_M = 4;  // tiles are walked in groups of 4 tile rows
   const int in_group = GROUP_M * p.tiles_n;
+  // (BATCHED: ks is the item's product index; there are no K ranges)
   auto tile_origin = [&](int ord, int& m0, int& n0, int& ks) __attribute__((always_inline)) {  // ord-th item of this work-group
     const int item = t_first + min(ord, n_my - 1) * t_step;
     ks = item / tiles_mn;
@@ -188,18 +201,26 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   };
 
   // ---- global side of the async copies: wave w fills row groups w + 4*j (8 rows of 128 B each), j = 0..7
-  const size_t ldb = (size_t)p.K * 2;  // bytes per operand row
+  const size_t ldb = BATCHED ? p.ldb : (size_t)p.K * 2;  // bytes per operand row
+  const size_t lda = BATCHED ? p.lda : ldb;
   uint32_t ga[kWaveCopies], gb[kWaveCopies];  // byte offsets of this lane's chunks from the operand bases
+  const unsigned char *copy_a = p.A, *copy_b = p.B;  // operand bases of the item the copy stream is in
   auto set_copy_tile = [&](int ord) __attribute__((always_inline)) {
     int m0, n0, ks;
     tile_origin(ord, m0, n0, ks);
-    const uint32_t k0 = (uint32_t)ks * (uint32_t)p.kc * 2u;  // byte offset of the item's K range inside a row
+    uint32_t k0 = (uint32_t)ks * (uint32_t)p.kc * 2u;  // byte offset of the item's K range inside a row
+    if constexpr (BATCHED) {
+      const int bo = ks / p.batch_inner, bi = ks - bo * p.batch_inner;
+      copy_a = p.A + (size_t)bo * p.a_so + (size_t)bi * p.a_si;
+      copy_b = p.B + (size_t)bo * p.b_so + (size_t)bi * p.b_si;
+      k0 = 0;
+    }
     const int lane = lane_now();
 #pragma unroll
     for (int j = 0; j < kWaveCopies; ++j) {
       const int r = (wave + 4 * j) * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ ((r >> 1) & 7);  // chunk that belongs at LDS position lane&7 of row r
-      ga[j] = (uint32_t)((size_t)min(m0 + r, p.M - 1) * ldb) + chunk * 16 + k0;
+      ga[j] = (uint32_t)((size_t)min(m0 + r, p.M - 1) * lda) + chunk * 16 + k0;
       if constexpr (!BPACK) gb[j] = (uint32_t)((size_t)min(n0 + r, p.N - 1) * ldb) + chunk * 16 + k0;
     }
   };
@@ -221,7 +242,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     }
     const uint32_t st = lds_base + (uint32_t)(c_stage * kStride) + (c & 1) * kTileBytes;
     const int j = c >> 1;
-    async_copy_16(((c & 1) ? p.B : p.A) + (size_t)c_kt * kRowBytes, (c & 1) ? gb[j] : ga[j], st + (wave + 4 * j) * 1024);
+    async_copy_16(((c & 1) ? copy_b : copy_a) + (size_t)c_kt * kRowBytes, (c & 1) ? gb[j] : ga[j], st + (wave + 4 * j) * 1024);
   };
   auto step_within_tile = [&]() __attribute__((always_inline)) {
     c_stage = next_of(c_stage);
@@ -289,7 +310,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     tile_origin(ord, m0, n0, ks);
     acc_read_fence();
     // partial tiles of K range ks go to slice ks of C (fp32, no bias: the caller's reduction adds it)
-    unsigned char* const Cs = (unsigned char*)p.C + (size_t)ks * (size_t)p.M * (size_t)p.N * sizeof(float);
+    unsigned char* Cs = (unsigned char*)p.C + (size_t)ks * (size_t)p.M * (size_t)p.N * sizeof(float);
+    if constexpr (BATCHED) {
+      const int bo = ks / p.batch_inner, bi = ks - bo * p.batch_inner;
+      Cs = (unsigned char*)p.C + (size_t)bo * p.c_so + (size_t)bi * p.c_si;
+    }
     const int lane = lane_now();
     const int r32 = lane & 31, kgrp = lane >> 5;
     const int rrow = lane >> 3, chunk = lane & 7;  // read side: row rrow + 8 * pass, 16-byte piece `chunk` of it
@@ -298,12 +323,13 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     const unsigned char* const stg_r = stg + rrow * kStgRow + chunk * 16;
     constexpr int kEsz = (OUT_DT == MASE_DT_F32) ? 4 : 2;
     constexpr int kVec = 16 / kEsz;  // elements per 16-byte piece
-    const bool vec_ok = ((p.N & (kVec - 1)) == 0) && ((((uintptr_t)p.C) & 15u) == 0);
+    // (BATCHED: the host has checked that the output base, its strides and its row stride are multiples of 16 bytes)
+    const bool vec_ok = BATCHED ? true : ((p.N & (kVec - 1)) == 0) && ((((uintptr_t)p.C) & 15u) == 0);
     // the wavefront's whole part of the tile lies inside C and takes 16-byte stores (wavefront-uniform)
     const bool interior = vec_ok && m0 + row_base + NI * 32 <= p.M && n0 + col_base + NJ * 32 <= p.N;
-    const size_t row_step = (size_t)p.N * kEsz;  // bytes from one output row to the next
+    const size_t row_step = BATCHED ? p.ldc : (size_t)p.N * kEsz;  // bytes from one output row to the next
     // where this lane's piece of row 0 of the wavefront's first band goes
-    unsigned char* const lane_c = Cs + ((size_t)(m0 + row_base + rrow) * p.N + (size_t)(n0 + col_base + chunk * kVec)) * kEsz;
+    unsigned char* const lane_c = Cs + (size_t)(m0 + row_base + rrow) * row_step + (size_t)(n0 + col_base + chunk * kVec) * kEsz;
     float bv[NJ][4][4];  // bias of the lane's columns
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
@@ -698,9 +724,10 @@ int persistent_grid_bf16(int total_tiles) {
 }
 
 // launch of the persistent kernel for the work items of p (tiles x K ranges), output dtype out_dtype
-int launch_gemm_bf16(const GemmParams& p, int out_dtype, hipStream_t st, bool bpack = false, bool bcodes = false) {
+int launch_gemm_bf16(const GemmParams& p, int out_dtype, hipStream_t st, bool bpack = false, bool bcodes = false,
+                     bool batched = false) {
   const size_t lds_bytes = (size_t)kLdsBytes;
-  const int nwg = persistent_grid_bf16(p.tiles_m * p.tiles_n * p.splits);
+  const int nwg = persistent_grid_bf16(p.tiles_m * p.tiles_n * (batched ? p.batches : p.splits));
   if (nwg <= 0) return MASE_ERR_LAUNCH;
   const dim3 grid((unsigned)nwg), block(kGemmThreads);
   const bool stream_fits = p.kc / BK >= S;
@@ -711,7 +738,25 @@ int launch_gemm_bf16(const GemmParams& p, int out_dtype, hipStream_t st, bool bp
     if (!set_dynamic_lds_once(attr_done, k, (int)lds_bytes)) return MASE_ERR_LAUNCH;                              \
     hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, STREAM_>), grid, block, lds_bytes, st, p);                       \
   } while (0)
-  if (bpack && bcodes) {
+  if (batched) {
+#define MASE_GEMM_LAUNCH_BATCHED(DT_, STREAM_)                                                                    \
+  do {                                                                                                            \
+    static std::atomic<uint64_t> attr_done{0};                                                                    \
+    const void* k = (const void*)gemm_bf16_tn_kernel<DT_, STREAM_, false, false, true>;                           \
+    if (!set_dynamic_lds_once(attr_done, k, (int)lds_bytes)) return MASE_ERR_LAUNCH;                              \
+    hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, STREAM_, false, false, true>), grid, block, lds_bytes, st, p);   \
+  } while (0)
+    if (stream_fits) {
+      if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH_BATCHED(MASE_DT_F32, true);
+      else if (out_dtype == MASE_DT_BF16) MASE_GEMM_LAUNCH_BATCHED(MASE_DT_BF16, true);
+      else MASE_GEMM_LAUNCH_BATCHED(MASE_DT_F16, true);
+    } else {
+      if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH_BATCHED(MASE_DT_F32, false);
+      else if (out_dtype == MASE_DT_BF16) MASE_GEMM_LAUNCH_BATCHED(MASE_DT_BF16, false);
+      else MASE_GEMM_LAUNCH_BATCHED(MASE_DT_F16, false);
+    }
+#undef MASE_GEMM_LAUNCH_BATCHED
+  } else if (bpack && bcodes) {
     if (!stream_fits || ((p.kc / BK) & 1) != 0) return MASE_ERR_SHAPE;
 #define MASE_GEMM_LAUNCH_C(DT_)                                                                                   \
   do {                                                                                                            \
@@ -856,6 +901,50 @@ extern "C" int mase_gemm_bf16_tn(const void* A, const void* B, const void* bias,
   p.splits = 1;
   p.kc = (int)K;
   return launch_gemm_bf16(p, out_dtype, (hipStream_t)stream);
+}
+
+extern "C" int mase_gemm_bf16_tn_batched(const void* A, const void* B, void* C, size_t batch_outer, size_t batch_inner,
+                                         size_t M, size_t N, size_t K, size_t lda, size_t ldb, size_t ldc,
+                                         size_t a_stride_outer, size_t a_stride_inner, size_t b_stride_outer,
+                                         size_t b_stride_inner, size_t c_stride_outer, size_t c_stride_inner,
+                                         int out_dtype, void* stream) {
+  using namespace mase;
+  if (M == 0 || N == 0 || batch_outer == 0 || batch_inner == 0) return MASE_OK;
+  if (A == nullptr || B == nullptr || C == nullptr) return MASE_ERR_NULL;
+  if (out_dtype < 0 || out_dtype > 2) return MASE_ERR_DTYPE;
+  if (K == 0 || (K % BK) != 0 || M > (1u << 30) || N > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
+  if (lda < K || ldb < K || ldc < N) return MASE_ERR_SHAPE;
+  const unsigned long long esz = out_dtype == MASE_DT_F32 ? 4 : 2;
+  // operand rows are fetched in 16-byte pieces at 32-bit byte offsets from the product's operand base; output pieces
+  // of 16 bytes are stored whole where they lie inside a row
+  if ((unsigned long long)M * lda * 2 > 0xFFFFFFFFull || (unsigned long long)N * ldb * 2 > 0xFFFFFFFFull) return MASE_ERR_SHAPE;
+  const unsigned long long tiles = (unsigned long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  if (tiles * batch_outer * batch_inner > (1ull << 30) || batch_inner > (1u << 30)) return MASE_ERR_SHAPE;
+  if (!aligned16(A) || !aligned16(B) || !aligned16(C)) return MASE_ERR_ALIGN;
+  if (lda % 8 || ldb % 8 || a_stride_outer % 8 || a_stride_inner % 8 || b_stride_outer % 8 || b_stride_inner % 8)
+    return MASE_ERR_ALIGN;
+  if ((ldc * esz) % 16 || (c_stride_outer * esz) % 16 || (c_stride_inner * esz) % 16) return MASE_ERR_ALIGN;
+  GemmParams p;
+  p.A = (const unsigned char*)A;
+  p.B = (const unsigned char*)B;
+  p.Bs = nullptr;
+  p.bias = nullptr;
+  p.C = C;
+  p.M = (int)M;
+  p.N = (int)N;
+  p.K = (int)K;
+  p.bias_dtype = 0;
+  p.tiles_m = (int)((M + BM - 1) / BM);
+  p.tiles_n = (int)((N + BN - 1) / BN);
+  p.splits = 1;
+  p.kc = (int)K;
+  p.batches = (int)(batch_outer * batch_inner);
+  p.batch_inner = (int)batch_inner;
+  p.a_so = a_stride_outer * 2; p.a_si = a_stride_inner * 2;
+  p.b_so = b_stride_outer * 2; p.b_si = b_stride_inner * 2;
+  p.c_so = c_stride_outer * esz; p.c_si = c_stride_inner * esz;
+  p.lda = lda * 2; p.ldb = ldb * 2; p.ldc = ldc * esz;
+  return launch_gemm_bf16(p, out_dtype, (hipStream_t)stream, false, false, true);
 }
 
 extern "C" size_t mase_gemm_bf16_tn_splitk_workspace_bytes(size_t M, size_t N, size_t K) {

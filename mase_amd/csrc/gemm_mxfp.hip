@@ -51,12 +51,15 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 // one wavefront-wide async copy HBM/L2 -> LDS: lane i's BYTES bytes at base + off_i land at LDS address
 // lds_addr + BYTES*i (base and lds_addr wavefront-uniform, off_i a 32-bit byte offset)
 template <int BYTES>
+// (m0 is written inside the statement and not listed as clobbered: the compiler keeps no value in m0 across
+// statements on this target, it reloads m0 before each use of its own, and rejects the name in a clobber list as a
+// reserved register)
 __device__ __forceinline__ void async_copy(const unsigned char* base, uint32_t off, uint32_t lds_addr) {
   const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_addr);
   if constexpr (BYTES == 16)
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
   else
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
 }
 
 template <int N>

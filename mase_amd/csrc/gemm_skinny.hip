@@ -43,9 +43,12 @@ __device__ __forceinline__ int sk_lds_off(int row, int chunk) { return row * 128
 
 // one wavefront-wide 1 KB async copy (issued from inline assembly and tracked by hand with s_waitcnt vmcnt, for the
 // reasons given in gemm_bf16.hip); M0 = LDS address, nothing else in this kernel uses M0
+// (m0 is written inside the statement and not listed as clobbered: the compiler keeps no value in m0 across
+// statements on this target, it reloads m0 before each use of its own, and rejects the name in a clobber list as a
+// reserved register)
 __device__ __forceinline__ void sk_async_copy(const unsigned char* base, uint32_t off, uint32_t lds_addr) {
   const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_addr);
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
 }
 
 template <int N>
@@ -171,7 +174,7 @@ struct SkinnyQParams {
 
 __device__ __forceinline__ void sk_async_copy4(const unsigned char* base, uint32_t off, uint32_t lds_addr) {
   const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_addr);
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
 }
 
 // four codes of one dword -> two registers of two bf16 values each (code * scale, exact)

@@ -2,9 +2,11 @@
 reference's ``chop/nn/quantized/functional/matmul.py:437-512``: both operands are MX-quantized along their *last*
 dimension (``block_dim=-1``; for ``y`` that is N, not the contraction dimension), then multiplied.
 
-The quantizers are the HIP kernels.  A plain 2-D product whose quantized operands are exact in bf16 (MXINT up to 8
-bits, every MXFP format) runs on the bf16 matrix-core kernel with fp32 accumulation; batched products go to the
-library's batched GEMM in the tensors' dtype, as the reference's ``torch.matmul`` / ``torch.bmm`` do.
+The quantizers are the HIP kernels.  A product whose quantized operands are exact in bf16 (MXINT up to 8 bits, every
+MXFP format) runs on the bf16 matrix-core kernel of this package with fp32 accumulation: 2-D operands on
+``mase_gemm_bf16_tn``, batched operands with equal leading dimensions on ``mase_gemm_bf16_tn_batched``.  Anything else
+(broadcast leading dimensions, wider mantissas, gradients recorded) goes to ``torch.matmul`` / ``torch.bmm`` as in the
+reference.
 """
 from __future__ import annotations
 
@@ -12,7 +14,7 @@ from functools import partial
 
 import torch
 
-from ..._gemm import gemm_bf16_tn
+from ..._gemm import gemm_bf16_tn, matmul_bf16
 from ...quantizers import mxfp_quantizer, mxint_quantizer
 
 matmul_mapping = {"matmul": torch.matmul, "bmm": torch.bmm}
@@ -23,6 +25,12 @@ def _product(x, y, style, exact_in_bf16):
             and x.dtype in (torch.float32, torch.bfloat16, torch.float16) and x.numel() > 0 and y.numel() > 0
             and not (torch.is_grad_enabled() and (x.requires_grad or y.requires_grad))):
         return gemm_bf16_tn(x.to(torch.bfloat16), y.t().to(torch.bfloat16), None, x.dtype)
+    if (exact_in_bf16 and x.dim() == y.dim() >= 3 and x.is_cuda and x.dtype == y.dtype
+            and x.dtype in (torch.float32, torch.bfloat16, torch.float16)
+            and not (torch.is_grad_enabled() and (x.requires_grad or y.requires_grad))):
+        out = matmul_bf16(x.to(torch.bfloat16), y.to(torch.bfloat16), out_dtype=x.dtype)
+        if out is not None:
+            return out
     return matmul_mapping[style](x, y)
 
 

@@ -6,8 +6,9 @@ of the reference's ``chop/nn/quantized/modules/llama/attention.py:130-457`` (``L
 The reference derives these classes from the ``transformers`` Llama modules; here they are plain ``nn.Module``s with
 the same parameter names (``q_proj/k_proj/v_proj/o_proj``, ``gate_proj/up_proj/down_proj``, ``weight``), so a state
 dict of the original module loads with ``strict=True`` and no ``transformers`` import is needed.  ``config`` is any
-object with the Llama config fields read below (a ``LlamaConfig`` works).  Every quantizer is a HIP kernel; the
-contractions are the library's batched GEMMs, the operations the reference performs at those points.
+object with the Llama config fields read below (a ``LlamaConfig`` works).  Every quantizer is a HIP kernel; the two
+batched contractions (query x keys, probabilities x values: ``torch.matmul`` in the reference) run on the batched
+matrix-core kernel of this package for bf16 operands (``mase_gemm_bf16_tn_batched``) and on ``torch.matmul`` otherwise.
 
 What is quantized (``q_config`` sub-dicts, each with an optional ``bypass``):
   ``rope``      cos/sin tables, minifloat cast                       (attention.py:163-177)
@@ -26,6 +27,7 @@ from typing import Optional, Tuple
 import torch
 from torch import Tensor, nn
 
+from ..._gemm import matmul_bf16
 from ...quantizers import mxfp_quantizer, mxint_quantizer
 from ...quantizers import _ops
 from ...quantizers._ops import attn_softmax_mx, attn_softmax_mx_supported, minifloat_mx_qdq
@@ -57,6 +59,25 @@ def _mx_quantizer(kind: str, config: dict):
                    block_dim=-1)
 
 
+def _matmul(x, y, out=None):
+    """``torch.matmul(x, y)``; bf16 device operands with equal leading dimensions run on the batched matrix-core kernel
+    of this package (same arithmetic as the library's bf16 product: exact products, fp32 sums, one rounding)"""
+    r = matmul_bf16(x, y, out=out) if x.is_cuda and x.dtype == torch.bfloat16 else None
+    return torch.matmul(x, y) if r is None else r
+
+
+def _value_product(probabilities, value_states):
+    """``matmul(probabilities, value_states).transpose(1, 2).contiguous()``: [batch, tokens, heads, head_dim]; the own
+    kernel writes that layout directly"""
+    B, H, S, _ = probabilities.shape
+    D = value_states.shape[-1]
+    if probabilities.is_cuda and probabilities.dtype == torch.bfloat16 and (D * 2) % 16 == 0:
+        out = torch.empty((B, S, H, D), dtype=probabilities.dtype, device=probabilities.device)
+        if matmul_bf16(probabilities, value_states, out=out.transpose(1, 2)) is not None:
+            return out
+    return torch.matmul(probabilities, value_states).transpose(1, 2).contiguous()
+
+
 def _eager_attention_forward(kind, module, query, key, value, attention_mask, scaling, dropout=0.0, qk_bypass=False,
                              qk_config=None, av_bypass=False, av_config=None, softmax_bypass=False, softmax_config=None,
                              **kwargs):
@@ -64,12 +85,11 @@ def _eager_attention_forward(kind, module, query, key, value, attention_mask, sc
     value_states = repeat_kv(value, module.num_key_value_groups)
     if not qk_bypass:
         query = _mx_quantizer(kind, qk_config)(query)
-    scores = torch.matmul(query, key_states.transpose(2, 3))
+    scores = _matmul(query, key_states.transpose(2, 3))
     fused = _fused_probabilities(kind, module, scores, key_states, attention_mask, scaling, dropout, av_bypass, av_config,
                                  softmax_bypass, softmax_config)
     if fused is not None:
-        attn_output = torch.matmul(fused, value_states).transpose(1, 2).contiguous()
-        return attn_output, fused
+        return _value_product(fused, value_states), fused
     attn_weights = scores * scaling
     if attention_mask is not None:
         causal_mask = attention_mask[:, :, :, : key_states.shape[-2]]
@@ -81,9 +101,7 @@ def _eager_attention_forward(kind, module, query, key, value, attention_mask, sc
     attn_weights = nn.functional.dropout(attn_weights, p=dropout, training=module.training)
     if not av_bypass:
         attn_weights = _mx_quantizer(kind, av_config)(attn_weights)
-    attn_output = torch.matmul(attn_weights, value_states)
-    attn_output = attn_output.transpose(1, 2).contiguous()
-    return attn_output, attn_weights
+    return _value_product(attn_weights, value_states), attn_weights
 
 
 def _fused_probabilities(kind, module, scores, key_states, attention_mask, scaling, dropout, av_bypass, av_config,

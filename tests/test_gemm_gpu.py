@@ -284,3 +284,79 @@ def test_gemm_with_the_weight_as_mxint8_codes_in_fragment_order(dev, M, N, K):
                 assert float((got.float() - want.float()).abs().max() / want.float().abs().max()) < tol, (dt, rep)
             else:
                 assert torch.equal(got, want), (dt, rep, float((got.float() - want.float()).abs().max()))
+
+
+@pytest.mark.parametrize("B,H,S,T,D", [(2, 3, 100, 72, 64), (1, 4, 256, 256, 128), (2, 8, 520, 300, 128), (1, 1, 1, 64, 64),
+                                       (3, 5, 33, 513, 192)])
+def test_gemm_bf16_tn_batched_on_attention_layouts(dev, B, H, S, T, D):
+    """The two contractions of an attention block on the layouts the modules hand over: query and output as [batch,
+    heads, tokens, d] views of [batch, tokens, heads, d] memory, keys contiguous per head.  Small-integer operands make
+    every partial sum exact, so each product must equal the integer product bit for bit; random operands are held
+    to the rounding of the bf16 output against a float64 product."""
+    from mase_amd._gemm import gemm_bf16_tn_batched, gemm_bf16_tn_batched_supported, matmul_bf16
+
+    g = torch.Generator().manual_seed(B * 100 + S + T)
+    print(f"batched gemm B={B} H={H} S={S} T={T} D={D}", flush=True)
+    qi = torch.randint(-8, 9, (B, S, H, D), generator=g).float()
+    ki = torch.randint(-8, 9, (B, H, T, D), generator=g).float()
+    q = qi.bfloat16().to(dev).transpose(1, 2)          # [B, H, S, D] view, row stride H * D
+    k = ki.bfloat16().to(dev)
+    assert gemm_bf16_tn_batched_supported(q, k)
+    want = qi.transpose(1, 2) @ ki.transpose(-1, -2)   # exact: |sums| <= 64 * D
+    for dt in (torch.float32, torch.bfloat16):
+        got = gemm_bf16_tn_batched(q, k, out_dtype=dt)
+        assert got.shape == (B, H, S, T) and got.dtype == dt
+        assert torch.equal(got.cpu().float(), want.to(dt).float())
+    # scores x values through matmul_bf16 (values [B, H, T, D] are copied into rows of T; T is padded to a multiple of
+    # 64 when it is not one), written into [B, S, H, D] memory
+    pi = torch.randint(0, 5, (B, H, S, T), generator=g).float()
+    vi = torch.randint(-8, 9, (B, T, H, D), generator=g).float()
+    p, v = pi.bfloat16().to(dev), vi.bfloat16().to(dev).transpose(1, 2)
+    out = torch.full((B, S, H, D), 7.0, dtype=torch.bfloat16, device=dev)
+    r = matmul_bf16(p, v, out=out.transpose(1, 2))
+    assert r is not None and r.data_ptr() == out.data_ptr()
+    assert torch.equal(out.cpu().float(), (pi @ vi.transpose(1, 2)).transpose(1, 2).bfloat16().float())
+    # random operands
+    a = torch.randn(B, H, S, D, generator=g).bfloat16()
+    b = torch.randn(B, H, T, D, generator=g).bfloat16()
+    ref = a.double() @ b.double().transpose(-1, -2)
+    assert rel_err(gemm_bf16_tn_batched(a.to(dev), b.to(dev), out_dtype=torch.float32).cpu(), ref) < 2e-6
+    assert rel_err(gemm_bf16_tn_batched(a.to(dev), b.to(dev)).cpu(), ref) < 4e-3
+
+
+def test_matmul_bf16_shapes_it_takes_and_leaves(dev):
+    from mase_amd._gemm import matmul_bf16
+
+    g = torch.Generator().manual_seed(3)
+    x = torch.randint(-4, 5, (6, 40, 100), generator=g).float()     # contraction length 100: padded to 128
+    y = torch.randint(-4, 5, (6, 100, 24), generator=g).float()
+    got = matmul_bf16(x.bfloat16().to(dev), y.bfloat16().to(dev), out_dtype=torch.float32)
+    assert got.shape == (6, 40, 24) and torch.equal(got.cpu(), x @ y)
+    got16 = matmul_bf16(x.bfloat16().to(dev), y.bfloat16().to(dev))   # 24 bf16 = 48 bytes per row: a whole number of pieces
+    assert torch.equal(got16.cpu().float(), (x @ y).bfloat16().float())
+    y1 = torch.randint(-4, 5, (6, 100, 3), generator=g).float()      # 3 bf16 per row: the result's rows are padded
+    got3 = matmul_bf16(x.bfloat16().to(dev), y1.bfloat16().to(dev))
+    assert got3.shape == (6, 40, 3) and torch.equal(got3.cpu().float(), (x @ y1).bfloat16().float())
+    # not taken: broadcast leading dimensions, other dtypes, 2-D operands, CPU tensors
+    assert matmul_bf16(x[:1].bfloat16().to(dev), y.bfloat16().to(dev)) is None
+    assert matmul_bf16(x.to(dev), y.to(dev)) is None
+    assert matmul_bf16(x[0].bfloat16().to(dev), y[0].bfloat16().to(dev)) is None
+    assert matmul_bf16(x.bfloat16(), y.bfloat16()) is None
+
+
+def test_batched_gemm_c_abi_checks(dev):
+    from mase_amd import _lib
+
+    lib = _lib.load()
+    a = torch.zeros(2, 64, 64, device=dev).bfloat16()
+    c = torch.zeros(2, 64, 64, device=dev).bfloat16()
+    call = lambda **kw: lib.mase_gemm_bf16_tn_batched(*[{**dict(A=a.data_ptr(), B=a.data_ptr(), C=c.data_ptr(), bo=1, bi=2, M=64, N=64,
+                                                                K=64, lda=64, ldb=64, ldc=64, aso=0, asi=4096, bso=0, bsi=4096,
+                                                                cso=0, csi=4096, dt=1, st=None), **kw}[k]
+                                                         for k in ("A", "B", "C", "bo", "bi", "M", "N", "K", "lda", "ldb", "ldc", "aso",
+                                                                   "asi", "bso", "bsi", "cso", "csi", "dt", "st")])
+    assert call() == 0
+    assert call(K=96) == -2 and call(lda=32) == -2 and call(ldc=60) == -2       # shape
+    assert call(lda=68) == -3 and call(csi=4100) == -3 and call(A=a.data_ptr() + 2) == -3   # alignment
+    assert call(A=None) == -1 and call(dt=5) == -4
+    assert call(bo=0) == 0 and call(M=0) == 0

@@ -378,3 +378,35 @@ def test_qwen3_registry_and_pass(dev):
     assert isinstance(net.self_attn, Qwen3AttentionMXInt) and isinstance(net.mlp, Qwen3MLPMXInt)
     assert isinstance(net.norm, Qwen3RMSNormMinifloat)
     assert torch.equal(net.self_attn.q_norm.weight.data, wq)
+
+
+@pytest.mark.parametrize("kind", ["mxint", "mxfp"])
+def test_attention_contractions_run_on_the_batched_kernel_of_this_package(dev, monkeypatch, kind):
+    """bf16 modules: query x keys and probabilities x values both go through mase_gemm_bf16_tn_batched (prefill, and
+    decode against a cache whose length is not a multiple of 64); torch.matmul is not called at all.  fp32 modules keep
+    torch.matmul: their keys and values are not bf16 values."""
+    from mase_amd import _gemm
+    from mase_amd.quantized import LlamaAttentionMXFP, LlamaAttentionMXInt
+
+    cls, q = (LlamaAttentionMXInt, Q_INT) if kind == "mxint" else (LlamaAttentionMXFP, Q_FP)
+    calls = []
+    real = _gemm.gemm_bf16_tn_batched
+    monkeypatch.setattr(_gemm, "gemm_bf16_tn_batched", lambda a, b, **kw: (calls.append((tuple(a.shape), tuple(b.shape))), real(a, b, **kw))[1])
+    library = []
+    real_matmul = torch.matmul
+    monkeypatch.setattr(torch, "matmul", lambda *a, **k: (library.append(1), real_matmul(*a, **k))[1])
+    for dtype, own in ((torch.bfloat16, True), (torch.float32, False)):
+        m = cls(CFG, layer_idx=0, q_config=q).to(dtype)
+        m.load_state_dict(seeded(m, 5, dtype))
+        m = m.to(dev).eval()
+        B, S = 2, 70
+        x = torch.randn(B, S, CFG.hidden_size, generator=torch.Generator().manual_seed(6)).to(dtype).to(dev)
+        cos, sin = (t.to(dev) for t in rope_tables(B, S, CFG.head_dim, dtype))
+        calls.clear(), library.clear()
+        with torch.no_grad():
+            m(x, (cos, sin), causal_mask(B, S, S, dtype).to(dev))
+        if own:
+            # head_dim 32 is padded to one K tile of 64; 70 keys to 128
+            assert calls == [((B, 8, S, 64), (B, 8, S, 64)), ((B, 8, S, 128), (B, 8, CFG.head_dim, 128))] and library == []
+        else:
+            assert calls == [] and len(library) == 2

@@ -106,3 +106,32 @@ def test_quantized_softmax_silu_rope_kvcache(dev, dtype):
         c, s_ = q(cos).unsqueeze(1), q(sin).unsqueeze(1)
         rot = lambda u: torch.cat((-u[..., 32:], u[..., :32]), -1)
         assert rel_err(qe, x * c + rot(x) * s_) < tol and rel_err(ke, (x * 2) * c + rot(x * 2) * s_) < tol
+
+
+def test_batched_products_run_on_the_kernel_of_this_package(dev, monkeypatch):
+    """bmm_mx* and matmul_mx* on batched operands: the quantized operands are exact in bf16, so the product runs on
+    mase_gemm_bf16_tn_batched whatever the tensors' dtype (fp32 results keep fp32 accumulation, rounded once);
+    9-bit MXINT mantissas and broadcast leading dimensions stay with torch."""
+    from mase_amd import _gemm
+    from mase_amd.quantized import bmm_mxint, matmul_mxfp, matmul_mxint
+
+    calls = []
+    real = _gemm.gemm_bf16_tn_batched
+    monkeypatch.setattr(_gemm, "gemm_bf16_tn_batched", lambda a, b, **kw: (calls.append(kw.get("out_dtype")), real(a, b, **kw))[1])
+    g = torch.Generator().manual_seed(13)
+    x = torch.randn(4, 50, 96, generator=g)
+    y = torch.randn(4, 96, 64, generator=g)
+    with torch.no_grad():
+        for dtype in (torch.float32, torch.bfloat16):
+            xd, yd = x.to(dtype).to(dev), y.to(dtype).to(dev)
+            calls.clear()
+            got = bmm_mxint(xd, yd, MXINT)
+            assert calls == [dtype] and got.dtype == dtype
+            assert rel_err(got, OM.matmul_mxint(x.to(dtype), y.to(dtype), MXINT, "bmm")) < (1e-5 if dtype == torch.float32 else 1e-2)
+            matmul_mxfp(xd, yd, MXFP)
+            assert len(calls) == 2
+        calls.clear()
+        wide = dict(MXINT, data_in_width=9)
+        matmul_mxint(x.to(dev), y.to(dev), wide)            # 9-bit mantissas are not bf16 values
+        matmul_mxint(x[:1].to(dev), y.to(dev), MXINT)        # broadcast over the batch
+        assert calls == []
