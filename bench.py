@@ -19,6 +19,8 @@ Secondary workloads (other rows of the path, same JSON; --dtype bf16|f32|f16 whe
     decode_linear  LinearMXInt 8192 -> 28672 for 16 tokens (weight-streaming kernel); decode_linear_packed: the same
                    with the weight streamed as int8 codes + scale bytes; decode_linear_mxfp4: LinearMXFP with e2m1
                    weights on the block-scaled MFMA
+    bmm_scores   the score product q k^T of an attention block on the batched matrix-core kernel (bound by writing
+                 the scores)
     copy         calibration copy
 Prints ONE JSON line.  `value` is algorithmic GB/s (Q-DQ) or TFLOP/s (Linear) over the whole timed region;
 `roofline` is for the dominant kernel, timed with HIP events on the launch stream; `cpu_baseline` is the CPU
@@ -675,6 +677,55 @@ class AttnProb(Workload):
                 "kind": "port", "sample": f"{n} passes of the separate tensor operations over 2 heads [1,2,2048,2048], {dt*1e3:.0f} ms each"}
 
 
+class BmmScores(Workload):
+    """the score product of a quantized attention block on its own: q [8, 32, 2048, 128] (a view of [batch, tokens,
+    heads, 128] memory, already MXINT8-quantized along the head dimension) times k^T, bf16 scores written to memory:
+    mase_gemm_bf16_tn_batched.  Bound by writing the [2048, 2048] score matrix of every head."""
+    name = "bmm_scores"
+    default_steps, default_warmup = 100, 10
+    unit = "GB/s"
+    dtype = "bf16"
+    kernel = "gemm_bf16_tn_kernel"
+    shape = (8, 32, 2048, 128)
+    metric = ("batched score product q k^T of an attention block (algorithmic bytes: 2 B per operand element read + 2 B "
+              "per score written)")
+    config = {"workload": "q, k bf16 [8,32,2048,128] as views of [batch, tokens, heads, 128], MXINT8 values, seed 9; scores "
+                          "bf16 [8,32,2048,2048]"}
+
+    def setup(self, torch, dev, n_buffers):
+        from mase_amd._gemm import gemm_bf16_tn_batched
+        from mase_amd.quantizers import _ops
+
+        self.op = gemm_bf16_tn_batched
+        B, H, T, D = self.shape
+        g = torch.Generator(device=dev).manual_seed(9)
+        mk = lambda: _ops.mxint_qdq(torch.randn(B, T, H, D, device=dev, generator=g).bfloat16(), 32, 8, -1, 8).transpose(1, 2)
+        self.sets = [(mk(), mk()) for _ in range(2)]
+        self.outs = [torch.empty(B, H, T, T, dtype=torch.bfloat16, device=dev) for _ in range(2)]
+
+    def step(self, i):
+        q, k = self.sets[i % 2]
+        self.out = self.op(q, k, out=self.outs[i % 2])
+
+    def work_per_step(self):
+        B, H, T, D = self.shape
+        return float(2 * B * H * T * D * 2 + B * H * T * T * 2)
+
+    def cpu_baseline(self, torch, budget_s):
+        q, k = (t[:1, :2].float().cpu() for t in self.sets[0])  # 2 heads of one batch item
+        t0 = time.perf_counter()
+        n = 0
+        while True:
+            torch.matmul(q, k.transpose(-1, -2))
+            n += 1
+            if time.perf_counter() - t0 > budget_s or n >= 50:
+                break
+        dt = (time.perf_counter() - t0) / n
+        T, D = self.shape[2], self.shape[3]
+        return {"value": 2 * (2 * T * D * 4 + T * T * 4) / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                "sample": f"{n} torch.matmul calls over 2 heads in fp32 (bytes counted at 4 B per element), {dt*1e3:.1f} ms each"}
+
+
 class AttentionCausal(Workload):
     """the decoder layer's attention core on its own: causal softmax(q k^T / sqrt(d)) v, bf16, batch 8 x 32 heads x 2048
     tokens x 128, operands as strided views of [batch, tokens, heads, 128] memory (what the projections produce)"""
@@ -835,7 +886,7 @@ class DecodeLinearMxfp4(Workload):
 
 WORKLOADS = {w.name: w for w in (MxintClipSearch, BfpQdq, MxintQdq, MxintLinear, MxintLinearCodes, MxfpLinear, DecoderLayerMxint, CopyBytes, IntegerQdq,
                                  MinifloatDenormQdq, MinifloatIeeeQdq, MinifloatMxQdq, MxfpQdq, AttnProb, DecodeLinear,
-                                 DecodeLinearPacked, DecodeLinearMxfp4, AttentionCausal, MfmaRateZeros, MfmaRateRandom, MfmaF8F4RateZeros,
+                                 DecodeLinearPacked, DecodeLinearMxfp4, AttentionCausal, BmmScores, MfmaRateZeros, MfmaRateRandom, MfmaF8F4RateZeros,
                                  MfmaF8F4RateRandom)}
 
 

@@ -372,6 +372,16 @@ int mase_attention_causal_fused(const void* q, const void* k, const void* v, voi
                                 size_t cs_stride_b, size_t cs_stride_t, int element_bits, const uint32_t* log2_tab,
                                 void* stream);
 
+/* Transposed copy of the trailing two dimensions of a 16-bit tensor: in[o][i][r][c] (row stride in_stride_row, batch
+ * strides in_stride_outer / in_stride_inner, all in elements, columns contiguous) -> out[o][i][c][r] contiguous with r
+ * padded with zeros to rows_padded (the next multiple of 64).  Prepares the second operand of the reference's
+ * torch.matmul / torch.bmm calls ([K, N] rows: the values of an attention block,
+ * nn/quantized/modules/llama/attention.py:449; y of bmm_mx*, nn/quantized/functional/matmul.py:437-512) for
+ * mase_gemm_bf16_tn_batched, which contracts rows with rows.  cols % 8 == 0; strides multiples of 8; pointers 16-byte
+ * aligned; at most 65535 batch items per call. */
+int mase_transpose16(const void* in, void* out, size_t batch_outer, size_t batch_inner, size_t rows, size_t cols,
+                     size_t rows_padded, size_t in_stride_outer, size_t in_stride_inner, size_t in_stride_row, void* stream);
+
 /* Rotary embedding out = x * cos + rotate_half(x) * sin for x [B, H, T, D] with the last dimension contiguous and
  * element strides (x_stride_b, x_stride_h, x_stride_t); out has the same strides; cos / sin tables [B or 1, T, D] with
  * strides (cs_stride_b, cs_stride_t), cs_stride_b = 0 for one table shared by the batch.  Products and sum are rounded to

@@ -182,6 +182,27 @@ def gemm_bf16_tn_batched(a: Tensor, b: Tensor, out_dtype: torch.dtype | None = N
     return out
 
 
+def transpose_last2(y: Tensor, rows_padded: int) -> Tensor:
+    """``y[..., K, N] -> [..., N, rows_padded]`` contiguous, columns K .. rows_padded - 1 zero (``mase_transpose16``
+    when the layout allows it: 16-bit elements, N a multiple of 8, last dimension contiguous, strides multiples of 8,
+    leading dimensions addressable by two nested indices; a strided copy of the library otherwise)"""
+    K, N = y.shape[-2], y.shape[-1]
+    out = torch.empty(y.shape[:-2] + (N, rows_padded), dtype=y.dtype, device=y.device)
+    split = _batch_strides(y)
+    if (y.is_cuda and y.element_size() == 2 and N % 8 == 0 and y.stride(-1) == 1 and rows_padded % 64 == 0
+            and 0 <= rows_padded - K < 64 and split is not None and split[0] * split[1] <= 65535
+            and not any(st % 8 for st in y.stride()[:-1]) and y.data_ptr() % 16 == 0):
+        n_outer, n_inner, s_outer, s_inner = split
+        rc = _lib.load().mase_transpose16(y.data_ptr(), out.data_ptr(), n_outer, n_inner, K, N, rows_padded, s_outer, s_inner,
+                                          y.stride(-2), _lib.stream_ptr(y))
+        _lib.check(rc, "mase_transpose16")
+        return out
+    if rows_padded != K:
+        out[..., K:].zero_()
+    out[..., :K].copy_(y.transpose(-1, -2))
+    return out
+
+
 def matmul_bf16(x: Tensor, y: Tensor, out: Tensor | None = None, out_dtype: torch.dtype | None = None) -> Tensor | None:
     """``torch.matmul(x, y)`` for bf16 device tensors x [..., M, K], y [..., K, N] with equal leading dimensions on the
     batched matrix-core kernel of this package (fp32 accumulation, one rounding to ``out_dtype``, bf16 unless given), or None when the operands do
@@ -198,9 +219,7 @@ def matmul_bf16(x: Tensor, y: Tensor, out: Tensor | None = None, out_dtype: torc
     if y.stride(-2) == 1 and not pad and y.stride(-1) >= K:  # already rows of K (a transposed view)
         yt = y.transpose(-1, -2)
     else:
-        yt = torch.zeros(y.shape[:-2] + (y.shape[-1], K + pad), dtype=y.dtype, device=y.device) if pad else \
-            torch.empty(y.shape[:-2] + (y.shape[-1], K), dtype=y.dtype, device=y.device)
-        yt[..., :K].copy_(y.transpose(-1, -2))
+        yt = transpose_last2(y, K + pad)
     if pad:
         x = torch.nn.functional.pad(x, (0, pad))
     elif x.stride(-1) != 1 or any(st % 8 for st in x.stride()[:-1]) or x.data_ptr() % 16:

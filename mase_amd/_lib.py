@@ -36,6 +36,7 @@ SIGNATURES = {
     "mase_minifloat_mx_qdq": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "mase_mxfp_qdq": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mase_gemm_bf16_tn": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_int, c_int, c_void_p]),
+    "mase_transpose16": (c_int, [c_void_p, c_void_p] + [c_size_t] * 8 + [c_void_p]),
     "mase_gemm_bf16_tn_batched": (c_int, [c_void_p, c_void_p, c_void_p] + [c_size_t] * 14 + [c_int, c_void_p]),
     "mase_gemm_bf16_tn_splitk_workspace_bytes": (c_size_t, [c_size_t, c_size_t, c_size_t]),
     "mase_gemm_bf16_tn_splitk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_int, c_int, c_void_p, c_size_t, c_void_p]),

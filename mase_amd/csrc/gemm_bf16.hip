@@ -154,18 +154,25 @@ __device__ __forceinline__ void load_2_untracked(uint32_t& dst, uint32_t off, co
 // BATCHED (plain form only): the work items are the output tiles of `batches` independent products with strided
 // operands (the score and value products of an attention block, torch.bmm): an item's operand bases and its output
 // base follow from its product index; rows of A, B and C have the strides lda, ldb, ldc.
-template <int OUT_DT, bool STREAM, bool BPACK = false, bool BCODES = false, bool BATCHED = false>
+// HALFN (plain form only): output tiles of 256 x 128 for products with at most 128 columns (the value product of an
+// attention block with head dimension 128), where a 256-wide tile would spend half of its matrix instructions on
+// columns that do not exist.  The wavefronts split the tile 2 x 2 into 128 rows x 64 columns (4 x 2 MFMA tiles, 8
+// MFMAs per K step); B's stage holds 128 rows.
+template <int OUT_DT, bool STREAM, bool BPACK = false, bool BCODES = false, bool BATCHED = false, bool HALFN = false>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p) {
-  constexpr int NI = BPACK ? 8 : 4, NJ = BPACK ? 2 : 4;  // MFMA tiles of a wavefront: rows x columns
+  constexpr int NI = BPACK ? 8 : 4, NJ = (BPACK || HALFN) ? 2 : 4;  // MFMA tiles of a wavefront: rows x columns
+  constexpr int kBN = HALFN ? 128 : BN;                           // columns of an output tile
+  constexpr int kCopiesB = HALFN ? kWaveCopies / 2 : kWaveCopies;  // copies of B per wavefront per K tile
   static_assert(!BCODES || BPACK, "codes come in fragment order");
   static_assert(!BATCHED || !BPACK, "the batched form takes row-major operands");
+  static_assert(!HALFN || !BPACK, "the narrow tile exists in the plain form");
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int tid = threadIdx.x;
   const int lane_id = tid & 63;
   const int lane = lane_id;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
-  const int row_base = BPACK ? 0 : wm * 128, col_base = BPACK ? wave * 64 : wn * 128;  // the wavefront's part of the tile
+  const int row_base = BPACK ? 0 : wm * 128, col_base = BPACK ? wave * 64 : wn * (HALFN ? 64 : 128);  // the wavefront's part of the tile
   const int nk = p.kc / BK;
 
   // ---- this work-group's output tiles.  Work-groups are dealt to the 8 XCDs round-robin; when the counts
@@ -197,7 +204,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     const int first_m = (t / in_group) * GROUP_M;
     const int gsz = min(p.tiles_m - first_m, GROUP_M);
     m0 = (first_m + (t % in_group) % gsz) * BM;
-    n0 = ((t % in_group) / gsz) * BN;
+    n0 = ((t % in_group) / gsz) * kBN;
   };
 
   // ---- global side of the async copies: wave w fills row groups w + 4*j (8 rows of 128 B each), j = 0..7
@@ -239,6 +246,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   auto issue_copy = [&](int c) __attribute__((always_inline)) {
     if constexpr (BPACK) {
       if (c & 1) return;  // B does not pass through LDS
+    }
+    if constexpr (HALFN) {
+      if ((c & 1) && (c >> 1) >= kCopiesB) return;  // B's stage holds 128 rows: row groups 0..15
     }
     const uint32_t st = lds_base + (uint32_t)(c_stage * kStride) + (c & 1) * kTileBytes;
     const int j = c >> 1;
@@ -293,7 +303,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
       const unsigned char* st = lds + stage * kStride;
       return __builtin_bit_cast(bf16x8_t, *(const uint4*)(st + lds_off(f * 32 + frag_row, s * 2 + kgrp)));
     } else {
-      const unsigned char* st = lds + stage * kStride + ((f < 4) ? (wm * 128) * kRowBytes : kTileBytes + (wn * 128) * kRowBytes);
+      const unsigned char* st = lds + stage * kStride + ((f < 4) ? (wm * 128) * kRowBytes : kTileBytes + (wn * (HALFN ? 64 : 128)) * kRowBytes);
       return __builtin_bit_cast(bf16x8_t, *(const uint4*)(st + lds_off((f & 3) * 32 + frag_row, s * 2 + kgrp)));
     }
   };
@@ -522,11 +532,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     b_kt = 1;
     wait_vmcnt<0>();
   } else {
-    wait_vmcnt<kCopies>();  // K tile 0 landed; K tile 1 may still be in flight
+    wait_vmcnt<kWaveCopies + kCopiesB>();  // K tile 0 landed; K tile 1 may still be in flight
   }
   asm volatile("s_barrier" ::: "memory");
 #pragma unroll
-  for (int f = 0; f < 8; ++f) fr[0][f] = load_frag(0, 0, f);
+  for (int f = 0; f < (HALFN ? 6 : 8); ++f) fr[0][f] = load_frag(0, 0, f);
   int stage = 0;
   // BPACK form of the K iteration.  The wavefront has two kinds of loads in flight, the B fragment loads into
   // registers and the A copies into LDS.  Each kind retires in order, but the two kinds do NOT retire in order with
@@ -670,6 +680,44 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     advance();
     stage ^= 1;
   };
+  // HALFN form of the plain K iteration: 8 MFMAs per step, MFMA t on (A row tile t / 2, B column tile t % 2); fragment
+  // sets hold 6 fragments (4 of A, then 2 of B); the 12 copies of the K tile after next go out one per MFMA slot of
+  // steps 2 and 3 (slots of the 4 copies that B does not have stay empty)
+  auto k_iteration_h = [&](auto&& advance) __attribute__((always_inline)) {
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) {
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        acc[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[s][4 + (t & 1)], fr[s][t >> 1],
+                                                                     acc[t >> 1][t & 1], 0, 0, 0);
+        if (s == 0) {
+          if (t < 6) fr[1][t] = load_frag(stage, 1, t);
+        } else if (s == 1) {
+          if (t < 6) {
+            fr[2][t] = load_frag(stage, 2, t);
+            fr[3][t] = load_frag(stage, 3, t);
+          }
+        } else if (s == 2) {
+          if (t < 6) fr[0][t] = load_frag(stage ^ 1, 0, t);
+          issue_copy(t);
+        } else {
+          issue_copy(8 + t);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (s == 1) {
+        wait_vmcnt<0>();
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    advance();
+    stage ^= 1;
+  };
+  auto k_iter_plain = [&](auto&& advance) __attribute__((always_inline)) {
+    if constexpr (HALFN) k_iteration_h(advance);
+    else k_iteration(advance);
+  };
   for (int ord = 0; ord < n_my; ++ord) {
     if constexpr (BPACK) {
       // two K tiles per trip (the fragment buffers alternate); the copy stream as in the plain form below, the B
@@ -696,14 +744,14 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     } else if constexpr (STREAM) {
       // the copy stream stands at K tile S of this output tile (or, if nk == S, at K tile 0 of the next)
 #pragma unroll 1
-      for (int kt = 0; kt < nk - S; ++kt) k_iteration(step_within_tile);
+      for (int kt = 0; kt < nk - S; ++kt) k_iter_plain(step_within_tile);
       // it moves on to the next output tile (past the last one: harmless re-copies of its first K tiles)
       set_copy_tile(ord + 1);
       c_kt = 0;
 #pragma unroll 1
-      for (int kt = 0; kt < S; ++kt) k_iteration(step_within_tile);
+      for (int kt = 0; kt < S; ++kt) k_iter_plain(step_within_tile);
     } else {
-      for (int kt = 0; kt < nk; ++kt) k_iteration(advance_copy_stream);
+      for (int kt = 0; kt < nk; ++kt) k_iter_plain(advance_copy_stream);
     }
     epilogue(ord);
     zero_acc();
@@ -739,22 +787,26 @@ int launch_gemm_bf16(const GemmParams& p, int out_dtype, hipStream_t st, bool bp
     hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, STREAM_>), grid, block, lds_bytes, st, p);                       \
   } while (0)
   if (batched) {
-#define MASE_GEMM_LAUNCH_BATCHED(DT_, STREAM_)                                                                    \
+    const bool halfn = p.N <= 128;  // the caller has counted tiles_n in tiles of 128 columns then
+#define MASE_GEMM_LAUNCH_BATCHED(DT_, STREAM_, HALFN_)                                                            \
   do {                                                                                                            \
     static std::atomic<uint64_t> attr_done{0};                                                                    \
-    const void* k = (const void*)gemm_bf16_tn_kernel<DT_, STREAM_, false, false, true>;                           \
+    const void* k = (const void*)gemm_bf16_tn_kernel<DT_, STREAM_, false, false, true, HALFN_>;                   \
     if (!set_dynamic_lds_once(attr_done, k, (int)lds_bytes)) return MASE_ERR_LAUNCH;                              \
-    hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, STREAM_, false, false, true>), grid, block, lds_bytes, st, p);   \
+    hipLaunchKernelGGL((gemm_bf16_tn_kernel<DT_, STREAM_, false, false, true, HALFN_>), grid, block, lds_bytes,   \
+                       st, p);                                                                                    \
   } while (0)
-    if (stream_fits) {
-      if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH_BATCHED(MASE_DT_F32, true);
-      else if (out_dtype == MASE_DT_BF16) MASE_GEMM_LAUNCH_BATCHED(MASE_DT_BF16, true);
-      else MASE_GEMM_LAUNCH_BATCHED(MASE_DT_F16, true);
-    } else {
-      if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH_BATCHED(MASE_DT_F32, false);
-      else if (out_dtype == MASE_DT_BF16) MASE_GEMM_LAUNCH_BATCHED(MASE_DT_BF16, false);
-      else MASE_GEMM_LAUNCH_BATCHED(MASE_DT_F16, false);
-    }
+#define MASE_GEMM_LAUNCH_BATCHED_DT(STREAM_, HALFN_)                                                              \
+  do {                                                                                                            \
+    if (out_dtype == MASE_DT_F32) MASE_GEMM_LAUNCH_BATCHED(MASE_DT_F32, STREAM_, HALFN_);                         \
+    else if (out_dtype == MASE_DT_BF16) MASE_GEMM_LAUNCH_BATCHED(MASE_DT_BF16, STREAM_, HALFN_);                  \
+    else MASE_GEMM_LAUNCH_BATCHED(MASE_DT_F16, STREAM_, HALFN_);                                                  \
+  } while (0)
+    if (stream_fits && halfn) MASE_GEMM_LAUNCH_BATCHED_DT(true, true);
+    else if (stream_fits) MASE_GEMM_LAUNCH_BATCHED_DT(true, false);
+    else if (halfn) MASE_GEMM_LAUNCH_BATCHED_DT(false, true);
+    else MASE_GEMM_LAUNCH_BATCHED_DT(false, false);
+#undef MASE_GEMM_LAUNCH_BATCHED_DT
 #undef MASE_GEMM_LAUNCH_BATCHED
   } else if (bpack && bcodes) {
     if (!stream_fits || ((p.kc / BK) & 1) != 0) return MASE_ERR_SHAPE;
@@ -918,7 +970,8 @@ extern "C" int mase_gemm_bf16_tn_batched(const void* A, const void* B, void* C, 
   // operand rows are fetched in 16-byte pieces at 32-bit byte offsets from the product's operand base; output pieces
   // of 16 bytes are stored whole where they lie inside a row
   if ((unsigned long long)M * lda * 2 > 0xFFFFFFFFull || (unsigned long long)N * ldb * 2 > 0xFFFFFFFFull) return MASE_ERR_SHAPE;
-  const unsigned long long tiles = (unsigned long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  const size_t bn = N <= 128 ? 128 : BN;  // products of at most 128 columns take output tiles of 256 x 128
+  const unsigned long long tiles = (unsigned long long)((M + BM - 1) / BM) * ((N + bn - 1) / bn);
   if (tiles * batch_outer * batch_inner > (1ull << 30) || batch_inner > (1u << 30)) return MASE_ERR_SHAPE;
   if (!aligned16(A) || !aligned16(B) || !aligned16(C)) return MASE_ERR_ALIGN;
   if (lda % 8 || ldb % 8 || a_stride_outer % 8 || a_stride_inner % 8 || b_stride_outer % 8 || b_stride_inner % 8)
@@ -935,7 +988,7 @@ extern "C" int mase_gemm_bf16_tn_batched(const void* A, const void* B, void* C, 
   p.K = (int)K;
   p.bias_dtype = 0;
   p.tiles_m = (int)((M + BM - 1) / BM);
-  p.tiles_n = (int)((N + BN - 1) / BN);
+  p.tiles_n = (int)((N + bn - 1) / bn);
   p.splits = 1;
   p.kc = (int)K;
   p.batches = (int)(batch_outer * batch_inner);

@@ -360,3 +360,34 @@ def test_batched_gemm_c_abi_checks(dev):
     assert call(lda=68) == -3 and call(csi=4100) == -3 and call(A=a.data_ptr() + 2) == -3   # alignment
     assert call(A=None) == -1 and call(dt=5) == -4
     assert call(bo=0) == 0 and call(M=0) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_transpose_last2_with_zero_padding(dev, dtype):
+    """mase_transpose16 against the tensor operation: views of [batch, tokens, heads, d] memory, ragged row counts
+    (padded with zeros to a multiple of 64), column counts that are not a multiple of the 64-wide tile, 3-D operands"""
+    from mase_amd import _gemm
+
+    g = torch.Generator().manual_seed(21)
+    cases = [torch.randn(2, 70, 3, 128, generator=g).to(dtype).to(dev).transpose(1, 2),   # [2, 3, 70, 128] view
+             torch.randn(5, 200, 72, generator=g).to(dtype).to(dev),
+             torch.randn(1, 2, 64, 8, generator=g).to(dtype).to(dev),
+             torch.randn(4, 130, 136, generator=g).to(dtype).to(dev)[:, :, :104]]
+    for y in cases:
+        K = y.shape[-2]
+        padded = (K + 63) // 64 * 64
+        got = _gemm.transpose_last2(y, padded)
+        assert got.shape == y.shape[:-2] + (y.shape[-1], padded) and got.is_contiguous()
+        assert torch.equal(got[..., :K], y.transpose(-1, -2))
+        assert bool((got[..., K:] == 0).all())
+    # what the kernel does not take goes through the library's copy with the same result
+    odd = torch.randn(3, 50, 12, generator=g).to(dtype).to(dev)      # 12 columns: not a multiple of 8
+    got = _gemm.transpose_last2(odd, 64)
+    assert torch.equal(got[..., :50], odd.transpose(-1, -2)) and bool((got[..., 50:] == 0).all())
+    lib = _gemm._lib.load()
+    a = torch.zeros(64, 64, dtype=dtype, device=dev)
+    assert lib.mase_transpose16(a.data_ptr(), a.data_ptr(), 1, 1, 64, 12, 64, 0, 0, 64, None) == -2
+    assert lib.mase_transpose16(a.data_ptr(), a.data_ptr(), 1, 1, 60, 64, 128, 0, 0, 64, None) == -2
+    assert lib.mase_transpose16(a.data_ptr(), a.data_ptr(), 1, 1, 64, 64, 64, 0, 0, 60, None) == -2
+    assert lib.mase_transpose16(a.data_ptr(), a.data_ptr(), 1, 1, 64, 64, 64, 4, 0, 64, None) == -3
+    assert lib.mase_transpose16(None, a.data_ptr(), 1, 1, 64, 64, 64, 0, 0, 64, None) == -1
