@@ -141,6 +141,58 @@ def minifloat_mx_decode(code: int, E: int, F: int, is_finite: bool):
     return (-v if sgn else v), sgn
 
 
+def minifloat_mx_value(xv: float, E: int, F: int, finite: bool, mode: str):
+    """What ``_minifloat_mx/fake.py:11-149`` (encode, then decode) computes for one finite fp32 value, stated on the
+    VALUE in exact rationals, with no bit field in sight: |x| = m 2^e; modes other than "rz" first drop what lies below
+    2^(e-15); r = the fraction in units of 2^(e-F) rounded in the mode on the magnitude; a fraction that rounds up to
+    2^F gives 2^(e+1) when e + bias is even and 2^e when it is odd (into the Inf code at the top of a format that has
+    one); e = -bias truncates to the subnormal grid (r = 0: zero; r = 2^F: 2^-bias); below that, and below 2^-126,
+    zero; above the top exponent the largest magnitude.  Returns (Fraction | "inf", negative).  The derivation and the
+    sweep that holds the vectorised restatement to it are in tests/test_minifloat_mx_value_pins.py."""
+    bias = 2 ** (E - 1) - 1
+    emax = (2 ** E - 1 if finite else 2 ** E - 2) - bias
+    neg = xv < 0
+    a = Fraction(abs(xv))
+    if a < Fraction(1, 2 ** 126):
+        return Fraction(0), neg
+    e = 0
+    while Fraction(2) ** (e + 1) <= a:
+        e += 1
+    while Fraction(2) ** e > a:
+        e -= 1
+    p = lambda k: Fraction(2) ** k
+    xt = a if mode == "rz" else (a / p(e - 15)).__floor__() * p(e - 15)
+    u = p(e - F)
+    q = (xt - p(e)) / u
+    fl = q.__floor__()
+    if mode == "rn":
+        rem = q - fl
+        r = fl + (1 if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1) else 0)
+    elif mode == "ru":
+        r = fl + (1 if q != fl else 0)
+    else:
+        r = fl
+    if e < -bias:
+        return Fraction(0), neg
+    if e > emax:
+        if emax + bias == 0:
+            return (2 ** F - 1) * p(1 - bias - F), neg
+        return (2 - p(-F)) * p(emax), neg
+    if e == -bias:
+        if r == 0:
+            return Fraction(0), neg
+        if r == 2 ** F:
+            return p(-bias), neg
+        return ((r + 2 ** F) // 2) * p(1 - bias - F), neg
+    if r == 2 ** F:
+        if (e + bias) % 2 == 1:
+            return p(e), neg
+        if not finite and e + bias + 1 == 2 ** E - 1:
+            return "inf", neg
+        return p(e + 1), neg
+    return (2 ** F + r) * u, neg
+
+
 def minifloat_representable(E: int, F: int, is_finite: bool):
     """all non-negative finite values of the format under the reference's decode"""
     vals = set()

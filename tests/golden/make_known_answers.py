@@ -137,6 +137,39 @@ def main():
             out["block_fp_bf16"].append({"width": width, "exponent_width": 8, "block": 16,
                                          "x": [bf16_bits(x) | 0 if not (x == 0 and str(x).startswith("-")) else 0x8000 for x in xs],
                                          "y": ys})
+    # the bit-level cast of the MX formats in the regions where the source's arithmetic departs from round-to-nearest
+    # (carry out of the fraction in odd / even exponent fields, exponent field 0, below 2^-bias, saturation, the low 8
+    # mantissa bits dropped before rounding).  Expected values from the value-domain statement in exact rationals
+    # (S.minifloat_mx_value), cross-checked here against the integer restatement of the bit fields.
+    out["minifloat_mx"] = []
+    rng2 = random.Random(77)
+    for (E, F) in ((4, 3), (5, 2), (2, 3), (3, 2), (2, 1), (1, 2)):
+        bias = (1 << (E - 1)) - 1
+        for finite in (True, False):
+            top = ((1 << E) - 1 if finite else (1 << E) - 2) - bias
+            xs = []
+            for e in sorted({-bias - 1, -bias, -bias + 1, -bias + 2, 0, top - 1, top, top + 1}):
+                if not -126 <= e <= 127:
+                    continue
+                for frac in (0.0, 1.0 - 2.0 ** -(F + 1), 1.0 - 2.0 ** -(F + 2), 2.0 ** -(F + 1), 2.0 ** -(F + 1) + 2.0 ** -23,
+                             2.0 ** -(F + 1) + 2.0 ** -15, 3 * 2.0 ** -(F + 1), rng2.random(), rng2.random()):
+                    xs.append(f32((1.0 + frac) * 2.0 ** e))
+            xs += [0.0, -0.0, 1e-40, -1e-40, 3.0e38, -3.0e38]
+            xs = [x if i % 3 else -x for i, x in enumerate(xs)]
+            for mode in ("rn", "ru", "rd", "rz"):
+                ys = []
+                for x in xs:
+                    v, neg = S.minifloat_mx_value(x, E, F, finite, mode)
+                    code = S.minifloat_mx_encode(bits(x), E, F, finite, mode)
+                    v2, sgn2 = S.minifloat_mx_decode(code, E, F, finite)
+                    if v == "inf":
+                        assert v2 in ("inf", "-inf"), (x, E, F, finite, mode)
+                        ys.append(0xFF800000 if neg else 0x7F800000)
+                        continue
+                    assert abs(v2) == v and bool(sgn2) == bool(neg), (x, E, F, finite, mode, v, v2)
+                    ys.append(frac_bits(v, negative_zero=(v == 0 and neg)) | (0x80000000 if (neg and v != 0) else 0))
+                out["minifloat_mx"].append({"exp_bits": E, "frac_bits": F, "is_finite": finite, "round_mode": mode,
+                                            "x": [bits(x) for x in xs], "y": ys})
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "known_answers.json")
     with open(path, "w") as f:
         json.dump(out, f, separators=(",", ":"))

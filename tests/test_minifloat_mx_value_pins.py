@@ -41,6 +41,7 @@ import pytest
 import torch
 
 import oracle as O
+from oracle.scalar import minifloat_mx_value as closed_form_fraction
 
 FORMATS = [(4, 3), (5, 2), (2, 3), (3, 2), (2, 1), (1, 2)]  # mxfp/meta.py:41
 MODES = ["rn", "ru", "rd", "rz"]
@@ -114,52 +115,6 @@ def closed_form(x: np.ndarray, E: int, F: int, finite: bool, mode: str, mutant: 
         val = np.where(inf_in, inf_value, val)
         val = np.where(nan_in, largest, val)
     return np.where(neg, -val, val)
-
-
-def closed_form_fraction(xv: float, E: int, F: int, finite: bool, mode: str):
-    """the same statement on one finite value in exact rationals; returns (Fraction | 'inf', negative)"""
-    bias = 2 ** (E - 1) - 1
-    emax = (2 ** E - 1 if finite else 2 ** E - 2) - bias
-    neg = xv < 0
-    a = Fraction(abs(xv))
-    if a < Fraction(1, 2 ** 126):
-        return Fraction(0), neg
-    e = 0
-    while Fraction(2) ** (e + 1) <= a:
-        e += 1
-    while Fraction(2) ** e > a:
-        e -= 1
-    p = lambda k: Fraction(2) ** k
-    xt = a if mode == "rz" else (a / p(e - 15)).__floor__() * p(e - 15)
-    u = p(e - F)
-    q = (xt - p(e)) / u
-    fl = q.__floor__()
-    if mode == "rn":
-        rem = q - fl
-        r = fl + (1 if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1) else 0)
-    elif mode == "ru":
-        r = fl + (1 if q != fl else 0)
-    else:
-        r = fl
-    if e < -bias:
-        return Fraction(0), neg
-    if e > emax:
-        if emax + bias == 0:
-            return (2 ** F - 1) * p(1 - bias - F), neg
-        return (2 - p(-F)) * p(emax), neg
-    if e == -bias:
-        if r == 0:
-            return Fraction(0), neg
-        if r == 2 ** F:
-            return p(-bias), neg
-        return ((r + 2 ** F) // 2) * p(1 - bias - F), neg
-    if r == 2 ** F:
-        if (e + bias) % 2 == 1:
-            return p(e), neg
-        if not finite and e + bias + 1 == 2 ** E - 1:
-            return "inf", neg
-        return p(e + 1), neg
-    return (2 ** F + r) * u, neg
 
 
 def swept_bits(E: int, F: int) -> np.ndarray:
