@@ -22,22 +22,27 @@ constexpr int kThreads = 256;
 __device__ __forceinline__ float bits2f(uint32_t b) { return __builtin_bit_cast(float, b); }
 __device__ __forceinline__ uint32_t f2bits(float f) { return __builtin_bit_cast(uint32_t, f); }
 
-// fp32 -> bf16 bits, round-to-nearest-even (NaN kept quiet)
-// fp32 -> bf16, round-to-nearest-even, with the hardware conversion of this part (two values per instruction,
-// first operand in the low half); NaN stays NaN
+// fp32 -> bf16, round-to-nearest-even, with the hardware conversion of this part (v_cvt_pk_bf16_f32: two values per
+// instruction, first operand in the low half); NaN stays NaN.  Written as a vector conversion, which the compiler
+// selects that instruction for, and not as the instruction by name: a vector instruction that reads the result of a
+// transcendental one (v_exp_f32, v_rcp_f32, ...) needs a wait state between the two on this part, which the compiler
+// inserts for instructions it knows and cannot for the text of an asm statement (seen as a wrong conversion of the
+// second of two exponentials, now and then).
 __device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
-  uint32_t r;
-  asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
-  return r;
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) { return f32x2_to_bf16x2_bits(f, 0.0f) & 0xFFFFu; }
 __device__ __forceinline__ float round_to_bf16(float f) { return bits2f(f32x2_to_bf16x2_bits(0.0f, f) & 0xFFFF0000u); }
 // fp32 -> fp16 bits, round-to-nearest-even.  Issued as an explicit instruction: when the compiler sees
 // "(half)(a * b)" it fuses the pair into a mixed-precision fma with a +0 addend, which turns a -0 product
-// into +0 and so loses the sign of zero that the reference keeps.
+// into +0 and so loses the sign of zero that the reference keeps.  The s_nop is the wait state that a reader of a
+// transcendental instruction's result needs (see above); the compiler does not look inside the statement.
 __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
   uint32_t h;
-  asm("v_cvt_f16_f32 %0, %1" : "=v"(h) : "v"(f));
+  asm("s_nop 0\n\tv_cvt_f16_f32 %0, %1" : "=v"(h) : "v"(f));
   return h & 0xFFFFu;
 }
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {

@@ -112,9 +112,11 @@ __device__ __forceinline__ float acc_read(float a) {
 }
 // The compiler separates a matrix instruction from a read of its result by the wait states the part requires, but it does
 // not look inside acc_read's assembly.  An epilogue therefore starts with this: more wait states than the longest
-// matrix instruction needs (19), issued after the K loop's last matrix instruction and, both being volatile assembly,
-// before the first acc_read.
-__device__ __forceinline__ void acc_read_fence() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
+// matrix instruction needs (19) plus the time the last matrix instructions may spend queued behind the ones before them,
+// issued after the K loop's last matrix instruction and, both being volatile assembly, before the first acc_read.
+__device__ __forceinline__ void acc_read_fence() {
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+}
 
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
