@@ -44,3 +44,37 @@ def test_linear_forward_replays_from_a_graph(dev, kind):
         torch.cuda.synchronize()
         assert torch.equal(static_y.view(torch.int16), eager_y.view(torch.int16))
         assert torch.equal(static_q.view(torch.int16), eager_q.view(torch.int16))
+
+
+@pytest.mark.parametrize("kind", ["mxint", "mxint-codes", "mxfp4"])
+def test_decode_sized_forward_replays_from_a_graph(dev, kind):
+    """16 rows of activations take the weight-streaming kernels (split-K partial sums in a workspace + a reduction):
+    the forward is recorded once and replayed with new inputs, with eager work and synchronisation between replays."""
+    from mase_amd.quantized import LinearMXFP, LinearMXInt
+
+    g = torch.Generator().manual_seed(22)
+    w = torch.randn(1536, 2048, generator=g) * 0.02
+    if kind == "mxfp4":
+        m = LinearMXFP(2048, 1536, bias=True, device=dev, dtype=torch.bfloat16, config=dict(MXFP))
+    else:
+        cfg = dict(MXINT, packed_decode=(kind == "mxint-codes"))
+        m = LinearMXInt(2048, 1536, bias=True, device=dev, dtype=torch.bfloat16, config=cfg)
+    m.load_state_dict({"weight": w.bfloat16(), "bias": (torch.randn(1536, generator=g) * 0.1).bfloat16()})
+    xs = [torch.randn(16, 2048, generator=g).bfloat16().to(dev) for _ in range(3)]
+    static_x = xs[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        m(static_x)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_y = m(static_x)
+    for x in xs + xs[:1]:
+        static_x.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager_y = m(x)
+        torch.cuda.synchronize()
+        assert torch.equal(static_y.view(torch.int16), eager_y.view(torch.int16))
