@@ -826,7 +826,7 @@ class DecodeLinear(Workload):
 class DecodeLinearPacked(DecodeLinear):
     """the same forward with the weight streamed as MXINT8 codes + scale bytes (config packed_decode)"""
     name = "decode_linear_packed"
-    kernel = "gemm_skinny_mxint8_partial_kernel"
+    kernel = "gemm_skinny_mxint8_shared_kernel"
     metric = ("MXINT8 Linear forward for 16 tokens, weight streamed as int8 codes + scale bytes (algorithmic bytes: "
               "1.03125 B per weight, read once)")
     config = {"workload": "LinearMXInt 8192 -> 28672 with packed_decode, 16 tokens, bf16, weights N(0,0.02) seed 7"}

@@ -35,7 +35,7 @@ struct SkinnyParams {
   const unsigned char* B;   // [N, K] bf16
   float* P;                 // [KS, M, N] fp32 partial results
   int M, N, K;
-  int kc;                   // K elements per split (multiple of 64)
+  int kc;                   // K elements per K range (multiple of 64); the last range holds what is left of K
 };
 
 // as in gemm_bf16.hip: 16-byte chunk `chunk` of row `row` (rows of 128 bytes), conflict-free for ds_read_b128
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_partial_kernel(Ski
   const unsigned char* abase = p.A + (size_t)ks * p.kc * 2;
   unsigned char* ring = lds + wave * (kSkStages * kSkStageBytes);
   const uint32_t ring_addr = (uint32_t)(uintptr_t)(lptr_t)ring;
-  const int chunks = p.kc / kSkChunk;
+  const int chunks = min(p.kc, p.K - ks * p.kc) / kSkChunk;
   // Work-group b walks its K range starting at chunk b mod chunks and wraps around (its four wavefronts stay in step
   // and share their reads of A).  Weight rows lie K*2 bytes apart,
   // for the usual K a power of two: wavefronts walking in step would all ask for the same few memory channels at any
@@ -169,7 +169,7 @@ struct SkinnyQParams {
   const unsigned char* Bs;   // [N, K/32] scale bytes
   float* P;
   int M, N, K;
-  int kc;                    // K elements per split (multiple of 128)
+  int kc;                    // K elements per K range (multiple of 128); the last range holds what is left of K
 };
 
 __device__ __forceinline__ void sk_async_copy4(const unsigned char* base, uint32_t off, uint32_t lds_addr) {
@@ -222,9 +222,11 @@ __global__ __launch_bounds__(kSqThreads) void gemm_skinny_mxint8_partial_kernel(
   const unsigned char* abase = p.A + (size_t)ks * p.kc * 2;
   unsigned char* ring = lds + wave * (S * G::kStageBytes);
   const uint32_t ring_addr = (uint32_t)(uintptr_t)(lptr_t)ring;
-  const int chunks = p.kc / kSqChunk;
+  const int chunks = min(p.kc, p.K - ks * p.kc) / kSqChunk;
+  const int rot = (int)((unsigned)blockIdx.x % (unsigned)chunks);  // rotated start, as in the bf16 kernel
   auto issue = [&](int c) __attribute__((always_inline)) {  // chunk c (clamped: past the end re-copies the last chunk)
-    const int cc = min(c, chunks - 1);
+    int cc = min(c, chunks - 1) + rot;
+    cc = cc >= chunks ? cc - chunks : cc;
     const uint32_t st = ring_addr + (uint32_t)((c % S) * G::kStageBytes);
 #pragma unroll
     for (int j = 0; j < 4; ++j) sk_async_copy(cbase + (size_t)cc * 128, offc[j], st + j * 1024);
@@ -284,6 +286,128 @@ __global__ __launch_bounds__(kSqThreads) void gemm_skinny_mxint8_partial_kernel(
   }
 }
 
+
+// The same kernel with the chunk of A shared by the work-group's four wavefronts instead of copied once per wavefront:
+// a stage holds the four wavefronts' code chunks and scale bytes and ONE chunk of A, so the ring is about twice as deep
+// in the same LDS and A crosses the vector-memory path once per work-group, at the price of one barrier per chunk (each
+// wavefront copies a quarter of A's chunk, waits for its own copies and meets the others).  Used for more than 8 rows
+// of A, where A's chunk is as large as a wavefront's codes or larger (measured on 28672 x 8192, reduction included:
+// 16 rows 67 -> 57 us, 32 rows 76 -> 60 us; with 8 rows or fewer the kernel above, whose ring is then deeper, is as fast
+// or faster).
+template <int XC>
+struct SqsGeom {
+  static constexpr int kWaveBytes = 32 * 128 + 256;            // codes and scale bytes of one wavefront's chunk
+  static constexpr int kABytes = XC * 8 * 256;                 // the chunk of A: 8 XC rows x 128 bf16
+  static constexpr int kStageBytes = kSqWaves * kWaveBytes + kABytes;
+  static constexpr int kACopies = (2 * XC + kSqWaves - 1) / kSqWaves;  // of A, per wavefront
+  static constexpr int kCopies = 4 + 1 + kACopies;
+  static constexpr int kFit = (160 * 1024) / kStageBytes;
+  static constexpr int kStages = kFit > 8 ? 8 : kFit;
+  static constexpr int kLdsBytes = kStages * kStageBytes;
+};
+
+template <int XC>
+__global__ __launch_bounds__(kSqThreads) void gemm_skinny_mxint8_shared_kernel(SkinnyQParams p) {
+  using G = SqsGeom<XC>;
+  constexpr int S = G::kStages;
+  static_assert((S - 1) * G::kCopies < 64, "outstanding copies must fit the 6-bit counter");
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  const int r = lane & 31, g = lane >> 5;
+  const int n0 = ((int)blockIdx.x * kSqWaves + wave) * 32;  // rows beyond N are clamped: every wavefront reaches the barriers
+  const int ks = blockIdx.y;
+  uint32_t offc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = 8 * j + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    offc[j] = (uint32_t)((size_t)min(n0 + row, p.N - 1) * (size_t)p.K) + chunk * 16;
+  }
+  const uint32_t offs = (uint32_t)((size_t)min(n0 + r, p.N - 1) * (size_t)(p.K / 32));
+  // A: copy j (0 .. 2*XC-1) moves rows 4j .. 4j+3 (256 bytes each); this wavefront issues copies wave, wave + 4, ...
+  // clamped to the last one (a repeated copy writes the same bytes to the same place)
+  uint32_t offa[G::kACopies];
+  int ja[G::kACopies];
+#pragma unroll
+  for (int i = 0; i < G::kACopies; ++i) {
+    ja[i] = min(wave + kSqWaves * i, 2 * XC - 1);
+    const int row = 4 * ja[i] + (lane >> 4);
+    const int chunk = (lane & 15) ^ (row & 15);
+    offa[i] = (uint32_t)((size_t)min(row, p.M - 1) * (size_t)p.K * 2) + chunk * 16;
+  }
+  const unsigned char* cbase = p.Bc + (size_t)ks * p.kc;
+  const unsigned char* sbase = p.Bs + (size_t)ks * (p.kc / 32);
+  const unsigned char* abase = p.A + (size_t)ks * p.kc * 2;
+  const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)lds;
+  const int chunks = min(p.kc, p.K - ks * p.kc) / kSqChunk;
+  const int rot = (int)((unsigned)blockIdx.x % (unsigned)chunks);
+  constexpr int kOffA = kSqWaves * G::kWaveBytes;
+  auto issue = [&](int c) __attribute__((always_inline)) {  // chunk c (clamped: past the end re-copies the last chunk)
+    int cc = min(c, chunks - 1) + rot;
+    cc = cc >= chunks ? cc - chunks : cc;
+    const uint32_t st = lds_addr + (uint32_t)((c % S) * G::kStageBytes);
+    const uint32_t mine = st + (uint32_t)(wave * G::kWaveBytes);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sk_async_copy(cbase + (size_t)cc * 128, offc[j], mine + j * 1024);
+    sk_async_copy4(sbase + (size_t)cc * 4, offs, mine + 4096);
+#pragma unroll
+    for (int i = 0; i < G::kACopies; ++i) sk_async_copy(abase + (size_t)cc * 256, offa[i], st + kOffA + ja[i] * 1024);
+  };
+
+  f32x16_t acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+  for (int c = 0; c < S - 1; ++c) issue(c);
+  const int arow = min(r, 8 * XC - 1);
+  for (int c = 0; c < chunks; ++c) {
+    // This wavefront's copies of chunk c have landed; behind the barrier so have the others' (their parts of A), and
+    // every wavefront has finished reading chunk c - 1, whose stage the copies issued next overwrite.
+    sk_wait_vmcnt<(S - 2) * G::kCopies>();
+    __builtin_amdgcn_s_barrier();
+    issue(c + S - 1);
+    const unsigned char* st = lds + (c % S) * G::kStageBytes;
+    const unsigned char* mine = st + wave * G::kWaveBytes;
+    const uint32_t sc4 = *(const uint32_t*)(mine + 4096 + r * 4);  // the row's 4 scale bytes of this chunk
+    float scale4[4], bias4[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const uint32_t sb = (sc4 >> (8 * b)) & 0xFFu;
+      scale4[b] = bits2f(sb >= 8u ? (sb - 7u) << 23 : 0u);
+      bias4[b] = -128.0f * scale4[b];
+    }
+#pragma unroll
+    for (int step = 0; step < 8; ++step) {
+      const uint2 cw = *(const uint2*)(mine + r * 128 + ((step ^ ((r >> 1) & 7)) << 4) + g * 8);
+      const uint4 xv = *(const uint4*)(st + kOffA + arow * 256 + (((2 * step + g) ^ (arow & 15)) << 4));
+      const float scale = scale4[step >> 1], bias = bias4[step >> 1];
+      uint4 wv;
+      codes4_to_bf16(cw.x, scale, bias, wv.x, wv.y);
+      codes4_to_bf16(cw.y, scale, bias, wv.z, wv.w);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wv), __builtin_bit_cast(bf16x8_t, xv), acc,
+                                                    0, 0, 0);
+    }
+  }
+  sk_wait_vmcnt<0>();  // no copy may still be in flight towards LDS when the wavefront retires
+  float* out = p.P + (size_t)ks * p.M * p.N;
+  const int m = r;
+  if (m < p.M && n0 < p.N) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int n = n0 + q * 8 + g * 4;
+      float* o = out + (size_t)m * p.N + n;
+      if (n + 3 < p.N && (p.N & 3) == 0) {
+        *(float4*)o = make_float4(acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (n + j < p.N) o[j] = acc[q * 4 + j];
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // The few-rows product on packed MXFP operands with the block-scaled matrix instruction: activations as e4m3 / e5m2
 // codes [M, K] and weights as e2m1 codes [N, K/2] (two per byte), one E8M0 scale byte per 32 elements each (the
@@ -311,7 +435,8 @@ struct SkinnyFParams {
   const unsigned char* Ws;   // [N, K/32]
   float* P;
   int M, N, K;
-  int kc;                    // K elements per split (multiple of 128)
+  int kc;                    // K elements per K range (multiple of 128); the last range holds what is left of K
+  int rotate;                // slab kernel: work-group b starts at chunk b mod chunks (pays with a single K range)
 };
 
 template <int XC, int CBSZ>
@@ -350,7 +475,7 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_mxfp4_partial_kern
   const unsigned char* xsbase = p.Xs + (size_t)ks * (p.kc / 32);
   unsigned char* ring = lds + wave * (S * G::kStageBytes);
   const uint32_t ring_addr = (uint32_t)(uintptr_t)(lptr_t)ring;
-  const int chunks = p.kc / 128;
+  const int chunks = min(p.kc, p.K - ks * p.kc) / 128;
   constexpr int kOffWs = G::kWBytes, kOffX = G::kWBytes + G::kScaleBytes, kOffXs = kOffX + G::kXBytes;
   auto issue = [&](int c) __attribute__((always_inline)) {  // chunk c (clamped: past the end re-copies the last chunk)
     const int cc = min(c, chunks - 1);
@@ -425,7 +550,7 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_mxfp4_slab_kernel(
   const int r = lane & 31, g = lane >> 5;
   const int n0 = ((int)blockIdx.x * 4 + wave) * 32;  // rows beyond N are clamped: every wavefront reaches the barrier
   const int ks = blockIdx.y;
-  const int nch = p.kc / 256;
+  const int nch = min(p.kc, p.K - ks * p.kc) / 256;
   const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)lds;
   const uint32_t xcodes_addr = lds_addr, xscales_addr = lds_addr + (uint32_t)(XR * p.kc);
   const unsigned char* xcodes = lds;
@@ -463,8 +588,13 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_mxfp4_slab_kernel(
   const uint32_t offws = (uint32_t)((size_t)min(n0 + (lane >> 1), p.N - 1) * (size_t)(p.K / 32)) + (uint32_t)((lane & 1) * 4);
   const unsigned char* wbase = p.Wc + (size_t)ks * (p.kc / 2);
   const unsigned char* wsbase = p.Ws + (size_t)ks * (p.kc / 32);
+  // with one K range per weight row the work-groups start at different chunks, as in the bf16 kernel (28672 x 8192,
+  // 8 tokens, reduction included: 33.5 -> 31 us); with two ranges the rotation costs time (36.5 -> 39.5 us), so the
+  // host asks for it only with one
+  const int rot = p.rotate ? (int)((unsigned)blockIdx.x % (unsigned)nch) : 0;
   auto issue = [&](int c) __attribute__((always_inline)) {  // chunk c (clamped: past the end re-copies the last chunk)
-    const int cc = min(c, nch - 1);
+    int cc = min(c, nch - 1) + rot;
+    cc = cc >= nch ? cc - nch : cc;
     const uint32_t st = ring_addr + (uint32_t)((c % S) * kSlabStageBytes);
 #pragma unroll
     for (int j = 0; j < 4; ++j) sk_async_copy(wbase + (size_t)cc * 128, offw[j], st + j * 1024);
@@ -485,9 +615,11 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_mxfp4_slab_kernel(
     issue(c + S - 1);
     sk_wait_vmcnt<(S - 1) * kSlabCopies>();  // chunk c has landed; the later ones may be in flight
     const unsigned char* st = ring + (c % S) * kSlabStageBytes;
-    const unsigned char* xc = xcodes + c * (XR * 256) + xrow * 256;
+    int cx = c + rot;  // the chunk of the slab that goes with the weights of this stage
+    cx = cx >= nch ? cx - nch : cx;
+    const unsigned char* xc = xcodes + cx * (XR * 256) + xrow * 256;
     const uint2 swv = *(const uint2*)(st + 4096 + r * 8);
-    const uint2 sxv = *(const uint2*)(xscales + c * 256 + xrow * 8);
+    const uint2 sxv = *(const uint2*)(xscales + cx * 256 + xrow * 8);
 #pragma unroll
     for (int step = 0; step < 4; ++step) {
       const uint4 x0 = *(const uint4*)(xc + (((step * 4 + g) ^ xsw) << 4));
@@ -521,15 +653,19 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_mxfp4_slab_kernel(
 
 int skinny_splits(int M, int N, int K, int n_cu);
 
-// K ranges of the slab kernel: at least as many as the LDS needs (slab rows * kc + kc <= 160 KB - rings), then as many
-// as skinny_splits would take; each a whole number of 256-element chunks
+// K elements per range when `chunks` chunks of `chunk` elements are cut into `splits` ranges: equal ranges of whole
+// chunks, the last one possibly shorter
+int range_elems(int K, int chunk, int splits) { return ((K / chunk) + splits - 1) / splits * chunk; }
+
+// K ranges of the slab kernel: at least as many as the LDS needs (slab rows * kc + kc <= 160 KB - rings) and as
+// skinny_splits would take; ranges of whole 256-element chunks, none of them empty
 int slab_splits(int rows8, int M, int N, int K, int n_cu) {
   const int chunks = K / 256;
   const int kc_max = ((kSlabLdsMax - kSlabRingBytes) / (rows8 + 1)) / 256 * 256;
-  int want = skinny_splits(M, N, K / 2, n_cu);
-  for (int s = 1; s <= chunks; ++s) {
-    if (chunks % s != 0) continue;
-    if (K / s <= kc_max && s >= want) return s;
+  const int want = skinny_splits(M, N, K / 2, n_cu);
+  for (int s = want; s < chunks; ++s) {
+    const int kc = range_elems(K, 256, s);
+    if (kc <= kc_max && (s - 1) * kc < K) return s;
   }
   return chunks;
 }
@@ -555,7 +691,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_reduce_kernel(const float* __
   else ((uint16_t*)C)[i] = (uint16_t)f32_to_f16_bits(s);
 }
 
-// K ranges (each a whole number of 64-element chunks, all equal).  A work-group takes the CU's whole LDS, so the
+// Number of K ranges for a K of `K / 64` chunks (kernels with longer chunks pass a proportionally smaller K): ranges of
+// ceil(chunks / ranges) chunks, the last one possibly shorter.  A work-group takes the CU's whole LDS, so the
 // work-groups run in rounds of n_cu; the number of ranges is chosen for the smallest estimated time
 //   rounds * (time of one work-group, proportional to its K range)  scaled by  (1 + partial-result traffic / B's bytes)
 // where the partial results cost ranges * rows * N * 8 bytes against N * K * 2 of B; ties go to fewer ranges.
@@ -566,13 +703,18 @@ int skinny_splits(int M, int N, int K, int n_cu) {
   const int rows = M < 32 ? M : 32;
   int best = 1;
   double best_cost = 1e300;
-  for (int s = 1; s <= chunks && s <= 64; ++s) {
-    if (chunks % s != 0) continue;
+  int last_s = 0;
+  for (int len = chunks; len >= 1; --len) {  // candidate range lengths, longest first = fewest ranges first
+    const int s = (chunks + len - 1) / len;
+    if (s == last_s) continue;
+    last_s = s;
+    if (s > 64) break;
+    const int range = (chunks + s - 1) / s;
     const long wgs = (long)groups * s;
     const long rounds = (wgs + n_cu - 1) / n_cu;
     const double overhead = 4.0 * s * rows / (double)K;
     // a short K range leaves the ring's start-up (a few chunks) exposed
-    const double per_wg = (double)(chunks / s) + 4.0;
+    const double per_wg = (double)range + 4.0;
     const double cost = (double)rounds * per_wg * (1.0 + overhead);
     if (cost < best_cost * 0.999) { best_cost = cost; best = s; }
   }
@@ -626,7 +768,7 @@ extern "C" int mase_gemm_bf16_skinny(const void* A, const void* B, const void* b
   p.B = (const unsigned char*)B;
   p.N = (int)N;
   p.K = (int)K;
-  p.kc = (int)K / splits;
+  p.kc = range_elems((int)K, kSkChunk, splits);
   // one pass per group of 32 rows of A; the partial results of a group form a [splits, rows, N] block, and the
   // blocks of successive groups are laid out so that together they read as [splits, M, N] per group offset
   for (size_t m0 = 0; m0 < M; m0 += 32) {
@@ -679,11 +821,15 @@ extern "C" int mase_gemm_mxint8_skinny(const void* A, const int8_t* B_codes, con
   hipStream_t st = (hipStream_t)stream;
   static std::atomic<uint64_t> attr_done{0};
   if (!device_setup_done(attr_done)) {
-    const void* ks[4] = {(const void*)gemm_skinny_mxint8_partial_kernel<1>, (const void*)gemm_skinny_mxint8_partial_kernel<2>,
-                         (const void*)gemm_skinny_mxint8_partial_kernel<3>, (const void*)gemm_skinny_mxint8_partial_kernel<4>};
-    const int sz[4] = {SqGeom<1>::kLdsBytes, SqGeom<2>::kLdsBytes, SqGeom<3>::kLdsBytes, SqGeom<4>::kLdsBytes};
-    for (int i = 0; i < 4; ++i)
-      if (hipFuncSetAttribute(ks[i], hipFuncAttributeMaxDynamicSharedMemorySize, sz[i]) != hipSuccess)
+    // up to 8 rows of A: a ring per wavefront; more: the chunk of A shared by the work-group
+    if (hipFuncSetAttribute((const void*)gemm_skinny_mxint8_partial_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            SqGeom<1>::kLdsBytes) != hipSuccess)
+      return MASE_ERR_LAUNCH;
+    const void* kh[3] = {(const void*)gemm_skinny_mxint8_shared_kernel<2>, (const void*)gemm_skinny_mxint8_shared_kernel<3>,
+                         (const void*)gemm_skinny_mxint8_shared_kernel<4>};
+    const int szh[3] = {SqsGeom<2>::kLdsBytes, SqsGeom<3>::kLdsBytes, SqsGeom<4>::kLdsBytes};
+    for (int i = 0; i < 3; ++i)
+      if (hipFuncSetAttribute(kh[i], hipFuncAttributeMaxDynamicSharedMemorySize, szh[i]) != hipSuccess)
         return MASE_ERR_LAUNCH;
     mark_device_setup_done(attr_done);
   }
@@ -693,7 +839,7 @@ extern "C" int mase_gemm_mxint8_skinny(const void* A, const int8_t* B_codes, con
   p.Bs = (const unsigned char*)B_scales;
   p.N = (int)N;
   p.K = (int)K;
-  p.kc = (int)K / splits;
+  p.kc = range_elems((int)K, kSqChunk, splits);
   for (size_t m0 = 0; m0 < M; m0 += 32) {
     const size_t rows = (M - m0 < 32) ? (M - m0) : 32;
     p.A = (const unsigned char*)A + m0 * K * 2;
@@ -701,9 +847,9 @@ extern "C" int mase_gemm_mxint8_skinny(const void* A, const int8_t* B_codes, con
     p.M = (int)rows;
     const int xc = (int)(rows + 7) / 8;
     if (xc == 1) hipLaunchKernelGGL(gemm_skinny_mxint8_partial_kernel<1>, grid, block, SqGeom<1>::kLdsBytes, st, p);
-    else if (xc == 2) hipLaunchKernelGGL(gemm_skinny_mxint8_partial_kernel<2>, grid, block, SqGeom<2>::kLdsBytes, st, p);
-    else if (xc == 3) hipLaunchKernelGGL(gemm_skinny_mxint8_partial_kernel<3>, grid, block, SqGeom<3>::kLdsBytes, st, p);
-    else hipLaunchKernelGGL(gemm_skinny_mxint8_partial_kernel<4>, grid, block, SqGeom<4>::kLdsBytes, st, p);
+    else if (xc == 2) hipLaunchKernelGGL(gemm_skinny_mxint8_shared_kernel<2>, grid, block, SqsGeom<2>::kLdsBytes, st, p);
+    else if (xc == 3) hipLaunchKernelGGL(gemm_skinny_mxint8_shared_kernel<3>, grid, block, SqsGeom<3>::kLdsBytes, st, p);
+    else hipLaunchKernelGGL(gemm_skinny_mxint8_shared_kernel<4>, grid, block, SqsGeom<4>::kLdsBytes, st, p);
     const size_t mn_g = rows * N;
     const dim3 rgrid_g((unsigned)blocks_for(mn_g, 256));
     void* Cg = (unsigned char*)C + m0 * N * (out_dtype == MASE_DT_F32 ? 4 : 2);
@@ -783,7 +929,8 @@ extern "C" int mase_gemm_mxfp4_skinny(const void* A_codes, const void* A_scales,
   p.Ws = (const unsigned char*)B_scales;
   p.N = (int)N;
   p.K = (int)K;
-  p.kc = (int)K / splits;
+  p.kc = range_elems((int)K, slab ? 256 : 128, splits);
+  p.rotate = (slab && splits == 1) ? 1 : 0;
   for (size_t m0 = 0; m0 < M; m0 += 32) {
     const size_t rows = (M - m0 < 32) ? (M - m0) : 32;
     p.Xc = (const unsigned char*)A_codes + m0 * K;

@@ -98,10 +98,11 @@ def test_gemm_wrappers_split_oversized_activations(dev, monkeypatch):
 
 
 @pytest.mark.parametrize("M", [1, 7, 32, 33, 64, 100, 128])
-@pytest.mark.parametrize("N,K", [(33, 64), (256, 4096), (4100, 1024), (11008, 4096), (4096, 11008)])
+@pytest.mark.parametrize("N,K", [(33, 64), (256, 4096), (4100, 1024), (11008, 4096), (4096, 11008), (520, 2368), (2048, 5504)])
 def test_gemm_few_rows_takes_the_weight_streaming_kernel(dev, M, N, K):
     """M <= 128: the kernel that splits N and K over the chip and adds the K ranges in a fixed order.  Exact on
-    small-integer operands, within fp32 summation error on random ones, and reproducible run to run."""
+    small-integer operands, within fp32 summation error on random ones, and reproducible run to run.  K = 2368 and
+    5504 are 37 and 86 chunks: no equal cut into ranges exists, the last range is shorter."""
     from mase_amd import _gemm
 
     assert M <= _gemm.SKINNY_MAX_ROWS
@@ -131,7 +132,7 @@ def test_gemm_few_rows_with_mxint8_coded_weights(dev, M):
     from mase_amd.quantizers import _ops
 
     g = torch.Generator().manual_seed(M)
-    for (N, K) in [(256, 128), (4096, 4096), (1000, 1152), (11008, 4096)]:
+    for (N, K) in [(256, 128), (4096, 4096), (1000, 1152), (11008, 4096), (300, 5504), (2048, 3968)]:  # 43, 31 chunks: unequal K ranges
         w = (torch.randn(N, K, generator=g) * 0.05)
         w[3] *= 2.0 ** -40            # a row of tiny blocks (small scale bytes)
         w[5, :64] = 0.0               # all-zero blocks

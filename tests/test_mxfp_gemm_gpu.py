@@ -209,7 +209,7 @@ def test_gemm_mxfp4_few_rows_streams_the_weight_codes(dev, afmt, M):
     from mase_amd._gemm import gemm_mxfp4_skinny, gemm_mxfp_scaled, mxfp_pack
 
     g = torch.Generator().manual_seed(M * 7 + afmt[0])
-    for (N, K) in [(64, 128), (4096, 4096), (1000, 1152), (11008, 2048)]:
+    for (N, K) in [(64, 128), (4096, 4096), (1000, 1152), (11008, 2048), (512, 7936), (4096, 11008)]:  # 31, 43 chunks: unequal K ranges
         a = torch.randn(M, K, generator=g)
         a[:, 5] *= 20
         b = torch.randn(N, K, generator=g) * 0.02
