@@ -839,7 +839,7 @@ class DecodeLinearMxfp4(Workload):
     name = "decode_linear_mxfp4"
     unit = "GB/s"
     dtype = "fp8"
-    kernel = "gemm_skinny_mxfp4_slab_kernel"
+    kernel = "gemm_skinny_mxfp4_shared_kernel"
     M, N, K = 16, 28672, 8192
     metric = ("MXFP4-weight Linear forward for 16 tokens (algorithmic bytes: e2m1 codes + E8M0 scales, 0.53125 B per "
               "weight, read once)")

@@ -7,8 +7,9 @@
 // (whole 128-byte lines per row, several stages in flight to cover the HBM latency; no barrier anywhere: nothing
 // is shared between wavefronts), multiplies with v_mfma_f32_32x32x16_bf16 and writes a 32 x M partial result;
 // a second small kernel adds the partial results of the K ranges in a fixed order (deterministic, no atomics),
-// adds the bias and converts.  More than 32 rows of A take one pass per group of 32 (B then comes from the
-// last-level cache on the later passes).
+// adds the bias and converts; with a single K range the first kernel does that itself and the second is not
+// launched.  More than 32 rows of A take one pass per group of 32 (B then comes from the last-level cache on the
+// later passes).
 #include "common.hpp"
 
 namespace mase {
@@ -30,10 +31,76 @@ struct SkGeom {
   static constexpr int kLdsBytes = 4 * kStages * kStageBytes;  // per work-group of 4 wavefronts
 };
 
+// Where a kernel's 32 x M result goes.  With several K ranges: partial sums [range][M][N] in the workspace, which the
+// reduce kernel adds in order.  With a single range the kernel finishes the job itself (C != null): the value the
+// reduce kernel would compute from the one partial sum (0 + sum, + bias), converted and written to C, and no second
+// launch.
+struct SkinnyOut {
+  float* P;           // [ranges, M, N] fp32 partial results
+  void* C;            // [M, N] in out_dtype, or null
+  const void* bias;   // [N] in bias_dtype, or null
+  int out_dtype, bias_dtype;
+};
+
+__device__ __forceinline__ float skinny_bias(const void* bias, int dt, int col) {
+  if (dt == MASE_DT_F32) return ((const float*)bias)[col];
+  if (dt == MASE_DT_BF16) return bits2f((uint32_t)((const uint16_t*)bias)[col] << 16);
+  return f16_bits_to_f32(((const uint16_t*)bias)[col]);
+}
+
+__device__ __forceinline__ float skinny_finish(const SkinnyOut& o, float sum, int col) {
+  float s = 0.0f;
+  s += sum;  // as the reduce kernel starts from zero: a sum of -0 comes out as +0 either way
+  if (o.bias != nullptr) s += skinny_bias(o.bias, o.bias_dtype, col);
+  return s;
+}
+
+__device__ __forceinline__ uint32_t skinny_to16(int dt, float v) {
+  return dt == MASE_DT_BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+}
+
+// element (m, n) of the result, from a lane that holds single elements
+__device__ __forceinline__ void skinny_put(const SkinnyOut& o, int ks, int M, int N, int m, int n, float sum) {
+  const size_t i = (size_t)m * N + n;
+  if (o.C == nullptr) {
+    o.P[(size_t)ks * M * N + i] = sum;
+  } else {
+    const float v = skinny_finish(o, sum, n);
+    if (o.out_dtype == MASE_DT_F32) ((float*)o.C)[i] = v;
+    else ((uint16_t*)o.C)[i] = (uint16_t)skinny_to16(o.out_dtype, v);
+  }
+}
+
+// elements (m, n .. n + 3) of the result, from a lane that holds four consecutive columns
+__device__ __forceinline__ void skinny_put4(const SkinnyOut& o, int ks, int M, int N, int m, int n, float s0, float s1,
+                                            float s2, float s3) {
+  if (n + 3 < N && (N & 3) == 0) {
+    const size_t i = (size_t)m * N + n;
+    if (o.C == nullptr) {
+      *(float4*)(o.P + (size_t)ks * M * N + i) = make_float4(s0, s1, s2, s3);
+    } else {
+      const float v0 = skinny_finish(o, s0, n), v1 = skinny_finish(o, s1, n + 1), v2 = skinny_finish(o, s2, n + 2),
+                  v3 = skinny_finish(o, s3, n + 3);
+      if (o.out_dtype == MASE_DT_F32) {
+        *(float4*)((float*)o.C + i) = make_float4(v0, v1, v2, v3);
+      } else {
+        const int dt = o.out_dtype;
+        *(uint2*)((uint16_t*)o.C + i) = make_uint2(skinny_to16(dt, v0) | (skinny_to16(dt, v1) << 16),
+                                                   skinny_to16(dt, v2) | (skinny_to16(dt, v3) << 16));
+      }
+    }
+  } else {
+    const float sv[4] = {s0, s1, s2, s3};
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (n + j < N) skinny_put(o, ks, M, N, m, n + j, sv[j]);
+  }
+}
+
 struct SkinnyParams {
   const unsigned char* A;   // [M, K] bf16, M <= 32 (this pass's rows)
   const unsigned char* B;   // [N, K] bf16
-  float* P;                 // [KS, M, N] fp32 partial results
+  SkinnyOut o;
   int M, N, K;
   int kc;                   // K elements per K range (multiple of 64); the last range holds what is left of K
 };
@@ -123,21 +190,11 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_partial_kernel(Ski
   sk_wait_vmcnt<0>();  // no copy may still be in flight towards LDS when the wavefront retires
   // acc[q*4 + j] = sum_k B[n0 + q*8 + g*4 + j][k] * A[r][k]: for this lane's row m = r of A, four consecutive
   // columns n per q
-  float* out = p.P + (size_t)ks * p.M * p.N;
   const int m = r;
   if (m < p.M) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int n = n0 + q * 8 + g * 4;
-      float* o = out + (size_t)m * p.N + n;
-      if (n + 3 < p.N && (p.N & 3) == 0) {
-        *(float4*)o = make_float4(acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if (n + j < p.N) o[j] = acc[q * 4 + j];
-      }
-    }
+    for (int q = 0; q < 4; ++q)
+      skinny_put4(p.o, ks, p.M, p.N, m, n0 + q * 8 + g * 4, acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]);
   }
 }
 
@@ -167,7 +224,7 @@ struct SkinnyQParams {
   const unsigned char* A;    // [M, K] bf16, M <= 32
   const unsigned char* Bc;   // [N, K] int8 codes
   const unsigned char* Bs;   // [N, K/32] scale bytes
-  float* P;
+  SkinnyOut o;
   int M, N, K;
   int kc;                    // K elements per K range (multiple of 128); the last range holds what is left of K
 };
@@ -268,21 +325,11 @@ __global__ __launch_bounds__(kSqThreads) void gemm_skinny_mxint8_partial_kernel(
     }
   }
   sk_wait_vmcnt<0>();  // no copy may still be in flight towards LDS when the wavefront retires
-  float* out = p.P + (size_t)ks * p.M * p.N;
   const int m = r;
   if (m < p.M) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int n = n0 + q * 8 + g * 4;
-      float* o = out + (size_t)m * p.N + n;
-      if (n + 3 < p.N && (p.N & 3) == 0) {
-        *(float4*)o = make_float4(acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if (n + j < p.N) o[j] = acc[q * 4 + j];
-      }
-    }
+    for (int q = 0; q < 4; ++q)
+      skinny_put4(p.o, ks, p.M, p.N, m, n0 + q * 8 + g * 4, acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]);
   }
 }
 
@@ -390,21 +437,11 @@ __global__ __launch_bounds__(kSqThreads) void gemm_skinny_mxint8_shared_kernel(S
     }
   }
   sk_wait_vmcnt<0>();  // no copy may still be in flight towards LDS when the wavefront retires
-  float* out = p.P + (size_t)ks * p.M * p.N;
   const int m = r;
   if (m < p.M && n0 < p.N) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int n = n0 + q * 8 + g * 4;
-      float* o = out + (size_t)m * p.N + n;
-      if (n + 3 < p.N && (p.N & 3) == 0) {
-        *(float4*)o = make_float4(acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if (n + j < p.N) o[j] = acc[q * 4 + j];
-      }
-    }
+    for (int q = 0; q < 4; ++q)
+      skinny_put4(p.o, ks, p.M, p.N, m, n0 + q * 8 + g * 4, acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]);
   }
 }
 
@@ -433,10 +470,10 @@ struct SkinnyFParams {
   const unsigned char* Xs;   // [M, K/32]
   const unsigned char* Wc;   // [N, K/2] e2m1 codes
   const unsigned char* Ws;   // [N, K/32]
-  float* P;
+  SkinnyOut o;
   int M, N, K;
   int kc;                    // K elements per K range (multiple of 128); the last range holds what is left of K
-  int rotate;                // slab kernel: work-group b starts at chunk b mod chunks (pays with a single K range)
+  int rotate;                // shared-chunk kernel: work-group b starts at chunk b mod chunks (pays with a single K range)
 };
 
 template <int XC, int CBSZ>
@@ -516,7 +553,6 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_mxfp4_partial_kern
   }
   sk_wait_vmcnt<0>();  // no copy may still be in flight towards LDS when the wavefront retires
   // acc[q*4 + j] = C[token q*8 + g*4 + j][weight row n0 + r]
-  float* out = p.P + (size_t)ks * p.M * p.N;
   const int n = n0 + r;
   if (n < p.N) {
 #pragma unroll
@@ -524,59 +560,48 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_mxfp4_partial_kern
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int m = q * 8 + g * 4 + j;
-        if (m < p.M) out[(size_t)m * p.N + n] = acc[q * 4 + j];
+        if (m < p.M) skinny_put(p.o, ks, p.M, p.N, m, n, acc[q * 4 + j]);
       }
   }
 }
 
-// The same product with the activation codes of the work-group's K range resident in LDS.  The kernel above copies
-// the activation chunk once per wavefront and chunk, which doubles its copy instructions, and reads the weight rows in
-// 64-byte pieces.  Here the work-group first copies its [rows, kc] slab of activation codes and scales into LDS (shared
-// by the 4 wavefronts, one barrier), and the per-wavefront rings carry weights only, in chunks of 256 elements of K
-// (128 bytes per weight row, 5 copies per 4 KB).  LDS: slab rows*kc + kc bytes, rings 4 x kSlabStages x 4352 bytes;
-// the host picks the number of K ranges so that this fits.  K % 256 == 0.
-// Slab layout: [chunk][row][256 B] with the 16-byte granule j of a row stored at position j ^ (row & 15), so that the
-// 16 lanes a ds_read_b128 serves together (16 rows, same granule) fall into different banks; scales [chunk][32][8 B].
-constexpr int kSlabStages = 5, kSlabStageBytes = 4096 + 256, kSlabCopies = 5;
-constexpr int kSlabRingBytes = 4 * kSlabStages * kSlabStageBytes;
-constexpr int kSlabLdsMax = 160 * 1024;
+// The same product with the chunk of activation codes shared by the work-group's four wavefronts.  The kernel above
+// copies the activation chunk once per wavefront and chunk, which doubles its copy instructions, and reads the weight
+// rows in 64-byte pieces.  Here a stage of the ring holds the four wavefronts' weight chunks of 256 elements of K
+// (128 bytes per weight row, 4 copies per 4 KB, plus their scale bytes) and ONE chunk of activation codes and scales,
+// of which each wavefront copies a quarter; one barrier per chunk makes the parts visible and frees the stage that
+// the next copies overwrite.  Nothing grows with K, so one K range serves any K where the weight has enough rows to
+// fill the chip, and every work-group starts up once (28672 x 8192, reduction included: 16 tokens 32 us, 32 tokens
+// 36 us; a form that kept the activations of the whole K range in LDS needed two ranges for 16 tokens and four for 32:
+// 38 and 48 us).  K % 256 == 0.
+// Activation chunk layout: [row][256 B] with the 16-byte granule j of a row stored at position j ^ (row & 15), so that
+// the 16 lanes a ds_read_b128 serves together (16 rows, same granule) fall into different banks; scales [32][8 B].
+template <int XC>
+struct SfsGeom {
+  static constexpr int kWaveBytes = 4096 + 256;                 // weight codes and scale bytes of one wavefront's chunk
+  static constexpr int kXBytes = XC * 8 * 256;                  // the chunk of activation codes: 8 XC rows x 256
+  static constexpr int kXsBytes = 256;                          // their scale bytes: [32 rows][8]
+  static constexpr int kStageBytes = 4 * kWaveBytes + kXBytes + kXsBytes;
+  static constexpr int kXCopies = (2 * XC + 3) / 4;             // of the activation codes, per wavefront
+  static constexpr int kCopies = 4 + 1 + kXCopies + 1;
+  static constexpr int kFit = (160 * 1024) / kStageBytes;
+  static constexpr int kStages = kFit > 8 ? 8 : kFit;
+  static constexpr int kLdsBytes = kStages * kStageBytes;
+};
 
 template <int XC, int CBSZ>
-__global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_mxfp4_slab_kernel(SkinnyFParams p) {
-  constexpr int XR = 8 * XC, S = kSlabStages;
+__global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_mxfp4_shared_kernel(SkinnyFParams p) {
+  using G = SfsGeom<XC>;
+  constexpr int XR = 8 * XC, S = G::kStages;
+  static_assert((S - 1) * G::kCopies < 64, "outstanding copies must fit the 6-bit counter");
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
   const int r = lane & 31, g = lane >> 5;
-  const int n0 = ((int)blockIdx.x * 4 + wave) * 32;  // rows beyond N are clamped: every wavefront reaches the barrier
+  const int n0 = ((int)blockIdx.x * 4 + wave) * 32;  // rows beyond N are clamped: every wavefront reaches the barriers
   const int ks = blockIdx.y;
   const int nch = min(p.kc, p.K - ks * p.kc) / 256;
   const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)lds;
-  const uint32_t xcodes_addr = lds_addr, xscales_addr = lds_addr + (uint32_t)(XR * p.kc);
-  const unsigned char* xcodes = lds;
-  const unsigned char* xscales = lds + XR * p.kc;
-  unsigned char* ring = lds + XR * p.kc + p.kc + wave * (S * kSlabStageBytes);
-  const uint32_t ring_addr = xscales_addr + (uint32_t)p.kc + (uint32_t)(wave * (S * kSlabStageBytes));
-
-  // activation slab: copy t moves rows 4q .. 4q+3 of chunk c (t = c * (XR/4) + q); lane -> row 4q + lane/16, slot lane%16
-  {
-    const unsigned char* xbase = p.Xc + (size_t)ks * p.kc;
-    const int total = nch * (XR / 4);
-    for (int t0 = 0; t0 < total; t0 += 4) {
-      const int t = min(t0 + wave, total - 1);
-      const int c = t / (XR / 4), q = t % (XR / 4);
-      const int row = 4 * q + (lane >> 4);
-      const int gran = (lane & 15) ^ (row & 15);
-      const uint32_t off = (uint32_t)((size_t)min(row, p.M - 1) * (size_t)p.K) + (uint32_t)(gran * 16);
-      sk_async_copy(xbase + (size_t)c * 256, off, xcodes_addr + (uint32_t)(c * (XR * 256) + q * 1024));
-    }
-    const unsigned char* xsbase = p.Xs + (size_t)ks * (p.kc / 32);
-    const uint32_t offs = (uint32_t)((size_t)min(lane >> 1, p.M - 1) * (size_t)(p.K / 32)) + (uint32_t)((lane & 1) * 4);
-    for (int c0 = 0; c0 < nch; c0 += 4) {
-      const int c = min(c0 + wave, nch - 1);
-      sk_async_copy4(xsbase + (size_t)c * 8, offs, xscales_addr + (uint32_t)(c * 256));
-    }
-  }
   // weights: copy j (0..3) moves rows 8j .. 8j+7 (128 bytes per row per chunk); scales: lane -> row lane/2, dword lane%2
   uint32_t offw[4];
 #pragma unroll
@@ -586,45 +611,62 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_mxfp4_slab_kernel(
     offw[j] = (uint32_t)((size_t)min(n0 + row, p.N - 1) * (size_t)(p.K / 2)) + (uint32_t)(gran * 16);
   }
   const uint32_t offws = (uint32_t)((size_t)min(n0 + (lane >> 1), p.N - 1) * (size_t)(p.K / 32)) + (uint32_t)((lane & 1) * 4);
+  // activations: copy q (0 .. 2*XC-1) moves rows 4q .. 4q+3 (256 bytes per row per chunk): lane -> row 4q + lane/16,
+  // granule lane%16 stored at position granule ^ (row & 15); this wavefront issues copies wave, wave + 4, ... clamped to
+  // the last one (a repeated copy writes the same bytes to the same place)
+  uint32_t offx[G::kXCopies];
+  int qx[G::kXCopies];
+#pragma unroll
+  for (int i = 0; i < G::kXCopies; ++i) {
+    qx[i] = min(wave + 4 * i, 2 * XC - 1);
+    const int row = 4 * qx[i] + (lane >> 4);
+    const int gran = (lane & 15) ^ (row & 15);
+    offx[i] = (uint32_t)((size_t)min(row, p.M - 1) * (size_t)p.K) + (uint32_t)(gran * 16);
+  }
+  const uint32_t offxs = (uint32_t)((size_t)min(lane >> 1, p.M - 1) * (size_t)(p.K / 32)) + (uint32_t)((lane & 1) * 4);
   const unsigned char* wbase = p.Wc + (size_t)ks * (p.kc / 2);
   const unsigned char* wsbase = p.Ws + (size_t)ks * (p.kc / 32);
-  // with one K range per weight row the work-groups start at different chunks, as in the bf16 kernel (28672 x 8192,
-  // 8 tokens, reduction included: 33.5 -> 31 us); with two ranges the rotation costs time (36.5 -> 39.5 us), so the
-  // host asks for it only with one
+  const unsigned char* xbase = p.Xc + (size_t)ks * p.kc;
+  const unsigned char* xsbase = p.Xs + (size_t)ks * (p.kc / 32);
+  // with one K range per weight row the work-groups start at different chunks, as in the bf16 kernel (16 tokens:
+  // 34 -> 32 us); with several ranges the rotation gains nothing or costs time, so the host asks for it only with one
   const int rot = p.rotate ? (int)((unsigned)blockIdx.x % (unsigned)nch) : 0;
+  constexpr int kOffX = 4 * G::kWaveBytes, kOffXs = kOffX + G::kXBytes;
   auto issue = [&](int c) __attribute__((always_inline)) {  // chunk c (clamped: past the end re-copies the last chunk)
     int cc = min(c, nch - 1) + rot;
     cc = cc >= nch ? cc - nch : cc;
-    const uint32_t st = ring_addr + (uint32_t)((c % S) * kSlabStageBytes);
+    const uint32_t st = lds_addr + (uint32_t)((c % S) * G::kStageBytes);
+    const uint32_t mine = st + (uint32_t)(wave * G::kWaveBytes);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) sk_async_copy(wbase + (size_t)cc * 128, offw[j], st + j * 1024);
-    sk_async_copy4(wsbase + (size_t)cc * 8, offws, st + 4096);
+    for (int j = 0; j < 4; ++j) sk_async_copy(wbase + (size_t)cc * 128, offw[j], mine + j * 1024);
+    sk_async_copy4(wsbase + (size_t)cc * 8, offws, mine + 4096);
+#pragma unroll
+    for (int i = 0; i < G::kXCopies; ++i) sk_async_copy(xbase + (size_t)cc * 256, offx[i], st + kOffX + qx[i] * 1024);
+    sk_async_copy4(xsbase + (size_t)cc * 8, offxs, st + kOffXs);  // by every wavefront alike: the counts stay uniform
   };
   f32x16_t acc;
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
 #pragma unroll
   for (int c = 0; c < S - 1; ++c) issue(c);
-  // the slab's copies are older than the ring's: with at most the ring's in flight, this wavefront's part of the slab has
-  // landed; the barrier makes the other wavefronts' parts visible
-  sk_wait_vmcnt<(S - 1) * kSlabCopies>();
-  __builtin_amdgcn_s_barrier();
   const int xrow = min(r, XR - 1);
   const int xsw = xrow & 15, wsw = (r >> 1) & 7;
   for (int c = 0; c < nch; ++c) {
+    // This wavefront's copies of chunk c have landed; behind the barrier so have the others' (their parts of the
+    // activations), and every wavefront has finished reading chunk c - 1, whose stage the copies issued next overwrite.
+    sk_wait_vmcnt<(S - 2) * G::kCopies>();
+    __builtin_amdgcn_s_barrier();
     issue(c + S - 1);
-    sk_wait_vmcnt<(S - 1) * kSlabCopies>();  // chunk c has landed; the later ones may be in flight
-    const unsigned char* st = ring + (c % S) * kSlabStageBytes;
-    int cx = c + rot;  // the chunk of the slab that goes with the weights of this stage
-    cx = cx >= nch ? cx - nch : cx;
-    const unsigned char* xc = xcodes + cx * (XR * 256) + xrow * 256;
-    const uint2 swv = *(const uint2*)(st + 4096 + r * 8);
-    const uint2 sxv = *(const uint2*)(xscales + cx * 256 + xrow * 8);
+    const unsigned char* st = lds + (c % S) * G::kStageBytes;
+    const unsigned char* mine = st + wave * G::kWaveBytes;
+    const unsigned char* xc = st + kOffX + xrow * 256;
+    const uint2 swv = *(const uint2*)(mine + 4096 + r * 8);
+    const uint2 sxv = *(const uint2*)(st + kOffXs + xrow * 8);
 #pragma unroll
     for (int step = 0; step < 4; ++step) {
       const uint4 x0 = *(const uint4*)(xc + (((step * 4 + g) ^ xsw) << 4));
       const uint4 x1 = *(const uint4*)(xc + (((step * 4 + 2 + g) ^ xsw) << 4));
-      const uint4 w0 = *(const uint4*)(st + r * 128 + (((step * 2 + g) ^ wsw) << 4));
+      const uint4 w0 = *(const uint4*)(mine + r * 128 + (((step * 2 + g) ^ wsw) << 4));
       const int sw = (int)((step < 2 ? swv.x : swv.y) >> (8 * g));
       const int sx = (int)((step < 2 ? sxv.x : sxv.y) >> (8 * g));
       i32x8_t a, b;
@@ -638,7 +680,6 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_mxfp4_slab_kernel(
   }
   sk_wait_vmcnt<0>();  // no copy may still be in flight towards LDS when the wavefront retires
   // acc[q*4 + j] = C[token q*8 + g*4 + j][weight row n0 + r]
-  float* out = p.P + (size_t)ks * p.M * p.N;
   const int n = n0 + r;
   if (n < p.N) {
 #pragma unroll
@@ -646,10 +687,11 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_mxfp4_slab_kernel(
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int m = q * 8 + g * 4 + j;
-        if (m < p.M) out[(size_t)m * p.N + n] = acc[q * 4 + j];
+        if (m < p.M) skinny_put(p.o, ks, p.M, p.N, m, n, acc[q * 4 + j]);
       }
   }
 }
+
 
 int skinny_splits(int M, int N, int K, int n_cu);
 
@@ -657,23 +699,14 @@ int skinny_splits(int M, int N, int K, int n_cu);
 // chunks, the last one possibly shorter
 int range_elems(int K, int chunk, int splits) { return ((K / chunk) + splits - 1) / splits * chunk; }
 
-// K ranges of the slab kernel: at least as many as the LDS needs (slab rows * kc + kc <= 160 KB - rings) and as
-// skinny_splits would take; ranges of whole 256-element chunks, none of them empty
-int slab_splits(int rows8, int M, int N, int K, int n_cu) {
+// K ranges of the shared-chunk MXFP4 kernel: as many as skinny_splits would take, in whole 256-element chunks, none
+// of them empty
+int mxfp4_shared_splits(int M, int N, int K, int n_cu) {
   const int chunks = K / 256;
-  const int kc_max = ((kSlabLdsMax - kSlabRingBytes) / (rows8 + 1)) / 256 * 256;
   const int want = skinny_splits(M, N, K / 2, n_cu);
-  for (int s = want; s < chunks; ++s) {
-    const int kc = range_elems(K, 256, s);
-    if (kc <= kc_max && (s - 1) * kc < K) return s;
-  }
+  for (int s = want; s < chunks; ++s)
+    if ((s - 1) * range_elems(K, 256, s) < K) return s;
   return chunks;
-}
-
-__device__ __forceinline__ float skinny_bias(const void* bias, int dt, int col) {
-  if (dt == MASE_DT_F32) return ((const float*)bias)[col];
-  if (dt == MASE_DT_BF16) return bits2f((uint32_t)((const uint16_t*)bias)[col] << 16);
-  return f16_bits_to_f32(((const uint16_t*)bias)[col]);
 }
 
 // C[m][n] = sum over the K ranges, in order, of P[ks][m][n]  (+ bias[n]), converted to the output dtype
@@ -719,6 +752,31 @@ int skinny_splits(int M, int N, int K, int n_cu) {
     if (cost < best_cost * 0.999) { best_cost = cost; best = s; }
   }
   return best;
+}
+
+// The tail of a pass over up to 32 rows of A: with one K range and a 16-byte aligned output block the kernel has
+// written C itself; otherwise the reduce kernel adds the ranges.
+void skinny_launch_reduce(const SkinnyOut& o, void* Cg, const void* bias, int out_dtype, int bias_dtype, size_t rows, size_t N,
+                          int splits, hipStream_t st) {
+  if (o.C != nullptr) return;
+  const size_t mn_g = rows * N;
+  const dim3 rgrid_g((unsigned)blocks_for(mn_g, 256));
+  if (out_dtype == MASE_DT_F32)
+    hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_F32>, rgrid_g, dim3(256), 0, st, o.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
+  else if (out_dtype == MASE_DT_BF16)
+    hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_BF16>, rgrid_g, dim3(256), 0, st, o.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
+  else
+    hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_F16>, rgrid_g, dim3(256), 0, st, o.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
+}
+
+SkinnyOut skinny_out(float* P, void* Cg, const void* bias, int out_dtype, int bias_dtype, int splits) {
+  SkinnyOut o;
+  o.P = P;
+  o.C = (splits == 1 && aligned16(Cg)) ? Cg : nullptr;
+  o.bias = bias;
+  o.out_dtype = out_dtype;
+  o.bias_dtype = bias_dtype;
+  return o;
 }
 
 int skinny_cu_count() {
@@ -774,22 +832,15 @@ extern "C" int mase_gemm_bf16_skinny(const void* A, const void* B, const void* b
   for (size_t m0 = 0; m0 < M; m0 += 32) {
     const size_t rows = (M - m0 < 32) ? (M - m0) : 32;
     p.A = (const unsigned char*)A + m0 * K * 2;
-    p.P = (float*)workspace + (size_t)splits * m0 * N;
+    void* Cg = (unsigned char*)C + m0 * N * (out_dtype == MASE_DT_F32 ? 4 : 2);
+    p.o = skinny_out((float*)workspace + (size_t)splits * m0 * N, Cg, bias, out_dtype, bias_dtype, splits);
     p.M = (int)rows;
     const int xc = (int)(rows + 7) / 8;
     if (xc == 1) hipLaunchKernelGGL(gemm_skinny_partial_kernel<1>, grid, block, SkGeom<1>::kLdsBytes, st, p);
     else if (xc == 2) hipLaunchKernelGGL(gemm_skinny_partial_kernel<2>, grid, block, SkGeom<2>::kLdsBytes, st, p);
     else if (xc == 3) hipLaunchKernelGGL(gemm_skinny_partial_kernel<3>, grid, block, SkGeom<3>::kLdsBytes, st, p);
     else hipLaunchKernelGGL(gemm_skinny_partial_kernel<4>, grid, block, SkGeom<4>::kLdsBytes, st, p);
-    const size_t mn_g = rows * N;
-    const dim3 rgrid_g((unsigned)blocks_for(mn_g, 256));
-    void* Cg = (unsigned char*)C + m0 * N * (out_dtype == MASE_DT_F32 ? 4 : 2);
-    if (out_dtype == MASE_DT_F32)
-      hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_F32>, rgrid_g, dim3(256), 0, st, p.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
-    else if (out_dtype == MASE_DT_BF16)
-      hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_BF16>, rgrid_g, dim3(256), 0, st, p.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
-    else
-      hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_F16>, rgrid_g, dim3(256), 0, st, p.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
+    skinny_launch_reduce(p.o, Cg, bias, out_dtype, bias_dtype, rows, N, splits, st);
   }
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
@@ -843,34 +894,24 @@ extern "C" int mase_gemm_mxint8_skinny(const void* A, const int8_t* B_codes, con
   for (size_t m0 = 0; m0 < M; m0 += 32) {
     const size_t rows = (M - m0 < 32) ? (M - m0) : 32;
     p.A = (const unsigned char*)A + m0 * K * 2;
-    p.P = (float*)workspace + (size_t)splits * m0 * N;
+    void* Cg = (unsigned char*)C + m0 * N * (out_dtype == MASE_DT_F32 ? 4 : 2);
+    p.o = skinny_out((float*)workspace + (size_t)splits * m0 * N, Cg, bias, out_dtype, bias_dtype, splits);
     p.M = (int)rows;
     const int xc = (int)(rows + 7) / 8;
     if (xc == 1) hipLaunchKernelGGL(gemm_skinny_mxint8_partial_kernel<1>, grid, block, SqGeom<1>::kLdsBytes, st, p);
     else if (xc == 2) hipLaunchKernelGGL(gemm_skinny_mxint8_shared_kernel<2>, grid, block, SqsGeom<2>::kLdsBytes, st, p);
     else if (xc == 3) hipLaunchKernelGGL(gemm_skinny_mxint8_shared_kernel<3>, grid, block, SqsGeom<3>::kLdsBytes, st, p);
     else hipLaunchKernelGGL(gemm_skinny_mxint8_shared_kernel<4>, grid, block, SqsGeom<4>::kLdsBytes, st, p);
-    const size_t mn_g = rows * N;
-    const dim3 rgrid_g((unsigned)blocks_for(mn_g, 256));
-    void* Cg = (unsigned char*)C + m0 * N * (out_dtype == MASE_DT_F32 ? 4 : 2);
-    if (out_dtype == MASE_DT_F32)
-      hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_F32>, rgrid_g, dim3(256), 0, st, p.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
-    else if (out_dtype == MASE_DT_BF16)
-      hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_BF16>, rgrid_g, dim3(256), 0, st, p.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
-    else
-      hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_F16>, rgrid_g, dim3(256), 0, st, p.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
+    skinny_launch_reduce(p.o, Cg, bias, out_dtype, bias_dtype, rows, N, splits, st);
   }
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
 
 namespace mase {
 namespace {
-// K % 256 == 0 takes the slab kernel (the same number of K ranges for every pass of 32 rows), other K the ring-only one
+// K % 256 == 0 takes the shared-chunk kernel, other K the ring-only one
 int mxfp4_skinny_splits(size_t M, size_t N, size_t K, int n_cu) {
-  if (K % 256 == 0) {
-    const int rows = (int)(M < 32 ? M : 32);
-    return slab_splits((rows + 7) / 8 * 8, (int)M, (int)N, (int)K, n_cu);
-  }
+  if (K % 256 == 0) return mxfp4_shared_splits((int)M, (int)N, (int)K, n_cu);
   return skinny_splits((int)M, (int)N, (int)(K / 2), n_cu);
 }
 }  // namespace
@@ -900,18 +941,19 @@ extern "C" int mase_gemm_mxfp4_skinny(const void* A_codes, const void* A_scales,
   const int n_cu = skinny_cu_count();
   if (n_cu <= 0) return MASE_ERR_LAUNCH;
   const int splits = mxfp4_skinny_splits(M, N, K, n_cu);
-  const bool slab = (K % 256) == 0;
+  const bool shared = (K % 256) == 0;
   const size_t need = (size_t)splits * M * N * sizeof(float);
   if (workspace == nullptr || workspace_bytes < need || (((uintptr_t)workspace) & 15u) != 0) return MASE_ERR_WORKSPACE;
   hipStream_t st = (hipStream_t)stream;
   static std::atomic<uint64_t> attr_done{0};
   if (!device_setup_done(attr_done)) {
-    const void* sl[8] = {(const void*)gemm_skinny_mxfp4_slab_kernel<1, 0>, (const void*)gemm_skinny_mxfp4_slab_kernel<2, 0>,
-                         (const void*)gemm_skinny_mxfp4_slab_kernel<3, 0>, (const void*)gemm_skinny_mxfp4_slab_kernel<4, 0>,
-                         (const void*)gemm_skinny_mxfp4_slab_kernel<1, 1>, (const void*)gemm_skinny_mxfp4_slab_kernel<2, 1>,
-                         (const void*)gemm_skinny_mxfp4_slab_kernel<3, 1>, (const void*)gemm_skinny_mxfp4_slab_kernel<4, 1>};
+    const void* sh[8] = {(const void*)gemm_skinny_mxfp4_shared_kernel<1, 0>, (const void*)gemm_skinny_mxfp4_shared_kernel<2, 0>,
+                         (const void*)gemm_skinny_mxfp4_shared_kernel<3, 0>, (const void*)gemm_skinny_mxfp4_shared_kernel<4, 0>,
+                         (const void*)gemm_skinny_mxfp4_shared_kernel<1, 1>, (const void*)gemm_skinny_mxfp4_shared_kernel<2, 1>,
+                         (const void*)gemm_skinny_mxfp4_shared_kernel<3, 1>, (const void*)gemm_skinny_mxfp4_shared_kernel<4, 1>};
+    const int shsz[4] = {SfsGeom<1>::kLdsBytes, SfsGeom<2>::kLdsBytes, SfsGeom<3>::kLdsBytes, SfsGeom<4>::kLdsBytes};
     for (int i = 0; i < 8; ++i)
-      if (hipFuncSetAttribute(sl[i], hipFuncAttributeMaxDynamicSharedMemorySize, kSlabLdsMax) != hipSuccess)
+      if (hipFuncSetAttribute(sh[i], hipFuncAttributeMaxDynamicSharedMemorySize, shsz[i & 3]) != hipSuccess)
         return MASE_ERR_LAUNCH;
     const void* ks[8] = {(const void*)gemm_skinny_mxfp4_partial_kernel<1, 0>, (const void*)gemm_skinny_mxfp4_partial_kernel<2, 0>,
                          (const void*)gemm_skinny_mxfp4_partial_kernel<3, 0>, (const void*)gemm_skinny_mxfp4_partial_kernel<4, 0>,
@@ -929,21 +971,23 @@ extern "C" int mase_gemm_mxfp4_skinny(const void* A_codes, const void* A_scales,
   p.Ws = (const unsigned char*)B_scales;
   p.N = (int)N;
   p.K = (int)K;
-  p.kc = range_elems((int)K, slab ? 256 : 128, splits);
-  p.rotate = (slab && splits == 1) ? 1 : 0;
+  p.kc = range_elems((int)K, shared ? 256 : 128, splits);
+  p.rotate = (shared && splits == 1) ? 1 : 0;
   for (size_t m0 = 0; m0 < M; m0 += 32) {
     const size_t rows = (M - m0 < 32) ? (M - m0) : 32;
     p.Xc = (const unsigned char*)A_codes + m0 * K;
     p.Xs = (const unsigned char*)A_scales + m0 * (K / 32);
-    p.P = (float*)workspace + (size_t)splits * m0 * N;
+    void* Cg = (unsigned char*)C + m0 * N * (out_dtype == MASE_DT_F32 ? 4 : 2);
+    p.o = skinny_out((float*)workspace + (size_t)splits * m0 * N, Cg, bias, out_dtype, bias_dtype, splits);
     p.M = (int)rows;
     const int xc = (int)(rows + 7) / 8;
-    const unsigned slab_lds = (unsigned)(8 * xc * p.kc + p.kc + kSlabRingBytes);
 #define MASE_SF_LAUNCH(XC_)                                                                                           \
   do {                                                                                                                \
-    if (slab) {                                                                                                       \
-      if (a_format == 0) hipLaunchKernelGGL((gemm_skinny_mxfp4_slab_kernel<XC_, 0>), grid, block, slab_lds, st, p);   \
-      else hipLaunchKernelGGL((gemm_skinny_mxfp4_slab_kernel<XC_, 1>), grid, block, slab_lds, st, p);                 \
+    if (shared) {                                                                                                     \
+      if (a_format == 0)                                                                                              \
+        hipLaunchKernelGGL((gemm_skinny_mxfp4_shared_kernel<XC_, 0>), grid, block, SfsGeom<XC_>::kLdsBytes, st, p);   \
+      else                                                                                                            \
+        hipLaunchKernelGGL((gemm_skinny_mxfp4_shared_kernel<XC_, 1>), grid, block, SfsGeom<XC_>::kLdsBytes, st, p);   \
     } else if (a_format == 0) {                                                                                       \
       hipLaunchKernelGGL((gemm_skinny_mxfp4_partial_kernel<XC_, 0>), grid, block, SfGeom<XC_>::kLdsBytes, st, p);     \
     } else {                                                                                                          \
@@ -955,15 +999,7 @@ extern "C" int mase_gemm_mxfp4_skinny(const void* A_codes, const void* A_scales,
     else if (xc == 3) MASE_SF_LAUNCH(3);
     else MASE_SF_LAUNCH(4);
 #undef MASE_SF_LAUNCH
-    const size_t mn_g = rows * N;
-    const dim3 rgrid_g((unsigned)blocks_for(mn_g, 256));
-    void* Cg = (unsigned char*)C + m0 * N * (out_dtype == MASE_DT_F32 ? 4 : 2);
-    if (out_dtype == MASE_DT_F32)
-      hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_F32>, rgrid_g, dim3(256), 0, st, p.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
-    else if (out_dtype == MASE_DT_BF16)
-      hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_BF16>, rgrid_g, dim3(256), 0, st, p.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
-    else
-      hipLaunchKernelGGL(gemm_skinny_reduce_kernel<MASE_DT_F16>, rgrid_g, dim3(256), 0, st, p.P, Cg, bias, bias_dtype, mn_g, (int)N, splits);
+    skinny_launch_reduce(p.o, Cg, bias, out_dtype, bias_dtype, rows, N, splits, st);
   }
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
