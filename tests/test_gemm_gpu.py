@@ -159,6 +159,44 @@ def test_gemm_few_rows_with_mxint8_coded_weights(dev, M):
     assert torch.equal(got.cpu(), ai @ wi.T)
 
 
+@pytest.mark.parametrize("kind", ["bf16", "mxint8", "mxfp4"])
+@pytest.mark.parametrize("M,N,K", [(16, 32768, 256), (5, 32766, 512), (40, 33001, 256)])
+def test_gemm_few_rows_single_k_range_finishes_the_output_in_the_kernel(dev, kind, M, N, K):
+    """Wide weights with a short K take one K range: no reduction kernel runs, the weight-streaming kernel adds the
+    bias and converts itself.  For every output and bias dtype the result must be the fp32 result plus the bias,
+    rounded once; N = 32766 and 33001 take the scalar stores, 40 rows two passes."""
+    from mase_amd import _gemm, _lib
+    from mase_amd.quantizers import _ops
+
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(M + N + K)
+    a = torch.randn(M, K, generator=g).bfloat16().to(dev)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(dev)
+    if kind == "bf16":
+        wb = w.bfloat16()
+        assert lib.mase_gemm_bf16_skinny_workspace_bytes(M, N, K) == M * N * 4   # one K range
+        run = lambda bias, dt: _gemm.gemm_bf16_tn(a, wb, bias, dt)
+    elif kind == "mxint8":
+        _, codes, scales = _ops.mxint_qdq(w, 32, 8, 1, 8, pack=True, out_dtype=torch.bfloat16)
+        codes, scales = codes.view(N, K), scales.view(N, K // 32)
+        assert lib.mase_gemm_mxint8_skinny_workspace_bytes(M, N, K) == M * N * 4
+        run = lambda bias, dt: _gemm.gemm_mxint8_skinny(a, codes, scales, bias, dt)
+    else:
+        ac, asc = _gemm.mxfp_pack(a, 4, 3)
+        bc, bsc = _gemm.mxfp_pack(w, 2, 1)
+        assert lib.mase_gemm_mxfp4_skinny_workspace_bytes(M, N, K) == M * N * 4
+        run = lambda bias, dt: _gemm.gemm_mxfp4_skinny(ac, asc, (4, 3), bc, bsc, bias, dt)
+    y32 = run(None, torch.float32)
+    assert torch.isfinite(y32).all() and float(y32.abs().max()) > 0
+    for bias_dt in (torch.float32, torch.bfloat16, torch.float16):
+        bias = torch.randn(N, generator=g).to(bias_dt).to(dev)
+        for out_dt in (torch.float32, torch.bfloat16, torch.float16):
+            got = run(bias, out_dt)
+            want = (y32 + bias.float()).to(out_dt)
+            assert torch.equal(got.view(torch.int32 if out_dt == torch.float32 else torch.int16),
+                               want.view(torch.int32 if out_dt == torch.float32 else torch.int16)), (bias_dt, out_dt)
+
+
 @pytest.mark.parametrize("M", [129, 256, 300, 512, 1000])
 def test_gemm_a_few_hundred_rows_cuts_k_into_work_items(dev, M):
     """mase_gemm_bf16_tn_splitk through the dispatch of gemm_bf16_tn: exact on integer operands, agrees with fp64
