@@ -233,7 +233,8 @@ int mase_gemm_mxint8_tn_packed(const void* A, const void* code_image, const void
 /* The same product for few rows of A (M <= 128, the token-by-token shape of serving): bound by streaming B once
  * from HBM.  The work is split over N and over K ranges; the partial results of the K ranges go through
  * `workspace` (device memory, 16-byte aligned, at least mase_gemm_bf16_skinny_workspace_bytes(M, N, K) bytes, which
- * is at most 64*M*N*4) and are added in a fixed order, so results are reproducible.  K % 64 == 0.
+ * is at most 64*M*N*4) and are added in a fixed order, so results are reproducible; when one K range is enough
+ * (wide weights) the workspace is not touched and the output is written by the first kernel.  K % 64 == 0.
  * Replaces the same F.linear as mase_gemm_bf16_tn (nn/quantized/modules/linear.py:972, :895). */
 size_t mase_gemm_bf16_skinny_workspace_bytes(size_t M, size_t N, size_t K);
 int mase_gemm_bf16_skinny(const void* A, const void* B, const void* bias, void* C, size_t M, size_t N, size_t K,
