@@ -521,6 +521,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     for (int i = 0; i < 8; ++i) load_8_untracked(fbc[0][i >> 1][i & 1], boff[i & 1], b_kbase + (size_t)(i >> 1) * 512);
     b_kt = 1;
     wait_vmcnt<0>();
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       set_scale(0, 0, j);
@@ -533,6 +534,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     for (int i = 0; i < 4 * NJ; ++i) load_16_untracked(fb[0][i / NJ][i % NJ], boff[i % NJ], b_kbase + (size_t)(i / NJ) * 1024);
     b_kt = 1;
     wait_vmcnt<0>();
+    __builtin_amdgcn_sched_barrier(0);
   } else {
     wait_vmcnt<kWaveCopies + kCopiesB>();  // K tile 0 landed; K tile 1 may still be in flight
   }
@@ -570,6 +572,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
       else if (s == 1) wait_vmcnt<12>();
       else if (s == 2) wait_vmcnt<10>();
       else wait_vmcnt<8>();
+      // A matrix instruction has no side effect the compiler would order against the wait: without this it hoists the
+      // step's first one above the wait that proves its fragment.
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int t = 0; t < 16; ++t) {
         acc[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[NB][s][t & 1], fr[s][t >> 1],
@@ -616,6 +621,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
       else if (s == 1) wait_vmcnt<12>();
       else if (s == 2) wait_vmcnt<10>();
       else wait_vmcnt<6>();
+      __builtin_amdgcn_sched_barrier(0);  // nothing that reads the codes or scales may be hoisted above the wait
 #pragma unroll
       for (int t = 0; t < 16; ++t) {
         acc[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
