@@ -118,9 +118,12 @@ __device__ __forceinline__ void sk_async_copy(const unsigned char* base, uint32_
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(m0v) : "memory");
 }
 
+// The empty statement behind the wait keeps the compiler from moving an LDS read of the copied data in front of it
+// (the wait itself is not a memory operation to the compiler).
 template <int N>
 __device__ __forceinline__ void sk_wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8) | ((N >> 4) << 14));
+  asm volatile("" ::: "memory");
 }
 
 template <int XC>
