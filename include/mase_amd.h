@@ -26,6 +26,7 @@
  *   mase_silu_mul_minifloat nn/quantized/modules/llama/mlp.py:60-62 (silu_minifloat(gate) * up)
  *   mase_rmsnorm_mxint, mase_silu_mul_mxint   the two above followed by the consumer LinearMXInt's activation
  *                           quantizer (nn/quantized/modules/linear.py:956-972) in the same pass
+ *   mase_silu_mul_mxint_lut, mase_silu_table  mase_silu_mul_mxint for 16-bit tensors with silu read from a table
  *   mase_add_rmsnorm_mxint  models/llama/modeling_llama.py:901-905 (residual addition, then the norm as above)
  *   mase_attn_softmax_mx    nn/quantized/modules/llama/attention.py:363-392 (scores -> quantized probabilities)
  *   mase_attention_causal   models/llama/modeling_llama.py:362-480 (the attention core on unquantized q, k, v)
@@ -337,6 +338,16 @@ int mase_rmsnorm_mxint(const void* x, const void* weight, void* out, size_t rows
                        int element_bits, const uint32_t* log2_tab, void* stream);
 int mase_silu_mul_mxint(const void* gate, const void* up, void* out, size_t numel, int dtype, int element_bits,
                         const uint32_t* log2_tab, void* stream);
+
+/* The same operation for 16-bit tensors with R(silu(gate)) read from a table of its 65536 possible values, which
+ * mase_silu_table fills once per dtype (bf16 or fp16; 128 KB of device memory, 16-byte aligned) with the expression
+ * mase_silu_mul_mxint evaluates per element: same results bit for bit, without the exponential and the division per
+ * element (a third of that kernel's time on large tensors).  The table sits in LDS, one work-group per CU.
+ * Same call site as mase_silu_mul_mxint (nn/quantized/modules/llama/mlp.py:60-62 followed by the activation quantizer of
+ * nn/quantized/modules/linear.py:956-972). */
+int mase_silu_table(void* table, int dtype, void* stream);
+int mase_silu_mul_mxint_lut(const void* gate, const void* up, void* out, size_t numel, int dtype, int element_bits,
+                            const uint32_t* log2_tab, const void* silu_table, void* stream);
 
 /* The residual addition of a pre-norm block followed by mase_rmsnorm_mxint, in one pass: sum_out = x + residual (rounded
  * to dtype, as the tensor addition rounds it) and out = mxint_quantizer(rmsnorm(sum_out)) as above

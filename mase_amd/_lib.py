@@ -57,6 +57,8 @@ SIGNATURES = {
     "mase_add_rmsnorm_mxint": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_float, c_int,
                                       c_void_p, c_void_p]),
     "mase_silu_mul_mxint": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_void_p, c_void_p]),
+    "mase_silu_table": (c_int, [c_void_p, c_int, c_void_p]),
+    "mase_silu_mul_mxint_lut": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "mase_mxint_clip_search": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mase_mxfp_clip_search": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mase_mxint_clip_candidates": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),

@@ -216,6 +216,66 @@ __global__ __launch_bounds__(kRowThreads) void silu_mul_kernel(SiluMulParams p) 
   if (live) store_vec8<DT>(p.out, i * 8, y);
 }
 
+// silu(gate) * up for 16-bit tensors with silu read from a table.  R(silu(g)) is a function of the 16 bits of g alone,
+// and evaluating it (an exponential and a division per element) costs the kernel above a third of its time; here the
+// table of all 65536 results (filled once per dtype by silu_table_kernel with the very expression the kernel above
+// evaluates, so the results are the same bit for bit) sits in LDS, 128 KB, one work-group of 16 wavefronts per CU,
+// each walking the tensor with the stride of the grid.
+constexpr int kLutThreads = 1024;
+
+template <int DT>
+__global__ __launch_bounds__(256) void silu_table_kernel(uint16_t* __restrict__ table) {
+  using TR = DTypeTraits<DT>;
+  static_assert(DT != MASE_DT_F32, "a table over the 16 bits of a value");
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;  // the grid covers exactly 65536 patterns
+  float v[8], y[8];
+  TR::unpack(make_uint4(i, 0u, 0u, 0u), v);  // element 0: the low half of the first dword
+#pragma unroll
+  for (int j = 0; j < 8; ++j) y[j] = TR::round(silu_f32(v[j]));
+  table[i] = (uint16_t)(TR::pack(y).x & 0xFFFFu);
+}
+
+struct SiluLutParams {
+  const uint4* gate;
+  const uint4* up;
+  uint4* out;
+  size_t n8;
+  const uint4* table;   // 65536 x 16 bits
+  MxintParams mx;
+};
+
+template <int DT>
+__global__ __launch_bounds__(kLutThreads) void silu_mul_lut_kernel(SiluLutParams p) {
+  using TR = DTypeTraits<DT>;
+  extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
+  for (int i = threadIdx.x; i < 65536 * 2 / 16; i += kLutThreads) ((uint4*)lut)[i] = p.table[i];
+  WaveLog2 meta;
+  meta.init(p.mx.tab, 0);
+  __syncthreads();
+  const size_t stride = (size_t)gridDim.x * kLutThreads;
+  // the loop bound is the same for all lanes of a wavefront: every lane takes part in the block maximum
+  for (size_t base = (size_t)blockIdx.x * kLutThreads + (threadIdx.x & ~63u); base < p.n8; base += stride) {
+    const size_t i = base + (threadIdx.x & 63u);
+    const bool live = i < p.n8;
+    uint4 gq = make_uint4(0, 0, 0, 0), uq = make_uint4(0, 0, 0, 0);
+    if (live) {
+      gq = load_nt(p.gate + i);
+      uq = load_nt(p.up + i);
+    }
+    const uint32_t gw[4] = {gq.x, gq.y, gq.z, gq.w};
+    uint32_t sw[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sw[j] = (uint32_t)lut[gw[j] & 0xFFFFu] | ((uint32_t)lut[gw[j] >> 16] << 16);
+    float s[8], u[8], y[8];
+    TR::unpack(make_uint4(sw[0], sw[1], sw[2], sw[3]), s);
+    TR::unpack(uq, u);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) y[j] = TR::round(s[j] * u[j]);
+    mxint_block32<DT>(y, p.mx, meta);
+    if (live) store_nt(p.out + i, TR::pack(y));
+  }
+}
+
 struct RopeParams {
   const void* x;
   const void* cos;
@@ -416,6 +476,50 @@ extern "C" int mase_silu_mul_mxint(const void* gate, const void* up, void* out, 
     case MASE_DT_BF16: hipLaunchKernelGGL((silu_mul_kernel<MASE_DT_BF16, true>), grid, block, 0, st, p); break;
     default: hipLaunchKernelGGL((silu_mul_kernel<MASE_DT_F16, true>), grid, block, 0, st, p); break;
   }
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+extern "C" int mase_silu_table(void* table, int dtype, void* stream) {
+  using namespace mase;
+  if (table == nullptr) return MASE_ERR_NULL;
+  if (!aligned16(table)) return MASE_ERR_ALIGN;
+  if (dtype != MASE_DT_BF16 && dtype != MASE_DT_F16) return MASE_ERR_DTYPE;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == MASE_DT_BF16) hipLaunchKernelGGL((silu_table_kernel<MASE_DT_BF16>), dim3(256), dim3(256), 0, st, (uint16_t*)table);
+  else hipLaunchKernelGGL((silu_table_kernel<MASE_DT_F16>), dim3(256), dim3(256), 0, st, (uint16_t*)table);
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+extern "C" int mase_silu_mul_mxint_lut(const void* gate, const void* up, void* out, size_t numel, int dtype,
+                                       int element_bits, const uint32_t* log2_tab, const void* silu_table, void* stream) {
+  using namespace mase;
+  if (numel == 0) return MASE_OK;
+  if (gate == nullptr || up == nullptr || out == nullptr || log2_tab == nullptr || silu_table == nullptr) return MASE_ERR_NULL;
+  if (numel % 32 != 0) return MASE_ERR_SHAPE;
+  if (!aligned16(gate) || !aligned16(up) || !aligned16(out) || !aligned16(silu_table)) return MASE_ERR_ALIGN;
+  if (dtype != MASE_DT_BF16 && dtype != MASE_DT_F16) return MASE_ERR_DTYPE;
+  SiluLutParams p{};
+  p.gate = (const uint4*)gate;
+  p.up = (const uint4*)up;
+  p.out = (uint4*)out;
+  p.n8 = numel / 8;
+  p.table = (const uint4*)silu_table;
+  if (!fill_mxint(p.mx, element_bits, dtype, log2_tab)) return MASE_ERR_PARAM;
+  const int n_cu = device_cu_count();
+  if (n_cu <= 0) return MASE_ERR_LAUNCH;
+  constexpr int kLutBytes = 65536 * 2;
+  static std::atomic<uint64_t> attr_done{0};
+  if (!device_setup_done(attr_done)) {
+    if (hipFuncSetAttribute((const void*)silu_mul_lut_kernel<MASE_DT_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, kLutBytes) != hipSuccess ||
+        hipFuncSetAttribute((const void*)silu_mul_lut_kernel<MASE_DT_F16>, hipFuncAttributeMaxDynamicSharedMemorySize, kLutBytes) != hipSuccess)
+      return MASE_ERR_LAUNCH;
+    mark_device_setup_done(attr_done);
+  }
+  const size_t wgs_needed = blocks_for(p.n8, (size_t)kLutThreads);
+  const dim3 grid((unsigned)(wgs_needed < (size_t)n_cu ? wgs_needed : (size_t)n_cu)), block(kLutThreads);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == MASE_DT_BF16) hipLaunchKernelGGL((silu_mul_lut_kernel<MASE_DT_BF16>), grid, block, kLutBytes, st, p);
+  else hipLaunchKernelGGL((silu_mul_lut_kernel<MASE_DT_F16>), grid, block, kLutBytes, st, p);
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
 

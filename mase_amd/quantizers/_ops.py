@@ -387,14 +387,41 @@ def add_rmsnorm_mxint(x: Tensor, residual: Tensor, weight: Tensor, eps: float, e
     return s, out
 
 
-def silu_mul_mxint(gate: Tensor, up: Tensor, element_bits: int) -> Tensor:
+SILU_TABLE_MIN_NUMEL = 1 << 23  # from here on the table form of silu * up pays for loading its 128 KB per CU
+_silu_tables: dict = {}
+
+
+def silu_table(dtype: torch.dtype, device: torch.device) -> Tensor:
+    """R(silu(x)) for every 16-bit pattern x of ``dtype`` (bf16 / fp16), computed on the device by
+    ``mase_silu_table`` with the expression the element-wise kernel evaluates; cached per dtype and device."""
+    key = (dtype, str(device))
+    if key not in _silu_tables:
+        lib = _lib.load()
+        tab = torch.empty(65536, dtype=torch.int16, device=device)
+        _lib.check(lib.mase_silu_table(tab.data_ptr(), _lib.DTYPE_CODE[dtype], _lib.stream_ptr(tab)), "mase_silu_table")
+        _silu_tables[key] = tab
+    return _silu_tables[key]
+
+
+def silu_mul_mxint(gate: Tensor, up: Tensor, element_bits: int, use_table: bool | None = None) -> Tensor:
     """``mxint_quantizer(silu(gate) * up, block 32 along the last dimension, element_bits)`` in one pass
-    (``mase_silu_mul_mxint``); the last dimension must be a multiple of 32."""
+    (``mase_silu_mul_mxint``); the last dimension must be a multiple of 32.  Large 16-bit tensors take the form that
+    reads silu from a table (``mase_silu_mul_mxint_lut``, same bits); ``use_table`` forces either form."""
     _lib.require_device(gate, "silu_mul_mxint")
     lib = _lib.load()
     assert silu_mul_supported(gate, up) and gate.shape[-1] % 32 == 0
     g, u = _contig(gate), _contig(up)
     out = torch.empty_like(g)
+    sixteen = g.dtype in (torch.bfloat16, torch.float16)
+    if use_table is None:
+        use_table = sixteen and g.numel() >= SILU_TABLE_MIN_NUMEL
+    if use_table:
+        assert sixteen, "the table form exists for 16-bit tensors"
+        rc = lib.mase_silu_mul_mxint_lut(g.data_ptr(), u.data_ptr(), out.data_ptr(), g.numel(), _lib.dtype_code(g),
+                                         int(element_bits), log2_table(g.dtype, g.device).data_ptr(),
+                                         silu_table(g.dtype, g.device).data_ptr(), _lib.stream_ptr(g))
+        _lib.check(rc, "mase_silu_mul_mxint_lut")
+        return out
     rc = lib.mase_silu_mul_mxint(g.data_ptr(), u.data_ptr(), out.data_ptr(), g.numel(), _lib.dtype_code(g),
                                  int(element_bits), log2_table(g.dtype, g.device).data_ptr(), _lib.stream_ptr(g))
     _lib.check(rc, "mase_silu_mul_mxint")

@@ -149,7 +149,33 @@ def test_norm_and_silu_product_written_in_the_consumers_mxint_form(dev, dtype, b
         up[-1, -32:] *= 1e4 if dtype != torch.float16 else 50.0
         gd, ud = gate.to(dev), up.to(dev)
         want = _ops.mxint_qdq(_ops.silu_mul_minifloat(gd, ud), 32, bits, -1, 8)
-        assert_bits_equal(_ops.silu_mul_mxint(gd, ud, bits), want, f"silu_mul_mxint {dtype} {rows}x{cols}")
+        assert_bits_equal(_ops.silu_mul_mxint(gd, ud, bits, use_table=False), want, f"silu_mul_mxint {dtype} {rows}x{cols}")
+        if dtype != torch.float32:  # the form that reads silu from a table: the same bits
+            assert_bits_equal(_ops.silu_mul_mxint(gd, ud, bits, use_table=True), want, f"silu_mul_mxint table {dtype} {rows}x{cols}")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_silu_table_form_for_every_gate_pattern_and_at_size(dev, dtype):
+    """mase_silu_mul_mxint_lut against mase_silu_mul_mxint bit for bit: every 16-bit pattern as the gate (NaNs and
+    infinities included), non-finite and huge second factors, a tensor large enough that the dispatch picks the table
+    form by itself (more work-groups' worth of vectors than CUs, a ragged last wavefront)"""
+    from mase_amd.quantizers import _ops
+    from helpers import assert_bits_equal
+
+    g = torch.Generator().manual_seed(17)
+    gate = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype).reshape(2048, 32).to(dev)
+    for scale in (1.0, 1e3 if dtype == torch.float16 else 1e30):
+        up = (torch.randn(2048, 32, generator=g) * scale).to(dtype).to(dev)
+        up[5, 3] = float("inf")
+        up[6, 4] = float("nan")
+        for bits in (8, 4, 2):
+            assert_bits_equal(_ops.silu_mul_mxint(gate, up, bits, use_table=True),
+                              _ops.silu_mul_mxint(gate, up, bits, use_table=False), f"table form, all gates, {dtype} bits {bits}")
+    rows, cols = 4099, 2144   # 8.8 M elements: above the dispatch threshold, not a multiple of the grid's stride
+    assert rows * cols >= _ops.SILU_TABLE_MIN_NUMEL
+    gate = (torch.randn(rows, cols, generator=g) * 2.5).to(dtype).to(dev)
+    up = torch.randn(rows, cols, generator=g).to(dtype).to(dev)
+    assert_bits_equal(_ops.silu_mul_mxint(gate, up, 8), _ops.silu_mul_mxint(gate, up, 8, use_table=False), f"table form at size, {dtype}")
 
 
 # the last two: enough (batch, head) pairs per XCD for the persistent form of the kernel (2 and 4 items per work-group)
