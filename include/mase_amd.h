@@ -207,9 +207,11 @@ int mase_gemm_bf16_tn_splitk(const void* A, const void* B, const void* bias, voi
 /* The same product with B given as the fragment-ordered image written by mase_gemm_bf16_pack_b (a weight is packed
  * once when it is loaded): B's fragments then go from the cache straight into registers instead of through LDS, which
  * the kernel otherwise shares between the copies arriving and the fragment reads.  K % 128 == 0; the image takes
- * mase_gemm_bf16_packed_bytes(N, K) = ceil(N/32)*32*K*2 bytes (below 4 GiB), 16-byte aligned.  Same results as
- * mase_gemm_bf16_tn (the same products added in the same order).  Replaces the same F.linear
- * (nn/quantized/modules/linear.py:972, :895). */
+ * mase_gemm_bf16_packed_bytes(N, K) = ceil(N/32)*32*K*2 bytes (below 4 GiB), 16-byte aligned; the packer takes any
+ * K % 32 == 0.  The same exact products with fp32 accumulation as mase_gemm_bf16_tn, added in another order (this kernel
+ * computes with the 16x16x32 matrix instruction, 32 products per instruction where mase_gemm_bf16_tn adds 16): equal to
+ * fp32 rounding of the sums, bit-identical where every partial sum is exact (small integers).  Replaces the same
+ * F.linear (nn/quantized/modules/linear.py:972, :895). */
 size_t mase_gemm_bf16_packed_bytes(size_t N, size_t K);
 int mase_gemm_bf16_pack_b(const void* B, void* B_packed, size_t N, size_t K, void* stream);
 int mase_gemm_bf16_tn_packed(const void* A, const void* B_packed, const void* bias, void* C, size_t M, size_t N,

@@ -34,7 +34,7 @@ def gemm_bf16_pack_b(b: Tensor) -> Tensor:
     b = b.contiguous()
     N, K = b.shape
     nbytes = lib.mase_gemm_bf16_packed_bytes(N, K)
-    assert nbytes > 0, "K must be a multiple of 16"
+    assert nbytes > 0, "K must be a multiple of 32"
     out = torch.empty(nbytes, dtype=torch.uint8, device=b.device)
     _lib.check(lib.mase_gemm_bf16_pack_b(b.data_ptr(), out.data_ptr(), N, K, _lib.stream_ptr(b)), "mase_gemm_bf16_pack_b")
     return out

@@ -31,6 +31,7 @@ namespace {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int S = 2;                              // LDS stages
@@ -118,6 +119,18 @@ __device__ __forceinline__ void acc_read_fence() {
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 }
 
+// acc += B fragment x A fragment with v_mfma_f32_16x16x32_bf16, the accumulator tied to accumulation registers.  Through
+// the compiler's builtin the 64 four-register accumulators of the K loop are not kept in place from one trip to the next
+// (the loop then opens with some 270 register moves).  As assembly the compiler inserts no wait states for it: an
+// accumulator is read again 64 matrix instructions after it was written, the fragments come from loads (completed by
+// s_waitcnt), the epilogue starts with acc_read_fence and zeroing ends with acc_write_fence.
+__device__ __forceinline__ void mfma16_acc(f32x4_t& acc, const bf16x8_t& b, const bf16x8_t& a) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
+}
+// wait states between a write of an accumulation register by an ordinary instruction and a matrix instruction that
+// reads it as its addend (the part requires 2)
+__device__ __forceinline__ void acc_write_fence() { asm volatile("s_nop 3" ::: "memory"); }
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   // gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14 ; leave the others at max
@@ -162,7 +175,11 @@ __device__ __forceinline__ void load_2_untracked(uint32_t& dst, uint32_t off, co
 // MFMAs per K step); B's stage holds 128 rows.
 template <int OUT_DT, bool STREAM, bool BPACK = false, bool BCODES = false, bool BATCHED = false, bool HALFN = false>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p) {
-  constexpr int NI = BPACK ? 8 : 4, NJ = (BPACK || HALFN) ? 2 : 4;  // MFMA tiles of a wavefront: rows x columns
+  constexpr int NI = BPACK ? 8 : 4, NJ = (BPACK || HALFN) ? 2 : 4;  // 32 x 32 tiles of a wavefront: rows x columns
+  // The bf16 image form computes with v_mfma_f32_16x16x32_bf16 (16 x 4 tiles of 16 x 16 per wavefront, two K steps of
+  // 32 per K tile): the same multiply-adds per cycle as the 32x32x16 instruction on paper, but under the board's power
+  // limit the part sustains a clock about 8 % higher on it (measured with both instructions on random operands).
+  constexpr bool MI16 = BPACK && !BCODES;
   constexpr int kBN = HALFN ? 128 : BN;                           // columns of an output tile
   constexpr int kCopiesB = HALFN ? kWaveCopies / 2 : kWaveCopies;  // copies of B per wavefront per K tile
   static_assert(!BCODES || BPACK, "codes come in fragment order");
@@ -273,14 +290,25 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     }
   };
 
-  f32x16_t acc[NI][NJ];
+  f32x16_t acc[MI16 ? 1 : NI][MI16 ? 1 : NJ];
+  f32x4_t acc16[MI16 ? 16 : 1][MI16 ? 4 : 1];  // MI16: [row tile of 16][column tile of 16]
   auto zero_acc = [&]() __attribute__((always_inline)) {
+    if constexpr (MI16) {
 #pragma unroll
-    for (int i = 0; i < NI; ++i)
+      for (int i = 0; i < 16; ++i)
 #pragma unroll
-      for (int j = 0; j < NJ; ++j)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+          for (int r = 0; r < 4; ++r) acc16[i][j][r] = 0.0f;
+      acc_write_fence();
+    } else {
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    }
   };
   zero_acc();
 
@@ -296,12 +324,16 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // The lane's row and K group within a fragment, which every LDS read of the K loop is addressed with.  Set again
   // from the lane number after each epilogue rather than kept across it: what lives across the epilogue's register
   // demand gets spilled (see lane_now).
-  int frag_row = lane & 31;
-  int kgrp = lane >> 5;
+  int frag_row = MI16 ? (lane & 15) : (lane & 31);
+  int kgrp = MI16 ? (lane >> 4) : (lane >> 5);
   // fragment f (0..3: A row tile f, 4..7: B column tile f-4) of K step s of the K tile in `stage`
-  // (BPACK: f = 0..7, A row tile f of the whole tile)
+  // (BPACK: f = 0..7, A row tile f of the whole tile; MI16: s = quarter q of the K tile, fragment = rows
+  // 128 * (q % 2) + 16 * f .. + 16 at K 32 * (q / 2) .. + 32, lane l supplying row l % 16, K 8 * (l / 16) .. + 8)
   auto load_frag = [&](int stage, int s, int f) __attribute__((always_inline)) -> bf16x8_t {
-    if constexpr (BPACK) {
+    if constexpr (MI16) {
+      const unsigned char* st = lds + stage * kStride;
+      return __builtin_bit_cast(bf16x8_t, *(const uint4*)(st + lds_off(((s & 1) * 8 + f) * 16 + frag_row, (s >> 1) * 4 + kgrp)));
+    } else if constexpr (BPACK) {
       const unsigned char* st = lds + stage * kStride;
       return __builtin_bit_cast(bf16x8_t, *(const uint4*)(st + lds_off(f * 32 + frag_row, s * 2 + kgrp)));
     } else {
@@ -317,6 +349,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // bytes: 64 columns of a 16-bit output, 32 of an fp32 one), from which every lane takes 16 consecutive bytes, so that
   // a store instruction writes 8 rows of 128 contiguous bytes.  Only lanes of one wavefront exchange data (its LDS
   // accesses execute in order, and the writes are waited for before the reads are issued): no barrier.
+  // MI16: acc16[i][j][rr] is C[row, col] with row = i*16 + lane%16 and col = j*16 + (lane/16)*4 + rr; a band of 32 rows
+  // is made of the row tiles 2b and 2b + 1.
   auto epilogue = [&](int ord) __attribute__((always_inline)) {
     int m0, n0, ks;
     tile_origin(ord, m0, n0, ks);
@@ -328,7 +362,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
       Cs = (unsigned char*)p.C + (size_t)bo * p.c_so + (size_t)bi * p.c_si;
     }
     const int lane = lane_now();
-    const int r32 = lane & 31, kgrp = lane >> 5;
+    const int r32 = MI16 ? (lane & 15) : (lane & 31), kgrp = MI16 ? (lane >> 4) : (lane >> 5);
     const int rrow = lane >> 3, chunk = lane & 7;  // read side: row rrow + 8 * pass, 16-byte piece `chunk` of it
     unsigned char* const stg = lds + S * kStageBytes + wave * kStgWave;
     unsigned char* const stg_w = stg + r32 * kStgRow;
@@ -357,7 +391,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
           for (int q = 0; q < 4; ++q)
 #pragma unroll
             for (int rr = 0; rr < 4; ++rr) {
-              const int col = n0 + col_base + j * 32 + q * 8 + kgrp * 4 + rr;
+              // (MI16: bv[j][q] belongs to column tile 2 * j + q / 2 of 16; q % 2 is not used)
+              const int col = MI16 ? n0 + col_base + (2 * j + (q >> 1)) * 16 + kgrp * 4 + rr
+                                   : n0 + col_base + j * 32 + q * 8 + kgrp * 4 + rr;
+              if (MI16 && (q & 1)) continue;
               if (col < p.N) bv[j][q][rr] = load_bias(p.bias, decltype(dtc)::value, col);
             }
       };
@@ -380,9 +417,19 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
         const int j = jb * kBandTiles + jj;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const float v[4] = {acc_read(acc[i][j][q * 4 + 0]) + bv[j][q][0], acc_read(acc[i][j][q * 4 + 1]) + bv[j][q][1],
-                              acc_read(acc[i][j][q * 4 + 2]) + bv[j][q][2], acc_read(acc[i][j][q * 4 + 3]) + bv[j][q][3]};
-          unsigned char* const dst = stg_w + (jj * 32 + q * 8 + kgrp * 4) * kEsz;
+          // MI16: q = 2 * (column tile of 16 within the 32 columns j) + (row tile of 16 within the band)
+          const int i16 = 2 * i + (q & 1), j16 = 2 * j + (q >> 1);
+          const float* const bq = bv[j][MI16 ? (q & 2) : q];
+          float v[4];
+          if constexpr (MI16) {
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) v[rr] = acc_read(acc16[i16][j16][rr]) + bq[rr];
+          } else {
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) v[rr] = acc_read(acc[i][j][q * 4 + rr]) + bq[rr];
+          }
+          unsigned char* const dst = MI16 ? stg_w + (q & 1) * 16 * kStgRow + (jj * 32 + (q >> 1) * 16 + kgrp * 4) * kEsz
+                                          : stg_w + (jj * 32 + q * 8 + kgrp * 4) * kEsz;
           if constexpr (OUT_DT == MASE_DT_F32) {
             *(uint4*)dst = make_uint4(f2bits(v[0]), f2bits(v[1]), f2bits(v[2]), f2bits(v[3]));
           } else if constexpr (OUT_DT == MASE_DT_BF16) {
@@ -461,8 +508,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // The epilogue's stores count in vmcnt like the copies, so the first hand-over of an output tile also waits
   // for the previous tile's stores to be acknowledged.
   bf16x8_t fr[4][8];
-  // BPACK: B fragments of two K tiles (the one in use and the one being loaded): [buffer][K step][column tile].
-  // Image layout: 1 KB blocks [column tile of 32][K step of 16][lane][8 bf16], lane l = column l % 32, K 8*(l/32)..+8.
+  // BPACK: B fragments of two K tiles (the one in use and the one being loaded): [buffer][2 * K step + column tile / 2]
+  // [column tile % 2].  Image layout: 1 KB blocks [column tile of 16][K step of 32][lane][8 bf16], lane l = column
+  // l % 16, K 8*(l/16)..+8.
   bf16x8_t fb[(BPACK && !BCODES) ? 2 : 1][(BPACK && !BCODES) ? 4 : 1][NJ];
   // BCODES: the codes of two K tiles [buffer][K step][column tile] (8 per lane), their scale bytes [buffer][column
   // tile] (the two blocks of 32 a K tile holds, for the lane's column) and the widened fragments of two K steps
@@ -480,6 +528,17 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     const int lane = lane_now();
     const int nt_last = (p.N + 31) / 32 - 1;
     constexpr uint32_t kFragBytes = BCODES ? 512u : 1024u;  // one fragment of a wavefront: 8 codes or 8 bf16 per lane
+    if constexpr (MI16) {
+      // four column tiles of 16; the image holds a multiple of 32 columns (those beyond N are zero)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const size_t ct = (size_t)min((n0 + col_base) / 16 + j, 2 * nt_last + 1);
+        boff[j] = (uint32_t)(ct * (size_t)(p.K / 32) * 1024u) + (uint32_t)lane * 16u;
+      }
+      b_kbase = p.B + (size_t)ks * (size_t)(p.kc / 32) * 1024u;
+      b_kt = 0;
+      return;
+    }
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       const size_t ct = (size_t)min((n0 + col_base) / 32 + j, nt_last);
@@ -531,7 +590,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   } else if constexpr (BPACK) {
     set_b_tile(0);
 #pragma unroll
-    for (int i = 0; i < 4 * NJ; ++i) load_16_untracked(fb[0][i / NJ][i % NJ], boff[i % NJ], b_kbase + (size_t)(i / NJ) * 1024);
+    for (int i = 0; i < 8; ++i) load_16_untracked(fb[0][i >> 1][i & 1], boff[i & 3], b_kbase + (size_t)(i >> 2) * 1024);
     b_kt = 1;
     wait_vmcnt<0>();
     __builtin_amdgcn_sched_barrier(0);
@@ -551,49 +610,61 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // three K tiles ahead, so when a hand-over needs the next K tile, the 16 copies of the two K tiles after it have
   // been issued, and the hand-over waits for "at most 16 outstanding": the next K tile has landed (its copies are older
   // than those 16), while the young copies and up to that many B loads fly on across the barrier.  The B fragments are
-  // proven the same way, by counting the *register loads* issued after them: at the head of step s the two fragments
-  // of the step (loads 2s+1, 2s+2 of the 8 issued one K tile ago) have landed once at most 6 / 12 / 10 / 8 loads are
-  // outstanding (the rest of their batch, plus from step 1 on the 8 of the next batch issued during step 0).
-  // Per step 16 MFMAs, MFMA t on (A row tile t / 2, B column tile t % 2):
-  //   step 0: MFMAs on fr[0]; LDS reads of step 1 (8) and the 8 B loads of the next K tile (their registers were last
-  //           read one K tile ago), one each per MFMA slot 0..7
-  //   step 1: MFMAs on fr[1]; LDS reads of steps 2 and 3 (16); the 8 A copies of the K tile three ahead into the stage
-  //           vacated at the previous hand-over, one every other MFMA slot
-  //   step 2: MFMAs on fr[2]; then the hand-over: at most 16 loads outstanding, own LDS reads complete, barrier
-  //   step 3: MFMAs on fr[3]; LDS reads of step 0 of the next K tile (8)
+  // proven the same way, by counting the *register loads* issued after them.
+  // bf16 image (MI16): a K tile is four quarters q of 32 matrix instructions 16x16x32: K step q / 2 (32 of the 64 K),
+  // rows 128 * (q % 2) .. + 128 (8 row tiles of 16) times the 4 column tiles of 16.  Slot t of a quarter (16 slots)
+  // issues the two instructions of row tile t / 2 on the column tiles 2 * (t % 2) and 2 * (t % 2) + 1, with the other
+  // work between them.  The B loads of a K tile are issued in the order [K step][column tile]; quarters 0 and 1 need
+  // the first four (proven by "at most 4 outstanding" at the head of the K tile: the other four of the batch are
+  // younger), quarters 2 and 3 the last four (at most 8 outstanding at the head of quarter 2: the 8 of the next batch,
+  // issued during quarter 0, are younger).
+  //   quarter 0: LDS reads of quarter 1 (8) and the 8 B loads of the next K tile (their registers were last read one K
+  //              tile ago), one each per slot 0..7
+  //   quarter 1: LDS reads of quarters 2 and 3 (16); the first 4 of the 8 A copies of the K tile three ahead into the
+  //              stage vacated at the previous hand-over, one every fourth slot
+  //   quarter 2: the other 4 A copies; then the hand-over: at most 16 loads outstanding, own LDS reads complete, barrier
+  //   quarter 3: LDS reads of quarter 0 of the next K tile (8)
+  // A wait "at most n outstanding" completes everything but the n youngest operations of either kind.  With all 8 A
+  // copies issued in quarter 1 the 8 youngest at the head of quarter 2 were those copies, and the wait there also
+  // completed the B loads issued in quarter 0, a third of a K tile after their issue: 8 % of the time at K = 11008,
+  // where the B image comes from further away.  With 4 copies issued after that wait, the 8 youngest at the wait are 4
+  // copies and the last 4 B loads.
   // Stores of an epilogue only make the waits of the next output tile's first K tile conservative.
   auto k_iteration_b = [&](auto&& advance, auto bufc) __attribute__((always_inline)) {
     constexpr int NB = decltype(bufc)::value;
-    const unsigned char* bsrc = b_kbase + (size_t)b_kt * 4096;
+    const unsigned char* bsrc = b_kbase + (size_t)b_kt * 2048;
     const int stage_next = next_of(stage);
 #pragma unroll
-    for (int s = 0; s < kSteps; ++s) {
-      if (s == 0) wait_vmcnt<6>();
-      else if (s == 1) wait_vmcnt<12>();
-      else if (s == 2) wait_vmcnt<10>();
-      else wait_vmcnt<8>();
+    for (int q = 0; q < 4; ++q) {
+      if (q == 0) wait_vmcnt<4>();
+      else if (q == 2) wait_vmcnt<8>();
       // A matrix instruction has no side effect the compiler would order against the wait: without this it hoists the
-      // step's first one above the wait that proves its fragment.
+      // quarter's first one above the wait that proves its fragment.
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int t = 0; t < 16; ++t) {
-        acc[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[NB][s][t & 1], fr[s][t >> 1],
-                                                                     acc[t >> 1][t & 1], 0, 0, 0);
-        if (s == 0) {
-          if (t < 8) {
-            fr[1][t] = load_frag(stage, 1, t);
-            load_16_untracked(fb[NB ^ 1][t >> 1][t & 1], boff[t & 1], bsrc + (size_t)(t >> 1) * 1024);
-          }
-        } else if (s == 1) {
+        const int it = (q & 1) * 8 + (t >> 1), jt = 2 * (t & 1), fx = (q >> 1) * 2 + (t & 1);
+        mfma16_acc(acc16[it][jt], fb[NB][fx][0], fr[q][t >> 1]);
+        if (q == 0) {
+          if (t < 8) fr[1][t] = load_frag(stage, 1, t);
+        } else if (q == 1) {
           if (t < 8) fr[2][t] = load_frag(stage, 2, t);
           else fr[3][t - 8] = load_frag(stage, 3, t - 8);
-          if (t & 1) issue_copy(t - 1);
-        } else if (s == 3) {
+        } else if (q == 3) {
           if (t < 8) fr[0][t] = load_frag(stage_next, 0, t);
         }
         __builtin_amdgcn_sched_barrier(0);
+        mfma16_acc(acc16[it][jt + 1], fb[NB][fx][1], fr[q][t >> 1]);
+        if (q == 0) {
+          if (t < 8) load_16_untracked(fb[NB ^ 1][t >> 1][t & 1], boff[t & 3], bsrc + (size_t)(t >> 2) * 1024);
+        } else if (q == 1) {
+          if ((t & 3) == 3) issue_copy((t >> 2) * 2);
+        } else if (q == 2) {
+          if ((t & 3) == 1) issue_copy(8 + (t >> 2) * 2);
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
-      if (s == 2) {
+      if (q == 2) {
         wait_vmcnt<(kStagesB - 2) * kWaveCopies>();
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
@@ -765,8 +836,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     zero_acc();
     {
       const int l = lane_now();
-      frag_row = l & 31;
-      kgrp = l >> 5;
+      frag_row = MI16 ? (l & 15) : (l & 31);
+      kgrp = MI16 ? (l >> 4) : (l >> 5);
     }
   }
   wait_vmcnt<0>();  // no copy may still be in flight towards LDS when the work-group retires
@@ -870,19 +941,19 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
   else ((uint16_t*)C)[i] = (uint16_t)f32_to_f16_bits(s);
 }
 
-// B[N, K] row-major -> fragment-ordered image: 1 KB blocks [column tile of 32][K step of 16][lane][8 bf16]; lane l
-// of a block holds B[tile*32 + l%32][step*16 + 8*(l/32) .. +8], rows beyond N are zero
+// B[N, K] row-major -> fragment-ordered image: 1 KB blocks [column tile of 16][K step of 32][lane][8 bf16]; lane l
+// of a block holds B[tile*16 + l%16][step*32 + 8*(l/16) .. +8], rows beyond N (the image holds a multiple of 32) are zero
 __global__ __launch_bounds__(256) void gemm_pack_b_kernel(const uint4* __restrict__ B, uint4* __restrict__ out, int N,
                                                           int K, size_t granules) {
   const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (g >= granules) return;
   const int lane = (int)(g & 63);
   const size_t blk = g >> 6;
-  const int steps = K / 16;
+  const int steps = K / 32;
   const int nt = (int)(blk / (size_t)steps), ks = (int)(blk % (size_t)steps);
-  const int row = nt * 32 + (lane & 31);
+  const int row = nt * 16 + (lane & 15);
   uint4 v = make_uint4(0, 0, 0, 0);
-  if (row < N) v = B[((size_t)row * K + (size_t)ks * 16 + 8 * (lane >> 5)) / 8];
+  if (row < N) v = B[((size_t)row * K + (size_t)ks * 32 + 8 * (lane >> 4)) / 8];
   out[g] = v;
 }
 
@@ -1059,7 +1130,7 @@ extern "C" int mase_gemm_bf16_tn_splitk(const void* A, const void* B, const void
 }
 
 extern "C" size_t mase_gemm_bf16_packed_bytes(size_t N, size_t K) {
-  if (N == 0 || K == 0 || (K % 16) != 0) return 0;
+  if (N == 0 || K == 0 || (K % 32) != 0) return 0;
   return ((N + 31) / 32) * 32 * K * 2;
 }
 
@@ -1067,7 +1138,7 @@ extern "C" int mase_gemm_bf16_pack_b(const void* B, void* B_packed, size_t N, si
   using namespace mase;
   if (N == 0 || K == 0) return MASE_OK;
   if (B == nullptr || B_packed == nullptr) return MASE_ERR_NULL;
-  if ((K % 16) != 0 || N > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
+  if ((K % 32) != 0 || N > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
   if (!aligned16(B) || !aligned16(B_packed)) return MASE_ERR_ALIGN;
   const size_t granules = mase_gemm_bf16_packed_bytes(N, K) / 16;
   hipLaunchKernelGGL(gemm_pack_b_kernel, dim3(blocks_for(granules, (size_t)256)), dim3(256), 0, (hipStream_t)stream,

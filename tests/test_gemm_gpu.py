@@ -232,27 +232,51 @@ def test_gemm_a_few_hundred_rows_cuts_k_into_work_items(dev, M):
                                    (4100, 4200, 640), (16384, 1024, 4096), (1000, 33, 128),
                                    (16384, 4096, 11008), (16384, 11008, 4096), (16131, 4096, 11008), (3000, 600, 11008)])
 def test_gemm_with_the_weight_in_fragment_order_is_the_same_product(dev, M, N, K):
-    """mase_gemm_bf16_tn_packed against mase_gemm_bf16_tn on the same operands: the same products in the same order,
-    so bit-identical (random operands; the bias and every output dtype), one to several output tiles per work-group,
-    ragged M and N, 1 to 86 pairs of K tiles (K = 11008 and N = 11008 at 16384 rows are the decoder layer's
-    down / gate / up projections at batch 8 x seq 2048), and against an fp32 product"""
+    """mase_gemm_bf16_tn_packed against mase_gemm_bf16_tn on the same operands.  The two kernels add the products of a
+    dot product in different orders (matrix instructions of K = 32 against K = 16), so: (1) on small-integer operands,
+    where every partial sum is exact in fp32 whatever the order, the results are bit-identical, and equal to the integer
+    product (the bias and every output dtype); (2) on random operands they agree to fp32 rounding of the sum, and
+    every launch gives the same bits.  One to several output tiles per work-group, ragged M and N, 1 to 86 pairs of K
+    tiles (K = 11008 and N = 11008 at 16384 rows are the decoder layer's down / gate / up projections at batch 8 x seq
+    2048)."""
     from mase_amd._gemm import gemm_bf16_pack_b, gemm_bf16_packed_b_supported, gemm_bf16_tn
 
     g = torch.Generator().manual_seed(M + N + K)
-    a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
-    b = (torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16).to(dev)
     bias = torch.randn(N, generator=g).to(dev)
     print(f"packed-B gemm M={M} N={N} K={K}", flush=True)
     assert gemm_bf16_packed_b_supported(N, K) == (K % 128 == 0)
+    big = M * N * K > (1 << 36)
+    # (1) integers of magnitude <= 8 and <= 15: |sum| <= 120 * 11008 < 2^24
+    a = torch.randint(-8, 9, (M, K), generator=g).to(torch.bfloat16).to(dev)
+    b = torch.randint(-15, 16, (N, K), generator=g).to(torch.bfloat16).to(dev)
     bp = gemm_bf16_pack_b(b)
     assert bp.numel() == (N + 31) // 32 * 32 * K * 2
     for dt, bs in ((torch.float32, None), (torch.bfloat16, bias), (torch.float16, bias.to(torch.float16))):
         want = gemm_bf16_tn(a, b, bs, dt)
         # several launches: the kernel's loads are tracked by hand, and a mistake there shows up as a few wrong tiles
         # in some launches only
-        for rep in range(4 if M * N * K > (1 << 36) else 2):
+        for rep in range(4 if big else 2):
             got = gemm_bf16_tn(a, b, bs, dt, b_packed=bp)
             assert torch.equal(got, want), (dt, rep, float((got.float() - want.float()).abs().max()))
+    if K % 128 == 0 and M * N <= (1 << 24):
+        exact = (a.double() @ b.double().t()).float()   # every value an integer below 2^24
+        assert torch.equal(gemm_bf16_tn(a, b, None, torch.float32, b_packed=bp), exact)
+    # (2) random operands
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
+    b = (torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+    bp = gemm_bf16_pack_b(b)
+    for dt, bs in ((torch.float32, None), (torch.bfloat16, bias)):
+        want = gemm_bf16_tn(a, b, bs, dt).float()
+        first = None
+        for rep in range(3 if big else 2):
+            got = gemm_bf16_tn(a, b, bs, dt, b_packed=bp)
+            if first is None:
+                first = got
+            assert torch.equal(got, first), (dt, rep)
+        # fp32: rounding of the partial sums; bf16: the two fp32 sums may round to neighbouring bf16 values
+        tol = 2e-6 if dt == torch.float32 else 2.0 ** -7
+        err = float(((first.float() - want).abs() / (want.abs() + want.abs().max() * 0.02)).max())
+        assert err < tol * 8, (dt, err)
     if K % 128 == 0 and M > 512:
         ref = (a.float() @ b.float().t())
         assert float((gemm_bf16_tn(a, b, None, torch.float32, b_packed=bp) - ref).abs().max() / ref.abs().max()) < 1e-5
@@ -268,8 +292,9 @@ def test_gemm_output_not_on_a_16_byte_boundary(dev, dt):
     lib = _lib.load()
     M, N, K = 512, 520, 256  # two tile columns in full and a ragged third; N a multiple of 8
     g = torch.Generator().manual_seed(7)
-    a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
-    b = (torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+    # small integers: every partial sum is exact, so the two kernels (which add in different orders) agree bit for bit
+    a = torch.randint(-8, 9, (M, K), generator=g).to(torch.bfloat16).to(dev)
+    b = torch.randint(-15, 16, (N, K), generator=g).to(torch.bfloat16).to(dev)
     bias = torch.randn(N, generator=g).to(dev)
     bp = gemm_bf16_pack_b(b)
     want = gemm_bf16_tn(a, b, bias, dt, b_packed=bp)
