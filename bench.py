@@ -207,6 +207,7 @@ class _MfmaIssueRate(Workload):
     instruction = "v_mfma_f32_32x32x16_bf16"
     flop_per_instruction = 2.0 * 32 * 32 * 16
     nominal_cycles = 32
+    instructions_per_iter = 8
 
     def setup(self, torch, dev, n_buffers):
         import bench_support
@@ -216,7 +217,7 @@ class _MfmaIssueRate(Workload):
         self._lib = _lib
         self.out = torch.empty(self.work_groups * 512 + 4, dtype=torch.float32, device=dev)
         self.metric = f"matrix-core issue rate of {self.instruction} on register operands (no memory traffic)"
-        self.config = {"workload": f"{self.work_groups} work-groups x 8 wavefronts x {8 * self.iters} instructions, operands: "
+        self.config = {"workload": f"{self.work_groups} work-groups x 8 wavefronts x {self.instructions_per_iter * self.iters} instructions, operands: "
                                    + ("zeros" if self.operands == 0 else self.random_kind)}
         self.fn = getattr(self.lib, self.entry)
 
@@ -227,14 +228,14 @@ class _MfmaIssueRate(Workload):
                                 self.operands, self._lib.stream_ptr(self.out)), "probe")
 
     def work_per_step(self):
-        return float(self.work_groups * 8 * 8 * self.iters) * self.flop_per_instruction
+        return float(self.work_groups * 8 * self.instructions_per_iter * self.iters) * self.flop_per_instruction
 
     def extra(self, torch):
         """shader clock during the last launch, from the kernel's own two counters (first wavefront's loop)"""
         cyc, ticks = self.out[-4:].view(torch.int64).tolist()
         rate_khz = int(self.lib.bench_constant_rate_counter_khz())
         secs = ticks / (rate_khz * 1e3)
-        return {"shader_clock_ghz_in_loop": round(cyc / secs / 1e9, 3), "cycles_per_instruction_of_first_wavefront": round(cyc / (8.0 * self.iters), 2),
+        return {"shader_clock_ghz_in_loop": round(cyc / secs / 1e9, 3), "cycles_per_instruction_of_first_wavefront": round(cyc / (float(self.instructions_per_iter) * self.iters), 2),
                 "constant_rate_counter_khz": rate_khz}
 
 
@@ -245,6 +246,26 @@ class MfmaRateZeros(_MfmaIssueRate):
 
 class MfmaRateRandom(_MfmaIssueRate):
     name = "mfma_rate_random"
+    operands = 2
+
+
+class _Mfma16IssueRate(_MfmaIssueRate):
+    """the same for v_mfma_f32_16x16x32_bf16, the instruction of the tiled GEMM on the fragment-ordered weight"""
+    kernel = "probe_mfma_bf16_16x16_kernel"
+    entry = "bench_probe_mfma_bf16_16x16"
+    instruction = "v_mfma_f32_16x16x32_bf16"
+    flop_per_instruction = 2.0 * 16 * 16 * 32
+    nominal_cycles = 16
+    instructions_per_iter = 16
+
+
+class Mfma16RateZeros(_Mfma16IssueRate):
+    name = "mfma16_rate_zeros"
+    operands = 0
+
+
+class Mfma16RateRandom(_Mfma16IssueRate):
+    name = "mfma16_rate_random"
     operands = 2
 
 
@@ -886,7 +907,7 @@ class DecodeLinearMxfp4(Workload):
 
 WORKLOADS = {w.name: w for w in (MxintClipSearch, BfpQdq, MxintQdq, MxintLinear, MxintLinearCodes, MxfpLinear, DecoderLayerMxint, CopyBytes, IntegerQdq,
                                  MinifloatDenormQdq, MinifloatIeeeQdq, MinifloatMxQdq, MxfpQdq, AttnProb, DecodeLinear,
-                                 DecodeLinearPacked, DecodeLinearMxfp4, AttentionCausal, BmmScores, MfmaRateZeros, MfmaRateRandom, MfmaF8F4RateZeros,
+                                 DecodeLinearPacked, DecodeLinearMxfp4, AttentionCausal, BmmScores, MfmaRateZeros, MfmaRateRandom, Mfma16RateZeros, Mfma16RateRandom, MfmaF8F4RateZeros,
                                  MfmaF8F4RateRandom)}
 
 

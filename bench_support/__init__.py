@@ -15,6 +15,7 @@ SOURCE = os.path.join(DIR, "probes.hip")
 SIGNATURES = {
     "bench_copy_bytes": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "bench_probe_mfma_bf16": (c_int, [c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p]),
+    "bench_probe_mfma_bf16_16x16": (c_int, [c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p]),
     "bench_probe_mfma_f8f4": (c_int, [c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p]),
     "bench_constant_rate_counter_khz": (c_int, []),
 }

@@ -2,7 +2,8 @@
 // library or its C ABI, and without counterpart in the reference.
 //   bench_copy_bytes               plain streaming copy: the achievable-bandwidth ceiling and the scale of the hardware
 //                                  byte counters
-//   bench_probe_mfma_bf16 / _f8f4  issue rate of the matrix instruction on register operands, nothing else running
+//   bench_probe_mfma_bf16 / _bf16_16x16 / _f8f4  issue rate of a matrix instruction on register operands, nothing else
+//                                  running
 //   bench_constant_rate_counter_khz
 // Status codes: 0 ok, negative = the product library's error codes (include/mase_amd.h).
 //
@@ -62,6 +63,57 @@ __global__ __launch_bounds__(512) void probe_mfma_bf16_kernel(float* out, int it
   for (int c = 0; c < 2; ++c)
 #pragma unroll
     for (int k = 0; k < 16; ++k) r += acc[c][k];
+  const long long c1 = __builtin_readcyclecounter(), w1 = wall_clock64();
+  out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = r;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    long long* t = (long long*)(out + (size_t)gridDim.x * blockDim.x);
+    t[0] = c1 - c0;
+    t[1] = w1 - w0;
+  }
+}
+
+// The same for v_mfma_f32_16x16x32_bf16, the instruction of the tiled GEMM on the fragment-ordered weight: the same
+// multiply-adds per cycle (16 instructions of half the work per iteration), on four times as many accumulator chains
+// of a quarter of the size.  With varying operand bits it is held back less than the 32x32x16 instruction.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(512) void probe_mfma_bf16_16x16_kernel(float* out, int iters, int operands) {
+  const int lane = threadIdx.x & 63;
+  bf16x8_t a[4], b[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t h1 = probe_hash(threadIdx.x * 64 + s * 8 + i + blockIdx.x * 7919), h2 = probe_hash(h1 + 12345);
+      float va = 0.0f, vb = 0.0f;
+      if (operands == 1) { va = (float)((lane + i) & 7); vb = (float)((lane - i) & 3); }
+      if (operands == 2) {
+        va = (float)(int)(h1 >> 8) * (1.0f / 4194304.0f) - 2.0f;
+        vb = (float)(int)(h2 >> 8) * (1.0f / 4194304.0f) - 2.0f;
+      }
+      a[s][i] = (__bf16)va;
+      b[s][i] = (__bf16)vb;
+    }
+  f32x4_t acc[8];
+#pragma unroll
+  for (int c = 0; c < 8; ++c)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[c][r] = 0.0f;
+  const long long c0 = __builtin_readcyclecounter(), w0 = wall_clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int c = 2 * s, d = (2 * s + 4) & 7;
+      acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s], b[s], acc[c], 0, 0, 0);
+      acc[c + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[(s + 1) & 3], b[s], acc[c + 1], 0, 0, 0);
+      acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[(s + 2) & 3], b[s], acc[d], 0, 0, 0);
+      acc[d + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[(s + 3) & 3], b[s], acc[d + 1], 0, 0, 0);
+    }
+  }
+  float r = 0.0f;
+#pragma unroll
+  for (int c = 0; c < 8; ++c)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) r += acc[c][k];
   const long long c1 = __builtin_readcyclecounter(), w1 = wall_clock64();
   out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = r;
   if (blockIdx.x == 0 && threadIdx.x == 0) {
@@ -150,6 +202,21 @@ extern "C" int bench_probe_mfma_bf16(void* out, size_t out_bytes, int work_group
   const int threads = 256 * wavefronts_per_simd;
   if (out_bytes < (size_t)work_groups * threads * sizeof(float) + 16 || !aligned16(out)) return MASE_ERR_WORKSPACE;
   hipLaunchKernelGGL(probe_mfma_bf16_kernel, dim3((unsigned)work_groups), dim3((unsigned)threads), 0, (hipStream_t)stream,
+                     (float*)out, iters, operands);
+  return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
+}
+
+// as bench_probe_mfma_bf16, with v_mfma_f32_16x16x32_bf16 (16 * iters instructions per wavefront)
+extern "C" int bench_probe_mfma_bf16_16x16(void* out, size_t out_bytes, int work_groups, int wavefronts_per_simd, int iters,
+                                          int operands, void* stream) {
+  using namespace mase;
+  if (out == nullptr) return MASE_ERR_NULL;
+  if (work_groups < 1 || work_groups > 65536 || (wavefronts_per_simd != 1 && wavefronts_per_simd != 2) || iters < 1 || iters > kMaxProbeIters ||
+      operands < 0 || operands > 2)
+    return MASE_ERR_PARAM;
+  const int threads = 256 * wavefronts_per_simd;
+  if (out_bytes < (size_t)work_groups * threads * sizeof(float) + 16 || !aligned16(out)) return MASE_ERR_WORKSPACE;
+  hipLaunchKernelGGL(probe_mfma_bf16_16x16_kernel, dim3((unsigned)work_groups), dim3((unsigned)threads), 0, (hipStream_t)stream,
                      (float*)out, iters, operands);
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
