@@ -220,9 +220,9 @@ int mase_gemm_bf16_tn_packed(const void* A, const void* B_packed, const void* bi
 /* The tiled product with B held as an MXINT8 weight in fragment order: the code image and the scale image written by
  * mase_gemm_mxint8_pack_b from int8 codes [N, K] and scale bytes [N, K/32] (value = code * 2^(scale - 134): the packed
  * outputs of mase_mxint_qdq with element_bits 8, block 32).  1.03 bytes per weight in memory and on the way in; the
- * codes are widened to the same bf16 values in registers, so the result is that of mase_gemm_bf16_tn on the dequantized
- * weight (the same products added in the same order) as long as every scale byte is at least 8 (weights of 2^-119 and
- * less are taken as zero).  K % 128 == 0; images 16-byte / 2-byte aligned, the code image below 4 GiB.
+ * codes are widened to the same bf16 values in registers, so the result is that of mase_gemm_bf16_tn_packed on the
+ * dequantized weight (the same products added in the same order, bit for bit) as long as every scale byte is at least 8
+ * (weights of 2^-119 and less are taken as zero).  K % 128 == 0; images 16-byte / 8-byte aligned, the code image below 4 GiB.
  * _code_bytes / _scale_bytes: sizes of the two images (0 when K % 128 != 0).  Replaces the F.linear of
  * LinearMXInt.forward (nn/quantized/modules/linear.py:972) with the weight dequantized on the way into the matrix
  * instruction instead of beforehand. */

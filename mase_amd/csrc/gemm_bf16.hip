@@ -148,6 +148,9 @@ __device__ __forceinline__ void load_16_untracked(bf16x8_t& dst, uint32_t off, c
 __device__ __forceinline__ void load_8_untracked(uint2& dst, uint32_t off, const unsigned char* base) {
   asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(dst) : "v"(off), "s"(base) : "memory");
 }
+__device__ __forceinline__ void load_4_untracked(uint32_t& dst, uint32_t off, const unsigned char* base) {
+  asm volatile("global_load_dword %0, %1, %2" : "=v"(dst) : "v"(off), "s"(base) : "memory");
+}
 __device__ __forceinline__ void load_2_untracked(uint32_t& dst, uint32_t off, const unsigned char* base) {
   asm volatile("global_load_ushort %0, %1, %2" : "=v"(dst) : "v"(off), "s"(base) : "memory");
 }
@@ -157,15 +160,16 @@ __device__ __forceinline__ void load_2_untracked(uint32_t& dst, uint32_t off, co
 // BPACK (with STREAM, an even number of K tiles): B is the fragment-ordered image of mase_gemm_bf16_pack_b and its
 // fragments go from L2 straight into registers, one K tile ahead of the MFMAs that use them; only A passes through
 // LDS, in four stages of 32 KB (the copies landing in LDS while the wavefronts read their fragments is what holds the
-// plain kernel back).  The four wavefronts then split the 256 x 256 tile 1 x 4 (each 256 rows x 64 columns: 8 x 2 MFMA
-// tiles) instead of 2 x 2 (128 x 128: 4 x 4), so that no two wavefronts load the same B fragments: the CU's
+// plain kernel back).  The four wavefronts then split the 256 x 256 tile 1 x 4 (each 256 rows x 64 columns: 16 x 4
+// tiles of v_mfma_f32_16x16x32_bf16) instead of 2 x 2 (128 x 128), so that no two wavefronts load the same B fragments: the CU's
 // vector-memory path carries 32 KB of B per K tile next to A's 32 KB (64 KB with the 2 x 2 split, measured 5 % slower),
 // at the price of each wavefront reading all of A from LDS.  That path, not the matrix pipe, is what the K loop waits
 // for.
 // BCODES (with BPACK): B is an MXINT8 weight as codes + scale bytes in fragment order (mase_gemm_mxint8_pack_b): half
 // the bytes of the bf16 image in memory and on the way in; the codes are widened to the same bf16 operand values in
-// registers, one K step ahead of the MFMAs that use them (code + 128 as an unsigned byte -> v_cvt_f32_ubyte -> one fma
-// that removes the 128 and applies the block's power-of-two scale -> the upper half of the exact fp32 product).
+// registers, a K step (half a K tile) ahead of the MFMAs that use them (code + 128 as an unsigned byte ->
+// v_cvt_f32_ubyte -> one fma that removes the 128 and applies the block's power-of-two scale -> the upper half of the
+// exact fp32 product).
 // BATCHED (plain form only): the work items are the output tiles of `batches` independent products with strided
 // operands (the score and value products of an attention block, torch.bmm): an item's operand bases and its output
 // base follow from its product index; rows of A, B and C have the strides lda, ldb, ldc.
@@ -176,10 +180,10 @@ __device__ __forceinline__ void load_2_untracked(uint32_t& dst, uint32_t off, co
 template <int OUT_DT, bool STREAM, bool BPACK = false, bool BCODES = false, bool BATCHED = false, bool HALFN = false>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p) {
   constexpr int NI = BPACK ? 8 : 4, NJ = (BPACK || HALFN) ? 2 : 4;  // 32 x 32 tiles of a wavefront: rows x columns
-  // The bf16 image form computes with v_mfma_f32_16x16x32_bf16 (16 x 4 tiles of 16 x 16 per wavefront, two K steps of
+  // The fragment-ordered forms compute with v_mfma_f32_16x16x32_bf16 (16 x 4 tiles of 16 x 16 per wavefront, two K steps of
   // 32 per K tile): the same multiply-adds per cycle as the 32x32x16 instruction on paper, but under the board's power
   // limit the part sustains a clock about 8 % higher on it (measured with both instructions on random operands).
-  constexpr bool MI16 = BPACK && !BCODES;
+  constexpr bool MI16 = BPACK;
   constexpr int kBN = HALFN ? 128 : BN;                           // columns of an output tile
   constexpr int kCopiesB = HALFN ? kWaveCopies / 2 : kWaveCopies;  // copies of B per wavefront per K tile
   static_assert(!BCODES || BPACK, "codes come in fragment order");
@@ -511,13 +515,15 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // BPACK: B fragments of two K tiles (the one in use and the one being loaded): [buffer][2 * K step + column tile / 2]
   // [column tile % 2].  Image layout: 1 KB blocks [column tile of 16][K step of 32][lane][8 bf16], lane l = column
   // l % 16, K 8*(l/16)..+8.
-  bf16x8_t fb[(BPACK && !BCODES) ? 2 : 1][(BPACK && !BCODES) ? 4 : 1][NJ];
-  // BCODES: the codes of two K tiles [buffer][K step][column tile] (8 per lane), their scale bytes [buffer][column
-  // tile] (the two blocks of 32 a K tile holds, for the lane's column) and the widened fragments of two K steps
+  bf16x8_t fb[(BPACK && !BCODES) ? 2 : 1][(BPACK && !BCODES) ? 4 : 1][2];
+  // BCODES: the codes of two K tiles [buffer][2 * K step + column tile / 2][column tile % 2] (8 per lane: K step of 32,
+  // column tile of 16, lane l = column l % 16, K 8 * (l / 16) .. + 8), the scale bytes of the lane's column in the four
+  // column tiles [buffer][K step] (byte ct = column tile ct) and the widened fragments of the two K steps [K step][column
+  // tile]
   uint2 fbc[BCODES ? 2 : 1][BCODES ? 4 : 1][2];
   uint32_t fsc[BCODES ? 2 : 1][2];
-  uint4 fbq[2][2];
-  uint32_t soff[2];          // BCODES: this lane's byte offset of K tile 0 of its four column tiles in the scale image
+  uint4 fbq[BCODES ? 2 : 1][BCODES ? 4 : 1];
+  uint32_t soff = 0;         // BCODES: this lane's byte offset of K tile 0 of its 64 columns in the scale image
   const unsigned char* s_kbase = p.Bs;
   uint32_t boff[4];          // this lane's byte offset of K step 0 of its four column tiles
   const unsigned char* b_kbase = p.B;  // image address of K tile 0 of the K range of the output tile being loaded
@@ -528,64 +534,93 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     const int lane = lane_now();
     const int nt_last = (p.N + 31) / 32 - 1;
     constexpr uint32_t kFragBytes = BCODES ? 512u : 1024u;  // one fragment of a wavefront: 8 codes or 8 bf16 per lane
-    if constexpr (MI16) {
+    {
       // four column tiles of 16; the image holds a multiple of 32 columns (those beyond N are zero)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const size_t ct = (size_t)min((n0 + col_base) / 16 + j, 2 * nt_last + 1);
-        boff[j] = (uint32_t)(ct * (size_t)(p.K / 32) * 1024u) + (uint32_t)lane * 16u;
+        boff[j] = (uint32_t)(ct * (size_t)(p.K / 32) * kFragBytes) + (uint32_t)lane * (kFragBytes / 64u);
       }
-      b_kbase = p.B + (size_t)ks * (size_t)(p.kc / 32) * 1024u;
+      b_kbase = p.B + (size_t)ks * (size_t)(p.kc / 32) * kFragBytes;
+      if constexpr (BCODES) {
+        // scale image: 128-byte blocks [64 columns][K tile][column % 16][K step][column / 16]
+        const size_t g64 = (size_t)min((n0 + col_base) / 64, (p.N + 63) / 64 - 1);
+        soff = (uint32_t)(g64 * (size_t)(p.K / 64) * 128u) + (uint32_t)(lane & 15) * 8u;
+        s_kbase = p.Bs + (size_t)ks * (size_t)(p.kc / 64) * 128u;
+      }
       b_kt = 0;
-      return;
     }
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const size_t ct = (size_t)min((n0 + col_base) / 32 + j, nt_last);
-      boff[j] = (uint32_t)(ct * (size_t)(p.K / 16) * kFragBytes) + (uint32_t)lane * (kFragBytes / 64u);
-      if constexpr (BCODES) soff[j] = (uint32_t)(ct * (size_t)(p.K / 64) * 64u) + (uint32_t)(lane & 31) * 2u;
-    }
-    b_kbase = p.B + (size_t)ks * (size_t)(p.kc / 16) * kFragBytes;
-    if constexpr (BCODES) s_kbase = p.Bs + (size_t)ks * (size_t)(p.kc / 64) * 64u;
-    b_kt = 0;
   };
-  // BCODES: widening of the fragment of column tile j, K step st of the K tile in code buffer `buf` into fragment set
-  // `set`; `half` 0 / 1 = the first / second four codes.  The scale byte of a step is byte st / 2 of the lane's two.
-  // The widening is issued in pieces small enough to hide between two MFMAs (which leave room for about seven VALU
-  // instructions): set_scale puts the scale of block `blk` (0 / 1) of column tile j of the K tile in buffer `buf`, and
-  // the -128 * scale that removes the code offset, into wsc / wbs; widen_quarter makes register q (0..3: two codes) of
-  // the fragment of column tile j, K step st ((code - 128) * scale is exact in fp32 and has at most 8 significant
-  // bits, so the upper half of the fp32 value is the bf16 value).
-  float wsc[2], wbs[2];
-  auto set_scale = [&](int buf, int blk, int j) __attribute__((always_inline)) {
-    const uint32_t sb = (fsc[buf][j] >> (8 * blk)) & 0xFFu;
-    wsc[j] = bits2f(sb >= 8u ? (sb - 7u) << 23 : 0u);  // 2^(sb - 134)
-    wbs[j] = -128.0f * wsc[j];
+  // BCODES: the loads of one half of a K tile's codes (K step st: its scale dword and its four fragments), and the
+  // widening.  set_scale puts the scale of the lane's column in column tile ct (K step st of the K tile in buffer
+  // `buf`), and the -128 * scale that removes the code offset, into wsc / wbs; widen_quarter makes register r (0..3:
+  // two codes) of the fragment of column tile ct ((code - 128) * scale is exact in fp32 and has at most 8 significant
+  // bits, so the upper half of the fp32 value is the bf16 value).  A quarter register is 5 vector instructions.
+  float wsc[4], wbs[4];
+  auto load_codes_half = [&](int buf, int st, int i, const unsigned char* csrc, const unsigned char* ssrc) __attribute__((always_inline)) {
+    // i = 0: the scale dword; i = 1..4: the codes of column tile i - 1
+    if (i == 0) load_4_untracked(fsc[buf][st], soff + (uint32_t)st * 4u, ssrc);
+    else load_8_untracked(fbc[buf][st * 2 + ((i - 1) >> 1)][(i - 1) & 1], boff[i - 1], csrc + (size_t)st * 512);
   };
-  auto widen_quarter = [&](int set, int buf, int st, int j, int q) __attribute__((always_inline)) {
-    const uint32_t u = (q & 2) ? fbc[buf][st][j].y : fbc[buf][st][j].x;
-    const float f0 = __builtin_fmaf((float)((q & 1) ? (u >> 16) & 0xFFu : u & 0xFFu), wsc[j], wbs[j]);
-    const float f1 = __builtin_fmaf((float)((q & 1) ? u >> 24 : (u >> 8) & 0xFFu), wsc[j], wbs[j]);
-    const uint32_t r = __builtin_amdgcn_perm(f2bits(f1), f2bits(f0), 0x07060302u);  // the upper halves: two bf16
-    if (q == 0) fbq[set][j].x = r;
-    else if (q == 1) fbq[set][j].y = r;
-    else if (q == 2) fbq[set][j].z = r;
-    else fbq[set][j].w = r;
+  // (each in two parts, one for either gap of a slot: three vector instructions fit between two matrix instructions.
+  // The parts are volatile assembly: plain arithmetic has no ordering against the matrix instructions or the scheduling
+  // barriers when the compiler lays the block out, and it gathered both parts of a slot in one gap.)
+  uint32_t wsb = 0;
+  float wc0 = 0.0f, wc1 = 0.0f;
+  auto set_scale_a = [&](int buf, int st, int ct) __attribute__((always_inline)) {
+    const uint32_t w = fsc[buf][st];
+    if (ct == 0) asm volatile("v_bfe_u32 %0, %1, 0, 8\n\tv_max_u32 %0, 7, %0" : "=v"(wsb) : "v"(w));
+    else if (ct == 1) asm volatile("v_bfe_u32 %0, %1, 8, 8\n\tv_max_u32 %0, 7, %0" : "=v"(wsb) : "v"(w));
+    else if (ct == 2) asm volatile("v_bfe_u32 %0, %1, 16, 8\n\tv_max_u32 %0, 7, %0" : "=v"(wsb) : "v"(w));
+    else asm volatile("v_bfe_u32 %0, %1, 24, 8\n\tv_max_u32 %0, 7, %0" : "=v"(wsb) : "v"(w));
+  };
+  auto set_scale_b = [&](int ct) __attribute__((always_inline)) {
+    // 2^(scale byte - 134), 0 for scale bytes below 8; and -128 times that
+    asm volatile("v_lshl_add_u32 %0, %2, 23, %3\n\tv_mul_f32 %1, 0xc3000000, %0"
+                 : "=&v"(wsc[ct]), "=v"(wbs[ct])
+                 : "v"(wsb), "v"(0xFC800000u));
+  };
+  auto set_scale = [&](int buf, int st, int ct) __attribute__((always_inline)) {
+    set_scale_a(buf, st, ct);
+    set_scale_b(ct);
+  };
+  auto widen_quarter_a = [&](int buf, int st, int ct, int r) __attribute__((always_inline)) {
+    const uint2 c = fbc[buf][st * 2 + (ct >> 1)][ct & 1];
+    const uint32_t u = (r & 2) ? c.y : c.x;
+    if (r & 1) asm volatile("v_cvt_f32_ubyte2 %0, %2\n\tv_cvt_f32_ubyte3 %1, %2" : "=&v"(wc0), "=v"(wc1) : "v"(u));
+    else asm volatile("v_cvt_f32_ubyte0 %0, %2\n\tv_cvt_f32_ubyte1 %1, %2" : "=&v"(wc0), "=v"(wc1) : "v"(u));
+  };
+  auto widen_quarter_b = [&](int st, int ct, int r) __attribute__((always_inline)) {
+    uint32_t v;  // the upper halves of the two products: two bf16
+    asm volatile("v_fma_f32 %0, %0, %3, %4\n\tv_fma_f32 %1, %1, %3, %4\n\tv_perm_b32 %2, %1, %0, %5"
+                 : "+v"(wc0), "+v"(wc1), "=v"(v)
+                 : "v"(wsc[ct]), "v"(wbs[ct]), "s"(0x07060302u));
+    if (r == 0) fbq[st][ct].x = v;
+    else if (r == 1) fbq[st][ct].y = v;
+    else if (r == 2) fbq[st][ct].z = v;
+    else fbq[st][ct].w = v;
+  };
+  auto widen_quarter = [&](int buf, int st, int ct, int r) __attribute__((always_inline)) {
+    widen_quarter_a(buf, st, ct, r);
+    widen_quarter_b(st, ct, r);
   };
   if constexpr (BCODES) {
+    // K tiles 0 and 1 in full; K step 0 of K tile 0 widened
     set_b_tile(0);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) load_2_untracked(fsc[0][j], soff[j], s_kbase);
+    for (int b = 0; b < 2; ++b)
 #pragma unroll
-    for (int i = 0; i < 8; ++i) load_8_untracked(fbc[0][i >> 1][i & 1], boff[i & 1], b_kbase + (size_t)(i >> 1) * 512);
-    b_kt = 1;
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int i = 0; i < 5; ++i) load_codes_half(b, st, i, b_kbase + (size_t)b * 1024, s_kbase + (size_t)b * 128);
+    b_kt = 2;
     wait_vmcnt<0>();
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      set_scale(0, 0, j);
+    for (int ct = 0; ct < 4; ++ct) {
+      set_scale(0, 0, ct);
 #pragma unroll
-      for (int q = 0; q < 4; ++q) widen_quarter(0, 0, 0, j, q);
+      for (int r = 0; r < 4; ++r) widen_quarter(0, 0, ct, r);
     }
   } else if constexpr (BPACK) {
     set_b_tile(0);
@@ -674,53 +709,67 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     stage = stage_next;
     ++b_kt;
   };
-  // BCODES form: as the BPACK form, with 2 scale loads and 8 code loads per K tile (step 0, slots 0..7: the scale of
-  // column tile t first in slots 0 and 1, then the codes of K step t / 2, column tile t % 2) and the widening of K
-  // step s + 1 (of step 0 of the next K tile during step 3) spread over the MFMA slots of step s, two codes at a
-  // time.  A step's codes must have landed one step earlier than in the BPACK form; counting the register loads issued after them (batch order S0 C0 S1 C1 C2 .. C7): codes of step 1 (C2, C3):
-  // 4 at the head of the K tile; step 2 (C4, C5): 2 + the 10 of the next batch at the head of step 1; step 3: 10 at
-  // the head of step 2; scales and codes of step 0 of the next K tile (S0 .. C1 of the batch issued during step 0):
-  // 6 at the head of step 3.
+  // BCODES form.  The matrix instructions of quarter q read the widened fragments fbq[q / 2][column tile]; the codes
+  // themselves are read only by the widening, so a half of a code buffer is free again as soon as its K step has been
+  // widened, and the loads run a K tile and a half ahead of their use with two buffers:
+  //   quarter 0: LDS reads of quarters 1 and 2 (16); slots 0..4: the loads of K step 0 of the K tile after next (scale
+  //              dword + 4 fragments of 8 bytes per lane) into this buffer's K step 0 half (widened during quarter 3 of
+  //              the previous K tile); before slot 12: K step 1 of this K tile has landed; slots 12..15: its scales
+  //   quarter 1: LDS reads of quarter 3 (8); widening of K step 1 of this K tile, one quarter register per slot; 4 A copies
+  //   quarter 2: slots 0..4: the loads of K step 1 of the K tile after next into this buffer's K step 1 half; 4 A
+  //              copies; before slot 12: K step 0 of the next K tile has landed; slots 12..15: its scales; hand-over
+  //   quarter 3: LDS reads of quarter 0 of the next K tile (8); widening of K step 0 of the next K tile
+  // Register loads in issue order: .. H0(k+1) H1(k+1) | H0(k+2) [quarter 0] H1(k+2) [quarter 2] with 5 loads per half.
+  // The wait in quarter 0 needs H1(k), after which H0(k+1), H1(k+1), H0(k+2) = 15 register loads were issued; the wait
+  // in quarter 2 needs H0(k+1), followed by H1(k+1), H0(k+2), H1(k+2) = 15: "at most 15 outstanding" both times.  What
+  // these waits complete besides is at least three quarters of a K tile old.  The hand-over is the one of the bf16
+  // image form (the 16 youngest of the A copies belong to later K tiles).
   auto k_iteration_c = [&](auto&& advance, auto bufc) __attribute__((always_inline)) {
     constexpr int NB = decltype(bufc)::value;
-    const unsigned char* bsrc = b_kbase + (size_t)b_kt * 2048;
-    const unsigned char* ssrc = s_kbase + (size_t)b_kt * 64;
+    const unsigned char* bsrc = b_kbase + (size_t)b_kt * 1024;
+    const unsigned char* ssrc = s_kbase + (size_t)b_kt * 128;
     const int stage_next = next_of(stage);
 #pragma unroll
-    for (int s = 0; s < kSteps; ++s) {
-      if (s == 0) wait_vmcnt<4>();
-      else if (s == 1) wait_vmcnt<12>();
-      else if (s == 2) wait_vmcnt<10>();
-      else wait_vmcnt<6>();
-      __builtin_amdgcn_sched_barrier(0);  // nothing that reads the codes or scales may be hoisted above the wait
+    for (int q = 0; q < 4; ++q) {
 #pragma unroll
       for (int t = 0; t < 16; ++t) {
-        acc[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            __builtin_bit_cast(bf16x8_t, fbq[s & 1][t & 1]), fr[s][t >> 1], acc[t >> 1][t & 1], 0, 0, 0);
-        // slots 0, 1 of the steps after which the block of 32 changes: the scales the next step's codes take; slots
-        // 2, 4, .., 14, 15: quarter u = 0..7 (column tile u / 4, register u % 4) of the next step's fragments
-        if ((s & 1) && t < 2) set_scale(s == 1 ? NB : NB ^ 1, s == 1 ? 1 : 0, t);
-        const int u = (t == 15) ? 7 : ((t >= 2 && !(t & 1)) ? (t - 2) >> 1 : -1);
-        if (u >= 0) {
-          if (s < 3) widen_quarter((s + 1) & 1, NB, s + 1, u >> 2, u & 3);
-          else widen_quarter(0, NB ^ 1, 0, u >> 2, u & 3);
+        if ((q == 0 || q == 2) && t == 12) {
+          wait_vmcnt<15>();
+          __builtin_amdgcn_sched_barrier(0);  // nothing that reads the codes or scales may be hoisted above the wait
         }
-        if (s == 0) {
-          if (t < 8) {
-            fr[1][t] = load_frag(stage, 1, t);
-            if (t < 2) load_2_untracked(fsc[NB ^ 1][t], soff[t], ssrc);
-            load_8_untracked(fbc[NB ^ 1][t >> 1][t & 1], boff[t & 1], bsrc + (size_t)(t >> 1) * 512);
-          }
-        } else if (s == 1) {
-          if (t < 8) fr[2][t] = load_frag(stage, 2, t);
-          else fr[3][t - 8] = load_frag(stage, 3, t - 8);
-          if (t & 1) issue_copy(t - 1);
-        } else if (s == 3) {
+        const int it = (q & 1) * 8 + (t >> 1), jt = 2 * (t & 1);
+        mfma16_acc(acc16[it][jt], __builtin_bit_cast(bf16x8_t, fbq[q >> 1][jt]), fr[q][t >> 1]);
+        if (q == 0) {
+          if (t < 8) fr[1][t] = load_frag(stage, 1, t);
+          else fr[2][t - 8] = load_frag(stage, 2, t - 8);
+          if (t >= 12) set_scale_a(NB, 1, t - 12);
+        } else if (q == 1) {
+          if (t < 8) fr[3][t] = load_frag(stage, 3, t);
+          widen_quarter_a(NB, 1, t >> 2, t & 3);
+        } else if (q == 2) {
+          if (t >= 12) set_scale_a(NB ^ 1, 0, t - 12);
+        } else {
           if (t < 8) fr[0][t] = load_frag(stage_next, 0, t);
+          widen_quarter_a(NB ^ 1, 0, t >> 2, t & 3);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mfma16_acc(acc16[it][jt + 1], __builtin_bit_cast(bf16x8_t, fbq[q >> 1][jt + 1]), fr[q][t >> 1]);
+        if (q == 0) {
+          if (t < 5) load_codes_half(NB, 0, t, bsrc, ssrc);
+          if (t >= 12) set_scale_b(t - 12);
+        } else if (q == 1) {
+          widen_quarter_b(1, t >> 2, t & 3);
+          if ((t & 3) == 3) issue_copy((t >> 2) * 2);
+        } else if (q == 2) {
+          if (t < 5) load_codes_half(NB, 1, t, bsrc, ssrc);
+          else if (t < 12 && (t & 1)) issue_copy(8 + ((t - 5) >> 1) * 2);
+          if (t >= 12) set_scale_b(t - 12);
+        } else {
+          widen_quarter_b(0, t >> 2, t & 3);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
-      if (s == 2) {
+      if (q == 2) {
         wait_vmcnt<(kStagesB - 2) * kWaveCopies>();
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
@@ -816,8 +865,14 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
       }
 #pragma unroll 1
       for (; kt < nk; kt += 2) {
+        // the B stream moves on to the next output tile: one K tile ahead (bf16 image), two ahead (codes)
+        if constexpr (BCODES) {
+          if (kt + 2 >= nk) set_b_tile(ord + 1);
+        }
         iter(std::integral_constant<int, 0>{}, advance_copy_stream);
-        if (kt + 2 >= nk) set_b_tile(ord + 1);
+        if constexpr (!BCODES) {
+          if (kt + 2 >= nk) set_b_tile(ord + 1);
+        }
         iter(std::integral_constant<int, 1>{}, advance_copy_stream);
       }
     } else if constexpr (STREAM) {
@@ -958,36 +1013,46 @@ __global__ __launch_bounds__(256) void gemm_pack_b_kernel(const uint4* __restric
 }
 
 // MXINT8 weight [N, K] (int8 codes, one scale byte per 32 along K) -> fragment-ordered images for the BCODES kernel:
-// codes: 512-byte blocks [column tile of 32][K step of 16][lane][8 bytes], lane l of a block holding the codes of
-// column tile*32 + l%32 at K = step*16 + 8*(l/32) .. +8, each plus 128 (an unsigned byte); columns beyond N hold 128
-// (zero).  scales: 64-byte blocks [column tile][K tile of 64][column][2 bytes] (the scale bytes of the K tile's two
-// blocks of 32).
-__global__ __launch_bounds__(256) void gemm_pack_codes_kernel(const uint2* __restrict__ codes, const uint8_t* __restrict__ scales,
-                                                              uint2* __restrict__ img, uint16_t* __restrict__ simg, int N,
+// codes: 512-byte blocks [column tile of 16][K step of 32][lane][8 bytes], lane l of a block holding the codes of
+// column tile*16 + l%16 at K = step*32 + 8*(l/16) .. +8, each plus 128 (an unsigned byte); columns beyond N (the image
+// holds a multiple of 32) hold 128 (zero).  scales: 128-byte blocks [64 columns][K tile of 64][column % 16][8 bytes],
+// byte 4 * s + c of a lane's eight = the scale byte of column 64 * group + 16 * c + column % 16 in block 2 * tile + s;
+// columns beyond N (the image holds a multiple of 64) have scale 0.
+__global__ __launch_bounds__(256) void gemm_pack_codes_kernel(const uint2* __restrict__ codes, uint2* __restrict__ img, int N,
                                                               int K, size_t granules) {
   const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (g >= granules) return;
   const int lane = (int)(g & 63);
   const size_t blk = g >> 6;
-  const int steps = K / 16;
+  const int steps = K / 32;
   const int nt = (int)(blk / (size_t)steps), ks = (int)(blk % (size_t)steps);
-  const int row = nt * 32 + (lane & 31);
+  const int row = nt * 16 + (lane & 15);
   uint2 v = make_uint2(0x80808080u, 0x80808080u);
   if (row < N) {
-    v = codes[((size_t)row * K + (size_t)ks * 16 + 8 * (lane >> 5)) / 8];
+    v = codes[((size_t)row * K + (size_t)ks * 32 + 8 * (lane >> 4)) / 8];
     v.x ^= 0x80808080u;
     v.y ^= 0x80808080u;
   }
   img[g] = v;
-  if ((ks & 3) == 0 && lane < 32) {  // one lane per column writes the K tile's two scale bytes
-    const int kt = ks >> 2;
-    uint16_t sc = 0;
-    if (row < N) {
-      const uint8_t* sp = scales + (size_t)row * (K / 32) + (size_t)kt * 2;
-      sc = (uint16_t)sp[0] | ((uint16_t)sp[1] << 8);
+}
+// one work-item per (64 columns, K tile, column % 16): its eight scale bytes
+__global__ __launch_bounds__(256) void gemm_pack_scales_kernel(const uint8_t* __restrict__ scales, uint2* __restrict__ simg, int N,
+                                                               int K, size_t items) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= items) return;
+  const int c16 = (int)(g & 15);
+  const size_t blk = g >> 4;
+  const int ktiles = K / 64;
+  const int g64 = (int)(blk / (size_t)ktiles), kt = (int)(blk % (size_t)ktiles);
+  uint32_t w[2] = {0u, 0u};
+#pragma unroll
+  for (int st = 0; st < 2; ++st)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int row = g64 * 64 + c * 16 + c16;
+      if (row < N) w[st] |= (uint32_t)scales[(size_t)row * (K / 32) + (size_t)kt * 2 + st] << (8 * c);
     }
-    simg[((size_t)nt * (K / 64) + kt) * 32 + lane] = sc;
-  }
+  simg[g] = make_uint2(w[0], w[1]);
 }
 
 // K ranges for a product whose output tiles alone would leave most CUs idle: as many as fill the machine once, each a
@@ -1180,7 +1245,7 @@ extern "C" size_t mase_gemm_mxint8_packed_code_bytes(size_t N, size_t K) {
 
 extern "C" size_t mase_gemm_mxint8_packed_scale_bytes(size_t N, size_t K) {
   if (N == 0 || K == 0 || (K % 128) != 0) return 0;
-  return ((N + 31) / 32) * 32 * (K / 32);
+  return ((N + 63) / 64) * 64 * (K / 32);
 }
 
 extern "C" int mase_gemm_mxint8_pack_b(const int8_t* codes, const uint8_t* scales, void* code_image, void* scale_image,
@@ -1189,10 +1254,13 @@ extern "C" int mase_gemm_mxint8_pack_b(const int8_t* codes, const uint8_t* scale
   if (N == 0 || K == 0) return MASE_OK;
   if (codes == nullptr || scales == nullptr || code_image == nullptr || scale_image == nullptr) return MASE_ERR_NULL;
   if ((K % 128) != 0 || N > (1u << 30) || K > (1u << 30)) return MASE_ERR_SHAPE;
-  if ((((uintptr_t)codes) & 7u) != 0 || !aligned16(code_image) || (((uintptr_t)scale_image) & 1u) != 0) return MASE_ERR_ALIGN;
+  if ((((uintptr_t)codes) & 7u) != 0 || !aligned16(code_image) || (((uintptr_t)scale_image) & 7u) != 0) return MASE_ERR_ALIGN;
   const size_t granules = mase_gemm_mxint8_packed_code_bytes(N, K) / 8;
   hipLaunchKernelGGL(gemm_pack_codes_kernel, dim3(blocks_for(granules, (size_t)256)), dim3(256), 0, (hipStream_t)stream,
-                     (const uint2*)codes, scales, (uint2*)code_image, (uint16_t*)scale_image, (int)N, (int)K, granules);
+                     (const uint2*)codes, (uint2*)code_image, (int)N, (int)K, granules);
+  const size_t items = mase_gemm_mxint8_packed_scale_bytes(N, K) / 8;
+  hipLaunchKernelGGL(gemm_pack_scales_kernel, dim3(blocks_for(items, (size_t)256)), dim3(256), 0, (hipStream_t)stream,
+                     scales, (uint2*)scale_image, (int)N, (int)K, items);
   return hipGetLastError() == hipSuccess ? MASE_OK : MASE_ERR_LAUNCH;
 }
 
@@ -1206,7 +1274,7 @@ extern "C" int mase_gemm_mxint8_tn_packed(const void* A, const void* code_image,
   if ((unsigned long long)M * K * 2 > 0xFFFFFFFFull ||
       (unsigned long long)mase_gemm_mxint8_packed_code_bytes(N, K) > 0xFFFFFFFFull)
     return MASE_ERR_SHAPE;
-  if (!aligned16(A) || !aligned16(code_image) || (((uintptr_t)scale_image) & 1u) != 0) return MASE_ERR_ALIGN;
+  if (!aligned16(A) || !aligned16(code_image) || (((uintptr_t)scale_image) & 7u) != 0) return MASE_ERR_ALIGN;
   if (out_dtype < 0 || out_dtype > 2 || (bias != nullptr && (bias_dtype < 0 || bias_dtype > 2))) return MASE_ERR_DTYPE;
   GemmParams p;
   p.A = (const unsigned char*)A;

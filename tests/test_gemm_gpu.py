@@ -319,10 +319,11 @@ def test_gemm_output_not_on_a_16_byte_boundary(dev, dt):
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (512, 768, 256), (300, 200, 384), (4096, 4096, 1024), (130, 4096, 512),
                                    (4100, 4200, 640), (16384, 1024, 4096), (16384, 4096, 11008), (16131, 11008, 4096)])
 def test_gemm_with_the_weight_as_mxint8_codes_in_fragment_order(dev, M, N, K):
-    """mase_gemm_mxint8_tn_packed (weight as int8 codes + scale bytes, widened in registers) against mase_gemm_bf16_tn
-    on the dequantized weight: the operands the matrix instruction sees are the same bf16 values, so the results are
-    bit-identical, for every output dtype, with a bias, ragged M and N, several launches"""
-    from mase_amd._gemm import gemm_bf16_tn, gemm_mxint8_pack_b, gemm_mxint8_tn_packed
+    """mase_gemm_mxint8_tn_packed (weight as int8 codes + scale bytes, widened in registers) against
+    mase_gemm_bf16_tn_packed on the dequantized weight: the operands the matrix instruction sees are the same bf16
+    values and the products are added in the same order, so the results are bit-identical, for every output dtype, with
+    a bias, ragged M and N, several launches"""
+    from mase_amd._gemm import gemm_bf16_pack_b, gemm_bf16_tn, gemm_mxint8_pack_b, gemm_mxint8_tn_packed
     from mase_amd.quantizers import _ops
 
     g = torch.Generator().manual_seed(M + N + K + 1)
@@ -334,13 +335,14 @@ def test_gemm_with_the_weight_as_mxint8_codes_in_fragment_order(dev, M, N, K):
     print(f"mxint8-codes gemm M={M} N={N} K={K}", flush=True)
     deq, codes, scales = _ops.mxint_qdq(w.to(dev), 32, 8, 1, 8, pack=True, out_dtype=torch.bfloat16)
     img, simg = gemm_mxint8_pack_b(codes.view(N, K), scales.view(N, K // 32))
-    assert img.numel() == (N + 31) // 32 * 32 * K and simg.numel() == (N + 31) // 32 * 32 * (K // 32)
+    assert img.numel() == (N + 31) // 32 * 32 * K and simg.numel() == (N + 63) // 64 * 64 * (K // 32)
     from mase_amd import _lib
 
     # a few hundred rows: gemm_bf16_tn cuts K into ranges there and adds the partial sums in another order
     split = _lib.load().mase_gemm_bf16_tn_splitk_workspace_bytes(M, N, K) > 0
+    bp = gemm_bf16_pack_b(deq.view(N, K))
     for dt, bs in ((torch.float32, None), (torch.bfloat16, bias), (torch.float16, bias.to(torch.float16))):
-        want = gemm_bf16_tn(a, deq.view(N, K), bs, dt)
+        want = gemm_bf16_tn(a, deq.view(N, K), bs, dt, b_packed=bp)
         for rep in range(3 if M * N * K > (1 << 36) else 2):
             got = gemm_mxint8_tn_packed(a, img, simg, N, bs, dt)
             if split:
