@@ -445,15 +445,27 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
         }
       }
     };
-    // (Staging band b + 1 between the issue of band b's reads and their use was measured: no gain, more registers.)
+    // Staging band b + 1 between the issue of band b's reads and their use (the LDS executes a wavefront's accesses in
+    // the order of issue, so the next band can be written behind the reads while their data is on its way) pays where
+    // the epilogue is a large part of the kernel, the batched form with its few K tiles per output tile (score product
+    // of an attention block: 6 % faster); with long K loops it was measured without gain or slightly slower.
+    constexpr bool kPipeBands = BATCHED;
+    if constexpr (kPipeBands) stage_band(0);
 #pragma unroll
     for (int b = 0; b < kBands; ++b) {
       const int i = b / kBandsPerRowTile, jb = b % kBandsPerRowTile;
-      stage_band(b);
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the band is in LDS before any lane reads it
+      if constexpr (!kPipeBands) {
+        stage_band(b);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the band is in LDS before any lane reads it
+      }
       uint4 w[4];
 #pragma unroll
       for (int ps = 0; ps < 4; ++ps) w[ps] = *(const uint4*)(stg_r + ps * 8 * kStgRow);
+      if constexpr (kPipeBands) {
+        asm volatile("" ::: "memory");
+        if (b + 1 < kBands) stage_band(b + 1);
+        asm volatile("" ::: "memory");
+      }
       // streaming stores: the output is not read again by this kernel and should not displace operand panels
       unsigned char* const dst0 = lane_c + (size_t)(i * 32) * row_step + jb * 128;
       if (__builtin_expect(interior, 1)) {
