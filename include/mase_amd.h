@@ -208,10 +208,9 @@ int mase_gemm_bf16_tn_splitk(const void* A, const void* B, const void* bias, voi
  * once when it is loaded): B's fragments then go from the cache straight into registers instead of through LDS, which
  * the kernel otherwise shares between the copies arriving and the fragment reads.  K % 128 == 0; the image takes
  * mase_gemm_bf16_packed_bytes(N, K) = ceil(N/32)*32*K*2 bytes (below 4 GiB), 16-byte aligned; the packer takes any
- * K % 32 == 0.  The same exact products with fp32 accumulation as mase_gemm_bf16_tn, added in another order (this kernel
- * computes with the 16x16x32 matrix instruction, 32 products per instruction where mase_gemm_bf16_tn adds 16): equal to
- * fp32 rounding of the sums, bit-identical where every partial sum is exact (small integers).  Replaces the same
- * F.linear (nn/quantized/modules/linear.py:972, :895). */
+ * K % 32 == 0.  Same results as mase_gemm_bf16_tn (the same products added in the same order: both compute with the
+ * 16x16x32 matrix instruction, K step by K step).  Replaces the same F.linear (nn/quantized/modules/linear.py:972,
+ * :895). */
 size_t mase_gemm_bf16_packed_bytes(size_t N, size_t K);
 int mase_gemm_bf16_pack_b(const void* B, void* B_packed, size_t N, size_t K, void* stream);
 int mase_gemm_bf16_tn_packed(const void* A, const void* B_packed, const void* bias, void* C, size_t M, size_t N,
@@ -220,7 +219,7 @@ int mase_gemm_bf16_tn_packed(const void* A, const void* B_packed, const void* bi
 /* The tiled product with B held as an MXINT8 weight in fragment order: the code image and the scale image written by
  * mase_gemm_mxint8_pack_b from int8 codes [N, K] and scale bytes [N, K/32] (value = code * 2^(scale - 134): the packed
  * outputs of mase_mxint_qdq with element_bits 8, block 32).  1.03 bytes per weight in memory and on the way in; the
- * codes are widened to the same bf16 values in registers, so the result is that of mase_gemm_bf16_tn_packed on the
+ * codes are widened to the same bf16 values in registers, so the result is that of mase_gemm_bf16_tn on the
  * dequantized weight (the same products added in the same order, bit for bit) as long as every scale byte is at least 8
  * (weights of 2^-119 and less are taken as zero).  K % 128 == 0; images 16-byte / 8-byte aligned, the code image below 4 GiB.
  * _code_bytes / _scale_bytes: sizes of the two images (0 when K % 128 != 0).  Replaces the F.linear of

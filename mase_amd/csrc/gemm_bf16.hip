@@ -1,14 +1,14 @@
 // C[M,N] = A[M,K] * B[N,K]^T (+ bias[N]) on gfx950 matrix cores: bf16 operands, fp32 accumulation.
 //
 // This is the contraction behind the MX Linear forward.  Both operands are K-major (activations [tokens, K],
-// weights [out, K]), which is the layout v_mfma_f32_32x32x16_bf16 wants: lane l supplies 8 consecutive
-// K-elements of row/column l%32, K-group l/32.  MXINT8 and MXFP values are exactly representable in bf16
+// weights [out, K]), which is the layout v_mfma_f32_16x16x32_bf16 wants: lane l supplies 8 consecutive
+// K-elements of row/column l%16, K-group l/16 (v_mfma_f32_32x32x16_bf16, used by the narrow form: l%32, l/32).  MXINT8 and MXFP values are exactly representable in bf16
 // (<= 8 significant bits times a power of two), so feeding them as bf16 computes the same real-number dot
 // products as the reference's fp32 GEMM on the quantize-dequantized operands; only the summation order
 // differs.
 //
-// Schedule: 256x256 output tile (4 wavefronts, 2x2, 128x128 each = 4x4 MFMA tiles, or 1x4, 256x64 each = 8x2 MFMA
-// tiles, when B comes in fragment order; 256 accumulator registers per lane either way), K tile 64 so that every operand row of a tile is one full 128-byte cache line (64-byte rows made
+// Schedule: 256x256 output tile (4 wavefronts, 2x2, 128x128 each = 8x8 MFMA tiles of 16x16, or 1x4, 256x64 each =
+// 16x4 tiles, when B comes in fragment order; 256 accumulator registers per lane either way), K tile 64 so that every operand row of a tile is one full 128-byte cache line (64-byte rows made
 // the L1 fetch every line twice and bound the loop), two LDS stages of 64 KB.  Operand tiles go from HBM/L2
 // straight into LDS with global_load_lds_dwordx4 (no staging registers, no ds_write).  A wavefront-wide copy
 // deposits 64 consecutive 16-byte chunks = 8 LDS rows of 128 B, so the bank-conflict swizzle is applied on
@@ -180,10 +180,10 @@ __device__ __forceinline__ void load_2_untracked(uint32_t& dst, uint32_t off, co
 template <int OUT_DT, bool STREAM, bool BPACK = false, bool BCODES = false, bool BATCHED = false, bool HALFN = false>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p) {
   constexpr int NI = BPACK ? 8 : 4, NJ = (BPACK || HALFN) ? 2 : 4;  // 32 x 32 tiles of a wavefront: rows x columns
-  // The fragment-ordered forms compute with v_mfma_f32_16x16x32_bf16 (16 x 4 tiles of 16 x 16 per wavefront, two K steps of
-  // 32 per K tile): the same multiply-adds per cycle as the 32x32x16 instruction on paper, but under the board's power
+  // All forms but the narrow one compute with v_mfma_f32_16x16x32_bf16 (16 x 4 or 8 x 8 tiles of 16 x 16 per wavefront,
+  // two K steps of 32 per K tile): the same multiply-adds per cycle as the 32x32x16 instruction on paper, but under the board's power
   // limit the part sustains a clock about 8 % higher on it (measured with both instructions on random operands).
-  constexpr bool MI16 = BPACK;
+  constexpr bool MI16 = !HALFN;
   constexpr int kBN = HALFN ? 128 : BN;                           // columns of an output tile
   constexpr int kCopiesB = HALFN ? kWaveCopies / 2 : kWaveCopies;  // copies of B per wavefront per K tile
   static_assert(!BCODES || BPACK, "codes come in fragment order");
@@ -295,13 +295,14 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   };
 
   f32x16_t acc[MI16 ? 1 : NI][MI16 ? 1 : NJ];
-  f32x4_t acc16[MI16 ? 16 : 1][MI16 ? 4 : 1];  // MI16: [row tile of 16][column tile of 16]
+  constexpr int NI16 = MI16 ? 2 * NI : 1, NJ16 = MI16 ? 2 * NJ : 1;
+  f32x4_t acc16[NI16][NJ16];  // MI16: [row tile of 16][column tile of 16]
   auto zero_acc = [&]() __attribute__((always_inline)) {
     if constexpr (MI16) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i)
+      for (int i = 0; i < NI16; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < NJ16; ++j)
 #pragma unroll
           for (int r = 0; r < 4; ++r) acc16[i][j][r] = 0.0f;
       acc_write_fence();
@@ -333,8 +334,14 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // fragment f (0..3: A row tile f, 4..7: B column tile f-4) of K step s of the K tile in `stage`
   // (BPACK: f = 0..7, A row tile f of the whole tile; MI16: s = quarter q of the K tile, fragment = rows
   // 128 * (q % 2) + 16 * f .. + 16 at K 32 * (q / 2) .. + 32, lane l supplying row l % 16, K 8 * (l / 16) .. + 8)
+  // plain form with 16 x 16 tiles: fragment f (0..7: A row tile f of the wavefront's 128 rows, 8..15: B column tile
+  // f - 8 of its 128 columns) of K step ks (32 of the K tile's 64)
+  auto load_frag16 = [&](int stage, int ks, int f) __attribute__((always_inline)) -> bf16x8_t {
+    const unsigned char* st = lds + stage * kStride + ((f < 8) ? (wm * 128) * kRowBytes : kTileBytes + (wn * 128) * kRowBytes);
+    return __builtin_bit_cast(bf16x8_t, *(const uint4*)(st + lds_off((f & 7) * 16 + frag_row, ks * 4 + kgrp)));
+  };
   auto load_frag = [&](int stage, int s, int f) __attribute__((always_inline)) -> bf16x8_t {
-    if constexpr (MI16) {
+    if constexpr (MI16 && BPACK) {
       const unsigned char* st = lds + stage * kStride;
       return __builtin_bit_cast(bf16x8_t, *(const uint4*)(st + lds_off(((s & 1) * 8 + f) * 16 + frag_row, (s >> 1) * 4 + kgrp)));
     } else if constexpr (BPACK) {
@@ -503,18 +510,18 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   };
 
   // Software pipeline, written out instruction by instruction and pinned with scheduling barriers, because a
-  // wavefront issues in order: an MFMA occupies the matrix pipe for 32 cycles, and whatever else has to be
-  // issued (LDS reads of later K steps, async copies of the K tile after next) must sit *between* MFMAs to be
-  // free.  Per K tile: 4 steps of 16 MFMAs, one fragment set fr[s] per step:
-  //   step 0: MFMAs on fr[0], interleaved with the 8 LDS reads of step 1
-  //   step 1: MFMAs on fr[1], interleaved with the 16 LDS reads of steps 2 and 3
-  //   hand-over (after the MFMAs of step 1 are issued): this wavefront's reads of the K tile are complete
+  // wavefront issues in order: an MFMA occupies the matrix pipe for 16 cycles (32 for the 32x32x16 instruction of
+  // the narrow form), and whatever else has to be issued (LDS reads of later K steps, async copies of the K tile after
+  // next) must sit *between* MFMAs to be free.  Per K tile, in the plain forms: four quarters (steps, in the narrow
+  // form) of matrix instructions:
+  //   quarters 0, 1: interleaved with the LDS reads of the fragments the rest of the K tile needs
+  //   hand-over (after the MFMAs of quarter 1 are issued): this wavefront's reads of the K tile are complete
   //     (lgkmcnt) and its copies of the next K tile have landed (vmcnt); barrier -> the next K tile is visible
   //     to all and nobody reads this one's stage any more
-  //   steps 2, 3: MFMAs on fr[2], fr[3], interleaved with the LDS reads of step 0 of the next K tile and the 16
-  //     copies of the K tile after next into the stage just vacated, one every other MFMA slot.
-  // Handing the stage over half-way through the K tile (which costs two more fragment sets) lets the copies be
-  // issued over two steps instead of one: issued in a burst their data arrives in a burst, the LDS is then busy
+  //   quarters 2, 3: interleaved with the LDS reads of the next K tile's first fragments and the 16 copies of the K
+  //     tile after next into the stage just vacated, one every other slot.
+  // Handing the stage over half-way through the K tile (which costs more fragment registers) lets the copies be
+  // issued over two quarters instead of one: issued in a burst their data arrives in a burst, the LDS is then busy
   // with the writes when the wavefronts want their fragment reads, and the wavefronts drift apart (measured:
   // the barrier costs nothing without the copies and a quarter of the loop with them in a 16-slot burst).
   // The barrier is a bare s_barrier: the fence of __syncthreads() would wait for all copies in flight.
@@ -645,8 +652,17 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     wait_vmcnt<kWaveCopies + kCopiesB>();  // K tile 0 landed; K tile 1 may still be in flight
   }
   asm volatile("s_barrier" ::: "memory");
+  if constexpr (MI16 && !BPACK) {
+    // fragment registers of the plain form: fr[q][0..3] = the four A row tiles of quarter q (K step q / 2, rows
+    // 64 * (q % 2) .. + 64 of the wavefront's 128), fr[2 * ks + c / 4][4 + c % 4] = B column tile c of K step ks
 #pragma unroll
-  for (int f = 0; f < (HALFN ? 6 : 8); ++f) fr[0][f] = load_frag(0, 0, f);
+    for (int f = 0; f < 4; ++f) fr[0][f] = load_frag16(0, 0, f);
+#pragma unroll
+    for (int c = 0; c < 8; ++c) fr[c >> 2][4 + (c & 3)] = load_frag16(0, 0, 8 + c);
+  } else {
+#pragma unroll
+    for (int f = 0; f < (HALFN ? 6 : 8); ++f) fr[0][f] = load_frag(0, 0, f);
+  }
   int stage = 0;
   // BPACK form of the K iteration.  The wavefront has two kinds of loads in flight, the B fragment loads into
   // registers and the A copies into LDS.  Each kind retires in order, but the two kinds do NOT retire in order with
@@ -791,27 +807,40 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     stage = stage_next;
     ++b_kt;
   };
+  // Plain form (both operands through LDS, wavefronts 2 x 2: 8 x 8 tiles of 16 x 16 each).  A K tile is four quarters
+  // of 32 matrix instructions: K step q / 2, A row tiles 4 * (q % 2) .. + 4 against the 8 B column tiles; slot t of a
+  // quarter issues row tile t / 4 against the column tiles 2 * (t % 4) and 2 * (t % 4) + 1.
+  //   quarter 0: the 16 LDS reads the rest of this K tile needs (A of quarter 1; A of quarter 2 and B of K step 1)
+  //   quarter 1: the 4 reads of A of quarter 3; then the hand-over as described above
+  //   quarter 2: the 12 reads of the next K tile's quarter 0 (A) and K step 0 (B); 8 of the 16 copies
+  //   quarter 3: the other 8 copies
   auto k_iteration = [&](auto&& advance) __attribute__((always_inline)) {
 #pragma unroll
-    for (int s = 0; s < kSteps; ++s) {
+    for (int q = 0; q < 4; ++q) {
 #pragma unroll
       for (int t = 0; t < 16; ++t) {
-        acc[t >> 2][t & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[s][4 + (t & 3)], fr[s][t >> 2],
-                                                                     acc[t >> 2][t & 3], 0, 0, 0);
-        if (s == 0) {
-          if (t < 8) fr[1][t] = load_frag(stage, 1, t);
-        } else if (s == 1) {
-          if (t < 8) fr[2][t] = load_frag(stage, 2, t);
-          else fr[3][t - 8] = load_frag(stage, 3, t - 8);
-        } else if (s == 2) {
-          if (t < 8) fr[0][t] = load_frag(stage ^ 1, 0, t);
+        const int ks = q >> 1, it = (q & 1) * 4 + (t >> 2), jt = 2 * (t & 3);
+        mfma16_acc(acc16[it][jt], fr[2 * ks + (jt >> 2)][4 + (jt & 3)], fr[q][t >> 2]);
+        if (q == 0) {
+          if (t < 4) fr[1][t] = load_frag16(stage, 0, 4 + t);
+          else if (t < 8) fr[2][t - 4] = load_frag16(stage, 1, t - 4);
+          else fr[2 + ((t - 8) >> 2)][4 + ((t - 8) & 3)] = load_frag16(stage, 1, t);
+        } else if (q == 1) {
+          if (t < 4) fr[3][t] = load_frag16(stage, 1, 4 + t);
+        } else if (q == 2) {
+          if (t < 4) fr[0][t] = load_frag16(stage ^ 1, 0, t);
+          else if (t < 12) fr[(t - 4) >> 2][4 + ((t - 4) & 3)] = load_frag16(stage ^ 1, 0, 4 + t);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mfma16_acc(acc16[it][jt + 1], fr[2 * ks + ((jt + 1) >> 2)][4 + ((jt + 1) & 3)], fr[q][t >> 2]);
+        if (q == 2) {
           if (t & 1) issue_copy(t >> 1);
-        } else {
+        } else if (q == 3) {
           if (t & 1) issue_copy(8 + (t >> 1));
         }
         __builtin_amdgcn_sched_barrier(0);
       }
-      if (s == 1) {
+      if (q == 1) {
         wait_vmcnt<0>();
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
