@@ -2,7 +2,7 @@
 //
 // This is the contraction behind the MX Linear forward.  Both operands are K-major (activations [tokens, K],
 // weights [out, K]), which is the layout v_mfma_f32_16x16x32_bf16 wants: lane l supplies 8 consecutive
-// K-elements of row/column l%16, K-group l/16 (v_mfma_f32_32x32x16_bf16, used by the narrow form: l%32, l/32).  MXINT8 and MXFP values are exactly representable in bf16
+// K-elements of row/column l%16, K-group l/16.  MXINT8 and MXFP values are exactly representable in bf16
 // (<= 8 significant bits times a power of two), so feeding them as bf16 computes the same real-number dot
 // products as the reference's fp32 GEMM on the quantize-dequantized operands; only the summation order
 // differs.
@@ -30,7 +30,6 @@ namespace mase {
 namespace {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int BM = 256, BN = 256, BK = 64;
@@ -42,7 +41,6 @@ constexpr int kTileBytes = BM * kRowBytes;        // 32 KB per operand per stage
 constexpr int kStageBytes = 2 * kTileBytes;       // A then B
 constexpr int kWaveCopies = kTileBytes / 1024 / 4;  // copies per wavefront per operand per K tile = 8
 constexpr int kCopies = 2 * kWaveCopies;          // async copies one wavefront issues per K tile = 16
-constexpr int kSteps = BK / 16;                   // MFMA K steps per K tile = 4
 // epilogue staging, separate from the stages: per wavefront 32 rows of 128 bytes, row stride 144 bytes (16-byte
 // accesses of 16 consecutive rows at one column offset then fall on 64 different banks)
 constexpr int kStgRow = 144;
@@ -175,15 +173,14 @@ __device__ __forceinline__ void load_2_untracked(uint32_t& dst, uint32_t off, co
 // base follow from its product index; rows of A, B and C have the strides lda, ldb, ldc.
 // HALFN (plain form only): output tiles of 256 x 128 for products with at most 128 columns (the value product of an
 // attention block with head dimension 128), where a 256-wide tile would spend half of its matrix instructions on
-// columns that do not exist.  The wavefronts split the tile 2 x 2 into 128 rows x 64 columns (4 x 2 MFMA tiles, 8
+// columns that do not exist.  The wavefronts split the tile 2 x 2 into 128 rows x 64 columns (8 x 4 MFMA tiles, 32
 // MFMAs per K step); B's stage holds 128 rows.
 template <int OUT_DT, bool STREAM, bool BPACK = false, bool BCODES = false, bool BATCHED = false, bool HALFN = false>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p) {
   constexpr int NI = BPACK ? 8 : 4, NJ = (BPACK || HALFN) ? 2 : 4;  // 32 x 32 tiles of a wavefront: rows x columns
-  // All forms but the narrow one compute with v_mfma_f32_16x16x32_bf16 (16 x 4 or 8 x 8 tiles of 16 x 16 per wavefront,
-  // two K steps of 32 per K tile): the same multiply-adds per cycle as the 32x32x16 instruction on paper, but under the board's power
+  // All forms compute with v_mfma_f32_16x16x32_bf16 (16 x 4, 8 x 8 or 8 x 4 tiles of 16 x 16 per wavefront, two K
+  // steps of 32 per K tile): the same multiply-adds per cycle as the 32x32x16 instruction on paper, but under the board's power
   // limit the part sustains a clock about 8 % higher on it (measured with both instructions on random operands).
-  constexpr bool MI16 = !HALFN;
   constexpr int kBN = HALFN ? 128 : BN;                           // columns of an output tile
   constexpr int kCopiesB = HALFN ? kWaveCopies / 2 : kWaveCopies;  // copies of B per wavefront per K tile
   static_assert(!BCODES || BPACK, "codes come in fragment order");
@@ -294,26 +291,16 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     }
   };
 
-  f32x16_t acc[MI16 ? 1 : NI][MI16 ? 1 : NJ];
-  constexpr int NI16 = MI16 ? 2 * NI : 1, NJ16 = MI16 ? 2 * NJ : 1;
-  f32x4_t acc16[NI16][NJ16];  // MI16: [row tile of 16][column tile of 16]
+  constexpr int NI16 = 2 * NI, NJ16 = 2 * NJ;
+  f32x4_t acc16[NI16][NJ16];  // [row tile of 16][column tile of 16]
   auto zero_acc = [&]() __attribute__((always_inline)) {
-    if constexpr (MI16) {
 #pragma unroll
-      for (int i = 0; i < NI16; ++i)
+    for (int i = 0; i < NI16; ++i)
 #pragma unroll
-        for (int j = 0; j < NJ16; ++j)
+      for (int j = 0; j < NJ16; ++j)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) acc16[i][j][r] = 0.0f;
-      acc_write_fence();
-    } else {
-#pragma unroll
-      for (int i = 0; i < NI; ++i)
-#pragma unroll
-        for (int j = 0; j < NJ; ++j)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-    }
+        for (int r = 0; r < 4; ++r) acc16[i][j][r] = 0.0f;
+    acc_write_fence();
   };
   zero_acc();
 
@@ -329,39 +316,29 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // The lane's row and K group within a fragment, which every LDS read of the K loop is addressed with.  Set again
   // from the lane number after each epilogue rather than kept across it: what lives across the epilogue's register
   // demand gets spilled (see lane_now).
-  int frag_row = MI16 ? (lane & 15) : (lane & 31);
-  int kgrp = MI16 ? (lane >> 4) : (lane >> 5);
-  // fragment f (0..3: A row tile f, 4..7: B column tile f-4) of K step s of the K tile in `stage`
-  // (BPACK: f = 0..7, A row tile f of the whole tile; MI16: s = quarter q of the K tile, fragment = rows
-  // 128 * (q % 2) + 16 * f .. + 16 at K 32 * (q / 2) .. + 32, lane l supplying row l % 16, K 8 * (l / 16) .. + 8)
-  // plain form with 16 x 16 tiles: fragment f (0..7: A row tile f of the wavefront's 128 rows, 8..15: B column tile
-  // f - 8 of its 128 columns) of K step ks (32 of the K tile's 64)
+  int frag_row = lane & 15;
+  int kgrp = lane >> 4;
+  // plain forms: fragment f (0..7: A row tile f of the wavefront's 128 rows, 8..15: B column tile f - 8 of its 128
+  // columns; narrow form: 8..11 of its 64 columns) of K step ks (32 of the K tile's 64)
   auto load_frag16 = [&](int stage, int ks, int f) __attribute__((always_inline)) -> bf16x8_t {
-    const unsigned char* st = lds + stage * kStride + ((f < 8) ? (wm * 128) * kRowBytes : kTileBytes + (wn * 128) * kRowBytes);
+    const unsigned char* st = lds + stage * kStride + ((f < 8) ? (wm * 128) * kRowBytes : kTileBytes + (wn * (HALFN ? 64 : 128)) * kRowBytes);
     return __builtin_bit_cast(bf16x8_t, *(const uint4*)(st + lds_off((f & 7) * 16 + frag_row, ks * 4 + kgrp)));
   };
-  auto load_frag = [&](int stage, int s, int f) __attribute__((always_inline)) -> bf16x8_t {
-    if constexpr (MI16 && BPACK) {
-      const unsigned char* st = lds + stage * kStride;
-      return __builtin_bit_cast(bf16x8_t, *(const uint4*)(st + lds_off(((s & 1) * 8 + f) * 16 + frag_row, (s >> 1) * 4 + kgrp)));
-    } else if constexpr (BPACK) {
-      const unsigned char* st = lds + stage * kStride;
-      return __builtin_bit_cast(bf16x8_t, *(const uint4*)(st + lds_off(f * 32 + frag_row, s * 2 + kgrp)));
-    } else {
-      const unsigned char* st = lds + stage * kStride + ((f < 4) ? (wm * 128) * kRowBytes : kTileBytes + (wn * (HALFN ? 64 : 128)) * kRowBytes);
-      return __builtin_bit_cast(bf16x8_t, *(const uint4*)(st + lds_off((f & 3) * 32 + frag_row, s * 2 + kgrp)));
-    }
+  // fragment-ordered forms (only A passes through LDS): fragment f of quarter q of the K tile = rows
+  // 128 * (q % 2) + 16 * f .. + 16 of the whole tile at K 32 * (q / 2) .. + 32, lane l supplying row l % 16, K
+  // 8 * (l / 16) .. + 8
+  auto load_frag = [&](int stage, int q, int f) __attribute__((always_inline)) -> bf16x8_t {
+    const unsigned char* st = lds + stage * kStride;
+    return __builtin_bit_cast(bf16x8_t, *(const uint4*)(st + lds_off(((q & 1) * 8 + f) * 16 + frag_row, (q >> 1) * 4 + kgrp)));
   };
 
   // ---- epilogue of one output tile.  The MFMAs take the B fragment as their first operand, so the accumulators hold
-  // the tile transposed: acc[i][j][q*4 + rr] is C[row, col] with row = i*32 + lane%32 and
-  // col = j*32 + q*8 + (lane/32)*4 + rr, i.e. a lane holds runs of four consecutive columns of one row.  Bias is added
+  // the tile transposed: acc16[i][j][rr] is C[row, col] with row = i*16 + lane%16 and col = j*16 + (lane/16)*4 + rr,
+  // i.e. a lane holds runs of four consecutive columns of one row; a band of 32 rows is made of two row tiles.  Bias is added
   // and the value converted in registers; the runs then pass through the wavefront's own staging rows (32 rows of 128
   // bytes: 64 columns of a 16-bit output, 32 of an fp32 one), from which every lane takes 16 consecutive bytes, so that
   // a store instruction writes 8 rows of 128 contiguous bytes.  Only lanes of one wavefront exchange data (its LDS
   // accesses execute in order, and the writes are waited for before the reads are issued): no barrier.
-  // MI16: acc16[i][j][rr] is C[row, col] with row = i*16 + lane%16 and col = j*16 + (lane/16)*4 + rr; a band of 32 rows
-  // is made of the row tiles 2b and 2b + 1.
   auto epilogue = [&](int ord) __attribute__((always_inline)) {
     int m0, n0, ks;
     tile_origin(ord, m0, n0, ks);
@@ -373,7 +350,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
       Cs = (unsigned char*)p.C + (size_t)bo * p.c_so + (size_t)bi * p.c_si;
     }
     const int lane = lane_now();
-    const int r32 = MI16 ? (lane & 15) : (lane & 31), kgrp = MI16 ? (lane >> 4) : (lane >> 5);
+    const int r32 = lane & 15, kgrp = lane >> 4;
     const int rrow = lane >> 3, chunk = lane & 7;  // read side: row rrow + 8 * pass, 16-byte piece `chunk` of it
     unsigned char* const stg = lds + S * kStageBytes + wave * kStgWave;
     unsigned char* const stg_w = stg + r32 * kStgRow;
@@ -402,10 +379,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
           for (int q = 0; q < 4; ++q)
 #pragma unroll
             for (int rr = 0; rr < 4; ++rr) {
-              // (MI16: bv[j][q] belongs to column tile 2 * j + q / 2 of 16; q % 2 is not used)
-              const int col = MI16 ? n0 + col_base + (2 * j + (q >> 1)) * 16 + kgrp * 4 + rr
-                                   : n0 + col_base + j * 32 + q * 8 + kgrp * 4 + rr;
-              if (MI16 && (q & 1)) continue;
+              // (bv[j][q] belongs to column tile 2 * j + q / 2 of 16; odd q are not used)
+              const int col = n0 + col_base + (2 * j + (q >> 1)) * 16 + kgrp * 4 + rr;
+              if (q & 1) continue;
               if (col < p.N) bv[j][q][rr] = load_bias(p.bias, decltype(dtc)::value, col);
             }
       };
@@ -428,19 +404,13 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
         const int j = jb * kBandTiles + jj;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          // MI16: q = 2 * (column tile of 16 within the 32 columns j) + (row tile of 16 within the band)
+          // q = 2 * (column tile of 16 within the 32 columns j) + (row tile of 16 within the band)
           const int i16 = 2 * i + (q & 1), j16 = 2 * j + (q >> 1);
-          const float* const bq = bv[j][MI16 ? (q & 2) : q];
+          const float* const bq = bv[j][q & 2];
           float v[4];
-          if constexpr (MI16) {
 #pragma unroll
-            for (int rr = 0; rr < 4; ++rr) v[rr] = acc_read(acc16[i16][j16][rr]) + bq[rr];
-          } else {
-#pragma unroll
-            for (int rr = 0; rr < 4; ++rr) v[rr] = acc_read(acc[i][j][q * 4 + rr]) + bq[rr];
-          }
-          unsigned char* const dst = MI16 ? stg_w + (q & 1) * 16 * kStgRow + (jj * 32 + (q >> 1) * 16 + kgrp * 4) * kEsz
-                                          : stg_w + (jj * 32 + q * 8 + kgrp * 4) * kEsz;
+          for (int rr = 0; rr < 4; ++rr) v[rr] = acc_read(acc16[i16][j16][rr]) + bq[rr];
+          unsigned char* const dst = stg_w + (q & 1) * 16 * kStgRow + (jj * 32 + (q >> 1) * 16 + kgrp * 4) * kEsz;
           if constexpr (OUT_DT == MASE_DT_F32) {
             *(uint4*)dst = make_uint4(f2bits(v[0]), f2bits(v[1]), f2bits(v[2]), f2bits(v[3]));
           } else if constexpr (OUT_DT == MASE_DT_BF16) {
@@ -510,10 +480,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   };
 
   // Software pipeline, written out instruction by instruction and pinned with scheduling barriers, because a
-  // wavefront issues in order: an MFMA occupies the matrix pipe for 16 cycles (32 for the 32x32x16 instruction of
-  // the narrow form), and whatever else has to be issued (LDS reads of later K steps, async copies of the K tile after
-  // next) must sit *between* MFMAs to be free.  Per K tile, in the plain forms: four quarters (steps, in the narrow
-  // form) of matrix instructions:
+  // wavefront issues in order: an MFMA occupies the matrix pipe for 16 cycles, and whatever else has to be issued (LDS reads of later K steps, async copies of the K tile after
+  // next) must sit *between* MFMAs to be free.  Per K tile, in the plain forms: four quarters of matrix instructions:
   //   quarters 0, 1: interleaved with the LDS reads of the fragments the rest of the K tile needs
   //   hand-over (after the MFMAs of quarter 1 are issued): this wavefront's reads of the K tile are complete
   //     (lgkmcnt) and its copies of the next K tile have landed (vmcnt); barrier -> the next K tile is visible
@@ -652,16 +620,22 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     wait_vmcnt<kWaveCopies + kCopiesB>();  // K tile 0 landed; K tile 1 may still be in flight
   }
   asm volatile("s_barrier" ::: "memory");
-  if constexpr (MI16 && !BPACK) {
-    // fragment registers of the plain form: fr[q][0..3] = the four A row tiles of quarter q (K step q / 2, rows
+  if constexpr (!BPACK) {
+    // fragment registers of the plain forms: fr[q][0..3] = the four A row tiles of quarter q (K step q / 2, rows
     // 64 * (q % 2) .. + 64 of the wavefront's 128), fr[2 * ks + c / 4][4 + c % 4] = B column tile c of K step ks
 #pragma unroll
     for (int f = 0; f < 4; ++f) fr[0][f] = load_frag16(0, 0, f);
+    if constexpr (HALFN) {
+      // narrow form: four B column tiles per K step, fr[2 * ks + c / 2][4 + c % 2]
 #pragma unroll
-    for (int c = 0; c < 8; ++c) fr[c >> 2][4 + (c & 3)] = load_frag16(0, 0, 8 + c);
+      for (int c = 0; c < 4; ++c) fr[c >> 1][4 + (c & 1)] = load_frag16(0, 0, 8 + c);
+    } else {
+#pragma unroll
+      for (int c = 0; c < 8; ++c) fr[c >> 2][4 + (c & 3)] = load_frag16(0, 0, 8 + c);
+    }
   } else {
 #pragma unroll
-    for (int f = 0; f < (HALFN ? 6 : 8); ++f) fr[0][f] = load_frag(0, 0, f);
+    for (int f = 0; f < 8; ++f) fr[0][f] = load_frag(0, 0, f);
   }
   int stage = 0;
   // BPACK form of the K iteration.  The wavefront has two kinds of loads in flight, the B fragment loads into
@@ -674,7 +648,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
   // been issued, and the hand-over waits for "at most 16 outstanding": the next K tile has landed (its copies are older
   // than those 16), while the young copies and up to that many B loads fly on across the barrier.  The B fragments are
   // proven the same way, by counting the *register loads* issued after them.
-  // bf16 image (MI16): a K tile is four quarters q of 32 matrix instructions 16x16x32: K step q / 2 (32 of the 64 K),
+  // bf16 image: a K tile is four quarters q of 32 matrix instructions 16x16x32: K step q / 2 (32 of the 64 K),
   // rows 128 * (q % 2) .. + 128 (8 row tiles of 16) times the 4 column tiles of 16.  Slot t of a quarter (16 slots)
   // issues the two instructions of row tile t / 2 on the column tiles 2 * (t % 2) and 2 * (t % 2) + 1, with the other
   // work between them.  The B loads of a K tile are issued in the order [K step][column tile]; quarters 0 and 1 need
@@ -849,32 +823,41 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     advance();
     stage ^= 1;
   };
-  // HALFN form of the plain K iteration: 8 MFMAs per step, MFMA t on (A row tile t / 2, B column tile t % 2); fragment
-  // sets hold 6 fragments (4 of A, then 2 of B); the 12 copies of the K tile after next go out one per MFMA slot of
-  // steps 2 and 3 (slots of the 4 copies that B does not have stay empty)
+  // Narrow form (output tiles of 256 x 128; wavefronts 2 x 2: 8 x 4 tiles of 16 x 16 each): quarters of 16 matrix
+  // instructions in 8 slots, slot t on row tile t / 2 of the quarter's four against the column tiles 2 * (t % 2) and
+  // 2 * (t % 2) + 1; fr[q][0..3] = A of quarter q, fr[2 * ks + c / 2][4 + c % 2] = B column tile c of K step ks.
+  //   quarter 0: the 12 LDS reads the rest of the K tile needs (A of quarters 1 and 2 in the first gap of a slot, B of
+  //              K step 1 in the second); quarter 1: A of quarter 3; hand-over
+  //   quarters 2, 3: the 8 reads of the next K tile's quarter 0 and K step 0; the 12 copies of the K tile after next,
+  //              one per slot (slots of the 4 copies that B does not have stay empty)
   auto k_iteration_h = [&](auto&& advance) __attribute__((always_inline)) {
 #pragma unroll
-    for (int s = 0; s < kSteps; ++s) {
+    for (int q = 0; q < 4; ++q) {
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
-        acc[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[s][4 + (t & 1)], fr[s][t >> 1],
-                                                                     acc[t >> 1][t & 1], 0, 0, 0);
-        if (s == 0) {
-          if (t < 6) fr[1][t] = load_frag(stage, 1, t);
-        } else if (s == 1) {
-          if (t < 6) {
-            fr[2][t] = load_frag(stage, 2, t);
-            fr[3][t] = load_frag(stage, 3, t);
-          }
-        } else if (s == 2) {
-          if (t < 6) fr[0][t] = load_frag(stage ^ 1, 0, t);
+        const int ks = q >> 1, it = (q & 1) * 4 + (t >> 1), jt = 2 * (t & 1);
+        mfma16_acc(acc16[it][jt], fr[2 * ks + (jt >> 1)][4], fr[q][t >> 1]);
+        if (q == 0) {
+          if (t < 4) fr[1][t] = load_frag16(stage, 0, 4 + t);
+          else fr[2][t - 4] = load_frag16(stage, 1, t - 4);
+        } else if (q == 1) {
+          if (t < 4) fr[3][t] = load_frag16(stage, 1, 4 + t);
+        } else if (q == 2) {
+          if (t < 4) fr[0][t] = load_frag16(stage ^ 1, 0, t);
+          else fr[(t - 4) >> 1][4 + ((t - 4) & 1)] = load_frag16(stage ^ 1, 0, 8 + (t - 4));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mfma16_acc(acc16[it][jt + 1], fr[2 * ks + (jt >> 1)][5], fr[q][t >> 1]);
+        if (q == 0) {
+          if (t < 4) fr[2 + (t >> 1)][4 + (t & 1)] = load_frag16(stage, 1, 8 + t);
+        } else if (q == 2) {
           issue_copy(t);
-        } else {
+        } else if (q == 3) {
           issue_copy(8 + t);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
-      if (s == 1) {
+      if (q == 1) {
         wait_vmcnt<0>();
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
@@ -932,8 +915,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_tn_kernel(GemmParams p
     zero_acc();
     {
       const int l = lane_now();
-      frag_row = MI16 ? (l & 15) : (l & 31);
-      kgrp = MI16 ? (l >> 4) : (l >> 5);
+      frag_row = l & 15;
+      kgrp = l >> 4;
     }
   }
   wait_vmcnt<0>();  // no copy may still be in flight towards LDS when the work-group retires
