@@ -120,7 +120,10 @@ __device__ __forceinline__ int select_key(const int* key, int P) {
 // Candidates with the same exponent are the same candidate, and with the first-minimum rule only the first of them
 // can win: a work-item evaluates each distinct exponent once (typically 3 of the 11), in percentile order.
 template <int DT, int B>
-__global__ __launch_bounds__(64) void mxint_clip_search_kernel(const void* __restrict__ in, const void* __restrict__ ref,
+// (Blocks of 32: the allocator is asked for three wavefronts per SIMD, i.e. at most 168 registers; left alone it takes
+// 186 to 216 and two wavefronts fit.  bf16: 267 -> 222 us on 8 x 2048 x 4096, same results; the fp16 form would spill
+// and was measured slower, so it keeps its registers.)
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu((B == 32 && DT != MASE_DT_F16) ? 3 : 1))) void mxint_clip_search_kernel(const void* __restrict__ in, const void* __restrict__ ref,
                                                                void* __restrict__ out, uint8_t* __restrict__ choice,
                                                                size_t n_blocks, MxintParams p) {
   using TR = DTypeTraits<DT>;
@@ -177,7 +180,7 @@ __global__ __launch_bounds__(64) void mxint_clip_search_kernel(const void* __res
 }
 
 template <int DT, int B>
-__global__ __launch_bounds__(64) void mxfp_clip_search_kernel(const void* __restrict__ in, const void* __restrict__ ref,
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(B == 32 ? 3 : 1))) void mxfp_clip_search_kernel(const void* __restrict__ in, const void* __restrict__ ref,
                                                               void* __restrict__ out, uint8_t* __restrict__ choice,
                                                               size_t n_blocks, MxfpParams p) {
   using TR = DTypeTraits<DT>;
@@ -253,7 +256,7 @@ __global__ __launch_bounds__(64) void mxfp_clip_search_kernel(const void* __rest
 // element i of the tensor quantized with the scale of percentile P.  MXFP also writes the values the reference
 // scores, code / 2^(F-1) * 2^(scale - 127) on the integer codes with the power in uint8 arithmetic (see above).
 template <int DT, int B>
-__global__ __launch_bounds__(64) void mxint_clip_candidates_kernel(const void* __restrict__ in, void* __restrict__ cand,
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(B == 32 ? 3 : 1))) void mxint_clip_candidates_kernel(const void* __restrict__ in, void* __restrict__ cand,
                                                                    size_t n_blocks, MxintParams p) {
   using TR = DTypeTraits<DT>;
   constexpr int V = TR::kVec;
@@ -283,7 +286,7 @@ __global__ __launch_bounds__(64) void mxint_clip_candidates_kernel(const void* _
 }
 
 template <int DT, int B>
-__global__ __launch_bounds__(64) void mxfp_clip_candidates_kernel(const void* __restrict__ in, void* __restrict__ cand,
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(B == 32 ? 3 : 1))) void mxfp_clip_candidates_kernel(const void* __restrict__ in, void* __restrict__ cand,
                                                                   void* __restrict__ score, size_t n_blocks,
                                                                   MxfpParams p) {
   using TR = DTypeTraits<DT>;
